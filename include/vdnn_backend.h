@@ -1,0 +1,198 @@
+/* C ABI of the MI355X (gfx950) device back end of the vDNN engine.
+ *
+ * This is the lower boundary of the training hot path: everything the reference obtains from
+ * cuDNN, cuBLAS, cnmem and the CUDA runtime is reached through these entry points, and the C++
+ * host classes (Layer, Network) call nothing else.  Plain pointers and sizes only.
+ *
+ * Conventions
+ *   - every function returns an int status: VDNN_OK (0), VDNN_OOM (-1, the pool cannot serve a
+ *     request; mirrors ASSERT_EQ's -1 in layer.h:110-128), or a value < -1 for a hard error;
+ *     vdnn_last_error() holds a message for the last failure on the calling thread.
+ *   - tensors are fp32, NCHW; filters KCRS; convolution is cross-correlation, dilation 1
+ *     (vdnn.h:11-12, 19-20).
+ *   - a stream argument of NULL means the context's compute stream.
+ *   - kernels are asynchronous on their stream; nothing here synchronises unless it says so.
+ *   - a context created with VDNN_CTX_PLAN_ONLY touches no device: the pool hands out addresses of
+ *     a virtual range, copies and kernels return VDNN_OK without doing anything.  It exists so the
+ *     allocation schedule of a policy can be replayed on a machine without a GPU; it computes
+ *     nothing and is not a CPU implementation of the math.
+ *   - not thread-safe: one host thread per context, like the reference.
+ */
+#ifndef VDNN_AMD_BACKEND_H_
+#define VDNN_AMD_BACKEND_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VDNN_OK       0
+#define VDNN_OOM     (-1)
+#define VDNN_EINVAL  (-2)
+#define VDNN_EDEVICE (-3)
+
+#define VDNN_CTX_PLAN_ONLY 1
+
+/* passes of a convolution, for vdnn_conv_workspace_bytes */
+#define VDNN_PASS_FWD        0
+#define VDNN_PASS_BWD_DATA   1
+#define VDNN_PASS_BWD_FILTER 2
+
+typedef struct vdnn_ctx vdnn_ctx;
+typedef void* vdnn_stream_t; /* a hipStream_t */
+typedef void* vdnn_event_t;  /* a hipEvent_t */
+
+/* One layer's geometry: input n,c,h,w; filter k,r,s; padding and stride (the argument list of the
+ * reference's Layer constructor, layer.h:133-154). */
+typedef struct {
+    int n, c, h, w;
+    int k, r, s;
+    int pad_h, pad_w, stride_h, stride_w;
+} vdnn_shape_t;
+
+/* ---- context --------------------------------------------------------------------------------- */
+/* Replaces cudnnCreate/cublasCreate/cudaSetDevice (network.cu:16, 39-40; vdnn.cu:59). Creates the
+ * compute stream and the two copy streams. */
+int vdnn_ctx_create(vdnn_ctx** out, int device, int flags);
+int vdnn_ctx_destroy(vdnn_ctx* ctx);
+const char* vdnn_last_error(void);
+/* cudaGetDeviceProperties(...).totalGlobalMem (network.cu:35-36, 48). */
+int vdnn_device_mem_info(vdnn_ctx* ctx, size_t* free_bytes, size_t* total_bytes);
+int vdnn_device_synchronize(vdnn_ctx* ctx);
+/* Streams owned by the context: compute, device-to-host, host-to-device. The reference has
+ * stream_compute and one stream_memory (network.cu:41-42); copies get one stream per direction. */
+vdnn_stream_t vdnn_ctx_stream_compute(vdnn_ctx* ctx);
+vdnn_stream_t vdnn_ctx_stream_d2h(vdnn_ctx* ctx);
+vdnn_stream_t vdnn_ctx_stream_h2d(vdnn_ctx* ctx);
+
+/* ---- pooled device memory (replaces cnmem: network.cu:47-53, layer.cu:989-1011) --------------- */
+/* cnmemInit: reserve `bytes` of device memory once; all later requests are carved from it. */
+int vdnn_pool_init(vdnn_ctx* ctx, size_t bytes);
+/* cnmemFinalize (network.cu:103). Releases the reservation and every block in it. */
+int vdnn_pool_finalize(vdnn_ctx* ctx);
+/* cnmemMalloc. VDNN_OOM when no free block fits or the cap would be exceeded. */
+int vdnn_pool_malloc(vdnn_ctx* ctx, void** ptr, size_t bytes);
+/* cnmemFree. */
+int vdnn_pool_free(vdnn_ctx* ctx, void* ptr);
+/* cnmemMemGetInfo (network.cu:1069, 1098, 1129, 1176): free and total bytes of the pool. */
+int vdnn_pool_info(vdnn_ctx* ctx, size_t* free_bytes, size_t* total_bytes);
+/* High-water marks since the last reset: bytes in use, and the highest end offset handed out. */
+int vdnn_pool_peak(vdnn_ctx* ctx, size_t* peak_in_use, size_t* peak_extent);
+int vdnn_pool_reset_peak(vdnn_ctx* ctx);
+/* Artificial limit on bytes in use (0 = none); requests beyond it return VDNN_OOM. */
+int vdnn_pool_set_cap(vdnn_ctx* ctx, size_t cap_bytes);
+/* Number of live blocks (leak checks). */
+int vdnn_pool_live_blocks(vdnn_ctx* ctx, size_t* count);
+
+/* ---- streams, events, copies (replaces the CUDA runtime calls of layer.cu:969-987,
+ *      network.cu:918-934, 1090-1091, 1168-1169) --------------------------------------------- */
+int vdnn_stream_synchronize(vdnn_ctx* ctx, vdnn_stream_t stream);
+int vdnn_event_create(vdnn_ctx* ctx, vdnn_event_t* out, int with_timing);
+int vdnn_event_destroy(vdnn_ctx* ctx, vdnn_event_t ev);
+int vdnn_event_record(vdnn_ctx* ctx, vdnn_event_t ev, vdnn_stream_t stream);
+int vdnn_stream_wait_event(vdnn_ctx* ctx, vdnn_stream_t stream, vdnn_event_t ev);
+int vdnn_event_synchronize(vdnn_ctx* ctx, vdnn_event_t ev);
+int vdnn_event_elapsed_ms(vdnn_ctx* ctx, vdnn_event_t start, vdnn_event_t stop, float* ms);
+/* cudaMallocHost / cudaFreeHost: pinned staging buffers for offloaded tensors. */
+int vdnn_host_alloc_pinned(vdnn_ctx* ctx, void** ptr, size_t bytes);
+int vdnn_host_free_pinned(vdnn_ctx* ctx, void* ptr);
+/* cudaMemcpyAsync D2H (offloadSrcData, layer.cu:969-977) and H2D (prefetchPreviousSrcData,
+ * layer.cu:979-987). */
+int vdnn_memcpy_d2h_async(vdnn_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes, vdnn_stream_t stream);
+int vdnn_memcpy_h2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes, vdnn_stream_t stream);
+/* Blocking copies (cudaMemcpy: layer.cu:940-942, network.cu:827). */
+int vdnn_memcpy_d2h(vdnn_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);
+int vdnn_memcpy_h2d(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
+int vdnn_memcpy_d2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes, vdnn_stream_t stream);
+
+/* ---- convolution (replaces cuDNN: layer.cu:539-665) ------------------------------------------ */
+/* Output extent of a convolution or pooling window: (in + 2*pad - window)/stride + 1
+ * (cudnnGetConvolution2dForwardOutputDim layer.cu:208-216, cudnnGetPooling2dForwardOutputDim
+ * layer.cu:432-439). */
+int vdnn_out_dim(int in, int pad, int window, int stride);
+/* cudnnGetConvolution*WorkspaceSize (layer.cu:268-294). algo_mode is a vdnnAlgoMode_t value.
+ * VDNN_MEMORY_OPT_ALGO always returns 0. */
+size_t vdnn_conv_workspace_bytes(const vdnn_shape_t* shape, int algo_mode, int pass);
+/* cudnnConvolutionForward + cudnnAddTensor (layer.cu:560-582): y = x (*) w + bias[k], the bias is
+ * added once after the full reduction. bias may be NULL (no add). */
+int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                  const float* x, const float* w, const float* bias, float* y,
+                  void* workspace, size_t workspace_bytes);
+/* cudnnAddTensor alone (layer.cu:576-582): y[n,k,:,:] += bias[k]. */
+int vdnn_bias_add(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw, const float* bias, float* y);
+/* cudnnConvolutionBackwardData (layer.cu:616-625): dx = w^T (*) dy, alpha 1, beta 0. */
+int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                       const float* dy, const float* w, float* dx,
+                       void* workspace, size_t workspace_bytes);
+/* cudnnConvolutionBackwardBias with alpha=-lr, beta=1 (layer.cu:631-637):
+ * bias[k] += alpha * sum_{n,p,q} dy[n,k,p,q]. Fixed summation order. */
+int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape,
+                           const float* dy, float* bias, float alpha);
+/* cudnnConvolutionBackwardFilter with alpha=-lr, beta=1 (layer.cu:651-660):
+ * w[k,c,r,s] += alpha * sum_{n,p,q} dy[n,k,p,q] * x[n,c,p*sh-ph+r,q*sw-pw+s]. Fixed summation
+ * order (no floating-point atomics). */
+int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                             const float* x, const float* dy, float* w, float alpha,
+                             void* workspace, size_t workspace_bytes);
+
+/* ---- fully connected (replaces cuBLAS: layer.cu:667-764) ------------------------------------- */
+/* Sgemm(T,N) + rank-1 bias broadcast (layer.cu:677-706): y[n,o] = sum_i w[o,i] x[n,i] + bias[o].
+ * w is [c_out][c_in] row-major. */
+int vdnn_fc_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                const float* x, const float* w, const float* bias, float* y);
+/* Sgemm(N,N) (layer.cu:725-733): dx[n,i] = sum_o w[o,i] dy[n,o]. */
+int vdnn_fc_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                     const float* dy, const float* w, float* dx);
+/* Sgemm(N,T) alpha=-lr beta=1 (layer.cu:736-744): w[o,i] += alpha * sum_n x[n,i] dy[n,o]. */
+int vdnn_fc_bwd_weight_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                           const float* x, const float* dy, float* w, float alpha);
+/* Sgemm with a ones vector, alpha=-lr beta=1 (layer.cu:747-761): bias[o] += alpha * sum_n dy[n,o]. */
+int vdnn_fc_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out,
+                         const float* dy, float* bias, float alpha);
+
+/* ---- bandwidth-bound layers (replaces cuDNN: layer.cu:766-915) -------------------------------- */
+/* cudnnActivationForward, ReLU, NaN propagates (layer.cu:774-781, 380-385): y = x > 0 ? x : (x!=x ? x : 0). */
+int vdnn_relu_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y);
+/* cudnnActivationBackward (layer.cu:802-811): dx = x > 0 ? dy : 0. x may be NULL, then the test is
+ * y > 0, which selects the same elements. */
+int vdnn_relu_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, const float* y,
+                  const float* dy, float* dx);
+/* cudnnPoolingForward, max, NaN not propagated (layer.cu:875-882, 416-428). Window r x s. */
+int vdnn_maxpool_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* x, float* y);
+/* cudnnPoolingBackward (layer.cu:903-912): each window's dy goes to its first maximum in row-major
+ * window order; overlapping windows accumulate in row-major order of the windows. */
+int vdnn_maxpool_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape,
+                     const float* x, const float* y, const float* dy, float* dx);
+/* Cross-channel LRN, window 5, alpha 1e-4, beta 0.75, k 2 (no counterpart in the reference; the
+ * AlexNet configuration names it): scale = k + alpha/5 * sum_{|c'-c|<=2} x_c'^2, y = x * scale^-beta. */
+int vdnn_lrn_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const float* x, float* y);
+int vdnn_lrn_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw,
+                 const float* x, const float* y, const float* dy, float* dx);
+/* cudnnSoftmaxForward ACCURATE / INSTANCE (layer.cu:824-832): per sample over `classes`. */
+int vdnn_softmax_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* x, float* y);
+/* cudnnSoftmaxBackward (layer.cu:853-862): dx_i = y_i * (dy_i - sum_j dy_j y_j). */
+int vdnn_softmax_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes,
+                     const float* y, const float* dy, float* dx);
+/* calculateDiffTensor (network.cu:3-8): r = a - b. */
+int vdnn_sub(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* a, const float* b, float* r);
+/* fillVectorWithOnes generalised (layer.cu:33-38): p[i] = value. */
+int vdnn_fill(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float value, float* p);
+/* Fused softmax + cross-entropy on integer labels (no counterpart in the reference, which never
+ * forms a loss): prob = softmax(logits); loss[0] = -(1/n) sum_n log prob[n,label_n], summed in
+ * sample order by one workgroup. loss may be NULL. */
+int vdnn_softmax_ce_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* logits,
+                        const int32_t* labels, float* prob, float* loss);
+/* dlogits = (prob - onehot(label)) / n. */
+int vdnn_softmax_ce_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* prob,
+                        const int32_t* labels, float* dlogits);
+/* Mean cross-entropy of a probability tensor against a dense target (one-hot or soft):
+ * loss[0] = -(1/n) sum_n sum_c target[n,c] * log(max(prob[n,c], FLT_MIN)). Monitoring only. */
+int vdnn_cross_entropy_dense(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes,
+                             const float* prob, const float* target, float* loss);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
