@@ -1,0 +1,327 @@
+"""GPU parity: every HIP kernel against the CPU checker, through the C ABI.
+
+Tolerances: convolution and FC results are fp32 MFMA sums compared with the checker's float64
+accumulation: relative error (max |a-b| / max |b|) <= 1e-4, the bound the hot path is specified to.
+ReLU, max-pool, subtraction and fills are exact (bit-identical).
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+import vdnn_implementation_amd.backend as be
+from gpu_util import Dev, announce, conv_shape, gpu_conv_bwd_bias, gpu_conv_bwd_data, gpu_conv_bwd_filter, gpu_conv_fwd
+from util import assert_close, golden
+from vdnn_implementation_amd.backend import check, lib
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = be.Context(pool_bytes=6 << 30)
+    yield c
+    c.close()
+
+
+@pytest.fixture(autouse=True)
+def accurate_oracle():
+    oracle.set_accumulate_double(True)
+    yield
+    oracle.set_accumulate_double(False)
+
+
+CONV_GOLDEN = ["vgg_3x3_p1", "alex_11x11_s4", "alex_5x5_p2", "overfeat_5x5_p0", "overfeat_6x6_to_1x1",
+               "overfeat_1x1", "odd_3x3_s2_p1"]
+
+
+@pytest.mark.parametrize("name", CONV_GOLDEN)
+def test_conv_golden(ctx, name):
+    f = golden("conv_" + name)
+    g = conv_shape(f["geom"])
+    announce("conv golden", name, "fwd")
+    assert_close(gpu_conv_fwd(ctx, g, f["x"], f["w"], f["b"]), f["y"], TOL, "fwd")
+    announce("conv golden", name, "bwd_data")
+    assert_close(gpu_conv_bwd_data(ctx, g, f["dy"], f["w"]), f["dx"], TOL, "bwd data")
+    alpha = np.float32(-0.37)
+    announce("conv golden", name, "bwd_filter")
+    assert_close(gpu_conv_bwd_filter(ctx, g, f["x"], f["dy"], f["w"], alpha), f["w"] + alpha * f["dw"], TOL, "bwd filter")
+    announce("conv golden", name, "bwd_bias")
+    assert_close(gpu_conv_bwd_bias(ctx, g, f["dy"], f["b"], alpha), f["b"] + alpha * f["db"], TOL, "bwd bias")
+
+
+# (n, c, h, w, k, r, s, pad_h, pad_w, stride_h, stride_w): tile edges, several reduction slices, split reductions
+CONV_RANDOM = [
+    (3, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1),     # VGG-like, M = 64 tile
+    (2, 128, 14, 14, 256, 3, 3, 1, 1, 1, 1),   # M > 128: two row tiles
+    (2, 3, 32, 32, 64, 3, 3, 1, 1, 1, 1),      # first layer: 27-deep reduction, 3-row backward-data
+    (2, 70, 9, 13, 130, 3, 3, 1, 1, 1, 1),     # nothing divides the tiles
+    (2, 3, 67, 67, 96, 11, 11, 0, 0, 4, 4),    # AlexNet conv1 geometry
+    (2, 48, 27, 27, 96, 5, 5, 2, 2, 1, 1),     # AlexNet conv2 geometry
+    (2, 40, 12, 12, 72, 5, 5, 0, 0, 1, 1),     # OverFeat conv2 geometry
+    (5, 64, 6, 6, 200, 6, 6, 0, 0, 1, 1),      # OverFeat 6x6 -> 1x1
+    (9, 300, 1, 1, 150, 1, 1, 0, 0, 1, 1),     # OverFeat 1x1 on 1x1
+    (1, 16, 20, 24, 32, 3, 5, 1, 2, 2, 1),     # asymmetric everything
+]
+
+
+@pytest.mark.parametrize("geom", CONV_RANDOM, ids=lambda g: "x".join(map(str, g)))
+def test_conv_random_against_oracle(ctx, geom):
+    rng = np.random.default_rng(hash(geom) % (2 ** 31))
+    g, og = be.shape(*geom), oracle.shape(*geom)
+    x = rng.standard_normal((g.n, g.c, g.h, g.w)).astype(np.float32)
+    w = (rng.standard_normal((g.k, g.c, g.r, g.s)) * np.sqrt(2.0 / (g.c * g.r * g.s))).astype(np.float32)
+    b = rng.standard_normal(g.k).astype(np.float32)
+    want_y = oracle.conv_fwd(og, x, w, b)
+    announce("conv random", geom, "fwd")
+    assert_close(gpu_conv_fwd(ctx, g, x, w, b), want_y, TOL, "fwd")
+    dy = rng.standard_normal(want_y.shape).astype(np.float32)
+    announce("conv random", geom, "bwd_data")
+    assert_close(gpu_conv_bwd_data(ctx, g, dy, w), oracle.conv_bwd_data(og, dy, w), TOL, "bwd data")
+    # compare gradients, not weights: alpha = 1 on a zero filter
+    announce("conv random", geom, "bwd_filter")
+    zero = np.zeros_like(w)
+    assert_close(gpu_conv_bwd_filter(ctx, g, x, dy, zero, np.float32(1.0)), oracle.conv_bwd_filter_sgd(og, x, dy, zero, 1.0), TOL, "bwd filter")
+    announce("conv random", geom, "bwd_filter sgd")
+    got = gpu_conv_bwd_filter(ctx, g, x, dy, w, np.float32(-1e-5))
+    assert_close(got, oracle.conv_bwd_filter_sgd(og, x, dy, w, -1e-5), 1e-6, "fused sgd")
+    announce("conv random", geom, "bwd_bias")
+    assert_close(gpu_conv_bwd_bias(ctx, g, dy, b, np.float32(-0.5)), oracle.conv_bwd_bias_sgd(og, dy, b, -0.5), TOL, "bwd bias")
+
+
+def test_conv_results_do_not_depend_on_the_run(ctx):
+    """Split reductions are ordered: two runs give identical bits."""
+    geom = (4, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1)
+    rng = np.random.default_rng(5)
+    g = be.shape(*geom)
+    x = rng.standard_normal((4, 64, 28, 28)).astype(np.float32)
+    dy = rng.standard_normal((4, 64, 28, 28)).astype(np.float32)
+    w = rng.standard_normal((64, 64, 3, 3)).astype(np.float32)
+    announce("determinism bwd_filter")
+    a = gpu_conv_bwd_filter(ctx, g, x, dy, w, np.float32(-1e-3))
+    b = gpu_conv_bwd_filter(ctx, g, x, dy, w, np.float32(-1e-3))
+    assert np.array_equal(a, b)
+    announce("determinism bwd_bias")
+    assert np.array_equal(gpu_conv_bwd_bias(ctx, g, dy, w[:, 0, 0, 0], np.float32(1.0)), gpu_conv_bwd_bias(ctx, g, dy, w[:, 0, 0, 0], np.float32(1.0)))
+
+
+def _fc_all(ctx, x, w, b, dy, alpha):
+    n, cin = x.shape
+    cout = w.shape[0]
+    with Dev(ctx) as d:
+        dx_, dw_, db_, ddy = d.up(x), d.up(w), d.up(b), d.up(dy)
+        y, gx = d.empty((n, cout)), d.empty((n, cin))
+        check(lib.vdnn_fc_fwd(ctx.handle, None, n, cin, cout, dx_.ptr, dw_.ptr, db_.ptr, y.ptr))
+        check(lib.vdnn_fc_bwd_data(ctx.handle, None, n, cin, cout, ddy.ptr, dw_.ptr, gx.ptr))
+        check(lib.vdnn_fc_bwd_weight_sgd(ctx.handle, None, n, cin, cout, dx_.ptr, ddy.ptr, dw_.ptr, alpha))
+        check(lib.vdnn_fc_bwd_bias_sgd(ctx.handle, None, n, cout, ddy.ptr, db_.ptr, alpha))
+        return y.download((n, cout)), gx.download((n, cin)), dw_.download(w.shape), db_.download(b.shape)
+
+
+def test_fc_golden(ctx):
+    f = golden("fc")
+    alpha = np.float32(0.21)
+    announce("fc golden")
+    y, dx, w2, b2 = _fc_all(ctx, f["x"], f["w"], f["b"], f["dy"], alpha)
+    assert_close(y, f["y"], TOL)
+    assert_close(dx, f["dx"], TOL)
+    assert_close(w2, f["w"] + alpha * f["dw"], TOL)
+    assert_close(b2, f["b"] + alpha * f["db"], TOL)
+
+
+@pytest.mark.parametrize("n,cin,cout", [(128, 1000, 520), (64, 2304, 512), (32, 777, 1000), (5, 40, 33)])
+def test_fc_random_against_oracle(ctx, n, cin, cout):
+    rng = np.random.default_rng(n * 7 + cin)
+    x = rng.standard_normal((n, cin)).astype(np.float32)
+    w = (rng.standard_normal((cout, cin)) * np.sqrt(2.0 / cin)).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    dy = rng.standard_normal((n, cout)).astype(np.float32)
+    alpha = np.float32(-0.01)
+    announce("fc random", n, cin, cout)
+    y, dx, w2, b2 = _fc_all(ctx, x, w, b, dy, alpha)
+    assert_close(y, oracle.fc_fwd(x, w, b), TOL, "fwd")
+    assert_close(dx, oracle.fc_bwd_data(dy, w), TOL, "bwd data")
+    assert_close((w2.astype(np.float64) - w) / alpha, (oracle.fc_bwd_weight_sgd(x, dy, w, alpha).astype(np.float64) - w) / alpha, 1e-3, "dW")
+    assert_close(w2, oracle.fc_bwd_weight_sgd(x, dy, w, alpha), 1e-6, "fused sgd")
+    assert_close(b2, oracle.fc_bwd_bias_sgd(dy, b, alpha), 1e-6, "bias")
+
+
+@pytest.mark.parametrize("count", [1, 3, 4, 1023, 4096 * 33 + 5])
+def test_relu_is_exact(ctx, count):
+    rng = np.random.default_rng(count)
+    x = rng.standard_normal(count).astype(np.float32)
+    x[::7] = 0.0
+    if count > 16:
+        x[3], x[5], x[6], x[9] = np.nan, np.inf, -np.inf, -0.0
+    dy = rng.standard_normal(count).astype(np.float32)
+    announce("relu", count)
+    with Dev(ctx) as d:
+        a, g = d.up(x), d.up(dy)
+        y, dx, dx2 = d.empty(count), d.empty(count), d.empty(count)
+        check(lib.vdnn_relu_fwd(ctx.handle, None, count, a.ptr, y.ptr))
+        check(lib.vdnn_relu_bwd(ctx.handle, None, count, a.ptr, y.ptr, g.ptr, dx.ptr))
+        check(lib.vdnn_relu_bwd(ctx.handle, None, count, None, y.ptr, g.ptr, dx2.ptr))
+        gy, gdx, gdx2 = y.download(count), dx.download(count), dx2.download(count)
+    wy = oracle.relu_fwd(x)
+    assert np.array_equal(gy.view(np.uint32), wy.view(np.uint32))
+    wdx = oracle.relu_bwd(x, wy, dy)
+    assert np.array_equal(gdx, wdx)
+    assert np.array_equal(gdx2, wdx)  # from y alone: same elements selected
+
+
+POOLS = [(2, 3, 13, 15, 3, 2), (2, 3, 12, 12, 2, 2), (1, 2, 7, 9, 2, 2), (3, 5, 8, 16, 2, 2), (2, 4, 27, 27, 3, 2), (1, 2, 6, 10, 2, 2)]
+
+
+@pytest.mark.parametrize("n,c,h,w,win,stride", POOLS)
+@pytest.mark.parametrize("ties", [False, True])
+def test_maxpool_is_exact(ctx, n, c, h, w, win, stride, ties):
+    rng = np.random.default_rng(h * 31 + w)
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    if ties:
+        x = np.maximum(np.round(x), 0).astype(np.float32)  # post-ReLU-like data full of equal values
+    g, og = be.shape(n, c, h, w, 0, win, win, 0, 0, stride, stride), oracle.shape(n, c, h, w, 0, win, win, 0, 0, stride, stride)
+    wy = oracle.maxpool_fwd(og, x)
+    dy = rng.standard_normal(wy.shape).astype(np.float32)
+    announce("maxpool", (n, c, h, w, win, stride), "ties" if ties else "")
+    with Dev(ctx) as d:
+        a, gdy = d.up(x), d.up(dy)
+        y, dx = d.empty(wy.shape), d.empty(x.shape)
+        check(lib.vdnn_maxpool_fwd(ctx.handle, None, g, a.ptr, y.ptr))
+        check(lib.vdnn_maxpool_bwd(ctx.handle, None, g, a.ptr, y.ptr, gdy.ptr, dx.ptr))
+        gy, gdx = y.download(wy.shape), dx.download(x.shape)
+    assert np.array_equal(gy, wy)
+    assert np.array_equal(gdx, oracle.maxpool_bwd(og, x, wy, dy))
+
+
+def test_maxpool_golden(ctx):
+    for name in ("pool_3x3_s2", "pool_2x2_s2", "pool_2x2_s2_odd"):
+        f = golden(name)
+        g = conv_shape(f["geom"])
+        announce("maxpool golden", name)
+        with Dev(ctx) as d:
+            a, gdy = d.up(f["x"]), d.up(f["dy"])
+            y, dx = d.empty(f["y"].shape), d.empty(f["x"].shape)
+            check(lib.vdnn_maxpool_fwd(ctx.handle, None, g, a.ptr, y.ptr))
+            check(lib.vdnn_maxpool_bwd(ctx.handle, None, g, a.ptr, y.ptr, gdy.ptr, dx.ptr))
+            assert np.array_equal(y.download(f["y"].shape), f["y"])
+            assert_close(dx.download(f["x"].shape), f["dx"], 1e-7)
+
+
+@pytest.mark.parametrize("shape,scale", [((2, 9, 4, 5), 1.0), ((2, 9, 4, 5), 60.0), ((3, 96, 11, 13), 30.0), ((1, 3, 5, 5), 10.0)])
+def test_lrn(ctx, shape, scale):
+    rng = np.random.default_rng(int(scale) + shape[1])
+    x = (rng.standard_normal(shape) * scale).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    wy = oracle.lrn_fwd(x)
+    n, c, hw = shape[0], shape[1], shape[2] * shape[3]
+    announce("lrn", shape, scale)
+    with Dev(ctx) as d:
+        a, gdy = d.up(x), d.up(dy)
+        y, dx = d.empty(shape), d.empty(shape)
+        check(lib.vdnn_lrn_fwd(ctx.handle, None, n, c, hw, a.ptr, y.ptr))
+        check(lib.vdnn_lrn_bwd(ctx.handle, None, n, c, hw, a.ptr, y.ptr, gdy.ptr, dx.ptr))
+        gy, gdx = y.download(shape), dx.download(shape)
+    assert_close(gy, wy, 1e-5, "fwd")
+    assert_close(gdx, oracle.lrn_bwd(x, wy, dy), 1e-5, "bwd")
+    if shape == (2, 9, 4, 5):
+        f = golden("lrn" if scale == 1.0 else "lrn_large_inputs")
+        with Dev(ctx) as d:
+            a, gdy, gy_ = d.up(f["x"]), d.up(f["dy"]), d.up(f["y"])
+            y, dx = d.empty(shape), d.empty(shape)
+            check(lib.vdnn_lrn_fwd(ctx.handle, None, n, c, hw, a.ptr, y.ptr))
+            check(lib.vdnn_lrn_bwd(ctx.handle, None, n, c, hw, a.ptr, gy_.ptr, gdy.ptr, dx.ptr))
+            assert_close(y.download(shape), f["y"], 1e-5, "golden fwd")
+            assert_close(dx.download(shape), f["dx"], 1e-5, "golden bwd")
+
+
+@pytest.mark.parametrize("n,classes", [(5, 17), (128, 1000), (3, 1), (2, 257)])
+def test_softmax(ctx, n, classes):
+    rng = np.random.default_rng(classes)
+    x = (rng.standard_normal((n, classes)) * 4).astype(np.float32)
+    dy = rng.standard_normal((n, classes)).astype(np.float32)
+    wy = oracle.softmax_fwd(x)
+    announce("softmax", n, classes)
+    with Dev(ctx) as d:
+        a, gdy = d.up(x), d.up(dy)
+        y, dx = d.empty(x.shape), d.empty(x.shape)
+        check(lib.vdnn_softmax_fwd(ctx.handle, None, n, classes, a.ptr, y.ptr))
+        check(lib.vdnn_softmax_bwd(ctx.handle, None, n, classes, y.ptr, gdy.ptr, dx.ptr))
+        gy, gdx = y.download(x.shape), dx.download(x.shape)
+    assert_close(gy, wy, 1e-5, "fwd")
+    assert np.allclose(gy.sum(axis=1), 1.0, atol=1e-5)
+    assert_close(gdx, oracle.softmax_bwd(gy, dy), 1e-5, "bwd")
+
+
+def test_softmax_golden_and_ce(ctx):
+    f = golden("softmax")
+    n, classes = f["x"].shape
+    announce("softmax golden")
+    with Dev(ctx) as d:
+        a, gdy, gy = d.up(f["x"]), d.up(f["dy"]), d.up(f["y"])
+        y, dx = d.empty(f["x"].shape), d.empty(f["x"].shape)
+        check(lib.vdnn_softmax_fwd(ctx.handle, None, n, classes, a.ptr, y.ptr))
+        check(lib.vdnn_softmax_bwd(ctx.handle, None, n, classes, gy.ptr, gdy.ptr, dx.ptr))
+        assert_close(y.download(f["x"].shape), f["y"], 1e-5)
+        assert_close(dx.download(f["x"].shape), f["dx"], 1e-5)
+    f = golden("softmax_ce")
+    n, classes = f["x"].shape
+    announce("softmax-ce golden")
+    with Dev(ctx) as d:
+        a, lab = d.up(f["x"]), d.up(f["labels"], np.int32)
+        prob, dlog, loss, loss2, onehot = d.empty(f["x"].shape), d.empty(f["x"].shape), d.empty(1), d.empty(1), d.up(np.eye(classes, dtype=np.float32)[f["labels"]])
+        check(lib.vdnn_softmax_ce_fwd(ctx.handle, None, n, classes, a.ptr, lab.ptr, prob.ptr, loss.ptr))
+        check(lib.vdnn_softmax_ce_bwd(ctx.handle, None, n, classes, prob.ptr, lab.ptr, dlog.ptr))
+        check(lib.vdnn_cross_entropy_dense(ctx.handle, None, n, classes, prob.ptr, onehot.ptr, loss2.ptr))
+        assert_close(prob.download(f["x"].shape), f["prob"], 1e-5)
+        assert abs(loss.download(1)[0] - f["loss"][0]) <= 1e-5 * abs(f["loss"][0])
+        assert abs(loss2.download(1)[0] - f["loss"][0]) <= 1e-5 * abs(f["loss"][0])
+        assert_close(dlog.download(f["x"].shape), f["dx"], 1e-5)
+
+
+def test_sub_fill_bias_add_are_exact(ctx):
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal(100003).astype(np.float32)
+    b = rng.standard_normal(100003).astype(np.float32)
+    announce("sub/fill/bias_add")
+    with Dev(ctx) as d:
+        da, db, r, f = d.up(a), d.up(b), d.empty(a.shape), d.empty(777)
+        check(lib.vdnn_sub(ctx.handle, None, a.size, da.ptr, db.ptr, r.ptr))
+        check(lib.vdnn_fill(ctx.handle, None, 777, 1.0, f.ptr))
+        assert np.array_equal(r.download(a.shape), a - b)
+        assert np.array_equal(f.download(777), np.ones(777, np.float32))
+        y = rng.standard_normal((3, 5, 7, 2)).astype(np.float32)
+        bias = rng.standard_normal(5).astype(np.float32)
+        dy_, dbias = d.up(y), d.up(bias)
+        check(lib.vdnn_bias_add(ctx.handle, None, 3, 5, 14, dbias.ptr, dy_.ptr))
+        assert np.array_equal(dy_.download(y.shape), y + bias[None, :, None, None])
+
+
+def test_offload_prefetch_round_trip_is_byte_identical(ctx):
+    """offloadSrcData / prefetchPreviousSrcData (layer.cu:969-987): D2H into pinned memory on the
+    copy stream, H2D back into a fresh block; the bytes must survive unchanged."""
+    import zlib
+    rng = np.random.default_rng(1)
+    nbytes = 32 << 20
+    src = rng.integers(0, 256, nbytes, dtype=np.uint8)
+    h = ctx.handle
+    announce("offload/prefetch round trip")
+    with Dev(ctx) as d:
+        a = d.up(src, np.uint8)
+        host = C.c_void_p()
+        check(lib.vdnn_host_alloc_pinned(h, C.byref(host), nbytes))
+        ev = C.c_void_p()
+        check(lib.vdnn_event_create(h, C.byref(ev), 0))
+        check(lib.vdnn_memcpy_d2h_async(h, host, a.ptr, nbytes, lib.vdnn_ctx_stream_d2h(h)))
+        check(lib.vdnn_event_record(h, ev, lib.vdnn_ctx_stream_d2h(h)))
+        check(lib.vdnn_stream_wait_event(h, lib.vdnn_ctx_stream_h2d(h), ev))
+        b = d.empty(nbytes, np.uint8)
+        check(lib.vdnn_memcpy_h2d_async(h, b.ptr, host, nbytes, lib.vdnn_ctx_stream_h2d(h)))
+        check(lib.vdnn_stream_synchronize(h, lib.vdnn_ctx_stream_h2d(h)))
+        staged = np.ctypeslib.as_array(C.cast(host, C.POINTER(C.c_uint8)), shape=(nbytes,)).copy()
+        back = b.download(nbytes, np.uint8)
+        check(lib.vdnn_event_destroy(h, ev))
+        check(lib.vdnn_host_free_pinned(h, host))
+    assert zlib.crc32(staged.tobytes()) == zlib.crc32(src.tobytes())
+    assert np.array_equal(back, src)

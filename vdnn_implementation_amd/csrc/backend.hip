@@ -1,0 +1,315 @@
+// Context, pooled device memory, streams, events and copies of the device back end.
+#include "backend_internal.h"
+
+#include <cstring>
+
+namespace vdnn {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+// Virtual base of a plan-only pool: never dereferenced, only used for offset arithmetic.
+static constexpr uintptr_t kPlanBase = uintptr_t(1) << 44;
+
+} // namespace vdnn
+
+using namespace vdnn;
+
+extern "C" {
+
+const char* vdnn_last_error(void) { return g_error; }
+
+int vdnn_ctx_create(vdnn_ctx** out, int device, int flags) {
+    if (!out) { set_error("vdnn_ctx_create: null out"); return VDNN_EINVAL; }
+    *out = nullptr;
+    vdnn_ctx* ctx = new vdnn_ctx();
+    ctx->device = device;
+    ctx->plan_only = (flags & VDNN_CTX_PLAN_ONLY) != 0;
+    if (!ctx->plan_only) {
+        hipError_t e = hipSetDevice(device);
+        if (e != hipSuccess) {
+            set_error("hipSetDevice(%d) failed: %s", device, hipGetErrorString(e));
+            delete ctx;
+            return VDNN_EDEVICE;
+        }
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->num_cu = prop.multiProcessorCount;
+        // default priority on every stream
+        if (hipStreamCreateWithFlags(&ctx->compute, hipStreamNonBlocking) != hipSuccess ||
+            hipStreamCreateWithFlags(&ctx->d2h, hipStreamNonBlocking) != hipSuccess ||
+            hipStreamCreateWithFlags(&ctx->h2d, hipStreamNonBlocking) != hipSuccess) {
+            set_error("hipStreamCreate failed");
+            delete ctx;
+            return VDNN_EDEVICE;
+        }
+    }
+    *out = ctx;
+    return VDNN_OK;
+}
+
+int vdnn_ctx_destroy(vdnn_ctx* ctx) {
+    if (!ctx) return VDNN_OK;
+    vdnn_pool_finalize(ctx);
+    if (!ctx->plan_only) {
+        (void)hipDeviceSynchronize();
+        if (ctx->compute) (void)hipStreamDestroy(ctx->compute);
+        if (ctx->d2h) (void)hipStreamDestroy(ctx->d2h);
+        if (ctx->h2d) (void)hipStreamDestroy(ctx->h2d);
+    }
+    delete ctx;
+    return VDNN_OK;
+}
+
+int vdnn_device_mem_info(vdnn_ctx* ctx, size_t* free_bytes, size_t* total_bytes) {
+    VDNN_REQUIRE(ctx && free_bytes && total_bytes, "null argument");
+    if (ctx->plan_only) {
+        *total_bytes = size_t(288) << 30; // MI355X HBM3E
+        *free_bytes = *total_bytes;
+        return VDNN_OK;
+    }
+    VDNN_HIP(hipMemGetInfo(free_bytes, total_bytes));
+    return VDNN_OK;
+}
+
+int vdnn_device_synchronize(vdnn_ctx* ctx) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only) return VDNN_OK;
+    VDNN_HIP(hipDeviceSynchronize());
+    return VDNN_OK;
+}
+
+vdnn_stream_t vdnn_ctx_stream_compute(vdnn_ctx* ctx) { return ctx ? ctx->compute : nullptr; }
+vdnn_stream_t vdnn_ctx_stream_d2h(vdnn_ctx* ctx) { return ctx ? ctx->d2h : nullptr; }
+vdnn_stream_t vdnn_ctx_stream_h2d(vdnn_ctx* ctx) { return ctx ? ctx->h2d : nullptr; }
+
+/* ---- pool ----------------------------------------------------------------------------------- */
+int vdnn_pool_init(vdnn_ctx* ctx, size_t bytes) {
+    VDNN_REQUIRE(ctx, "null context");
+    VDNN_REQUIRE(!ctx->pool.initialised(), "pool already initialised");
+    VDNN_REQUIRE(bytes > kReduceScratchBytes, "pool smaller than the reduction staging area");
+    if (ctx->plan_only) {
+        ctx->pool.init(kPlanBase, bytes);
+    } else {
+        hipError_t e = hipMalloc(&ctx->pool_base, bytes);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            set_error("vdnn_pool_init: hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+            ctx->pool_base = nullptr;
+            return VDNN_OOM;
+        }
+        ctx->pool.init((uintptr_t)ctx->pool_base, bytes);
+    }
+    uintptr_t s = ctx->pool.allocate(kReduceScratchBytes);
+    ctx->reduce_scratch = (float*)s;
+    ctx->reduce_scratch_bytes = kReduceScratchBytes;
+    return VDNN_OK;
+}
+
+int vdnn_pool_finalize(vdnn_ctx* ctx) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (!ctx->pool.initialised()) return VDNN_OK;
+    if (!ctx->plan_only && ctx->pool_base) {
+        (void)hipDeviceSynchronize();
+        (void)hipFree(ctx->pool_base);
+    }
+    ctx->pool_base = nullptr;
+    ctx->reduce_scratch = nullptr;
+    ctx->reduce_scratch_bytes = 0;
+    ctx->pool.clear();
+    return VDNN_OK;
+}
+
+int vdnn_pool_malloc(vdnn_ctx* ctx, void** ptr, size_t bytes) {
+    VDNN_REQUIRE(ctx && ptr, "null argument");
+    VDNN_REQUIRE(ctx->pool.initialised(), "pool not initialised");
+    uintptr_t p = ctx->pool.allocate(bytes);
+    if (!p) {
+        *ptr = nullptr;
+        set_error("vdnn_pool_malloc: out of memory for %zu bytes (in use %zu of %zu, cap %zu, largest free %zu)",
+                  bytes, ctx->pool.in_use(), ctx->pool.total(), ctx->pool.cap(), ctx->pool.largest_free());
+        return VDNN_OOM;
+    }
+    *ptr = (void*)p;
+    return VDNN_OK;
+}
+
+int vdnn_pool_free(vdnn_ctx* ctx, void* ptr) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (!ptr) return VDNN_OK;
+    VDNN_REQUIRE(ctx->pool.release((uintptr_t)ptr), "pointer is not a live pool block");
+    return VDNN_OK;
+}
+
+int vdnn_pool_info(vdnn_ctx* ctx, size_t* free_bytes, size_t* total_bytes) {
+    VDNN_REQUIRE(ctx && free_bytes && total_bytes, "null argument");
+    *total_bytes = ctx->pool.total();
+    *free_bytes = ctx->pool.total() - ctx->pool.in_use();
+    return VDNN_OK;
+}
+
+int vdnn_pool_peak(vdnn_ctx* ctx, size_t* peak_in_use, size_t* peak_extent) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (peak_in_use) *peak_in_use = ctx->pool.peak_in_use();
+    if (peak_extent) *peak_extent = ctx->pool.peak_extent();
+    return VDNN_OK;
+}
+
+int vdnn_pool_reset_peak(vdnn_ctx* ctx) {
+    VDNN_REQUIRE(ctx, "null context");
+    ctx->pool.reset_peak();
+    return VDNN_OK;
+}
+
+int vdnn_pool_set_cap(vdnn_ctx* ctx, size_t cap_bytes) {
+    VDNN_REQUIRE(ctx, "null context");
+    ctx->pool.set_cap(cap_bytes);
+    return VDNN_OK;
+}
+
+int vdnn_pool_live_blocks(vdnn_ctx* ctx, size_t* count) {
+    VDNN_REQUIRE(ctx && count, "null argument");
+    *count = ctx->pool.live_blocks();
+    return VDNN_OK;
+}
+
+/* ---- streams, events, copies ------------------------------------------------------------------ */
+int vdnn_stream_synchronize(vdnn_ctx* ctx, vdnn_stream_t stream) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only) return VDNN_OK;
+    VDNN_HIP(hipStreamSynchronize(stream_of(ctx, stream)));
+    return VDNN_OK;
+}
+
+int vdnn_event_create(vdnn_ctx* ctx, vdnn_event_t* out, int with_timing) {
+    VDNN_REQUIRE(ctx && out, "null argument");
+    *out = nullptr;
+    if (ctx->plan_only) return VDNN_OK;
+    hipEvent_t ev;
+    VDNN_HIP(hipEventCreateWithFlags(&ev, with_timing ? hipEventDefault : hipEventDisableTiming));
+    *out = ev;
+    return VDNN_OK;
+}
+
+int vdnn_event_destroy(vdnn_ctx* ctx, vdnn_event_t ev) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only || !ev) return VDNN_OK;
+    VDNN_HIP(hipEventDestroy((hipEvent_t)ev));
+    return VDNN_OK;
+}
+
+int vdnn_event_record(vdnn_ctx* ctx, vdnn_event_t ev, vdnn_stream_t stream) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only) return VDNN_OK;
+    VDNN_REQUIRE(ev, "null event");
+    VDNN_HIP(hipEventRecord((hipEvent_t)ev, stream_of(ctx, stream)));
+    return VDNN_OK;
+}
+
+int vdnn_stream_wait_event(vdnn_ctx* ctx, vdnn_stream_t stream, vdnn_event_t ev) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only) return VDNN_OK;
+    VDNN_REQUIRE(ev, "null event");
+    VDNN_HIP(hipStreamWaitEvent(stream_of(ctx, stream), (hipEvent_t)ev, 0));
+    return VDNN_OK;
+}
+
+int vdnn_event_synchronize(vdnn_ctx* ctx, vdnn_event_t ev) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only) return VDNN_OK;
+    VDNN_REQUIRE(ev, "null event");
+    VDNN_HIP(hipEventSynchronize((hipEvent_t)ev));
+    return VDNN_OK;
+}
+
+int vdnn_event_elapsed_ms(vdnn_ctx* ctx, vdnn_event_t start, vdnn_event_t stop, float* ms) {
+    VDNN_REQUIRE(ctx && ms, "null argument");
+    *ms = 0.0f;
+    if (ctx->plan_only) return VDNN_OK;
+    VDNN_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return VDNN_OK;
+}
+
+int vdnn_host_alloc_pinned(vdnn_ctx* ctx, void** ptr, size_t bytes) {
+    VDNN_REQUIRE(ctx && ptr, "null argument");
+    *ptr = nullptr;
+    if (ctx->plan_only) {
+        // a distinct non-null token per request; never dereferenced
+        static uintptr_t next = uintptr_t(1) << 45;
+        *ptr = (void*)next;
+        next += (bytes + 4095) / 4096 * 4096 + 4096;
+        return VDNN_OK;
+    }
+    hipError_t e = hipHostMalloc(ptr, bytes, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("hipHostMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+        *ptr = nullptr;
+        return VDNN_OOM;
+    }
+    return VDNN_OK;
+}
+
+int vdnn_host_free_pinned(vdnn_ctx* ctx, void* ptr) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only || !ptr) return VDNN_OK;
+    VDNN_HIP(hipHostFree(ptr));
+    return VDNN_OK;
+}
+
+int vdnn_memcpy_d2h_async(vdnn_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes, vdnn_stream_t stream) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only || bytes == 0) return VDNN_OK;
+    VDNN_REQUIRE(dst_host && src_dev, "null pointer");
+    VDNN_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, stream ? (hipStream_t)stream : ctx->d2h));
+    return VDNN_OK;
+}
+
+int vdnn_memcpy_h2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes, vdnn_stream_t stream) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only || bytes == 0) return VDNN_OK;
+    VDNN_REQUIRE(dst_dev && src_host, "null pointer");
+    VDNN_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, stream ? (hipStream_t)stream : ctx->h2d));
+    return VDNN_OK;
+}
+
+int vdnn_memcpy_d2h(vdnn_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only || bytes == 0) return VDNN_OK;
+    VDNN_REQUIRE(dst_host && src_dev, "null pointer");
+    VDNN_HIP(hipDeviceSynchronize());
+    VDNN_HIP(hipMemcpy(dst_host, src_dev, bytes, hipMemcpyDeviceToHost));
+    return VDNN_OK;
+}
+
+int vdnn_memcpy_h2d(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only || bytes == 0) return VDNN_OK;
+    VDNN_REQUIRE(dst_dev && src_host, "null pointer");
+    VDNN_HIP(hipDeviceSynchronize());
+    VDNN_HIP(hipMemcpy(dst_dev, src_host, bytes, hipMemcpyHostToDevice));
+    VDNN_HIP(hipDeviceSynchronize());
+    return VDNN_OK;
+}
+
+int vdnn_memcpy_d2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes, vdnn_stream_t stream) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only || bytes == 0) return VDNN_OK;
+    VDNN_REQUIRE(dst_dev && src_dev, "null pointer");
+    VDNN_HIP(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, stream_of(ctx, stream)));
+    return VDNN_OK;
+}
+
+int vdnn_out_dim(int in, int pad, int window, int stride) {
+    if (stride <= 0 || window <= 0) return 0;
+    const int t = in + 2 * pad - window;
+    if (t < 0) return 0;
+    return t / stride + 1;
+}
+
+} // extern "C"

@@ -1,0 +1,599 @@
+// Bandwidth-bound layers: ReLU, max-pool, LRN, softmax, bias add / bias gradient, the first-diff
+// subtraction, fills and the ordered reduction of split partial sums.
+// Replaces cudnnActivation*/cudnnPooling*/cudnnSoftmax*/cudnnAddTensor/cudnnConvolutionBackwardBias
+// (layer.cu:576-582, 631-637, 766-915) and the reference's two own kernels (layer.cu:33-38,
+// network.cu:3-8). All reductions have a fixed order: results do not depend on timing.
+#include "backend_internal.h"
+
+#include <cfloat>
+
+namespace vdnn {
+
+constexpr int EB = 256; // threads per workgroup
+
+static inline unsigned grid_for(size_t items, int per_block, int max_blocks) {
+    size_t b = (items + per_block - 1) / per_block;
+    if (b < 1) b = 1;
+    if (b > (size_t)max_blocks) b = max_blocks;
+    return (unsigned)b;
+}
+
+// ---- wavefront / workgroup reductions (fixed tree order) -----------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+// every thread returns the workgroup-wide result; EB == 256 -> 4 wavefronts
+__device__ __forceinline__ float block_sum(float v, float* sh) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) sh[wave] = v;
+    __syncthreads();
+    return (sh[0] + sh[1]) + (sh[2] + sh[3]);
+}
+__device__ __forceinline__ float block_max(float v, float* sh) {
+    v = wave_max(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) sh[wave] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+}
+
+// ---- ReLU ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float relu1(float v) { return v > 0.0f ? v : (v != v ? v : 0.0f); }
+
+__global__ void __launch_bounds__(EB) relu_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, size_t n4, size_t n) {
+    const size_t stride = (size_t)gridDim.x * EB;
+    const float4* x4 = (const float4*)x;
+    float4* y4 = (float4*)y;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < n4; i += stride) {
+        float4 v = x4[i];
+        v.x = relu1(v.x); v.y = relu1(v.y); v.z = relu1(v.z); v.w = relu1(v.w);
+        y4[i] = v;
+    }
+    for (size_t i = n4 * 4 + (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) y[i] = relu1(x[i]);
+}
+
+__global__ void __launch_bounds__(EB) relu_bwd_kernel(const float* __restrict__ t, const float* __restrict__ dy,
+                                                      float* __restrict__ dx, size_t n4, size_t n) {
+    const size_t stride = (size_t)gridDim.x * EB;
+    const float4* t4 = (const float4*)t;
+    const float4* d4 = (const float4*)dy;
+    float4* o4 = (float4*)dx;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < n4; i += stride) {
+        const float4 a = t4[i], d = d4[i];
+        float4 o;
+        o.x = a.x > 0.0f ? d.x : 0.0f; o.y = a.y > 0.0f ? d.y : 0.0f;
+        o.z = a.z > 0.0f ? d.z : 0.0f; o.w = a.w > 0.0f ? d.w : 0.0f;
+        o4[i] = o;
+    }
+    for (size_t i = n4 * 4 + (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) dx[i] = t[i] > 0.0f ? dy[i] : 0.0f;
+}
+
+// ---- elementwise helpers ------------------------------------------------------------------------
+__global__ void __launch_bounds__(EB) sub_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ r, size_t n) {
+    const size_t stride = (size_t)gridDim.x * EB;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) r[i] = a[i] - b[i];
+}
+__global__ void __launch_bounds__(EB) fill_kernel(float* __restrict__ p, float v, size_t n) {
+    const size_t stride = (size_t)gridDim.x * EB;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) p[i] = v;
+}
+// y[n,k,:] += bias[k]; one workgroup row per (n,k) plane chunk
+__global__ void __launch_bounds__(EB) bias_add_kernel(float* __restrict__ y, const float* __restrict__ bias, int K, int hw, size_t total) {
+    const size_t stride = (size_t)gridDim.x * EB;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
+        const int k = (int)((i / hw) % K);
+        y[i] += bias[k];
+    }
+}
+
+// out[i] = (accumulate ? out[i] : 0) + alpha * (p[0][i] + p[1][i] + ...) (+ bias[i % ncols]); split order fixed
+__global__ void __launch_bounds__(EB) reduce_splits_kernel(float* __restrict__ out, const float* __restrict__ partial, size_t count,
+                                                           int splits, float alpha, int accumulate, const float* __restrict__ bias_j, int ncols) {
+    const size_t stride = (size_t)gridDim.x * EB;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < count; i += stride) {
+        float s = partial[i];
+        for (int k = 1; k < splits; k++) s += partial[(size_t)k * count + i];
+        float r = alpha * s;
+        if (accumulate) r = out[i] + r;
+        if (bias_j) r += bias_j[i % ncols];
+        out[i] = r;
+    }
+}
+
+int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
+                         int splits, float alpha, int accumulate, const float* bias_j, int ncols) {
+    hipLaunchKernelGGL(reduce_splits_kernel, dim3(grid_for(count, EB, ctx->num_cu * 8)), dim3(EB), 0, stream,
+                       out, partial, count, splits, alpha, accumulate, bias_j, ncols);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+// ---- bias gradient of a convolution: bias[k] += alpha * sum_{n,pq} dy[n,k,pq] -------------------
+// stage 1: workgroup (k, split) sums samples [n0, n1) of channel k into partial[k*splits + split]
+__global__ void __launch_bounds__(EB) bias_grad_partial_kernel(const float* __restrict__ dy, float* __restrict__ partial,
+                                                               int N, int K, int PQ, int splits, int n_per_split) {
+    __shared__ float sh[4];
+    const int k = blockIdx.x / splits, sp = blockIdx.x % splits;
+    const int n0 = sp * n_per_split, n1 = min(N, n0 + n_per_split);
+    float acc = 0.0f;
+    for (int n = n0; n < n1; n++) {
+        const float* p = dy + ((size_t)n * K + k) * PQ;
+        for (int i = threadIdx.x; i < PQ; i += EB) acc += p[i];
+    }
+    acc = block_sum(acc, sh);
+    if (threadIdx.x == 0) partial[blockIdx.x] = acc;
+}
+// stage 2: one thread per channel adds its partials in split order
+__global__ void __launch_bounds__(EB) bias_grad_final_kernel(const float* __restrict__ partial, float* __restrict__ bias, int K, int splits, float alpha) {
+    const int k = blockIdx.x * EB + threadIdx.x;
+    if (k >= K) return;
+    float s = 0.0f;
+    for (int i = 0; i < splits; i++) s += partial[(size_t)k * splits + i];
+    bias[k] = bias[k] + alpha * s;
+}
+
+// bias[o] += alpha * sum_n dy[n,o]
+__global__ void __launch_bounds__(EB) fc_bias_grad_kernel(const float* __restrict__ dy, float* __restrict__ bias, int N, int Cout, float alpha) {
+    const int o = blockIdx.x * EB + threadIdx.x;
+    if (o >= Cout) return;
+    float s = 0.0f;
+    for (int n = 0; n < N; n++) s += dy[(size_t)n * Cout + o];
+    bias[o] = bias[o] + alpha * s;
+}
+
+// ---- max pooling --------------------------------------------------------------------------------
+struct PoolGeo { int N, C, H, W, R, S, P, Q, ph, pw, sh, sw; };
+
+__global__ void __launch_bounds__(EB) maxpool_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, PoolGeo g, size_t total) {
+    const size_t stride = (size_t)gridDim.x * EB;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
+        const int q = (int)(i % g.Q);
+        const size_t t = i / g.Q;
+        const int p = (int)(t % g.P);
+        const size_t nc = t / g.P;
+        const float* xp = x + nc * g.H * g.W;
+        float m = -FLT_MAX;
+        for (int r = 0; r < g.R; r++) {
+            const int ih = p * g.sh - g.ph + r;
+            if (ih < 0 || ih >= g.H) continue;
+            for (int s = 0; s < g.S; s++) {
+                const int iw = q * g.sw - g.pw + s;
+                if (iw < 0 || iw >= g.W) continue;
+                const float v = xp[(size_t)ih * g.W + iw];
+                if (v > m) m = v;
+            }
+        }
+        y[i] = m;
+    }
+}
+
+// 2x2 stride 2, no padding, even extents, W % 4 == 0: one thread makes two outputs from two float4 rows
+__global__ void __launch_bounds__(EB) maxpool2x2_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, int H, int W, size_t total_pairs) {
+    const int Q2 = W / 4, P = H / 2;
+    const size_t stride = (size_t)gridDim.x * EB;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total_pairs; i += stride) {
+        const int q2 = (int)(i % Q2);
+        const size_t t = i / Q2;
+        const int p = (int)(t % P);
+        const size_t nc = t / P;
+        const float* r0 = x + (nc * H + 2 * (size_t)p) * W + 4 * (size_t)q2;
+        const float4 a = *(const float4*)r0, b = *(const float4*)(r0 + W);
+        float m0 = -FLT_MAX, m1 = -FLT_MAX;
+        if (a.x > m0) m0 = a.x; if (a.y > m0) m0 = a.y; if (b.x > m0) m0 = b.x; if (b.y > m0) m0 = b.y;
+        if (a.z > m1) m1 = a.z; if (a.w > m1) m1 = a.w; if (b.z > m1) m1 = b.z; if (b.w > m1) m1 = b.w;
+        float2 o; o.x = m0; o.y = m1;
+        *(float2*)(y + (nc * P + p) * (size_t)(W / 2) + 2 * (size_t)q2) = o;
+    }
+}
+
+// argmax of window (p,q) with the forward's comparison: first strict maximum in row-major order;
+// the first valid position if nothing exceeds -FLT_MAX
+__device__ __forceinline__ int window_argmax(const float* __restrict__ xp, const PoolGeo& g, int p, int q) {
+    float m = -FLT_MAX;
+    int arg = -1;
+    for (int r = 0; r < g.R; r++) {
+        const int ih = p * g.sh - g.ph + r;
+        if (ih < 0 || ih >= g.H) continue;
+        for (int s = 0; s < g.S; s++) {
+            const int iw = q * g.sw - g.pw + s;
+            if (iw < 0 || iw >= g.W) continue;
+            const float v = xp[(size_t)ih * g.W + iw];
+            if (arg < 0) arg = ih * g.W + iw;
+            if (v > m) { m = v; arg = ih * g.W + iw; }
+        }
+    }
+    return arg;
+}
+
+// gather form: one thread per input element, windows visited in row-major order
+__global__ void __launch_bounds__(EB) maxpool_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ dx,
+                                                         PoolGeo g, size_t total) {
+    const size_t stride = (size_t)gridDim.x * EB;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
+        const int w = (int)(i % g.W);
+        const size_t t = i / g.W;
+        const int h = (int)(t % g.H);
+        const size_t nc = t / g.H;
+        const float* xp = x + nc * g.H * g.W;
+        const float* dyp = dy + nc * g.P * g.Q;
+        // windows containing (h,w): p*sh - ph <= h <= p*sh - ph + R - 1
+        int p_lo = h + g.ph - g.R + 1; p_lo = p_lo <= 0 ? 0 : (p_lo + g.sh - 1) / g.sh;
+        int p_hi = (h + g.ph) / g.sh; if (p_hi > g.P - 1) p_hi = g.P - 1;
+        int q_lo = w + g.pw - g.S + 1; q_lo = q_lo <= 0 ? 0 : (q_lo + g.sw - 1) / g.sw;
+        int q_hi = (w + g.pw) / g.sw; if (q_hi > g.Q - 1) q_hi = g.Q - 1;
+        const int self = h * g.W + w;
+        float acc = 0.0f;
+        for (int p = p_lo; p <= p_hi; p++)
+            for (int q = q_lo; q <= q_hi; q++)
+                if (window_argmax(xp, g, p, q) == self) acc += dyp[(size_t)p * g.Q + q];
+        dx[i] = acc;
+    }
+}
+
+// 2x2 stride 2 exact cover: one thread per pair of windows, writes all eight inputs
+__global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ dx,
+                                                            int H, int W, size_t total_pairs) {
+    const int Q2 = W / 4, P = H / 2;
+    const size_t stride = (size_t)gridDim.x * EB;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total_pairs; i += stride) {
+        const int q2 = (int)(i % Q2);
+        const size_t t = i / Q2;
+        const int p = (int)(t % P);
+        const size_t nc = t / P;
+        const size_t off = (nc * H + 2 * (size_t)p) * W + 4 * (size_t)q2;
+        const float4 a = *(const float4*)(x + off), b = *(const float4*)(x + off + W);
+        const float2 d = *(const float2*)(dy + (nc * P + p) * (size_t)(W / 2) + 2 * (size_t)q2);
+        // window 0: a.x a.y / b.x b.y ; window 1: a.z a.w / b.z b.w ; first strict maximum wins
+        int s0 = 0; float m0 = -FLT_MAX;
+        if (a.x > m0) { m0 = a.x; s0 = 0; } if (a.y > m0) { m0 = a.y; s0 = 1; }
+        if (b.x > m0) { m0 = b.x; s0 = 2; } if (b.y > m0) { m0 = b.y; s0 = 3; }
+        int s1 = 0; float m1 = -FLT_MAX;
+        if (a.z > m1) { m1 = a.z; s1 = 0; } if (a.w > m1) { m1 = a.w; s1 = 1; }
+        if (b.z > m1) { m1 = b.z; s1 = 2; } if (b.w > m1) { m1 = b.w; s1 = 3; }
+        float4 oa, ob;
+        oa.x = s0 == 0 ? d.x : 0.0f; oa.y = s0 == 1 ? d.x : 0.0f; ob.x = s0 == 2 ? d.x : 0.0f; ob.y = s0 == 3 ? d.x : 0.0f;
+        oa.z = s1 == 0 ? d.y : 0.0f; oa.w = s1 == 1 ? d.y : 0.0f; ob.z = s1 == 2 ? d.y : 0.0f; ob.w = s1 == 3 ? d.y : 0.0f;
+        *(float4*)(dx + off) = oa;
+        *(float4*)(dx + off + W) = ob;
+    }
+}
+
+// ---- LRN across channels: window 5, alpha 1e-4, beta 0.75, k 2 -------------------------------------
+#define LRN_A5 (1e-4f / 5.0f)
+#define LRN_BETA 0.75f
+#define LRN_KC 2.0f
+
+__global__ void __launch_bounds__(EB) lrn_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int hw, size_t total) {
+    const size_t stride = (size_t)gridDim.x * EB;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
+        const int c = (int)((i / hw) % C);
+        float ss = 0.0f;
+#pragma unroll
+        for (int d = -2; d <= 2; d++) {
+            const int cc = c + d;
+            if (cc < 0 || cc >= C) continue;
+            const float v = x[(long)i + (long)d * hw];
+            ss += v * v;
+        }
+        const float scale = LRN_KC + LRN_A5 * ss;
+        y[i] = x[i] * powf(scale, -LRN_BETA);
+    }
+}
+
+__global__ void __launch_bounds__(EB) lrn_bwd_kernel(const float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ dy,
+                                                     float* __restrict__ dx, int C, int hw, size_t total) {
+    const size_t stride = (size_t)gridDim.x * EB;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
+        const int c = (int)((i / hw) % C);
+        float xs[9]; // x^2 of channels c-4 .. c+4
+#pragma unroll
+        for (int d = -4; d <= 4; d++) {
+            const int cc = c + d;
+            float v = 0.0f;
+            if (cc >= 0 && cc < C) v = x[(long)i + (long)d * hw];
+            xs[d + 4] = v * v;
+        }
+        float t = 0.0f, scale_c = 1.0f;
+#pragma unroll
+        for (int d = -2; d <= 2; d++) {
+            const int cc = c + d;
+            // scale of channel cc: its own window, taken in ascending channel order
+            float ss = 0.0f;
+#pragma unroll
+            for (int e = -2; e <= 2; e++) ss += xs[d + e + 4];
+            const float scale = LRN_KC + LRN_A5 * ss;
+            if (d == 0) scale_c = scale;
+            if (cc < 0 || cc >= C) continue;
+            const long o = (long)i + (long)d * hw;
+            t += dy[o] * y[o] / scale;
+        }
+        dx[i] = dy[i] * powf(scale_c, -LRN_BETA) - (2.0f * 1e-4f * LRN_BETA / 5.0f) * x[i] * t;
+    }
+}
+
+// ---- softmax (one workgroup per sample) -------------------------------------------------------------
+__global__ void __launch_bounds__(EB) softmax_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, int classes) {
+    __shared__ float sh[4];
+    const float* xr = x + (size_t)blockIdx.x * classes;
+    float* yr = y + (size_t)blockIdx.x * classes;
+    float m = -FLT_MAX;
+    for (int j = threadIdx.x; j < classes; j += EB) m = fmaxf(m, xr[j]);
+    m = block_max(m, sh);
+    float s = 0.0f;
+    for (int j = threadIdx.x; j < classes; j += EB) {
+        const float e = expf(xr[j] - m);
+        yr[j] = e;
+        s += e;
+    }
+    s = block_sum(s, sh);
+    const float inv = 1.0f / s;
+    for (int j = threadIdx.x; j < classes; j += EB) yr[j] *= inv;
+}
+
+__global__ void __launch_bounds__(EB) softmax_bwd_kernel(const float* __restrict__ y, const float* __restrict__ dy, float* __restrict__ dx, int classes) {
+    __shared__ float sh[4];
+    const size_t base = (size_t)blockIdx.x * classes;
+    float dot = 0.0f;
+    for (int j = threadIdx.x; j < classes; j += EB) dot += dy[base + j] * y[base + j];
+    dot = block_sum(dot, sh);
+    for (int j = threadIdx.x; j < classes; j += EB) dx[base + j] = y[base + j] * (dy[base + j] - dot);
+}
+
+// per-sample -log p[label] into sample_loss[n]
+__global__ void __launch_bounds__(EB) nll_label_kernel(const float* __restrict__ prob, const int32_t* __restrict__ labels, float* __restrict__ sample_loss, int n, int classes) {
+    const int i = blockIdx.x * EB + threadIdx.x;
+    if (i >= n) return;
+    const int lab = labels[i];
+    float p = (lab >= 0 && lab < classes) ? prob[(size_t)i * classes + lab] : 1.0f;
+    sample_loss[i] = -logf(fmaxf(p, FLT_MIN));
+}
+// per-sample -sum_c target*log p
+__global__ void __launch_bounds__(EB) ce_dense_kernel(const float* __restrict__ prob, const float* __restrict__ target, float* __restrict__ sample_loss, int classes) {
+    __shared__ float sh[4];
+    const size_t base = (size_t)blockIdx.x * classes;
+    float s = 0.0f;
+    for (int j = threadIdx.x; j < classes; j += EB) {
+        const float t = target[base + j];
+        if (t != 0.0f) s -= t * logf(fmaxf(prob[base + j], FLT_MIN));
+    }
+    s = block_sum(s, sh);
+    if (threadIdx.x == 0) sample_loss[blockIdx.x] = s;
+}
+// loss[0] = mean of sample_loss, summed in sample order by one workgroup
+__global__ void __launch_bounds__(EB) mean_kernel(const float* __restrict__ v, float* __restrict__ out, int n) {
+    __shared__ float sh[4];
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < n; i += EB) s += v[i];
+    s = block_sum(s, sh);
+    if (threadIdx.x == 0) out[0] = s / (float)n;
+}
+__global__ void __launch_bounds__(EB) softmax_ce_bwd_kernel(const float* __restrict__ prob, const int32_t* __restrict__ labels, float* __restrict__ d, int classes, float inv_n, size_t total) {
+    const size_t stride = (size_t)gridDim.x * EB;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
+        const int n = (int)(i / classes), j = (int)(i % classes);
+        d[i] = (prob[i] - (labels[n] == j ? 1.0f : 0.0f)) * inv_n;
+    }
+}
+
+static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+} // namespace vdnn
+
+using namespace vdnn;
+
+extern "C" {
+
+int vdnn_relu_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(x && y, "null tensor");
+    if (count == 0) return VDNN_OK;
+    const size_t n4 = (aligned16(x) && aligned16(y)) ? count / 4 : 0;
+    hipLaunchKernelGGL(relu_fwd_kernel, dim3(grid_for(n4 ? n4 : count, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), x, y, n4, count);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_relu_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, const float* y, const float* dy, float* dx) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    const float* t = x ? x : y;
+    VDNN_REQUIRE(t && dy && dx, "null tensor");
+    if (count == 0) return VDNN_OK;
+    const size_t n4 = (aligned16(t) && aligned16(dy) && aligned16(dx)) ? count / 4 : 0;
+    hipLaunchKernelGGL(relu_bwd_kernel, dim3(grid_for(n4 ? n4 : count, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), t, dy, dx, n4, count);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_sub(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* a, const float* b, float* r) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(a && b && r, "null tensor");
+    if (count == 0) return VDNN_OK;
+    hipLaunchKernelGGL(sub_kernel, dim3(grid_for(count, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), a, b, r, count);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_fill(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float value, float* p) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(p, "null tensor");
+    if (count == 0) return VDNN_OK;
+    hipLaunchKernelGGL(fill_kernel, dim3(grid_for(count, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), p, value, count);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_bias_add(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw, const float* bias, float* y) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(bias && y && n > 0 && k > 0 && hw > 0, "bad argument");
+    const size_t total = (size_t)n * k * hw;
+    hipLaunchKernelGGL(bias_add_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), y, bias, k, hw, total);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* dy, float* bias, float alpha) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(shape && dy && bias, "null argument");
+    const int N = shape->n, K = shape->k;
+    const int P = vdnn_out_dim(shape->h, shape->pad_h, shape->r, shape->stride_h);
+    const int Q = vdnn_out_dim(shape->w, shape->pad_w, shape->s, shape->stride_w);
+    VDNN_REQUIRE(N > 0 && K > 0 && P > 0 && Q > 0, "bad geometry");
+    // split the batch so that K*splits workgroups fill the chip; geometry depends on the shape only
+    int splits = (4 * ctx->num_cu + K - 1) / K;
+    if (splits > N) splits = N;
+    if (splits < 1) splits = 1;
+    const int per = (N + splits - 1) / splits;
+    splits = (N + per - 1) / per;
+    VDNN_REQUIRE((size_t)K * splits * sizeof(float) <= ctx->reduce_scratch_bytes, "staging area too small");
+    hipStream_t st = stream_of(ctx, stream);
+    hipLaunchKernelGGL(bias_grad_partial_kernel, dim3(K * splits), dim3(EB), 0, st, dy, ctx->reduce_scratch, N, K, P * Q, splits, per);
+    VDNN_LAUNCH_CHECK();
+    hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB - 1) / EB), dim3(EB), 0, st, ctx->reduce_scratch, bias, K, splits, alpha);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_fc_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const float* dy, float* bias, float alpha) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(dy && bias && n > 0 && c_out > 0, "bad argument");
+    hipLaunchKernelGGL(fc_bias_grad_kernel, dim3((c_out + EB - 1) / EB), dim3(EB), 0, stream_of(ctx, stream), dy, bias, n, c_out, alpha);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+static bool pool_geo(const vdnn_shape_t* s, PoolGeo& g) {
+    g.N = s->n; g.C = s->c; g.H = s->h; g.W = s->w; g.R = s->r; g.S = s->s;
+    g.ph = s->pad_h; g.pw = s->pad_w; g.sh = s->stride_h; g.sw = s->stride_w;
+    if (g.N <= 0 || g.C <= 0 || g.H <= 0 || g.W <= 0 || g.R <= 0 || g.S <= 0 || g.sh <= 0 || g.sw <= 0 || g.ph < 0 || g.pw < 0) return false;
+    g.P = vdnn_out_dim(g.H, g.ph, g.R, g.sh);
+    g.Q = vdnn_out_dim(g.W, g.pw, g.S, g.sw);
+    return g.P > 0 && g.Q > 0 && (long)g.H * g.W < (1l << 31);
+}
+
+static bool pool_is_2x2_exact(const PoolGeo& g, const void* a, const void* b, const void* c) {
+    return g.R == 2 && g.S == 2 && g.sh == 2 && g.sw == 2 && g.ph == 0 && g.pw == 0 && g.H % 2 == 0 && g.W % 4 == 0 &&
+           aligned16(a) && aligned16(b) && (!c || aligned16(c));
+}
+
+int vdnn_maxpool_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* x, float* y) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    PoolGeo g;
+    VDNN_REQUIRE(shape && pool_geo(shape, g), "unsupported pooling geometry");
+    VDNN_REQUIRE(x && y, "null tensor");
+    hipStream_t st = stream_of(ctx, stream);
+    if (pool_is_2x2_exact(g, x, y, nullptr)) {
+        const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
+        hipLaunchKernelGGL(maxpool2x2_fwd_kernel, dim3(grid_for(pairs, EB, ctx->num_cu * 16)), dim3(EB), 0, st, x, y, g.H, g.W, pairs);
+    } else {
+        const size_t total = (size_t)g.N * g.C * g.P * g.Q;
+        hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, st, x, y, g, total);
+    }
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_maxpool_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape,
+                     const float* x, const float* y, const float* dy, float* dx) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    (void)y; // the winner of each window is recomputed from x with the forward's comparison
+    PoolGeo g;
+    VDNN_REQUIRE(shape && pool_geo(shape, g), "unsupported pooling geometry");
+    VDNN_REQUIRE(x && dy && dx, "null tensor");
+    hipStream_t st = stream_of(ctx, stream);
+    if (pool_is_2x2_exact(g, x, dx, dy) && (g.W / 2) % 2 == 0) {
+        const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
+        hipLaunchKernelGGL(maxpool2x2_bwd_kernel, dim3(grid_for(pairs, EB, ctx->num_cu * 16)), dim3(EB), 0, st, x, dy, dx, g.H, g.W, pairs);
+    } else {
+        const size_t total = (size_t)g.N * g.C * g.H * g.W;
+        hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, st, x, dy, dx, g, total);
+    }
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_lrn_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const float* x, float* y) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(x && y && n > 0 && c > 0 && hw > 0, "bad argument");
+    const size_t total = (size_t)n * c * hw;
+    hipLaunchKernelGGL(lrn_fwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), x, y, c, hw, total);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_lrn_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const float* x, const float* y, const float* dy, float* dx) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(x && y && dy && dx && n > 0 && c > 0 && hw > 0, "bad argument");
+    const size_t total = (size_t)n * c * hw;
+    hipLaunchKernelGGL(lrn_bwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), x, y, dy, dx, c, hw, total);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_softmax_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* x, float* y) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(x && y && n > 0 && classes > 0, "bad argument");
+    hipLaunchKernelGGL(softmax_fwd_kernel, dim3(n), dim3(EB), 0, stream_of(ctx, stream), x, y, classes);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_softmax_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* y, const float* dy, float* dx) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(y && dy && dx && n > 0 && classes > 0, "bad argument");
+    hipLaunchKernelGGL(softmax_bwd_kernel, dim3(n), dim3(EB), 0, stream_of(ctx, stream), y, dy, dx, classes);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_softmax_ce_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* logits,
+                        const int32_t* labels, float* prob, float* loss) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(logits && labels && prob && n > 0 && classes > 0, "bad argument");
+    hipStream_t st = stream_of(ctx, stream);
+    hipLaunchKernelGGL(softmax_fwd_kernel, dim3(n), dim3(EB), 0, st, logits, prob, classes);
+    VDNN_LAUNCH_CHECK();
+    if (loss) {
+        VDNN_REQUIRE((size_t)n * sizeof(float) <= ctx->reduce_scratch_bytes, "staging area too small");
+        hipLaunchKernelGGL(nll_label_kernel, dim3((n + EB - 1) / EB), dim3(EB), 0, st, prob, labels, ctx->reduce_scratch, n, classes);
+        VDNN_LAUNCH_CHECK();
+        hipLaunchKernelGGL(mean_kernel, dim3(1), dim3(EB), 0, st, ctx->reduce_scratch, loss, n);
+        VDNN_LAUNCH_CHECK();
+    }
+    return VDNN_OK;
+}
+
+int vdnn_softmax_ce_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* prob,
+                        const int32_t* labels, float* dlogits) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(prob && labels && dlogits && n > 0 && classes > 0, "bad argument");
+    const size_t total = (size_t)n * classes;
+    hipLaunchKernelGGL(softmax_ce_bwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream),
+                       prob, labels, dlogits, classes, 1.0f / (float)n, total);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_cross_entropy_dense(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes,
+                             const float* prob, const float* target, float* loss) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(prob && target && loss && n > 0 && classes > 0, "bad argument");
+    VDNN_REQUIRE((size_t)n * sizeof(float) <= ctx->reduce_scratch_bytes, "staging area too small");
+    hipStream_t st = stream_of(ctx, stream);
+    hipLaunchKernelGGL(ce_dense_kernel, dim3(n), dim3(EB), 0, st, prob, target, ctx->reduce_scratch, classes);
+    VDNN_LAUNCH_CHECK();
+    hipLaunchKernelGGL(mean_kernel, dim3(1), dim3(EB), 0, st, ctx->reduce_scratch, loss, n);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+} // extern "C"

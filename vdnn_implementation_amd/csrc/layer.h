@@ -1,0 +1,259 @@
+// One layer of a network: geometry, parameter and activation pointers, forward/backward, the
+// offload/prefetch copies. Mirrors the reference's class Layer (layer.h:130-342): same public
+// method names, argument order and return convention (0 ok, -1 out of memory when isDynamic).
+// Everything device-side is reached through the C ABI of include/vdnn_backend.h; the cuDNN/cuBLAS
+// descriptors of the reference have no counterpart (geometry is a plain vdnn_shape_t).
+#pragma once
+#include <cassert>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <string>
+#include <vector>
+
+#include "vdnn.h"
+#include "vdnn_backend.h"
+
+/* Macro related to kernel execution (layer.h:32) */
+#define CEIL(a, b) (((a) + (b) - 1) / (b))
+
+/* Error conventions of layer.h:60-128: assertion-style aborts outside dynamic mode */
+#define M_ASSERT(EXPR, MESSAGE)                                                        \
+    do {                                                                               \
+        if (!(EXPR)) {                                                                 \
+            fprintf(stderr, "Assertion failed: %s (%s:%d)\n", MESSAGE, __FILE__, __LINE__); \
+            abort();                                                                   \
+        }                                                                              \
+    } while (0)
+
+#define FatalError(s)                                                                  \
+    do {                                                                               \
+        fprintf(stderr, "%s\n%s:%d\nAborting...\n", std::string(s).c_str(), __FILE__, __LINE__); \
+        exit(EXIT_FAILURE);                                                            \
+    } while (0)
+
+/* checkCUDNN / checkCUBLAS / checkCudaErrors / checkCuda collapse into one check of the back end's
+ * status (layer.h:72-107) */
+#define checkVDNN(status)                                                              \
+    do {                                                                               \
+        int s_ = (status);                                                             \
+        if (s_ != VDNN_OK) {                                                           \
+            fprintf(stderr, "vDNN back end failure %d: %s\n", s_, vdnn_last_error());  \
+            FatalError("back end failure");                                            \
+        }                                                                              \
+    } while (0)
+
+/* layer.h:109-128: pool status -> 0 / -1 (out of memory) / -2; aborts outside dynamic mode */
+inline int ASSERT_EQ(int result, bool isDynamicMode = false) {
+    if (!isDynamicMode) {
+        if (result != VDNN_OK) {
+            fprintf(stderr, "\n[POOL FAILED with error %d: %s]\n", result, vdnn_last_error());
+            abort();
+        }
+        return 0;
+    }
+    if (result == VDNN_OOM) return -1;
+    if (result == VDNN_OK) return 0;
+    return -2;
+}
+
+/* The two handle types of the reference's constructors (cudnnHandle_t*, cublasHandle_t*) survive as
+ * two distinct thin types over the same back-end context. */
+struct vdnnConvHandle_t { vdnn_ctx* ctx; };
+struct vdnnGemmHandle_t { vdnn_ctx* ctx; };
+
+class Layer {
+public:
+    Layer(
+        vdnn_t            _vdnnMode,
+        vdnnAlgoMode_t    _vdnnAlgoMode,
+        Layer_t           _layerType,
+        vdnnConvHandle_t* _convHandle,
+        vdnn_stream_t*    _stream_compute,
+        vdnn_stream_t*    _stream_memory,
+        int _id,
+        int _n, int _c, int _h, int _w,
+        int _pad_h, int _pad_w, int _stride_h, int _stride_w,
+        int _k, int _r, int _s);
+    Layer(
+        vdnn_t            _vdnnMode,
+        vdnnAlgoMode_t    _vdnnAlgoMode,
+        Layer_t           _layerType,
+        vdnnGemmHandle_t* _gemmHandle,
+        vdnn_stream_t*    _stream_compute,
+        vdnn_stream_t*    _stream_memory,
+        int _id,
+        int _n, int _c, int _h, int _w,
+        int _pad_h, int _pad_w, int _stride_h, int _stride_w,
+        int _k, int _r, int _s);
+    ~Layer();
+    Layer(const Layer&) = delete;
+    Layer& operator=(const Layer&) = delete;
+
+    // Seed of the synthetic initialisation (the reference draws from std::random_device).
+    static void     setInitSeed(uint64_t seed) { initSeed = seed; }
+    static uint64_t getInitSeed() { return initSeed; }
+    // Per-layer shape dump on stdout like the reference's constructors (layer.cu:96-101, 474-484)
+    static void     setVerbose(bool v) { verbose = v; }
+
+    // Seeded initialisation of filter/bias: He-normal filters, zero biases
+    void    initializeConvolutionFilterAndBias();
+    void    initializeFullyConnectedFilterAndBias();
+
+    // Algorithm selection: memory-optimal (no workspace) or perf-optimal (workspace) kernel variants
+    void    findMemOptFwdAlgo();
+    void    findMemOptBwdFilterAlgo();
+    void    findMemOptBwdDataAlgo();
+    void    findPerfOptFwdAlgo();
+    void    findPerfOptBwdFilterAlgo();
+    void    findPerfOptBwdDataAlgo();
+    void    findDynamicAlgo();
+
+    // General fwd/bwd function
+    int     forward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workSpace, bool isDynamic);
+    int     backward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
+                     void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
+
+    // CONV layer
+    int     convolutionForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workSpace, bool isDynamic);
+    int     convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
+                                void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
+    // FC_GEMM layer
+    int     fullyConnectedForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workSpace, bool isDynamic);
+    int     fullyConnectedBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
+                                   void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
+    // Activation (RELU) layer
+    int     activationForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workSpace, bool isDynamic);
+    int     activationBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
+                               void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
+    // SOFTMAX layer
+    int     softmaxForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workSpace, bool isDynamic);
+    int     softmaxBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
+                            void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
+    // POOL layer
+    int     poolingForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workSpace, bool isDynamic);
+    int     poolingBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
+                            void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
+    // LRN layer (addition)
+    int     lrnForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workSpace, bool isDynamic);
+    int     lrnBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
+                        void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
+    // CONCATENATE layer (empty in the reference, layer.cu:917-923)
+    int     concatenateForward();
+    int     concatenateBackward();
+
+    // Offloading and prefetching functions
+    void    offloadSrcData(bool* _offloaded, DATATYPE** _offloadedSrcData_h);
+    void    prefetchPreviousSrcData(DATATYPE* _prefetchedSrcData_h, void* _srcDataToPrefetch, unsigned long _prefetch_bytes);
+
+    // Allocate device memory from the pool (the reference's names, layer.cu:989-1011)
+    int     cnmemMallocSrcData(bool isDynamic);
+    int     cnmemMallocDstData(bool isDynamic);
+    int     cnmemMallocDiffData(bool isDynamic);
+    int     cnmemMallocGradData(bool isDynamic);
+
+    // Copy pointers
+    void    copySrcData(void* _srcData)   { srcData = _srcData;   }
+    void    copyDstData(void* _dstData)   { dstData = _dstData;   }
+    void    copyDiffData(void* _diffData) { diffData = _diffData; }
+    void    copyGradData(void* _gradData) { gradData = _gradData; }
+
+    /* Set functions */
+    void    setVdnnMode(vdnn_t _vdnnMode) { vdnnMode = _vdnnMode; }
+    void    setAlgoMode(vdnnAlgoMode_t m);
+    // Event the offload copy waits for (srcData fully written) and the events this layer's copies
+    // signal; owned by the Network. Null events mean "no ordering needed" (plan-only contexts).
+    void    setSrcReadyEvent(vdnn_event_t e)     { srcReadyEvent = e; }
+    void    setOffloadDoneEvent(vdnn_event_t e)  { offloadDoneEvent = e; }
+    void    setPrefetchEvents(vdnn_event_t blockFree, vdnn_event_t hostReady, vdnn_event_t done) {
+        prefetchBlockFreeEvent = blockFree; prefetchHostReadyEvent = hostReady; prefetchDoneEvent = done;
+    }
+
+    /* Get functions */
+    Layer_t LayerType()              { return layerType; }
+    int     LayerId()                { return layerId; }
+    void*   SrcData()                { return srcData;  }
+    void*   DstData()                { return dstData;  }
+    void*   DiffData()               { return diffData; }
+    void*   GradData()               { return gradData; }
+    void*   FilterData()             { return filterData; }
+    void*   BiasData()               { return biasData; }
+    int     InputN()                 { return n_in;  }
+    int     InputC()                 { return c_in;  }
+    int     InputH()                 { return h_in;  }
+    int     InputW()                 { return w_in;  }
+    int     OutputN()                { return n_out; }
+    int     OutputC()                { return c_out; }
+    int     OutputH()                { return h_out; }
+    int     OutputW()                { return w_out; }
+    // element counts are size_t: the reference's int overflows from VGG16 batch 256 on (layer.h:240)
+    size_t  SrcDataSize()            { return (size_t)n_in * c_in * h_in * w_in;      }
+    size_t  DstDataSize()            { return (size_t)n_out * c_out * h_out * w_out;  }
+    size_t  FwdWorkSpaceSize()       { return fwdWorkSpaceSize;       }
+    size_t  BwdDataWorkSpaceSize()   { return bwdDataWorkSpaceSize;   }
+    size_t  BwdFilterWorkSpaceSize() { return bwdFilterWorkSpaceSize; }
+    size_t  FilterDataSize()         { return hasParams() ? (size_t)k * c_in * r * s : 0; }
+    size_t  BiasDataSize()           { return hasParams() ? (size_t)c_out : 0; }
+    bool    hasParams() const        { return layerType == FC_GEMM || layerType == CONV || layerType == FC_CONV; }
+    const vdnn_shape_t& Shape() const { return shape; }
+    vdnnAlgoMode_t AlgoMode() const  { return vdnnAlgoMode; }
+    int     RefCntFwd()              { return refCntFwd; }
+    int     RefCntBwd()              { return refCntBwd; }
+
+    /* Reference Count Management (unused by the three networks, kept for interface parity) */
+    void    decrementRefCntFwd()  { assert(refCntFwd > 0);  refCntFwd--; }
+    void    decrementRefCntBwd()  { assert(refCntBwd > 0);  refCntBwd--; }
+
+    /* For debugging */
+    void    printDstData();
+    void    printFilterData();
+
+private:
+    void    construct(vdnn_ctx* _ctx);
+    int     mallocWorkSpace(void* shared, size_t bytes, void** cur, bool isDynamic);
+    void    freeWorkSpace(void* shared, size_t bytes, void* cur, bool isDynamic);
+
+    static uint64_t initSeed;
+    static bool     verbose;
+
+    /* General layer info */
+    vdnn_t         vdnnMode;
+    vdnnAlgoMode_t vdnnAlgoMode;
+    Layer_t        layerType;
+    int            layerId;
+    vdnn_ctx*      ctx;
+
+    /* Input NCHW, filter, output NCHW */
+    int n_in, c_in, h_in, w_in;
+    int pad_h, pad_w, stride_h, stride_w, k, r, s;
+    int n_out, c_out, h_out, w_out;
+    vdnn_shape_t shape;
+
+    /* Workspace size */
+    size_t fwdWorkSpaceSize, bwdDataWorkSpaceSize, bwdFilterWorkSpaceSize;
+
+    /* Streams */
+    vdnn_stream_t* stream_compute;
+    vdnn_stream_t* stream_memory;
+
+    /* Pointers to memory (data) */
+    void* srcData;    // x
+    void* filterData; // w
+    void* biasData;   // bias
+    void* dstData;    // y
+    void* diffData;   // dy
+    void* gradData;   // dx
+
+    /* Ordering of the copies */
+    vdnn_event_t srcReadyEvent, offloadDoneEvent;
+    vdnn_event_t prefetchBlockFreeEvent, prefetchHostReadyEvent, prefetchDoneEvent;
+
+    /* Connection to other layers (GoogLeNet plumbing of the reference, unused) */
+    std::vector<int> producerLayerId, consumerLayerId;
+    int  refCntFwd, refCntBwd;
+    bool inPlaceOp, insideInceptionModule, headOfFork, tailOfFork;
+    int  forkId, concatenateChannelOffset;
+
+    vdnnConvHandle_t* convHandle;
+    vdnnGemmHandle_t* gemmHandle;
+};
