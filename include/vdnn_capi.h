@@ -1,0 +1,95 @@
+/* C ABI over the C++ host classes (Network, Layer): what a foreign-function binding of the
+ * reference's upper boundary needs. The reference exposes C++ classes only (network.h:15-95,
+ * layer.h:130-255, constructed by main at vdnn.cu:69); each entry point names the member it wraps.
+ * Status: 0 ok, -1 out of memory (dynamic mode), other failures abort like the reference's macros.
+ */
+#ifndef VDNN_AMD_CAPI_H_
+#define VDNN_AMD_CAPI_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct vdnn_network vdnn_network;
+
+typedef struct {
+    uint64_t seed;
+    size_t   pool_bytes;   /* 0: sized from the layer table */
+    size_t   cap_bytes;    /* 0: no artificial limit */
+    int      plan_only;    /* replay the allocation schedule without a device */
+    int      host_sync;    /* synchronise both streams after every layer (network.cu:1090-1091) */
+    int      capture;      /* keep host copies of every layer's dstData / gradData */
+    int      verbose;
+    int      device;
+} vdnn_network_options;
+
+typedef struct {
+    int type;              /* Layer_t */
+    int n, c, h, w;
+    int pad_h, pad_w, stride_h, stride_w;
+    int k, r, s;
+    int n_out, c_out, h_out, w_out; /* filled in by vdnn_network_layer_spec; ignored on input */
+} vdnn_layer_spec;
+
+typedef struct {
+    size_t peak_bytes_in_use, peak_extent, offload_bytes, prefetch_bytes, pinned_bytes, pool_bytes, weight_bytes;
+} vdnn_network_stats;
+
+void vdnn_network_default_options(vdnn_network_options* o);
+/* Network::Network (network.cu:10-92); cnn is a CNN_t, policy a vdnn_t, algo a vdnnAlgoMode_t */
+vdnn_network* vdnn_network_create(int cnn, int policy, int algo, int batch, const vdnn_network_options* o);
+/* a network from an explicit table (Network::setLayersCustomCNN is an empty stub, network.cu:815-817) */
+vdnn_network* vdnn_network_create_custom(const vdnn_layer_spec* layers, int num_layers, int policy, int algo,
+                                         const vdnn_network_options* o);
+void vdnn_network_destroy(vdnn_network* net);
+/* Network::forwardPropagation / backwardPropagation (network.cu:1056-1191) */
+int  vdnn_network_forward(vdnn_network* net, int is_dynamic);
+int  vdnn_network_backward(vdnn_network* net, int is_dynamic);
+void vdnn_network_synchronize(vdnn_network* net);
+float vdnn_network_loss(vdnn_network* net);
+int  vdnn_network_num_layers(vdnn_network* net);
+int  vdnn_network_batch(vdnn_network* net);
+int  vdnn_network_policy(vdnn_network* net);
+int  vdnn_network_algo(vdnn_network* net);
+int  vdnn_network_layer_spec(vdnn_network* net, int l, vdnn_layer_spec* out);
+/* Network::getInputSize / getOutputSize (network.h:56-57) */
+size_t vdnn_network_input_size(vdnn_network* net);
+size_t vdnn_network_output_size(vdnn_network* net);
+void vdnn_network_set_input(vdnn_network* net, const float* host);
+void vdnn_network_get_input(vdnn_network* net, float* host);
+void vdnn_network_set_labels(vdnn_network* net, const int32_t* labels);
+void vdnn_network_set_label_tensor(vdnn_network* net, const float* host);
+int  vdnn_network_set_layer_params(vdnn_network* net, int l, const float* filter, const float* bias);
+int  vdnn_network_get_layer_params(vdnn_network* net, int l, float* filter, float* bias);
+size_t vdnn_network_filter_count(vdnn_network* net, int l);
+size_t vdnn_network_bias_count(vdnn_network* net, int l);
+/* host copies taken during the last step when options.capture is set; returns the element count */
+size_t vdnn_network_captured_dst(vdnn_network* net, int l, float* host, size_t capacity);
+size_t vdnn_network_captured_grad(vdnn_network* net, int l, float* host, size_t capacity);
+void vdnn_network_stats_get(vdnn_network* net, vdnn_network_stats* out);
+void vdnn_network_reset_peak(vdnn_network* net);
+/* Network::isOffload[] after setVdnnType (network.cu:875-940) */
+int  vdnn_network_is_offloaded(vdnn_network* net, int l);
+/* (backward layer, prefetched layer) pairs of the last backward, Network::findPrefetchLayer
+ * (network.cu:1198-1208); returns the number of pairs */
+int  vdnn_network_prefetch_trace(vdnn_network* net, int* bwd_layer, int* prefetched_layer, int capacity);
+/* Network::findMaxDxDySize / findMaxWorkSpaceSize (network.cu:1010-1040), bytes */
+size_t vdnn_network_max_dxdy_bytes(vdnn_network* net);
+size_t vdnn_network_max_workspace_bytes(vdnn_network* net);
+/* the context of the network, for calling include/vdnn_backend.h directly (timing events) */
+struct vdnn_ctx* vdnn_network_context(vdnn_network* net);
+/* parseVdnnInputs (vdnn.cu:8-54): 0 on success, -1 for an unknown word */
+int vdnn_parse_cnn(const char* word, int* cnn);
+int vdnn_parse_policy(const char* word, int* policy);
+int vdnn_parse_algo(const char* word, int* algo);
+/* host-side seeded generator, so a binding can reproduce the synthetic tensors */
+void vdnn_seeded_fill_normal(float* p, size_t count, uint64_t seed, uint64_t stream, float mean, float stddev);
+void vdnn_seeded_fill_labels(int32_t* p, size_t count, uint64_t seed, uint64_t stream, int classes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

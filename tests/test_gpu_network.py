@@ -1,0 +1,189 @@
+"""GPU parity of whole training steps through the Network C ABI.
+
+ 1. a small network with every layer kind against a torch-autograd fixture;
+ 2. every memory policy, with events or with the reference's per-layer host syncs, gives
+    bit-identical loss, gradients and post-step filters to BASELINE;
+ 3. the reference's networks (reduced batch) against the CPU checker, layer by layer:
+    outputs to 1e-4 relative (max norm); gradients to 1e-4 relative in the L2 norm with at most
+    1e-4 of the elements off by more than 1e-3 of the tensor's maximum (a ReLU or max-pool
+    decision that flips on a last-bit difference changes single elements by O(1));
+ 4. an offloaded and prefetched tensor is byte-identical (the network input after a step).
+"""
+import numpy as np
+import pytest
+
+import oracle
+from gpu_util import announce
+from test_oracle_net import load_small_net, small_net_layers
+from util import assert_close, golden, rel_err
+from vdnn_implementation_amd import (ALEXNET, ALEXNET_LRN, BASELINE, OVERFEAT, VDNN_ALL, VDNN_CONV, VDNN_MEMORY_OPT_ALGO,
+                                     VDNN_NONE, VDNN_PERF_OPT_ALGO, VGG16_128, enums)
+from vdnn_implementation_amd.network import Network, layer_spec
+
+pytestmark = pytest.mark.gpu
+POLICIES = [BASELINE, VDNN_NONE, VDNN_CONV, VDNN_ALL]
+
+
+def small_specs(n=4):
+    return [layer_spec(enums.FC_CONV, n, 3, 20, 20, 1, 1, 8, 3), layer_spec(enums.RELU, n, 8, 20, 20),
+            layer_spec(enums.LRN, n, 8, 20, 20), layer_spec(enums.POOL, n, 8, 20, 20, 0, 2, 0, 2),
+            layer_spec(enums.FC_CONV, n, 8, 10, 10, 2, 1, 12, 5), layer_spec(enums.RELU, n, 12, 10, 10),
+            layer_spec(enums.POOL, n, 12, 10, 10, 0, 2, 0, 3), layer_spec(enums.FC_GEMM, n, 192, 1, 1, 0, 0, 20, 1),
+            layer_spec(enums.RELU, n, 20, 1, 1), layer_spec(enums.FC_GEMM, n, 20, 1, 1, 0, 0, 10, 1),
+            layer_spec(enums.SOFTMAX, n, 10, 1, 1)]
+
+
+@pytest.mark.parametrize("policy", POLICIES)
+def test_small_net_against_torch_autograd(policy):
+    f = golden("small_net")
+    announce("small net golden, policy", policy)
+    with Network(layers=small_specs(), policy=policy, capture=True) as net:
+        net.set_input(f["x"])
+        net.set_labels(f["labels"])
+        for l in (0, 4, 7, 9):
+            net.set_params(l, f["w%d" % l], f["b%d" % l])
+        assert net.forwardPropagation() == 0
+        assert abs(net.loss() - float(f["ce"])) <= 1e-4 * abs(float(f["ce"]))
+        assert net.backwardPropagation() == 0
+        for l in range(net.num_layers):
+            assert_close(net.captured_dst(l).reshape(f["dst%d" % l].shape), f["dst%d" % l], 1e-4, "dst %d" % l)
+        assert_close(net.captured_grad(0), f["dx"], 1e-4, "dx")
+        for l in range(1, net.num_layers):
+            want = f["ddst%d" % (l - 1)]
+            assert_close(net.captured_grad(l).reshape(want.shape), want, 1e-4, "grad %d" % l)
+        for l in (0, 4, 7, 9):
+            w, b = net.get_params(l)
+            dw = (w.astype(np.float64).reshape(f["w%d" % l].shape) - f["w%d" % l]) / -1e-5
+            assert_close(dw, f["dw%d" % l], 2e-2, "dw %d" % l)  # bounded by fp32 rounding of w + 1e-5*dw
+
+
+def run_steps(net, steps):
+    out = {"loss": [], "grads": [], "dsts": []}
+    for _ in range(steps):
+        assert net.forwardPropagation() == 0
+        out["loss"].append(np.float32(net.loss()))
+        assert net.backwardPropagation() == 0
+        out["grads"].append([net.captured_grad(l) for l in range(net.num_layers)])
+        out["dsts"].append([net.captured_dst(l) for l in range(net.num_layers)])
+    out["params"] = [net.get_params(l) for l in range(net.num_layers) if net.has_params(l)]
+    out["input"] = net.get_input()
+    return out
+
+
+def assert_bit_identical(a, b, what):
+    assert [x.tobytes() for x in a["loss"]] == [x.tobytes() for x in b["loss"]], what + ": loss"
+    for s, (ga, gb) in enumerate(zip(a["grads"], b["grads"])):
+        for l, (x, y) in enumerate(zip(ga, gb)):
+            assert np.array_equal(x.view(np.uint32), y.view(np.uint32)), "%s: step %d gradient of layer %d" % (what, s, l)
+    for s, (da, db) in enumerate(zip(a["dsts"], b["dsts"])):
+        for l, (x, y) in enumerate(zip(da, db)):
+            assert np.array_equal(x.view(np.uint32), y.view(np.uint32)), "%s: step %d output of layer %d" % (what, s, l)
+    for i, ((wa, ba), (wb, bb)) in enumerate(zip(a["params"], b["params"])):
+        assert np.array_equal(wa.view(np.uint32), wb.view(np.uint32)) and np.array_equal(ba.view(np.uint32), bb.view(np.uint32)), "%s: params %d" % (what, i)
+    assert np.array_equal(a["input"].view(np.uint32), b["input"].view(np.uint32)), what + ": input after the step"
+
+
+@pytest.mark.parametrize("cnn,batch,algo", [(None, 4, VDNN_MEMORY_OPT_ALGO), (ALEXNET_LRN, 4, VDNN_MEMORY_OPT_ALGO),
+                                            (OVERFEAT, 3, VDNN_MEMORY_OPT_ALGO), (VGG16_128, 2, VDNN_PERF_OPT_ALGO)])
+def test_policies_are_bit_identical_to_baseline(cnn, batch, algo):
+    def make(policy, host_sync=False):
+        if cnn is None:
+            return Network(layers=small_specs(batch), policy=policy, algo=algo, capture=True, seed=3, host_sync=host_sync)
+        return Network(cnn, policy, algo, batch, capture=True, seed=3, host_sync=host_sync)
+
+    announce("policies bit-identical", cnn, batch, "BASELINE")
+    with make(BASELINE) as net:
+        base = run_steps(net, 2)
+        x0 = None
+    assert all(np.isfinite(v) for v in base["loss"])
+    for policy in (VDNN_NONE, VDNN_CONV, VDNN_ALL):
+        for host_sync in (False, True):
+            announce("policies bit-identical", cnn, batch, "policy", policy, "host_sync", host_sync)
+            with make(policy, host_sync) as net:
+                got = run_steps(net, 2)
+            assert_bit_identical(got, base, "policy %d host_sync %s" % (policy, host_sync))
+
+
+def grad_close(got, want, what):
+    got = got.astype(np.float64).ravel()
+    want = want.astype(np.float64).ravel()
+    l2 = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    assert l2 <= 1e-4, "%s: relative L2 error %.3e" % (what, l2)
+    bad = np.count_nonzero(np.abs(got - want) > 1e-3 * np.max(np.abs(want)))
+    assert bad <= max(1, int(1e-4 * want.size)), "%s: %d of %d elements off" % (what, bad, want.size)
+
+
+@pytest.mark.parametrize("cnn,batch,policy,algo", [
+    (ALEXNET_LRN, 2, BASELINE, VDNN_MEMORY_OPT_ALGO),   # the CPU-runnable configuration, reduced batch
+    (ALEXNET, 2, VDNN_ALL, VDNN_MEMORY_OPT_ALGO),
+    (OVERFEAT, 2, VDNN_CONV, VDNN_MEMORY_OPT_ALGO),
+    (VGG16_128, 1, VDNN_ALL, VDNN_PERF_OPT_ALGO),
+])
+def test_reference_networks_against_the_checker(cnn, batch, policy, algo):
+    seed = 11
+    o = oracle.Net(cnn=cnn, batch=batch)
+    o.init_seeded(seed)
+    oracle.set_accumulate_double(True)
+    try:
+        announce("network vs checker", cnn, batch, policy, algo)
+        with Network(cnn, policy, algo, batch, capture=True, seed=seed) as net:
+            # the product's own seeded draw equals the checker's, bit for bit
+            assert np.array_equal(net.get_input().view(np.uint32), o.input().view(np.uint32))
+            for l in range(net.num_layers):
+                if net.has_params(l):
+                    w, b = net.get_params(l)
+                    assert np.array_equal(w.view(np.uint32), o.filter(l).view(np.uint32)) and np.array_equal(b, o.bias(l))
+            w_before = {l: o.filter(l).copy() for l in range(o.num_layers) if o.filter(l) is not None}
+            want_loss = o.forward()
+            assert net.forwardPropagation() == 0
+            assert abs(net.loss() - want_loss) <= 1e-4 * abs(want_loss)
+            o.backward()
+            assert net.backwardPropagation() == 0
+            for l in range(net.num_layers):
+                assert_close(net.captured_dst(l), o.dst(l), 1e-4, "dst of layer %d" % l)
+            for l in range(net.num_layers):
+                grad_close(net.captured_grad(l), o.grad(l), "grad of layer %d" % l)
+            for l, w0 in w_before.items():
+                w, b = net.get_params(l)
+                assert_close(w, o.filter(l), 1e-6, "filter of layer %d after the step" % l)
+                assert_close(b, o.bias(l), 1e-6, "bias of layer %d after the step" % l)
+                # the update itself: (w_new - w_old) / -lr, limited by fp32 rounding of w
+                dw_got = (w.astype(np.float64) - w0) / -1e-5
+                dw_want = (o.filter(l).astype(np.float64) - w0) / -1e-5
+                if np.max(np.abs(dw_want)) > 1.0:
+                    l2 = np.linalg.norm(dw_got - dw_want) / np.linalg.norm(dw_want)
+                    assert l2 <= 5e-2, "dW of layer %d: %.3e" % (l, l2)
+            # offloaded then prefetched: the input block went to the host and back
+            assert np.array_equal(net.get_input().view(np.uint32), o.input().view(np.uint32))
+            st = net.stats()
+            if policy in (VDNN_ALL, VDNN_CONV):
+                assert st["offload_bytes"] == st["prefetch_bytes"] > 0
+    finally:
+        oracle.set_accumulate_double(False)
+        o.close()
+
+
+def test_offload_moves_the_bytes_the_schedule_says():
+    announce("offload byte counts, VGG16 batch 2")
+    with Network(VGG16_128, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 2, seed=5) as net:
+        x0 = net.get_input()
+        assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
+        st = net.stats()
+        want = sum(int(np.prod(net.src_shape(l))) * 4 for l in range(net.num_layers - 1))
+        assert st["offload_bytes"] == st["prefetch_bytes"] == want == st["pinned_bytes"]
+        assert np.array_equal(net.get_input().view(np.uint32), x0.view(np.uint32))
+        assert net.prefetch_trace() == [(l, l - 1) for l in range(36, 0, -1)]
+
+
+def test_out_of_memory_under_a_cap_returns_minus_one_on_the_device():
+    announce("cap: VDNN_NONE cannot fit, VDNN_ALL can")
+    with Network(VGG16_128, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 4, seed=5) as net:
+        assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
+        need = net.stats()["peak_bytes_in_use"]
+        loss_all = net.loss()
+    cap = int(need * 1.03)
+    with Network(VGG16_128, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 4, seed=5, cap_bytes=cap) as net:
+        assert net.forwardPropagation(True) == 0 and net.backwardPropagation(True) == 0
+        assert np.float32(net.loss()).tobytes() == np.float32(loss_all).tobytes()
+    with Network(VGG16_128, VDNN_NONE, VDNN_MEMORY_OPT_ALGO, 4, seed=5, cap_bytes=cap) as net:
+        assert net.forwardPropagation(True) == -1

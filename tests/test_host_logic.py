@@ -1,0 +1,282 @@
+"""Host logic without a GPU: the C ABI library loads and exports every declared symbol, the pool
+allocator, the policy setup, the prefetch scheduler and the allocation schedule replayed on a
+plan-only context (no kernels run, nothing is computed), the seeded generator against the checker's.
+"""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+import oracle
+import vdnn_implementation_amd.backend as be
+from vdnn_implementation_amd import (ALEXNET, ALEXNET_LRN, BASELINE, OVERFEAT, VDNN_ALL, VDNN_CONV, VDNN_DYNAMIC_ALGO,
+                                     VDNN_MEMORY_OPT_ALGO, VDNN_NONE, VDNN_PERF_OPT_ALGO, VGG16_64, VGG16_128, VGG16_256)
+from vdnn_implementation_amd import enums
+from vdnn_implementation_amd.backend import check, lib
+from vdnn_implementation_amd.network import CAPI_SYMBOLS, Network, layer_spec, parse
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GB = 1e9
+
+
+def declared_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return set(re.findall(r"\b(vdnn_[a-z0-9_]+)\s*\(", text))
+
+
+def test_library_exports_every_declared_symbol():
+    for header, table in (("vdnn_backend.h", be.BACKEND_SYMBOLS), ("vdnn_capi.h", CAPI_SYMBOLS)):
+        names = declared_functions(header)
+        assert names, header
+        for n in names:
+            assert hasattr(lib, n), "%s declares %s but the library does not export it" % (header, n)
+        assert names == set(table), (names ^ set(table))
+
+
+def test_enum_values_match_the_reference_header():
+    # vdnn.h:23-61
+    assert (BASELINE, VDNN_NONE, VDNN_ALL, VDNN_CONV) == (0, 1, 2, 3)
+    assert (VDNN_MEMORY_OPT_ALGO, VDNN_PERF_OPT_ALGO, VDNN_DYNAMIC_ALGO) == (0, 1, 2)
+    assert (enums.FC_GEMM, enums.CONV, enums.FC_CONV, enums.RELU, enums.SOFTMAX, enums.POOL) == (0, 1, 2, 3, 6, 7)
+    assert (ALEXNET, OVERFEAT, VGG16_64, VGG16_128, VGG16_256) == (0, 1, 3, 4, 5)
+    text = open(os.path.join(ROOT, "include", "vdnn.h")).read()
+    for name, val in (("VDNN_CONV", 3), ("VDNN_DYNAMIC_ALGO", 2), ("POOL", 7), ("VGG16_256", 5), ("LRN", 10)):
+        assert re.search(r"\b%s\s*=\s*%d\b" % (name, val), text)
+
+
+def test_command_line_words():
+    assert parse("VGG16_128", "VDNN_ALL", "VDNN_MEMORY_OPT_ALGO") == (VGG16_128, VDNN_ALL, VDNN_MEMORY_OPT_ALGO)
+    assert parse("ALEXNET", "VDNN_NONE", "VDNN_PERF_OPT_ALGO") == (ALEXNET, VDNN_NONE, VDNN_PERF_OPT_ALGO)
+    assert parse("OVERFEAT", "BASELINE", "VDNN_DYNAMIC_ALGO") == (OVERFEAT, BASELINE, VDNN_DYNAMIC_ALGO)
+    with pytest.raises(ValueError):
+        parse("RESNET", "BASELINE", "VDNN_MEMORY_OPT_ALGO")
+    exe = os.path.join(ROOT, "vdnn_implementation_amd", "bin", "vdnn")
+    out = subprocess.run([exe, "VGG16_64", "VDNN_CONV", "VDNN_MEMORY_OPT_ALGO", "--plan"], capture_output=True, text=True)
+    assert out.returncode == 0 and "CNN Model Type: VGG16_64" in out.stdout and '"batch": 64' in out.stdout
+    bad = subprocess.run([exe, "VGG16_64", "VDNN_SOME", "VDNN_MEMORY_OPT_ALGO", "--plan"], capture_output=True, text=True)
+    assert bad.returncode != 0 and "VDNN type must be one of" in bad.stderr
+
+
+# ---- pool allocator ---------------------------------------------------------------------------------
+def test_pool_best_fit_coalescing_peak_and_cap():
+    ctx = be.Context(plan_only=True, pool_bytes=256 << 20)
+    base_free, total = ctx.pool_info()
+    assert total == 256 << 20 and total - base_free == 64 << 20  # the staging area is taken at init
+    a, b, c = ctx.alloc(1 << 20), ctx.alloc(3 << 20), ctx.alloc(1 << 20)
+    assert ctx.pool_info()[0] == base_free - (5 << 20)
+    assert a.ptr % 512 == 0 and b.ptr == a.ptr + (1 << 20) and c.ptr == b.ptr + (3 << 20)
+    pb = b.ptr
+    b.free()
+    d = ctx.alloc(2 << 20)          # best fit: the 3 MiB hole, not the tail
+    assert d.ptr == pb
+    e = ctx.alloc(1 << 20)          # the remaining 1 MiB of the hole
+    assert e.ptr == pb + (2 << 20)
+    peak, extent = ctx.pool_peak()
+    assert peak == (64 << 20) + (5 << 20)
+    for x in (a, c, d, e):
+        x.free()
+    assert ctx.pool_info()[0] == base_free and ctx.live_blocks() == 1
+    big = ctx.alloc(base_free)      # fully coalesced again
+    big.free()
+    with pytest.raises(be.OutOfMemory):
+        ctx.alloc(base_free + 512)
+    check(lib.vdnn_pool_set_cap(ctx.handle, (64 << 20) + (10 << 20)))
+    x = ctx.alloc(8 << 20)
+    with pytest.raises(be.OutOfMemory):
+        ctx.alloc(4 << 20)
+    x.free()
+    assert lib.vdnn_pool_free(ctx.handle, C.c_void_p(12345)) == be.VDNN_EINVAL  # not a live block
+    tiny = ctx.alloc(1)
+    assert ctx.pool_info()[0] == base_free - 512  # 512-byte granularity
+    tiny.free()
+    ctx.close()
+
+
+def test_pool_fragmentation_is_visible_in_the_extent():
+    ctx = be.Context(plan_only=True, pool_bytes=128 << 20)
+    blocks = [ctx.alloc(1 << 20) for _ in range(8)]
+    for b in blocks[::2]:
+        b.free()
+    with_holes = ctx.alloc(2 << 20)  # no 2 MiB hole: goes to the tail
+    assert with_holes.ptr > blocks[-1].ptr
+    in_use, extent = ctx.pool_peak()
+    assert extent >= in_use
+    ctx.close()
+
+
+# ---- policy setup (network.cu:875-940) and prefetch scheduler (network.cu:1198-1208) -----------------
+def plan(cnn, policy, algo=VDNN_MEMORY_OPT_ALGO, batch=0, **kw):
+    return Network(cnn, policy, algo, batch, plan_only=True, **kw)
+
+
+def conv_layers(net):
+    return [l for l, s in enumerate(net.specs) if s.type in (enums.FC_CONV, enums.CONV)]
+
+
+@pytest.mark.parametrize("cnn,layers", [(ALEXNET, 19), (ALEXNET_LRN, 21), (OVERFEAT, 19), (VGG16_128, 37)])
+def test_offload_sets(cnn, layers):
+    for policy in (BASELINE, VDNN_NONE):
+        with plan(cnn, policy, batch=2) as net:
+            assert net.num_layers == layers
+            assert not any(net.is_offloaded(l) for l in range(layers))
+    with plan(cnn, VDNN_ALL, batch=2) as net:
+        assert [net.is_offloaded(l) for l in range(layers)] == [True] * (layers - 1) + [False]
+        pinned = sum(int(np.prod(net.src_shape(l))) * 4 for l in range(layers - 1))
+        assert net.stats()["pinned_bytes"] == pinned
+    with plan(cnn, VDNN_CONV, batch=2) as net:
+        assert [l for l in range(layers) if net.is_offloaded(l)] == conv_layers(net)
+
+
+def step(net):
+    assert net.forwardPropagation() == 0
+    assert net.backwardPropagation() == 0
+
+
+def test_prefetch_sequences():
+    # derived by replaying network.cu:1198-1208 on the reference's tables
+    with plan(VGG16_128, VDNN_ALL, batch=1) as net:
+        step(net)
+        assert net.prefetch_trace() == [(l, l - 1) for l in range(36, 0, -1)]
+    with plan(VGG16_128, VDNN_CONV, batch=1) as net:
+        step(net)
+        assert net.prefetch_trace() == [(36, 28), (28, 26), (26, 24), (24, 21), (21, 19), (19, 17), (17, 14), (14, 12),
+                                        (12, 10), (10, 7), (7, 5), (5, 2), (2, 0)]
+    with plan(ALEXNET, VDNN_CONV, batch=1) as net:
+        step(net)
+        assert net.prefetch_trace() == [(18, 10), (10, 8), (8, 6), (6, 3), (3, 0)]
+    with plan(OVERFEAT, VDNN_CONV, batch=1) as net:
+        step(net)
+        assert net.prefetch_trace() == [(18, 17), (17, 15), (15, 13), (13, 10), (10, 8), (8, 6), (6, 3), (3, 0)]
+    for cnn in (ALEXNET, OVERFEAT, ALEXNET_LRN):
+        with plan(cnn, VDNN_ALL, batch=1) as net:
+            step(net)
+            L = net.num_layers
+            assert net.prefetch_trace() == [(l, l - 1) for l in range(L - 1, 0, -1)]
+    with plan(VGG16_128, VDNN_NONE, batch=1) as net:
+        step(net)
+        assert net.prefetch_trace() == []
+
+
+STAGING = 64 << 20  # reduction staging area, taken from the pool at start
+
+
+def test_peak_memory_of_the_literal_schedule_vgg16_128():
+    """Replay of the reference's allocation schedule, 4-byte elements, no convolution workspace:
+    BASELINE 18.58 GB, VDNN_NONE 15.38, VDNN_CONV 11.11, VDNN_ALL 8.85 (weights 0.553 GB included).
+    The figures below add the 64 MiB staging area and 512-byte rounding; VDNN_ALL is 77 MB lower
+    because the input block is released after its offload instead of being leaked."""
+    want = {BASELINE: 18.58, VDNN_NONE: 15.38, VDNN_CONV: 11.11, VDNN_ALL: 8.85}
+    got = {}
+    for policy in want:
+        with plan(VGG16_128, policy) as net:
+            assert net.batch == 128
+            step(net)
+            got[policy] = net.stats()
+            peak = (got[policy]["peak_bytes_in_use"] - STAGING) / GB
+            assert abs(peak - want[policy]) < 0.09, (policy, peak)
+            step(net)  # a second step must not grow the pool: nothing leaks
+            assert net.stats()["peak_bytes_in_use"] == got[policy]["peak_bytes_in_use"]
+    assert got[VDNN_ALL]["offload_bytes"] == got[VDNN_ALL]["prefetch_bytes"] == 14741667840
+    assert abs(got[VDNN_CONV]["offload_bytes"] / GB - 4.65) < 0.01
+    assert got[VDNN_CONV]["offload_bytes"] == got[VDNN_CONV]["prefetch_bytes"]
+    assert got[BASELINE]["peak_bytes_in_use"] / got[VDNN_ALL]["peak_bytes_in_use"] > 2.09
+    assert abs(got[BASELINE]["weight_bytes"] / GB - 0.553) < 0.001
+
+
+def test_peak_memory_other_configs():
+    for cnn, batch, base, allp in ((VGG16_64, 0, 9.57, 4.70), (OVERFEAT, 128, 1.90, 1.37), (ALEXNET, 32, 0.53, 0.44)):
+        with plan(cnn, BASELINE, batch=batch) as net:
+            step(net)
+            assert abs((net.stats()["peak_bytes_in_use"] - STAGING) / GB - base) < 0.03
+        with plan(cnn, VDNN_ALL, batch=batch) as net:
+            step(net)
+            # lower than the literal replay by one input block (released after its offload, not leaked)
+            input_gb = net.getInputSize() * 4 / GB
+            assert abs((net.stats()["peak_bytes_in_use"] - STAGING) / GB - (allp - input_gb)) < 0.012
+
+
+def test_byte_counts_do_not_overflow_at_batch_256():
+    # the reference's int byte math overflows here (network.cu:1010-1023, layer.h:240)
+    with plan(VGG16_256, BASELINE) as net:
+        assert net.batch == 256
+        assert net.findMaxDxDySize() == 256 * 64 * 224 * 224 * 4 > 2 ** 31
+        step(net)
+
+
+def test_blocks_are_all_returned():
+    for policy in (VDNN_NONE, VDNN_CONV, VDNN_ALL):
+        with plan(ALEXNET_LRN, policy, batch=4) as net:
+            ctxh = net.context
+            n0 = C.c_size_t()
+            lib.vdnn_pool_live_blocks(ctxh, C.byref(n0))
+            for _ in range(3):
+                step(net)
+            n1 = C.c_size_t()
+            lib.vdnn_pool_live_blocks(ctxh, C.byref(n1))
+            assert n1.value == n0.value
+
+
+def test_cap_makes_baseline_fail_cleanly_where_vdnn_all_fits():
+    """The out-of-memory path of layer.h:110-128: in dynamic mode a failed pool request travels up as
+    -1 through Layer::forward and forwardPropagation."""
+    with plan(VGG16_64, VDNN_ALL) as net:
+        step(net)
+        need_all = net.stats()["peak_bytes_in_use"]
+    cap = int(need_all * 1.05)
+    with plan(VGG16_64, VDNN_ALL, cap_bytes=cap) as net:
+        assert net.forwardPropagation(True) == 0 and net.backwardPropagation(True) == 0
+    with plan(VGG16_64, VDNN_NONE, cap_bytes=cap) as net:
+        assert net.forwardPropagation(True) == -1
+
+
+def test_dynamic_algo_ladder():
+    # network.cu:946-1008: with room to spare the first rung that fits is (VDNN_NONE, PERF_OPT)
+    with plan(ALEXNET, BASELINE, VDNN_DYNAMIC_ALGO, batch=8) as net:
+        assert (net.policy, net.algo) == (VDNN_NONE, VDNN_PERF_OPT_ALGO)
+    with plan(VGG16_64, VDNN_ALL) as net:
+        step(net)
+        need_all = net.stats()["peak_bytes_in_use"]
+    with plan(VGG16_64, VDNN_CONV) as net:
+        step(net)
+        need_conv = net.stats()["peak_bytes_in_use"]
+    # room for VDNN_CONV but not VDNN_NONE
+    with plan(VGG16_64, BASELINE, VDNN_DYNAMIC_ALGO, cap_bytes=int(need_conv * 1.02)) as net:
+        assert (net.policy, net.algo) == (VDNN_CONV, VDNN_PERF_OPT_ALGO)
+    with plan(VGG16_64, BASELINE, VDNN_DYNAMIC_ALGO, cap_bytes=int(need_all * 1.02)) as net:
+        assert net.policy == VDNN_ALL
+
+
+def test_custom_table_shape_inference_and_sanity():
+    layers = [layer_spec(enums.FC_CONV, 2, 3, 20, 20, 1, 1, 8, 3), layer_spec(enums.RELU, 2, 8, 20, 20),
+              layer_spec(enums.POOL, 2, 8, 20, 20, 0, 2, 0, 2), layer_spec(enums.FC_GEMM, 2, 800, 1, 1, 0, 0, 10, 1),
+              layer_spec(enums.SOFTMAX, 2, 10, 1, 1)]
+    with Network(layers=layers, policy=VDNN_ALL, plan_only=True) as net:
+        assert net.dst_shape(0) == (2, 8, 20, 20) and net.dst_shape(2) == (2, 8, 10, 10) and net.dst_shape(3) == (2, 10, 1, 1)
+        step(net)
+        assert net.prefetch_trace() == [(4, 3), (3, 2), (2, 1), (1, 0)]
+
+
+# ---- seeded generator: the host code's draw equals the checker's, bit for bit ------------------------
+def test_seeded_generator_matches_the_checker():
+    for seed, stream, std in ((1, 1, 1.0), (77, 100, 0.0589), (2 ** 40 + 3, 136, 0.0147)):
+        a = np.empty(50000, np.float32)
+        lib.vdnn_seeded_fill_normal(a.ctypes.data_as(C.POINTER(C.c_float)), a.size, seed, stream, 0.0, std)
+        assert np.array_equal(a.view(np.uint32), oracle.fill_normal(a.size, seed, stream, 0.0, std).view(np.uint32))
+    lab = np.empty(1000, np.int32)
+    lib.vdnn_seeded_fill_labels(lab.ctypes.data_as(C.POINTER(C.c_int32)), lab.size, 9, 2, 1000)
+    assert np.array_equal(lab, oracle.fill_labels(1000, 9, 2, 1000))
+
+
+def test_tables_agree_with_the_checker():
+    for cnn in (ALEXNET, ALEXNET_LRN, OVERFEAT, VGG16_128):
+        o = oracle.Net(cnn=cnn, batch=2)
+        with plan(cnn, BASELINE, batch=2) as net:
+            assert net.num_layers == o.num_layers
+            for l in range(net.num_layers):
+                assert net.specs[l].type == o.desc[l].type
+                assert net.src_shape(l) == o.src_shape(l) and net.dst_shape(l) == o.dst_shape(l)
+        o.close()

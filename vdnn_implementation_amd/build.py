@@ -42,9 +42,11 @@ def _compile(src, force):
     obj = os.path.join(OBJ, src + ".o")
     if not force and not _deps_newer(obj, [path]):
         return obj
-    cmd = [HIPCC] + COMMON + (DEVICE_FLAGS if src.endswith(".hip") else ["-x", "c++"]) + ["-c", path, "-o", obj]
-    if not src.endswith(".hip"):
-        cmd = [HIPCC] + COMMON + ["-c", path, "-o", obj]
+    if src.endswith(".hip"):
+        cmd = [HIPCC] + COMMON + DEVICE_FLAGS + ["-c", path, "-o", obj]
+    else:
+        # host code: no contraction, so the seeded generator rounds the same way everywhere
+        cmd = [HIPCC] + COMMON + ["-ffp-contract=off", "-c", path, "-o", obj]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
@@ -65,7 +67,7 @@ def build(force=False, verbose=True):
         subprocess.check_call(cmd)
     cli = os.path.join(CSRC, CLI_SOURCE)
     if os.path.exists(cli) and (force or _deps_newer(BIN, [cli, LIB])):
-        cmd = [HIPCC] + COMMON + [cli, "-o", BIN, "-L" + PKG, "-lvdnn_amd", "-Wl,-rpath,$ORIGIN/.."]
+        cmd = [HIPCC] + COMMON + ["-ffp-contract=off", cli, "-o", BIN, "-L" + PKG, "-lvdnn_amd", "-Wl,-rpath,$ORIGIN/.."]
         subprocess.check_call(cmd)
     if verbose:
         print("built", LIB)

@@ -95,6 +95,8 @@ public:
     static uint64_t getInitSeed() { return initSeed; }
     // Per-layer shape dump on stdout like the reference's constructors (layer.cu:96-101, 474-484)
     static void     setVerbose(bool v) { verbose = v; }
+    // Plan-only networks allocate the parameter blocks but skip drawing and uploading their values
+    static void     setSkipParameterValues(bool v) { skipParameterValues = v; }
 
     // Seeded initialisation of filter/bias: He-normal filters, zero biases
     void    initializeConvolutionFilterAndBias();
@@ -197,6 +199,8 @@ public:
     bool    hasParams() const        { return layerType == FC_GEMM || layerType == CONV || layerType == FC_CONV; }
     const vdnn_shape_t& Shape() const { return shape; }
     vdnnAlgoMode_t AlgoMode() const  { return vdnnAlgoMode; }
+    vdnnConvHandle_t* ConvHandle()   { return convHandle; }
+    vdnnGemmHandle_t* GemmHandle()   { return gemmHandle; }
     int     RefCntFwd()              { return refCntFwd; }
     int     RefCntBwd()              { return refCntBwd; }
 
@@ -215,6 +219,7 @@ private:
 
     static uint64_t initSeed;
     static bool     verbose;
+    static bool     skipParameterValues;
 
     /* General layer info */
     vdnn_t         vdnnMode;

@@ -1,0 +1,669 @@
+// Network: tables, policy setup, forward/backward drivers, prefetch scheduler.
+// Control flow follows the reference's network.cu (cited per function). Differences that change no
+// value: copies are ordered against compute with events instead of two host-side stream syncs per
+// layer (options.hostSync restores those), byte counts are size_t, the input block is released after
+// its offload like every other offloaded tensor (the reference leaks one input-sized block per
+// step, network.cu:1156/1185), and everything is torn down in the destructor.
+#include "network.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "seeded_init.h"
+
+namespace {
+
+bool is_conv(Layer_t t) { return t == FC_CONV || t == CONV; }
+
+struct TableBuilder {
+    std::vector<LayerSpec>& t;
+    int n;
+    void conv(int c, int hw, int pad, int stride, int k, int r, bool forceMemOpt = false) {
+        t.push_back(LayerSpec{FC_CONV, n, c, hw, hw, pad, pad, stride, stride, k, r, r, forceMemOpt});
+    }
+    void relu(int c, int hw) { t.push_back(LayerSpec{RELU, n, c, hw, hw, 0, 0, 0, 0, 0, 0, 0, false}); }
+    void lrn(int c, int hw) { t.push_back(LayerSpec{LRN, n, c, hw, hw, 0, 0, 0, 0, 0, 0, 0, false}); }
+    void pool(int c, int hw, int win) { t.push_back(LayerSpec{POOL, n, c, hw, hw, 0, 0, 2, 2, 0, win, win, false}); }
+    void fc(int cin, int cout) { t.push_back(LayerSpec{FC_GEMM, n, cin, 1, 1, 0, 0, 0, 0, cout, 1, 1, false}); }
+    void softmax(int c) { t.push_back(LayerSpec{SOFTMAX, n, c, 1, 1, 0, 0, 0, 0, 0, 0, 0, false}); }
+};
+
+/* network.cu:156-323 (19 layers); withLrn adds conv-ReLU-LRN-pool normalisation after the first two
+ * convolutions (21 layers) */
+void table_alexnet(std::vector<LayerSpec>& t, int n, bool withLrn) {
+    TableBuilder b{t, n};
+    b.conv(3, 227, 0, 4, 96, 11);  b.relu(96, 55);  if (withLrn) b.lrn(96, 55);  b.pool(96, 55, 3);
+    b.conv(96, 27, 2, 1, 256, 5);  b.relu(256, 27); if (withLrn) b.lrn(256, 27); b.pool(256, 27, 3);
+    b.conv(256, 13, 1, 1, 384, 3); b.relu(384, 13);
+    b.conv(384, 13, 1, 1, 384, 3); b.relu(384, 13);
+    b.conv(384, 13, 1, 1, 256, 3); b.relu(256, 13); b.pool(256, 13, 3);
+    b.fc(9216, 4096); b.relu(4096, 1);
+    b.fc(4096, 4096); b.relu(4096, 1);
+    b.fc(4096, 1000); b.softmax(1000);
+}
+
+/* network.cu:325-495: the three classifier layers are convolutions pinned to the memory-optimal mode */
+void table_overfeat(std::vector<LayerSpec>& t, int n) {
+    TableBuilder b{t, n};
+    b.conv(3, 231, 0, 4, 96, 11);    b.relu(96, 56);   b.pool(96, 56, 2);
+    b.conv(96, 28, 0, 1, 256, 5);    b.relu(256, 24);  b.pool(256, 24, 2);
+    b.conv(256, 12, 1, 1, 512, 3);   b.relu(512, 12);
+    b.conv(512, 12, 1, 1, 1024, 3);  b.relu(1024, 12);
+    b.conv(1024, 12, 1, 1, 1024, 3); b.relu(1024, 12); b.pool(1024, 12, 2);
+    b.conv(1024, 6, 0, 1, 3072, 6, true); b.relu(3072, 1);
+    b.conv(3072, 1, 0, 1, 4096, 1, true); b.relu(4096, 1);
+    b.conv(4096, 1, 0, 1, 1000, 1, true); b.softmax(1000);
+}
+
+/* network.cu:501-813 */
+void table_vgg16(std::vector<LayerSpec>& t, int n) {
+    TableBuilder b{t, n};
+    const int stages[5][3] = {{64, 2, 224}, {128, 2, 112}, {256, 3, 56}, {512, 3, 28}, {512, 3, 14}}; // channels, convs, extent
+    int c = 3;
+    for (const auto& st : stages) {
+        for (int i = 0; i < st[1]; i++) { b.conv(c, st[2], 1, 1, st[0], 3); b.relu(st[0], st[2]); c = st[0]; }
+        b.pool(st[0], st[2], 2);
+    }
+    b.fc(512 * 7 * 7, 4096); b.relu(4096, 1);
+    b.fc(4096, 4096);        b.relu(4096, 1);
+    b.fc(4096, 1000);        b.softmax(1000);
+}
+
+size_t spec_src_count(const LayerSpec& s) { return (size_t)s.n * s.c * s.h * s.w; }
+
+void spec_out(const LayerSpec& s, int& n, int& c, int& h, int& w) {
+    n = s.n;
+    switch (s.type) {
+    case FC_GEMM: c = s.k; h = 1; w = 1; break;
+    case CONV: case FC_CONV: c = s.k; h = vdnn_out_dim(s.h, s.pad_h, s.r, s.stride_h); w = vdnn_out_dim(s.w, s.pad_w, s.s, s.stride_w); break;
+    case POOL: c = s.c; h = vdnn_out_dim(s.h, s.pad_h, s.r, s.stride_h); w = vdnn_out_dim(s.w, s.pad_w, s.s, s.stride_w); break;
+    default: c = s.c; h = s.h; w = s.w; break;
+    }
+}
+
+size_t spec_dst_count(const LayerSpec& s) {
+    int n, c, h, w;
+    spec_out(s, n, c, h, w);
+    return (size_t)n * c * h * w;
+}
+
+} // namespace
+
+std::vector<LayerSpec> Network::tableFor(CNN_t cnn, int batch) {
+    std::vector<LayerSpec> t;
+    switch (cnn) {
+    case ALEXNET: table_alexnet(t, batch, false); break;
+    case ALEXNET_LRN: table_alexnet(t, batch, true); break;
+    case OVERFEAT: table_overfeat(t, batch); break;
+    case VGG16_64: case VGG16_128: case VGG16_256: case VGG16_512: table_vgg16(t, batch); break;
+    default: break; // GOOGLENET and CUSTOM_CNN are empty stubs in the reference (network.cu:497-499, 815-817)
+    }
+    return t;
+}
+
+Network::Network(CNN_t _cnnType, vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode, int _batchSize)
+    : cnnType(_cnnType), options(), batchSize(_batchSize), customTable(false) {
+    construct(_vdnnType, _algoMode);
+}
+
+Network::Network(CNN_t _cnnType, vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode, int _batchSize, const NetworkOptions& _options)
+    : cnnType(_cnnType), options(_options), batchSize(_batchSize), customTable(false) {
+    construct(_vdnnType, _algoMode);
+}
+
+Network::Network(const std::vector<LayerSpec>& table, vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode, const NetworkOptions& _options)
+    : cnnType(CUSTOM_CNN), options(_options), batchSize(table.empty() ? 0 : table[0].n), customTable(true), specs(table) {
+    construct(_vdnnType, _algoMode);
+}
+
+/* network.cu:10-92 */
+void Network::construct(vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) {
+    vdnnType = _vdnnType;
+    algoMode = _algoMode;
+    numLayers = 0;
+    inputData = labelData = networkDiffData = networkGradData = workSpace = nullptr;
+    lossData = nullptr;
+    inputResident = false;
+    for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
+        layer[i] = nullptr;
+        isOffload[i] = isPrefetched[i] = false;
+        offloadedSrcData_h[i] = nullptr;
+        evFwdDone[i] = evOffloadDone[i] = evBlockFree[i] = evPrefetchDone[i] = nullptr;
+    }
+
+    /* context = handles + streams (network.cu:39-42) */
+    ctx = nullptr;
+    checkVDNN(vdnn_ctx_create(&ctx, options.device, options.planOnly ? VDNN_CTX_PLAN_ONLY : 0));
+    convHandle.ctx = ctx;
+    gemmHandle.ctx = ctx;
+    stream_compute = vdnn_ctx_stream_compute(ctx);
+    stream_memory = vdnn_ctx_stream_d2h(ctx);
+    Layer::setInitSeed(options.seed);
+    Layer::setVerbose(options.verbose);
+    Layer::setSkipParameterValues(options.planOnly);
+
+    if (_algoMode == VDNN_DYNAMIC_ALGO) {
+        /* network.cu:59-78: start from (VDNN_ALL, memory-optimal), then walk the ladder */
+        algoMode = VDNN_MEMORY_OPT_ALGO;
+        vdnnType = VDNN_ALL;
+        setLayers(cnnType);
+        setVdnnType(VDNN_ALL);
+        allocIoBuffers();
+        vdnnDynamicAlgo();
+    } else {
+        setLayers(cnnType);
+        setVdnnType(vdnnType);
+        allocIoBuffers();
+    }
+}
+
+Network::~Network() {
+    if (ctx) vdnn_device_synchronize(ctx);
+    releasePolicyBuffers();
+    releaseLayers();
+    for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
+        for (vdnn_event_t* e : {&evFwdDone[i], &evOffloadDone[i], &evBlockFree[i], &evPrefetchDone[i]}) {
+            if (*e) vdnn_event_destroy(ctx, *e);
+            *e = nullptr;
+        }
+    }
+    if (ctx) {
+        vdnn_pool_finalize(ctx);
+        vdnn_ctx_destroy(ctx);
+    }
+}
+
+void Network::releaseLayers() {
+    for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
+        delete layer[i];
+        layer[i] = nullptr;
+    }
+    numLayers = 0;
+}
+
+void Network::releasePolicyBuffers() {
+    for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
+        if (offloadedSrcData_h[i]) vdnn_host_free_pinned(ctx, offloadedSrcData_h[i]);
+        offloadedSrcData_h[i] = nullptr;
+        isOffload[i] = isPrefetched[i] = false;
+    }
+}
+
+/* network.cu:101-132: drop every allocation, rebuild layers and buffers for a new configuration */
+void Network::reset(CNN_t _cnnType, vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) {
+    vdnn_device_synchronize(ctx);
+    releasePolicyBuffers();
+    releaseLayers();
+    vdnn_pool_finalize(ctx); /* cnmemFinalize: everything carved from the pool is gone */
+    inputData = labelData = networkDiffData = networkGradData = workSpace = nullptr;
+    lossData = nullptr;
+    inputResident = false;
+    cnnType = _cnnType;
+    algoMode = _algoMode;
+    vdnnType = _vdnnType;
+    setLayers(_cnnType);
+    setVdnnType(_vdnnType);
+    allocIoBuffers();
+}
+
+/* network.cu:47-53 reserves floor(totalGlobalMem / 1e9) GB. On a 288 GB device that would take the
+ * whole card for a network that needs a fraction of it, so the reservation is sized from the layer
+ * table instead: everything BASELINE keeps resident plus slack; options.poolBytes overrides. */
+void Network::initPool() {
+    size_t bytes = options.poolBytes;
+    if (bytes == 0) {
+        size_t sum = 0, maxAct = 0;
+        for (const LayerSpec& s : specs) {
+            const size_t src = spec_src_count(s), dst = spec_dst_count(s);
+            sum += dst;
+            maxAct = std::max(maxAct, std::max(src, dst));
+            if (s.type == FC_GEMM || is_conv(s.type)) sum += (size_t)s.k * s.c * s.r * s.s + s.k;
+        }
+        sum += spec_src_count(specs[0]) * 2 + spec_dst_count(specs.back()) * 2 + 3 * maxAct;
+        bytes = sum * sizeof(DATATYPE);
+        bytes += bytes / 8 + (size_t(384) << 20); // rounding of ~100 blocks, staging area, headroom
+        size_t freeB = 0, totalB = 0;
+        checkVDNN(vdnn_device_mem_info(ctx, &freeB, &totalB));
+        const size_t limit = freeB - freeB / 16;
+        if (bytes > limit) bytes = limit;
+    }
+    ASSERT_EQ(vdnn_pool_init(ctx, bytes));
+    if (options.capBytes) checkVDNN(vdnn_pool_set_cap(ctx, options.capBytes));
+}
+
+/* network.cu:134-154 */
+void Network::setLayers(CNN_t _cnnType) {
+    cnnType = _cnnType;
+    if (_cnnType == ALEXNET || _cnnType == ALEXNET_LRN) setLayersAlexnet();
+    else if (_cnnType == OVERFEAT) setLayersOverfeat();
+    else if (_cnnType == GOOGLENET) setLayersGooglenet();
+    else if (_cnnType == VGG16_64) setLayersVgg16(64);
+    else if (_cnnType == VGG16_128) setLayersVgg16(128);
+    else if (_cnnType == VGG16_256) setLayersVgg16(256);
+    else if (_cnnType == VGG16_512) setLayersVgg16(512);
+    else if (_cnnType == CUSTOM_CNN) setLayersCustomCNN();
+    else M_ASSERT(false, "Invalid CNN Type!");
+    if (options.verbose) printf("-------------------------------------------------------\n\n");
+    sanityCheck();
+}
+
+void Network::setLayersAlexnet() {
+    specs = tableFor(cnnType, batchSize);
+    buildLayers();
+}
+
+void Network::setLayersOverfeat() {
+    specs = tableFor(OVERFEAT, batchSize);
+    buildLayers();
+}
+
+void Network::setLayersGooglenet() {
+    M_ASSERT(false, "GOOGLENET is an empty stub in the reference (network.cu:497-499); not available");
+}
+
+/* network.cu:501-503: the VGG16 variants carry their batch in the enum; a batch given to the
+ * constructor that differs from the default overrides it (addition, used for small test batches) */
+void Network::setLayersVgg16(int givenBatch) {
+    if (batchSize == DEFAULT_BATCH_SIZE || batchSize <= 0) batchSize = givenBatch;
+    specs = tableFor(VGG16_128, batchSize);
+    buildLayers();
+}
+
+void Network::setLayersCustomCNN() {
+    M_ASSERT(customTable && !specs.empty(), "CUSTOM_CNN needs an explicit layer table");
+    buildLayers();
+}
+
+/* Creates the Layer objects of `specs` (the bodies of the reference's setLayers* functions). */
+void Network::buildLayers() {
+    M_ASSERT(!specs.empty() && (int)specs.size() <= DEFAULT_NUM_LAYER, "layer table empty or too long");
+    numLayers = (int)specs.size();
+    batchSize = specs[0].n;
+    n_in = specs[0].n; c_in = specs[0].c; h_in = specs[0].h; w_in = specs[0].w;
+    spec_out(specs.back(), n_out, c_out, h_out, w_out);
+    initPool();
+    for (int l = 0; l < numLayers; l++) {
+        const LayerSpec& s = specs[l];
+        const vdnnAlgoMode_t mode = s.forceMemOpt ? VDNN_MEMORY_OPT_ALGO : algoMode;
+        if (s.type == FC_GEMM)
+            layer[l] = new Layer(vdnnType, mode, s.type, &gemmHandle, &stream_compute, &stream_memory, l,
+                                 s.n, s.c, s.h, s.w, s.pad_h, s.pad_w, s.stride_h, s.stride_w, s.k, s.r, s.s);
+        else
+            layer[l] = new Layer(vdnnType, mode, s.type, &convHandle, &stream_compute, &stream_memory, l,
+                                 s.n, s.c, s.h, s.w, s.pad_h, s.pad_w, s.stride_h, s.stride_w, s.k, s.r, s.s);
+    }
+    capDst.assign(numLayers, {});
+    capGrad.assign(numLayers, {});
+}
+
+/* network.cu:819-829: the reference draws U(-0.01, 0.01) from an unseeded generator on every call;
+ * here the draw is seeded (stream 1) and N(0,1) */
+void Network::randomInitializeData(void* data, size_t size) {
+    std::vector<DATATYPE> data_h(size);
+    vdnn::seeded_fill_normal(data_h.data(), size, options.seed, 1, 0.0f, 1.0f);
+    checkVDNN(vdnn_memcpy_h2d(ctx, data, data_h.data(), sizeof(DATATYPE) * size));
+}
+
+/* network.cu:831-873 */
+void Network::sanityCheck() {
+    for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
+        if (i < numLayers) { M_ASSERT(layer[i] != NULL, "Not enough layers!"); }
+        else { M_ASSERT(layer[i] == NULL, "Too many layers!"); }
+    }
+    M_ASSERT((layer[0]->InputN() == n_in && layer[0]->InputC() == c_in && layer[0]->InputH() == h_in && layer[0]->InputW() == w_in),
+             "Layer 0 input and network input have different dimensions");
+    M_ASSERT((layer[numLayers - 1]->OutputN() == n_out && layer[numLayers - 1]->OutputC() == c_out &&
+              layer[numLayers - 1]->OutputH() == h_out && layer[numLayers - 1]->OutputW() == w_out),
+             "Layer L output and network output have different dimensions");
+    for (int i = 0; i < numLayers - 1; i++) {
+        bool check;
+        if (layer[i + 1]->LayerType() == FC_GEMM) {
+            check = layer[i]->DstDataSize() == layer[i + 1]->SrcDataSize();
+        } else {
+            check = layer[i]->OutputN() == layer[i + 1]->InputN() && layer[i]->OutputC() == layer[i + 1]->InputC() &&
+                    layer[i]->OutputH() == layer[i + 1]->InputH() && layer[i]->OutputW() == layer[i + 1]->InputW();
+        }
+        if (!check) {
+            printf("Sanity check error at layer %d and %d!\n", i, i + 1);
+            M_ASSERT(0, "Sanity check error!");
+        }
+    }
+}
+
+/* network.cu:875-940 */
+void Network::setVdnnType(vdnn_t newVdnnType) {
+    vdnnType = newVdnnType;
+    for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
+        isOffload[i] = false;
+        isPrefetched[i] = false;
+        if (offloadedSrcData_h[i] != NULL) vdnn_host_free_pinned(ctx, offloadedSrcData_h[i]);
+        offloadedSrcData_h[i] = NULL;
+        if (layer[i] != NULL) layer[i]->setVdnnMode(newVdnnType);
+    }
+    lastStats.pinnedBytes = 0;
+
+    auto offload = [&](int l) {
+        isOffload[l] = true;
+        const size_t bytes = layer[l]->SrcDataSize() * sizeof(DATATYPE);
+        checkVDNN(vdnn_host_alloc_pinned(ctx, (void**)&offloadedSrcData_h[l], bytes));
+        lastStats.pinnedBytes += bytes;
+    };
+
+    switch (newVdnnType) {
+    case BASELINE: {
+        /* one dx/dy ping-pong pair and one workspace, each sized for the largest user */
+        const size_t dxdySize = findMaxDxDySize();
+        ASSERT_EQ(vdnn_pool_malloc(ctx, &networkDiffData, dxdySize));
+        ASSERT_EQ(vdnn_pool_malloc(ctx, &networkGradData, dxdySize));
+        const size_t workSpaceSize = findMaxWorkSpaceSize();
+        if (workSpaceSize > 0) ASSERT_EQ(vdnn_pool_malloc(ctx, &workSpace, workSpaceSize));
+    } break;
+    case VDNN_NONE:
+        break;
+    case VDNN_ALL:
+        for (int l = 0; l < numLayers - 1; l++) offload(l);
+        break;
+    case VDNN_CONV:
+        for (int l = 0; l < numLayers - 1; l++)
+            if (is_conv(layer[l]->LayerType())) offload(l);
+        break;
+    }
+
+    if (newVdnnType != BASELINE) {
+        for (int l = 0; l < numLayers; l++)
+            for (vdnn_event_t* e : {&evFwdDone[l], &evOffloadDone[l], &evBlockFree[l], &evPrefetchDone[l]})
+                if (!*e) checkVDNN(vdnn_event_create(ctx, e, 0));
+    }
+}
+
+/* network.cu:942-944 is empty in the reference; here it switches every convolution's variant */
+void Network::setAlgoType(vdnnAlgoMode_t newAlgoMode) {
+    algoMode = newAlgoMode;
+    for (int l = 0; l < numLayers; l++)
+        if (!specs[l].forceMemOpt) layer[l]->setAlgoMode(newAlgoMode);
+}
+
+/* network.cu:87-90: input and label tensors; plus the loss scalar and the seeded contents */
+void Network::allocIoBuffers() {
+    ASSERT_EQ(vdnn_pool_malloc(ctx, &inputData, sizeof(DATATYPE) * getInputSize()));
+    ASSERT_EQ(vdnn_pool_malloc(ctx, &labelData, sizeof(DATATYPE) * getOutputSize()));
+    ASSERT_EQ(vdnn_pool_malloc(ctx, (void**)&lossData, sizeof(DATATYPE)));
+    if (!options.planOnly) {
+        inputHost.resize(getInputSize());
+        vdnn::seeded_fill_normal(inputHost.data(), inputHost.size(), options.seed, 1, 0.0f, 1.0f);
+        checkVDNN(vdnn_memcpy_h2d(ctx, inputData, inputHost.data(), sizeof(DATATYPE) * inputHost.size()));
+        const int classes = c_out * h_out * w_out;
+        std::vector<int32_t> lab((size_t)n_out);
+        vdnn::seeded_fill_labels(lab.data(), lab.size(), options.seed, 2, classes);
+        setLabels(lab.data());
+    }
+    inputResident = true;
+}
+
+/* network.cu:946-1008 */
+void Network::vdnnDynamicAlgo() {
+    int ret = 0;
+    if (options.verbose) printf("\n1. Test VDNN_ALL and VDNN_MEMORY_OPT_ALGO\n");
+    if (forwardPropagation(true) < 0 || backwardPropagation(true) < 0) {
+        printf("This CNN model cannot be trained\n");
+        M_ASSERT(0, "This CNN model cannot be trained");
+    }
+    const vdnn_t ladder[3] = {VDNN_NONE, VDNN_CONV, VDNN_ALL};
+    const char* names[3] = {"VDNN_NONE", "VDNN_CONV", "VDNN_ALL"};
+    for (int i = 0; i < 3; i++) {
+        if (options.verbose) printf("\n%d. Test %s and VDNN_PERF_OPT_ALGO\n", i + 2, names[i]);
+        reset(cnnType, ladder[i], VDNN_PERF_OPT_ALGO);
+        ret = forwardPropagation(true);
+        if (ret >= 0) ret = backwardPropagation(true);
+        if (ret >= 0) {
+            reset(cnnType, ladder[i], VDNN_PERF_OPT_ALGO);
+            if (options.verbose) printf("%s and VDNN_PERF_OPT_ALGO Passed!\n", names[i]);
+            return;
+        }
+    }
+    if (options.verbose) printf("\n5. Dynamic Algorithm with VDNN_ALL\n");
+    reset(cnnType, VDNN_ALL, VDNN_PERF_OPT_ALGO);
+    for (int id = 0; id < DEFAULT_NUM_LAYER; id++) {
+        if (layer[id] == NULL) continue;
+        if (is_conv(layer[id]->LayerType())) layer[id]->findDynamicAlgo();
+    }
+}
+
+/* network.cu:1010-1023 */
+size_t Network::findMaxDxDySize() {
+    size_t ret = 0;
+    for (int i = 0; i < numLayers; i++) ret = std::max(ret, layer[i]->SrcDataSize());
+    ret = std::max(ret, layer[numLayers - 1]->DstDataSize());
+    return ret * sizeof(DATATYPE);
+}
+
+/* network.cu:1025-1040 */
+size_t Network::findMaxWorkSpaceSize() {
+    size_t ret = 0;
+    for (int i = 0; i < numLayers; i++) {
+        if (!is_conv(layer[i]->LayerType())) continue;
+        ret = std::max(ret, layer[i]->FwdWorkSpaceSize());
+        ret = std::max(ret, layer[i]->BwdDataWorkSpaceSize());
+        ret = std::max(ret, layer[i]->BwdFilterWorkSpaceSize());
+    }
+    return ret;
+}
+
+/* network.cu:1042-1054: result = first - second on the compute stream (the reference launches it on
+ * the default stream and redraws the label here; the label is fixed at construction instead) */
+void Network::calculateFirstDiffData(void* result, void* first, void* second) {
+    checkVDNN(vdnn_sub(ctx, stream_compute, getOutputSize(), (const float*)first, (const float*)second, (float*)result));
+}
+
+void Network::printUsage(const char* tag, int l, size_t workspace) {
+    if (!options.verbose) return;
+    size_t freeB = 0, totalB = 0;
+    vdnn_pool_info(ctx, &freeB, &totalB);
+    printf("[%s] Layer %d, Free Memory: %lu, Total Memory: %lu, Memory Usage: %lu\n", tag, l,
+           (unsigned long)freeB, (unsigned long)totalB, (unsigned long)(totalB - freeB + workspace));
+}
+
+void Network::captureLayer(int l, bool grad) {
+    if (!options.capture || options.planOnly) return;
+    std::vector<float>& dstv = grad ? capGrad[l] : capDst[l];
+    const size_t count = grad ? layer[l]->SrcDataSize() : layer[l]->DstDataSize();
+    dstv.resize(count);
+    checkVDNN(vdnn_memcpy_d2h(ctx, dstv.data(), grad ? layer[l]->GradData() : layer[l]->DstData(), count * sizeof(float)));
+}
+
+/* network.cu:1090-1091, 1168-1169 */
+void Network::afterLayerSync() {
+    checkVDNN(vdnn_stream_synchronize(ctx, stream_compute));
+    checkVDNN(vdnn_stream_synchronize(ctx, stream_memory));
+    checkVDNN(vdnn_stream_synchronize(ctx, vdnn_ctx_stream_h2d(ctx)));
+}
+
+/* network.cu:1056-1110 */
+int Network::forwardPropagation(bool isDynamic) {
+    M_ASSERT(inputResident && inputData, "forwardPropagation needs the input on the device (run backwardPropagation after a forward)");
+    lastStats.offloadBytes = 0;
+    if (vdnnType == BASELINE) {
+        for (int l = 0; l < numLayers; l++) {
+            layer[l]->copySrcData(l == 0 ? inputData : layer[l - 1]->DstData());
+            if (layer[l]->forward(isOffload, offloadedSrcData_h, workSpace, isDynamic) < 0) return -1;
+            captureLayer(l, false);
+            printUsage("Fwd", l, layer[l]->FwdWorkSpaceSize());
+        }
+    } else {
+        /* everything enqueued so far (the previous step's last prefetch included) precedes this event */
+        checkVDNN(vdnn_event_record(ctx, evBlockFree[0], stream_compute));
+        for (int l = 0; l < numLayers; l++) {
+            layer[l]->copySrcData(l == 0 ? inputData : layer[l - 1]->DstData());
+            if (isOffload[l]) {
+                layer[l]->setSrcReadyEvent(l == 0 ? evBlockFree[0] : evFwdDone[l - 1]);
+                layer[l]->setOffloadDoneEvent(evOffloadDone[l]);
+            }
+
+            /* Forward propagation */
+            if (layer[l]->forward(isOffload, offloadedSrcData_h, workSpace, isDynamic) < 0) return -1;
+            checkVDNN(vdnn_event_record(ctx, evFwdDone[l], stream_compute));
+            captureLayer(l, false);
+
+            /* The reference synchronises both streams on the host here. Ordering is what matters:
+               the block may be recycled once this layer's kernels (stream order) and its offload
+               copy (event) are done with it. */
+            if (options.hostSync) afterLayerSync();
+            else if (isOffload[l]) checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evOffloadDone[l]));
+
+            /* Release srcData of this layer. The reference keeps layer 0's block and later allocates
+               a second one for its prefetch; releasing it here avoids that leak. */
+            if (isOffload[l]) {
+                lastStats.offloadBytes += layer[l]->SrcDataSize() * sizeof(DATATYPE);
+                ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->SrcData()), isDynamic);
+                if (l == 0) { inputData = nullptr; inputResident = false; }
+            }
+            printUsage("Fwd", l, layer[l]->FwdWorkSpaceSize());
+        }
+    }
+    /* addition: mean cross-entropy of the output against the target, for monitoring */
+    checkVDNN(vdnn_cross_entropy_dense(ctx, stream_compute, n_out, c_out * h_out * w_out,
+                                       (const float*)layer[numLayers - 1]->DstData(), (const float*)labelData, lossData));
+    return 0;
+}
+
+/* network.cu:1112-1191 */
+int Network::backwardPropagation(bool isDynamic) {
+    lastStats.prefetchBytes = 0;
+    prefetchLog.clear();
+    if (vdnnType == BASELINE) {
+        calculateFirstDiffData(networkDiffData, layer[numLayers - 1]->DstData(), labelData);
+        for (int l = numLayers - 1; l >= 0; l--) {
+            if (l == numLayers - 1) {
+                layer[l]->copyDiffData(networkDiffData);
+                layer[l]->copyGradData(networkGradData);
+            } else {
+                layer[l]->copyDiffData(layer[l + 1]->GradData());
+                layer[l]->copyGradData(layer[l + 1]->DiffData());
+            }
+            if (layer[l]->backward(-1, NULL, NULL, 0, workSpace, isDynamic) < 0) return -1;
+            captureLayer(l, true);
+            printUsage("Bwd", l, layer[l]->BwdDataWorkSpaceSize() + layer[l]->BwdFilterWorkSpaceSize());
+        }
+    } else {
+        resetIsPrefetchedArray();
+        if (layer[numLayers - 1]->cnmemMallocDiffData(isDynamic) < 0) return -1;
+        calculateFirstDiffData(layer[numLayers - 1]->DiffData(), layer[numLayers - 1]->DstData(), labelData);
+
+        for (int l = numLayers - 1; l >= 0; l--) {
+            if (l != numLayers - 1) {
+                layer[l]->copyDiffData(layer[l + 1]->GradData());
+                layer[l]->copyDstData(layer[l + 1]->SrcData());
+            }
+            /* this layer reads its own srcData: if that was prefetched, the copy must have landed */
+            if (!options.hostSync && isPrefetched[l]) checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evPrefetchDone[l]));
+
+            int prefId = l == 0 ? -1 : findPrefetchLayer(l);
+            if (prefId >= 0) {
+                if (layer[prefId]->cnmemMallocSrcData(isDynamic) < 0) return -1;
+                layer[l]->setPrefetchEvents(evBlockFree[prefId], evOffloadDone[prefId], evPrefetchDone[prefId]);
+                const size_t bytes = sizeof(DATATYPE) * layer[prefId]->SrcDataSize();
+                if (layer[l]->backward(prefId, offloadedSrcData_h[prefId], layer[prefId]->SrcData(), bytes, workSpace, isDynamic) < 0) return -1;
+                lastStats.prefetchBytes += bytes;
+                prefetchLog.emplace_back(l, prefId);
+                if (prefId == 0) { inputData = layer[0]->SrcData(); inputResident = true; }
+            } else {
+                if (layer[l]->backward(-1, NULL, NULL, 0, workSpace, isDynamic) < 0) return -1;
+            }
+            captureLayer(l, true);
+
+            if (options.hostSync) afterLayerSync();
+
+            /* Release dstData and diffData: every reader is already enqueued on the compute stream */
+            ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DstData()), isDynamic);
+            ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DiffData()), isDynamic);
+            printUsage("Bwd", l, layer[l]->BwdDataWorkSpaceSize() + layer[l]->BwdFilterWorkSpaceSize());
+        }
+        ASSERT_EQ(vdnn_pool_free(ctx, layer[0]->GradData()), isDynamic);
+        inputData = layer[0]->SrcData(); /* network.cu:1185 */
+        inputResident = true;
+    }
+    return 0;
+}
+
+/* network.cu:1193-1196 */
+void Network::resetIsPrefetchedArray() {
+    for (int i = 0; i < DEFAULT_NUM_LAYER; i++) isPrefetched[i] = false;
+}
+
+/* network.cu:1198-1208: scan downward from currLayerId-1; the first layer that is offloaded and not
+ * yet prefetched is the one to fetch; stop at the first convolution that is not eligible */
+int Network::findPrefetchLayer(int currLayerId) {
+    for (int id = currLayerId - 1; id >= 0; id--) {
+        if (isOffload[id] == true && isPrefetched[id] == false) {
+            isPrefetched[id] = true;
+            return id;
+        } else if (is_conv(layer[id]->LayerType())) {
+            return -1;
+        }
+    }
+    return -1;
+}
+
+/* ---- additions ------------------------------------------------------------------------------ */
+void Network::setInput(const float* host) {
+    M_ASSERT(inputResident && inputData, "input block is not resident");
+    if (options.planOnly) return;
+    inputHost.assign(host, host + getInputSize());
+    checkVDNN(vdnn_memcpy_h2d(ctx, inputData, host, sizeof(DATATYPE) * getInputSize()));
+}
+
+void Network::getInput(float* host) {
+    M_ASSERT(inputResident && inputData, "input block is not resident");
+    checkVDNN(vdnn_memcpy_d2h(ctx, host, inputData, sizeof(DATATYPE) * getInputSize()));
+}
+
+void Network::setLabels(const int32_t* labels) {
+    const int classes = c_out * h_out * w_out;
+    std::vector<float> dense((size_t)n_out * classes, 0.0f);
+    for (int i = 0; i < n_out; i++) {
+        M_ASSERT(labels[i] >= 0 && labels[i] < classes, "label out of range");
+        dense[(size_t)i * classes + labels[i]] = 1.0f;
+    }
+    setLabelTensor(dense.data());
+}
+
+void Network::setLabelTensor(const float* host) {
+    if (options.planOnly) return;
+    checkVDNN(vdnn_memcpy_h2d(ctx, labelData, host, sizeof(DATATYPE) * getOutputSize()));
+}
+
+int Network::setLayerParams(int l, const float* filter, const float* bias) {
+    if (l < 0 || l >= numLayers || !layer[l]->hasParams()) return -1;
+    if (filter) checkVDNN(vdnn_memcpy_h2d(ctx, layer[l]->FilterData(), filter, layer[l]->FilterDataSize() * sizeof(float)));
+    if (bias) checkVDNN(vdnn_memcpy_h2d(ctx, layer[l]->BiasData(), bias, layer[l]->BiasDataSize() * sizeof(float)));
+    return 0;
+}
+
+int Network::getLayerParams(int l, float* filter, float* bias) {
+    if (l < 0 || l >= numLayers || !layer[l]->hasParams()) return -1;
+    if (filter) checkVDNN(vdnn_memcpy_d2h(ctx, filter, layer[l]->FilterData(), layer[l]->FilterDataSize() * sizeof(float)));
+    if (bias) checkVDNN(vdnn_memcpy_d2h(ctx, bias, layer[l]->BiasData(), layer[l]->BiasDataSize() * sizeof(float)));
+    return 0;
+}
+
+float Network::loss() {
+    float v = 0.0f;
+    if (options.planOnly) return v;
+    checkVDNN(vdnn_memcpy_d2h(ctx, &v, lossData, sizeof(float)));
+    return v;
+}
+
+void Network::synchronize() { checkVDNN(vdnn_device_synchronize(ctx)); }
+
+NetworkStats Network::stats() {
+    NetworkStats s = lastStats;
+    vdnn_pool_peak(ctx, &s.peakBytesInUse, &s.peakExtent);
+    size_t freeB = 0;
+    vdnn_pool_info(ctx, &freeB, &s.poolBytes);
+    s.weightBytes = 0;
+    for (int l = 0; l < numLayers; l++) s.weightBytes += (layer[l]->FilterDataSize() + layer[l]->BiasDataSize()) * sizeof(float);
+    return s;
+}
+
+void Network::resetPeak() { vdnn_pool_reset_peak(ctx); }

@@ -1,0 +1,176 @@
+// Network: layer tables, memory-policy setup, forward/backward drivers and the prefetch scheduler.
+// Mirrors the reference's class Network (network.h:15-95): same public method names and return
+// convention. Additions (marked) cover what the reference cannot do: seeded data, a loss value,
+// tensor capture for parity checks, usage statistics, real teardown.
+#pragma once
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "layer.h"
+
+/* Optional settings of a Network (addition). The reference's constructor takes none of these. */
+struct NetworkOptions {
+    uint64_t seed = 1;           // seed of inputs, labels and filters
+    size_t   poolBytes = 0;      // size of the device pool; 0 = sized from the layer table
+    size_t   capBytes = 0;       // artificial limit on pool bytes in use; 0 = none
+    bool     planOnly = false;   // replay the allocation schedule without a device
+    bool     hostSync = false;   // synchronise both streams after every layer like the reference
+                                 // (network.cu:1090-1091, 1168-1169) instead of ordering by events
+    bool     capture = false;    // keep host copies of every layer's dstData and gradData
+    bool     verbose = false;    // the reference's per-layer printouts
+    int      device = DEFAULT_DEVICE;
+};
+
+/* One row of a layer table (the argument list of the reference's Layer constructor). */
+struct LayerSpec {
+    Layer_t type;
+    int n, c, h, w;
+    int pad_h, pad_w, stride_h, stride_w;
+    int k, r, s;
+    bool forceMemOpt; // OverFeat's FC-as-conv layers ignore the algorithm mode (network.cu:449, 465, 481)
+};
+
+/* Per-step statistics (addition). */
+struct NetworkStats {
+    size_t peakBytesInUse = 0;     // pool high-water mark (bytes in use)
+    size_t peakExtent = 0;         // highest pool offset handed out
+    size_t offloadBytes = 0;       // bytes copied device-to-host by the last forward
+    size_t prefetchBytes = 0;      // bytes copied host-to-device by the last backward
+    size_t pinnedBytes = 0;        // pinned host memory held for offloaded tensors
+    size_t poolBytes = 0;
+    size_t weightBytes = 0;
+};
+
+class Network {
+public:
+    Network(
+        CNN_t          _cnnType,
+        vdnn_t         _vdnnType,
+        vdnnAlgoMode_t _algoMode,
+        int            _batchSize = DEFAULT_BATCH_SIZE);
+    /* addition: explicit options */
+    Network(CNN_t _cnnType, vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode, int _batchSize, const NetworkOptions& _options);
+    /* addition: a network from an explicit layer table (the reference's CUSTOM_CNN is an empty stub) */
+    Network(const std::vector<LayerSpec>& table, vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode, const NetworkOptions& _options);
+    ~Network();
+    Network(const Network&) = delete;
+    Network& operator=(const Network&) = delete;
+
+    /* Reset network */
+    void            reset(CNN_t _cnnType, vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode);
+
+    /* Setup */
+    void            setLayers(CNN_t _cnnType);
+    void            setLayersAlexnet();
+    void            setLayersOverfeat();
+    void            setLayersGooglenet();
+    void            setLayersVgg16(int givenBatch);
+    void            setLayersCustomCNN();
+    void            randomInitializeData(void* data, size_t size);
+    void            sanityCheck();
+    void            setVdnnType(vdnn_t newVdnnType);
+    void            setAlgoType(vdnnAlgoMode_t newAlgoMode);
+    void            vdnnDynamicAlgo();
+
+    /* Find max dx, dy, workspace size (bytes) */
+    size_t          findMaxDxDySize();
+    size_t          findMaxWorkSpaceSize();
+
+    /* Computation for training network */
+    void            calculateFirstDiffData(void* result, void* first, void* second);
+    int             forwardPropagation(bool isDynamic = false);
+    int             backwardPropagation(bool isDynamic = false);
+
+    /* Find prefetch layer */
+    void            resetIsPrefetchedArray();
+    int             findPrefetchLayer(int currLayerId);
+
+    /* Get functions */
+    Layer**         layerArray()            { return layer;              }
+    DATATYPE**      offloadedSrcDataArray() { return offloadedSrcData_h; }
+    size_t          getInputSize()          { return (size_t)n_in * c_in * h_in * w_in;     }
+    size_t          getOutputSize()         { return (size_t)n_out * c_out * h_out * w_out; }
+
+    /* ---- additions ---- */
+    int             numLayersCount() const  { return numLayers; }
+    int             batch() const           { return batchSize; }
+    vdnn_t          policy() const          { return vdnnType; }
+    vdnnAlgoMode_t  algo() const            { return algoMode; }
+    vdnn_ctx*       context()               { return ctx; }
+    bool            isOffloaded(int l) const { return isOffload[l]; }
+    // synthetic data: N(0,1) input, integer labels in [0, classes) as a one-hot target, seeded filters
+    void            setInput(const float* host);
+    void            setLabels(const int32_t* labels);
+    void            setLabelTensor(const float* host);
+    void            getInput(float* host);
+    int             setLayerParams(int l, const float* filter, const float* bias);
+    int             getLayerParams(int l, float* filter, float* bias);
+    // mean cross-entropy of the last forward's output against the target (waits for the device)
+    float           loss();
+    void            synchronize();
+    NetworkStats    stats();
+    void            resetPeak();
+    // host copies of dstData / gradData of layer l taken during the last step (options.capture)
+    const std::vector<float>& capturedDst(int l) const { return capDst[l]; }
+    const std::vector<float>& capturedGrad(int l) const { return capGrad[l]; }
+    // the sequence (backward layer, prefetched layer) of the last backward
+    const std::vector<std::pair<int, int>>& prefetchTrace() const { return prefetchLog; }
+    const std::vector<LayerSpec>& table() const { return specs; }
+    static std::vector<LayerSpec> tableFor(CNN_t cnn, int batch);
+
+private:
+    void            construct(vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode);
+    void            initPool();
+    void            buildLayers();
+    void            releaseLayers();
+    void            releasePolicyBuffers();
+    void            allocIoBuffers();
+    void            captureLayer(int l, bool grad);
+    void            afterLayerSync();
+    void            printUsage(const char* tag, int l, size_t workspace);
+
+    CNN_t               cnnType;
+    vdnn_t              vdnnType;
+    vdnnAlgoMode_t      algoMode;
+    NetworkOptions      options;
+    vdnn_ctx*           ctx;
+    vdnnConvHandle_t    convHandle;   // in place of cudnnHandle
+    vdnnGemmHandle_t    gemmHandle;   // in place of cublasHandle
+    vdnn_stream_t       stream_compute;
+    vdnn_stream_t       stream_memory; // device-to-host copies; host-to-device copies use the context's third stream
+    int                 batchSize;
+    int                 numLayers;
+    bool                customTable;
+
+    /* Input / Output */
+    int n_in, c_in, h_in, w_in;
+    int n_out, c_out, h_out, w_out;
+
+    /* Data */
+    void*               inputData;
+    void*               labelData;
+    void*               networkDiffData;
+    void*               networkGradData;
+    void*               workSpace;
+    float*              lossData;          // one float on the device (addition)
+    std::vector<float>  inputHost;         // the seeded input, kept for re-upload (addition)
+
+    /* Layers */
+    std::vector<LayerSpec> specs;
+    Layer*              layer[DEFAULT_NUM_LAYER];
+    bool                isOffload[DEFAULT_NUM_LAYER];
+    bool                isPrefetched[DEFAULT_NUM_LAYER];
+    DATATYPE*           offloadedSrcData_h[DEFAULT_NUM_LAYER];
+
+    /* Events that order the copy streams against the compute stream (addition) */
+    vdnn_event_t        evFwdDone[DEFAULT_NUM_LAYER];     // compute: layer l's forward kernels enqueued
+    vdnn_event_t        evOffloadDone[DEFAULT_NUM_LAYER]; // d2h: srcData of layer l is in pinned memory
+    vdnn_event_t        evBlockFree[DEFAULT_NUM_LAYER];   // compute: everything enqueued before the prefetch of l
+    vdnn_event_t        evPrefetchDone[DEFAULT_NUM_LAYER];// h2d: srcData of layer l is back on the device
+    bool                inputResident;                     // inputData currently holds the input (addition)
+
+    NetworkStats        lastStats;
+    std::vector<std::vector<float>> capDst, capGrad;
+    std::vector<std::pair<int, int>> prefetchLog;
+};
