@@ -1,0 +1,137 @@
+"""Headline benchmark: VGG16, fp32, batch 128, one MI355X.
+
+A step is one forwardPropagation + backwardPropagation (SGD fused into the backward kernels) on
+seeded synthetic data. BASELINE, VDNN_NONE, VDNN_CONV and VDNN_ALL run back to back; `value` is the
+VDNN_ALL images/s, the other policies and the ratio to BASELINE ride along in `policies`.
+The roofline entry is the convolution kernel class with the largest share of device time, timed with
+HIP events around every launch on the compute stream during the timed steps. The CPU baseline is the
+C checker under oracle/ (a port of the same layer math) on the host cores, at a reduced batch.
+
+One JSON line on stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP32_MFMA_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
+FLOP_PER_IMAGE = 92.82e9  # 3 passes over 13 convolutions and 3 FC layers
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed):
+    net = Network(cnn, policy, algo, batch, seed=seed)
+    try:
+        for _ in range(warmup):
+            assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
+        net.synchronize()
+        net.reset_peak()
+        be.profile_enable(net.context, True)
+        net.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
+        net.synchronize()
+        dt = time.perf_counter() - t0
+        prof = be.profile_collect(net.context)
+        be.profile_enable(net.context, False)
+        st = net.stats()
+        loss = net.loss()
+    finally:
+        net.close()
+    return {"ms_per_step": dt * 1e3 / steps, "images_per_s": batch * steps / dt, "loss": loss,
+            "peak_hbm_gb": st["peak_bytes_in_use"] / 1e9, "offload_gb_per_step": st["offload_bytes"] / 1e9,
+            "prefetch_gb_per_step": st["prefetch_bytes"] / 1e9, "pinned_gb": st["pinned_bytes"] / 1e9}, prof
+
+
+def cpu_baseline(batch):
+    """The checker's training step on the host cores, VGG16 at a reduced batch."""
+    import oracle
+    threads = min(16, os.cpu_count() or 1)
+    oracle.set_threads(threads)
+    net = oracle.Net(cnn=4, batch=batch)
+    net.init_seeded(1)
+    t0 = time.perf_counter()
+    net.forward()
+    net.backward()
+    dt = time.perf_counter() - t0
+    net.close()
+    return {"value": batch / dt, "unit": "images/s", "cores": threads, "kind": "port",
+            "sample": "one VGG16 fp32 step (forward+backward+SGD) at batch %d instead of 128, %.1f s" % (batch, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--batch", type=int, default=128)
+    ap.add_argument("--algo", default="VDNN_MEMORY_OPT_ALGO")
+    ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL")
+    ap.add_argument("--cpu-batch", type=int, default=4)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
+        sys.exit(2)
+
+    import vdnn_implementation_amd.backend as be
+    from vdnn_implementation_amd import enums
+    from vdnn_implementation_amd.network import Network, parse
+
+    cnn = enums.VGG16_128
+    results, profiles = {}, {}
+    for name in args.policies.split(","):
+        _, policy, algo = parse("VGG16_128", name, args.algo)
+        log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
+        results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1)
+        log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
+            results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))
+
+    head = "VDNN_ALL" if "VDNN_ALL" in results else list(results)[-1]
+    base = results.get("BASELINE")
+    # dominant kernel: the convolution class with the most device time under the headline policy
+    prof = profiles[head]
+    conv = {k: v for k, v in prof.items() if k.startswith("conv_") and v["flops"] > 0}
+    dom = max(conv, key=lambda k: conv[k]["ms"])
+    d = conv[dom]
+    achieved = d["flops"] / (d["ms"] * 1e-3) / 1e12
+    conv_all_tf = sum(v["flops"] for v in conv.values()) / (sum(v["ms"] for v in conv.values()) * 1e-3) / 1e12
+    kernels = {k: {"launches": v["launches"], "avg_ms": v["ms"] / max(v["launches"], 1),
+                   "tflops": (v["flops"] / (v["ms"] * 1e-3) / 1e12) if v["flops"] else None,
+                   "gbs": (v["bytes"] / (v["ms"] * 1e-3) / 1e9) if v["bytes"] else None}
+               for k, v in sorted(prof.items(), key=lambda kv: -kv[1]["ms"])}
+    out = {
+        "metric": "VGG16-128 train img/s (VDNN_ALL vs BASELINE); peak HBM GB; conv MFMA util",
+        "value": results[head]["images_per_s"], "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": results[head]["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic (seeded N(0,1) inputs, integer labels, He-normal filters)",
+        "config": {"workload": "VGG16 fp32 batch %d, one SGD step (fwd+bwd), policy %s, %s" % (args.batch, head, args.algo),
+                   "batch": args.batch, "policy": head, "algo": args.algo},
+        "policies": results,
+        "vdnn_all_vs_baseline_speed": (results[head]["images_per_s"] / base["images_per_s"]) if base else None,
+        "peak_hbm_reduction_vs_baseline": (base["peak_hbm_gb"] / results[head]["peak_hbm_gb"]) if base else None,
+        "losses_bit_identical": len({results[k]["loss"] for k in results}) == 1,
+        "conv_mfma_util": conv_all_tf / FP32_MFMA_PEAK_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "avg_launch_ms": d["ms"] / d["launches"], "launches": d["launches"]},
+        "kernels": kernels,
+        "step_mfma_frac": args.batch * FLOP_PER_IMAGE / (results[head]["ms_per_step"] * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+    }
+    if not args.no_cpu_baseline:
+        log("[bench] CPU baseline: checker, VGG16 batch %d" % args.cpu_batch)
+        out["cpu_baseline"] = cpu_baseline(args.cpu_batch)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -192,6 +192,22 @@ int vdnn_softmax_ce_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes,
 int vdnn_cross_entropy_dense(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes,
                              const float* prob, const float* target, float* loss);
 
+/* ---- per-kernel timing (no counterpart in the reference, whose _PROFILE_* macros are unused:
+ *      layer.h:34-38) ---------------------------------------------------------------------------
+ * While enabled, every kernel launch of this library is bracketed by two events on its own stream.
+ * vdnn_profile_collect synchronises the device and returns one entry per kernel class: launches,
+ * summed duration, and the algorithmic work of those launches (floating-point operations for the
+ * MFMA kernels, bytes that must cross HBM for the bandwidth-bound ones). */
+typedef struct {
+    char   name[48];
+    unsigned long long launches;
+    double ms;
+    double flops;
+    double bytes;
+} vdnn_profile_entry;
+int vdnn_profile_enable(vdnn_ctx* ctx, int on);
+int vdnn_profile_collect(vdnn_ctx* ctx, vdnn_profile_entry* out, int capacity, int* count);
+
 #ifdef __cplusplus
 }
 #endif

@@ -40,6 +40,11 @@ def shape(n, c, h, w, k=0, r=0, s=0, pad_h=0, pad_w=0, stride_h=1, stride_w=1):
     return Shape(n, c, h, w, k, r, s, pad_h, pad_w, stride_h, stride_w)
 
 
+class ProfileEntry(C.Structure):
+    _fields_ = [("name", C.c_char * 48), ("launches", C.c_ulonglong), ("ms", C.c_double), ("flops", C.c_double),
+                ("bytes", C.c_double)]
+
+
 _vp, _sz, _i, _f = C.c_void_p, C.c_size_t, C.c_int, C.c_float
 _S = C.POINTER(Shape)
 _psz = C.POINTER(C.c_size_t)
@@ -101,6 +106,8 @@ BACKEND_SYMBOLS = {
     "vdnn_softmax_ce_fwd": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _vp]),
     "vdnn_softmax_ce_bwd": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp]),
     "vdnn_cross_entropy_dense": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp]),
+    "vdnn_profile_enable": (_i, [_vp, _i]),
+    "vdnn_profile_collect": (_i, [_vp, C.POINTER(ProfileEntry), _i, C.POINTER(_i)]),
 }
 
 for _name, (_res, _args) in BACKEND_SYMBOLS.items():
@@ -116,6 +123,19 @@ def check(status):
     if status == VDNN_OOM:
         raise OutOfMemory(status, msg)
     raise BackendError(status, msg)
+
+
+def profile_enable(ctx_handle, on):
+    check(lib.vdnn_profile_enable(ctx_handle, int(on)))
+
+
+def profile_collect(ctx_handle):
+    """{kernel class: {launches, ms, flops, bytes}} since profiling was enabled (synchronises)."""
+    arr = (ProfileEntry * 64)()
+    n = _i()
+    check(lib.vdnn_profile_collect(ctx_handle, arr, 64, C.byref(n)))
+    return {arr[i].name.decode(): {"launches": int(arr[i].launches), "ms": arr[i].ms, "flops": arr[i].flops, "bytes": arr[i].bytes}
+            for i in range(min(n.value, 64))}
 
 
 class DeviceBuffer:

@@ -14,6 +14,17 @@ void set_error(const char* fmt, ...) {
     va_end(ap);
 }
 
+hipEvent_t prof_take_event(vdnn_ctx* ctx) {
+    if (!ctx->prof_free_events.empty()) {
+        hipEvent_t e = ctx->prof_free_events.back();
+        ctx->prof_free_events.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+}
+
 // Virtual base of a plan-only pool: never dereferenced, only used for offset arithmetic.
 static constexpr uintptr_t kPlanBase = uintptr_t(1) << 44;
 
@@ -58,6 +69,8 @@ int vdnn_ctx_destroy(vdnn_ctx* ctx) {
     vdnn_pool_finalize(ctx);
     if (!ctx->plan_only) {
         (void)hipDeviceSynchronize();
+        for (auto& r : ctx->prof_records) { (void)hipEventDestroy(r.start); (void)hipEventDestroy(r.stop); }
+        for (auto e : ctx->prof_free_events) (void)hipEventDestroy(e);
         if (ctx->compute) (void)hipStreamDestroy(ctx->compute);
         if (ctx->d2h) (void)hipStreamDestroy(ctx->d2h);
         if (ctx->h2d) (void)hipStreamDestroy(ctx->h2d);
@@ -302,6 +315,40 @@ int vdnn_memcpy_d2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_dev, siz
     if (ctx->plan_only || bytes == 0) return VDNN_OK;
     VDNN_REQUIRE(dst_dev && src_dev, "null pointer");
     VDNN_HIP(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, stream_of(ctx, stream)));
+    return VDNN_OK;
+}
+
+int vdnn_profile_enable(vdnn_ctx* ctx, int on) {
+    VDNN_REQUIRE(ctx, "null context");
+    if (ctx->plan_only) return VDNN_OK;
+    VDNN_HIP(hipDeviceSynchronize());
+    for (auto& r : ctx->prof_records) { ctx->prof_free_events.push_back(r.start); ctx->prof_free_events.push_back(r.stop); }
+    ctx->prof_records.clear();
+    ctx->profiling = on != 0;
+    return VDNN_OK;
+}
+
+int vdnn_profile_collect(vdnn_ctx* ctx, vdnn_profile_entry* out, int capacity, int* count) {
+    VDNN_REQUIRE(ctx && count, "null argument");
+    *count = 0;
+    if (ctx->plan_only) return VDNN_OK;
+    VDNN_HIP(hipDeviceSynchronize());
+    std::vector<vdnn_profile_entry> agg;
+    for (const auto& r : ctx->prof_records) {
+        float ms = 0.0f;
+        VDNN_HIP(hipEventElapsedTime(&ms, r.start, r.stop));
+        size_t i = 0;
+        for (; i < agg.size(); i++) if (strcmp(agg[i].name, r.name) == 0) break;
+        if (i == agg.size()) {
+            vdnn_profile_entry e;
+            memset(&e, 0, sizeof(e));
+            strncpy(e.name, r.name, sizeof(e.name) - 1);
+            agg.push_back(e);
+        }
+        agg[i].launches += 1; agg[i].ms += ms; agg[i].flops += r.flops; agg[i].bytes += r.bytes;
+    }
+    *count = (int)agg.size();
+    for (int i = 0; i < (int)agg.size() && i < capacity; i++) if (out) out[i] = agg[i];
     return VDNN_OK;
 }
 

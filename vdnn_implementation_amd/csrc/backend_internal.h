@@ -4,6 +4,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <vector>
 
 #include "../../include/vdnn_backend.h"
 #include "pool.h"
@@ -19,6 +20,11 @@ struct vdnn_ctx {
     float* reduce_scratch = nullptr;
     size_t reduce_scratch_bytes = 0;
     int num_cu = 256;
+    // per-kernel timing (vdnn_profile_*)
+    struct ProfRecord { const char* name; hipEvent_t start, stop; double flops, bytes; };
+    bool profiling = false;
+    std::vector<ProfRecord> prof_records;
+    std::vector<hipEvent_t> prof_free_events;
 };
 
 namespace vdnn {
@@ -28,6 +34,23 @@ static constexpr size_t kReduceScratchBytes = size_t(64) << 20;
 void set_error(const char* fmt, ...);
 
 inline hipStream_t stream_of(vdnn_ctx* ctx, vdnn_stream_t s) { return s ? (hipStream_t)s : ctx->compute; }
+
+hipEvent_t prof_take_event(vdnn_ctx* ctx);
+
+// Brackets the launches made during its lifetime with two timing events when profiling is on.
+// `name` must be a string literal (it is kept by pointer).
+struct ProfScope {
+    vdnn_ctx* ctx; hipStream_t stream; size_t index; bool active;
+    ProfScope(vdnn_ctx* c, hipStream_t s, const char* name, double flops, double bytes) : ctx(c), stream(s), index(0), active(c->profiling) {
+        if (!active) return;
+        vdnn_ctx::ProfRecord r{name, prof_take_event(c), prof_take_event(c), flops, bytes};
+        if (!r.start || !r.stop) { active = false; return; }
+        (void)hipEventRecord(r.start, stream);
+        index = c->prof_records.size();
+        c->prof_records.push_back(r);
+    }
+    ~ProfScope() { if (active) (void)hipEventRecord(ctx->prof_records[index].stop, stream); }
+};
 
 } // namespace vdnn
 

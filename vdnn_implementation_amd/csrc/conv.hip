@@ -235,10 +235,17 @@ static GemmDims make_dims(int M, int N, int K, int TM, int TN, int splits) {
     return d;
 }
 
+// names of the kernel classes in the timing report: {pass}_{tile}
+struct PassNames { const char* t64; const char* t128; };
+static const PassNames kFwdNames{"conv_fwd_64x256", "conv_fwd_128x128"};
+static const PassNames kBwdDataNames{"conv_bwd_data_64x256", "conv_bwd_data_128x128"};
+static const PassNames kBwdFilterNames{"conv_bwd_filter_64x256", "conv_bwd_filter_128x128"};
+
 template <int TM, int TN, class AL, class BL, class EP>
-static int launch_igemm(hipStream_t stream, const AL& al, const BL& bl, const EP& ep, const GemmDims& d) {
+static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, const AL& al, const BL& bl, const EP& ep, const GemmDims& d) {
     const long blocks = (long)d.mtiles * d.ntiles * d.splits;
     if (blocks <= 0 || blocks >= (1l << 31)) { set_error("igemm: grid of %ld workgroups out of range", blocks); return VDNN_EINVAL; }
+    ProfScope prof(ctx, stream, name, 2.0 * d.M * (double)d.N * d.K, 0.0);
     hipLaunchKernelGGL((igemm_kernel<TM, TN, AL, BL, EP>), dim3((unsigned)blocks), dim3(NT), 0, stream, al, bl, ep, d);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
@@ -246,9 +253,9 @@ static int launch_igemm(hipStream_t stream, const AL& al, const BL& bl, const EP
 
 // Tile shape by output-channel count: 64-row tiles for narrow layers, 128 otherwise.
 template <class AL, class BL, class EP>
-static int launch_by_m(hipStream_t stream, const AL& al, const BL& bl, const EP& ep, int M, int N, int K, int splits) {
-    if (M <= 64) return launch_igemm<64, 256>(stream, al, bl, ep, make_dims(M, N, K, 64, 256, splits));
-    return launch_igemm<128, 128>(stream, al, bl, ep, make_dims(M, N, K, 128, 128, splits));
+static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names, const AL& al, const BL& bl, const EP& ep, int M, int N, int K, int splits) {
+    if (M <= 64) return launch_igemm<64, 256>(ctx, stream, names.t64, al, bl, ep, make_dims(M, N, K, 64, 256, splits));
+    return launch_igemm<128, 128>(ctx, stream, names.t128, al, bl, ep, make_dims(M, N, K, 128, 128, splits));
 }
 
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
@@ -280,7 +287,7 @@ int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape
     LoadDense<true> al{w, (long)g.C * g.R * g.S, 1, g.K};
     LoadIm2colPix<0> bl{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W};
     StoreNCHW ep{y, bias, g.P * g.Q};
-    return launch_by_m(st, al, bl, ep, g.K, g.N * g.P * g.Q, g.C * g.R * g.S, 1);
+    return launch_by_m(ctx, st, kFwdNames, al, bl, ep, g.K, g.N * g.P * g.Q, g.C * g.R * g.S, 1);
 }
 
 int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
@@ -297,10 +304,10 @@ int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* 
     const int M = g.C, N = g.N * g.H * g.W, K = g.K * g.R * g.S;
     if (g.sh == 1 && g.sw == 1) {
         LoadIm2colPix<1> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, (long)g.K * g.P * g.Q};
-        return launch_by_m(st, al, bl, ep, M, N, K, 1);
+        return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K, 1);
     }
     LoadIm2colPix<2> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.K * g.P * g.Q};
-    return launch_by_m(st, al, bl, ep, M, N, K, 1);
+    return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K, 1);
 }
 
 int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
@@ -333,7 +340,7 @@ int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sha
     LoadDyRed al{dy, g.K, g.P * g.Q};
     LoadIm2colRed bl{x, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N};
     StoreDense ep{w, staging, nullptr, (long)N, (long)M * N, alpha, 1};
-    int rc = M <= 64 ? launch_igemm<64, 256>(st, al, bl, ep, d) : launch_igemm<128, 128>(st, al, bl, ep, d);
+    int rc = M <= 64 ? launch_igemm<64, 256>(ctx, st, kBwdFilterNames.t64, al, bl, ep, d) : launch_igemm<128, 128>(ctx, st, kBwdFilterNames.t128, al, bl, ep, d);
     if (rc != VDNN_OK) return rc;
     if (d.splits > 1) return launch_reduce_splits(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, 1, nullptr, 0);
     return VDNN_OK;

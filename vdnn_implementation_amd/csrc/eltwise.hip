@@ -112,6 +112,7 @@ __global__ void __launch_bounds__(EB) reduce_splits_kernel(float* __restrict__ o
 
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
                          int splits, float alpha, int accumulate, const float* bias_j, int ncols) {
+    ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)count * (splits + 2));
     hipLaunchKernelGGL(reduce_splits_kernel, dim3(grid_for(count, EB, ctx->num_cu * 8)), dim3(EB), 0, stream,
                        out, partial, count, splits, alpha, accumulate, bias_j, ncols);
     VDNN_LAUNCH_CHECK();
@@ -398,6 +399,7 @@ int vdnn_relu_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float
     VDNN_REQUIRE(x && y, "null tensor");
     if (count == 0) return VDNN_OK;
     const size_t n4 = (aligned16(x) && aligned16(y)) ? count / 4 : 0;
+    ProfScope prof(ctx, stream_of(ctx, stream), "relu_fwd", 0.0, 8.0 * (double)count);
     hipLaunchKernelGGL(relu_fwd_kernel, dim3(grid_for(n4 ? n4 : count, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), x, y, n4, count);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
@@ -409,6 +411,7 @@ int vdnn_relu_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float
     VDNN_REQUIRE(t && dy && dx, "null tensor");
     if (count == 0) return VDNN_OK;
     const size_t n4 = (aligned16(t) && aligned16(dy) && aligned16(dx)) ? count / 4 : 0;
+    ProfScope prof(ctx, stream_of(ctx, stream), "relu_bwd", 0.0, 12.0 * (double)count);
     hipLaunchKernelGGL(relu_bwd_kernel, dim3(grid_for(n4 ? n4 : count, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), t, dy, dx, n4, count);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
@@ -456,6 +459,7 @@ int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape
     splits = (N + per - 1) / per;
     VDNN_REQUIRE((size_t)K * splits * sizeof(float) <= ctx->reduce_scratch_bytes, "staging area too small");
     hipStream_t st = stream_of(ctx, stream);
+    ProfScope prof(ctx, st, "conv_bwd_bias", 0.0, 4.0 * (double)N * K * P * Q);
     hipLaunchKernelGGL(bias_grad_partial_kernel, dim3(K * splits), dim3(EB), 0, st, dy, ctx->reduce_scratch, N, K, P * Q, splits, per);
     VDNN_LAUNCH_CHECK();
     hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB - 1) / EB), dim3(EB), 0, st, ctx->reduce_scratch, bias, K, splits, alpha);
@@ -491,6 +495,7 @@ int vdnn_maxpool_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* sh
     VDNN_REQUIRE(shape && pool_geo(shape, g), "unsupported pooling geometry");
     VDNN_REQUIRE(x && y, "null tensor");
     hipStream_t st = stream_of(ctx, stream);
+    ProfScope prof(ctx, st, "maxpool_fwd", 0.0, 4.0 * ((double)g.N * g.C * g.H * g.W + (double)g.N * g.C * g.P * g.Q));
     if (pool_is_2x2_exact(g, x, y, nullptr)) {
         const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
         hipLaunchKernelGGL(maxpool2x2_fwd_kernel, dim3(grid_for(pairs, EB, ctx->num_cu * 16)), dim3(EB), 0, st, x, y, g.H, g.W, pairs);
@@ -510,6 +515,7 @@ int vdnn_maxpool_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* sh
     VDNN_REQUIRE(shape && pool_geo(shape, g), "unsupported pooling geometry");
     VDNN_REQUIRE(x && dy && dx, "null tensor");
     hipStream_t st = stream_of(ctx, stream);
+    ProfScope prof(ctx, st, "maxpool_bwd", 0.0, 4.0 * (2.0 * g.N * g.C * g.H * g.W + (double)g.N * g.C * g.P * g.Q));
     if (pool_is_2x2_exact(g, x, dx, dy) && (g.W / 2) % 2 == 0) {
         const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
         hipLaunchKernelGGL(maxpool2x2_bwd_kernel, dim3(grid_for(pairs, EB, ctx->num_cu * 16)), dim3(EB), 0, st, x, dy, dx, g.H, g.W, pairs);
@@ -525,6 +531,7 @@ int vdnn_lrn_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, cons
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && y && n > 0 && c > 0 && hw > 0, "bad argument");
     const size_t total = (size_t)n * c * hw;
+    ProfScope prof(ctx, stream_of(ctx, stream), "lrn_fwd", 0.0, 8.0 * (double)total);
     hipLaunchKernelGGL(lrn_fwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), x, y, c, hw, total);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
@@ -534,6 +541,7 @@ int vdnn_lrn_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, cons
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && y && dy && dx && n > 0 && c > 0 && hw > 0, "bad argument");
     const size_t total = (size_t)n * c * hw;
+    ProfScope prof(ctx, stream_of(ctx, stream), "lrn_bwd", 0.0, 16.0 * (double)total);
     hipLaunchKernelGGL(lrn_bwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), x, y, dy, dx, c, hw, total);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;

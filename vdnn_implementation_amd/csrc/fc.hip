@@ -11,7 +11,7 @@ int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const fl
 // Out[M][N] (row stride ld_out) = alpha * A*B (+ Out) (+ bias per column); reduction split into
 // ordered partial sums when the tile grid alone cannot fill the chip.
 template <class AL, class BL>
-static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const AL& al, const BL& bl, int M, int N, int K,
+static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const char* name, const AL& al, const BL& bl, int M, int N, int K,
                    float* out, long ld_out, float alpha, int accumulate, const float* bias_j) {
     if (ld_out != N) { set_error("fc_gemm: output must be dense"); return VDNN_EINVAL; }
     const int TM = M <= 64 ? 64 : 128, TN = M <= 64 ? 256 : 128;
@@ -31,6 +31,7 @@ static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const AL& al, const BL& bl, in
     d.splits = (K + kchunk - 1) / kchunk;
     StoreDense ep{out, ctx->reduce_scratch, d.splits > 1 ? nullptr : bias_j, ld_out, (long)M * N, alpha, accumulate};
     const long blocks = (long)d.mtiles * d.ntiles * d.splits;
+    ProfScope prof(ctx, st, name, 2.0 * M * (double)N * K, 0.0);
     if (TM == 64) hipLaunchKernelGGL((igemm_kernel<64, 256, AL, BL, StoreDense>), dim3((unsigned)blocks), dim3(NT), 0, st, al, bl, ep, d);
     else hipLaunchKernelGGL((igemm_kernel<128, 128, AL, BL, StoreDense>), dim3((unsigned)blocks), dim3(NT), 0, st, al, bl, ep, d);
     VDNN_LAUNCH_CHECK();
@@ -51,7 +52,7 @@ int vdnn_fc_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
     VDNN_REQUIRE(x && w && y && n > 0 && c_in > 0 && c_out > 0, "bad argument");
     LoadDense<true> al{x, (long)c_in, 1, n};
     LoadDense<true> bl{w, (long)c_in, 1, c_out};
-    return fc_gemm(ctx, stream_of(ctx, stream), al, bl, n, c_out, c_in, y, c_out, 1.0f, 0, bias);
+    return fc_gemm(ctx, stream_of(ctx, stream), "fc_fwd", al, bl, n, c_out, c_in, y, c_out, 1.0f, 0, bias);
 }
 
 // dx[n][i] = sum_o dy[n][o] * w[o][i]                 (Sgemm(N,N), layer.cu:725-733)
@@ -61,7 +62,7 @@ int vdnn_fc_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c
     VDNN_REQUIRE(dy && w && dx && n > 0 && c_in > 0 && c_out > 0, "bad argument");
     LoadDense<true> al{dy, (long)c_out, 1, n};
     LoadDense<false> bl{w, 1, (long)c_in, c_in};
-    return fc_gemm(ctx, stream_of(ctx, stream), al, bl, n, c_in, c_out, dx, c_in, 1.0f, 0, nullptr);
+    return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_data", al, bl, n, c_in, c_out, dx, c_in, 1.0f, 0, nullptr);
 }
 
 // w[o][i] += alpha * sum_n dy[n][o] * x[n][i]         (Sgemm(N,T) alpha=-lr beta=1, layer.cu:736-744)
@@ -71,7 +72,7 @@ int vdnn_fc_bwd_weight_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in,
     VDNN_REQUIRE(x && dy && w && n > 0 && c_in > 0 && c_out > 0, "bad argument");
     LoadDense<false> al{dy, 1, (long)c_out, c_out};
     LoadDense<false> bl{x, 1, (long)c_in, c_in};
-    return fc_gemm(ctx, stream_of(ctx, stream), al, bl, c_out, c_in, n, w, c_in, alpha, 1, nullptr);
+    return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_weight", al, bl, c_out, c_in, n, w, c_in, alpha, 1, nullptr);
 }
 
 } // extern "C"
