@@ -44,6 +44,8 @@ struct LoadIm2colPix {
     int OH, OW;      // extent of the output pixel grid
     int R, S, ph, pw, sh, sw;
     long sample_stride; // channels_of_src * Hs * Ws
+    FastDiv divRS, divS;
+    const float* zeros; // a readable zero: masked taps are loaded from here
     struct State {
         const float* base;
         int off0, ih0, iw0;
@@ -83,17 +85,19 @@ struct LoadIm2colPix {
         const int RS = R * S, plane = Hs * Ws;
         // every lane of a wavefront shares kk: keep the tap arithmetic on the scalar unit
         const int kbase = __builtin_amdgcn_readfirstlane(kk0 + tid / T);
+        // branch-free, and nothing depends on the loaded value until it is written to LDS
 #pragma unroll
         for (int i = 0; i < L::NLOAD; i++) {
             const int kk = kbase + (NT / T) * i;
-            const int ch = kk / RS, rs = kk - ch * RS;
-            const int tr = rs / S, ts = rs - tr * S;
-            const bool ok = kk < kend && ((st.rowmask >> tr) & (st.colmask >> ts) & 1u);
+            const int ch = divRS.div(kk), rs = kk - ch * RS;
+            const int tr = divS.div(rs), ts = rs - tr * S;
+            const bool ok = (kk < kend) & (((st.rowmask >> tr) & (st.colmask >> ts) & 1u) != 0);
             int off;
             if (MODE == 0) off = st.off0 + ch * plane + tr * Ws + ts;
             else if (MODE == 1) off = st.off0 + ch * plane - tr * Ws - ts;
             else off = ch * plane + ((st.ih0 - tr) / sh) * Ws + (st.iw0 - ts) / sw;
-            r[i] = ok ? st.base[off] : 0.0f;
+            const float* p = ok ? st.base + off : zeros;
+            r[i] = *p;
         }
     }
 };
@@ -103,6 +107,7 @@ struct LoadFilterT {
     static constexpr bool RED_MAJOR = true;
     const float* w;
     int C, RS;
+    const float* zeros;
     struct State { int row0; };
     template <int T>
     __device__ __forceinline__ void init(State& st, int row0, int, int) const { st.row0 = row0; }
@@ -115,7 +120,9 @@ struct LoadFilterT {
 #pragma unroll
         for (int i = 0; i < L::NLOAD; i++) {
             const int c = st.row0 + L::row_of(tid, i);
-            r[i] = (kk < kend && c < C) ? w[kbase + (long)c * RS] : 0.0f;
+            const bool ok = (kk < kend) & (c < C);
+            const float* p = ok ? w + (kbase + (long)c * RS) : zeros;
+            r[i] = *p;
         }
     }
 };
@@ -125,6 +132,7 @@ struct LoadDyRed {
     static constexpr bool RED_MAJOR = true;
     const float* dy;
     int K, PQ;
+    const float* zeros;
     struct State { int row0; };
     template <int T>
     __device__ __forceinline__ void init(State& st, int row0, int, int) const { st.row0 = row0; }
@@ -139,7 +147,9 @@ struct LoadDyRed {
 #pragma unroll
         for (int i = 0; i < L::NLOAD; i++) {
             const int m = st.row0 + L::row_of(tid, i);
-            r[i] = (kok && m < K) ? base[(long)m * PQ] : 0.0f;
+            const bool ok = kok & (m < K);
+            const float* p = ok ? base + (long)m * PQ : zeros;
+            r[i] = *p;
         }
     }
 };
@@ -151,6 +161,7 @@ struct LoadIm2colRed {
     const float* x;
     int C, H, W, R, S, P, Q, ph, pw, sh, sw;
     int ncols; // C*R*S
+    const float* zeros;
     static constexpr int MAXROWS = 256 * KB / NT; // rows per thread for the widest tile
     struct State {
         int joff[MAXROWS]; // c*H*W + r*W + s, or -1 when the column is out of range
@@ -184,13 +195,15 @@ struct LoadIm2colRed {
         const int n = kc / PQ, pq = kc - n * PQ;
         const int p = pq / Q, q = pq - p * Q;
         const int ih0 = p * sh - ph, iw0 = q * sw - pw;
-        const float* base = x + (long)n * C * H * W + ih0 * W + iw0;
+        const float* sample = x + (long)n * C * H * W;
+        const int poff = ih0 * W + iw0;
 #pragma unroll
         for (int i = 0; i < L::NLOAD; i++) {
             const int tr = st.jrs[i] >> 8, ts = st.jrs[i] & 255;
             const int ih = ih0 + tr, iw = iw0 + ts;
-            const bool ok = kok && st.joff[i] >= 0 && ih >= 0 && ih < H && iw >= 0 && iw < W;
-            r[i] = ok ? base[st.joff[i]] : 0.0f;
+            const bool ok = kok & (st.joff[i] >= 0) & ((unsigned)ih < (unsigned)H) & ((unsigned)iw < (unsigned)W);
+            const float* p = ok ? sample + (poff + st.joff[i]) : zeros;
+            r[i] = *p;
         }
     }
 };
@@ -284,8 +297,8 @@ int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(x && w && y, "null tensor");
     hipStream_t st = stream_of(ctx, stream);
-    LoadDense<true> al{w, (long)g.C * g.R * g.S, 1, g.K};
-    LoadIm2colPix<0> bl{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W};
+    LoadDense<true> al{w, (long)g.C * g.R * g.S, 1, g.K, ctx->zeros};
+    LoadIm2colPix<0> bl{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, FastDiv::make(g.R * g.S), FastDiv::make(g.S), ctx->zeros};
     StoreNCHW ep{y, bias, g.P * g.Q};
     return launch_by_m(ctx, st, kFwdNames, al, bl, ep, g.K, g.N * g.P * g.Q, g.C * g.R * g.S, 1);
 }
@@ -299,14 +312,14 @@ int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* 
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(dy && w && dx, "null tensor");
     hipStream_t st = stream_of(ctx, stream);
-    LoadFilterT al{w, g.C, g.R * g.S};
+    LoadFilterT al{w, g.C, g.R * g.S, ctx->zeros};
     StoreNCHW ep{dx, nullptr, g.H * g.W};
     const int M = g.C, N = g.N * g.H * g.W, K = g.K * g.R * g.S;
     if (g.sh == 1 && g.sw == 1) {
-        LoadIm2colPix<1> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, (long)g.K * g.P * g.Q};
+        LoadIm2colPix<1> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, (long)g.K * g.P * g.Q, FastDiv::make(g.R * g.S), FastDiv::make(g.S), ctx->zeros};
         return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K, 1);
     }
-    LoadIm2colPix<2> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.K * g.P * g.Q};
+    LoadIm2colPix<2> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.K * g.P * g.Q, FastDiv::make(g.R * g.S), FastDiv::make(g.S), ctx->zeros};
     return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K, 1);
 }
 
@@ -337,8 +350,8 @@ int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sha
     if (want > by_mem) want = by_mem;
     if (want < 1) want = 1;
     GemmDims d = make_dims(M, N, (int)Kred, TM, TN, (int)want);
-    LoadDyRed al{dy, g.K, g.P * g.Q};
-    LoadIm2colRed bl{x, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N};
+    LoadDyRed al{dy, g.K, g.P * g.Q, ctx->zeros};
+    LoadIm2colRed bl{x, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N, ctx->zeros};
     StoreDense ep{w, staging, nullptr, (long)N, (long)M * N, alpha, 1};
     int rc = M <= 64 ? launch_igemm<64, 256>(ctx, st, kBwdFilterNames.t64, al, bl, ep, d) : launch_igemm<128, 128>(ctx, st, kBwdFilterNames.t128, al, bl, ep, d);
     if (rc != VDNN_OK) return rc;

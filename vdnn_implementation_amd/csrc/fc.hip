@@ -50,8 +50,8 @@ int vdnn_fc_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
                 const float* x, const float* w, const float* bias, float* y) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && w && y && n > 0 && c_in > 0 && c_out > 0, "bad argument");
-    LoadDense<true> al{x, (long)c_in, 1, n};
-    LoadDense<true> bl{w, (long)c_in, 1, c_out};
+    LoadDense<true> al{x, (long)c_in, 1, n, ctx->zeros};
+    LoadDense<true> bl{w, (long)c_in, 1, c_out, ctx->zeros};
     return fc_gemm(ctx, stream_of(ctx, stream), "fc_fwd", al, bl, n, c_out, c_in, y, c_out, 1.0f, 0, bias);
 }
 
@@ -60,8 +60,8 @@ int vdnn_fc_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c
                      const float* dy, const float* w, float* dx) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(dy && w && dx && n > 0 && c_in > 0 && c_out > 0, "bad argument");
-    LoadDense<true> al{dy, (long)c_out, 1, n};
-    LoadDense<false> bl{w, 1, (long)c_in, c_in};
+    LoadDense<true> al{dy, (long)c_out, 1, n, ctx->zeros};
+    LoadDense<false> bl{w, 1, (long)c_in, c_in, ctx->zeros};
     return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_data", al, bl, n, c_in, c_out, dx, c_in, 1.0f, 0, nullptr);
 }
 
@@ -70,8 +70,8 @@ int vdnn_fc_bwd_weight_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in,
                            const float* x, const float* dy, float* w, float alpha) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && dy && w && n > 0 && c_in > 0 && c_out > 0, "bad argument");
-    LoadDense<false> al{dy, 1, (long)c_out, c_out};
-    LoadDense<false> bl{x, 1, (long)c_in, c_in};
+    LoadDense<false> al{dy, 1, (long)c_out, c_out, ctx->zeros};
+    LoadDense<false> bl{x, 1, (long)c_in, c_in, ctx->zeros};
     return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_weight", al, bl, c_out, c_in, n, w, c_in, alpha, 1, nullptr);
 }
 

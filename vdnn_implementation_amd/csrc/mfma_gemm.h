@@ -36,6 +36,21 @@ __device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
     return start + idx;
 }
 
+// Division of a small non-negative integer by a loop-invariant divisor as a multiply-high with the
+// 33-bit constant ceil(2^32 / d), kept as (hi, lo) so that d == 1 needs no branch.
+// Exact while x * d < 2^32 (callers bound x below 2^24 and d by 256).
+struct FastDiv {
+    unsigned lo, hi;
+    __host__ __device__ static FastDiv make(int divisor) {
+        const unsigned long long m = (0x100000000ull + (unsigned)divisor - 1) / (unsigned)divisor;
+        FastDiv f;
+        f.lo = (unsigned)m;
+        f.hi = (unsigned)(m >> 32);
+        return f;
+    }
+    __device__ __forceinline__ int div(int x) const { return (int)(__umulhi((unsigned)x, lo) + (unsigned)x * hi); }
+};
+
 template <int T, bool RED_MAJOR>
 struct LdsLayout {
     static constexpr int ROW_STRIDE = RED_MAJOR ? (KB + 1) : 1;
@@ -55,19 +70,27 @@ template <int A_RS, int A_KS, int B_RS, int B_KS>
 __device__ __forceinline__ void mfma_slice(const float* __restrict__ As, const float* __restrict__ Bs,
                                            floatx16 (&acc)[2][2], int lane) {
     const int l32 = lane & 31, lk = lane >> 5;
+    // operand fragments of step t+1 are read from LDS while the four MFMAs of step t execute
+    float a[2][2], b[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) a[0][i] = As[(i * 32 + l32) * A_RS + lk * A_KS];
+#pragma unroll
+    for (int j = 0; j < 2; j++) b[0][j] = Bs[(j * 32 + l32) * B_RS + lk * B_KS];
 #pragma unroll
     for (int t = 0; t < KB / 2; t++) {
-        const int k = 2 * t + lk;
-        float a[2], b[2];
+        const int cur = t & 1, nxt = cur ^ 1;
+        if (t + 1 < KB / 2) {
+            const int k = 2 * (t + 1) + lk;
 #pragma unroll
-        for (int i = 0; i < 2; i++) a[i] = As[(i * 32 + l32) * A_RS + k * A_KS];
+            for (int i = 0; i < 2; i++) a[nxt][i] = As[(i * 32 + l32) * A_RS + k * A_KS];
 #pragma unroll
-        for (int j = 0; j < 2; j++) b[j] = Bs[(j * 32 + l32) * B_RS + k * B_KS];
+            for (int j = 0; j < 2; j++) b[nxt][j] = Bs[(j * 32 + l32) * B_RS + k * B_KS];
+        }
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i], b[cur][j], acc[i][j], 0, 0, 0);
     }
 }
 
@@ -148,18 +171,21 @@ struct LoadDense {
     const float* base;
     long ld_row, ld_k;
     int rows; // valid rows
+    const float* zeros; // a readable zero: elements outside the matrix are loaded from here
     struct State { int row0; };
     template <int T>
     __device__ __forceinline__ void init(State& st, int row0, int, int) const { st.row0 = row0; }
     template <int T>
     __device__ __forceinline__ void load(const State& st, int kk0, int kend, int tid, float (&r)[LdsLayout<T, RED_MAJOR>::NLOAD]) const {
         using L = LdsLayout<T, RED_MAJOR>;
+        // branch-free, and nothing depends on the loaded value until it is written to LDS
 #pragma unroll
         for (int i = 0; i < L::NLOAD; i++) {
             const int row = st.row0 + L::row_of(tid, i);
             const int kk = kk0 + L::kk_of(tid, i);
-            const bool ok = row < rows && kk < kend;
-            r[i] = ok ? base[(long)row * ld_row + (long)kk * ld_k] : 0.0f;
+            const bool ok = (row < rows) & (kk < kend);
+            const float* p = ok ? base + ((long)row * ld_row + (long)kk * ld_k) : zeros;
+            r[i] = *p;
         }
     }
 };
