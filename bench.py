@@ -27,8 +27,8 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed):
-    net = Network(cnn, policy, algo, batch, seed=seed)
+def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False):
+    net = Network(cnn, policy, algo, batch, seed=seed, refined=refined)
     try:
         for _ in range(warmup):
             assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
@@ -47,9 +47,21 @@ def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed):
         loss = net.loss()
     finally:
         net.close()
-    return {"ms_per_step": dt * 1e3 / steps, "images_per_s": batch * steps / dt, "loss": loss,
-            "peak_hbm_gb": st["peak_bytes_in_use"] / 1e9, "offload_gb_per_step": st["offload_bytes"] / 1e9,
-            "prefetch_gb_per_step": st["prefetch_bytes"] / 1e9, "pinned_gb": st["pinned_bytes"] / 1e9}, prof
+    res = {"ms_per_step": dt * 1e3 / steps, "images_per_s": batch * steps / dt, "loss": loss,
+           "peak_hbm_gb": st["peak_bytes_in_use"] / 1e9, "offload_gb_per_step": st["offload_bytes"] / 1e9,
+           "prefetch_gb_per_step": st["prefetch_bytes"] / 1e9, "pinned_gb": st["pinned_bytes"] / 1e9}
+    # host link: busy time and rate of the copies, and how much of the copy time ran under compute
+    copies = [prof[k] for k in ("offload_d2h", "prefetch_h2d") if k in prof]
+    if copies:
+        copy_ms = sum(c["ms"] for c in copies)
+        kernel_ms = sum(v["ms"] for k, v in prof.items() if k not in ("offload_d2h", "prefetch_h2d"))
+        res["d2h_gbs"] = prof["offload_d2h"]["bytes"] / (prof["offload_d2h"]["ms"] * 1e-3) / 1e9
+        res["h2d_gbs"] = prof["prefetch_h2d"]["bytes"] / (prof["prefetch_h2d"]["ms"] * 1e-3) / 1e9
+        res["copy_busy_ms_per_step"] = copy_ms / steps
+        res["kernel_busy_ms_per_step"] = kernel_ms / steps
+        # step = kernels + copies - overlap + idle  =>  overlap >= kernels + copies - step
+        res["overlap_fraction_lower_bound"] = max(0.0, min(1.0, (kernel_ms + copy_ms - dt * 1e3) / copy_ms))
+    return res, prof
 
 
 def cpu_baseline(batch):
@@ -75,7 +87,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--algo", default="VDNN_MEMORY_OPT_ALGO")
-    ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL")
+    ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined")
     ap.add_argument("--cpu-batch", type=int, default=24)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -90,17 +102,21 @@ def main():
     cnn = enums.VGG16_128
     results, profiles = {}, {}
     for name in args.policies.split(","):
-        _, policy, algo = parse("VGG16_128", name, args.algo)
+        # "+refined": the same policy with the value-preserving lifetime refinements switched on
+        word, _, suffix = name.partition("+")
+        _, policy, algo = parse("VGG16_128", word, args.algo)
         log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
-        results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1)
+        results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1,
+                                                   refined=(suffix == "refined"))
         log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
             results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))
 
-    head = "VDNN_ALL" if "VDNN_ALL" in results else list(results)[-1]
+    head = "VDNN_ALL" if "VDNN_ALL" in results else list(results)[0]
     base = results.get("BASELINE")
     # dominant kernel: the convolution class with the most device time under the headline policy
     prof = profiles[head]
     conv = {k: v for k, v in prof.items() if k.startswith("conv_") and v["flops"] > 0}
+    prof = {k: v for k, v in prof.items() if v["ms"] > 0}
     dom = max(conv, key=lambda k: conv[k]["ms"])
     d = conv[dom]
     achieved = d["flops"] / (d["ms"] * 1e-3) / 1e12
@@ -119,6 +135,10 @@ def main():
         "policies": results,
         "vdnn_all_vs_baseline_speed": (results[head]["images_per_s"] / base["images_per_s"]) if base else None,
         "peak_hbm_reduction_vs_baseline": (base["peak_hbm_gb"] / results[head]["peak_hbm_gb"]) if base else None,
+        "refined_vdnn_all_vs_baseline_speed": (results["VDNN_ALL+refined"]["images_per_s"] / base["images_per_s"])
+        if base and "VDNN_ALL+refined" in results else None,
+        "refined_peak_hbm_reduction_vs_baseline": (base["peak_hbm_gb"] / results["VDNN_ALL+refined"]["peak_hbm_gb"])
+        if base and "VDNN_ALL+refined" in results else None,
         "losses_bit_identical": len({results[k]["loss"] for k in results}) == 1,
         "conv_mfma_util": conv_all_tf / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",

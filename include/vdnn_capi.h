@@ -24,6 +24,7 @@ typedef struct {
     int      capture;      /* keep host copies of every layer's dstData / gradData */
     int      verbose;
     int      device;
+    int      refined_lifetimes; /* value-preserving lifetime refinements of the vDNN policies (0 = literal schedule) */
 } vdnn_network_options;
 
 typedef struct {

@@ -86,10 +86,10 @@ def assert_bit_identical(a, b, what):
 @pytest.mark.parametrize("cnn,batch,algo", [(None, 4, VDNN_MEMORY_OPT_ALGO), (ALEXNET_LRN, 4, VDNN_MEMORY_OPT_ALGO),
                                             (OVERFEAT, 3, VDNN_MEMORY_OPT_ALGO), (VGG16_128, 2, VDNN_PERF_OPT_ALGO)])
 def test_policies_are_bit_identical_to_baseline(cnn, batch, algo):
-    def make(policy, host_sync=False):
+    def make(policy, host_sync=False, refined=False):
         if cnn is None:
-            return Network(layers=small_specs(batch), policy=policy, algo=algo, capture=True, seed=3, host_sync=host_sync)
-        return Network(cnn, policy, algo, batch, capture=True, seed=3, host_sync=host_sync)
+            return Network(layers=small_specs(batch), policy=policy, algo=algo, capture=True, seed=3, host_sync=host_sync, refined=refined)
+        return Network(cnn, policy, algo, batch, capture=True, seed=3, host_sync=host_sync, refined=refined)
 
     announce("policies bit-identical", cnn, batch, "BASELINE")
     with make(BASELINE) as net:
@@ -102,6 +102,12 @@ def test_policies_are_bit_identical_to_baseline(cnn, batch, algo):
             with make(policy, host_sync) as net:
                 got = run_steps(net, 2)
             assert_bit_identical(got, base, "policy %d host_sync %s" % (policy, host_sync))
+        # the lifetime refinements (dead ReLU inputs released, early release of unread outputs,
+        # in-place ReLU backward) change no value either
+        announce("policies bit-identical", cnn, batch, "policy", policy, "refined lifetimes")
+        with make(policy, refined=True) as net:
+            got = run_steps(net, 2)
+        assert_bit_identical(got, base, "policy %d refined" % policy)
 
 
 def layer_forward_on_checker(spec, src, w, b):

@@ -282,6 +282,7 @@ int vdnn_memcpy_d2h_async(vdnn_ctx* ctx, void* dst_host, const void* src_dev, si
     VDNN_REQUIRE(ctx, "null context");
     if (ctx->plan_only || bytes == 0) return VDNN_OK;
     VDNN_REQUIRE(dst_host && src_dev, "null pointer");
+    ProfScope prof(ctx, stream ? (hipStream_t)stream : ctx->d2h, "offload_d2h", 0.0, (double)bytes);
     VDNN_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, stream ? (hipStream_t)stream : ctx->d2h));
     return VDNN_OK;
 }
@@ -290,6 +291,7 @@ int vdnn_memcpy_h2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, si
     VDNN_REQUIRE(ctx, "null context");
     if (ctx->plan_only || bytes == 0) return VDNN_OK;
     VDNN_REQUIRE(dst_dev && src_host, "null pointer");
+    ProfScope prof(ctx, stream ? (hipStream_t)stream : ctx->h2d, "prefetch_h2d", 0.0, (double)bytes);
     VDNN_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, stream ? (hipStream_t)stream : ctx->h2d));
     return VDNN_OK;
 }

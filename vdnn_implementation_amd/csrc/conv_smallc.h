@@ -1,0 +1,137 @@
+// Backward data for layers with at most four input channels (the first layer of each network),
+// on the vector ALU: the implicit GEMM would have only C <= 4 output rows.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "conv_loaders.h"
+
+namespace vdnn {
+
+// ---- backward data for layers with at most four input channels (the first layer of each network) --
+// The implicit GEMM has only C <= 4 output rows, which would fill 3/64 of an MFMA tile; instead one
+// thread produces all channels of one input pixel with vector FMAs, summing over (k, r, s) in that
+// order. Filters are staged through LDS eight output channels at a time as [k][tap] -> float4 of the
+// (zero padded) input channels, so every lane reads the same address (broadcast).
+constexpr int SMALLC_KC = 8;
+constexpr int SMALLC_MAXTAPS = 128;
+
+template <bool STRIDE1>
+__global__ void __launch_bounds__(256) conv_bwd_data_smallc_kernel(const float* __restrict__ dy, const float* __restrict__ w,
+                                                                   float* __restrict__ dx, const ConvGeo g) {
+    __shared__ float4 ws[SMALLC_KC][SMALLC_MAXTAPS];
+    const int tid = threadIdx.x;
+    const int RS = g.R * g.S;
+    const long pix = (long)blockIdx.x * 256 + tid;
+    const long total = (long)g.N * g.H * g.W;
+    const bool live = pix < total;
+    const long pc = live ? pix : 0;
+    const int n = (int)(pc / (g.H * g.W));
+    const int hw = (int)(pc - (long)n * g.H * g.W);
+    const int h = hw / g.W, x = hw - h * g.W;
+    const int th = h + g.ph, tw = x + g.pw;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k0 = 0; k0 < g.K; k0 += SMALLC_KC) {
+        __syncthreads();
+        for (int i = tid; i < SMALLC_KC * RS; i += 256) {
+            const int kk = i / RS, tap = i - kk * RS;
+            float v[4] = {0.f, 0.f, 0.f, 0.f};
+            if (k0 + kk < g.K)
+                for (int c = 0; c < g.C; c++) v[c] = w[((long)(k0 + kk) * g.C + c) * RS + tap];
+            ws[kk][tap] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+        __syncthreads();
+        if (!live) continue;
+        const int kmax = min(SMALLC_KC, g.K - k0);
+        for (int kk = 0; kk < kmax; kk++) {
+            const float* dyp = dy + ((long)n * g.K + k0 + kk) * g.P * g.Q;
+            for (int r = 0; r < g.R; r++) {
+                int p = th - r;
+                if (STRIDE1) {
+                    if ((unsigned)p >= (unsigned)g.P) continue;
+                } else {
+                    if (p < 0 || p % g.sh != 0) continue;
+                    p /= g.sh;
+                    if (p >= g.P) continue;
+                }
+                const float* row = dyp + (long)p * g.Q;
+                for (int s = 0; s < g.S; s++) {
+                    int q = tw - s;
+                    if (STRIDE1) {
+                        if ((unsigned)q >= (unsigned)g.Q) continue;
+                    } else {
+                        if (q < 0 || q % g.sw != 0) continue;
+                        q /= g.sw;
+                        if (q >= g.Q) continue;
+                    }
+                    const float d = row[q];
+                    const float4 f = ws[kk][r * g.S + s];
+                    acc.x += d * f.x; acc.y += d * f.y; acc.z += d * f.z; acc.w += d * f.w;
+                }
+            }
+        }
+    }
+    if (!live) return;
+    float* o = dx + (long)n * g.C * g.H * g.W + hw;
+    const long plane = (long)g.H * g.W;
+    o[0] = acc.x;
+    if (g.C > 1) o[plane] = acc.y;
+    if (g.C > 2) o[2 * plane] = acc.z;
+    if (g.C > 3) o[3 * plane] = acc.w;
+}
+
+// The same, for a compile-time window at stride 1 (VGG's 3x3): fully unrolled and branch-free. Taps
+// outside dy are read from a clamped position and replaced by zero. The filter values of one output
+// channel are wave-uniform, so they are fetched with scalar loads straight from global memory.
+template <int RC, int SC, int CC>
+__global__ void __launch_bounds__(256) conv_bwd_data_smallc_s1_kernel(const float* __restrict__ dy, const float* __restrict__ w,
+                                                                      float* __restrict__ dx, const ConvGeo g) {
+    constexpr int RS = RC * SC;
+    const int tid = threadIdx.x;
+    const long pix = (long)blockIdx.x * 256 + tid;
+    const long total = (long)g.N * g.H * g.W;
+    const bool live = pix < total;
+    const long pc = live ? pix : 0;
+    const int n = (int)(pc / (g.H * g.W));
+    const int hw = (int)(pc - (long)n * g.H * g.W);
+    const int h = hw / g.W, x = hw - h * g.W;
+    int rowoff[RC], col[SC];
+    bool rowok[RC], colok[SC];
+#pragma unroll
+    for (int r = 0; r < RC; r++) {
+        const int p = h + g.ph - r;
+        rowok[r] = (unsigned)p < (unsigned)g.P;
+        rowoff[r] = rowok[r] ? p * g.Q : 0;
+    }
+#pragma unroll
+    for (int s = 0; s < SC; s++) {
+        const int q = x + g.pw - s;
+        colok[s] = (unsigned)q < (unsigned)g.Q;
+        col[s] = colok[s] ? q : 0;
+    }
+    float acc[CC];
+#pragma unroll
+    for (int c = 0; c < CC; c++) acc[c] = 0.f;
+    const long kstride = (long)g.P * g.Q;
+    const float* dyp = dy + (long)n * g.K * kstride;
+    for (int k = 0; k < g.K; k++, dyp += kstride) {
+        const float* wk = w + (long)k * CC * RS; // uniform: scalar loads
+#pragma unroll
+        for (int r = 0; r < RC; r++) {
+            const float* row = dyp + rowoff[r];
+#pragma unroll
+            for (int s = 0; s < SC; s++) {
+                const float v = row[col[s]];
+                const float d = (rowok[r] & colok[s]) ? v : 0.0f;
+#pragma unroll
+                for (int c = 0; c < CC; c++) acc[c] += d * wk[c * RS + r * SC + s];
+            }
+        }
+    }
+    if (!live) return;
+    float* o = dx + (long)n * CC * g.H * g.W + hw;
+    const long plane = (long)g.H * g.W;
+#pragma unroll
+    for (int c = 0; c < CC; c++) o[c * plane] = acc[c];
+}
+
+} // namespace vdnn

@@ -8,12 +8,13 @@ namespace vdnn {
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
                          int splits, float alpha, int accumulate, const float* bias_j, int ncols);
 
-// Out[M][N] (row stride ld_out) = alpha * A*B (+ Out) (+ bias per column); reduction split into
+static inline bool fc_aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// Out[M][N] (dense, row stride N) = alpha * A*B (+ Out) (+ bias per column); the reduction is split into
 // ordered partial sums when the tile grid alone cannot fill the chip.
 template <class AL, class BL>
 static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const char* name, const AL& al, const BL& bl, int M, int N, int K,
-                   float* out, long ld_out, float alpha, int accumulate, const float* bias_j) {
-    if (ld_out != N) { set_error("fc_gemm: output must be dense"); return VDNN_EINVAL; }
+                   float* out, float alpha, int accumulate, const float* bias_j) {
     const int TM = M <= 64 ? 64 : 128, TN = M <= 64 ? 256 : 128;
     const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
     long want = (4l * ctx->num_cu + tiles - 1) / tiles;
@@ -29,7 +30,7 @@ static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const char* name, const AL& al
     kchunk = (kchunk + KB - 1) / KB * KB;
     d.kchunk = kchunk;
     d.splits = (K + kchunk - 1) / kchunk;
-    StoreDense ep{out, ctx->reduce_scratch, d.splits > 1 ? nullptr : bias_j, ld_out, (long)M * N, alpha, accumulate};
+    StoreDense ep{out, ctx->reduce_scratch, d.splits > 1 ? nullptr : bias_j, (long)N, (long)M * N, alpha, accumulate};
     const long blocks = (long)d.mtiles * d.ntiles * d.splits;
     ProfScope prof(ctx, st, name, 2.0 * M * (double)N * K, 0.0);
     if (TM == 64) hipLaunchKernelGGL((igemm_kernel<64, 256, AL, BL, StoreDense>), dim3((unsigned)blocks), dim3(NT), 0, st, al, bl, ep, d);
@@ -43,6 +44,8 @@ static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const char* name, const AL& al
 
 using namespace vdnn;
 
+#define FC_REQUIRE_SMALL(elems) VDNN_REQUIRE((long)(elems) * 4 < 0x7FFF0000l, "matrix of 2 GiB or more")
+
 extern "C" {
 
 // y[n][o] = sum_i x[n][i] * w[o][i] + bias[o]        (Sgemm(T,N) + bias broadcast, layer.cu:677-706)
@@ -50,9 +53,15 @@ int vdnn_fc_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
                 const float* x, const float* w, const float* bias, float* y) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && w && y && n > 0 && c_in > 0 && c_out > 0, "bad argument");
-    LoadDense<true> al{x, (long)c_in, 1, n, ctx->zeros};
-    LoadDense<true> bl{w, (long)c_in, 1, c_out, ctx->zeros};
-    return fc_gemm(ctx, stream_of(ctx, stream), "fc_fwd", al, bl, n, c_out, c_in, y, c_out, 1.0f, 0, bias);
+    FC_REQUIRE_SMALL((long)n * c_in); FC_REQUIRE_SMALL((long)c_out * c_in);
+    const unsigned xb = (unsigned)((long)n * c_in * 4), wb = (unsigned)((long)c_out * c_in * 4);
+    hipStream_t st = stream_of(ctx, stream);
+    if (c_in % 4 == 0 && fc_aligned16(x) && fc_aligned16(w)) {
+        LoadDenseRed<true> al{x, (long)c_in, n, xb}, bl{w, (long)c_in, c_out, wb};
+        return fc_gemm(ctx, st, "fc_fwd", al, bl, n, c_out, c_in, y, 1.0f, 0, bias);
+    }
+    LoadDenseRed<false> al{x, (long)c_in, n, xb}, bl{w, (long)c_in, c_out, wb};
+    return fc_gemm(ctx, st, "fc_fwd", al, bl, n, c_out, c_in, y, 1.0f, 0, bias);
 }
 
 // dx[n][i] = sum_o dy[n][o] * w[o][i]                 (Sgemm(N,N), layer.cu:725-733)
@@ -60,9 +69,16 @@ int vdnn_fc_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c
                      const float* dy, const float* w, float* dx) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(dy && w && dx && n > 0 && c_in > 0 && c_out > 0, "bad argument");
-    LoadDense<true> al{dy, (long)c_out, 1, n, ctx->zeros};
-    LoadDense<false> bl{w, 1, (long)c_in, c_in, ctx->zeros};
-    return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_data", al, bl, n, c_in, c_out, dx, c_in, 1.0f, 0, nullptr);
+    FC_REQUIRE_SMALL((long)n * c_out); FC_REQUIRE_SMALL((long)c_out * c_in);
+    const unsigned db = (unsigned)((long)n * c_out * 4), wb = (unsigned)((long)c_out * c_in * 4);
+    hipStream_t st = stream_of(ctx, stream);
+    LoadDenseRow bl{w, (long)c_in, c_in, wb};
+    if (c_out % 4 == 0 && fc_aligned16(dy)) {
+        LoadDenseRed<true> al{dy, (long)c_out, n, db};
+        return fc_gemm(ctx, st, "fc_bwd_data", al, bl, n, c_in, c_out, dx, 1.0f, 0, nullptr);
+    }
+    LoadDenseRed<false> al{dy, (long)c_out, n, db};
+    return fc_gemm(ctx, st, "fc_bwd_data", al, bl, n, c_in, c_out, dx, 1.0f, 0, nullptr);
 }
 
 // w[o][i] += alpha * sum_n dy[n][o] * x[n][i]         (Sgemm(N,T) alpha=-lr beta=1, layer.cu:736-744)
@@ -70,9 +86,10 @@ int vdnn_fc_bwd_weight_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in,
                            const float* x, const float* dy, float* w, float alpha) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && dy && w && n > 0 && c_in > 0 && c_out > 0, "bad argument");
-    LoadDense<false> al{dy, 1, (long)c_out, c_out, ctx->zeros};
-    LoadDense<false> bl{x, 1, (long)c_in, c_in, ctx->zeros};
-    return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_weight", al, bl, c_out, c_in, n, w, c_in, alpha, 1, nullptr);
+    FC_REQUIRE_SMALL((long)n * c_out); FC_REQUIRE_SMALL((long)n * c_in);
+    LoadDenseRow al{dy, (long)c_out, c_out, (unsigned)((long)n * c_out * 4)};
+    LoadDenseRow bl{x, (long)c_in, c_in, (unsigned)((long)n * c_in * 4)};
+    return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_weight", al, bl, c_out, c_in, n, w, alpha, 1, nullptr);
 }
 
 } // extern "C"

@@ -305,7 +305,8 @@ int Layer::activationForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, v
 int Layer::activationBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h, void* _srcDataToPrefetch,
                               unsigned long _prefetch_bytes, void*, bool isDynamic) {
     if (vdnnMode != BASELINE) {
-        if (cnmemMallocGradData(isDynamic) < 0) return -1;
+        if (inPlaceOp) gradData = diffData; /* elementwise: dx may overwrite dy */
+        else if (cnmemMallocGradData(isDynamic) < 0) return -1;
     }
     if (vdnnMode != BASELINE && _layer_id_to_prefetch >= 0)
         prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);

@@ -162,6 +162,9 @@ public:
 
     /* Set functions */
     void    setVdnnMode(vdnn_t _vdnnMode) { vdnnMode = _vdnnMode; }
+    // ReLU only: backward writes dx over dy instead of into a freshly allocated gradData
+    void    setInPlaceOp(bool v) { inPlaceOp = v; }
+    bool    InPlaceOp() const { return inPlaceOp; }
     void    setAlgoMode(vdnnAlgoMode_t m);
     // Event the offload copy waits for (srcData fully written) and the events this layer's copies
     // signal; owned by the Network. Null events mean "no ordering needed" (plan-only contexts).

@@ -9,21 +9,34 @@
 // ever exists as LDS tiles). Loads for slice s+1 are issued into registers before slice s is
 // multiplied, then written to the other LDS buffer: one barrier per slice.
 //
-// LDS layouts (chosen so both the global-load lane order and the MFMA operand reads are
-// bank-conflict free):
-//   reduction-major operand (lanes of a load run along kk):  lds[row * (KB+1) + kk]
-//   row-major operand       (lanes of a load run along the row/column index): lds[kk * T + row]
+// The matrix pipe and the vector ALU of a SIMD do not overlap well, so every vector instruction in
+// the loop costs MFMA time. The loaders therefore fetch through buffer descriptors: an element that
+// must read as zero (outside the matrix, a padding tap, beyond the reduction range) is given an
+// out-of-range offset and the hardware returns 0 - no branch, no select, and nothing depends on the
+// loaded value until it is written to LDS. Uniform parts of an address go into the scalar offset.
+//
+// LDS layouts:
+//   reduction-major operand (a thread's load runs along kk): lds[row * (KB+4) + kk], moved as
+//       128-bit chunks of four consecutive kk where the source allows
+//   row-major operand (lanes run along the row/column index): lds[kk * T + row]
 // MFMA operand mapping for 32x32x2: lane l supplies A[i = l%32][k = l/32] and B[k = l/32][j = l%32];
-// result register v of lane l is D[8*(v/4) + 4*(l/32) + v%4][l%32].
+// result register v of lane l is D[8*(v/4) + 4*(l/32) + v%4][l%32]. The order in which the KB
+// reduction indices of a slice are consumed is free as long as A and B agree: step (g, i) uses
+// k = 8g + 4*(l/32) + i, so a lane's four values of a reduction-major operand are one 128-bit read.
 #pragma once
 #include <hip/hip_runtime.h>
 
 namespace vdnn {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int KB = 16;   // reduction depth of one LDS slice
-constexpr int NT = 256;  // threads per workgroup
+constexpr int KB = 16;              // reduction depth of one LDS slice
+constexpr int NT = 256;             // threads per workgroup
+constexpr int RED_STRIDE = KB + 4;  // row stride of a reduction-major LDS tile (80 bytes: 128-bit reads of 8 consecutive rows hit 8 different bank groups)
+constexpr int OOB = -1;             // byte offset that is out of range for every descriptor
+constexpr int SENT = 0x40000000;    // out-of-range marker that survives one addition of a second offset below 1 GiB
+constexpr unsigned MAX_SUM_RANGE = 0x40000000u; // descriptors addressed with summed offsets must be smaller than this
 
 // MI355X has 8 XCDs, each with its own L2; consecutive workgroup ids are dealt round-robin to the
 // XCDs. Remap so that consecutive *logical* tiles (which share operand tiles) land on one XCD.
@@ -51,46 +64,70 @@ struct FastDiv {
     __device__ __forceinline__ int div(int x) const { return (int)(__umulhi((unsigned)x, lo) + (unsigned)x * hi); }
 };
 
+// ---- buffer descriptors: loads that return 0 outside [0, bytes) ----------------------------------
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+// voff: per-lane byte offset; soff: wave-uniform byte offset. Out of range if voff + soff >= bytes
+// (no 32-bit wrap-around: OOB + anything stays out of range).
+__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+__device__ __forceinline__ floatx4 buf_load4(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+// Descriptor range for `bytes` remaining after the base, clamped to what a descriptor can hold.
+__device__ __forceinline__ unsigned clamp_range(long bytes) {
+    return bytes <= 0 ? 0u : (bytes > 0xFFFFFFF0l ? 0xFFFFFFF0u : (unsigned)bytes);
+}
+
+// ---- LDS tile geometry ------------------------------------------------------------------------------
 template <int T, bool RED_MAJOR>
-struct LdsLayout {
-    static constexpr int ROW_STRIDE = RED_MAJOR ? (KB + 1) : 1;
-    static constexpr int K_STRIDE = RED_MAJOR ? 1 : T;
-    static constexpr int SIZE = RED_MAJOR ? T * (KB + 1) : KB * T;
-    static constexpr int NLOAD = T * KB / NT; // elements each thread moves per slice
-    // element i of a thread: (row, kk) within the tile
-    __device__ static __forceinline__ int row_of(int tid, int i) { return RED_MAJOR ? (tid / KB + (NT / KB) * i) : (tid % T); }
-    __device__ static __forceinline__ int kk_of(int tid, int i) { return RED_MAJOR ? (tid % KB) : (tid / T + (NT / T) * i); }
-    __device__ static __forceinline__ void store(float* lds, int tid, const float (&r)[NLOAD]) {
-#pragma unroll
-        for (int i = 0; i < NLOAD; i++) lds[row_of(tid, i) * ROW_STRIDE + kk_of(tid, i) * K_STRIDE] = r[i];
-    }
+struct LdsTile {
+    static constexpr int SIZE = RED_MAJOR ? T * RED_STRIDE : KB * T;
+    static constexpr int ROW_STRIDE = RED_MAJOR ? RED_STRIDE : 1;
 };
 
-template <int A_RS, int A_KS, int B_RS, int B_KS>
+// Four reduction values (k = 8g + 4*lk + i, i = 0..3) of row l32 of a 32-row tile at `tile`.
+template <int T, bool RED_MAJOR>
+__device__ __forceinline__ floatx4 read_frag(const float* tile, int l32, int lk, int g) {
+    if (RED_MAJOR) {
+        return *(const floatx4*)(tile + l32 * RED_STRIDE + 8 * g + 4 * lk);
+    } else {
+        const float* p = tile + (8 * g + 4 * lk) * T + l32;
+        floatx4 v;
+        v.x = p[0]; v.y = p[T]; v.z = p[2 * T]; v.w = p[3 * T];
+        return v;
+    }
+}
+
+template <int TM, int TN, bool A_RED, bool B_RED>
 __device__ __forceinline__ void mfma_slice(const float* __restrict__ As, const float* __restrict__ Bs,
                                            floatx16 (&acc)[2][2], int lane) {
     const int l32 = lane & 31, lk = lane >> 5;
-    // operand fragments of step t+1 are read from LDS while the four MFMAs of step t execute
-    float a[2][2], b[2][2];
+    constexpr int A_TILE = 32 * LdsTile<TM, A_RED>::ROW_STRIDE, B_TILE = 32 * LdsTile<TN, B_RED>::ROW_STRIDE;
+    // fragments of group g+1 are read from LDS while the MFMAs of group g execute
+    floatx4 a[2][2], b[2][2];
 #pragma unroll
-    for (int i = 0; i < 2; i++) a[0][i] = As[(i * 32 + l32) * A_RS + lk * A_KS];
+    for (int i = 0; i < 2; i++) a[0][i] = read_frag<TM, A_RED>(As + i * A_TILE, l32, lk, 0);
 #pragma unroll
-    for (int j = 0; j < 2; j++) b[0][j] = Bs[(j * 32 + l32) * B_RS + lk * B_KS];
+    for (int j = 0; j < 2; j++) b[0][j] = read_frag<TN, B_RED>(Bs + j * B_TILE, l32, lk, 0);
 #pragma unroll
-    for (int t = 0; t < KB / 2; t++) {
-        const int cur = t & 1, nxt = cur ^ 1;
-        if (t + 1 < KB / 2) {
-            const int k = 2 * (t + 1) + lk;
+    for (int g = 0; g < KB / 8; g++) {
+        const int cur = g & 1, nxt = cur ^ 1;
+        if (g + 1 < KB / 8) {
 #pragma unroll
-            for (int i = 0; i < 2; i++) a[nxt][i] = As[(i * 32 + l32) * A_RS + k * A_KS];
+            for (int i = 0; i < 2; i++) a[nxt][i] = read_frag<TM, A_RED>(As + i * A_TILE, l32, lk, g + 1);
 #pragma unroll
-            for (int j = 0; j < 2; j++) b[nxt][j] = Bs[(j * 32 + l32) * B_RS + k * B_KS];
+            for (int j = 0; j < 2; j++) b[nxt][j] = read_frag<TN, B_RED>(Bs + j * B_TILE, l32, lk, g + 1);
         }
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int e = 0; e < 4; e++)
 #pragma unroll
-            for (int j = 0; j < 2; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i], b[cur][j], acc[i][j], 0, 0, 0);
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][e], b[cur][j][e], acc[i][j], 0, 0, 0);
     }
 }
 
@@ -103,10 +140,10 @@ struct GemmDims {
 template <int TM, int TN, class AL, class BL, class EP>
 __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, const EP ep, const GemmDims d) {
     static_assert(TM % 64 == 0 && TN % 64 == 0 && (TM / 64) * (TN / 64) == 4, "four 64x64 wave tiles");
-    using LA = LdsLayout<TM, AL::RED_MAJOR>;
-    using LB = LdsLayout<TN, BL::RED_MAJOR>;
-    __shared__ float As[2][LA::SIZE];
-    __shared__ float Bs[2][LB::SIZE];
+    using LA = LdsTile<TM, AL::RED_MAJOR>;
+    using LB = LdsTile<TN, BL::RED_MAJOR>;
+    __shared__ __attribute__((aligned(16))) float As[2][LA::SIZE];
+    __shared__ __attribute__((aligned(16))) float Bs[2][LB::SIZE];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -120,10 +157,10 @@ __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, con
     const int k_begin = ks * d.kchunk;
     const int k_end = min(d.K, k_begin + d.kchunk);
 
-    typename AL::State sa;
-    typename BL::State sb;
-    al.template init<TM>(sa, m0, tid, d.M);
-    bl.template init<TN>(sb, j0, tid, d.N);
+    typename AL::template State<TM> sa;
+    typename BL::template State<TN> sb;
+    al.template init<TM>(sa, m0, tid, d.M, k_begin);
+    bl.template init<TN>(sb, j0, tid, d.N, k_begin);
 
     floatx16 acc[2][2];
 #pragma unroll
@@ -134,14 +171,15 @@ __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, con
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
     const int wm0 = (wave % (TM / 64)) * 64, wn0 = (wave / (TM / 64)) * 64;
-    float ra[LA::NLOAD], rb[LB::NLOAD];
+    typename AL::template Regs<TM> ra;
+    typename BL::template Regs<TN> rb;
 
     const int nslices = (k_end - k_begin + KB - 1) / KB;
     if (nslices > 0) {
         al.template load<TM>(sa, k_begin, k_end, tid, ra);
         bl.template load<TN>(sb, k_begin, k_end, tid, rb);
-        LA::store(As[0], tid, ra);
-        LB::store(Bs[0], tid, rb);
+        AL::template store<TM>(As[0], tid, ra);
+        BL::template store<TN>(Bs[0], tid, rb);
     }
     __syncthreads();
     for (int s = 0; s < nslices; s++) {
@@ -152,11 +190,10 @@ __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, con
             al.template load<TM>(sa, kk0, k_end, tid, ra);
             bl.template load<TN>(sb, kk0, k_end, tid, rb);
         }
-        mfma_slice<LA::ROW_STRIDE, LA::K_STRIDE, LB::ROW_STRIDE, LB::K_STRIDE>(
-            As[cur] + wm0 * LA::ROW_STRIDE, Bs[cur] + wn0 * LB::ROW_STRIDE, acc, lane);
+        mfma_slice<TM, TN, AL::RED_MAJOR, BL::RED_MAJOR>(As[cur] + wm0 * LA::ROW_STRIDE, Bs[cur] + wn0 * LB::ROW_STRIDE, acc, lane);
         if (more) {
-            LA::store(As[cur ^ 1], tid, ra);
-            LB::store(Bs[cur ^ 1], tid, rb);
+            AL::template store<TM>(As[cur ^ 1], tid, ra);
+            BL::template store<TN>(Bs[cur ^ 1], tid, rb);
         }
         __syncthreads();
     }
@@ -164,29 +201,93 @@ __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, con
     ep.store(acc, m0 + wm0, j0 + wn0, lane, ks, d);
 }
 
-// ---- dense operand: element (row, kk) at base[row*ld_row + kk*ld_k] -----------------------------
-template <bool RED_MAJOR_>
-struct LoadDense {
-    static constexpr bool RED_MAJOR = RED_MAJOR_;
+// ---- dense reduction-major operand: element (row, kk) at base[row*ld + kk] -------------------------
+// VEC4: rows are 16-byte aligned and the reduction range is a multiple of four, so a thread moves
+// 128-bit chunks (thread t: chunk t%4 of rows t/4 + 64*i). Otherwise 32-bit elements
+// (thread t: kk t%16 of rows t/16 + 16*i).
+template <bool VEC4>
+struct LoadDenseRed {
+    static constexpr bool RED_MAJOR = true;
     const float* base;
-    long ld_row, ld_k;
-    int rows; // valid rows
-    const float* zeros; // a readable zero: elements outside the matrix are loaded from here
-    struct State { int row0; };
+    long ld;          // elements between rows
+    int rows;         // valid rows
+    unsigned bytes;   // extent of the matrix in bytes (below 2 GiB)
+    template <int T> struct Regs { floatx4 v[T / 64]; float s[VEC4 ? 1 : T / 16]; };
+    template <int T> struct State { int vrow[VEC4 ? T / 64 : T / 16]; __amdgpu_buffer_rsrc_t rsrc; };
     template <int T>
-    __device__ __forceinline__ void init(State& st, int row0, int, int) const { st.row0 = row0; }
-    template <int T>
-    __device__ __forceinline__ void load(const State& st, int kk0, int kend, int tid, float (&r)[LdsLayout<T, RED_MAJOR>::NLOAD]) const {
-        using L = LdsLayout<T, RED_MAJOR>;
-        // branch-free, and nothing depends on the loaded value until it is written to LDS
+    __device__ __forceinline__ void init(State<T>& st, int row0, int tid, int, int) const {
+        st.rsrc = make_rsrc(base, bytes);
+        if (VEC4) {
 #pragma unroll
-        for (int i = 0; i < L::NLOAD; i++) {
-            const int row = st.row0 + L::row_of(tid, i);
-            const int kk = kk0 + L::kk_of(tid, i);
-            const bool ok = (row < rows) & (kk < kend);
-            const float* p = ok ? base + ((long)row * ld_row + (long)kk * ld_k) : zeros;
-            r[i] = *p;
+            for (int i = 0; i < T / 64; i++) {
+                const int row = row0 + (tid >> 2) + 64 * i;
+                st.vrow[i] = row < rows ? (int)(((long)row * ld + 4 * (tid & 3)) * 4) : OOB;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < T / 16; i++) {
+                const int row = row0 + (tid >> 4) + 16 * i;
+                st.vrow[i] = row < rows ? (int)(((long)row * ld + (tid & 15)) * 4) : OOB;
+            }
         }
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int kk0, int kend, int tid, Regs<T>& r) const {
+        const int soff = kk0 * 4;
+        // only the last slice of a range can be partial; there a thread past the end reads out of range
+        const bool tail = kk0 + KB > kend;
+        if (VEC4) {
+            const bool dead = tail && (kk0 + 4 * (tid & 3) >= kend);
+#pragma unroll
+            for (int i = 0; i < T / 64; i++) r.v[i] = buf_load4(st.rsrc, dead ? OOB : st.vrow[i], soff);
+        } else {
+            const bool dead = tail && (kk0 + (tid & 15) >= kend);
+#pragma unroll
+            for (int i = 0; i < T / 16; i++) r.s[i] = buf_load(st.rsrc, dead ? OOB : st.vrow[i], soff);
+        }
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(float* lds, int tid, const Regs<T>& r) {
+        if (VEC4) {
+#pragma unroll
+            for (int i = 0; i < T / 64; i++) *(floatx4*)(lds + ((tid >> 2) + 64 * i) * RED_STRIDE + 4 * (tid & 3)) = r.v[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < T / 16; i++) lds[((tid >> 4) + 16 * i) * RED_STRIDE + (tid & 15)] = r.s[i];
+        }
+    }
+};
+
+// ---- dense row-major operand: element (row, kk) at base[kk*ld_k + row] ------------------------------
+// lanes run along rows (coalesced); the reduction index is wave-uniform and lives in the scalar offset
+struct LoadDenseRow {
+    static constexpr bool RED_MAJOR = false;
+    const float* base;
+    long ld_k;        // elements between consecutive kk
+    int rows;
+    unsigned bytes;   // extent in bytes (below 2 GiB)
+    template <int T> struct Regs { float s[T * KB / NT]; };
+    template <int T> struct State { int vrow; __amdgpu_buffer_rsrc_t rsrc; };
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int row0, int tid, int, int) const {
+        st.rsrc = make_rsrc(base, bytes);
+        const int row = row0 + tid % T;
+        st.vrow = row < rows ? row * 4 : OOB;
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int kk0, int kend, int tid, Regs<T>& r) const {
+        const int kbase = __builtin_amdgcn_readfirstlane(kk0 + tid / T);
+#pragma unroll
+        for (int i = 0; i < T * KB / NT; i++) {
+            const int kk = kbase + (NT / T) * i;
+            const int soff = kk < kend ? (int)((long)kk * ld_k * 4) : 0x7FFFFFF0;
+            r.s[i] = buf_load(st.rsrc, st.vrow, soff);
+        }
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(float* lds, int tid, const Regs<T>& r) {
+#pragma unroll
+        for (int i = 0; i < T * KB / NT; i++) lds[(tid / T + (NT / T) * i) * T + tid % T] = r.s[i];
     }
 };
 

@@ -128,6 +128,7 @@ void Network::construct(vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) {
     for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
         layer[i] = nullptr;
         isOffload[i] = isPrefetched[i] = false;
+        dropSrcAfterFwd[i] = false;
         offloadedSrcData_h[i] = nullptr;
         evFwdDone[i] = evOffloadDone[i] = evBlockFree[i] = evPrefetchDone[i] = nullptr;
     }
@@ -337,13 +338,28 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
     for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
         isOffload[i] = false;
         isPrefetched[i] = false;
+        dropSrcAfterFwd[i] = false;
         if (offloadedSrcData_h[i] != NULL) vdnn_host_free_pinned(ctx, offloadedSrcData_h[i]);
         offloadedSrcData_h[i] = NULL;
-        if (layer[i] != NULL) layer[i]->setVdnnMode(newVdnnType);
+        if (layer[i] != NULL) {
+            layer[i]->setVdnnMode(newVdnnType);
+            layer[i]->setInPlaceOp(false);
+        }
     }
     lastStats.pinnedBytes = 0;
+    /* refined lifetimes: a ReLU layer's input is dead once its forward has run (never layer 0: the
+       network input outlives the step) and its backward runs in place */
+    const bool refined = options.refinedLifetimes && newVdnnType != BASELINE;
+    if (refined) {
+        for (int l = 0; l < numLayers; l++) {
+            if (layer[l]->LayerType() != RELU) continue;
+            layer[l]->setInPlaceOp(true);
+            if (l > 0) dropSrcAfterFwd[l] = true;
+        }
+    }
 
     auto offload = [&](int l) {
+        if (dropSrcAfterFwd[l]) return; /* released, not moved: nothing reads it again */
         isOffload[l] = true;
         const size_t bytes = layer[l]->SrcDataSize() * sizeof(DATATYPE);
         checkVDNN(vdnn_host_alloc_pinned(ctx, (void**)&offloadedSrcData_h[l], bytes));
@@ -517,6 +533,10 @@ int Network::forwardPropagation(bool isDynamic) {
                 lastStats.offloadBytes += layer[l]->SrcDataSize() * sizeof(DATATYPE);
                 ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->SrcData()), isDynamic);
                 if (l == 0) { inputData = nullptr; inputResident = false; }
+            } else if (dropSrcAfterFwd[l]) {
+                /* refined lifetimes: every reader (this layer's forward) is already enqueued */
+                ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->SrcData()), isDynamic);
+                layer[l]->copySrcData(nullptr);
             }
             printUsage("Fwd", l, layer[l]->FwdWorkSpaceSize());
         }
@@ -555,6 +575,18 @@ int Network::backwardPropagation(bool isDynamic) {
                 layer[l]->copyDiffData(layer[l + 1]->GradData());
                 layer[l]->copyDstData(layer[l + 1]->SrcData());
             }
+            /* refined lifetimes: convolution, FC and pooling backward never read their output, so
+               its block (the next layer's srcData) goes back to the pool before anything is
+               allocated for this layer */
+            bool dstReleased = false;
+            if (options.refinedLifetimes && l != numLayers - 1) {
+                const Layer_t t = layer[l]->LayerType();
+                if (is_conv(t) || t == FC_GEMM || t == POOL) {
+                    ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DstData()), isDynamic);
+                    layer[l]->copyDstData(nullptr);
+                    dstReleased = true;
+                }
+            }
             /* this layer reads its own srcData: if that was prefetched, the copy must have landed */
             if (!options.hostSync && isPrefetched[l]) checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evPrefetchDone[l]));
 
@@ -574,9 +606,11 @@ int Network::backwardPropagation(bool isDynamic) {
 
             if (options.hostSync) afterLayerSync();
 
-            /* Release dstData and diffData: every reader is already enqueued on the compute stream */
-            ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DstData()), isDynamic);
-            ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DiffData()), isDynamic);
+            /* Release dstData and diffData: every reader is already enqueued on the compute stream.
+               An in-place ReLU's diffData is its gradData and lives on as the next layer's diffData. */
+            if (!dstReleased) ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DstData()), isDynamic);
+            if (!(layer[l]->InPlaceOp() && layer[l]->GradData() == layer[l]->DiffData()))
+                ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DiffData()), isDynamic);
             printUsage("Bwd", l, layer[l]->BwdDataWorkSpaceSize() + layer[l]->BwdFilterWorkSpaceSize());
         }
         ASSERT_EQ(vdnn_pool_free(ctx, layer[0]->GradData()), isDynamic);

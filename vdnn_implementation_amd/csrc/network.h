@@ -19,6 +19,13 @@ struct NetworkOptions {
                                  // (network.cu:1090-1091, 1168-1169) instead of ordering by events
     bool     capture = false;    // keep host copies of every layer's dstData and gradData
     bool     verbose = false;    // the reference's per-layer printouts
+    // Value-preserving lifetime refinements of the vDNN policies (off = the reference's literal
+    // schedule): (1) a tensor no backward kernel reads is released instead of kept or offloaded:
+    // the input of a ReLU layer, whose backward needs only its output (y > 0 selects the same
+    // elements as x > 0); (2) the output of a convolution, FC or pooling layer is released before
+    // that layer's backward instead of after it (those backward kernels never read y);
+    // (3) a ReLU layer writes dx over dy instead of into a new block.
+    bool     refinedLifetimes = false;
     int      device = DEFAULT_DEVICE;
 };
 
@@ -161,6 +168,7 @@ private:
     Layer*              layer[DEFAULT_NUM_LAYER];
     bool                isOffload[DEFAULT_NUM_LAYER];
     bool                isPrefetched[DEFAULT_NUM_LAYER];
+    bool                dropSrcAfterFwd[DEFAULT_NUM_LAYER]; // refined lifetimes: srcData is dead after forward
     DATATYPE*           offloadedSrcData_h[DEFAULT_NUM_LAYER];
 
     /* Events that order the copy streams against the compute stream (addition) */

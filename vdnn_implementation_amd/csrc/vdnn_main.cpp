@@ -54,6 +54,7 @@ int main(int argc, char** argv) {
         else if (!strcmp(argv[i], "--cap-gb")) opt.capBytes = (size_t)(atof(need("--cap-gb needs a value")) * 1e9);
         else if (!strcmp(argv[i], "--host-sync")) opt.hostSync = true;
         else if (!strcmp(argv[i], "--plan")) opt.planOnly = true;
+        else if (!strcmp(argv[i], "--refined")) opt.refinedLifetimes = true;
         else if (!strcmp(argv[i], "--verbose")) opt.verbose = true;
         else M_ASSERT(0, "unknown flag");
     }

@@ -14,7 +14,7 @@ _ip = C.POINTER(C.c_int32)
 
 class Options(C.Structure):
     _fields_ = [("seed", C.c_uint64), ("pool_bytes", _sz), ("cap_bytes", _sz), ("plan_only", _i), ("host_sync", _i),
-                ("capture", _i), ("verbose", _i), ("device", _i)]
+                ("capture", _i), ("verbose", _i), ("device", _i), ("refined_lifetimes", _i)]
 
 
 class LayerSpec(C.Structure):
@@ -86,11 +86,13 @@ class Network:
     explicit table instead of one of the built-in networks."""
 
     def __init__(self, cnn=None, policy=enums.BASELINE, algo=enums.VDNN_MEMORY_OPT_ALGO, batch=0, layers=None, seed=1,
-                 pool_bytes=0, cap_bytes=0, plan_only=False, host_sync=False, capture=False, verbose=False, device=0):
+                 pool_bytes=0, cap_bytes=0, plan_only=False, host_sync=False, capture=False, verbose=False, device=0,
+                 refined=False):
         o = Options()
         lib.vdnn_network_default_options(C.byref(o))
         o.seed, o.pool_bytes, o.cap_bytes = seed, int(pool_bytes), int(cap_bytes)
         o.plan_only, o.host_sync, o.capture, o.verbose, o.device = int(plan_only), int(host_sync), int(capture), int(verbose), device
+        o.refined_lifetimes = int(refined)
         if layers is not None:
             arr = (LayerSpec * len(layers))(*layers)
             self._h = lib.vdnn_network_create_custom(arr, len(layers), policy, algo, C.byref(o))
