@@ -9,6 +9,7 @@
 // and the tiles exist only in LDS.
 #include "backend_internal.h"
 #include "conv_loaders.h"
+#include "conv_loaders_tap.h"
 #include "conv_smallc.h"
 
 namespace vdnn {
@@ -127,6 +128,15 @@ int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape
     hipStream_t st = stream_of(ctx, stream);
     const int K = g.C * g.R * g.S;
     const unsigned wbytes = (unsigned)((long)g.K * K * 4);
+    if (g.R * g.S <= 32 && g.C % KB == 0) {
+        // blocked tap-major reduction: one slice = one tap x 16 input channels
+        const int RS = g.R * g.S;
+        LoadFilterTap<false> al{w, g.C * RS, RS, g.K, RS, wbytes, FastDiv::make(RS)};
+        LoadIm2colPixTap<0> bl{{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N,
+                                FastDiv::make(RS), FastDiv::make(g.S)}};
+        StoreNCHW ep{y, bias, g.P * g.Q};
+        return launch_by_m(ctx, st, kFwdNames, al, bl, ep, g.K, g.N * g.P * g.Q, K);
+    }
     if (K % 4 == 0 && aligned16(w)) {
         LoadDenseRed<true> al{w, (long)K, g.K, wbytes};
         return conv_fwd_with(ctx, st, g, al, x, bias, y);
@@ -165,6 +175,12 @@ int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* 
     const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S);
     const long sample = (long)g.K * g.P * g.Q;
     if (g.sh == 1 && g.sw == 1) {
+        if (RS <= 32 && g.K % KB == 0) {
+            // blocked tap-major reduction: one slice = one tap x 16 output channels
+            LoadFilterTap<true> alt{w, RS, g.C * RS, g.C, RS, (unsigned)((long)g.K * g.C * RS * 4), dRS};
+            LoadIm2colPixTap<1> bl{{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS}};
+            return launch_by_m(ctx, st, kBwdDataNames, alt, bl, ep, M, N, K);
+        }
         if (RS <= 32) {
             LoadIm2colPix<1, false> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS};
             return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K);
