@@ -91,6 +91,52 @@ def test_conv_random_against_oracle(ctx, geom):
     assert_close(gpu_conv_bwd_bias(ctx, g, dy, b, np.float32(-0.5)), oracle.conv_bwd_bias_sgd(og, dy, b, -0.5), TOL, "bwd bias")
 
 
+PERF_OPT_GEOMS = [
+    (3, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1),
+    (2, 128, 14, 14, 256, 3, 3, 1, 1, 1, 1),
+    (2, 48, 27, 27, 96, 5, 5, 2, 2, 1, 1),
+    (1, 16, 20, 24, 32, 3, 5, 1, 2, 2, 1),     # strided: forward packs, backward data does not
+    (2, 3, 32, 32, 64, 3, 3, 1, 1, 1, 1),      # three input channels: only backward filter has a variant
+    (128, 512, 28, 28, 512, 3, 3, 1, 1, 1, 1), # backward filter asks for more staging than the context owns
+]
+
+
+@pytest.mark.parametrize("geom", PERF_OPT_GEOMS, ids=lambda g: "x".join(map(str, g)))
+def test_conv_perf_opt_variants(ctx, geom):
+    """The workspace-using variants: forward and backward data read a re-laid-out filter bank in the
+    same reduction order, so they return the bits of the workspace-free kernels; backward filter may
+    split the reduction differently and is held to the tolerance against the checker."""
+    rng = np.random.default_rng(hash(geom) % (2 ** 31) + 1)
+    g, og = be.shape(*geom), oracle.shape(*geom)
+    n, c, h, w_, k, r, s_ = geom[:7]
+    filter_bytes = k * c * r * s_ * 4
+    fwd_ok = r * s_ <= 32 and c % 16 == 0
+    bwd_ok = c > 4 and geom[9] == 1 and geom[10] == 1 and r * s_ <= 32 and k % 16 == 0
+    assert lib.vdnn_conv_workspace_bytes(g, 0, 0) == lib.vdnn_conv_workspace_bytes(g, 0, 1) == lib.vdnn_conv_workspace_bytes(g, 0, 2) == 0
+    assert lib.vdnn_conv_workspace_bytes(g, 1, 0) == (filter_bytes if fwd_ok else 0)
+    assert lib.vdnn_conv_workspace_bytes(g, 1, 1) == (filter_bytes if bwd_ok else 0)
+    assert lib.vdnn_conv_workspace_bytes(g, 1, 2) % filter_bytes == 0
+    if geom[0] == 128:
+        assert lib.vdnn_conv_workspace_bytes(g, 1, 2) > (64 << 20)
+    x = rng.standard_normal((g.n, g.c, g.h, g.w)).astype(np.float32)
+    w = (rng.standard_normal((g.k, g.c, g.r, g.s)) * np.sqrt(2.0 / (g.c * g.r * g.s))).astype(np.float32)
+    b = rng.standard_normal(g.k).astype(np.float32)
+    announce("conv perf-opt", geom, "fwd")
+    y0, y1 = gpu_conv_fwd(ctx, g, x, w, b, algo=0), gpu_conv_fwd(ctx, g, x, w, b, algo=1)
+    assert np.array_equal(y0, y1)
+    dy = rng.standard_normal(y0.shape).astype(np.float32)
+    announce("conv perf-opt", geom, "bwd_data")
+    assert np.array_equal(gpu_conv_bwd_data(ctx, g, dy, w, algo=0), gpu_conv_bwd_data(ctx, g, dy, w, algo=1))
+    announce("conv perf-opt", geom, "bwd_filter")
+    zero = np.zeros_like(w)
+    got = gpu_conv_bwd_filter(ctx, g, x, dy, zero, np.float32(1.0), algo=1)
+    if n * c * h * w_ * k <= 2 ** 28:  # sizes the checker finishes in seconds
+        assert_close(got, oracle.conv_bwd_filter_sgd(og, x, dy, zero, 1.0), TOL, "bwd filter")
+        assert_close(y1, oracle.conv_fwd(og, x, w, b), TOL, "fwd")
+    else:
+        assert_close(got, gpu_conv_bwd_filter(ctx, g, x, dy, zero, np.float32(1.0), algo=0), TOL, "bwd filter, two split counts")
+
+
 def test_conv_results_do_not_depend_on_the_run(ctx):
     """Split reductions are ordered: two runs give identical bits."""
     geom = (4, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1)

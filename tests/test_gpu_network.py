@@ -250,3 +250,36 @@ def test_out_of_memory_under_a_cap_returns_minus_one_on_the_device():
         assert np.float32(net.loss()).tobytes() == np.float32(loss_all).tobytes()
     with Network(VGG16_128, VDNN_NONE, VDNN_MEMORY_OPT_ALGO, 4, seed=5, cap_bytes=cap) as net:
         assert net.forwardPropagation(True) == -1
+
+
+def _losses_and_stats(cnn, policy, algo, batch, steps=2, **kw):
+    with Network(cnn, policy, algo, batch, seed=11, **kw) as net:
+        losses = []
+        for _ in range(steps):
+            assert net.forwardPropagation() == 0
+            losses.append(np.float32(net.loss()).tobytes())
+            assert net.backwardPropagation() == 0
+        return losses, net.stats()
+
+
+@pytest.mark.parametrize("cnn,batch,algo,policies", [
+    (OVERFEAT, 128, VDNN_MEMORY_OPT_ALGO, [VDNN_CONV]),                     # OverFeat-fast, batch 128, VDNN_CONV
+    (VGG16_128, 64, VDNN_PERF_OPT_ALGO, [VDNN_ALL]),                        # VGG16, batch 64, VDNN_ALL, workspace kernels
+    (VGG16_128, 128, VDNN_MEMORY_OPT_ALGO, [VDNN_NONE, VDNN_CONV, VDNN_ALL]),  # the four-policy comparison
+], ids=["overfeat128_conv", "vgg16_64_all_perfopt", "vgg16_128_all_policies"])
+def test_full_size_configurations_keep_the_baseline_losses(cnn, batch, algo, policies):
+    """At full size no CPU result is affordable; what must hold at any size: every policy computes the
+    bits BASELINE computes (two steps, so the weight updates are covered), moves the bytes its
+    offload table says, and holds less device memory."""
+    announce("full size", cnn, batch, algo, "BASELINE")
+    base_losses, base_stats = _losses_and_stats(cnn, BASELINE, algo, batch)
+    assert all(np.isfinite(np.frombuffer(b, np.float32)[0]) for b in base_losses)
+    for policy in policies:
+        for refined in (False, True):
+            announce("full size", cnn, batch, algo, "policy", policy, "refined", refined)
+            losses, st = _losses_and_stats(cnn, policy, algo, batch, refined=refined)
+            assert losses == base_losses
+            assert st["offload_bytes"] == st["prefetch_bytes"]
+            if policy != VDNN_NONE:
+                assert st["offload_bytes"] > 0
+                assert st["peak_bytes_in_use"] < base_stats["peak_bytes_in_use"]

@@ -59,6 +59,8 @@ struct PassNames { const char* t64; const char* t128; };
 static const PassNames kFwdNames{"conv_fwd_64x256", "conv_fwd_128x128"};
 static const PassNames kBwdDataNames{"conv_bwd_data_64x256", "conv_bwd_data_128x128"};
 static const PassNames kBwdFilterNames{"conv_bwd_filter_64x256", "conv_bwd_filter_128x128"};
+static const PassNames kFwdPackedNames{"conv_fwd_packed_64x256", "conv_fwd_packed_128x128"};
+static const PassNames kBwdDataPackedNames{"conv_bwd_data_packed_64x256", "conv_bwd_data_packed_128x128"};
 
 template <int TM, int TN, class AL, class BL, class EP>
 static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, const AL& al, const BL& bl, const EP& ep, const GemmDims& d) {
@@ -102,6 +104,26 @@ static int conv_wgrad_with(vdnn_ctx* ctx, hipStream_t st, const AL& al, const BL
                   : launch_igemm<128, 128>(ctx, st, kBwdFilterNames.t128, al, bl, ep, d);
 }
 
+// Workspace planning has no context at hand: it assumes the 256 compute units of the target part.
+constexpr int kPlanningCUs = 256;
+constexpr size_t kDefaultStagingBytes = (size_t)64 << 20;
+constexpr size_t kMaxWgradWorkspace = (size_t)256 << 20;
+
+static bool packed_fwd_ok(const ConvGeo& g) { return g.R * g.S <= 32 && g.C % KB == 0; }
+static bool packed_bwd_data_ok(const ConvGeo& g) {
+    return g.C > 4 && g.sh == 1 && g.sw == 1 && g.R * g.S <= 32 && g.K % KB == 0;
+}
+
+static int launch_pack_filter(vdnn_ctx* ctx, hipStream_t st, const float* w, float* packed, int rows, int Cred, int RS,
+                              int row_stride, int red_stride) {
+    const long total = (long)rows * Cred * RS;
+    ProfScope prof(ctx, st, "conv_pack_filter", 0.0, 8.0 * (double)total);
+    hipLaunchKernelGGL(pack_filter_tap_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, packed, rows, Cred, RS,
+                       row_stride, red_stride, total);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
 } // namespace vdnn
 
 using namespace vdnn;
@@ -112,15 +134,30 @@ size_t vdnn_conv_workspace_bytes(const vdnn_shape_t* shape, int algo_mode, int p
     ConvGeo g;
     if (!shape || !geo_from_shape(shape, g)) return 0;
     if (algo_mode == 0 /* VDNN_MEMORY_OPT_ALGO */) return 0;
-    (void)pass;
-    return 0; // the workspace-using variants are selected per pass below once they exist
+    // Perf-optimal mode: forward and backward data re-lay the filter bank out for 128-bit operand
+    // loads; backward filter takes a staging area large enough for the split count that fills the chip.
+    const int RS = g.R * g.S;
+    const size_t filter_bytes = (size_t)g.K * g.C * RS * sizeof(float);
+    if (pass == 0) return packed_fwd_ok(g) ? filter_bytes : 0;
+    if (pass == 1) return packed_bwd_data_ok(g) ? filter_bytes : 0;
+    const int M = g.K, N = g.C * RS;
+    const bool narrow = M <= 64;
+    const int TM = narrow ? 64 : 128, TN = narrow ? 256 : 128;
+    const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
+    long cap = ((long)g.N * g.P * g.Q + 4 * KB - 1) / (4 * KB);
+    const long by_mem = (long)(kMaxWgradWorkspace / filter_bytes);
+    if (cap > by_mem) cap = by_mem;
+    const int want = choose_splits(tiles, (long)g.N * g.P * g.Q, cap, kPlanningCUs, filter_bytes, 2.0 * TM * TN * KB);
+    if (want <= 1) return 0;
+    const size_t need = (size_t)want * filter_bytes;
+    if (need <= kDefaultStagingBytes) return 0; // the context's own staging area already holds it
+    return need;
 }
 
 int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
                   const float* x, const float* w, const float* bias, float* y,
                   void* workspace, size_t workspace_bytes) {
     VDNN_KERNEL_PROLOGUE(ctx);
-    (void)algo_mode; (void)workspace; (void)workspace_bytes;
     ConvGeo g;
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(x && w && y, "null tensor");
@@ -131,10 +168,18 @@ int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape
     if (g.R * g.S <= 32 && g.C % KB == 0) {
         // blocked tap-major reduction: one slice = one tap x 16 input channels
         const int RS = g.R * g.S;
-        LoadFilterTap<false> al{w, g.C * RS, RS, g.K, RS, wbytes, FastDiv::make(RS)};
         LoadIm2colPixTap<0> bl{{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N,
                                 FastDiv::make(RS), FastDiv::make(g.S)}};
         StoreNCHW ep{y, bias, g.P * g.Q};
+        if (algo_mode == 1 && workspace && workspace_bytes >= wbytes && aligned16(workspace)) {
+            // perf-optimal: the filter bank, re-laid-out in the workspace, is a dense 128-bit operand
+            float* packed = (float*)workspace;
+            const int rc = launch_pack_filter(ctx, st, w, packed, g.K, g.C, RS, g.C * RS, RS);
+            if (rc != VDNN_OK) return rc;
+            LoadDenseRed<true> alp{packed, (long)K, g.K, wbytes};
+            return launch_by_m(ctx, st, kFwdPackedNames, alp, bl, ep, g.K, g.N * g.P * g.Q, K);
+        }
+        LoadFilterTap<false> al{w, g.C * RS, RS, g.K, RS, wbytes, FastDiv::make(RS)};
         return launch_by_m(ctx, st, kFwdNames, al, bl, ep, g.K, g.N * g.P * g.Q, K);
     }
     if (K % 4 == 0 && aligned16(w)) {
@@ -149,7 +194,6 @@ int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* 
                        const float* dy, const float* w, float* dx,
                        void* workspace, size_t workspace_bytes) {
     VDNN_KERNEL_PROLOGUE(ctx);
-    (void)algo_mode; (void)workspace; (void)workspace_bytes;
     ConvGeo g;
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(dy && w && dx, "null tensor");
@@ -177,8 +221,16 @@ int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* 
     if (g.sh == 1 && g.sw == 1) {
         if (RS <= 32 && g.K % KB == 0) {
             // blocked tap-major reduction: one slice = one tap x 16 output channels
-            LoadFilterTap<true> alt{w, RS, g.C * RS, g.C, RS, (unsigned)((long)g.K * g.C * RS * 4), dRS};
+            const unsigned wbytes = (unsigned)((long)g.K * g.C * RS * 4);
             LoadIm2colPixTap<1> bl{{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS}};
+            if (algo_mode == 1 && workspace && workspace_bytes >= wbytes && aligned16(workspace)) {
+                float* packed = (float*)workspace; // [c][(kb*RS + tap)*16 + l]
+                const int rc = launch_pack_filter(ctx, st, w, packed, g.C, g.K, RS, RS, g.C * RS);
+                if (rc != VDNN_OK) return rc;
+                LoadDenseRed<true> alp{packed, (long)K, g.C, wbytes};
+                return launch_by_m(ctx, st, kBwdDataPackedNames, alp, bl, ep, M, N, K);
+            }
+            LoadFilterTap<true> alt{w, RS, g.C * RS, g.C, RS, wbytes, dRS};
             return launch_by_m(ctx, st, kBwdDataNames, alt, bl, ep, M, N, K);
         }
         if (RS <= 32) {
@@ -213,13 +265,11 @@ int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sha
     size_t staging_bytes = ctx->reduce_scratch_bytes;
     if (workspace && workspace_bytes > staging_bytes) { staging = (float*)workspace; staging_bytes = workspace_bytes; }
     const size_t out_bytes = (size_t)M * N * sizeof(float);
-    long want = (4l * ctx->num_cu + tiles - 1) / tiles;
-    const long by_depth = (Kred + 4 * KB - 1) / (4 * KB); // at least four slices per split
-    if (want > by_depth) want = by_depth;
+    long cap = (Kred + 4 * KB - 1) / (4 * KB); // at least four slices per split
     const long by_mem = staging ? (long)(staging_bytes / out_bytes) : 1;
-    if (want > by_mem) want = by_mem;
-    if (want < 1) want = 1;
-    GemmDims d = make_dims(M, N, (int)Kred, TM, TN, (int)want);
+    if (cap > by_mem) cap = by_mem;
+    const int want = choose_splits(tiles, Kred, cap, ctx->num_cu, out_bytes, 2.0 * TM * TN * KB);
+    GemmDims d = make_dims(M, N, (int)Kred, TM, TN, want);
     // one split's samples of dy and of x are addressed through one descriptor with summed offsets
     const long nspan = d.kchunk / PQ + 2;
     VDNN_REQUIRE(nspan * g.K * PQ * 4 < (long)MAX_SUM_RANGE && nspan * g.C * g.H * g.W * 4 < (long)MAX_SUM_RANGE,

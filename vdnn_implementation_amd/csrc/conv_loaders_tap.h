@@ -86,3 +86,21 @@ struct LoadIm2colPixTap {
 };
 
 } // namespace vdnn
+
+namespace vdnn {
+
+// Filter bank re-laid-out for the blocked tap-major order (the workspace of the perf-optimal mode):
+// packed[row][(cb*RS + tap)*16 + l] = w[row*row_stride + (cb*16 + l)*red_stride + tap], so that the A
+// operand becomes a dense reduction-major matrix read with 128-bit loads.
+__global__ void __launch_bounds__(256) pack_filter_tap_kernel(const float* __restrict__ w, float* __restrict__ packed,
+                                                              int rows, int Cred, int RS, int row_stride, int red_stride, long total) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int per_row = Cred * RS;
+    const int row = (int)(i / per_row), kk = (int)(i - (long)row * per_row);
+    const int l = kk & 15, slice = kk >> 4;
+    const int cb = slice / RS, tap = slice - cb * RS;
+    packed[i] = w[(long)row * row_stride + (long)(cb * 16 + l) * red_stride + tap];
+}
+
+} // namespace vdnn

@@ -113,7 +113,7 @@ __global__ void __launch_bounds__(EB) reduce_splits_kernel(float* __restrict__ o
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
                          int splits, float alpha, int accumulate, const float* bias_j, int ncols) {
     ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)count * (splits + 2));
-    hipLaunchKernelGGL(reduce_splits_kernel, dim3(grid_for(count, EB, ctx->num_cu * 8)), dim3(EB), 0, stream,
+    hipLaunchKernelGGL(reduce_splits_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
                        out, partial, count, splits, alpha, accumulate, bias_j, ncols);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
@@ -127,9 +127,23 @@ __global__ void __launch_bounds__(EB) bias_grad_partial_kernel(const float* __re
     const int k = blockIdx.x / splits, sp = blockIdx.x % splits;
     const int n0 = sp * n_per_split, n1 = min(N, n0 + n_per_split);
     float acc = 0.0f;
-    for (int n = n0; n < n1; n++) {
-        const float* p = dy + ((size_t)n * K + k) * PQ;
-        for (int i = threadIdx.x; i < PQ; i += EB) acc += p[i];
+    if ((PQ & 3) == 0 && (((uintptr_t)dy & 15) == 0)) {
+        // 128-bit loads, four independent partial sums per thread (a fixed order, combined below)
+        float4 a4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        const int pq4 = PQ >> 2;
+        for (int n = n0; n < n1; n++) {
+            const float4* p = (const float4*)(dy + ((size_t)n * K + k) * PQ);
+            for (int i = threadIdx.x; i < pq4; i += EB) {
+                const float4 v = p[i];
+                a4.x += v.x; a4.y += v.y; a4.z += v.z; a4.w += v.w;
+            }
+        }
+        acc = (a4.x + a4.y) + (a4.z + a4.w);
+    } else {
+        for (int n = n0; n < n1; n++) {
+            const float* p = dy + ((size_t)n * K + k) * PQ;
+            for (int i = threadIdx.x; i < PQ; i += EB) acc += p[i];
+        }
     }
     acc = block_sum(acc, sh);
     if (threadIdx.x == 0) partial[blockIdx.x] = acc;
@@ -400,7 +414,7 @@ int vdnn_relu_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float
     if (count == 0) return VDNN_OK;
     const size_t n4 = (aligned16(x) && aligned16(y)) ? count / 4 : 0;
     ProfScope prof(ctx, stream_of(ctx, stream), "relu_fwd", 0.0, 8.0 * (double)count);
-    hipLaunchKernelGGL(relu_fwd_kernel, dim3(grid_for(n4 ? n4 : count, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), x, y, n4, count);
+    hipLaunchKernelGGL(relu_fwd_kernel, dim3(grid_for(n4 ? n4 : count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), x, y, n4, count);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
@@ -412,7 +426,7 @@ int vdnn_relu_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float
     if (count == 0) return VDNN_OK;
     const size_t n4 = (aligned16(t) && aligned16(dy) && aligned16(dx)) ? count / 4 : 0;
     ProfScope prof(ctx, stream_of(ctx, stream), "relu_bwd", 0.0, 12.0 * (double)count);
-    hipLaunchKernelGGL(relu_bwd_kernel, dim3(grid_for(n4 ? n4 : count, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), t, dy, dx, n4, count);
+    hipLaunchKernelGGL(relu_bwd_kernel, dim3(grid_for(n4 ? n4 : count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), t, dy, dx, n4, count);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
@@ -421,7 +435,7 @@ int vdnn_sub(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* a, 
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(a && b && r, "null tensor");
     if (count == 0) return VDNN_OK;
-    hipLaunchKernelGGL(sub_kernel, dim3(grid_for(count, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), a, b, r, count);
+    hipLaunchKernelGGL(sub_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), a, b, r, count);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
@@ -430,7 +444,7 @@ int vdnn_fill(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float value, fl
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(p, "null tensor");
     if (count == 0) return VDNN_OK;
-    hipLaunchKernelGGL(fill_kernel, dim3(grid_for(count, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), p, value, count);
+    hipLaunchKernelGGL(fill_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), p, value, count);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
@@ -439,7 +453,7 @@ int vdnn_bias_add(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw, con
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(bias && y && n > 0 && k > 0 && hw > 0, "bad argument");
     const size_t total = (size_t)n * k * hw;
-    hipLaunchKernelGGL(bias_add_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), y, bias, k, hw, total);
+    hipLaunchKernelGGL(bias_add_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), y, bias, k, hw, total);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
@@ -498,10 +512,10 @@ int vdnn_maxpool_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* sh
     ProfScope prof(ctx, st, "maxpool_fwd", 0.0, 4.0 * ((double)g.N * g.C * g.H * g.W + (double)g.N * g.C * g.P * g.Q));
     if (pool_is_2x2_exact(g, x, y, nullptr)) {
         const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
-        hipLaunchKernelGGL(maxpool2x2_fwd_kernel, dim3(grid_for(pairs, EB, ctx->num_cu * 16)), dim3(EB), 0, st, x, y, g.H, g.W, pairs);
+        hipLaunchKernelGGL(maxpool2x2_fwd_kernel, dim3(grid_for(pairs, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, y, g.H, g.W, pairs);
     } else {
         const size_t total = (size_t)g.N * g.C * g.P * g.Q;
-        hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, st, x, y, g, total);
+        hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, y, g, total);
     }
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
@@ -518,10 +532,10 @@ int vdnn_maxpool_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* sh
     ProfScope prof(ctx, st, "maxpool_bwd", 0.0, 4.0 * (2.0 * g.N * g.C * g.H * g.W + (double)g.N * g.C * g.P * g.Q));
     if (pool_is_2x2_exact(g, x, dx, dy) && (g.W / 2) % 2 == 0) {
         const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
-        hipLaunchKernelGGL(maxpool2x2_bwd_kernel, dim3(grid_for(pairs, EB, ctx->num_cu * 16)), dim3(EB), 0, st, x, dy, dx, g.H, g.W, pairs);
+        hipLaunchKernelGGL(maxpool2x2_bwd_kernel, dim3(grid_for(pairs, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g.H, g.W, pairs);
     } else {
         const size_t total = (size_t)g.N * g.C * g.H * g.W;
-        hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, st, x, dy, dx, g, total);
+        hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g, total);
     }
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
@@ -532,7 +546,7 @@ int vdnn_lrn_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, cons
     VDNN_REQUIRE(x && y && n > 0 && c > 0 && hw > 0, "bad argument");
     const size_t total = (size_t)n * c * hw;
     ProfScope prof(ctx, stream_of(ctx, stream), "lrn_fwd", 0.0, 8.0 * (double)total);
-    hipLaunchKernelGGL(lrn_fwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), x, y, c, hw, total);
+    hipLaunchKernelGGL(lrn_fwd_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), x, y, c, hw, total);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
@@ -542,7 +556,7 @@ int vdnn_lrn_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, cons
     VDNN_REQUIRE(x && y && dy && dx && n > 0 && c > 0 && hw > 0, "bad argument");
     const size_t total = (size_t)n * c * hw;
     ProfScope prof(ctx, stream_of(ctx, stream), "lrn_bwd", 0.0, 16.0 * (double)total);
-    hipLaunchKernelGGL(lrn_bwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream), x, y, dy, dx, c, hw, total);
+    hipLaunchKernelGGL(lrn_bwd_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), x, y, dy, dx, c, hw, total);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
@@ -585,7 +599,7 @@ int vdnn_softmax_ce_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes,
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(prob && labels && dlogits && n > 0 && classes > 0, "bad argument");
     const size_t total = (size_t)n * classes;
-    hipLaunchKernelGGL(softmax_ce_bwd_kernel, dim3(grid_for(total, EB, ctx->num_cu * 16)), dim3(EB), 0, stream_of(ctx, stream),
+    hipLaunchKernelGGL(softmax_ce_bwd_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream),
                        prob, labels, dlogits, classes, 1.0f / (float)n, total);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;

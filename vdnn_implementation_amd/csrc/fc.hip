@@ -17,12 +17,10 @@ static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const char* name, const AL& al
                    float* out, float alpha, int accumulate, const float* bias_j) {
     const int TM = M <= 64 ? 64 : 128, TN = M <= 64 ? 256 : 128;
     const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
-    long want = (4l * ctx->num_cu + tiles - 1) / tiles;
-    const long by_depth = ((long)K + 8 * KB - 1) / (8 * KB);
-    if (want > by_depth) want = by_depth;
+    long cap = ((long)K + 8 * KB - 1) / (8 * KB); // at least eight slices per split
     const long by_mem = (long)(ctx->reduce_scratch_bytes / ((size_t)M * N * sizeof(float)));
-    if (want > by_mem) want = by_mem;
-    if (want < 1) want = 1;
+    if (cap > by_mem) cap = by_mem;
+    const long want = choose_splits(tiles, K, cap, ctx->num_cu, (size_t)M * N * sizeof(float), 2.0 * TM * TN * KB);
     GemmDims d;
     d.M = M; d.N = N; d.K = K;
     d.mtiles = (M + TM - 1) / TM; d.ntiles = (N + TN - 1) / TN;

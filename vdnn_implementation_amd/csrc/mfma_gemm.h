@@ -137,6 +137,32 @@ struct GemmDims {
     int mtiles, ntiles, splits, kchunk;
 };
 
+// Number of reduction splits for a grid of `tiles` output tiles over a reduction of K, at most
+// max_splits. Measured on the part: workgroups are resident three to a compute unit, so a grid runs
+// fastest when it is a little under a multiple of the unit count, best a multiple of three units'
+// worth; one more workgroup than that starts a nearly empty round. The estimate below counts, per
+// compute unit, rounds x (slices per split + a fixed prologue/epilogue) with the measured efficiency
+// of a round count, plus the traffic of writing and re-reading one partial result per split.
+static inline int choose_splits(long tiles, long K, long max_splits, int num_cu, size_t out_bytes, double tile_flops_per_slice) {
+    if (max_splits < 1) max_splits = 1;
+    const long useful = 12l * num_cu / tiles + 1; // beyond twelve rounds the estimate only grows
+    if (max_splits > useful) max_splits = useful;
+    const double us_per_slice = tile_flops_per_slice / (118e6 / num_cu); // one unit at ~118 TFLOP/s / units
+    const double us_per_split = (double)out_bytes * 2.0 / 4e6;           // partials at ~4 TB/s
+    double best = 0.0;
+    int best_s = 1;
+    for (long s = 1; s <= max_splits; s++) {
+        long kchunk = (K + s - 1) / s;
+        kchunk = (kchunk + KB - 1) / KB * KB;
+        const long splits = (K + kchunk - 1) / kchunk;
+        const long rounds = (tiles * splits + num_cu - 1) / num_cu;
+        const double eff = rounds == 1 ? 0.72 : rounds == 2 ? 0.92 : rounds == 4 ? 0.93 : rounds % 3 == 0 ? 1.0 : 0.97;
+        const double cost = (double)rounds * (double)(kchunk / KB + 6) * us_per_slice / eff + (splits > 1 ? (double)splits * us_per_split : 0.0);
+        if (s == 1 || cost < best) { best = cost; best_s = (int)s; }
+    }
+    return best_s;
+}
+
 template <int TM, int TN, class AL, class BL, class EP>
 __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, const EP ep, const GemmDims d) {
     static_assert(TM % 64 == 0 && TN % 64 == 0 && (TM / 64) * (TN / 64) == 4, "four 64x64 wave tiles");
