@@ -22,6 +22,18 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
 FLOP_PER_IMAGE = 92.82e9  # 3 passes over 13 convolutions and 3 FC layers
 
+# Memory traffic per launch (bytes fetched into L2 plus bytes written back, averaged over a class's
+# launches in one step) of the three large convolution classes at the default workload (batch 128,
+# memory-optimal mode). Hardware counters cannot be read from inside this script: the figures come
+# from two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), whose summary is
+# kept under profiles/. FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0: what the same counters
+# read for the ReLU kernels of the same run, which move a known number of bytes.
+MEASURED_TRAFFIC_BYTES = {
+    "conv_fwd_128x128": 953.6e6,
+    "conv_bwd_data_128x128": 876.8e6,
+    "conv_bwd_filter_128x128": 1172.2e6,
+}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -113,8 +125,14 @@ def main():
 
     head = "VDNN_ALL" if "VDNN_ALL" in results else list(results)[0]
     base = results.get("BASELINE")
-    # dominant kernel: the convolution class with the most device time under the headline policy
-    prof = profiles[head]
+    # dominant kernel: the convolution class with the most device time over the timed steps of all
+    # policies of this run (the same launches a kernel trace of this command sees, warm-up aside)
+    prof = {}
+    for p in profiles.values():
+        for k, v in p.items():
+            acc = prof.setdefault(k, {"launches": 0, "ms": 0.0, "flops": 0.0, "bytes": 0.0})
+            for field in acc:
+                acc[field] += v[field]
     conv = {k: v for k, v in prof.items() if k.startswith("conv_") and v["flops"] > 0}
     prof = {k: v for k, v in prof.items() if v["ms"] > 0}
     dom = max(conv, key=lambda k: conv[k]["ms"])
@@ -142,7 +160,10 @@ def main():
         "losses_bit_identical": len({results[k]["loss"] for k in results}) == 1,
         "conv_mfma_util": conv_all_tf / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom) if args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" else None,
+                     "traffic_unit": "bytes per launch (L2 fetch + write-back, counters scaled by a known-size kernel)",
+                     "algorithmic_flop_per_launch": d["flops"] / d["launches"],
                      "avg_launch_ms": d["ms"] / d["launches"], "launches": d["launches"]},
         "kernels": kernels,
         "step_mfma_frac": args.batch * FLOP_PER_IMAGE / (results[head]["ms_per_step"] * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
