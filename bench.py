@@ -39,8 +39,8 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False):
-    net = Network(cnn, policy, algo, batch, seed=seed, refined=refined)
+def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0):
+    net = Network(cnn, policy, algo, batch, seed=seed, refined=refined, cap_bytes=cap_bytes)
     try:
         for _ in range(warmup):
             assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
@@ -100,6 +100,7 @@ def main():
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--algo", default="VDNN_MEMORY_OPT_ALGO")
     ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined")
+    ap.add_argument("--cap-gb", type=float, default=0.0, help="artificial limit on pool bytes in use (0 = none)")
     ap.add_argument("--cpu-batch", type=int, default=24)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -119,7 +120,7 @@ def main():
         _, policy, algo = parse("VGG16_128", word, args.algo)
         log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
         results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1,
-                                                   refined=(suffix == "refined"))
+                                                   refined=(suffix == "refined"), cap_bytes=int(args.cap_gb * 1e9))
         log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
             results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))
 

@@ -64,6 +64,9 @@ CONV_RANDOM = [
     (5, 64, 6, 6, 200, 6, 6, 0, 0, 1, 1),      # OverFeat 6x6 -> 1x1
     (9, 300, 1, 1, 150, 1, 1, 0, 0, 1, 1),     # OverFeat 1x1 on 1x1
     (1, 16, 20, 24, 32, 3, 5, 1, 2, 2, 1),     # asymmetric everything
+    (2, 4, 17, 19, 8, 3, 3, 1, 1, 2, 2),       # four input channels, strided: the vector-ALU filter gradient
+    (3, 1, 9, 9, 12, 3, 3, 0, 0, 1, 1),        # one input channel, no padding
+    (7, 3, 40, 36, 16, 3, 3, 1, 1, 1, 1),      # three input channels, several pixel chunks per sample
 ]
 
 

@@ -256,6 +256,33 @@ int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sha
     const int M = g.K, N = g.C * g.R * g.S, PQ = g.P * g.Q, RS = g.R * g.S;
     const long Kred = (long)g.N * PQ;
     VDNN_REQUIRE(Kred < (1l << 31), "reduction too long");
+    if (g.C <= 4 && g.R == 3 && g.S == 3 && g.K % 4 == 0 && ctx->reduce_scratch) {
+        // few input channels: vector-ALU kernel over chunks of output pixels, then the ordered chunk sum
+        const long total = Kred;
+        const size_t out_bytes = (size_t)M * N * sizeof(float);
+        long chunks = (total + 256 * 96 - 1) / (256 * 96);
+        const long by_mem = (long)(ctx->reduce_scratch_bytes / out_bytes);
+        if (chunks > by_mem) chunks = by_mem;
+        if (chunks < 1) chunks = 1;
+        long per = (total + chunks - 1) / chunks;
+        per = (per + 255) / 256 * 256;
+        chunks = (total + per - 1) / per;
+        const long blocks = chunks * (g.K / 4);
+        VDNN_REQUIRE(blocks < (1l << 31), "grid too large");
+        const PixelStep step{256 / PQ, (256 % PQ) / g.Q, (256 % PQ) % g.Q};
+        float* staging = ctx->reduce_scratch;
+        {
+            ProfScope prof(ctx, st, "conv_bwd_filter_smallc", 2.0 * (double)M * N * (double)Kred, 0.0);
+            switch (g.C) {
+            case 1: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<1, 4>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
+            case 2: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<2, 4>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
+            case 3: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<3, 4>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
+            default: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<4, 4>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
+            }
+            VDNN_LAUNCH_CHECK();
+        }
+        return launch_reduce_splits(ctx, st, w, staging, (size_t)M * N, (int)chunks, alpha, 1, nullptr, 0);
+    }
     // Split the (n,p,q) reduction so the grid fills the chip; partial sums go to a staging area and
     // are added in split order by a second kernel (no floating-point atomics).
     const bool narrow = M <= 64;

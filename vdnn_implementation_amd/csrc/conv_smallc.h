@@ -134,4 +134,93 @@ __global__ void __launch_bounds__(256) conv_bwd_data_smallc_s1_kernel(const floa
     for (int c = 0; c < CC; c++) o[c * plane] = acc[c];
 }
 
+// ---- backward filter for 3x3 layers with at most four input channels ------------------------------
+// The implicit GEMM has only C*9 <= 36 columns, which would fill a tenth of a 256-wide MFMA tile, and
+// the pass is bound by reading dy once. Lanes run along output pixels (coalesced dy and x reads); one
+// thread keeps the C*9 products of KG output channels in registers, walks its share of one chunk of
+// pixels, and the workgroup's sums go to partial[chunk][k][c][tap] in a fixed order (wavefront
+// shuffle tree, then the four wavefronts in order). The chunks are added in order by the split
+// reduction that also applies the SGD step.
+struct PixelStep { int dn, dp, dq; }; // 256 pixels = dn samples + dp rows + dq columns
+
+template <int CC, int KG>
+__global__ void __launch_bounds__(256) conv_bwd_filter_smallc3x3_kernel(const float* __restrict__ dy, const float* __restrict__ x,
+                                                                        float* __restrict__ partial, const ConvGeo g,
+                                                                        long pix_per_chunk, PixelStep step) {
+    constexpr int TAPS = CC * 9;
+    __shared__ float red[4][KG * TAPS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kgroups = g.K / KG;
+    const int kg = blockIdx.x % kgroups;
+    const long chunk = blockIdx.x / kgroups;
+    const long total = (long)g.N * g.P * g.Q;
+    const long pix0 = chunk * pix_per_chunk;
+    const long pix1 = pix0 + pix_per_chunk < total ? pix0 + pix_per_chunk : total;
+    const int PQ = g.P * g.Q;
+    long pix = pix0 + tid;
+    int n = (int)(pix / PQ);
+    int rem = (int)(pix - (long)n * PQ);
+    int p = rem / g.Q, q = rem - p * g.Q;
+
+    float acc[KG][TAPS];
+#pragma unroll
+    for (int j = 0; j < KG; j++)
+#pragma unroll
+        for (int t = 0; t < TAPS; t++) acc[j][t] = 0.0f;
+
+    const long plane = (long)g.H * g.W;
+    for (; pix < pix1; pix += 256) {
+        const int ih0 = p * g.sh - g.ph, iw0 = q * g.sw - g.pw;
+        const float* xs = x + (long)n * CC * plane;
+        float xv[TAPS];
+#pragma unroll
+        for (int r = 0; r < 3; r++) {
+            const int ih = ih0 + r;
+            const bool vr = (unsigned)ih < (unsigned)g.H;
+            const int ihc = vr ? ih : 0;
+#pragma unroll
+            for (int t = 0; t < 3; t++) {
+                const int iw = iw0 + t;
+                const bool v = vr & ((unsigned)iw < (unsigned)g.W);
+                const int iwc = ((unsigned)iw < (unsigned)g.W) ? iw : 0;
+#pragma unroll
+                for (int c = 0; c < CC; c++) {
+                    const float val = xs[c * plane + (long)ihc * g.W + iwc];
+                    xv[c * 9 + r * 3 + t] = v ? val : 0.0f;
+                }
+            }
+        }
+        const float* dyp = dy + ((long)n * g.K + kg * KG) * PQ + p * g.Q + q;
+#pragma unroll
+        for (int j = 0; j < KG; j++) {
+            const float d = dyp[(long)j * PQ];
+#pragma unroll
+            for (int t = 0; t < TAPS; t++) acc[j][t] += d * xv[t];
+        }
+        // advance 256 pixels
+        q += step.dq;
+        const int cq = q >= g.Q;
+        q -= cq ? g.Q : 0;
+        p += step.dp + cq;
+        const int cp = p >= g.P;
+        p -= cp ? g.P : 0;
+        n += step.dn + cp;
+    }
+
+#pragma unroll
+    for (int j = 0; j < KG; j++)
+#pragma unroll
+        for (int t = 0; t < TAPS; t++) {
+            float v = acc[j][t];
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+            if (lane == 0) red[wave][j * TAPS + t] = v;
+        }
+    __syncthreads();
+    if (tid < KG * TAPS) {
+        const float v = ((red[0][tid] + red[1][tid]) + red[2][tid]) + red[3][tid];
+        partial[chunk * ((long)g.K * TAPS) + (long)kg * KG * TAPS + tid] = v;
+    }
+}
+
 } // namespace vdnn
