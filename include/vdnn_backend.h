@@ -137,6 +137,16 @@ int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sha
                              const float* x, const float* dy, float* w, float alpha,
                              void* workspace, size_t workspace_bytes);
 
+/* The same two reductions with the optimizer step left out: db[k] = sum dy, dw = sum dy*x (beta = 0).
+ * The reference always fuses SGD into these calls (alpha=-lr, beta=1); a training loop that keeps
+ * gradients (to average them over devices, or to apply another optimizer) needs them separately.
+ * vdnn_sgd_apply then evaluates param += alpha * grad with the arithmetic of the fused calls, so
+ * the two routes give the same bits. */
+int vdnn_conv_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* dy, float* db);
+int vdnn_conv_bwd_filter(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                         const float* x, const float* dy, float* dw, void* workspace, size_t workspace_bytes);
+int vdnn_sgd_apply(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float alpha, const float* grad, float* param);
+
 /* ---- fully connected (replaces cuBLAS: layer.cu:667-764) ------------------------------------- */
 /* Sgemm(T,N) + rank-1 bias broadcast (layer.cu:677-706): y[n,o] = sum_i w[o,i] x[n,i] + bias[o].
  * w is [c_out][c_in] row-major. */
@@ -151,6 +161,10 @@ int vdnn_fc_bwd_weight_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in,
 /* Sgemm with a ones vector, alpha=-lr beta=1 (layer.cu:747-761): bias[o] += alpha * sum_n dy[n,o]. */
 int vdnn_fc_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out,
                          const float* dy, float* bias, float alpha);
+/* The two FC reductions without the optimizer step (see vdnn_conv_bwd_filter). */
+int vdnn_fc_bwd_weight(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                       const float* x, const float* dy, float* dw);
+int vdnn_fc_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const float* dy, float* db);
 
 /* ---- bandwidth-bound layers (replaces cuDNN: layer.cu:766-915) -------------------------------- */
 /* cudnnActivationForward, ReLU, NaN propagates (layer.cu:774-781, 380-385): y = x > 0 ? x : (x!=x ? x : 0). */
@@ -159,6 +173,13 @@ int vdnn_relu_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float
  * y > 0, which selects the same elements. */
 int vdnn_relu_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, const float* y,
                   const float* dy, float* dx);
+/* cudnnActivationForward/Backward with CUDNN_ACTIVATION_TANH / CUDNN_ACTIVATION_SIGMOID (mode chosen from
+ * the layer type at layer.cu:362-369; same call sites as ReLU, layer.cu:774-781, 802-811):
+ * y = tanh(x), dx = dy (1 - y^2); y = 1 / (1 + exp(-x)), dx = dy y (1 - y). Backward reads y, not x. */
+int vdnn_tanh_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y);
+int vdnn_tanh_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* y, const float* dy, float* dx);
+int vdnn_sigmoid_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y);
+int vdnn_sigmoid_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* y, const float* dy, float* dx);
 /* cudnnPoolingForward, max, NaN not propagated (layer.cu:875-882, 416-428). Window r x s. */
 int vdnn_maxpool_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* x, float* y);
 /* cudnnPoolingBackward (layer.cu:903-912): each window's dy goes to its first maximum in row-major

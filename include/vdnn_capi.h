@@ -25,6 +25,8 @@ typedef struct {
     int      verbose;
     int      device;
     int      refined_lifetimes; /* value-preserving lifetime refinements of the vDNN policies (0 = literal schedule) */
+    int      unfused_optimizer; /* keep dW / db per layer and step after backward instead of inside it (same bits) */
+    int      defer_optimizer;   /* with unfused_optimizer: backward leaves the step to vdnn_network_apply_gradients */
 } vdnn_network_options;
 
 typedef struct {
@@ -65,6 +67,11 @@ void vdnn_network_set_labels(vdnn_network* net, const int32_t* labels);
 void vdnn_network_set_label_tensor(vdnn_network* net, const float* host);
 int  vdnn_network_set_layer_params(vdnn_network* net, int l, const float* filter, const float* bias);
 int  vdnn_network_get_layer_params(vdnn_network* net, int l, float* filter, float* bias);
+/* unfused optimizer (no counterpart in the reference, which fuses SGD into backward: layer.cu:651-660, 736-761) */
+int  vdnn_network_get_layer_gradients(vdnn_network* net, int l, float* filter, float* bias);
+int  vdnn_network_apply_gradients(vdnn_network* net);
+/* `steps` training steps; writes the loss seen by each step's forward into losses[0..return) */
+int  vdnn_network_train(vdnn_network* net, int steps, int is_dynamic, float* losses);
 size_t vdnn_network_filter_count(vdnn_network* net, int l);
 size_t vdnn_network_bias_count(vdnn_network* net, int l);
 /* host copies taken during the last step when options.capture is set; returns the element count */

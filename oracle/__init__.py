@@ -66,6 +66,10 @@ _sig("orc_fc_bwd_weight_sgd", None, C.c_int, C.c_int, C.c_int, _f, _f, _f, C.c_f
 _sig("orc_fc_bwd_bias_sgd", None, C.c_int, C.c_int, _f, _f, C.c_float)
 _sig("orc_relu_fwd", None, C.c_size_t, _f, _f)
 _sig("orc_relu_bwd", None, C.c_size_t, _f, _f, _f, _f)
+for _name in ("orc_tanh_fwd", "orc_sigmoid_fwd"):
+    _sig(_name, None, C.c_size_t, _f, _f)
+for _name in ("orc_tanh_bwd", "orc_sigmoid_bwd"):
+    _sig(_name, None, C.c_size_t, _f, _f, _f)
 _sig("orc_maxpool_fwd", None, _S, _f, _f)
 _sig("orc_maxpool_bwd", None, _S, _f, _f, _f, _f)
 _sig("orc_lrn_fwd", None, C.c_int, C.c_int, C.c_int, _f, _f)
@@ -212,6 +216,36 @@ def relu_bwd(x, y, dy):
     dx = np.empty_like(dy)
     lib.orc_relu_bwd(dy.size, _p(x), _p(y), _p(dy), _p(dx))
     return dx
+
+
+def _act_fwd(fn, x):
+    x = _f32(x)
+    y = np.empty_like(x)
+    fn(x.size, _p(x), _p(y))
+    return y
+
+
+def _act_bwd(fn, y, dy):
+    y, dy = _f32(y), _f32(dy)
+    dx = np.empty_like(dy)
+    fn(dy.size, _p(y), _p(dy), _p(dx))
+    return dx
+
+
+def tanh_fwd(x):
+    return _act_fwd(lib.orc_tanh_fwd, x)
+
+
+def tanh_bwd(y, dy):
+    return _act_bwd(lib.orc_tanh_bwd, y, dy)
+
+
+def sigmoid_fwd(x):
+    return _act_fwd(lib.orc_sigmoid_fwd, x)
+
+
+def sigmoid_bwd(y, dy):
+    return _act_bwd(lib.orc_sigmoid_bwd, y, dy)
 
 
 def pool_out_shape(g):

@@ -397,6 +397,32 @@ void orc_relu_bwd(size_t count, const float* x, const float* y, const float* dy,
 }
 
 /* ---------------------------------------------------------------------------------------------
+ * tanh and sigmoid: cudnnActivationForward/Backward with CUDNN_ACTIVATION_TANH / _SIGMOID, selected
+ * by the layer type at layer.cu:362-369 and run through the same two call sites as ReLU
+ * (layer.cu:774-781, 802-811). Backward uses the output only: tanh' = 1 - y^2, sigmoid' = y (1 - y).
+ * Evaluated in double and rounded once.
+ * ------------------------------------------------------------------------------------------- */
+void orc_tanh_fwd(size_t count, const float* x, float* y) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) y[i] = (float)tanh((double)x[i]);
+}
+
+void orc_tanh_bwd(size_t count, const float* y, const float* dy, float* dx) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) dx[i] = (float)((double)dy[i] * (1.0 - (double)y[i] * (double)y[i]));
+}
+
+void orc_sigmoid_fwd(size_t count, const float* x, float* y) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) y[i] = (float)(1.0 / (1.0 + exp(-(double)x[i])));
+}
+
+void orc_sigmoid_bwd(size_t count, const float* y, const float* dy, float* dx) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) dx[i] = (float)((double)dy[i] * (double)y[i] * (1.0 - (double)y[i]));
+}
+
+/* ---------------------------------------------------------------------------------------------
  * Max pooling: CUDNN_POOLING_MAX, NOT_PROPAGATE_NAN (layer.cu:416-428, 875-882, 903-912).
  * Padding positions never win. Backward: dy of each window goes to the window's first maximum in
  * row-major order (PARITY UNPINNED tie rule, see header); windows are visited in row-major order

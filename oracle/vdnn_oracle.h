@@ -14,6 +14,8 @@
  *   bias add / bias grad / sub / fill: closed form
  *   fc fwd / bwd-data / bwd-weight   : numpy matmul
  *   relu                             : closed form incl. -0, NaN, inf
+ *   tanh / sigmoid fwd / bwd         : torch.tanh / torch.sigmoid + autograd in float64, special values,
+ *                                      the identities tanh(-x) = -tanh(x), sigmoid(x) + sigmoid(-x) = 1
  *   maxpool fwd / bwd                : torch max_pool2d + autograd fixtures on tie-free data
  *                                      (3x3 s2 overlapping and 2x2 s2); brute force.
  *                                      TIE RULE OF maxpool bwd: PARITY UNPINNED (cuDNN closed, no
@@ -74,6 +76,10 @@ void orc_fc_bwd_bias_sgd(int n, int c_out, const float* dy, float* bias, float a
 /* layer.cu:774-781, 802-811 */
 void orc_relu_fwd(size_t count, const float* x, float* y);
 void orc_relu_bwd(size_t count, const float* x, const float* y, const float* dy, float* dx);
+void orc_tanh_fwd(size_t count, const float* x, float* y);
+void orc_tanh_bwd(size_t count, const float* y, const float* dy, float* dx);
+void orc_sigmoid_fwd(size_t count, const float* x, float* y);
+void orc_sigmoid_bwd(size_t count, const float* y, const float* dy, float* dx);
 /* layer.cu:875-882, 903-912 */
 void orc_maxpool_fwd(const orc_shape* g, const float* x, float* y);
 void orc_maxpool_bwd(const orc_shape* g, const float* x, const float* y, const float* dy, float* dx);

@@ -7,7 +7,7 @@
 #include <stdlib.h>
 #include <string.h>
 
-enum { T_FC_GEMM = 0, T_CONV = 1, T_FC_CONV = 2, T_RELU = 3, T_SOFTMAX = 6, T_POOL = 7, T_LRN = 10 };
+enum { T_FC_GEMM = 0, T_CONV = 1, T_FC_CONV = 2, T_RELU = 3, T_TANH = 4, T_SIGMOID = 5, T_SOFTMAX = 6, T_POOL = 7, T_LRN = 10 };
 #define ORC_MAX_LAYERS 64
 #define ORC_LR 1e-5 /* vdnn.h:8 */
 
@@ -206,6 +206,8 @@ float orc_net_forward(orc_net* net) {
         case T_FC_GEMM: orc_fc_fwd(d->g.n, d->g.c, d->g.k, src, net->filter[l], net->bias[l], dst); break;
         case T_CONV: case T_FC_CONV: orc_conv_fwd(&d->g, src, net->filter[l], net->bias[l], dst); break;
         case T_RELU: orc_relu_fwd(src_count(d), src, dst); break;
+        case T_TANH: orc_tanh_fwd(src_count(d), src, dst); break;
+        case T_SIGMOID: orc_sigmoid_fwd(src_count(d), src, dst); break;
         case T_LRN: orc_lrn_fwd(d->g.n, d->g.c, d->g.h * d->g.w, src, dst); break;
         case T_POOL: orc_maxpool_fwd(&d->g, src, dst); break;
         case T_SOFTMAX: orc_softmax_fwd(d->g.n, d->g.c * d->g.h * d->g.w, src, dst); break;
@@ -244,6 +246,8 @@ void orc_net_backward(orc_net* net) {
             orc_conv_bwd_filter_sgd(&d->g, src, diff, net->filter[l], alpha);
             break;
         case T_RELU: orc_relu_bwd(src_count(d), src, dst, diff, grad); break;
+        case T_TANH: orc_tanh_bwd(src_count(d), dst, diff, grad); break;
+        case T_SIGMOID: orc_sigmoid_bwd(src_count(d), dst, diff, grad); break;
         case T_LRN: orc_lrn_bwd(d->g.n, d->g.c, d->g.h * d->g.w, src, dst, diff, grad); break;
         case T_POOL: orc_maxpool_bwd(&d->g, src, dst, diff, grad); break;
         case T_SOFTMAX: orc_softmax_bwd(d->g.n, d->g.c * d->g.h * d->g.w, dst, diff, grad); break;

@@ -220,6 +220,24 @@ def test_relu_is_exact(ctx, count):
     assert np.array_equal(gdx2, wdx)  # from y alone: same elements selected
 
 
+@pytest.mark.parametrize("count", [1, 5, 4096 * 9 + 3])
+def test_tanh_and_sigmoid(ctx, count):
+    rng = np.random.default_rng(count)
+    x = (rng.standard_normal(count) * 3).astype(np.float32)
+    x[: min(count, 4)] = np.array([0.0, 30.0, -30.0, -0.0], np.float32)[: min(count, 4)]
+    dy = rng.standard_normal(count).astype(np.float32)
+    for name, fwd, bwd in (("tanh", oracle.tanh_fwd, oracle.tanh_bwd), ("sigmoid", oracle.sigmoid_fwd, oracle.sigmoid_bwd)):
+        announce(name, count)
+        with Dev(ctx) as d:
+            dx_, ddy, y, gx = d.up(x), d.up(dy), d.empty((count,)), d.empty((count,))
+            check(getattr(lib, "vdnn_%s_fwd" % name)(ctx.handle, None, count, dx_.ptr, y.ptr))
+            check(getattr(lib, "vdnn_%s_bwd" % name)(ctx.handle, None, count, y.ptr, ddy.ptr, gx.ptr))
+            got_y, got_dx = y.download((count,)), gx.download((count,))
+        # float32 library functions against the checker's double evaluation: a few units in the last place
+        assert_close(got_y, fwd(x), 1e-6, name + " forward")
+        assert_close(got_dx, bwd(got_y, dy), 1e-6, name + " backward")
+
+
 POOLS = [(2, 3, 13, 15, 3, 2), (2, 3, 12, 12, 2, 2), (1, 2, 7, 9, 2, 2), (3, 5, 8, 16, 2, 2), (2, 4, 27, 27, 3, 2), (1, 2, 6, 10, 2, 2)]
 
 

@@ -120,6 +120,10 @@ def layer_forward_on_checker(spec, src, w, b):
         return oracle.fc_fwd(src.reshape(spec.n, -1), w.reshape(spec.k, -1), b).reshape(spec.n, spec.k, 1, 1)
     if t == enums.RELU:
         return oracle.relu_fwd(src)
+    if t == enums.TANH:
+        return oracle.tanh_fwd(src)
+    if t == enums.SIGMOID:
+        return oracle.sigmoid_fwd(src)
     if t == enums.LRN:
         return oracle.lrn_fwd(src)
     if t == enums.POOL:
@@ -142,6 +146,10 @@ def layer_backward_on_checker(spec, src, dst, dy, w, b):
                 oracle.fc_bwd_bias_sgd(dy2, b, alpha))
     if t == enums.RELU:
         return oracle.relu_bwd(src, dst, dy), None, None
+    if t == enums.TANH:
+        return oracle.tanh_bwd(dst, dy), None, None
+    if t == enums.SIGMOID:
+        return oracle.sigmoid_bwd(dst, dy), None, None
     if t == enums.LRN:
         return oracle.lrn_bwd(src, dst, dy), None, None
     if t == enums.POOL:
@@ -158,17 +166,38 @@ def layer_backward_on_checker(spec, src, dst, dy, w, b):
     (VGG16_128, 1, VDNN_ALL, VDNN_PERF_OPT_ALGO),
 ])
 def test_reference_networks_against_the_checker(cnn, batch, policy, algo):
+    check_network_against_the_checker(cnn, batch, policy, algo)
+
+
+def smooth_specs(n=3):
+    """A table with the two activation modes none of the reference's networks uses (layer.cu:362-369)."""
+    return [layer_spec(enums.FC_CONV, n, 3, 16, 16, 1, 1, 8, 3), layer_spec(enums.TANH, n, 8, 16, 16),
+            layer_spec(enums.POOL, n, 8, 16, 16, 0, 2, 0, 2), layer_spec(enums.FC_CONV, n, 8, 8, 8, 1, 1, 16, 3),
+            layer_spec(enums.SIGMOID, n, 16, 8, 8), layer_spec(enums.FC_GEMM, n, 1024, 1, 1, 0, 0, 24, 1),
+            layer_spec(enums.TANH, n, 24, 1, 1), layer_spec(enums.FC_GEMM, n, 24, 1, 1, 0, 0, 10, 1),
+            layer_spec(enums.SOFTMAX, n, 10, 1, 1)]
+
+
+@pytest.mark.parametrize("policy,refined", [(BASELINE, False), (VDNN_ALL, False), (VDNN_ALL, True)])
+def test_tanh_and_sigmoid_layers_against_the_checker(policy, refined):
+    check_network_against_the_checker(None, 3, policy, VDNN_MEMORY_OPT_ALGO, layers=smooth_specs(3), refined=refined)
+
+
+def check_network_against_the_checker(cnn, batch, policy, algo, layers=None, refined=False):
     """Layer by layer on identical inputs: each layer's output and gradients, computed by the checker
     from the tensors the GPU run fed that layer, within 1e-4 relative (max norm); exact for ReLU and
     max-pool. End to end (where a ReLU or pooling decision that flips on a last-bit difference moves
     single elements by O(1)) the loss must agree to 1e-4 and the input gradient to 2e-2 in L2."""
     seed = 11
-    o = oracle.Net(cnn=cnn, batch=batch)
+    o = oracle.Net(cnn=cnn, batch=batch) if layers is None else oracle.Net(layers=[
+        oracle.LayerDesc(s.type, oracle.Shape(s.n, s.c, s.h, s.w, s.k, s.r, s.s, s.pad_h, s.pad_w, s.stride_h, s.stride_w), 0, 0, 0, 0)
+        for s in layers])
     o.init_seeded(seed)
     oracle.set_accumulate_double(True)
     try:
         announce("network vs checker", cnn, batch, policy, algo)
-        with Network(cnn, policy, algo, batch, capture=True, seed=seed) as net:
+        with (Network(cnn, policy, algo, batch, capture=True, seed=seed) if layers is None else
+              Network(layers=layers, policy=policy, algo=algo, capture=True, seed=seed, refined=refined)) as net:
             # the product's own seeded draw equals the checker's, bit for bit
             x0 = net.get_input()
             assert np.array_equal(x0.view(np.uint32), o.input().view(np.uint32))
@@ -283,3 +312,43 @@ def test_full_size_configurations_keep_the_baseline_losses(cnn, batch, algo, pol
             if policy != VDNN_NONE:
                 assert st["offload_bytes"] > 0
                 assert st["peak_bytes_in_use"] < base_stats["peak_bytes_in_use"]
+
+
+def test_unfused_optimizer_gives_the_bits_of_the_fused_step():
+    """dW / db kept in buffers and applied after backward: same losses and parameters as the fused
+    update over three steps; with the step deferred, backward leaves the parameters alone."""
+    announce("unfused optimizer, small net + AlexNet batch 4")
+    for make in (lambda **kw: Network(layers=small_specs(4), policy=VDNN_ALL, algo=VDNN_MEMORY_OPT_ALGO, seed=3, **kw),
+                 lambda **kw: Network(ALEXNET, VDNN_CONV, VDNN_PERF_OPT_ALGO, 4, seed=3, **kw)):
+        with make() as fused:
+            want_losses = fused.train(3)
+            want = [fused.get_params(l) for l in range(fused.num_layers) if fused.has_params(l)]
+        with make(unfused_optimizer=True) as net:
+            got_losses = net.train(3)
+            got = [net.get_params(l) for l in range(net.num_layers) if net.has_params(l)]
+        assert got_losses.tobytes() == want_losses.tobytes() and len(got_losses) == 3
+        for (wa, ba), (wb, bb) in zip(got, want):
+            assert np.array_equal(wa.view(np.uint32), wb.view(np.uint32)) and np.array_equal(ba.view(np.uint32), bb.view(np.uint32))
+        with make(unfused_optimizer=True, defer_optimizer=True) as net:
+            layers = [l for l in range(net.num_layers) if net.has_params(l)]
+            before = [net.get_params(l) for l in layers]
+            assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
+            for l, (w0, b0) in zip(layers, before):
+                w1, b1 = net.get_params(l)
+                assert np.array_equal(w0, w1) and np.array_equal(b0, b1)
+            grads = [net.get_gradients(l) for l in layers]
+            assert net.applyGradients() == 0
+            lr = np.float32(-1e-5)
+            for l, (w0, b0), (dw, db) in zip(layers, before, grads):
+                w1, b1 = net.get_params(l)
+                assert np.abs(dw).max() > 0
+                # one fused multiply-add per element: within one rounding of the two-step float32 result
+                assert_close(w1, w0.astype(np.float64) + np.float64(lr) * dw, 1e-6, "w += alpha dW")
+                assert_close(b1, b0.astype(np.float64) + np.float64(lr) * db, 1e-6, "b += alpha db")
+            # after the deferred step the parameters are those of one fused step
+            with make() as fused:
+                fused.train(1)
+                for l in layers:
+                    wf, bf = fused.get_params(l)
+                    w1, b1 = net.get_params(l)
+                    assert np.array_equal(wf.view(np.uint32), w1.view(np.uint32)) and np.array_equal(bf.view(np.uint32), b1.view(np.uint32))

@@ -215,6 +215,23 @@ def test_refined_lifetimes_cut_peak_memory_threefold():
         assert net.stats()["peak_bytes_in_use"] == base
 
 
+def test_unfused_optimizer_costs_one_more_copy_of_the_parameters():
+    for policy in (BASELINE, VDNN_ALL):
+        with plan(VGG16_128, policy) as net:
+            step(net)
+            fused = net.stats()
+        with plan(VGG16_128, policy, unfused_optimizer=True) as net:
+            n0 = C.c_size_t()
+            lib.vdnn_pool_live_blocks(net.context, C.byref(n0))
+            step(net)
+            st = net.stats()
+            n1 = C.c_size_t()
+            lib.vdnn_pool_live_blocks(net.context, C.byref(n1))
+            assert n1.value == n0.value
+        extra = st["peak_bytes_in_use"] - fused["peak_bytes_in_use"]
+        assert abs(extra - fused["weight_bytes"]) < 64 * 512  # 32 parameter blocks, 512-byte granularity
+
+
 def test_peak_memory_other_configs():
     for cnn, batch, base, allp in ((VGG16_64, 0, 9.57, 4.70), (OVERFEAT, 128, 1.90, 1.37), (ALEXNET, 32, 0.53, 0.44)):
         with plan(cnn, BASELINE, batch=batch) as net:
@@ -268,7 +285,7 @@ def test_dynamic_algo_ladder():
     with plan(VGG16_64, VDNN_ALL) as net:
         step(net)
         need_all = net.stats()["peak_bytes_in_use"]
-    with plan(VGG16_64, VDNN_CONV) as net:
+    with plan(VGG16_64, VDNN_CONV, VDNN_PERF_OPT_ALGO) as net:  # the rung runs the workspace-using kernels
         step(net)
         need_conv = net.stats()["peak_bytes_in_use"]
     # room for VDNN_CONV but not VDNN_NONE

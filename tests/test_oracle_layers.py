@@ -229,3 +229,27 @@ def test_seeded_generator_is_pinned():
     assert lab.min() >= 0 and lab.max() <= 999 and len(np.unique(lab)) == 1000
     he = oracle.fill_normal(300000, 5, 100, 0.0, float(np.sqrt(2.0 / 576)))
     assert abs(he.std() - np.sqrt(2.0 / 576)) < 2e-4
+
+
+def test_tanh_and_sigmoid_against_torch_and_identities():
+    import torch
+    rng = np.random.default_rng(21)
+    x = (rng.standard_normal(4099) * 3).astype(np.float32)
+    dy = rng.standard_normal(4099).astype(np.float32)
+    for fwd, bwd, ref in ((oracle.tanh_fwd, oracle.tanh_bwd, torch.tanh), (oracle.sigmoid_fwd, oracle.sigmoid_bwd, torch.sigmoid)):
+        xt = torch.tensor(x.astype(np.float64), requires_grad=True)
+        yt = ref(xt)
+        yt.backward(torch.tensor(dy.astype(np.float64)))
+        y = fwd(x)
+        assert_close(y, yt.detach().numpy(), 1e-7, "forward")
+        # backward is a function of the (float32) output, as the library call is handed y
+        y64 = y.astype(np.float64)
+        want = dy * (1 - y64 * y64) if ref is torch.tanh else dy * y64 * (1 - y64)
+        assert_close(bwd(y, dy), want, 1e-7, "backward from y")
+        assert_close(bwd(y, dy), xt.grad.numpy(), 1e-5, "backward against autograd")
+    special = np.array([0.0, -0.0, np.inf, -np.inf, 200.0, -200.0], np.float32)
+    assert np.array_equal(oracle.tanh_fwd(special), np.array([0, -0.0, 1, -1, 1, -1], np.float32))
+    assert np.array_equal(oracle.sigmoid_fwd(special), np.array([0.5, 0.5, 1, 0, 1, 0], np.float32))
+    assert np.isnan(oracle.tanh_fwd(np.array([np.nan], np.float32))[0]) and np.isnan(oracle.sigmoid_fwd(np.array([np.nan], np.float32))[0])
+    assert np.array_equal(oracle.tanh_fwd(-x), -oracle.tanh_fwd(x))
+    assert_close(oracle.sigmoid_fwd(x).astype(np.float64) + oracle.sigmoid_fwd(-x), np.ones_like(x), 1e-7, "sigmoid(x) + sigmoid(-x)")

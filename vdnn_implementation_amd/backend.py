@@ -93,6 +93,15 @@ BACKEND_SYMBOLS = {
     "vdnn_fc_bwd_data": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
     "vdnn_fc_bwd_weight_sgd": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _f]),
     "vdnn_fc_bwd_bias_sgd": (_i, [_vp, _vp, _i, _i, _vp, _vp, _f]),
+    "vdnn_conv_bwd_bias": (_i, [_vp, _vp, _S, _vp, _vp]),
+    "vdnn_conv_bwd_filter": (_i, [_vp, _vp, _S, _i, _vp, _vp, _vp, _vp, _sz]),
+    "vdnn_fc_bwd_weight": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
+    "vdnn_fc_bwd_bias": (_i, [_vp, _vp, _i, _i, _vp, _vp]),
+    "vdnn_sgd_apply": (_i, [_vp, _vp, _sz, _f, _vp, _vp]),
+    "vdnn_tanh_fwd": (_i, [_vp, _vp, _sz, _vp, _vp]),
+    "vdnn_tanh_bwd": (_i, [_vp, _vp, _sz, _vp, _vp, _vp]),
+    "vdnn_sigmoid_fwd": (_i, [_vp, _vp, _sz, _vp, _vp]),
+    "vdnn_sigmoid_bwd": (_i, [_vp, _vp, _sz, _vp, _vp, _vp]),
     "vdnn_relu_fwd": (_i, [_vp, _vp, _sz, _vp, _vp]),
     "vdnn_relu_bwd": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _vp]),
     "vdnn_maxpool_fwd": (_i, [_vp, _vp, _S, _vp, _vp]),

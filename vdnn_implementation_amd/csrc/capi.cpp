@@ -15,6 +15,8 @@ static NetworkOptions to_options(const vdnn_network_options* o) {
     n.planOnly = o->plan_only != 0; n.hostSync = o->host_sync != 0; n.capture = o->capture != 0;
     n.verbose = o->verbose != 0; n.device = o->device;
     n.refinedLifetimes = o->refined_lifetimes != 0;
+    n.unfusedOptimizer = o->unfused_optimizer != 0;
+    n.deferOptimizer = o->defer_optimizer != 0;
     return n;
 }
 
@@ -24,7 +26,7 @@ void vdnn_network_default_options(vdnn_network_options* o) {
     if (!o) return;
     NetworkOptions d;
     o->seed = d.seed; o->pool_bytes = 0; o->cap_bytes = 0; o->plan_only = 0; o->host_sync = 0;
-    o->capture = 0; o->verbose = 0; o->device = d.device; o->refined_lifetimes = 0;
+    o->capture = 0; o->verbose = 0; o->device = d.device; o->refined_lifetimes = 0; o->unfused_optimizer = 0; o->defer_optimizer = 0;
 }
 
 vdnn_network* vdnn_network_create(int cnn, int policy, int algo, int batch, const vdnn_network_options* o) {
@@ -79,6 +81,13 @@ void vdnn_network_set_labels(vdnn_network* h, const int32_t* labels) { h->net->s
 void vdnn_network_set_label_tensor(vdnn_network* h, const float* host) { h->net->setLabelTensor(host); }
 int vdnn_network_set_layer_params(vdnn_network* h, int l, const float* f, const float* b) { return h->net->setLayerParams(l, f, b); }
 int vdnn_network_get_layer_params(vdnn_network* h, int l, float* f, float* b) { return h->net->getLayerParams(l, f, b); }
+int vdnn_network_get_layer_gradients(vdnn_network* h, int l, float* f, float* b) { return h->net->getLayerGradients(l, f, b); }
+int vdnn_network_apply_gradients(vdnn_network* h) { return h->net->applyGradients(); }
+int vdnn_network_train(vdnn_network* h, int steps, int is_dynamic, float* losses) {
+    const std::vector<float> v = h->net->train(steps, is_dynamic != 0);
+    if (losses) for (size_t i = 0; i < v.size(); i++) losses[i] = v[i];
+    return (int)v.size();
+}
 
 size_t vdnn_network_filter_count(vdnn_network* h, int l) {
     return (l < 0 || l >= h->net->numLayersCount()) ? 0 : h->net->layerArray()[l]->FilterDataSize();

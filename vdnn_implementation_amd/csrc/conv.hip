@@ -244,9 +244,10 @@ int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* 
     return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K);
 }
 
-int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
-                             const float* x, const float* dy, float* w, float alpha,
-                             void* workspace, size_t workspace_bytes) {
+// out = (accumulate ? out : 0) + alpha * dW
+static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                                const float* x, const float* dy, float* w, float alpha, int accumulate,
+                                void* workspace, size_t workspace_bytes) {
     VDNN_KERNEL_PROLOGUE(ctx);
     (void)algo_mode;
     ConvGeo g;
@@ -281,7 +282,7 @@ int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sha
             }
             VDNN_LAUNCH_CHECK();
         }
-        return launch_reduce_splits(ctx, st, w, staging, (size_t)M * N, (int)chunks, alpha, 1, nullptr, 0);
+        return launch_reduce_splits(ctx, st, w, staging, (size_t)M * N, (int)chunks, alpha, accumulate, nullptr, 0);
     }
     // Split the (n,p,q) reduction so the grid fills the chip; partial sums go to a staging area and
     // are added in split order by a second kernel (no floating-point atomics).
@@ -301,7 +302,7 @@ int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sha
     const long nspan = d.kchunk / PQ + 2;
     VDNN_REQUIRE(nspan * g.K * PQ * 4 < (long)MAX_SUM_RANGE && nspan * g.C * g.H * g.W * 4 < (long)MAX_SUM_RANGE,
                  "samples of one reduction split too large for one descriptor");
-    StoreDense ep{w, staging, nullptr, (long)N, (long)M * N, alpha, 1};
+    StoreDense ep{w, staging, nullptr, (long)N, (long)M * N, alpha, accumulate};
     const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S), dQ = FastDiv::make(g.Q);
     const bool vec = PQ % 4 == 0 && aligned16(dy);
     const bool big = RS > 32;
@@ -318,8 +319,19 @@ int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sha
     else VDNN_WGRAD(false, true);
 #undef VDNN_WGRAD
     if (rc != VDNN_OK) return rc;
-    if (d.splits > 1) return launch_reduce_splits(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, 1, nullptr, 0);
+    if (d.splits > 1) return launch_reduce_splits(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, accumulate, nullptr, 0);
     return VDNN_OK;
+}
+
+int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                             const float* x, const float* dy, float* w, float alpha,
+                             void* workspace, size_t workspace_bytes) {
+    return conv_bwd_filter_impl(ctx, stream, shape, algo_mode, x, dy, w, alpha, 1, workspace, workspace_bytes);
+}
+
+int vdnn_conv_bwd_filter(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                         const float* x, const float* dy, float* dw, void* workspace, size_t workspace_bytes) {
+    return conv_bwd_filter_impl(ctx, stream, shape, algo_mode, x, dy, dw, 1.0f, 0, workspace, workspace_bytes);
 }
 
 } // extern "C"

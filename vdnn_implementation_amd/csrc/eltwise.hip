@@ -78,6 +78,41 @@ __global__ void __launch_bounds__(EB) relu_bwd_kernel(const float* __restrict__ 
     for (size_t i = n4 * 4 + (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) dx[i] = t[i] > 0.0f ? dy[i] : 0.0f;
 }
 
+// ---- tanh / sigmoid: the other two activation modes of the layer (one float4 per thread) --------------
+// backward needs the output only: tanh' = 1 - y^2, sigmoid' = y (1 - y)
+template <int MODE> __device__ __forceinline__ float act1(float v) {
+    return MODE == 0 ? tanhf(v) : 1.0f / (1.0f + expf(-v));
+}
+template <int MODE> __device__ __forceinline__ float dact1(float y, float d) {
+    return MODE == 0 ? d * (1.0f - y * y) : d * (y * (1.0f - y));
+}
+
+template <int MODE>
+__global__ void __launch_bounds__(EB) act_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, size_t n4, size_t n) {
+    const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
+    if (i < n4) {
+        float4 v = ((const float4*)x)[i];
+        v.x = act1<MODE>(v.x); v.y = act1<MODE>(v.y); v.z = act1<MODE>(v.z); v.w = act1<MODE>(v.w);
+        ((float4*)y)[i] = v;
+    }
+    const size_t t = n4 * 4 + i;
+    if (t < n) y[t] = act1<MODE>(x[t]);
+}
+
+template <int MODE>
+__global__ void __launch_bounds__(EB) act_bwd_kernel(const float* __restrict__ y, const float* __restrict__ dy, float* __restrict__ dx,
+                                                     size_t n4, size_t n) {
+    const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
+    if (i < n4) {
+        const float4 a = ((const float4*)y)[i], d = ((const float4*)dy)[i];
+        float4 o;
+        o.x = dact1<MODE>(a.x, d.x); o.y = dact1<MODE>(a.y, d.y); o.z = dact1<MODE>(a.z, d.z); o.w = dact1<MODE>(a.w, d.w);
+        ((float4*)dx)[i] = o;
+    }
+    const size_t t = n4 * 4 + i;
+    if (t < n) dx[t] = dact1<MODE>(y[t], dy[t]);
+}
+
 // ---- elementwise helpers ------------------------------------------------------------------------
 __global__ void __launch_bounds__(EB) sub_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ r, size_t n) {
     const size_t stride = (size_t)gridDim.x * EB;
@@ -103,8 +138,7 @@ __global__ void __launch_bounds__(EB) reduce_splits_kernel(float* __restrict__ o
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < count; i += stride) {
         float s = partial[i];
         for (int k = 1; k < splits; k++) s += partial[(size_t)k * count + i];
-        float r = alpha * s;
-        if (accumulate) r = out[i] + r;
+        float r = accumulate ? __fmaf_rn(alpha, s, out[i]) : alpha * s; // one fused multiply-add on every route
         if (bias_j) r += bias_j[i % ncols];
         out[i] = r;
     }
@@ -117,6 +151,14 @@ int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const fl
                        out, partial, count, splits, alpha, accumulate, bias_j, ncols);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
+}
+
+// param[i] = fma(alpha, grad[i], param[i]), the expression the fused updates evaluate
+__global__ void __launch_bounds__(EB) sgd_apply_kernel(const float* __restrict__ grad, float* __restrict__ param, float alpha, size_t count) {
+    const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
+    if (i < count) {
+        param[i] = __fmaf_rn(alpha, grad[i], param[i]);
+    }
 }
 
 // ---- bias gradient of a convolution: bias[k] += alpha * sum_{n,pq} dy[n,k,pq] -------------------
@@ -149,21 +191,21 @@ __global__ void __launch_bounds__(EB) bias_grad_partial_kernel(const float* __re
     if (threadIdx.x == 0) partial[blockIdx.x] = acc;
 }
 // stage 2: one thread per channel adds its partials in split order
-__global__ void __launch_bounds__(EB) bias_grad_final_kernel(const float* __restrict__ partial, float* __restrict__ bias, int K, int splits, float alpha) {
+__global__ void __launch_bounds__(EB) bias_grad_final_kernel(const float* __restrict__ partial, float* __restrict__ bias, int K, int splits, float alpha, int accumulate) {
     const int k = blockIdx.x * EB + threadIdx.x;
     if (k >= K) return;
     float s = 0.0f;
     for (int i = 0; i < splits; i++) s += partial[(size_t)k * splits + i];
-    bias[k] = bias[k] + alpha * s;
+    bias[k] = accumulate ? __fmaf_rn(alpha, s, bias[k]) : alpha * s;
 }
 
 // bias[o] += alpha * sum_n dy[n,o]
-__global__ void __launch_bounds__(EB) fc_bias_grad_kernel(const float* __restrict__ dy, float* __restrict__ bias, int N, int Cout, float alpha) {
+__global__ void __launch_bounds__(EB) fc_bias_grad_kernel(const float* __restrict__ dy, float* __restrict__ bias, int N, int Cout, float alpha, int accumulate) {
     const int o = blockIdx.x * EB + threadIdx.x;
     if (o >= Cout) return;
     float s = 0.0f;
     for (int n = 0; n < N; n++) s += dy[(size_t)n * Cout + o];
-    bias[o] = bias[o] + alpha * s;
+    bias[o] = accumulate ? __fmaf_rn(alpha, s, bias[o]) : alpha * s;
 }
 
 // ---- max pooling --------------------------------------------------------------------------------
@@ -406,6 +448,32 @@ static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 using namespace vdnn;
 
+template <int MODE>
+static int act_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const char* name, size_t count, const float* x, float* y) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(x && y, "null tensor");
+    if (count == 0) return VDNN_OK;
+    const size_t n4 = (aligned16(x) && aligned16(y)) ? count / 4 : 0;
+    const size_t threads = n4 > count - n4 * 4 ? n4 : count - n4 * 4;
+    ProfScope prof(ctx, stream_of(ctx, stream), name, 0.0, 8.0 * (double)count);
+    hipLaunchKernelGGL(act_fwd_kernel<MODE>, dim3(grid_for(threads, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), x, y, n4, count);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+template <int MODE>
+static int act_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const char* name, size_t count, const float* y, const float* dy, float* dx) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(y && dy && dx, "null tensor");
+    if (count == 0) return VDNN_OK;
+    const size_t n4 = (aligned16(y) && aligned16(dy) && aligned16(dx)) ? count / 4 : 0;
+    const size_t threads = n4 > count - n4 * 4 ? n4 : count - n4 * 4;
+    ProfScope prof(ctx, stream_of(ctx, stream), name, 0.0, 12.0 * (double)count);
+    hipLaunchKernelGGL(act_bwd_kernel<MODE>, dim3(grid_for(threads, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), y, dy, dx, n4, count);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
 extern "C" {
 
 int vdnn_relu_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y) {
@@ -430,6 +498,11 @@ int vdnn_relu_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
+
+int vdnn_tanh_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y) { return act_fwd<0>(ctx, stream, "tanh_fwd", count, x, y); }
+int vdnn_tanh_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* y, const float* dy, float* dx) { return act_bwd<0>(ctx, stream, "tanh_bwd", count, y, dy, dx); }
+int vdnn_sigmoid_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y) { return act_fwd<1>(ctx, stream, "sigmoid_fwd", count, x, y); }
+int vdnn_sigmoid_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* y, const float* dy, float* dx) { return act_bwd<1>(ctx, stream, "sigmoid_bwd", count, y, dy, dx); }
 
 int vdnn_sub(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* a, const float* b, float* r) {
     VDNN_KERNEL_PROLOGUE(ctx);
@@ -458,7 +531,7 @@ int vdnn_bias_add(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw, con
     return VDNN_OK;
 }
 
-int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* dy, float* bias, float alpha) {
+static int conv_bwd_bias_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* dy, float* bias, float alpha, int accumulate) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(shape && dy && bias, "null argument");
     const int N = shape->n, K = shape->k;
@@ -476,15 +549,43 @@ int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape
     ProfScope prof(ctx, st, "conv_bwd_bias", 0.0, 4.0 * (double)N * K * P * Q);
     hipLaunchKernelGGL(bias_grad_partial_kernel, dim3(K * splits), dim3(EB), 0, st, dy, ctx->reduce_scratch, N, K, P * Q, splits, per);
     VDNN_LAUNCH_CHECK();
-    hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB - 1) / EB), dim3(EB), 0, st, ctx->reduce_scratch, bias, K, splits, alpha);
+    hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB - 1) / EB), dim3(EB), 0, st, ctx->reduce_scratch, bias, K, splits, alpha, accumulate);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* dy, float* bias, float alpha) {
+    return conv_bwd_bias_impl(ctx, stream, shape, dy, bias, alpha, 1);
+}
+
+int vdnn_conv_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* dy, float* db) {
+    return conv_bwd_bias_impl(ctx, stream, shape, dy, db, 1.0f, 0);
+}
+
+static int fc_bwd_bias_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const float* dy, float* bias, float alpha, int accumulate) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(dy && bias && n > 0 && c_out > 0, "bad argument");
+    hipLaunchKernelGGL(fc_bias_grad_kernel, dim3((c_out + EB - 1) / EB), dim3(EB), 0, stream_of(ctx, stream), dy, bias, n, c_out, alpha, accumulate);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
 int vdnn_fc_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const float* dy, float* bias, float alpha) {
+    return fc_bwd_bias_impl(ctx, stream, n, c_out, dy, bias, alpha, 1);
+}
+
+int vdnn_fc_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const float* dy, float* db) {
+    return fc_bwd_bias_impl(ctx, stream, n, c_out, dy, db, 1.0f, 0);
+}
+
+// param[i] += alpha * grad[i]: the optimizer step when gradients are kept instead of fused into backward
+int vdnn_sgd_apply(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float alpha, const float* grad, float* param) {
     VDNN_KERNEL_PROLOGUE(ctx);
-    VDNN_REQUIRE(dy && bias && n > 0 && c_out > 0, "bad argument");
-    hipLaunchKernelGGL(fc_bias_grad_kernel, dim3((c_out + EB - 1) / EB), dim3(EB), 0, stream_of(ctx, stream), dy, bias, n, c_out, alpha);
+    VDNN_REQUIRE(grad && param, "null tensor");
+    if (count == 0) return VDNN_OK;
+    hipStream_t st = stream_of(ctx, stream);
+    ProfScope prof(ctx, st, "sgd_apply", 0.0, 12.0 * (double)count);
+    hipLaunchKernelGGL(sgd_apply_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, st, grad, param, alpha, count);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }

@@ -90,4 +90,14 @@ int vdnn_fc_bwd_weight_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in,
     return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_weight", al, bl, c_out, c_in, n, w, alpha, 1, nullptr);
 }
 
+int vdnn_fc_bwd_weight(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                       const float* x, const float* dy, float* dw) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(x && dy && dw && n > 0 && c_in > 0 && c_out > 0, "bad argument");
+    FC_REQUIRE_SMALL((long)n * c_out); FC_REQUIRE_SMALL((long)n * c_in);
+    LoadDenseRow al{dy, (long)c_out, c_out, (unsigned)((long)n * c_out * 4)};
+    LoadDenseRow bl{x, (long)c_in, c_in, (unsigned)((long)n * c_in * 4)};
+    return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_weight", al, bl, c_out, c_in, n, dw, 1.0f, 0, nullptr);
+}
+
 } // extern "C"

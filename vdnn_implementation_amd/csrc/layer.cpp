@@ -63,6 +63,7 @@ void Layer::construct(vdnn_ctx* _ctx) {
     concatenateChannelOffset = 0;
     refCntFwd = refCntBwd = 0;
     srcData = filterData = biasData = dstData = diffData = gradData = nullptr;
+    filterGrad = biasGrad = nullptr;
     fwdWorkSpaceSize = bwdDataWorkSpaceSize = bwdFilterWorkSpaceSize = 0;
     srcReadyEvent = offloadDoneEvent = nullptr;
     prefetchBlockFreeEvent = prefetchHostReadyEvent = prefetchDoneEvent = nullptr;
@@ -83,13 +84,11 @@ void Layer::construct(vdnn_ctx* _ctx) {
         setAlgoMode(vdnnAlgoMode); /* layer.cu:255-294 */
         break;
     case RELU:
-    case SOFTMAX:
-    case LRN: /* layer.cu:301-304 */
-        n_out = n_in; c_out = c_in; h_out = h_in; w_out = w_in;
-        break;
     case TANH:
-    case SIGMOID:
-        M_ASSERT(false, "TANH and SIGMOID are enumerated by the reference but used by none of its networks; not built");
+    case SIGMOID: /* layer.cu:298-304: the three activation modes share one layer kind */
+    case SOFTMAX:
+    case LRN:
+        n_out = n_in; c_out = c_in; h_out = h_in; w_out = w_in;
         break;
     case POOL: /* layer.cu:432-439 */
         n_out = n_in; c_out = c_in;
@@ -125,6 +124,8 @@ void Layer::construct(vdnn_ctx* _ctx) {
 Layer::~Layer() {
     if (filterData) vdnn_pool_free(ctx, filterData);
     if (biasData) vdnn_pool_free(ctx, biasData);
+    if (filterGrad) vdnn_pool_free(ctx, filterGrad);
+    if (biasGrad) vdnn_pool_free(ctx, biasGrad);
     if (vdnnMode == BASELINE && dstData) vdnn_pool_free(ctx, dstData);
 }
 
@@ -171,7 +172,9 @@ int Layer::forward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workS
     case FC_GEMM: return fullyConnectedForward(_offloaded, _offloadedSrcData_h, workSpace, isDynamic);
     case CONV:
     case FC_CONV: return convolutionForward(_offloaded, _offloadedSrcData_h, workSpace, isDynamic);
-    case RELU: return activationForward(_offloaded, _offloadedSrcData_h, workSpace, isDynamic);
+    case RELU:
+    case TANH:
+    case SIGMOID: return activationForward(_offloaded, _offloadedSrcData_h, workSpace, isDynamic);
     case SOFTMAX: return softmaxForward(_offloaded, _offloadedSrcData_h, workSpace, isDynamic);
     case POOL: return poolingForward(_offloaded, _offloadedSrcData_h, workSpace, isDynamic);
     case LRN: return lrnForward(_offloaded, _offloadedSrcData_h, workSpace, isDynamic);
@@ -186,7 +189,9 @@ int Layer::backward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h, v
     case FC_GEMM: return fullyConnectedBackward(_layer_id_to_prefetch, _prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes, workSpace, isDynamic);
     case CONV:
     case FC_CONV: return convolutionBackward(_layer_id_to_prefetch, _prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes, workSpace, isDynamic);
-    case RELU: return activationBackward(_layer_id_to_prefetch, _prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes, workSpace, isDynamic);
+    case RELU:
+    case TANH:
+    case SIGMOID: return activationBackward(_layer_id_to_prefetch, _prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes, workSpace, isDynamic);
     case SOFTMAX: return softmaxBackward(_layer_id_to_prefetch, _prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes, workSpace, isDynamic);
     case POOL: return poolingBackward(_layer_id_to_prefetch, _prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes, workSpace, isDynamic);
     case LRN: return lrnBackward(_layer_id_to_prefetch, _prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes, workSpace, isDynamic);
@@ -255,11 +260,16 @@ int Layer::convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedS
     freeWorkSpace(workSpace, bwdDataWorkSpaceSize, curWorkSpace, isDynamic);
 
     /* Backward Bias Propagation: the learning rate is folded into the update */
-    checkVDNN(vdnn_conv_bwd_bias_sgd(ctx, *stream_compute, &shape, (const float*)diffData, (float*)biasData, lr));
+    if (filterGrad) checkVDNN(vdnn_conv_bwd_bias(ctx, *stream_compute, &shape, (const float*)diffData, (float*)biasGrad));
+    else checkVDNN(vdnn_conv_bwd_bias_sgd(ctx, *stream_compute, &shape, (const float*)diffData, (float*)biasData, lr));
 
     if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) return -1;
-    checkVDNN(vdnn_conv_bwd_filter_sgd(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
-                                       (float*)filterData, lr, curWorkSpace, bwdFilterWorkSpaceSize));
+    if (filterGrad)
+        checkVDNN(vdnn_conv_bwd_filter(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
+                                       (float*)filterGrad, curWorkSpace, bwdFilterWorkSpaceSize));
+    else
+        checkVDNN(vdnn_conv_bwd_filter_sgd(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
+                                           (float*)filterData, lr, curWorkSpace, bwdFilterWorkSpaceSize));
     freeWorkSpace(workSpace, bwdFilterWorkSpaceSize, curWorkSpace, isDynamic);
     return 0;
 }
@@ -286,8 +296,13 @@ int Layer::fullyConnectedBackward(int _layer_id_to_prefetch, DATATYPE* _prefetch
     if (vdnnMode != BASELINE && _layer_id_to_prefetch >= 0)
         prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);
     checkVDNN(vdnn_fc_bwd_data(ctx, *stream_compute, n_out, c_in, c_out, (const float*)diffData, (const float*)filterData, (float*)gradData));
-    checkVDNN(vdnn_fc_bwd_weight_sgd(ctx, *stream_compute, n_out, c_in, c_out, (const float*)srcData, (const float*)diffData, (float*)filterData, lr));
-    checkVDNN(vdnn_fc_bwd_bias_sgd(ctx, *stream_compute, n_out, c_out, (const float*)diffData, (float*)biasData, lr));
+    if (filterGrad) {
+        checkVDNN(vdnn_fc_bwd_weight(ctx, *stream_compute, n_out, c_in, c_out, (const float*)srcData, (const float*)diffData, (float*)filterGrad));
+        checkVDNN(vdnn_fc_bwd_bias(ctx, *stream_compute, n_out, c_out, (const float*)diffData, (float*)biasGrad));
+    } else {
+        checkVDNN(vdnn_fc_bwd_weight_sgd(ctx, *stream_compute, n_out, c_in, c_out, (const float*)srcData, (const float*)diffData, (float*)filterData, lr));
+        checkVDNN(vdnn_fc_bwd_bias_sgd(ctx, *stream_compute, n_out, c_out, (const float*)diffData, (float*)biasData, lr));
+    }
     return 0;
 }
 
@@ -296,7 +311,10 @@ int Layer::activationForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, v
     if (vdnnMode != BASELINE) {
         if (cnmemMallocDstData(isDynamic) < 0) return -1;
     }
-    checkVDNN(vdnn_relu_fwd(ctx, *stream_compute, SrcDataSize(), (const float*)srcData, (float*)dstData));
+    /* the activation mode follows the layer type (layer.cu:357-372) */
+    if (layerType == TANH) checkVDNN(vdnn_tanh_fwd(ctx, *stream_compute, SrcDataSize(), (const float*)srcData, (float*)dstData));
+    else if (layerType == SIGMOID) checkVDNN(vdnn_sigmoid_fwd(ctx, *stream_compute, SrcDataSize(), (const float*)srcData, (float*)dstData));
+    else checkVDNN(vdnn_relu_fwd(ctx, *stream_compute, SrcDataSize(), (const float*)srcData, (float*)dstData));
     if (_offloaded[layerId]) offloadSrcData(_offloaded, _offloadedSrcData_h);
     return 0;
 }
@@ -310,8 +328,13 @@ int Layer::activationBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSr
     }
     if (vdnnMode != BASELINE && _layer_id_to_prefetch >= 0)
         prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);
-    checkVDNN(vdnn_relu_bwd(ctx, *stream_compute, SrcDataSize(), (const float*)srcData, (const float*)dstData,
-                            (const float*)diffData, (float*)gradData));
+    if (layerType == TANH)
+        checkVDNN(vdnn_tanh_bwd(ctx, *stream_compute, SrcDataSize(), (const float*)dstData, (const float*)diffData, (float*)gradData));
+    else if (layerType == SIGMOID)
+        checkVDNN(vdnn_sigmoid_bwd(ctx, *stream_compute, SrcDataSize(), (const float*)dstData, (const float*)diffData, (float*)gradData));
+    else
+        checkVDNN(vdnn_relu_bwd(ctx, *stream_compute, SrcDataSize(), (const float*)srcData, (const float*)dstData,
+                                (const float*)diffData, (float*)gradData));
     return 0;
 }
 
@@ -397,6 +420,20 @@ void Layer::initializeConvolutionFilterAndBias() {
     vdnn::seeded_fill_normal(filterData_h.data(), filterDataSize, initSeed, 100 + 2 * (uint64_t)layerId, 0.0f, (float)std::sqrt(2.0 / fan_in));
     checkVDNN(vdnn_memcpy_h2d(ctx, filterData, filterData_h.data(), sizeof(DATATYPE) * filterDataSize));
     checkVDNN(vdnn_memcpy_h2d(ctx, biasData, biasData_h.data(), sizeof(DATATYPE) * biasDataSize));
+}
+
+/* addition: gradient buffers of a layer with parameters, for an optimizer step outside backward */
+void Layer::keepGradients() {
+    if (!filterData || filterGrad) return;
+    ASSERT_EQ(vdnn_pool_malloc(ctx, &filterGrad, sizeof(DATATYPE) * (size_t)k * c_in * r * s));
+    ASSERT_EQ(vdnn_pool_malloc(ctx, &biasGrad, sizeof(DATATYPE) * (size_t)k));
+}
+
+int Layer::applyGradients(DATATYPE alpha) {
+    if (!filterGrad) return 0;
+    checkVDNN(vdnn_sgd_apply(ctx, *stream_compute, (size_t)k * c_in * r * s, alpha, (const float*)filterGrad, (float*)filterData));
+    checkVDNN(vdnn_sgd_apply(ctx, *stream_compute, (size_t)k, alpha, (const float*)biasGrad, (float*)biasData));
+    return 0;
 }
 
 /* layer.cu:947-967 */

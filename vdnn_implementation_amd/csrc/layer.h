@@ -97,6 +97,12 @@ public:
     static void     setVerbose(bool v) { verbose = v; }
     // Plan-only networks allocate the parameter blocks but skip drawing and uploading their values
     static void     setSkipParameterValues(bool v) { skipParameterValues = v; }
+    /* addition: keep dW / db in buffers of their own instead of fusing the SGD step into backward
+     * (layer.cu:651-660, 736-761 fuse it); applyGradients then performs the step */
+    void            keepGradients();
+    int             applyGradients(DATATYPE alpha);
+    void*           FilterGrad()             { return filterGrad; }
+    void*           BiasGrad()               { return biasGrad; }
 
     // Seeded initialisation of filter/bias: He-normal filters, zero biases
     void    initializeConvolutionFilterAndBias();
@@ -248,6 +254,8 @@ private:
     void* srcData;    // x
     void* filterData; // w
     void* biasData;   // bias
+    void* filterGrad; // dW (only with keepGradients)
+    void* biasGrad;   // db
     void* dstData;    // y
     void* diffData;   // dy
     void* gradData;   // dx

@@ -344,8 +344,8 @@ struct StoreDense {
                     if (d.splits > 1) {
                         partial[(long)ks * partial_stride + idx] = a;
                     } else {
-                        float r = alpha * a;
-                        if (accumulate) r = out[idx] + r;
+                        // one fused multiply-add: every route to "out += alpha * sum" rounds the same way
+                        float r = accumulate ? __fmaf_rn(alpha, a, out[idx]) : alpha * a;
                         if (bias_j) r += bias_j[j];
                         out[idx] = r;
                     }

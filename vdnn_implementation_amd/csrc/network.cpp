@@ -219,7 +219,7 @@ void Network::initPool() {
             const size_t src = spec_src_count(s), dst = spec_dst_count(s);
             sum += dst;
             maxAct = std::max(maxAct, std::max(src, dst));
-            if (s.type == FC_GEMM || is_conv(s.type)) sum += (size_t)s.k * s.c * s.r * s.s + s.k;
+            if (s.type == FC_GEMM || is_conv(s.type)) sum += ((size_t)s.k * s.c * s.r * s.s + s.k) * (options.unfusedOptimizer ? 2 : 1);
         }
         sum += spec_src_count(specs[0]) * 2 + spec_dst_count(specs.back()) * 2 + 3 * maxAct;
         bytes = sum * sizeof(DATATYPE);
@@ -293,6 +293,7 @@ void Network::buildLayers() {
         else
             layer[l] = new Layer(vdnnType, mode, s.type, &convHandle, &stream_compute, &stream_memory, l,
                                  s.n, s.c, s.h, s.w, s.pad_h, s.pad_w, s.stride_h, s.stride_w, s.k, s.r, s.s);
+        if (options.unfusedOptimizer) layer[l]->keepGradients();
     }
     capDst.assign(numLayers, {});
     capGrad.assign(numLayers, {});
@@ -347,12 +348,13 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         }
     }
     lastStats.pinnedBytes = 0;
-    /* refined lifetimes: a ReLU layer's input is dead once its forward has run (never layer 0: the
+    /* refined lifetimes: an activation layer's input is dead once its forward has run (never layer 0: the
        network input outlives the step) and its backward runs in place */
     const bool refined = options.refinedLifetimes && newVdnnType != BASELINE;
     if (refined) {
         for (int l = 0; l < numLayers; l++) {
-            if (layer[l]->LayerType() != RELU) continue;
+            const Layer_t kind = layer[l]->LayerType(); /* all three activations differentiate from y alone */
+            if (kind != RELU && kind != TANH && kind != SIGMOID) continue;
             layer[l]->setInPlaceOp(true);
             if (l > 0) dropSrcAfterFwd[l] = true;
         }
@@ -617,7 +619,35 @@ int Network::backwardPropagation(bool isDynamic) {
         inputData = layer[0]->SrcData(); /* network.cu:1185 */
         inputResident = true;
     }
+    if (options.unfusedOptimizer && !options.deferOptimizer) return applyGradients();
     return 0;
+}
+
+/* addition: the optimizer step of unfusedOptimizer, with the reference's scalar (alpha = -lr, layer.cu:593) */
+int Network::applyGradients() {
+    const DATATYPE lr = LEARNING_RATE * -1.0f;
+    for (int l = 0; l < numLayers; l++)
+        if (layer[l]->applyGradients(lr) < 0) return -1;
+    return 0;
+}
+
+int Network::getLayerGradients(int l, float* filter, float* bias) {
+    if (l < 0 || l >= numLayers || !layer[l]->hasParams() || !layer[l]->FilterGrad()) return -1;
+    if (filter) checkVDNN(vdnn_memcpy_d2h(ctx, filter, layer[l]->FilterGrad(), layer[l]->FilterDataSize() * sizeof(float)));
+    if (bias) checkVDNN(vdnn_memcpy_d2h(ctx, bias, layer[l]->BiasGrad(), layer[l]->BiasDataSize() * sizeof(float)));
+    return 0;
+}
+
+/* addition: the reference's main runs one step (vdnn.cu:71-75); this is the loop around it */
+std::vector<float> Network::train(int steps, bool isDynamic) {
+    std::vector<float> losses;
+    for (int i = 0; i < steps; i++) {
+        if (forwardPropagation(isDynamic) < 0) break;
+        losses.push_back(loss());
+        if (backwardPropagation(isDynamic) < 0) break;
+        if (options.unfusedOptimizer && options.deferOptimizer && applyGradients() < 0) break;
+    }
+    return losses;
 }
 
 /* network.cu:1193-1196 */

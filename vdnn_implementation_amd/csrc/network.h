@@ -26,6 +26,12 @@ struct NetworkOptions {
     // that layer's backward instead of after it (those backward kernels never read y);
     // (3) a ReLU layer writes dx over dy instead of into a new block.
     bool     refinedLifetimes = false;
+    // Keep every layer's dW / db in buffers of their own and perform the SGD step after the last
+    // backward layer (applyGradients) instead of inside the backward kernels as the reference does
+    // (layer.cu:651-660, 736-761). Same bits as the fused step; what a data-parallel exchange or
+    // another optimizer needs. deferOptimizer leaves the step to the caller.
+    bool     unfusedOptimizer = false;
+    bool     deferOptimizer = false;
     int      device = DEFAULT_DEVICE;
 };
 
@@ -115,6 +121,11 @@ public:
     int             getLayerParams(int l, float* filter, float* bias);
     // mean cross-entropy of the last forward's output against the target (waits for the device)
     float           loss();
+    // the optimizer step of unfusedOptimizer: w += (-lr) * dW, b += (-lr) * db for every layer
+    int             applyGradients();
+    int             getLayerGradients(int l, float* filter, float* bias);
+    // `steps` training steps (forward, backward, optimizer); returns the loss before each step's update
+    std::vector<float> train(int steps, bool isDynamic = false);
     void            synchronize();
     NetworkStats    stats();
     void            resetPeak();

@@ -55,6 +55,7 @@ int main(int argc, char** argv) {
         else if (!strcmp(argv[i], "--host-sync")) opt.hostSync = true;
         else if (!strcmp(argv[i], "--plan")) opt.planOnly = true;
         else if (!strcmp(argv[i], "--refined")) opt.refinedLifetimes = true;
+        else if (!strcmp(argv[i], "--unfused")) opt.unfusedOptimizer = true;
         else if (!strcmp(argv[i], "--verbose")) opt.verbose = true;
         else M_ASSERT(0, "unknown flag");
     }

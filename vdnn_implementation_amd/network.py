@@ -14,7 +14,8 @@ _ip = C.POINTER(C.c_int32)
 
 class Options(C.Structure):
     _fields_ = [("seed", C.c_uint64), ("pool_bytes", _sz), ("cap_bytes", _sz), ("plan_only", _i), ("host_sync", _i),
-                ("capture", _i), ("verbose", _i), ("device", _i), ("refined_lifetimes", _i)]
+                ("capture", _i), ("verbose", _i), ("device", _i), ("refined_lifetimes", _i),
+                ("unfused_optimizer", _i), ("defer_optimizer", _i)]
 
 
 class LayerSpec(C.Structure):
@@ -50,6 +51,9 @@ CAPI_SYMBOLS = {
     "vdnn_network_set_label_tensor": (None, [_vp, _fp]),
     "vdnn_network_set_layer_params": (_i, [_vp, _i, _fp, _fp]),
     "vdnn_network_get_layer_params": (_i, [_vp, _i, _fp, _fp]),
+    "vdnn_network_get_layer_gradients": (_i, [_vp, _i, _fp, _fp]),
+    "vdnn_network_apply_gradients": (_i, [_vp]),
+    "vdnn_network_train": (_i, [_vp, _i, _i, _fp]),
     "vdnn_network_filter_count": (_sz, [_vp, _i]),
     "vdnn_network_bias_count": (_sz, [_vp, _i]),
     "vdnn_network_captured_dst": (_sz, [_vp, _i, _fp, _sz]),
@@ -87,12 +91,13 @@ class Network:
 
     def __init__(self, cnn=None, policy=enums.BASELINE, algo=enums.VDNN_MEMORY_OPT_ALGO, batch=0, layers=None, seed=1,
                  pool_bytes=0, cap_bytes=0, plan_only=False, host_sync=False, capture=False, verbose=False, device=0,
-                 refined=False):
+                 refined=False, unfused_optimizer=False, defer_optimizer=False):
         o = Options()
         lib.vdnn_network_default_options(C.byref(o))
         o.seed, o.pool_bytes, o.cap_bytes = seed, int(pool_bytes), int(cap_bytes)
         o.plan_only, o.host_sync, o.capture, o.verbose, o.device = int(plan_only), int(host_sync), int(capture), int(verbose), device
         o.refined_lifetimes = int(refined)
+        o.unfused_optimizer, o.defer_optimizer = int(unfused_optimizer), int(defer_optimizer)
         if layers is not None:
             arr = (LayerSpec * len(layers))(*layers)
             self._h = lib.vdnn_network_create_custom(arr, len(layers), policy, algo, C.byref(o))
@@ -201,6 +206,24 @@ class Network:
         assert w.size == lib.vdnn_network_filter_count(self._h, l)
         lib.vdnn_network_get_layer_params(self._h, l, w.ctypes.data_as(_fp), b.ctypes.data_as(_fp))
         return w, b
+
+    def get_gradients(self, l):
+        """dW, db of layer l from the last backward (needs unfused_optimizer)."""
+        s = self.specs[l]
+        w = np.empty((s.k, s.c, s.r, s.s), np.float32)
+        b = np.empty(lib.vdnn_network_bias_count(self._h, l), np.float32)
+        if lib.vdnn_network_get_layer_gradients(self._h, l, w.ctypes.data_as(_fp), b.ctypes.data_as(_fp)) != 0:
+            raise ValueError("layer %d keeps no gradients" % l)
+        return w, b
+
+    def applyGradients(self):
+        return lib.vdnn_network_apply_gradients(self._h)
+
+    def train(self, steps, is_dynamic=False):
+        """`steps` training steps; the loss seen by each step's forward."""
+        out = np.zeros(steps, np.float32)
+        done = lib.vdnn_network_train(self._h, int(steps), int(is_dynamic), out.ctypes.data_as(_fp))
+        return out[:done]
 
     def set_params(self, l, w=None, b=None):
         w = None if w is None else _f32(w)
