@@ -35,6 +35,14 @@ extern "C" {
 
 #define VDNN_CTX_PLAN_ONLY 1
 
+/* Element type of ACTIVATION tensors (layer inputs, outputs and their gradients: every `void*`
+ * tensor argument of the kernel entry points below). The reference fixes float (vdnn.h:11-12);
+ * bfloat16 storage halves the memory and the offload traffic. Filters, biases, their gradients and
+ * loss values are always float (`float*` arguments), and all arithmetic is float with float
+ * accumulation; a bfloat16 result is rounded once (to nearest, ties to even) when it is stored. */
+#define VDNN_DTYPE_F32  0
+#define VDNN_DTYPE_BF16 1
+
 /* passes of a convolution, for vdnn_conv_workspace_bytes */
 #define VDNN_PASS_FWD        0
 #define VDNN_PASS_BWD_DATA   1
@@ -57,6 +65,10 @@ typedef struct {
  * compute stream and the two copy streams. */
 int vdnn_ctx_create(vdnn_ctx** out, int device, int flags);
 int vdnn_ctx_destroy(vdnn_ctx* ctx);
+/* Element type of the activation tensors handed to later kernel calls on this context (default
+ * VDNN_DTYPE_F32). No counterpart in the reference (CUDNN_DATA_FLOAT is fixed, vdnn.h:12). */
+int vdnn_ctx_set_activation_dtype(vdnn_ctx* ctx, int dtype);
+int vdnn_ctx_activation_dtype(vdnn_ctx* ctx);
 const char* vdnn_last_error(void);
 /* cudaGetDeviceProperties(...).totalGlobalMem (network.cu:35-36, 48). */
 int vdnn_device_mem_info(vdnn_ctx* ctx, size_t* free_bytes, size_t* total_bytes);
@@ -118,23 +130,23 @@ size_t vdnn_conv_workspace_bytes(const vdnn_shape_t* shape, int algo_mode, int p
 /* cudnnConvolutionForward + cudnnAddTensor (layer.cu:560-582): y = x (*) w + bias[k], the bias is
  * added once after the full reduction. bias may be NULL (no add). */
 int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
-                  const float* x, const float* w, const float* bias, float* y,
+                  const void* x, const float* w, const float* bias, void* y,
                   void* workspace, size_t workspace_bytes);
 /* cudnnAddTensor alone (layer.cu:576-582): y[n,k,:,:] += bias[k]. */
-int vdnn_bias_add(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw, const float* bias, float* y);
+int vdnn_bias_add(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw, const float* bias, void* y);
 /* cudnnConvolutionBackwardData (layer.cu:616-625): dx = w^T (*) dy, alpha 1, beta 0. */
 int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
-                       const float* dy, const float* w, float* dx,
+                       const void* dy, const float* w, void* dx,
                        void* workspace, size_t workspace_bytes);
 /* cudnnConvolutionBackwardBias with alpha=-lr, beta=1 (layer.cu:631-637):
  * bias[k] += alpha * sum_{n,p,q} dy[n,k,p,q]. Fixed summation order. */
 int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape,
-                           const float* dy, float* bias, float alpha);
+                           const void* dy, float* bias, float alpha);
 /* cudnnConvolutionBackwardFilter with alpha=-lr, beta=1 (layer.cu:651-660):
  * w[k,c,r,s] += alpha * sum_{n,p,q} dy[n,k,p,q] * x[n,c,p*sh-ph+r,q*sw-pw+s]. Fixed summation
  * order (no floating-point atomics). */
 int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
-                             const float* x, const float* dy, float* w, float alpha,
+                             const void* x, const void* dy, float* w, float alpha,
                              void* workspace, size_t workspace_bytes);
 
 /* The same two reductions with the optimizer step left out: db[k] = sum dy, dw = sum dy*x (beta = 0).
@@ -142,76 +154,76 @@ int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sha
  * gradients (to average them over devices, or to apply another optimizer) needs them separately.
  * vdnn_sgd_apply then evaluates param += alpha * grad with the arithmetic of the fused calls, so
  * the two routes give the same bits. */
-int vdnn_conv_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* dy, float* db);
+int vdnn_conv_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* dy, float* db);
 int vdnn_conv_bwd_filter(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
-                         const float* x, const float* dy, float* dw, void* workspace, size_t workspace_bytes);
+                         const void* x, const void* dy, float* dw, void* workspace, size_t workspace_bytes);
 int vdnn_sgd_apply(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float alpha, const float* grad, float* param);
 
 /* ---- fully connected (replaces cuBLAS: layer.cu:667-764) ------------------------------------- */
 /* Sgemm(T,N) + rank-1 bias broadcast (layer.cu:677-706): y[n,o] = sum_i w[o,i] x[n,i] + bias[o].
  * w is [c_out][c_in] row-major. */
 int vdnn_fc_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
-                const float* x, const float* w, const float* bias, float* y);
+                const void* x, const float* w, const float* bias, void* y);
 /* Sgemm(N,N) (layer.cu:725-733): dx[n,i] = sum_o w[o,i] dy[n,o]. */
 int vdnn_fc_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
-                     const float* dy, const float* w, float* dx);
+                     const void* dy, const float* w, void* dx);
 /* Sgemm(N,T) alpha=-lr beta=1 (layer.cu:736-744): w[o,i] += alpha * sum_n x[n,i] dy[n,o]. */
 int vdnn_fc_bwd_weight_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
-                           const float* x, const float* dy, float* w, float alpha);
+                           const void* x, const void* dy, float* w, float alpha);
 /* Sgemm with a ones vector, alpha=-lr beta=1 (layer.cu:747-761): bias[o] += alpha * sum_n dy[n,o]. */
 int vdnn_fc_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out,
-                         const float* dy, float* bias, float alpha);
+                         const void* dy, float* bias, float alpha);
 /* The two FC reductions without the optimizer step (see vdnn_conv_bwd_filter). */
 int vdnn_fc_bwd_weight(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
-                       const float* x, const float* dy, float* dw);
-int vdnn_fc_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const float* dy, float* db);
+                       const void* x, const void* dy, float* dw);
+int vdnn_fc_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const void* dy, float* db);
 
 /* ---- bandwidth-bound layers (replaces cuDNN: layer.cu:766-915) -------------------------------- */
 /* cudnnActivationForward, ReLU, NaN propagates (layer.cu:774-781, 380-385): y = x > 0 ? x : (x!=x ? x : 0). */
-int vdnn_relu_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y);
+int vdnn_relu_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* x, void* y);
 /* cudnnActivationBackward (layer.cu:802-811): dx = x > 0 ? dy : 0. x may be NULL, then the test is
  * y > 0, which selects the same elements. */
-int vdnn_relu_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, const float* y,
-                  const float* dy, float* dx);
+int vdnn_relu_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* x, const void* y,
+                  const void* dy, void* dx);
 /* cudnnActivationForward/Backward with CUDNN_ACTIVATION_TANH / CUDNN_ACTIVATION_SIGMOID (mode chosen from
  * the layer type at layer.cu:362-369; same call sites as ReLU, layer.cu:774-781, 802-811):
  * y = tanh(x), dx = dy (1 - y^2); y = 1 / (1 + exp(-x)), dx = dy y (1 - y). Backward reads y, not x. */
-int vdnn_tanh_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y);
-int vdnn_tanh_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* y, const float* dy, float* dx);
-int vdnn_sigmoid_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y);
-int vdnn_sigmoid_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* y, const float* dy, float* dx);
+int vdnn_tanh_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* x, void* y);
+int vdnn_tanh_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* y, const void* dy, void* dx);
+int vdnn_sigmoid_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* x, void* y);
+int vdnn_sigmoid_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* y, const void* dy, void* dx);
 /* cudnnPoolingForward, max, NaN not propagated (layer.cu:875-882, 416-428). Window r x s. */
-int vdnn_maxpool_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* x, float* y);
+int vdnn_maxpool_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* x, void* y);
 /* cudnnPoolingBackward (layer.cu:903-912): each window's dy goes to its first maximum in row-major
  * window order; overlapping windows accumulate in row-major order of the windows. */
 int vdnn_maxpool_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape,
-                     const float* x, const float* y, const float* dy, float* dx);
+                     const void* x, const void* y, const void* dy, void* dx);
 /* Cross-channel LRN, window 5, alpha 1e-4, beta 0.75, k 2 (no counterpart in the reference; the
  * AlexNet configuration names it): scale = k + alpha/5 * sum_{|c'-c|<=2} x_c'^2, y = x * scale^-beta. */
-int vdnn_lrn_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const float* x, float* y);
+int vdnn_lrn_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const void* x, void* y);
 int vdnn_lrn_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw,
-                 const float* x, const float* y, const float* dy, float* dx);
+                 const void* x, const void* y, const void* dy, void* dx);
 /* cudnnSoftmaxForward ACCURATE / INSTANCE (layer.cu:824-832): per sample over `classes`. */
-int vdnn_softmax_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* x, float* y);
+int vdnn_softmax_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* x, void* y);
 /* cudnnSoftmaxBackward (layer.cu:853-862): dx_i = y_i * (dy_i - sum_j dy_j y_j). */
 int vdnn_softmax_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes,
-                     const float* y, const float* dy, float* dx);
+                     const void* y, const void* dy, void* dx);
 /* calculateDiffTensor (network.cu:3-8): r = a - b. */
-int vdnn_sub(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* a, const float* b, float* r);
+int vdnn_sub(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* a, const void* b, void* r);
 /* fillVectorWithOnes generalised (layer.cu:33-38): p[i] = value. */
-int vdnn_fill(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float value, float* p);
+int vdnn_fill(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float value, void* p);
 /* Fused softmax + cross-entropy on integer labels (no counterpart in the reference, which never
  * forms a loss): prob = softmax(logits); loss[0] = -(1/n) sum_n log prob[n,label_n], summed in
  * sample order by one workgroup. loss may be NULL. */
-int vdnn_softmax_ce_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* logits,
-                        const int32_t* labels, float* prob, float* loss);
+int vdnn_softmax_ce_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* logits,
+                        const int32_t* labels, void* prob, float* loss);
 /* dlogits = (prob - onehot(label)) / n. */
-int vdnn_softmax_ce_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* prob,
-                        const int32_t* labels, float* dlogits);
+int vdnn_softmax_ce_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* prob,
+                        const int32_t* labels, void* dlogits);
 /* Mean cross-entropy of a probability tensor against a dense target (one-hot or soft):
  * loss[0] = -(1/n) sum_n sum_c target[n,c] * log(max(prob[n,c], FLT_MIN)). Monitoring only. */
 int vdnn_cross_entropy_dense(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes,
-                             const float* prob, const float* target, float* loss);
+                             const void* prob, const void* target, float* loss);
 
 /* ---- per-kernel timing (no counterpart in the reference, whose _PROFILE_* macros are unused:
  *      layer.h:34-38) ---------------------------------------------------------------------------

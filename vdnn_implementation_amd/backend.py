@@ -53,6 +53,8 @@ _psz = C.POINTER(C.c_size_t)
 BACKEND_SYMBOLS = {
     "vdnn_ctx_create": (_i, [C.POINTER(_vp), _i, _i]),
     "vdnn_ctx_destroy": (_i, [_vp]),
+    "vdnn_ctx_set_activation_dtype": (_i, [_vp, _i]),
+    "vdnn_ctx_activation_dtype": (_i, [_vp]),
     "vdnn_last_error": (C.c_char_p, []),
     "vdnn_device_mem_info": (_i, [_vp, _psz, _psz]),
     "vdnn_device_synchronize": (_i, [_vp]),

@@ -64,6 +64,15 @@ int vdnn_ctx_create(vdnn_ctx** out, int device, int flags) {
     return VDNN_OK;
 }
 
+int vdnn_ctx_set_activation_dtype(vdnn_ctx* ctx, int dtype) {
+    VDNN_REQUIRE(ctx != nullptr, "null context");
+    VDNN_REQUIRE(dtype == VDNN_DTYPE_F32 || dtype == VDNN_DTYPE_BF16, "unknown element type");
+    ctx->act_dtype = dtype;
+    return VDNN_OK;
+}
+
+int vdnn_ctx_activation_dtype(vdnn_ctx* ctx) { return ctx ? ctx->act_dtype : VDNN_DTYPE_F32; }
+
 int vdnn_ctx_destroy(vdnn_ctx* ctx) {
     if (!ctx) return VDNN_OK;
     vdnn_pool_finalize(ctx);

@@ -23,6 +23,7 @@ struct vdnn_ctx {
     // kernels are loaded from here, so their loads need neither a branch nor a select afterwards
     const float* zeros = nullptr;
     int num_cu = 256;
+    int act_dtype = VDNN_DTYPE_F32;   // element type of activation tensors handed to the kernels
     // per-kernel timing (vdnn_profile_*)
     struct ProfRecord { const char* name; hipEvent_t start, stop; double flops, bytes; };
     bool profiling = false;
@@ -56,6 +57,9 @@ struct ProfScope {
 };
 
 } // namespace vdnn
+
+// activation tensors are float or bfloat16, as the context says; filters, biases and their gradients are float
+#define VDNN_BY_ACT(ctx, call_f32, call_bf16) ((ctx) && (ctx)->act_dtype == VDNN_DTYPE_BF16 ? (call_bf16) : (call_f32))
 
 #define VDNN_HIP(call)                                                                        \
     do {                                                                                      \

@@ -36,8 +36,8 @@ static bool geo_from_shape(const vdnn_shape_t* s, ConvGeo& g) {
 
 // samples one tile of `tile` pixels can touch, times the sample size: must stay below 2 GiB so that
 // per-lane byte offsets are positive ints and the exhausted-range scalar offset is out of range
-static bool pixel_tile_span_ok(long sample_elems, int opix, int tile) {
-    const long span = (long)(tile / opix + 2) * sample_elems * 4;
+static bool pixel_tile_span_ok(long sample_elems, int opix, int tile, int elem_bytes) {
+    const long span = (long)(tile / opix + 2) * sample_elems * elem_bytes;
     return span < 0x7FFF0000l;
 }
 
@@ -85,21 +85,21 @@ int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const fl
                          int splits, float alpha, int accumulate, const float* bias_j, int ncols);
 
 // forward with the given A loader (128-bit or 32-bit filter loads)
-template <class AL>
-static int conv_fwd_with(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const AL& al, const float* x, const float* bias, float* y) {
-    StoreNCHW ep{y, bias, g.P * g.Q};
+template <class AL, class E>
+static int conv_fwd_with(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const AL& al, const E* x, const float* bias, E* y) {
+    StoreNCHW<E> ep{y, bias, g.P * g.Q};
     const int M = g.K, N = g.N * g.P * g.Q, K = g.C * g.R * g.S;
     const FastDiv dRS = FastDiv::make(g.R * g.S), dS = FastDiv::make(g.S);
     if (g.R * g.S <= 32) {
-        LoadIm2colPix<0, false> bl{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N, dRS, dS};
+        LoadIm2colPix<0, false, E> bl{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N, dRS, dS};
         return launch_by_m(ctx, st, kFwdNames, al, bl, ep, M, N, K);
     }
-    LoadIm2colPix<0, true> bl{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N, dRS, dS};
+    LoadIm2colPix<0, true, E> bl{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N, dRS, dS};
     return launch_by_m(ctx, st, kFwdNames, al, bl, ep, M, N, K);
 }
 
 template <class AL, class BL>
-static int conv_wgrad_with(vdnn_ctx* ctx, hipStream_t st, const AL& al, const BL& bl, const StoreDense& ep, const GemmDims& d, bool narrow) {
+static int conv_wgrad_with(vdnn_ctx* ctx, hipStream_t st, const AL& al, const BL& bl, const StoreDense<float>& ep, const GemmDims& d, bool narrow) {
     return narrow ? launch_igemm<64, 256>(ctx, st, kBwdFilterNames.t64, al, bl, ep, d)
                   : launch_igemm<128, 128>(ctx, st, kBwdFilterNames.t128, al, bl, ep, d);
 }
@@ -128,49 +128,24 @@ static int launch_pack_filter(vdnn_ctx* ctx, hipStream_t st, const float* w, flo
 
 using namespace vdnn;
 
-extern "C" {
-
-size_t vdnn_conv_workspace_bytes(const vdnn_shape_t* shape, int algo_mode, int pass) {
-    ConvGeo g;
-    if (!shape || !geo_from_shape(shape, g)) return 0;
-    if (algo_mode == 0 /* VDNN_MEMORY_OPT_ALGO */) return 0;
-    // Perf-optimal mode: forward and backward data re-lay the filter bank out for 128-bit operand
-    // loads; backward filter takes a staging area large enough for the split count that fills the chip.
-    const int RS = g.R * g.S;
-    const size_t filter_bytes = (size_t)g.K * g.C * RS * sizeof(float);
-    if (pass == 0) return packed_fwd_ok(g) ? filter_bytes : 0;
-    if (pass == 1) return packed_bwd_data_ok(g) ? filter_bytes : 0;
-    const int M = g.K, N = g.C * RS;
-    const bool narrow = M <= 64;
-    const int TM = narrow ? 64 : 128, TN = narrow ? 256 : 128;
-    const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
-    long cap = ((long)g.N * g.P * g.Q + 4 * KB - 1) / (4 * KB);
-    const long by_mem = (long)(kMaxWgradWorkspace / filter_bytes);
-    if (cap > by_mem) cap = by_mem;
-    const int want = choose_splits(tiles, (long)g.N * g.P * g.Q, cap, kPlanningCUs, filter_bytes, 2.0 * TM * TN * KB);
-    if (want <= 1) return 0;
-    const size_t need = (size_t)want * filter_bytes;
-    if (need <= kDefaultStagingBytes) return 0; // the context's own staging area already holds it
-    return need;
-}
-
-int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
-                  const float* x, const float* w, const float* bias, float* y,
-                  void* workspace, size_t workspace_bytes) {
+template <class E>
+static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                         const E* x, const float* w, const float* bias, E* y,
+                         void* workspace, size_t workspace_bytes) {
     VDNN_KERNEL_PROLOGUE(ctx);
     ConvGeo g;
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(x && w && y, "null tensor");
-    VDNN_REQUIRE(pixel_tile_span_ok((long)g.C * g.H * g.W, g.P * g.Q, 256), "input samples too large for one tile's descriptor");
+    VDNN_REQUIRE(pixel_tile_span_ok((long)g.C * g.H * g.W, g.P * g.Q, 256, (int)sizeof(E)), "input samples too large for one tile's descriptor");
     hipStream_t st = stream_of(ctx, stream);
     const int K = g.C * g.R * g.S;
     const unsigned wbytes = (unsigned)((long)g.K * K * 4);
     if (g.R * g.S <= 32 && g.C % KB == 0) {
         // blocked tap-major reduction: one slice = one tap x 16 input channels
         const int RS = g.R * g.S;
-        LoadIm2colPixTap<0> bl{{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N,
+        LoadIm2colPixTap<0, E> bl{{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N,
                                 FastDiv::make(RS), FastDiv::make(g.S)}};
-        StoreNCHW ep{y, bias, g.P * g.Q};
+        StoreNCHW<E> ep{y, bias, g.P * g.Q};
         if (algo_mode == 1 && workspace && workspace_bytes >= wbytes && aligned16(workspace)) {
             // perf-optimal: the filter bank, re-laid-out in the workspace, is a dense 128-bit operand
             float* packed = (float*)workspace;
@@ -190,9 +165,10 @@ int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape
     return conv_fwd_with(ctx, st, g, al, x, bias, y);
 }
 
-int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
-                       const float* dy, const float* w, float* dx,
-                       void* workspace, size_t workspace_bytes) {
+template <class E>
+static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                              const E* dy, const float* w, E* dx,
+                              void* workspace, size_t workspace_bytes) {
     VDNN_KERNEL_PROLOGUE(ctx);
     ConvGeo g;
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
@@ -204,17 +180,17 @@ int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* 
         VDNN_REQUIRE(blocks < (1l << 31), "grid too large");
         ProfScope prof(ctx, st, "conv_bwd_data_smallc", 2.0 * g.C * (double)g.N * g.P * g.Q * g.K * g.R * g.S, 0.0);
         const bool s1_3x3 = g.sh == 1 && g.sw == 1 && g.R == 3 && g.S == 3;
-        if (s1_3x3 && g.C == 3) hipLaunchKernelGGL((conv_bwd_data_smallc_s1_kernel<3, 3, 3>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
-        else if (s1_3x3 && g.C == 4) hipLaunchKernelGGL((conv_bwd_data_smallc_s1_kernel<3, 3, 4>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
-        else if (g.sh == 1 && g.sw == 1) hipLaunchKernelGGL(conv_bwd_data_smallc_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
-        else hipLaunchKernelGGL(conv_bwd_data_smallc_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
+        if (s1_3x3 && g.C == 3) hipLaunchKernelGGL((conv_bwd_data_smallc_s1_kernel<3, 3, 3, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
+        else if (s1_3x3 && g.C == 4) hipLaunchKernelGGL((conv_bwd_data_smallc_s1_kernel<3, 3, 4, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
+        else if (g.sh == 1 && g.sw == 1) hipLaunchKernelGGL((conv_bwd_data_smallc_kernel<true, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
+        else hipLaunchKernelGGL((conv_bwd_data_smallc_kernel<false, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
         VDNN_LAUNCH_CHECK();
         return VDNN_OK;
     }
-    VDNN_REQUIRE(pixel_tile_span_ok((long)g.K * g.P * g.Q, g.H * g.W, 256), "output-gradient samples too large for one tile's descriptor");
+    VDNN_REQUIRE(pixel_tile_span_ok((long)g.K * g.P * g.Q, g.H * g.W, 256, (int)sizeof(E)), "output-gradient samples too large for one tile's descriptor");
     const int RS = g.R * g.S;
     LoadFilterT al{w, g.C, RS, (unsigned)((long)g.K * g.C * RS * 4), FastDiv::make(RS)};
-    StoreNCHW ep{dx, nullptr, g.H * g.W};
+    StoreNCHW<E> ep{dx, nullptr, g.H * g.W};
     const int M = g.C, N = g.N * g.H * g.W, K = g.K * RS;
     const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S);
     const long sample = (long)g.K * g.P * g.Q;
@@ -222,7 +198,7 @@ int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* 
         if (RS <= 32 && g.K % KB == 0) {
             // blocked tap-major reduction: one slice = one tap x 16 output channels
             const unsigned wbytes = (unsigned)((long)g.K * g.C * RS * 4);
-            LoadIm2colPixTap<1> bl{{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS}};
+            LoadIm2colPixTap<1, E> bl{{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS}};
             if (algo_mode == 1 && workspace && workspace_bytes >= wbytes && aligned16(workspace)) {
                 float* packed = (float*)workspace; // [c][(kb*RS + tap)*16 + l]
                 const int rc = launch_pack_filter(ctx, st, w, packed, g.C, g.K, RS, RS, g.C * RS);
@@ -234,19 +210,20 @@ int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* 
             return launch_by_m(ctx, st, kBwdDataNames, alt, bl, ep, M, N, K);
         }
         if (RS <= 32) {
-            LoadIm2colPix<1, false> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS};
+            LoadIm2colPix<1, false, E> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS};
             return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K);
         }
-        LoadIm2colPix<1, true> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS};
+        LoadIm2colPix<1, true, E> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS};
         return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K);
     }
-    LoadIm2colPix<2, true> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, g.sh, g.sw, sample, g.N, dRS, dS};
+    LoadIm2colPix<2, true, E> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, g.sh, g.sw, sample, g.N, dRS, dS};
     return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K);
 }
 
 // out = (accumulate ? out : 0) + alpha * dW
+template <class E>
 static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
-                                const float* x, const float* dy, float* w, float alpha, int accumulate,
+                                const E* x, const E* dy, float* w, float alpha, int accumulate,
                                 void* workspace, size_t workspace_bytes) {
     VDNN_KERNEL_PROLOGUE(ctx);
     (void)algo_mode;
@@ -275,10 +252,10 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
         {
             ProfScope prof(ctx, st, "conv_bwd_filter_smallc", 2.0 * (double)M * N * (double)Kred, 0.0);
             switch (g.C) {
-            case 1: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<1, 4>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
-            case 2: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<2, 4>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
-            case 3: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<3, 4>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
-            default: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<4, 4>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
+            case 1: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<1, 4, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
+            case 2: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<2, 4, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
+            case 3: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<3, 4, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
+            default: hipLaunchKernelGGL((conv_bwd_filter_smallc3x3_kernel<4, 4, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, x, staging, g, per, step); break;
             }
             VDNN_LAUNCH_CHECK();
         }
@@ -300,17 +277,17 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     GemmDims d = make_dims(M, N, (int)Kred, TM, TN, want);
     // one split's samples of dy and of x are addressed through one descriptor with summed offsets
     const long nspan = d.kchunk / PQ + 2;
-    VDNN_REQUIRE(nspan * g.K * PQ * 4 < (long)MAX_SUM_RANGE && nspan * g.C * g.H * g.W * 4 < (long)MAX_SUM_RANGE,
+    VDNN_REQUIRE(nspan * g.K * PQ * (long)sizeof(E) < (long)MAX_SUM_RANGE && nspan * g.C * g.H * g.W * (long)sizeof(E) < (long)MAX_SUM_RANGE,
                  "samples of one reduction split too large for one descriptor");
-    StoreDense ep{w, staging, nullptr, (long)N, (long)M * N, alpha, accumulate};
+    StoreDense<float> ep{w, staging, nullptr, (long)N, (long)M * N, alpha, accumulate};
     const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S), dQ = FastDiv::make(g.Q);
-    const bool vec = PQ % 4 == 0 && aligned16(dy);
+    const bool vec = PQ % 4 == 0 && aligned16(dy); // bf16: four elements are 8 bytes, covered by the same test
     const bool big = RS > 32;
     int rc;
 #define VDNN_WGRAD(VEC, BIG)                                                                                              \
     do {                                                                                                                  \
-        LoadDyRed<VEC> al{dy, g.N, g.K, PQ, d.kchunk, d.K};                                                               \
-        LoadIm2colRed<BIG> bl{x, g.N, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N, d.kchunk, d.K, dRS, dS, dQ}; \
+        LoadDyRed<VEC, E> al{dy, g.N, g.K, PQ, d.kchunk, d.K};                                                               \
+        LoadIm2colRed<BIG, E> bl{x, g.N, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N, d.kchunk, d.K, dRS, dS, dQ}; \
         rc = conv_wgrad_with(ctx, st, al, bl, ep, d, narrow);                                                             \
     } while (0)
     if (vec && !big) VDNN_WGRAD(true, false);
@@ -323,15 +300,57 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     return VDNN_OK;
 }
 
+extern "C" {
+
+size_t vdnn_conv_workspace_bytes(const vdnn_shape_t* shape, int algo_mode, int pass) {
+    ConvGeo g;
+    if (!shape || !geo_from_shape(shape, g)) return 0;
+    if (algo_mode == 0 /* VDNN_MEMORY_OPT_ALGO */) return 0;
+    // Perf-optimal mode: forward and backward data re-lay the filter bank out for 128-bit operand
+    // loads; backward filter takes a staging area large enough for the split count that fills the chip.
+    const int RS = g.R * g.S;
+    const size_t filter_bytes = (size_t)g.K * g.C * RS * sizeof(float);
+    if (pass == 0) return packed_fwd_ok(g) ? filter_bytes : 0;
+    if (pass == 1) return packed_bwd_data_ok(g) ? filter_bytes : 0;
+    const int M = g.K, N = g.C * RS;
+    const bool narrow = M <= 64;
+    const int TM = narrow ? 64 : 128, TN = narrow ? 256 : 128;
+    const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
+    long cap = ((long)g.N * g.P * g.Q + 4 * KB - 1) / (4 * KB);
+    const long by_mem = (long)(kMaxWgradWorkspace / filter_bytes);
+    if (cap > by_mem) cap = by_mem;
+    const int want = choose_splits(tiles, (long)g.N * g.P * g.Q, cap, kPlanningCUs, filter_bytes, 2.0 * TM * TN * KB);
+    if (want <= 1) return 0;
+    const size_t need = (size_t)want * filter_bytes;
+    if (need <= kDefaultStagingBytes) return 0; // the context's own staging area already holds it
+    return need;
+}
+
+int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                  const void* x, const float* w, const float* bias, void* y,
+                  void* workspace, size_t workspace_bytes) {
+    return VDNN_BY_ACT(ctx, conv_fwd_impl<float>(ctx, stream, shape, algo_mode, (const float*)x, w, bias, (float*)y, workspace, workspace_bytes),
+                       conv_fwd_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)x, w, bias, (bf16_t*)y, workspace, workspace_bytes));
+}
+
+int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                       const void* dy, const float* w, void* dx,
+                       void* workspace, size_t workspace_bytes) {
+    return VDNN_BY_ACT(ctx, conv_bwd_data_impl<float>(ctx, stream, shape, algo_mode, (const float*)dy, w, (float*)dx, workspace, workspace_bytes),
+                       conv_bwd_data_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)dy, w, (bf16_t*)dx, workspace, workspace_bytes));
+}
+
 int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
-                             const float* x, const float* dy, float* w, float alpha,
+                             const void* x, const void* dy, float* w, float alpha,
                              void* workspace, size_t workspace_bytes) {
-    return conv_bwd_filter_impl(ctx, stream, shape, algo_mode, x, dy, w, alpha, 1, workspace, workspace_bytes);
+    return VDNN_BY_ACT(ctx, conv_bwd_filter_impl<float>(ctx, stream, shape, algo_mode, (const float*)x, (const float*)dy, w, alpha, 1, workspace, workspace_bytes),
+                       conv_bwd_filter_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)x, (const bf16_t*)dy, w, alpha, 1, workspace, workspace_bytes));
 }
 
 int vdnn_conv_bwd_filter(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
-                         const float* x, const float* dy, float* dw, void* workspace, size_t workspace_bytes) {
-    return conv_bwd_filter_impl(ctx, stream, shape, algo_mode, x, dy, dw, 1.0f, 0, workspace, workspace_bytes);
+                         const void* x, const void* dy, float* dw, void* workspace, size_t workspace_bytes) {
+    return VDNN_BY_ACT(ctx, conv_bwd_filter_impl<float>(ctx, stream, shape, algo_mode, (const float*)x, (const float*)dy, dw, 1.0f, 0, workspace, workspace_bytes),
+                       conv_bwd_filter_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)x, (const bf16_t*)dy, dw, 1.0f, 0, workspace, workspace_bytes));
 }
 
 } // extern "C"

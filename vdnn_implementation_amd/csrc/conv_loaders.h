@@ -29,10 +29,11 @@ __device__ __forceinline__ unsigned valid_window_bits(int origin, int window, in
 // (ch, r, s) is wave-uniform and goes into the scalar offset, and the pixel's out-of-image taps are a
 // bit mask that is OR-ed into the offset as all-ones. BIGWIN: windows of more than 32 taps keep
 // separate row and column masks.
-template <int MODE, bool BIGWIN>
+template <int MODE, bool BIGWIN, class E = float>
 struct LoadIm2colPix {
     static constexpr bool RED_MAJOR = false;
-    const float* src;
+    static constexpr int ES = ElemBytes<E>::V;
+    const E* src;
     int Hs, Ws;      // extent of one source plane
     int OH, OW;      // extent of the output pixel grid
     int R, S, ph, pw, sh, sw;
@@ -61,22 +62,22 @@ struct LoadIm2colPix {
         if (MODE == 0) {
             shift = -((long)ph * Ws + pw);
             ih0 = oh * sh - ph; iw0 = ow * sw - pw;
-            st.vbase = (int)(((long)(n - n_first) * sample_elems + (long)oh * sh * Ws + ow * sw) * 4);
+            st.vbase = (int)(((long)(n - n_first) * sample_elems + (long)oh * sh * Ws + ow * sw) * ES);
         } else if (MODE == 1) {
             shift = (long)(ph - R + 1) * Ws + (pw - S + 1);
             ih0 = oh + ph; iw0 = ow + pw;
-            st.vbase = (int)(((long)(n - n_first) * sample_elems + (long)oh * Ws + ow) * 4);
+            st.vbase = (int)(((long)(n - n_first) * sample_elems + (long)oh * Ws + ow) * ES);
         } else {
             shift = 0;
             ih0 = oh + ph; iw0 = ow + pw;
-            st.vbase = (int)((long)(n - n_first) * sample_elems * 4);
+            st.vbase = (int)((long)(n - n_first) * sample_elems * ES);
         }
         st.ih0 = ih0; st.iw0 = iw0;
         // the descriptor covers only the samples this tile touches (the host checks that this is
         // below 2 GiB, so the scalar offset 0x7FFFFFF0 of an exhausted reduction range is out of range)
         int n_last = (j0 + T - 1) / opix;
         if (n_last > nsamples - 1) n_last = nsamples - 1;
-        st.rsrc = make_rsrc(src + first + shift, clamp_range(((long)(n_last - n_first + 1) * sample_elems - shift) * 4));
+        st.rsrc = make_rsrc(src + first + shift, clamp_range(((long)(n_last - n_first + 1) * sample_elems - shift) * ES));
         unsigned vrow = 0, vcol = 0; // valid taps
         for (int r = 0; r < R; r++) {
             bool ok;
@@ -110,14 +111,14 @@ struct LoadIm2colPix {
             const int ch = divRS.div(kk), rs = kk - ch * RS;
             const int tr = divS.div(rs), ts = rs - tr * S;
             int soff, voff;
-            if (MODE == 0) soff = (ch * plane + tr * Ws + ts) * 4;
-            else if (MODE == 1) soff = (ch * plane + (R - 1 - tr) * Ws + (S - 1 - ts)) * 4;
-            else soff = ch * plane * 4;
+            if (MODE == 0) soff = (ch * plane + tr * Ws + ts) * ES;
+            else if (MODE == 1) soff = (ch * plane + (R - 1 - tr) * Ws + (S - 1 - ts)) * ES;
+            else soff = ch * plane * ES;
             if (kk >= kend) soff = 0x7FFFFFF0;
             const int dead = BIGWIN || MODE == 2 ? (bit_to_all_ones(st.invrow, tr) | bit_to_all_ones(st.invcol, ts)) : bit_to_all_ones(st.inv, rs);
-            if (MODE == 2) voff = (st.vbase + (((st.ih0 - tr) / sh) * Ws + (st.iw0 - ts) / sw) * 4) | dead;
+            if (MODE == 2) voff = (st.vbase + (((st.ih0 - tr) / sh) * Ws + (st.iw0 - ts) / sw) * ES) | dead;
             else voff = st.vbase | dead;
-            r.s[i] = buf_load(st.rsrc, voff, soff);
+            r.s[i] = buf_load_e<E>(st.rsrc, voff, soff);
         }
     }
     template <int T>
@@ -181,10 +182,11 @@ struct PixelCursor {
 // ---- dy as the A operand of backward filter: A[k][(n,p,q)] = dy[n,k,p,q] -------------------------
 // The descriptor starts at the first sample of the workgroup's reduction range. VEC4 (plane size a
 // multiple of four): 128-bit chunks, thread t: chunk t%4 of rows t/4 + 64*i; else 32-bit elements.
-template <bool VEC4>
+template <bool VEC4, class E = float>
 struct LoadDyRed {
     static constexpr bool RED_MAJOR = true;
-    const float* dy;
+    static constexpr int ES = ElemBytes<E>::V;
+    const E* dy;
     int N, K, PQ;
     int kchunk, Ktot; // reduction indices per split and in total
     template <int T> struct Regs { floatx4 v[T / 64]; float s[VEC4 ? 1 : T / 16]; };
@@ -195,26 +197,26 @@ struct LoadDyRed {
         const int n_first = k_begin / PQ;
         int k_last = k_begin + kchunk; if (k_last > Ktot) k_last = Ktot;
         const int n_last = k_last > k_begin ? (k_last - 1) / PQ : n_first;
-        st.rsrc = make_rsrc(dy + (long)n_first * K * PQ, clamp_range((long)(n_last - n_first + 1) * K * PQ * 4));
+        st.rsrc = make_rsrc(dy + (long)n_first * K * PQ, clamp_range((long)(n_last - n_first + 1) * K * PQ * ES));
         st.kk = k_begin + (VEC4 ? 4 * (tid & 3) : (tid & 15));
         st.cur.init(st.kk, PQ, n_first);
         if (VEC4) {
 #pragma unroll
-            for (int i = 0; i < T / 64; i++) { const int m = row0 + (tid >> 2) + 64 * i; st.mrow[i] = m < K ? m * PQ * 4 : SENT; }
+            for (int i = 0; i < T / 64; i++) { const int m = row0 + (tid >> 2) + 64 * i; st.mrow[i] = m < K ? m * PQ * ES : SENT; }
         } else {
 #pragma unroll
-            for (int i = 0; i < T / 16; i++) { const int m = row0 + (tid >> 4) + 16 * i; st.mrow[i] = m < K ? m * PQ * 4 : SENT; }
+            for (int i = 0; i < T / 16; i++) { const int m = row0 + (tid >> 4) + 16 * i; st.mrow[i] = m < K ? m * PQ * ES : SENT; }
         }
     }
     template <int T>
     __device__ __forceinline__ void load(State<T>& st, int, int kend, int, Regs<T>& r) const {
-        const int npart = st.kk < kend ? (st.cur.n * K * PQ + st.cur.pq) * 4 : SENT;
+        const int npart = st.kk < kend ? (st.cur.n * K * PQ + st.cur.pq) * ES : SENT;
         if (VEC4) {
 #pragma unroll
-            for (int i = 0; i < T / 64; i++) r.v[i] = buf_load4(st.rsrc, st.mrow[i] + npart, 0);
+            for (int i = 0; i < T / 64; i++) r.v[i] = buf_load4_e<E>(st.rsrc, st.mrow[i] + npart, 0);
         } else {
 #pragma unroll
-            for (int i = 0; i < T / 16; i++) r.s[i] = buf_load(st.rsrc, st.mrow[i] + npart, 0);
+            for (int i = 0; i < T / 16; i++) r.s[i] = buf_load_e<E>(st.rsrc, st.mrow[i] + npart, 0);
         }
         st.kk += KB;
         st.cur.advance(PQ);
@@ -234,17 +236,18 @@ struct LoadDyRed {
 // ---- im2col operand of backward filter: B[(n,p,q)][(c,r,s)] = x[n,c,p*sh-ph+r,q*sw-pw+s] ---------
 // reduction-major: thread t owns pixel t%16 of the slice and columns t/16 + 16*i. Per slice it
 // derives the pixel's offset and its mask of out-of-image taps once; each column adds a constant.
-template <bool BIGWIN>
+template <bool BIGWIN, class E = float>
 struct LoadIm2colRed {
     static constexpr bool RED_MAJOR = true;
-    const float* x;
+    static constexpr int ES = ElemBytes<E>::V;
+    const E* x;
     int N, C, H, W, R, S, P, Q, ph, pw, sh, sw;
     int ncols; // C*R*S
     int kchunk, Ktot; // reduction indices per split and in total
     FastDiv divRS, divS, divQ;
     template <int T> struct Regs { float s[T / 16]; };
     template <int T> struct State {
-        int jconst[T / 16]; // (c*H*W + r*W + s) * 4, or SENT for a column outside the matrix
+        int jconst[T / 16]; // byte offset of (c*H*W + r*W + s), or SENT for a column outside the matrix
         int tap[T / 16];    // r*S + s (BIGWIN: r << 8 | s)
         PixelCursor cur; int kk;
         __amdgpu_buffer_rsrc_t rsrc;
@@ -257,7 +260,7 @@ struct LoadIm2colRed {
         const long shift = -((long)ph * W + pw);
         int k_last = k_begin + kchunk; if (k_last > Ktot) k_last = Ktot;
         const int n_last = k_last > k_begin ? (k_last - 1) / PQ : n_first;
-        st.rsrc = make_rsrc(x + (long)n_first * chw + shift, clamp_range(((long)(n_last - n_first + 1) * chw - shift) * 4));
+        st.rsrc = make_rsrc(x + (long)n_first * chw + shift, clamp_range(((long)(n_last - n_first + 1) * chw - shift) * ES));
         st.kk = k_begin + (tid & 15);
         st.cur.init(st.kk, PQ, n_first);
 #pragma unroll
@@ -266,7 +269,7 @@ struct LoadIm2colRed {
             if (j < ncols) {
                 const int c = divRS.div(j), rs = j - c * RS;
                 const int r = divS.div(rs), s = rs - r * S;
-                st.jconst[i] = (c * H * W + r * W + s) * 4;
+                st.jconst[i] = (c * H * W + r * W + s) * ES;
                 st.tap[i] = BIGWIN ? ((r << 8) | s) : rs;
             } else {
                 st.jconst[i] = SENT;
@@ -279,14 +282,14 @@ struct LoadIm2colRed {
         const int PQ = P * Q;
         const int p = divQ.div(st.cur.pq), q = st.cur.pq - p * Q;
         const int ih0 = p * sh - ph, iw0 = q * sw - pw;
-        const int pixbase = st.kk < kend ? (st.cur.n * C * H * W + p * sh * W + q * sw) * 4 : SENT;
+        const int pixbase = st.kk < kend ? (st.cur.n * C * H * W + p * sh * W + q * sw) * ES : SENT;
         const unsigned vrow = valid_window_bits(ih0, R, H), vcol = valid_window_bits(iw0, S, W);
         if (BIGWIN) {
             const unsigned invrow = ~vrow, invcol = ~vcol;
 #pragma unroll
             for (int i = 0; i < T / 16; i++) {
                 const int dead = bit_to_all_ones(invrow, st.tap[i] >> 8) | bit_to_all_ones(invcol, st.tap[i] & 255);
-                r.s[i] = buf_load(st.rsrc, (pixbase + st.jconst[i]) | dead, 0);
+                r.s[i] = buf_load_e<E>(st.rsrc, (pixbase + st.jconst[i]) | dead, 0);
             }
         } else {
             unsigned v = 0;
@@ -294,7 +297,7 @@ struct LoadIm2colRed {
             const unsigned inv = ~v;
 #pragma unroll
             for (int i = 0; i < T / 16; i++)
-                r.s[i] = buf_load(st.rsrc, (pixbase + st.jconst[i]) | bit_to_all_ones(inv, st.tap[i]), 0);
+                r.s[i] = buf_load_e<E>(st.rsrc, (pixbase + st.jconst[i]) | bit_to_all_ones(inv, st.tap[i]), 0);
         }
         st.kk += KB;
         st.cur.advance(PQ);
@@ -307,8 +310,9 @@ struct LoadIm2colRed {
 };
 
 // ---- result of forward / backward data: out[n][m][pix] = acc (+ bias[m]) --------------------------
+template <class E = float>
 struct StoreNCHW {
-    float* out;
+    E* out;
     const float* bias; // optional, per output channel
     int opix;          // pixels of one output plane
     __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int, const GemmDims& d) const {
@@ -318,7 +322,7 @@ struct StoreNCHW {
             const int j = j0 + jt * 32 + l32;
             if (j >= d.N) continue;
             const int n = j / opix, pix = j - n * opix;
-            float* o = out + (size_t)n * d.M * opix + pix;
+            E* o = out + (size_t)n * d.M * opix + pix;
 #pragma unroll
             for (int it = 0; it < 2; it++)
 #pragma unroll
@@ -327,7 +331,7 @@ struct StoreNCHW {
                     if (m >= d.M) continue;
                     float r = acc[it][jt][v];
                     if (bias) r += bias[m];
-                    o[(size_t)m * opix] = r;
+                    store_elem(o + (size_t)m * opix, r);
                 }
         }
     }

@@ -56,12 +56,13 @@ struct LoadFilterTap {
 
 // ---- im2col operand, columns = output pixels, tap-major reduction ------------------------------------
 // MODE 0: forward gather from x; MODE 1: backward data at stride 1 (src = dy). At most 32 taps.
-template <int MODE>
+template <int MODE, class E = float>
 struct LoadIm2colPixTap {
     static constexpr bool RED_MAJOR = false;
-    LoadIm2colPix<MODE, false> base; // geometry and per-pixel state are those of the channel-major loader
-    template <int T> using Regs = typename LoadIm2colPix<MODE, false>::template Regs<T>;
-    template <int T> using State = typename LoadIm2colPix<MODE, false>::template State<T>;
+    static constexpr int ES = ElemBytes<E>::V;
+    LoadIm2colPix<MODE, false, E> base; // geometry and per-pixel state are those of the channel-major loader
+    template <int T> using Regs = typename LoadIm2colPix<MODE, false, E>::template Regs<T>;
+    template <int T> using State = typename LoadIm2colPix<MODE, false, E>::template State<T>;
     template <int T>
     __device__ __forceinline__ void init(State<T>& st, int j0, int tid, int ncols, int k_begin) const {
         base.template init<T>(st, j0, tid, ncols, k_begin);
@@ -75,13 +76,13 @@ struct LoadIm2colPixTap {
         const int tapoff = MODE == 0 ? tr * base.Ws + ts : (base.R - 1 - tr) * base.Ws + (base.S - 1 - ts);
         const int voff = st.vbase | bit_to_all_ones(st.inv, tap);
         const int chb = ch0 + __builtin_amdgcn_readfirstlane(tid / T);
-        const int soff0 = (chb * plane + tapoff) * 4, step = (NT / T) * plane * 4;
+        const int soff0 = (chb * plane + tapoff) * ES, step = (NT / T) * plane * ES;
 #pragma unroll
-        for (int i = 0; i < T * KB / NT; i++) r.s[i] = buf_load(st.rsrc, voff, soff0 + i * step);
+        for (int i = 0; i < T * KB / NT; i++) r.s[i] = buf_load_e<E>(st.rsrc, voff, soff0 + i * step);
     }
     template <int T>
     __device__ static __forceinline__ void store(float* lds, int tid, const Regs<T>& r) {
-        LoadIm2colPix<MODE, false>::template store<T>(lds, tid, r);
+        LoadIm2colPix<MODE, false, E>::template store<T>(lds, tid, r);
     }
 };
 

@@ -15,9 +15,9 @@ namespace vdnn {
 constexpr int SMALLC_KC = 8;
 constexpr int SMALLC_MAXTAPS = 128;
 
-template <bool STRIDE1>
-__global__ void __launch_bounds__(256) conv_bwd_data_smallc_kernel(const float* __restrict__ dy, const float* __restrict__ w,
-                                                                   float* __restrict__ dx, const ConvGeo g) {
+template <bool STRIDE1, class E>
+__global__ void __launch_bounds__(256) conv_bwd_data_smallc_kernel(const E* __restrict__ dy, const float* __restrict__ w,
+                                                                   E* __restrict__ dx, const ConvGeo g) {
     __shared__ float4 ws[SMALLC_KC][SMALLC_MAXTAPS];
     const int tid = threadIdx.x;
     const int RS = g.R * g.S;
@@ -43,7 +43,7 @@ __global__ void __launch_bounds__(256) conv_bwd_data_smallc_kernel(const float* 
         if (!live) continue;
         const int kmax = min(SMALLC_KC, g.K - k0);
         for (int kk = 0; kk < kmax; kk++) {
-            const float* dyp = dy + ((long)n * g.K + k0 + kk) * g.P * g.Q;
+            const E* dyp = dy + ((long)n * g.K + k0 + kk) * g.P * g.Q;
             for (int r = 0; r < g.R; r++) {
                 int p = th - r;
                 if (STRIDE1) {
@@ -53,7 +53,7 @@ __global__ void __launch_bounds__(256) conv_bwd_data_smallc_kernel(const float* 
                     p /= g.sh;
                     if (p >= g.P) continue;
                 }
-                const float* row = dyp + (long)p * g.Q;
+                const E* row = dyp + (long)p * g.Q;
                 for (int s = 0; s < g.S; s++) {
                     int q = tw - s;
                     if (STRIDE1) {
@@ -63,7 +63,7 @@ __global__ void __launch_bounds__(256) conv_bwd_data_smallc_kernel(const float* 
                         q /= g.sw;
                         if (q >= g.Q) continue;
                     }
-                    const float d = row[q];
+                    const float d = load_elem(row + q);
                     const float4 f = ws[kk][r * g.S + s];
                     acc.x += d * f.x; acc.y += d * f.y; acc.z += d * f.z; acc.w += d * f.w;
                 }
@@ -71,20 +71,20 @@ __global__ void __launch_bounds__(256) conv_bwd_data_smallc_kernel(const float* 
         }
     }
     if (!live) return;
-    float* o = dx + (long)n * g.C * g.H * g.W + hw;
+    E* o = dx + (long)n * g.C * g.H * g.W + hw;
     const long plane = (long)g.H * g.W;
-    o[0] = acc.x;
-    if (g.C > 1) o[plane] = acc.y;
-    if (g.C > 2) o[2 * plane] = acc.z;
-    if (g.C > 3) o[3 * plane] = acc.w;
+    store_elem(o, acc.x);
+    if (g.C > 1) store_elem(o + plane, acc.y);
+    if (g.C > 2) store_elem(o + 2 * plane, acc.z);
+    if (g.C > 3) store_elem(o + 3 * plane, acc.w);
 }
 
 // The same, for a compile-time window at stride 1 (VGG's 3x3): fully unrolled and branch-free. Taps
 // outside dy are read from a clamped position and replaced by zero. The filter values of one output
 // channel are wave-uniform, so they are fetched with scalar loads straight from global memory.
-template <int RC, int SC, int CC>
-__global__ void __launch_bounds__(256) conv_bwd_data_smallc_s1_kernel(const float* __restrict__ dy, const float* __restrict__ w,
-                                                                      float* __restrict__ dx, const ConvGeo g) {
+template <int RC, int SC, int CC, class E>
+__global__ void __launch_bounds__(256) conv_bwd_data_smallc_s1_kernel(const E* __restrict__ dy, const float* __restrict__ w,
+                                                                      E* __restrict__ dx, const ConvGeo g) {
     constexpr int RS = RC * SC;
     const int tid = threadIdx.x;
     const long pix = (long)blockIdx.x * 256 + tid;
@@ -112,15 +112,15 @@ __global__ void __launch_bounds__(256) conv_bwd_data_smallc_s1_kernel(const floa
 #pragma unroll
     for (int c = 0; c < CC; c++) acc[c] = 0.f;
     const long kstride = (long)g.P * g.Q;
-    const float* dyp = dy + (long)n * g.K * kstride;
+    const E* dyp = dy + (long)n * g.K * kstride;
     for (int k = 0; k < g.K; k++, dyp += kstride) {
         const float* wk = w + (long)k * CC * RS; // uniform: scalar loads
 #pragma unroll
         for (int r = 0; r < RC; r++) {
-            const float* row = dyp + rowoff[r];
+            const E* row = dyp + rowoff[r];
 #pragma unroll
             for (int s = 0; s < SC; s++) {
-                const float v = row[col[s]];
+                const float v = load_elem(row + col[s]);
                 const float d = (rowok[r] & colok[s]) ? v : 0.0f;
 #pragma unroll
                 for (int c = 0; c < CC; c++) acc[c] += d * wk[c * RS + r * SC + s];
@@ -128,10 +128,10 @@ __global__ void __launch_bounds__(256) conv_bwd_data_smallc_s1_kernel(const floa
         }
     }
     if (!live) return;
-    float* o = dx + (long)n * CC * g.H * g.W + hw;
+    E* o = dx + (long)n * CC * g.H * g.W + hw;
     const long plane = (long)g.H * g.W;
 #pragma unroll
-    for (int c = 0; c < CC; c++) o[c * plane] = acc[c];
+    for (int c = 0; c < CC; c++) store_elem(o + c * plane, acc[c]);
 }
 
 // ---- backward filter for 3x3 layers with at most four input channels ------------------------------
@@ -143,8 +143,8 @@ __global__ void __launch_bounds__(256) conv_bwd_data_smallc_s1_kernel(const floa
 // reduction that also applies the SGD step.
 struct PixelStep { int dn, dp, dq; }; // 256 pixels = dn samples + dp rows + dq columns
 
-template <int CC, int KG>
-__global__ void __launch_bounds__(256) conv_bwd_filter_smallc3x3_kernel(const float* __restrict__ dy, const float* __restrict__ x,
+template <int CC, int KG, class E>
+__global__ void __launch_bounds__(256) conv_bwd_filter_smallc3x3_kernel(const E* __restrict__ dy, const E* __restrict__ x,
                                                                         float* __restrict__ partial, const ConvGeo g,
                                                                         long pix_per_chunk, PixelStep step) {
     constexpr int TAPS = CC * 9;
@@ -171,7 +171,7 @@ __global__ void __launch_bounds__(256) conv_bwd_filter_smallc3x3_kernel(const fl
     const long plane = (long)g.H * g.W;
     for (; pix < pix1; pix += 256) {
         const int ih0 = p * g.sh - g.ph, iw0 = q * g.sw - g.pw;
-        const float* xs = x + (long)n * CC * plane;
+        const E* xs = x + (long)n * CC * plane;
         float xv[TAPS];
 #pragma unroll
         for (int r = 0; r < 3; r++) {
@@ -185,15 +185,15 @@ __global__ void __launch_bounds__(256) conv_bwd_filter_smallc3x3_kernel(const fl
                 const int iwc = ((unsigned)iw < (unsigned)g.W) ? iw : 0;
 #pragma unroll
                 for (int c = 0; c < CC; c++) {
-                    const float val = xs[c * plane + (long)ihc * g.W + iwc];
+                    const float val = load_elem(xs + c * plane + (long)ihc * g.W + iwc);
                     xv[c * 9 + r * 3 + t] = v ? val : 0.0f;
                 }
             }
         }
-        const float* dyp = dy + ((long)n * g.K + kg * KG) * PQ + p * g.Q + q;
+        const E* dyp = dy + ((long)n * g.K + kg * KG) * PQ + p * g.Q + q;
 #pragma unroll
         for (int j = 0; j < KG; j++) {
-            const float d = dyp[(long)j * PQ];
+            const float d = load_elem(dyp + (long)j * PQ);
 #pragma unroll
             for (int t = 0; t < TAPS; t++) acc[j][t] += d * xv[t];
         }

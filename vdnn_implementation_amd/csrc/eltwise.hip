@@ -4,6 +4,7 @@
 // (layer.cu:576-582, 631-637, 766-915) and the reference's two own kernels (layer.cu:33-38,
 // network.cu:3-8). All reductions have a fixed order: results do not depend on timing.
 #include "backend_internal.h"
+#include "mfma_gemm.h"
 
 #include <cfloat>
 
@@ -47,38 +48,60 @@ __device__ __forceinline__ float block_max(float v, float* sh) {
     return fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
 }
 
+// ---- four / two consecutive activation elements as floats ----------------------------------------------
+// float: one 128-bit (64-bit) access; bfloat16: one 64-bit (32-bit) access. p must be aligned to the access.
+__device__ __forceinline__ float4 ld4(const float* p) { return *(const float4*)p; }
+__device__ __forceinline__ float4 ld4(const bf16_t* p) {
+    const uint2 w = *(const uint2*)p;
+    return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xFFFF0000u), __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xFFFF0000u));
+}
+__device__ __forceinline__ void st4(float* p, float4 v) { *(float4*)p = v; }
+__device__ __forceinline__ void st4(bf16_t* p, float4 v) {
+    uint2 w;
+    w.x = (unsigned)float_to_bf16_bits(v.x) | ((unsigned)float_to_bf16_bits(v.y) << 16);
+    w.y = (unsigned)float_to_bf16_bits(v.z) | ((unsigned)float_to_bf16_bits(v.w) << 16);
+    *(uint2*)p = w;
+}
+__device__ __forceinline__ float2 ld2(const float* p) { return *(const float2*)p; }
+__device__ __forceinline__ float2 ld2(const bf16_t* p) {
+    const unsigned w = *(const unsigned*)p;
+    return make_float2(__uint_as_float(w << 16), __uint_as_float(w & 0xFFFF0000u));
+}
+__device__ __forceinline__ void st2(float* p, float2 v) { *(float2*)p = v; }
+__device__ __forceinline__ void st2(bf16_t* p, float2 v) {
+    *(unsigned*)p = (unsigned)float_to_bf16_bits(v.x) | ((unsigned)float_to_bf16_bits(v.y) << 16);
+}
+
 // ---- ReLU ---------------------------------------------------------------------------------------
 __device__ __forceinline__ float relu1(float v) { return v > 0.0f ? v : (v != v ? v : 0.0f); }
 
-__global__ void __launch_bounds__(EB) relu_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, size_t n4, size_t n) {
+template <class E>
+__global__ void __launch_bounds__(EB) relu_fwd_kernel(const E* __restrict__ x, E* __restrict__ y, size_t n4, size_t n) {
     const size_t stride = (size_t)gridDim.x * EB;
-    const float4* x4 = (const float4*)x;
-    float4* y4 = (float4*)y;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < n4; i += stride) {
-        float4 v = x4[i];
+        float4 v = ld4(x + 4 * i);
         v.x = relu1(v.x); v.y = relu1(v.y); v.z = relu1(v.z); v.w = relu1(v.w);
-        y4[i] = v;
+        st4(y + 4 * i, v);
     }
-    for (size_t i = n4 * 4 + (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) y[i] = relu1(x[i]);
+    for (size_t i = n4 * 4 + (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) store_elem(y + i, relu1(load_elem(x + i)));
 }
 
-__global__ void __launch_bounds__(EB) relu_bwd_kernel(const float* __restrict__ t, const float* __restrict__ dy,
-                                                      float* __restrict__ dx, size_t n4, size_t n) {
+template <class E>
+__global__ void __launch_bounds__(EB) relu_bwd_kernel(const E* __restrict__ t, const E* __restrict__ dy,
+                                                      E* __restrict__ dx, size_t n4, size_t n) {
     const size_t stride = (size_t)gridDim.x * EB;
-    const float4* t4 = (const float4*)t;
-    const float4* d4 = (const float4*)dy;
-    float4* o4 = (float4*)dx;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < n4; i += stride) {
-        const float4 a = t4[i], d = d4[i];
+        const float4 a = ld4(t + 4 * i), d = ld4(dy + 4 * i);
         float4 o;
         o.x = a.x > 0.0f ? d.x : 0.0f; o.y = a.y > 0.0f ? d.y : 0.0f;
         o.z = a.z > 0.0f ? d.z : 0.0f; o.w = a.w > 0.0f ? d.w : 0.0f;
-        o4[i] = o;
+        st4(dx + 4 * i, o);
     }
-    for (size_t i = n4 * 4 + (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) dx[i] = t[i] > 0.0f ? dy[i] : 0.0f;
+    for (size_t i = n4 * 4 + (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride)
+        store_elem(dx + i, load_elem(t + i) > 0.0f ? load_elem(dy + i) : 0.0f);
 }
 
-// ---- tanh / sigmoid: the other two activation modes of the layer (one float4 per thread) --------------
+// ---- tanh / sigmoid: the other two activation modes of the layer (four elements per thread) -----------
 // backward needs the output only: tanh' = 1 - y^2, sigmoid' = y (1 - y)
 template <int MODE> __device__ __forceinline__ float act1(float v) {
     return MODE == 0 ? tanhf(v) : 1.0f / (1.0f + expf(-v));
@@ -87,70 +110,83 @@ template <int MODE> __device__ __forceinline__ float dact1(float y, float d) {
     return MODE == 0 ? d * (1.0f - y * y) : d * (y * (1.0f - y));
 }
 
-template <int MODE>
-__global__ void __launch_bounds__(EB) act_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, size_t n4, size_t n) {
+template <int MODE, class E>
+__global__ void __launch_bounds__(EB) act_fwd_kernel(const E* __restrict__ x, E* __restrict__ y, size_t n4, size_t n) {
     const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
     if (i < n4) {
-        float4 v = ((const float4*)x)[i];
+        float4 v = ld4(x + 4 * i);
         v.x = act1<MODE>(v.x); v.y = act1<MODE>(v.y); v.z = act1<MODE>(v.z); v.w = act1<MODE>(v.w);
-        ((float4*)y)[i] = v;
+        st4(y + 4 * i, v);
     }
     const size_t t = n4 * 4 + i;
-    if (t < n) y[t] = act1<MODE>(x[t]);
+    if (t < n) store_elem(y + t, act1<MODE>(load_elem(x + t)));
 }
 
-template <int MODE>
-__global__ void __launch_bounds__(EB) act_bwd_kernel(const float* __restrict__ y, const float* __restrict__ dy, float* __restrict__ dx,
+template <int MODE, class E>
+__global__ void __launch_bounds__(EB) act_bwd_kernel(const E* __restrict__ y, const E* __restrict__ dy, E* __restrict__ dx,
                                                      size_t n4, size_t n) {
     const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
     if (i < n4) {
-        const float4 a = ((const float4*)y)[i], d = ((const float4*)dy)[i];
+        const float4 a = ld4(y + 4 * i), d = ld4(dy + 4 * i);
         float4 o;
         o.x = dact1<MODE>(a.x, d.x); o.y = dact1<MODE>(a.y, d.y); o.z = dact1<MODE>(a.z, d.z); o.w = dact1<MODE>(a.w, d.w);
-        ((float4*)dx)[i] = o;
+        st4(dx + 4 * i, o);
     }
     const size_t t = n4 * 4 + i;
-    if (t < n) dx[t] = dact1<MODE>(y[t], dy[t]);
+    if (t < n) store_elem(dx + t, dact1<MODE>(load_elem(y + t), load_elem(dy + t)));
 }
 
 // ---- elementwise helpers ------------------------------------------------------------------------
-__global__ void __launch_bounds__(EB) sub_kernel(const float* __restrict__ a, const float* __restrict__ b, float* __restrict__ r, size_t n) {
+template <class E>
+__global__ void __launch_bounds__(EB) sub_kernel(const E* __restrict__ a, const E* __restrict__ b, E* __restrict__ r, size_t n) {
     const size_t stride = (size_t)gridDim.x * EB;
-    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) r[i] = a[i] - b[i];
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) store_elem(r + i, load_elem(a + i) - load_elem(b + i));
 }
-__global__ void __launch_bounds__(EB) fill_kernel(float* __restrict__ p, float v, size_t n) {
+template <class E>
+__global__ void __launch_bounds__(EB) fill_kernel(E* __restrict__ p, float v, size_t n) {
     const size_t stride = (size_t)gridDim.x * EB;
-    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) p[i] = v;
+    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) store_elem(p + i, v);
 }
 // y[n,k,:] += bias[k]; one workgroup row per (n,k) plane chunk
-__global__ void __launch_bounds__(EB) bias_add_kernel(float* __restrict__ y, const float* __restrict__ bias, int K, int hw, size_t total) {
+template <class E>
+__global__ void __launch_bounds__(EB) bias_add_kernel(E* __restrict__ y, const float* __restrict__ bias, int K, int hw, size_t total) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
         const int k = (int)((i / hw) % K);
-        y[i] += bias[k];
+        store_elem(y + i, load_elem(y + i) + bias[k]);
     }
 }
 
 // out[i] = (accumulate ? out[i] : 0) + alpha * (p[0][i] + p[1][i] + ...) (+ bias[i % ncols]); split order fixed
-__global__ void __launch_bounds__(EB) reduce_splits_kernel(float* __restrict__ out, const float* __restrict__ partial, size_t count,
+template <class E>
+__global__ void __launch_bounds__(EB) reduce_splits_kernel(E* __restrict__ out, const float* __restrict__ partial, size_t count,
                                                            int splits, float alpha, int accumulate, const float* __restrict__ bias_j, int ncols) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < count; i += stride) {
         float s = partial[i];
         for (int k = 1; k < splits; k++) s += partial[(size_t)k * count + i];
-        float r = accumulate ? __fmaf_rn(alpha, s, out[i]) : alpha * s; // one fused multiply-add on every route
+        float r = accumulate ? __fmaf_rn(alpha, s, load_elem(out + i)) : alpha * s; // one fused multiply-add on every route
         if (bias_j) r += bias_j[i % ncols];
-        out[i] = r;
+        store_elem(out + i, r);
     }
 }
 
-int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
-                         int splits, float alpha, int accumulate, const float* bias_j, int ncols) {
+template <class E>
+static int launch_reduce_splits_t(vdnn_ctx* ctx, hipStream_t stream, E* out, const float* partial, size_t count,
+                                  int splits, float alpha, int accumulate, const float* bias_j, int ncols) {
     ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)count * (splits + 2));
-    hipLaunchKernelGGL(reduce_splits_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
+    hipLaunchKernelGGL(reduce_splits_kernel<E>, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
                        out, partial, count, splits, alpha, accumulate, bias_j, ncols);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
+}
+int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
+                         int splits, float alpha, int accumulate, const float* bias_j, int ncols) {
+    return launch_reduce_splits_t(ctx, stream, out, partial, count, splits, alpha, accumulate, bias_j, ncols);
+}
+int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, size_t count,
+                         int splits, float alpha, int accumulate, const float* bias_j, int ncols) {
+    return launch_reduce_splits_t(ctx, stream, out, partial, count, splits, alpha, accumulate, bias_j, ncols);
 }
 
 // param[i] = fma(alpha, grad[i], param[i]), the expression the fused updates evaluate
@@ -163,28 +199,29 @@ __global__ void __launch_bounds__(EB) sgd_apply_kernel(const float* __restrict__
 
 // ---- bias gradient of a convolution: bias[k] += alpha * sum_{n,pq} dy[n,k,pq] -------------------
 // stage 1: workgroup (k, split) sums samples [n0, n1) of channel k into partial[k*splits + split]
-__global__ void __launch_bounds__(EB) bias_grad_partial_kernel(const float* __restrict__ dy, float* __restrict__ partial,
+template <class E>
+__global__ void __launch_bounds__(EB) bias_grad_partial_kernel(const E* __restrict__ dy, float* __restrict__ partial,
                                                                int N, int K, int PQ, int splits, int n_per_split) {
     __shared__ float sh[4];
     const int k = blockIdx.x / splits, sp = blockIdx.x % splits;
     const int n0 = sp * n_per_split, n1 = min(N, n0 + n_per_split);
     float acc = 0.0f;
     if ((PQ & 3) == 0 && (((uintptr_t)dy & 15) == 0)) {
-        // 128-bit loads, four independent partial sums per thread (a fixed order, combined below)
+        // four elements per access, four independent partial sums per thread (a fixed order, combined below)
         float4 a4 = make_float4(0.f, 0.f, 0.f, 0.f);
         const int pq4 = PQ >> 2;
         for (int n = n0; n < n1; n++) {
-            const float4* p = (const float4*)(dy + ((size_t)n * K + k) * PQ);
+            const E* p = dy + ((size_t)n * K + k) * PQ;
             for (int i = threadIdx.x; i < pq4; i += EB) {
-                const float4 v = p[i];
+                const float4 v = ld4(p + 4 * i);
                 a4.x += v.x; a4.y += v.y; a4.z += v.z; a4.w += v.w;
             }
         }
         acc = (a4.x + a4.y) + (a4.z + a4.w);
     } else {
         for (int n = n0; n < n1; n++) {
-            const float* p = dy + ((size_t)n * K + k) * PQ;
-            for (int i = threadIdx.x; i < PQ; i += EB) acc += p[i];
+            const E* p = dy + ((size_t)n * K + k) * PQ;
+            for (int i = threadIdx.x; i < PQ; i += EB) acc += load_elem(p + i);
         }
     }
     acc = block_sum(acc, sh);
@@ -200,25 +237,27 @@ __global__ void __launch_bounds__(EB) bias_grad_final_kernel(const float* __rest
 }
 
 // bias[o] += alpha * sum_n dy[n,o]
-__global__ void __launch_bounds__(EB) fc_bias_grad_kernel(const float* __restrict__ dy, float* __restrict__ bias, int N, int Cout, float alpha, int accumulate) {
+template <class E>
+__global__ void __launch_bounds__(EB) fc_bias_grad_kernel(const E* __restrict__ dy, float* __restrict__ bias, int N, int Cout, float alpha, int accumulate) {
     const int o = blockIdx.x * EB + threadIdx.x;
     if (o >= Cout) return;
     float s = 0.0f;
-    for (int n = 0; n < N; n++) s += dy[(size_t)n * Cout + o];
+    for (int n = 0; n < N; n++) s += load_elem(dy + (size_t)n * Cout + o);
     bias[o] = accumulate ? __fmaf_rn(alpha, s, bias[o]) : alpha * s;
 }
 
 // ---- max pooling --------------------------------------------------------------------------------
 struct PoolGeo { int N, C, H, W, R, S, P, Q, ph, pw, sh, sw; };
 
-__global__ void __launch_bounds__(EB) maxpool_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, PoolGeo g, size_t total) {
+template <class E>
+__global__ void __launch_bounds__(EB) maxpool_fwd_kernel(const E* __restrict__ x, E* __restrict__ y, PoolGeo g, size_t total) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
         const int q = (int)(i % g.Q);
         const size_t t = i / g.Q;
         const int p = (int)(t % g.P);
         const size_t nc = t / g.P;
-        const float* xp = x + nc * g.H * g.W;
+        const E* xp = x + nc * g.H * g.W;
         float m = -FLT_MAX;
         for (int r = 0; r < g.R; r++) {
             const int ih = p * g.sh - g.ph + r;
@@ -226,16 +265,17 @@ __global__ void __launch_bounds__(EB) maxpool_fwd_kernel(const float* __restrict
             for (int s = 0; s < g.S; s++) {
                 const int iw = q * g.sw - g.pw + s;
                 if (iw < 0 || iw >= g.W) continue;
-                const float v = xp[(size_t)ih * g.W + iw];
+                const float v = load_elem(xp + (size_t)ih * g.W + iw);
                 if (v > m) m = v;
             }
         }
-        y[i] = m;
+        store_elem(y + i, m);
     }
 }
 
-// 2x2 stride 2, no padding, even extents, W % 4 == 0: one thread makes two outputs from two float4 rows
-__global__ void __launch_bounds__(EB) maxpool2x2_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, int H, int W, size_t total_pairs) {
+// 2x2 stride 2, no padding, even extents, W % 4 == 0: one thread makes two outputs from two four-element rows
+template <class E>
+__global__ void __launch_bounds__(EB) maxpool2x2_fwd_kernel(const E* __restrict__ x, E* __restrict__ y, int H, int W, size_t total_pairs) {
     const int Q2 = W / 4, P = H / 2;
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total_pairs; i += stride) {
@@ -243,19 +283,20 @@ __global__ void __launch_bounds__(EB) maxpool2x2_fwd_kernel(const float* __restr
         const size_t t = i / Q2;
         const int p = (int)(t % P);
         const size_t nc = t / P;
-        const float* r0 = x + (nc * H + 2 * (size_t)p) * W + 4 * (size_t)q2;
-        const float4 a = *(const float4*)r0, b = *(const float4*)(r0 + W);
+        const E* r0 = x + (nc * H + 2 * (size_t)p) * W + 4 * (size_t)q2;
+        const float4 a = ld4(r0), b = ld4(r0 + W);
         float m0 = -FLT_MAX, m1 = -FLT_MAX;
         if (a.x > m0) m0 = a.x; if (a.y > m0) m0 = a.y; if (b.x > m0) m0 = b.x; if (b.y > m0) m0 = b.y;
         if (a.z > m1) m1 = a.z; if (a.w > m1) m1 = a.w; if (b.z > m1) m1 = b.z; if (b.w > m1) m1 = b.w;
         float2 o; o.x = m0; o.y = m1;
-        *(float2*)(y + (nc * P + p) * (size_t)(W / 2) + 2 * (size_t)q2) = o;
+        st2(y + (nc * P + p) * (size_t)(W / 2) + 2 * (size_t)q2, o);
     }
 }
 
 // argmax of window (p,q) with the forward's comparison: first strict maximum in row-major order;
 // the first valid position if nothing exceeds -FLT_MAX
-__device__ __forceinline__ int window_argmax(const float* __restrict__ xp, const PoolGeo& g, int p, int q) {
+template <class E>
+__device__ __forceinline__ int window_argmax(const E* __restrict__ xp, const PoolGeo& g, int p, int q) {
     float m = -FLT_MAX;
     int arg = -1;
     for (int r = 0; r < g.R; r++) {
@@ -264,7 +305,7 @@ __device__ __forceinline__ int window_argmax(const float* __restrict__ xp, const
         for (int s = 0; s < g.S; s++) {
             const int iw = q * g.sw - g.pw + s;
             if (iw < 0 || iw >= g.W) continue;
-            const float v = xp[(size_t)ih * g.W + iw];
+            const float v = load_elem(xp + (size_t)ih * g.W + iw);
             if (arg < 0) arg = ih * g.W + iw;
             if (v > m) { m = v; arg = ih * g.W + iw; }
         }
@@ -273,7 +314,8 @@ __device__ __forceinline__ int window_argmax(const float* __restrict__ xp, const
 }
 
 // gather form: one thread per input element, windows visited in row-major order
-__global__ void __launch_bounds__(EB) maxpool_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ dx,
+template <class E>
+__global__ void __launch_bounds__(EB) maxpool_bwd_kernel(const E* __restrict__ x, const E* __restrict__ dy, E* __restrict__ dx,
                                                          PoolGeo g, size_t total) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
@@ -281,8 +323,8 @@ __global__ void __launch_bounds__(EB) maxpool_bwd_kernel(const float* __restrict
         const size_t t = i / g.W;
         const int h = (int)(t % g.H);
         const size_t nc = t / g.H;
-        const float* xp = x + nc * g.H * g.W;
-        const float* dyp = dy + nc * g.P * g.Q;
+        const E* xp = x + nc * g.H * g.W;
+        const E* dyp = dy + nc * g.P * g.Q;
         // windows containing (h,w): p*sh - ph <= h <= p*sh - ph + R - 1
         int p_lo = h + g.ph - g.R + 1; p_lo = p_lo <= 0 ? 0 : (p_lo + g.sh - 1) / g.sh;
         int p_hi = (h + g.ph) / g.sh; if (p_hi > g.P - 1) p_hi = g.P - 1;
@@ -292,13 +334,14 @@ __global__ void __launch_bounds__(EB) maxpool_bwd_kernel(const float* __restrict
         float acc = 0.0f;
         for (int p = p_lo; p <= p_hi; p++)
             for (int q = q_lo; q <= q_hi; q++)
-                if (window_argmax(xp, g, p, q) == self) acc += dyp[(size_t)p * g.Q + q];
-        dx[i] = acc;
+                if (window_argmax(xp, g, p, q) == self) acc += load_elem(dyp + (size_t)p * g.Q + q);
+        store_elem(dx + i, acc);
     }
 }
 
 // 2x2 stride 2 exact cover: one thread per pair of windows, writes all eight inputs
-__global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ dx,
+template <class E>
+__global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const E* __restrict__ x, const E* __restrict__ dy, E* __restrict__ dx,
                                                             int H, int W, size_t total_pairs) {
     const int Q2 = W / 4, P = H / 2;
     const size_t stride = (size_t)gridDim.x * EB;
@@ -308,8 +351,8 @@ __global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const float* __restr
         const int p = (int)(t % P);
         const size_t nc = t / P;
         const size_t off = (nc * H + 2 * (size_t)p) * W + 4 * (size_t)q2;
-        const float4 a = *(const float4*)(x + off), b = *(const float4*)(x + off + W);
-        const float2 d = *(const float2*)(dy + (nc * P + p) * (size_t)(W / 2) + 2 * (size_t)q2);
+        const float4 a = ld4(x + off), b = ld4(x + off + W);
+        const float2 d = ld2(dy + (nc * P + p) * (size_t)(W / 2) + 2 * (size_t)q2);
         // window 0: a.x a.y / b.x b.y ; window 1: a.z a.w / b.z b.w ; first strict maximum wins
         int s0 = 0; float m0 = -FLT_MAX;
         if (a.x > m0) { m0 = a.x; s0 = 0; } if (a.y > m0) { m0 = a.y; s0 = 1; }
@@ -320,8 +363,8 @@ __global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const float* __restr
         float4 oa, ob;
         oa.x = s0 == 0 ? d.x : 0.0f; oa.y = s0 == 1 ? d.x : 0.0f; ob.x = s0 == 2 ? d.x : 0.0f; ob.y = s0 == 3 ? d.x : 0.0f;
         oa.z = s1 == 0 ? d.y : 0.0f; oa.w = s1 == 1 ? d.y : 0.0f; ob.z = s1 == 2 ? d.y : 0.0f; ob.w = s1 == 3 ? d.y : 0.0f;
-        *(float4*)(dx + off) = oa;
-        *(float4*)(dx + off + W) = ob;
+        st4(dx + off, oa);
+        st4(dx + off + W, ob);
     }
 }
 
@@ -330,7 +373,8 @@ __global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const float* __restr
 #define LRN_BETA 0.75f
 #define LRN_KC 2.0f
 
-__global__ void __launch_bounds__(EB) lrn_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int hw, size_t total) {
+template <class E>
+__global__ void __launch_bounds__(EB) lrn_fwd_kernel(const E* __restrict__ x, E* __restrict__ y, int C, int hw, size_t total) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
         const int c = (int)((i / hw) % C);
@@ -339,16 +383,17 @@ __global__ void __launch_bounds__(EB) lrn_fwd_kernel(const float* __restrict__ x
         for (int d = -2; d <= 2; d++) {
             const int cc = c + d;
             if (cc < 0 || cc >= C) continue;
-            const float v = x[(long)i + (long)d * hw];
+            const float v = load_elem(x + ((long)i + (long)d * hw));
             ss += v * v;
         }
         const float scale = LRN_KC + LRN_A5 * ss;
-        y[i] = x[i] * powf(scale, -LRN_BETA);
+        store_elem(y + i, load_elem(x + i) * powf(scale, -LRN_BETA));
     }
 }
 
-__global__ void __launch_bounds__(EB) lrn_bwd_kernel(const float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ dy,
-                                                     float* __restrict__ dx, int C, int hw, size_t total) {
+template <class E>
+__global__ void __launch_bounds__(EB) lrn_bwd_kernel(const E* __restrict__ x, const E* __restrict__ y, const E* __restrict__ dy,
+                                                     E* __restrict__ dx, int C, int hw, size_t total) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
         const int c = (int)((i / hw) % C);
@@ -357,7 +402,7 @@ __global__ void __launch_bounds__(EB) lrn_bwd_kernel(const float* __restrict__ x
         for (int d = -4; d <= 4; d++) {
             const int cc = c + d;
             float v = 0.0f;
-            if (cc >= 0 && cc < C) v = x[(long)i + (long)d * hw];
+            if (cc >= 0 && cc < C) v = load_elem(x + ((long)i + (long)d * hw));
             xs[d + 4] = v * v;
         }
         float t = 0.0f, scale_c = 1.0f;
@@ -372,56 +417,57 @@ __global__ void __launch_bounds__(EB) lrn_bwd_kernel(const float* __restrict__ x
             if (d == 0) scale_c = scale;
             if (cc < 0 || cc >= C) continue;
             const long o = (long)i + (long)d * hw;
-            t += dy[o] * y[o] / scale;
+            t += load_elem(dy + o) * load_elem(y + o) / scale;
         }
-        dx[i] = dy[i] * powf(scale_c, -LRN_BETA) - (2.0f * 1e-4f * LRN_BETA / 5.0f) * x[i] * t;
+        store_elem(dx + i, load_elem(dy + i) * powf(scale_c, -LRN_BETA) - (2.0f * 1e-4f * LRN_BETA / 5.0f) * load_elem(x + i) * t);
     }
 }
 
 // ---- softmax (one workgroup per sample) -------------------------------------------------------------
-__global__ void __launch_bounds__(EB) softmax_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, int classes) {
+template <class E>
+__global__ void __launch_bounds__(EB) softmax_fwd_kernel(const E* __restrict__ x, E* __restrict__ y, int classes) {
     __shared__ float sh[4];
-    const float* xr = x + (size_t)blockIdx.x * classes;
-    float* yr = y + (size_t)blockIdx.x * classes;
+    const E* xr = x + (size_t)blockIdx.x * classes;
+    E* yr = y + (size_t)blockIdx.x * classes;
     float m = -FLT_MAX;
-    for (int j = threadIdx.x; j < classes; j += EB) m = fmaxf(m, xr[j]);
+    for (int j = threadIdx.x; j < classes; j += EB) m = fmaxf(m, load_elem(xr + j));
     m = block_max(m, sh);
     float s = 0.0f;
-    for (int j = threadIdx.x; j < classes; j += EB) {
-        const float e = expf(xr[j] - m);
-        yr[j] = e;
-        s += e;
-    }
+    for (int j = threadIdx.x; j < classes; j += EB) s += expf(load_elem(xr + j) - m);
     s = block_sum(s, sh);
     const float inv = 1.0f / s;
-    for (int j = threadIdx.x; j < classes; j += EB) yr[j] *= inv;
+    // the exponentials are evaluated again rather than parked in y: a bfloat16 y is rounded once
+    for (int j = threadIdx.x; j < classes; j += EB) store_elem(yr + j, expf(load_elem(xr + j) - m) * inv);
 }
 
-__global__ void __launch_bounds__(EB) softmax_bwd_kernel(const float* __restrict__ y, const float* __restrict__ dy, float* __restrict__ dx, int classes) {
+template <class E>
+__global__ void __launch_bounds__(EB) softmax_bwd_kernel(const E* __restrict__ y, const E* __restrict__ dy, E* __restrict__ dx, int classes) {
     __shared__ float sh[4];
     const size_t base = (size_t)blockIdx.x * classes;
     float dot = 0.0f;
-    for (int j = threadIdx.x; j < classes; j += EB) dot += dy[base + j] * y[base + j];
+    for (int j = threadIdx.x; j < classes; j += EB) dot += load_elem(dy + base + j) * load_elem(y + base + j);
     dot = block_sum(dot, sh);
-    for (int j = threadIdx.x; j < classes; j += EB) dx[base + j] = y[base + j] * (dy[base + j] - dot);
+    for (int j = threadIdx.x; j < classes; j += EB) store_elem(dx + base + j, load_elem(y + base + j) * (load_elem(dy + base + j) - dot));
 }
 
 // per-sample -log p[label] into sample_loss[n]
-__global__ void __launch_bounds__(EB) nll_label_kernel(const float* __restrict__ prob, const int32_t* __restrict__ labels, float* __restrict__ sample_loss, int n, int classes) {
+template <class E>
+__global__ void __launch_bounds__(EB) nll_label_kernel(const E* __restrict__ prob, const int32_t* __restrict__ labels, float* __restrict__ sample_loss, int n, int classes) {
     const int i = blockIdx.x * EB + threadIdx.x;
     if (i >= n) return;
     const int lab = labels[i];
-    float p = (lab >= 0 && lab < classes) ? prob[(size_t)i * classes + lab] : 1.0f;
+    float p = (lab >= 0 && lab < classes) ? load_elem(prob + (size_t)i * classes + lab) : 1.0f;
     sample_loss[i] = -logf(fmaxf(p, FLT_MIN));
 }
 // per-sample -sum_c target*log p
-__global__ void __launch_bounds__(EB) ce_dense_kernel(const float* __restrict__ prob, const float* __restrict__ target, float* __restrict__ sample_loss, int classes) {
+template <class E>
+__global__ void __launch_bounds__(EB) ce_dense_kernel(const E* __restrict__ prob, const E* __restrict__ target, float* __restrict__ sample_loss, int classes) {
     __shared__ float sh[4];
     const size_t base = (size_t)blockIdx.x * classes;
     float s = 0.0f;
     for (int j = threadIdx.x; j < classes; j += EB) {
-        const float t = target[base + j];
-        if (t != 0.0f) s -= t * logf(fmaxf(prob[base + j], FLT_MIN));
+        const float t = load_elem(target + base + j);
+        if (t != 0.0f) s -= t * logf(fmaxf(load_elem(prob + base + j), FLT_MIN));
     }
     s = block_sum(s, sh);
     if (threadIdx.x == 0) sample_loss[blockIdx.x] = s;
@@ -434,11 +480,12 @@ __global__ void __launch_bounds__(EB) mean_kernel(const float* __restrict__ v, f
     s = block_sum(s, sh);
     if (threadIdx.x == 0) out[0] = s / (float)n;
 }
-__global__ void __launch_bounds__(EB) softmax_ce_bwd_kernel(const float* __restrict__ prob, const int32_t* __restrict__ labels, float* __restrict__ d, int classes, float inv_n, size_t total) {
+template <class E>
+__global__ void __launch_bounds__(EB) softmax_ce_bwd_kernel(const E* __restrict__ prob, const int32_t* __restrict__ labels, E* __restrict__ d, int classes, float inv_n, size_t total) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
         const int n = (int)(i / classes), j = (int)(i % classes);
-        d[i] = (prob[i] - (labels[n] == j ? 1.0f : 0.0f)) * inv_n;
+        store_elem(d + i, (load_elem(prob + i) - (labels[n] == j ? 1.0f : 0.0f)) * inv_n);
     }
 }
 
@@ -448,90 +495,93 @@ static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 using namespace vdnn;
 
-template <int MODE>
-static int act_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const char* name, size_t count, const float* x, float* y) {
+// ---- launchers, one instance per activation element type ----------------------------------------------
+template <class E>
+static int relu_fwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* xv, void* yv) {
     VDNN_KERNEL_PROLOGUE(ctx);
+    const E* x = (const E*)xv; E* y = (E*)yv;
     VDNN_REQUIRE(x && y, "null tensor");
     if (count == 0) return VDNN_OK;
     const size_t n4 = (aligned16(x) && aligned16(y)) ? count / 4 : 0;
-    const size_t threads = n4 > count - n4 * 4 ? n4 : count - n4 * 4;
-    ProfScope prof(ctx, stream_of(ctx, stream), name, 0.0, 8.0 * (double)count);
-    hipLaunchKernelGGL(act_fwd_kernel<MODE>, dim3(grid_for(threads, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), x, y, n4, count);
+    ProfScope prof(ctx, stream_of(ctx, stream), "relu_fwd", 0.0, 2.0 * sizeof(E) * (double)count);
+    hipLaunchKernelGGL(relu_fwd_kernel<E>, dim3(grid_for(n4 ? n4 : count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), x, y, n4, count);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-template <int MODE>
-static int act_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const char* name, size_t count, const float* y, const float* dy, float* dx) {
+template <class E>
+static int relu_bwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* xv, const void* yv, const void* dyv, void* dxv) {
     VDNN_KERNEL_PROLOGUE(ctx);
+    const E* t = (const E*)(xv ? xv : yv); const E* dy = (const E*)dyv; E* dx = (E*)dxv;
+    VDNN_REQUIRE(t && dy && dx, "null tensor");
+    if (count == 0) return VDNN_OK;
+    const size_t n4 = (aligned16(t) && aligned16(dy) && aligned16(dx)) ? count / 4 : 0;
+    ProfScope prof(ctx, stream_of(ctx, stream), "relu_bwd", 0.0, 3.0 * sizeof(E) * (double)count);
+    hipLaunchKernelGGL(relu_bwd_kernel<E>, dim3(grid_for(n4 ? n4 : count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), t, dy, dx, n4, count);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+template <int MODE, class E>
+static int act_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const char* name, size_t count, const void* xv, void* yv) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    const E* x = (const E*)xv; E* y = (E*)yv;
+    VDNN_REQUIRE(x && y, "null tensor");
+    if (count == 0) return VDNN_OK;
+    const size_t n4 = (aligned16(x) && aligned16(y)) ? count / 4 : 0;
+    const size_t threads = n4 > count - n4 * 4 ? n4 : count - n4 * 4;
+    ProfScope prof(ctx, stream_of(ctx, stream), name, 0.0, 2.0 * sizeof(E) * (double)count);
+    hipLaunchKernelGGL((act_fwd_kernel<MODE, E>), dim3(grid_for(threads, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), x, y, n4, count);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+template <int MODE, class E>
+static int act_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const char* name, size_t count, const void* yv, const void* dyv, void* dxv) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    const E* y = (const E*)yv; const E* dy = (const E*)dyv; E* dx = (E*)dxv;
     VDNN_REQUIRE(y && dy && dx, "null tensor");
     if (count == 0) return VDNN_OK;
     const size_t n4 = (aligned16(y) && aligned16(dy) && aligned16(dx)) ? count / 4 : 0;
     const size_t threads = n4 > count - n4 * 4 ? n4 : count - n4 * 4;
-    ProfScope prof(ctx, stream_of(ctx, stream), name, 0.0, 12.0 * (double)count);
-    hipLaunchKernelGGL(act_bwd_kernel<MODE>, dim3(grid_for(threads, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), y, dy, dx, n4, count);
+    ProfScope prof(ctx, stream_of(ctx, stream), name, 0.0, 3.0 * sizeof(E) * (double)count);
+    hipLaunchKernelGGL((act_bwd_kernel<MODE, E>), dim3(grid_for(threads, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), y, dy, dx, n4, count);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-extern "C" {
-
-int vdnn_relu_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y) {
-    VDNN_KERNEL_PROLOGUE(ctx);
-    VDNN_REQUIRE(x && y, "null tensor");
-    if (count == 0) return VDNN_OK;
-    const size_t n4 = (aligned16(x) && aligned16(y)) ? count / 4 : 0;
-    ProfScope prof(ctx, stream_of(ctx, stream), "relu_fwd", 0.0, 8.0 * (double)count);
-    hipLaunchKernelGGL(relu_fwd_kernel, dim3(grid_for(n4 ? n4 : count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), x, y, n4, count);
-    VDNN_LAUNCH_CHECK();
-    return VDNN_OK;
-}
-
-int vdnn_relu_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, const float* y, const float* dy, float* dx) {
-    VDNN_KERNEL_PROLOGUE(ctx);
-    const float* t = x ? x : y;
-    VDNN_REQUIRE(t && dy && dx, "null tensor");
-    if (count == 0) return VDNN_OK;
-    const size_t n4 = (aligned16(t) && aligned16(dy) && aligned16(dx)) ? count / 4 : 0;
-    ProfScope prof(ctx, stream_of(ctx, stream), "relu_bwd", 0.0, 12.0 * (double)count);
-    hipLaunchKernelGGL(relu_bwd_kernel, dim3(grid_for(n4 ? n4 : count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), t, dy, dx, n4, count);
-    VDNN_LAUNCH_CHECK();
-    return VDNN_OK;
-}
-
-int vdnn_tanh_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y) { return act_fwd<0>(ctx, stream, "tanh_fwd", count, x, y); }
-int vdnn_tanh_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* y, const float* dy, float* dx) { return act_bwd<0>(ctx, stream, "tanh_bwd", count, y, dy, dx); }
-int vdnn_sigmoid_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* x, float* y) { return act_fwd<1>(ctx, stream, "sigmoid_fwd", count, x, y); }
-int vdnn_sigmoid_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* y, const float* dy, float* dx) { return act_bwd<1>(ctx, stream, "sigmoid_bwd", count, y, dy, dx); }
-
-int vdnn_sub(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const float* a, const float* b, float* r) {
+template <class E>
+static int sub_t(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* a, const void* b, void* r) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(a && b && r, "null tensor");
     if (count == 0) return VDNN_OK;
-    hipLaunchKernelGGL(sub_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), a, b, r, count);
+    hipLaunchKernelGGL(sub_kernel<E>, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), (const E*)a, (const E*)b, (E*)r, count);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-int vdnn_fill(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float value, float* p) {
+template <class E>
+static int fill_t(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float value, void* p) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(p, "null tensor");
     if (count == 0) return VDNN_OK;
-    hipLaunchKernelGGL(fill_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), p, value, count);
+    hipLaunchKernelGGL(fill_kernel<E>, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), (E*)p, value, count);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-int vdnn_bias_add(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw, const float* bias, float* y) {
+template <class E>
+static int bias_add_t(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw, const float* bias, void* y) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(bias && y && n > 0 && k > 0 && hw > 0, "bad argument");
     const size_t total = (size_t)n * k * hw;
-    hipLaunchKernelGGL(bias_add_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), y, bias, k, hw, total);
+    hipLaunchKernelGGL(bias_add_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), (E*)y, bias, k, hw, total);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-static int conv_bwd_bias_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* dy, float* bias, float alpha, int accumulate) {
+template <class E>
+static int conv_bwd_bias_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* dy, float* bias, float alpha, int accumulate) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(shape && dy && bias, "null argument");
     const int N = shape->n, K = shape->k;
@@ -546,46 +596,19 @@ static int conv_bwd_bias_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
     splits = (N + per - 1) / per;
     VDNN_REQUIRE((size_t)K * splits * sizeof(float) <= ctx->reduce_scratch_bytes, "staging area too small");
     hipStream_t st = stream_of(ctx, stream);
-    ProfScope prof(ctx, st, "conv_bwd_bias", 0.0, 4.0 * (double)N * K * P * Q);
-    hipLaunchKernelGGL(bias_grad_partial_kernel, dim3(K * splits), dim3(EB), 0, st, dy, ctx->reduce_scratch, N, K, P * Q, splits, per);
+    ProfScope prof(ctx, st, "conv_bwd_bias", 0.0, (double)sizeof(E) * (double)N * K * P * Q);
+    hipLaunchKernelGGL(bias_grad_partial_kernel<E>, dim3(K * splits), dim3(EB), 0, st, (const E*)dy, ctx->reduce_scratch, N, K, P * Q, splits, per);
     VDNN_LAUNCH_CHECK();
     hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB - 1) / EB), dim3(EB), 0, st, ctx->reduce_scratch, bias, K, splits, alpha, accumulate);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* dy, float* bias, float alpha) {
-    return conv_bwd_bias_impl(ctx, stream, shape, dy, bias, alpha, 1);
-}
-
-int vdnn_conv_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* dy, float* db) {
-    return conv_bwd_bias_impl(ctx, stream, shape, dy, db, 1.0f, 0);
-}
-
-static int fc_bwd_bias_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const float* dy, float* bias, float alpha, int accumulate) {
+template <class E>
+static int fc_bwd_bias_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const void* dy, float* bias, float alpha, int accumulate) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(dy && bias && n > 0 && c_out > 0, "bad argument");
-    hipLaunchKernelGGL(fc_bias_grad_kernel, dim3((c_out + EB - 1) / EB), dim3(EB), 0, stream_of(ctx, stream), dy, bias, n, c_out, alpha, accumulate);
-    VDNN_LAUNCH_CHECK();
-    return VDNN_OK;
-}
-
-int vdnn_fc_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const float* dy, float* bias, float alpha) {
-    return fc_bwd_bias_impl(ctx, stream, n, c_out, dy, bias, alpha, 1);
-}
-
-int vdnn_fc_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const float* dy, float* db) {
-    return fc_bwd_bias_impl(ctx, stream, n, c_out, dy, db, 1.0f, 0);
-}
-
-// param[i] += alpha * grad[i]: the optimizer step when gradients are kept instead of fused into backward
-int vdnn_sgd_apply(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float alpha, const float* grad, float* param) {
-    VDNN_KERNEL_PROLOGUE(ctx);
-    VDNN_REQUIRE(grad && param, "null tensor");
-    if (count == 0) return VDNN_OK;
-    hipStream_t st = stream_of(ctx, stream);
-    ProfScope prof(ctx, st, "sgd_apply", 0.0, 12.0 * (double)count);
-    hipLaunchKernelGGL(sgd_apply_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, st, grad, param, alpha, count);
+    hipLaunchKernelGGL(fc_bias_grad_kernel<E>, dim3((c_out + EB - 1) / EB), dim3(EB), 0, stream_of(ctx, stream), (const E*)dy, bias, n, c_out, alpha, accumulate);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
@@ -604,90 +627,100 @@ static bool pool_is_2x2_exact(const PoolGeo& g, const void* a, const void* b, co
            aligned16(a) && aligned16(b) && (!c || aligned16(c));
 }
 
-int vdnn_maxpool_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const float* x, float* y) {
+template <class E>
+static int maxpool_fwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* xv, void* yv) {
     VDNN_KERNEL_PROLOGUE(ctx);
+    const E* x = (const E*)xv; E* y = (E*)yv;
     PoolGeo g;
     VDNN_REQUIRE(shape && pool_geo(shape, g), "unsupported pooling geometry");
     VDNN_REQUIRE(x && y, "null tensor");
     hipStream_t st = stream_of(ctx, stream);
-    ProfScope prof(ctx, st, "maxpool_fwd", 0.0, 4.0 * ((double)g.N * g.C * g.H * g.W + (double)g.N * g.C * g.P * g.Q));
+    ProfScope prof(ctx, st, "maxpool_fwd", 0.0, (double)sizeof(E) * ((double)g.N * g.C * g.H * g.W + (double)g.N * g.C * g.P * g.Q));
     if (pool_is_2x2_exact(g, x, y, nullptr)) {
         const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
-        hipLaunchKernelGGL(maxpool2x2_fwd_kernel, dim3(grid_for(pairs, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, y, g.H, g.W, pairs);
+        hipLaunchKernelGGL(maxpool2x2_fwd_kernel<E>, dim3(grid_for(pairs, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, y, g.H, g.W, pairs);
     } else {
         const size_t total = (size_t)g.N * g.C * g.P * g.Q;
-        hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, y, g, total);
+        hipLaunchKernelGGL(maxpool_fwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, y, g, total);
     }
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-int vdnn_maxpool_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape,
-                     const float* x, const float* y, const float* dy, float* dx) {
+template <class E>
+static int maxpool_bwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape,
+                         const void* xv, const void* yv, const void* dyv, void* dxv) {
     VDNN_KERNEL_PROLOGUE(ctx);
-    (void)y; // the winner of each window is recomputed from x with the forward's comparison
+    (void)yv; // the winner of each window is recomputed from x with the forward's comparison
+    const E* x = (const E*)xv; const E* dy = (const E*)dyv; E* dx = (E*)dxv;
     PoolGeo g;
     VDNN_REQUIRE(shape && pool_geo(shape, g), "unsupported pooling geometry");
     VDNN_REQUIRE(x && dy && dx, "null tensor");
     hipStream_t st = stream_of(ctx, stream);
-    ProfScope prof(ctx, st, "maxpool_bwd", 0.0, 4.0 * (2.0 * g.N * g.C * g.H * g.W + (double)g.N * g.C * g.P * g.Q));
+    ProfScope prof(ctx, st, "maxpool_bwd", 0.0, (double)sizeof(E) * (2.0 * g.N * g.C * g.H * g.W + (double)g.N * g.C * g.P * g.Q));
     if (pool_is_2x2_exact(g, x, dx, dy) && (g.W / 2) % 2 == 0) {
         const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
-        hipLaunchKernelGGL(maxpool2x2_bwd_kernel, dim3(grid_for(pairs, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g.H, g.W, pairs);
+        hipLaunchKernelGGL(maxpool2x2_bwd_kernel<E>, dim3(grid_for(pairs, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g.H, g.W, pairs);
     } else {
         const size_t total = (size_t)g.N * g.C * g.H * g.W;
-        hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g, total);
+        hipLaunchKernelGGL(maxpool_bwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g, total);
     }
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-int vdnn_lrn_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const float* x, float* y) {
+template <class E>
+static int lrn_fwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const void* x, void* y) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && y && n > 0 && c > 0 && hw > 0, "bad argument");
     const size_t total = (size_t)n * c * hw;
-    ProfScope prof(ctx, stream_of(ctx, stream), "lrn_fwd", 0.0, 8.0 * (double)total);
-    hipLaunchKernelGGL(lrn_fwd_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), x, y, c, hw, total);
+    ProfScope prof(ctx, stream_of(ctx, stream), "lrn_fwd", 0.0, 2.0 * sizeof(E) * (double)total);
+    hipLaunchKernelGGL(lrn_fwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), (const E*)x, (E*)y, c, hw, total);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-int vdnn_lrn_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const float* x, const float* y, const float* dy, float* dx) {
+template <class E>
+static int lrn_bwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const void* x, const void* y, const void* dy, void* dx) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && y && dy && dx && n > 0 && c > 0 && hw > 0, "bad argument");
     const size_t total = (size_t)n * c * hw;
-    ProfScope prof(ctx, stream_of(ctx, stream), "lrn_bwd", 0.0, 16.0 * (double)total);
-    hipLaunchKernelGGL(lrn_bwd_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), x, y, dy, dx, c, hw, total);
+    ProfScope prof(ctx, stream_of(ctx, stream), "lrn_bwd", 0.0, 4.0 * sizeof(E) * (double)total);
+    hipLaunchKernelGGL(lrn_bwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream),
+                       (const E*)x, (const E*)y, (const E*)dy, (E*)dx, c, hw, total);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-int vdnn_softmax_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* x, float* y) {
+template <class E>
+static int softmax_fwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* x, void* y) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && y && n > 0 && classes > 0, "bad argument");
-    hipLaunchKernelGGL(softmax_fwd_kernel, dim3(n), dim3(EB), 0, stream_of(ctx, stream), x, y, classes);
+    hipLaunchKernelGGL(softmax_fwd_kernel<E>, dim3(n), dim3(EB), 0, stream_of(ctx, stream), (const E*)x, (E*)y, classes);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-int vdnn_softmax_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* y, const float* dy, float* dx) {
+template <class E>
+static int softmax_bwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* y, const void* dy, void* dx) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(y && dy && dx && n > 0 && classes > 0, "bad argument");
-    hipLaunchKernelGGL(softmax_bwd_kernel, dim3(n), dim3(EB), 0, stream_of(ctx, stream), y, dy, dx, classes);
+    hipLaunchKernelGGL(softmax_bwd_kernel<E>, dim3(n), dim3(EB), 0, stream_of(ctx, stream), (const E*)y, (const E*)dy, (E*)dx, classes);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-int vdnn_softmax_ce_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* logits,
-                        const int32_t* labels, float* prob, float* loss) {
+template <class E>
+static int softmax_ce_fwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* logits,
+                            const int32_t* labels, void* prob, float* loss) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(logits && labels && prob && n > 0 && classes > 0, "bad argument");
     hipStream_t st = stream_of(ctx, stream);
-    hipLaunchKernelGGL(softmax_fwd_kernel, dim3(n), dim3(EB), 0, st, logits, prob, classes);
+    hipLaunchKernelGGL(softmax_fwd_kernel<E>, dim3(n), dim3(EB), 0, st, (const E*)logits, (E*)prob, classes);
     VDNN_LAUNCH_CHECK();
     if (loss) {
         VDNN_REQUIRE((size_t)n * sizeof(float) <= ctx->reduce_scratch_bytes, "staging area too small");
-        hipLaunchKernelGGL(nll_label_kernel, dim3((n + EB - 1) / EB), dim3(EB), 0, st, prob, labels, ctx->reduce_scratch, n, classes);
+        hipLaunchKernelGGL(nll_label_kernel<E>, dim3((n + EB - 1) / EB), dim3(EB), 0, st, (const E*)prob, labels, ctx->reduce_scratch, n, classes);
         VDNN_LAUNCH_CHECK();
         hipLaunchKernelGGL(mean_kernel, dim3(1), dim3(EB), 0, st, ctx->reduce_scratch, loss, n);
         VDNN_LAUNCH_CHECK();
@@ -695,28 +728,104 @@ int vdnn_softmax_ce_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes,
     return VDNN_OK;
 }
 
-int vdnn_softmax_ce_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const float* prob,
-                        const int32_t* labels, float* dlogits) {
+template <class E>
+static int softmax_ce_bwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* prob,
+                            const int32_t* labels, void* dlogits) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(prob && labels && dlogits && n > 0 && classes > 0, "bad argument");
     const size_t total = (size_t)n * classes;
-    hipLaunchKernelGGL(softmax_ce_bwd_kernel, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream),
-                       prob, labels, dlogits, classes, 1.0f / (float)n, total);
+    hipLaunchKernelGGL(softmax_ce_bwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream),
+                       (const E*)prob, labels, (E*)dlogits, classes, 1.0f / (float)n, total);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 
-int vdnn_cross_entropy_dense(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes,
-                             const float* prob, const float* target, float* loss) {
+template <class E>
+static int cross_entropy_dense_t(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes,
+                                 const void* prob, const void* target, float* loss) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(prob && target && loss && n > 0 && classes > 0, "bad argument");
     VDNN_REQUIRE((size_t)n * sizeof(float) <= ctx->reduce_scratch_bytes, "staging area too small");
     hipStream_t st = stream_of(ctx, stream);
-    hipLaunchKernelGGL(ce_dense_kernel, dim3(n), dim3(EB), 0, st, prob, target, ctx->reduce_scratch, classes);
+    hipLaunchKernelGGL(ce_dense_kernel<E>, dim3(n), dim3(EB), 0, st, (const E*)prob, (const E*)target, ctx->reduce_scratch, classes);
     VDNN_LAUNCH_CHECK();
     hipLaunchKernelGGL(mean_kernel, dim3(1), dim3(EB), 0, st, ctx->reduce_scratch, loss, n);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
+}
+
+// the same call for either activation element type
+#define ACT_CALL(fn, ...) VDNN_BY_ACT(ctx, fn<float>(__VA_ARGS__), fn<bf16_t>(__VA_ARGS__))
+
+extern "C" {
+
+int vdnn_relu_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* x, void* y) { return ACT_CALL(relu_fwd_t, ctx, stream, count, x, y); }
+int vdnn_relu_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* x, const void* y, const void* dy, void* dx) {
+    return ACT_CALL(relu_bwd_t, ctx, stream, count, x, y, dy, dx);
+}
+
+int vdnn_tanh_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* x, void* y) {
+    return VDNN_BY_ACT(ctx, (act_fwd<0, float>(ctx, stream, "tanh_fwd", count, x, y)), (act_fwd<0, bf16_t>(ctx, stream, "tanh_fwd", count, x, y)));
+}
+int vdnn_tanh_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* y, const void* dy, void* dx) {
+    return VDNN_BY_ACT(ctx, (act_bwd<0, float>(ctx, stream, "tanh_bwd", count, y, dy, dx)), (act_bwd<0, bf16_t>(ctx, stream, "tanh_bwd", count, y, dy, dx)));
+}
+int vdnn_sigmoid_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* x, void* y) {
+    return VDNN_BY_ACT(ctx, (act_fwd<1, float>(ctx, stream, "sigmoid_fwd", count, x, y)), (act_fwd<1, bf16_t>(ctx, stream, "sigmoid_fwd", count, x, y)));
+}
+int vdnn_sigmoid_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* y, const void* dy, void* dx) {
+    return VDNN_BY_ACT(ctx, (act_bwd<1, float>(ctx, stream, "sigmoid_bwd", count, y, dy, dx)), (act_bwd<1, bf16_t>(ctx, stream, "sigmoid_bwd", count, y, dy, dx)));
+}
+
+int vdnn_sub(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, const void* a, const void* b, void* r) { return ACT_CALL(sub_t, ctx, stream, count, a, b, r); }
+int vdnn_fill(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float value, void* p) { return ACT_CALL(fill_t, ctx, stream, count, value, p); }
+int vdnn_bias_add(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw, const float* bias, void* y) { return ACT_CALL(bias_add_t, ctx, stream, n, k, hw, bias, y); }
+
+int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* dy, float* bias, float alpha) {
+    return ACT_CALL(conv_bwd_bias_impl, ctx, stream, shape, dy, bias, alpha, 1);
+}
+int vdnn_conv_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* dy, float* db) {
+    return ACT_CALL(conv_bwd_bias_impl, ctx, stream, shape, dy, db, 1.0f, 0);
+}
+int vdnn_fc_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const void* dy, float* bias, float alpha) {
+    return ACT_CALL(fc_bwd_bias_impl, ctx, stream, n, c_out, dy, bias, alpha, 1);
+}
+int vdnn_fc_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const void* dy, float* db) {
+    return ACT_CALL(fc_bwd_bias_impl, ctx, stream, n, c_out, dy, db, 1.0f, 0);
+}
+
+// param[i] += alpha * grad[i]: the optimizer step when gradients are kept instead of fused into backward
+int vdnn_sgd_apply(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float alpha, const float* grad, float* param) {
+    VDNN_KERNEL_PROLOGUE(ctx);
+    VDNN_REQUIRE(grad && param, "null tensor");
+    if (count == 0) return VDNN_OK;
+    hipStream_t st = stream_of(ctx, stream);
+    ProfScope prof(ctx, st, "sgd_apply", 0.0, 12.0 * (double)count);
+    hipLaunchKernelGGL(sgd_apply_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, st, grad, param, alpha, count);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+int vdnn_maxpool_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* x, void* y) { return ACT_CALL(maxpool_fwd_t, ctx, stream, shape, x, y); }
+int vdnn_maxpool_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* x, const void* y, const void* dy, void* dx) {
+    return ACT_CALL(maxpool_bwd_t, ctx, stream, shape, x, y, dy, dx);
+}
+int vdnn_lrn_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const void* x, void* y) { return ACT_CALL(lrn_fwd_t, ctx, stream, n, c, hw, x, y); }
+int vdnn_lrn_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const void* x, const void* y, const void* dy, void* dx) {
+    return ACT_CALL(lrn_bwd_t, ctx, stream, n, c, hw, x, y, dy, dx);
+}
+int vdnn_softmax_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* x, void* y) { return ACT_CALL(softmax_fwd_t, ctx, stream, n, classes, x, y); }
+int vdnn_softmax_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* y, const void* dy, void* dx) {
+    return ACT_CALL(softmax_bwd_t, ctx, stream, n, classes, y, dy, dx);
+}
+int vdnn_softmax_ce_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* logits, const int32_t* labels, void* prob, float* loss) {
+    return ACT_CALL(softmax_ce_fwd_t, ctx, stream, n, classes, logits, labels, prob, loss);
+}
+int vdnn_softmax_ce_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* prob, const int32_t* labels, void* dlogits) {
+    return ACT_CALL(softmax_ce_bwd_t, ctx, stream, n, classes, prob, labels, dlogits);
+}
+int vdnn_cross_entropy_dense(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int classes, const void* prob, const void* target, float* loss) {
+    return ACT_CALL(cross_entropy_dense_t, ctx, stream, n, classes, prob, target, loss);
 }
 
 } // extern "C"

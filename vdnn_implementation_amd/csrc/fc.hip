@@ -7,14 +7,16 @@ namespace vdnn {
 
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
                          int splits, float alpha, int accumulate, const float* bias_j, int ncols);
+int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, size_t count,
+                         int splits, float alpha, int accumulate, const float* bias_j, int ncols);
 
 static inline bool fc_aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 // Out[M][N] (dense, row stride N) = alpha * A*B (+ Out) (+ bias per column); the reduction is split into
 // ordered partial sums when the tile grid alone cannot fill the chip.
-template <class AL, class BL>
+template <class AL, class BL, class EO>
 static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const char* name, const AL& al, const BL& bl, int M, int N, int K,
-                   float* out, float alpha, int accumulate, const float* bias_j) {
+                   EO* out, float alpha, int accumulate, const float* bias_j) {
     const int TM = M <= 64 ? 64 : 128, TN = M <= 64 ? 256 : 128;
     const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
     long cap = ((long)K + 8 * KB - 1) / (8 * KB); // at least eight slices per split
@@ -28,11 +30,11 @@ static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const char* name, const AL& al
     kchunk = (kchunk + KB - 1) / KB * KB;
     d.kchunk = kchunk;
     d.splits = (K + kchunk - 1) / kchunk;
-    StoreDense ep{out, ctx->reduce_scratch, d.splits > 1 ? nullptr : bias_j, (long)N, (long)M * N, alpha, accumulate};
+    StoreDense<EO> ep{out, ctx->reduce_scratch, d.splits > 1 ? nullptr : bias_j, (long)N, (long)M * N, alpha, accumulate};
     const long blocks = (long)d.mtiles * d.ntiles * d.splits;
     ProfScope prof(ctx, st, name, 2.0 * M * (double)N * K, 0.0);
-    if (TM == 64) hipLaunchKernelGGL((igemm_kernel<64, 256, AL, BL, StoreDense>), dim3((unsigned)blocks), dim3(NT), 0, st, al, bl, ep, d);
-    else hipLaunchKernelGGL((igemm_kernel<128, 128, AL, BL, StoreDense>), dim3((unsigned)blocks), dim3(NT), 0, st, al, bl, ep, d);
+    if (TM == 64) hipLaunchKernelGGL((igemm_kernel<64, 256, AL, BL, StoreDense<EO>>), dim3((unsigned)blocks), dim3(NT), 0, st, al, bl, ep, d);
+    else hipLaunchKernelGGL((igemm_kernel<128, 128, AL, BL, StoreDense<EO>>), dim3((unsigned)blocks), dim3(NT), 0, st, al, bl, ep, d);
     VDNN_LAUNCH_CHECK();
     if (d.splits > 1) return launch_reduce_splits(ctx, st, out, ctx->reduce_scratch, (size_t)M * N, d.splits, alpha, accumulate, bias_j, N);
     return VDNN_OK;
@@ -44,60 +46,79 @@ using namespace vdnn;
 
 #define FC_REQUIRE_SMALL(elems) VDNN_REQUIRE((long)(elems) * 4 < 0x7FFF0000l, "matrix of 2 GiB or more")
 
-extern "C" {
-
 // y[n][o] = sum_i x[n][i] * w[o][i] + bias[o]        (Sgemm(T,N) + bias broadcast, layer.cu:677-706)
-int vdnn_fc_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
-                const float* x, const float* w, const float* bias, float* y) {
+template <class E>
+static int fc_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                       const E* x, const float* w, const float* bias, E* y) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && w && y && n > 0 && c_in > 0 && c_out > 0, "bad argument");
     FC_REQUIRE_SMALL((long)n * c_in); FC_REQUIRE_SMALL((long)c_out * c_in);
-    const unsigned xb = (unsigned)((long)n * c_in * 4), wb = (unsigned)((long)c_out * c_in * 4);
+    const unsigned xb = (unsigned)((long)n * c_in * sizeof(E)), wb = (unsigned)((long)c_out * c_in * 4);
     hipStream_t st = stream_of(ctx, stream);
     if (c_in % 4 == 0 && fc_aligned16(x) && fc_aligned16(w)) {
-        LoadDenseRed<true> al{x, (long)c_in, n, xb}, bl{w, (long)c_in, c_out, wb};
+        LoadDenseRed<true, E> al{x, (long)c_in, n, xb};
+        LoadDenseRed<true> bl{w, (long)c_in, c_out, wb};
         return fc_gemm(ctx, st, "fc_fwd", al, bl, n, c_out, c_in, y, 1.0f, 0, bias);
     }
-    LoadDenseRed<false> al{x, (long)c_in, n, xb}, bl{w, (long)c_in, c_out, wb};
+    LoadDenseRed<false, E> al{x, (long)c_in, n, xb};
+    LoadDenseRed<false> bl{w, (long)c_in, c_out, wb};
     return fc_gemm(ctx, st, "fc_fwd", al, bl, n, c_out, c_in, y, 1.0f, 0, bias);
 }
 
 // dx[n][i] = sum_o dy[n][o] * w[o][i]                 (Sgemm(N,N), layer.cu:725-733)
-int vdnn_fc_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
-                     const float* dy, const float* w, float* dx) {
+template <class E>
+static int fc_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                            const E* dy, const float* w, E* dx) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(dy && w && dx && n > 0 && c_in > 0 && c_out > 0, "bad argument");
     FC_REQUIRE_SMALL((long)n * c_out); FC_REQUIRE_SMALL((long)c_out * c_in);
-    const unsigned db = (unsigned)((long)n * c_out * 4), wb = (unsigned)((long)c_out * c_in * 4);
+    const unsigned db = (unsigned)((long)n * c_out * sizeof(E)), wb = (unsigned)((long)c_out * c_in * 4);
     hipStream_t st = stream_of(ctx, stream);
-    LoadDenseRow bl{w, (long)c_in, c_in, wb};
+    LoadDenseRow<float> bl{w, (long)c_in, c_in, wb};
     if (c_out % 4 == 0 && fc_aligned16(dy)) {
-        LoadDenseRed<true> al{dy, (long)c_out, n, db};
+        LoadDenseRed<true, E> al{dy, (long)c_out, n, db};
         return fc_gemm(ctx, st, "fc_bwd_data", al, bl, n, c_in, c_out, dx, 1.0f, 0, nullptr);
     }
-    LoadDenseRed<false> al{dy, (long)c_out, n, db};
+    LoadDenseRed<false, E> al{dy, (long)c_out, n, db};
     return fc_gemm(ctx, st, "fc_bwd_data", al, bl, n, c_in, c_out, dx, 1.0f, 0, nullptr);
 }
 
-// w[o][i] += alpha * sum_n dy[n][o] * x[n][i]         (Sgemm(N,T) alpha=-lr beta=1, layer.cu:736-744)
-int vdnn_fc_bwd_weight_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
-                           const float* x, const float* dy, float* w, float alpha) {
+// out[o][i] = (accumulate ? out : 0) + alpha * sum_n dy[n][o] * x[n][i]   (Sgemm(N,T), layer.cu:736-744)
+template <class E>
+static int fc_bwd_weight_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                              const E* x, const E* dy, float* w, float alpha, int accumulate) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && dy && w && n > 0 && c_in > 0 && c_out > 0, "bad argument");
     FC_REQUIRE_SMALL((long)n * c_out); FC_REQUIRE_SMALL((long)n * c_in);
-    LoadDenseRow al{dy, (long)c_out, c_out, (unsigned)((long)n * c_out * 4)};
-    LoadDenseRow bl{x, (long)c_in, c_in, (unsigned)((long)n * c_in * 4)};
-    return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_weight", al, bl, c_out, c_in, n, w, alpha, 1, nullptr);
+    LoadDenseRow<E> al{dy, (long)c_out, c_out, (unsigned)((long)n * c_out * sizeof(E))};
+    LoadDenseRow<E> bl{x, (long)c_in, c_in, (unsigned)((long)n * c_in * sizeof(E))};
+    return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_weight", al, bl, c_out, c_in, n, w, alpha, accumulate, nullptr);
+}
+
+extern "C" {
+
+int vdnn_fc_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                const void* x, const float* w, const float* bias, void* y) {
+    return VDNN_BY_ACT(ctx, fc_fwd_impl<float>(ctx, stream, n, c_in, c_out, (const float*)x, w, bias, (float*)y),
+                       fc_fwd_impl<bf16_t>(ctx, stream, n, c_in, c_out, (const bf16_t*)x, w, bias, (bf16_t*)y));
+}
+
+int vdnn_fc_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                     const void* dy, const float* w, void* dx) {
+    return VDNN_BY_ACT(ctx, fc_bwd_data_impl<float>(ctx, stream, n, c_in, c_out, (const float*)dy, w, (float*)dx),
+                       fc_bwd_data_impl<bf16_t>(ctx, stream, n, c_in, c_out, (const bf16_t*)dy, w, (bf16_t*)dx));
+}
+
+int vdnn_fc_bwd_weight_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                           const void* x, const void* dy, float* w, float alpha) {
+    return VDNN_BY_ACT(ctx, fc_bwd_weight_impl<float>(ctx, stream, n, c_in, c_out, (const float*)x, (const float*)dy, w, alpha, 1),
+                       fc_bwd_weight_impl<bf16_t>(ctx, stream, n, c_in, c_out, (const bf16_t*)x, (const bf16_t*)dy, w, alpha, 1));
 }
 
 int vdnn_fc_bwd_weight(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
-                       const float* x, const float* dy, float* dw) {
-    VDNN_KERNEL_PROLOGUE(ctx);
-    VDNN_REQUIRE(x && dy && dw && n > 0 && c_in > 0 && c_out > 0, "bad argument");
-    FC_REQUIRE_SMALL((long)n * c_out); FC_REQUIRE_SMALL((long)n * c_in);
-    LoadDenseRow al{dy, (long)c_out, c_out, (unsigned)((long)n * c_out * 4)};
-    LoadDenseRow bl{x, (long)c_in, c_in, (unsigned)((long)n * c_in * 4)};
-    return fc_gemm(ctx, stream_of(ctx, stream), "fc_bwd_weight", al, bl, c_out, c_in, n, dw, 1.0f, 0, nullptr);
+                       const void* x, const void* dy, float* dw) {
+    return VDNN_BY_ACT(ctx, fc_bwd_weight_impl<float>(ctx, stream, n, c_in, c_out, (const float*)x, (const float*)dy, dw, 1.0f, 0),
+                       fc_bwd_weight_impl<bf16_t>(ctx, stream, n, c_in, c_out, (const bf16_t*)x, (const bf16_t*)dy, dw, 1.0f, 0));
 }
 
 } // extern "C"

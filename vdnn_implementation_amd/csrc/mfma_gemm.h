@@ -81,6 +81,43 @@ __device__ __forceinline__ unsigned clamp_range(long bytes) {
     return bytes <= 0 ? 0u : (bytes > 0xFFFFFFF0l ? 0xFFFFFFF0u : (unsigned)bytes);
 }
 
+// ---- element types of activation tensors -------------------------------------------------------------
+// Activations are float or bfloat16 in memory; every kernel computes in float. A bf16 value is the
+// upper half of the float with the same value; storing rounds to nearest, ties to even, NaN stays NaN.
+struct bf16_t { unsigned short bits; };
+template <class E> struct ElemBytes { static constexpr int V = (int)sizeof(E); };
+
+__host__ __device__ __forceinline__ float bf16_bits_to_float(unsigned bits) {
+    return __builtin_bit_cast(float, bits << 16);
+}
+__host__ __device__ __forceinline__ unsigned short float_to_bf16_bits(float f) {
+    unsigned u = __builtin_bit_cast(unsigned, f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (unsigned short)((u >> 16) | 0x40u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (unsigned short)(u >> 16);
+}
+__device__ __forceinline__ float load_elem(const float* p) { return *p; }
+__device__ __forceinline__ float load_elem(const bf16_t* p) { return bf16_bits_to_float(p->bits); }
+__device__ __forceinline__ void store_elem(float* p, float v) { *p = v; }
+__device__ __forceinline__ void store_elem(bf16_t* p, float v) { p->bits = float_to_bf16_bits(v); }
+
+// one element / four consecutive elements through a descriptor, as float (offsets in bytes)
+template <class E> __device__ __forceinline__ float buf_load_e(__amdgpu_buffer_rsrc_t r, int voff, int soff);
+template <> __device__ __forceinline__ float buf_load_e<float>(__amdgpu_buffer_rsrc_t r, int voff, int soff) { return buf_load(r, voff, soff); }
+template <> __device__ __forceinline__ float buf_load_e<bf16_t>(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    return bf16_bits_to_float((unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0));
+}
+template <class E> __device__ __forceinline__ floatx4 buf_load4_e(__amdgpu_buffer_rsrc_t r, int voff, int soff);
+template <> __device__ __forceinline__ floatx4 buf_load4_e<float>(__amdgpu_buffer_rsrc_t r, int voff, int soff) { return buf_load4(r, voff, soff); }
+template <> __device__ __forceinline__ floatx4 buf_load4_e<bf16_t>(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
+    const uintx2 w = __builtin_bit_cast(uintx2, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
+    floatx4 v;
+    v.x = __builtin_bit_cast(float, w.x << 16); v.y = __builtin_bit_cast(float, w.x & 0xFFFF0000u);
+    v.z = __builtin_bit_cast(float, w.y << 16); v.w = __builtin_bit_cast(float, w.y & 0xFFFF0000u);
+    return v;
+}
+
 // ---- LDS tile geometry ------------------------------------------------------------------------------
 template <int T, bool RED_MAJOR>
 struct LdsTile {
@@ -231,10 +268,11 @@ __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, con
 // VEC4: rows are 16-byte aligned and the reduction range is a multiple of four, so a thread moves
 // 128-bit chunks (thread t: chunk t%4 of rows t/4 + 64*i). Otherwise 32-bit elements
 // (thread t: kk t%16 of rows t/16 + 16*i).
-template <bool VEC4>
+template <bool VEC4, class E = float>
 struct LoadDenseRed {
     static constexpr bool RED_MAJOR = true;
-    const float* base;
+    static constexpr int ES = ElemBytes<E>::V;
+    const E* base;
     long ld;          // elements between rows
     int rows;         // valid rows
     unsigned bytes;   // extent of the matrix in bytes (below 2 GiB)
@@ -247,29 +285,29 @@ struct LoadDenseRed {
 #pragma unroll
             for (int i = 0; i < T / 64; i++) {
                 const int row = row0 + (tid >> 2) + 64 * i;
-                st.vrow[i] = row < rows ? (int)(((long)row * ld + 4 * (tid & 3)) * 4) : OOB;
+                st.vrow[i] = row < rows ? (int)(((long)row * ld + 4 * (tid & 3)) * ES) : OOB;
             }
         } else {
 #pragma unroll
             for (int i = 0; i < T / 16; i++) {
                 const int row = row0 + (tid >> 4) + 16 * i;
-                st.vrow[i] = row < rows ? (int)(((long)row * ld + (tid & 15)) * 4) : OOB;
+                st.vrow[i] = row < rows ? (int)(((long)row * ld + (tid & 15)) * ES) : OOB;
             }
         }
     }
     template <int T>
     __device__ __forceinline__ void load(State<T>& st, int kk0, int kend, int tid, Regs<T>& r) const {
-        const int soff = kk0 * 4;
+        const int soff = kk0 * ES;
         // only the last slice of a range can be partial; there a thread past the end reads out of range
         const bool tail = kk0 + KB > kend;
         if (VEC4) {
             const bool dead = tail && (kk0 + 4 * (tid & 3) >= kend);
 #pragma unroll
-            for (int i = 0; i < T / 64; i++) r.v[i] = buf_load4(st.rsrc, dead ? OOB : st.vrow[i], soff);
+            for (int i = 0; i < T / 64; i++) r.v[i] = buf_load4_e<E>(st.rsrc, dead ? OOB : st.vrow[i], soff);
         } else {
             const bool dead = tail && (kk0 + (tid & 15) >= kend);
 #pragma unroll
-            for (int i = 0; i < T / 16; i++) r.s[i] = buf_load(st.rsrc, dead ? OOB : st.vrow[i], soff);
+            for (int i = 0; i < T / 16; i++) r.s[i] = buf_load_e<E>(st.rsrc, dead ? OOB : st.vrow[i], soff);
         }
     }
     template <int T>
@@ -286,9 +324,11 @@ struct LoadDenseRed {
 
 // ---- dense row-major operand: element (row, kk) at base[kk*ld_k + row] ------------------------------
 // lanes run along rows (coalesced); the reduction index is wave-uniform and lives in the scalar offset
+template <class E = float>
 struct LoadDenseRow {
     static constexpr bool RED_MAJOR = false;
-    const float* base;
+    static constexpr int ES = ElemBytes<E>::V;
+    const E* base;
     long ld_k;        // elements between consecutive kk
     int rows;
     unsigned bytes;   // extent in bytes (below 2 GiB)
@@ -298,7 +338,7 @@ struct LoadDenseRow {
     __device__ __forceinline__ void init(State<T>& st, int row0, int tid, int, int) const {
         st.rsrc = make_rsrc(base, bytes);
         const int row = row0 + tid % T;
-        st.vrow = row < rows ? row * 4 : OOB;
+        st.vrow = row < rows ? row * ES : OOB;
     }
     template <int T>
     __device__ __forceinline__ void load(State<T>& st, int kk0, int kend, int tid, Regs<T>& r) const {
@@ -306,8 +346,8 @@ struct LoadDenseRow {
 #pragma unroll
         for (int i = 0; i < T * KB / NT; i++) {
             const int kk = kbase + (NT / T) * i;
-            const int soff = kk < kend ? (int)((long)kk * ld_k * 4) : 0x7FFFFFF0;
-            r.s[i] = buf_load(st.rsrc, st.vrow, soff);
+            const int soff = kk < kend ? (int)((long)kk * ld_k * ES) : 0x7FFFFFF0;
+            r.s[i] = buf_load_e<E>(st.rsrc, st.vrow, soff);
         }
     }
     template <int T>
@@ -319,8 +359,9 @@ struct LoadDenseRow {
 
 // ---- dense result: out[m*ld_m + j] = alpha*acc (+ old if accumulate) (+ bias[j]); or a split's
 //      partial sums to scratch[ks][m*ld_m + j] ------------------------------------------------------
+template <class E = float>
 struct StoreDense {
-    float* out;
+    E* out;
     float* partial;     // used when splits > 1
     const float* bias_j; // optional, indexed by column
     long ld_m;
@@ -345,9 +386,9 @@ struct StoreDense {
                         partial[(long)ks * partial_stride + idx] = a;
                     } else {
                         // one fused multiply-add: every route to "out += alpha * sum" rounds the same way
-                        float r = accumulate ? __fmaf_rn(alpha, a, out[idx]) : alpha * a;
+                        float r = accumulate ? __fmaf_rn(alpha, a, load_elem(out + idx)) : alpha * a;
                         if (bias_j) r += bias_j[j];
-                        out[idx] = r;
+                        store_elem(out + idx, r);
                     }
                 }
         }
