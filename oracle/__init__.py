@@ -66,7 +66,7 @@ _sig("orc_fc_bwd_weight_sgd", None, C.c_int, C.c_int, C.c_int, _f, _f, _f, C.c_f
 _sig("orc_fc_bwd_bias_sgd", None, C.c_int, C.c_int, _f, _f, C.c_float)
 _sig("orc_relu_fwd", None, C.c_size_t, _f, _f)
 _sig("orc_relu_bwd", None, C.c_size_t, _f, _f, _f, _f)
-for _name in ("orc_tanh_fwd", "orc_sigmoid_fwd"):
+for _name in ("orc_tanh_fwd", "orc_sigmoid_fwd", "orc_round_bf16"):
     _sig(_name, None, C.c_size_t, _f, _f)
 for _name in ("orc_tanh_bwd", "orc_sigmoid_bwd"):
     _sig(_name, None, C.c_size_t, _f, _f, _f)
@@ -230,6 +230,11 @@ def _act_bwd(fn, y, dy):
     dx = np.empty_like(dy)
     fn(dy.size, _p(y), _p(dy), _p(dx))
     return dx
+
+
+def round_bf16(x):
+    """x rounded to the nearest bfloat16 (ties to even), as float32."""
+    return _act_fwd(lib.orc_round_bf16, x)
 
 
 def tanh_fwd(x):

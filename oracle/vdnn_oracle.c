@@ -4,6 +4,7 @@
 
 #include <float.h>
 #include <math.h>
+#include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
 #ifdef _OPENMP
@@ -394,6 +395,27 @@ void orc_relu_bwd(size_t count, const float* x, const float* y, const float* dy,
     const float* t = x ? x : y;
 #pragma omp parallel for schedule(static)
     for (size_t i = 0; i < count; i++) dx[i] = (t[i] > 0.0f) ? dy[i] : 0.0f;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * bfloat16 storage (the reduced-precision configuration; the reference is float only, vdnn.h:11-12).
+ * A bfloat16 value is the float whose low 16 bits are zero. Rounding a float to it: to nearest, ties
+ * to even; infinities stay, NaN stays NaN (quiet). y[i] is x[i] rounded, still held as a float.
+ * ------------------------------------------------------------------------------------------- */
+void orc_round_bf16(size_t count, const float* x, float* y) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) {
+        uint32_t u;
+        memcpy(&u, &x[i], 4);
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u) {
+            u = (u | 0x00400000u) & 0xFFFF0000u;
+        } else {
+            const uint32_t lower = u & 0xFFFFu, odd = (u >> 16) & 1u;
+            u &= 0xFFFF0000u;
+            if (lower > 0x8000u || (lower == 0x8000u && odd)) u += 0x10000u;
+        }
+        memcpy(&y[i], &u, 4);
+    }
 }
 
 /* ---------------------------------------------------------------------------------------------

@@ -14,6 +14,8 @@
  *   bias add / bias grad / sub / fill: closed form
  *   fc fwd / bwd-data / bwd-weight   : numpy matmul
  *   relu                             : closed form incl. -0, NaN, inf
+ *   bfloat16 rounding                : torch's float32 -> bfloat16 conversion on random values, exact ties,
+ *                                      subnormals, infinities and NaN
  *   tanh / sigmoid fwd / bwd         : torch.tanh / torch.sigmoid + autograd in float64, special values,
  *                                      the identities tanh(-x) = -tanh(x), sigmoid(x) + sigmoid(-x) = 1
  *   maxpool fwd / bwd                : torch max_pool2d + autograd fixtures on tie-free data
@@ -76,6 +78,7 @@ void orc_fc_bwd_bias_sgd(int n, int c_out, const float* dy, float* bias, float a
 /* layer.cu:774-781, 802-811 */
 void orc_relu_fwd(size_t count, const float* x, float* y);
 void orc_relu_bwd(size_t count, const float* x, const float* y, const float* dy, float* dx);
+void orc_round_bf16(size_t count, const float* x, float* y);
 void orc_tanh_fwd(size_t count, const float* x, float* y);
 void orc_tanh_bwd(size_t count, const float* y, const float* dy, float* dx);
 void orc_sigmoid_fwd(size_t count, const float* x, float* y);

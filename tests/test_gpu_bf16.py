@@ -1,0 +1,223 @@
+"""GPU parity with bfloat16 activation storage, through the C ABI.
+
+Activation tensors are bfloat16 in memory, parameters float, arithmetic float with float accumulation;
+a result is rounded once when stored. The checker computes the same layer on the same (bfloat16-valued)
+inputs in double and the GPU result must lie within one bfloat16 unit in the last place of it
+(util.assert_close_bf16). ReLU, max-pool and subtraction have exactly representable results: bit-exact.
+"""
+import numpy as np
+import pytest
+
+import oracle
+import vdnn_implementation_amd.backend as be
+from gpu_util import announce
+from util import assert_close, assert_close_bf16, from_bf16_bits, to_bf16_bits
+from vdnn_implementation_amd.backend import check, lib
+
+pytestmark = pytest.mark.gpu
+BF16 = 1
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = be.Context(pool_bytes=4 << 30)
+    check(lib.vdnn_ctx_set_activation_dtype(c.handle, BF16))
+    assert lib.vdnn_ctx_activation_dtype(c.handle) == BF16
+    yield c
+    c.close()
+
+
+@pytest.fixture(autouse=True)
+def accurate_oracle():
+    oracle.set_accumulate_double(True)
+    yield
+    oracle.set_accumulate_double(False)
+
+
+class Dev:
+    def __init__(self, ctx):
+        self.ctx, self.bufs = ctx, []
+
+    def act(self, a):
+        """uploads a bfloat16-valued float32 array as bfloat16"""
+        b = self.ctx.to_device(to_bf16_bits(a), np.uint16)
+        self.bufs.append(b)
+        return b
+
+    def f32(self, a):
+        b = self.ctx.to_device(a, np.float32)
+        self.bufs.append(b)
+        return b
+
+    def empty_act(self, shape):
+        b = self.ctx.alloc(max(int(np.prod(shape)) * 2, 4))
+        self.bufs.append(b)
+        return b
+
+    def raw(self, nbytes):
+        b = self.ctx.alloc(max(nbytes, 4))
+        self.bufs.append(b)
+        return b
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        for b in self.bufs:
+            b.free()
+
+
+def get_act(buf, shape):
+    return from_bf16_bits(buf.download(shape, np.uint16))
+
+
+def rnd(rng, shape, scale=1.0):
+    return oracle.round_bf16((rng.standard_normal(shape) * scale).astype(np.float32))
+
+
+def ws(d, g, algo, which):
+    n = int(lib.vdnn_conv_workspace_bytes(g, algo, which))
+    return (d.raw(n).ptr, n) if n else (None, 0)
+
+
+CONV = [
+    (3, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1),     # blocked tap-major loaders, 64-row tile
+    (2, 128, 14, 14, 256, 3, 3, 1, 1, 1, 1),   # two row tiles
+    (2, 3, 32, 32, 64, 3, 3, 1, 1, 1, 1),      # three input channels: dense forward, vector-ALU backward passes
+    (2, 70, 9, 13, 130, 3, 3, 1, 1, 1, 1),     # nothing divides the tiles; odd plane size (scalar dy loads)
+    (2, 3, 67, 67, 96, 11, 11, 0, 0, 4, 4),    # AlexNet conv1: large window, stride 4
+    (2, 48, 27, 27, 96, 5, 5, 2, 2, 1, 1),     # AlexNet conv2
+    (5, 64, 6, 6, 200, 6, 6, 0, 0, 1, 1),      # OverFeat 6x6 -> 1x1
+    (1, 16, 20, 24, 32, 3, 5, 1, 2, 2, 1),     # asymmetric, strided backward data
+]
+
+
+@pytest.mark.parametrize("geom", CONV, ids=lambda g: "x".join(map(str, g)))
+@pytest.mark.parametrize("algo", [0, 1])
+def test_conv_bf16(ctx, geom, algo):
+    rng = np.random.default_rng(hash(geom) % (2 ** 31) + 7)
+    g, og = be.shape(*geom), oracle.shape(*geom)
+    x = rnd(rng, (g.n, g.c, g.h, g.w))
+    w = (rng.standard_normal((g.k, g.c, g.r, g.s)) * np.sqrt(2.0 / (g.c * g.r * g.s))).astype(np.float32)
+    b = rng.standard_normal(g.k).astype(np.float32)
+    want_y = oracle.conv_fwd(og, x, w, b)
+    dy = rnd(rng, want_y.shape)
+    with Dev(ctx) as d:
+        dx_, ddy, dw, db = d.act(x), d.act(dy), d.f32(w), d.f32(b)
+        y, gx = d.empty_act(want_y.shape), d.empty_act(x.shape)
+        announce("conv bf16", geom, "algo", algo, "fwd")
+        p, n = ws(d, g, algo, 0)
+        check(lib.vdnn_conv_fwd(ctx.handle, None, g, algo, dx_.ptr, dw.ptr, db.ptr, y.ptr, p, n))
+        assert_close_bf16(get_act(y, want_y.shape), want_y, "fwd")
+        announce("conv bf16", geom, "algo", algo, "bwd_data")
+        p, n = ws(d, g, algo, 1)
+        check(lib.vdnn_conv_bwd_data(ctx.handle, None, g, algo, ddy.ptr, dw.ptr, gx.ptr, p, n))
+        assert_close_bf16(get_act(gx, x.shape), oracle.conv_bwd_data(og, dy, w), "bwd data")
+        # parameter gradients stay float: the float tolerance applies
+        announce("conv bf16", geom, "algo", algo, "bwd_filter")
+        gw = d.f32(np.zeros_like(w))
+        p, n = ws(d, g, algo, 2)
+        check(lib.vdnn_conv_bwd_filter(ctx.handle, None, g, algo, dx_.ptr, ddy.ptr, gw.ptr, p, n))
+        assert_close(gw.download(w.shape), oracle.conv_bwd_filter_sgd(og, x, dy, np.zeros_like(w), 1.0), 1e-4, "bwd filter")
+        announce("conv bf16", geom, "algo", algo, "bwd_bias")
+        gb = d.f32(np.zeros_like(b))
+        check(lib.vdnn_conv_bwd_bias(ctx.handle, None, g, ddy.ptr, gb.ptr))
+        assert_close(gb.download(b.shape), oracle.conv_bwd_bias_sgd(og, dy, np.zeros_like(b), 1.0), 1e-4, "bwd bias")
+
+
+@pytest.mark.parametrize("n,cin,cout", [(128, 1000, 520), (64, 2304, 512), (5, 41, 33)])
+def test_fc_bf16(ctx, n, cin, cout):
+    rng = np.random.default_rng(n + cin)
+    x, dy = rnd(rng, (n, cin)), rnd(rng, (n, cout))
+    w = (rng.standard_normal((cout, cin)) / np.sqrt(cin)).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    announce("fc bf16", n, cin, cout)
+    with Dev(ctx) as d:
+        dx_, ddy, dw, db = d.act(x), d.act(dy), d.f32(w), d.f32(b)
+        y, gx, gw, gb = d.empty_act((n, cout)), d.empty_act((n, cin)), d.f32(np.zeros_like(w)), d.f32(np.zeros_like(b))
+        check(lib.vdnn_fc_fwd(ctx.handle, None, n, cin, cout, dx_.ptr, dw.ptr, db.ptr, y.ptr))
+        check(lib.vdnn_fc_bwd_data(ctx.handle, None, n, cin, cout, ddy.ptr, dw.ptr, gx.ptr))
+        check(lib.vdnn_fc_bwd_weight(ctx.handle, None, n, cin, cout, dx_.ptr, ddy.ptr, gw.ptr))
+        check(lib.vdnn_fc_bwd_bias(ctx.handle, None, n, cout, ddy.ptr, gb.ptr))
+        assert_close_bf16(get_act(y, (n, cout)), oracle.fc_fwd(x, w, b), "fc fwd")
+        assert_close_bf16(get_act(gx, (n, cin)), oracle.fc_bwd_data(dy, w), "fc bwd data")
+        assert_close(gw.download(w.shape), oracle.fc_bwd_weight_sgd(x, dy, np.zeros_like(w), 1.0), 1e-4, "fc dW")
+        assert_close(gb.download(b.shape), oracle.fc_bwd_bias_sgd(dy, np.zeros_like(b), 1.0), 1e-4, "fc db")
+
+
+@pytest.mark.parametrize("count", [1, 7, 4096 * 5 + 3])
+def test_elementwise_bf16(ctx, count):
+    rng = np.random.default_rng(count)
+    x, dy = rnd(rng, count, 2.0), rnd(rng, count)
+    x[: min(4, count)] = np.array([0.0, -0.0, np.inf, -1.0], np.float32)[: min(4, count)]
+    announce("elementwise bf16", count)
+    with Dev(ctx) as d:
+        dx_, ddy, y, gx = d.act(x), d.act(dy), d.empty_act(count), d.empty_act(count)
+        check(lib.vdnn_relu_fwd(ctx.handle, None, count, dx_.ptr, y.ptr))
+        got_y = get_act(y, count)
+        assert np.array_equal(got_y.view(np.uint32), oracle.relu_fwd(x).view(np.uint32))
+        check(lib.vdnn_relu_bwd(ctx.handle, None, count, dx_.ptr, y.ptr, ddy.ptr, gx.ptr))
+        assert np.array_equal(get_act(gx, count), oracle.relu_bwd(x, got_y, dy))
+        check(lib.vdnn_relu_bwd(ctx.handle, None, count, None, y.ptr, ddy.ptr, gx.ptr))
+        assert np.array_equal(get_act(gx, count), oracle.relu_bwd(x, got_y, dy))
+        check(lib.vdnn_sub(ctx.handle, None, count, dx_.ptr, ddy.ptr, y.ptr))
+        fin = np.isfinite(x)
+        assert np.array_equal(get_act(y, count)[fin], oracle.round_bf16(x - dy)[fin])
+        xs = np.where(fin, x, 1.0).astype(np.float32)
+        dxs = d.act(xs)
+        for name, fwd, bwd in (("tanh", oracle.tanh_fwd, oracle.tanh_bwd), ("sigmoid", oracle.sigmoid_fwd, oracle.sigmoid_bwd)):
+            check(getattr(lib, "vdnn_%s_fwd" % name)(ctx.handle, None, count, dxs.ptr, y.ptr))
+            gy = get_act(y, count)
+            assert_close_bf16(gy, fwd(xs), name)
+            check(getattr(lib, "vdnn_%s_bwd" % name)(ctx.handle, None, count, y.ptr, ddy.ptr, gx.ptr))
+            assert_close_bf16(get_act(gx, count), bwd(gy, dy), name + " bwd")
+        check(lib.vdnn_fill(ctx.handle, None, count, 0.3, y.ptr))
+        assert np.all(get_act(y, count) == oracle.round_bf16(np.float32([0.3]))[0])
+
+
+@pytest.mark.parametrize("n,c,h,w,win,stride", [(2, 8, 16, 16, 2, 2), (2, 5, 13, 13, 3, 2), (3, 4, 6, 10, 2, 2), (1, 3, 8, 12, 2, 2)])
+def test_maxpool_bf16_is_exact(ctx, n, c, h, w, win, stride):
+    rng = np.random.default_rng(h * w)
+    g = be.shape(n, c, h, w, 0, win, win, 0, 0, stride, stride)
+    og = oracle.shape(n, c, h, w, 0, win, win, 0, 0, stride, stride)
+    x = rnd(rng, (n, c, h, w))
+    want = oracle.maxpool_fwd(og, x)
+    dy = rnd(rng, want.shape)
+    announce("maxpool bf16", n, c, h, w, win, stride)
+    with Dev(ctx) as d:
+        dx_, ddy, y, gx = d.act(x), d.act(dy), d.empty_act(want.shape), d.empty_act(x.shape)
+        check(lib.vdnn_maxpool_fwd(ctx.handle, None, g, dx_.ptr, y.ptr))
+        assert np.array_equal(get_act(y, want.shape), want)
+        check(lib.vdnn_maxpool_bwd(ctx.handle, None, g, dx_.ptr, y.ptr, ddy.ptr, gx.ptr))
+        # overlapping windows add several dy: the sum is rounded once
+        assert_close_bf16(get_act(gx, x.shape), oracle.maxpool_bwd(og, x, want, dy), "pool bwd", ulps=0.51)
+
+
+def test_lrn_softmax_and_loss_bf16(ctx):
+    rng = np.random.default_rng(3)
+    x, dy = rnd(rng, (3, 24, 5, 7), 20.0), rnd(rng, (3, 24, 5, 7))
+    announce("lrn bf16")
+    with Dev(ctx) as d:
+        dx_, ddy, y, gx = d.act(x), d.act(dy), d.empty_act(x.shape), d.empty_act(x.shape)
+        check(lib.vdnn_lrn_fwd(ctx.handle, None, 3, 24, 35, dx_.ptr, y.ptr))
+        gy = get_act(y, x.shape)
+        assert_close_bf16(gy, oracle.lrn_fwd(x), "lrn fwd")
+        check(lib.vdnn_lrn_bwd(ctx.handle, None, 3, 24, 35, dx_.ptr, y.ptr, ddy.ptr, gx.ptr))
+        assert_close_bf16(get_act(gx, x.shape), oracle.lrn_bwd(x, gy, dy), "lrn bwd")
+    n, classes = 6, 1000
+    logits, dyl = rnd(rng, (n, classes), 3.0), rnd(rng, (n, classes))
+    labels = rng.integers(0, classes, n).astype(np.int32)
+    target = np.zeros((n, classes), np.float32)
+    target[np.arange(n), labels] = 1.0
+    announce("softmax bf16")
+    with Dev(ctx) as d:
+        dl, ddy, prob, gx, dt = d.act(logits), d.act(dyl), d.empty_act((n, classes)), d.empty_act((n, classes)), d.act(target)
+        loss = d.f32(np.zeros(1, np.float32))
+        check(lib.vdnn_softmax_fwd(ctx.handle, None, n, classes, dl.ptr, prob.ptr))
+        gp = get_act(prob, (n, classes))
+        assert_close_bf16(gp, oracle.softmax_fwd(logits), "softmax fwd")
+        check(lib.vdnn_softmax_bwd(ctx.handle, None, n, classes, prob.ptr, ddy.ptr, gx.ptr))
+        assert_close_bf16(get_act(gx, (n, classes)), oracle.softmax_bwd(gp, dyl), "softmax bwd")
+        check(lib.vdnn_cross_entropy_dense(ctx.handle, None, n, classes, prob.ptr, dt.ptr, loss.ptr))
+        want = float(np.mean(-np.log(gp[np.arange(n), labels].astype(np.float64))))
+        assert abs(loss.download((1,))[0] - want) <= 1e-5 * abs(want)

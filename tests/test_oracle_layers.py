@@ -253,3 +253,21 @@ def test_tanh_and_sigmoid_against_torch_and_identities():
     assert np.isnan(oracle.tanh_fwd(np.array([np.nan], np.float32))[0]) and np.isnan(oracle.sigmoid_fwd(np.array([np.nan], np.float32))[0])
     assert np.array_equal(oracle.tanh_fwd(-x), -oracle.tanh_fwd(x))
     assert_close(oracle.sigmoid_fwd(x).astype(np.float64) + oracle.sigmoid_fwd(-x), np.ones_like(x), 1e-7, "sigmoid(x) + sigmoid(-x)")
+
+
+def test_bf16_rounding_against_torch():
+    import torch
+    rng = np.random.default_rng(8)
+    x = np.concatenate([
+        (rng.standard_normal(20000) * 10.0 ** rng.integers(-30, 30, 20000)).astype(np.float32),
+        np.array([0.0, -0.0, 1.0, np.inf, -np.inf, 3.4028235e38, 1e-45, -1e-40], np.float32),
+        # exact ties: 1 + 2^-8 (even below: rounds down), 1 + 3*2^-8 (odd below: rounds up), and just past a tie
+        np.array([1.00390625, 1.01171875, np.nextafter(np.float32(1.00390625), np.float32(2))], np.float32)])
+    want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+    got = oracle.round_bf16(x)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert got[-3] == 1.0 and got[-2] == np.float32(1.015625) and got[-1] == np.float32(1.0078125)
+    assert np.isinf(oracle.round_bf16(np.array([3.4028235e38], np.float32))[0])
+    n = oracle.round_bf16(np.array([np.nan], np.float32))
+    assert np.isnan(n[0]) and not (n.view(np.uint32)[0] & 0xFFFF)
+    assert np.array_equal(oracle.round_bf16(got).view(np.uint32), got.view(np.uint32))  # idempotent
