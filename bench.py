@@ -39,8 +39,8 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0):
-    net = Network(cnn, policy, algo, batch, seed=seed, refined=refined, cap_bytes=cap_bytes)
+def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0, bf16=False):
+    net = Network(cnn, policy, algo, batch, seed=seed, refined=refined, cap_bytes=cap_bytes, bf16=bf16)
     try:
         for _ in range(warmup):
             assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
@@ -101,6 +101,7 @@ def main():
     ap.add_argument("--algo", default="VDNN_MEMORY_OPT_ALGO")
     ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined")
     ap.add_argument("--cap-gb", type=float, default=0.0, help="artificial limit on pool bytes in use (0 = none)")
+    ap.add_argument("--bf16", action="store_true", help="bfloat16 activation storage (float parameters and arithmetic)")
     ap.add_argument("--cpu-batch", type=int, default=24)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -120,7 +121,7 @@ def main():
         _, policy, algo = parse("VGG16_128", word, args.algo)
         log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
         results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1,
-                                                   refined=(suffix == "refined"), cap_bytes=int(args.cap_gb * 1e9))
+                                                   refined=(suffix == "refined"), cap_bytes=int(args.cap_gb * 1e9), bf16=args.bf16)
         log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
             results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))
 
@@ -148,8 +149,8 @@ def main():
         "metric": "VGG16-128 train img/s (VDNN_ALL vs BASELINE); peak HBM GB; conv MFMA util",
         "value": results[head]["images_per_s"], "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": results[head]["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic (seeded N(0,1) inputs, integer labels, He-normal filters)",
-        "config": {"workload": "VGG16 fp32 batch %d, one SGD step (fwd+bwd), policy %s, %s" % (args.batch, head, args.algo),
+        "dtype": "bf16 storage, f32 arithmetic" if args.bf16 else "f32", "data": "synthetic (seeded N(0,1) inputs, integer labels, He-normal filters)",
+        "config": {"workload": "VGG16 %s batch %d, one SGD step (fwd+bwd), policy %s, %s" % ("bf16-storage" if args.bf16 else "fp32", args.batch, head, args.algo),
                    "batch": args.batch, "policy": head, "algo": args.algo},
         "policies": results,
         "vdnn_all_vs_baseline_speed": (results[head]["images_per_s"] / base["images_per_s"]) if base else None,
@@ -162,7 +163,7 @@ def main():
         "conv_mfma_util": conv_all_tf / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom) if args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" else None,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom) if args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" and not args.bf16 else None,
                      "traffic_unit": "bytes per launch (L2 fetch + write-back, counters scaled by a known-size kernel)",
                      "algorithmic_flop_per_launch": d["flops"] / d["launches"],
                      "avg_launch_ms": d["ms"] / d["launches"], "launches": d["launches"]},

@@ -27,6 +27,7 @@ typedef struct {
     int      refined_lifetimes; /* value-preserving lifetime refinements of the vDNN policies (0 = literal schedule) */
     int      unfused_optimizer; /* keep dW / db per layer and step after backward instead of inside it (same bits) */
     int      defer_optimizer;   /* with unfused_optimizer: backward leaves the step to vdnn_network_apply_gradients */
+    int      data_type;         /* element type of activation tensors: VDNN_DTYPE_F32 (the reference, vdnn.h:11-12) or VDNN_DTYPE_BF16 */
 } vdnn_network_options;
 
 typedef struct {

@@ -90,6 +90,7 @@ _sig("orc_net_destroy", None, C.c_void_p)
 _sig("orc_net_num_layers", C.c_int, C.c_void_p)
 _sig("orc_net_layer_desc", None, C.c_void_p, C.c_int, C.POINTER(LayerDesc))
 _sig("orc_net_init_seeded", None, C.c_void_p, C.c_uint64)
+_sig("orc_net_set_bf16", None, C.c_void_p, C.c_int)
 _sig("orc_net_filter_count", C.c_size_t, C.c_void_p, C.c_int)
 _sig("orc_net_bias_count", C.c_size_t, C.c_void_p, C.c_int)
 for _n in ("orc_net_filter", "orc_net_bias", "orc_net_dst", "orc_net_grad"):
@@ -371,6 +372,9 @@ class Net:
         if not ptr or n == 0:
             return None
         return np.ctypeslib.as_array(ptr, shape=(n,)).reshape(shape)
+
+    def set_bf16(self, on=True):
+        lib.orc_net_set_bf16(self._h, int(on))
 
     def init_seeded(self, seed):
         lib.orc_net_init_seeded(self._h, seed)

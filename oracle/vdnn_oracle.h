@@ -125,6 +125,9 @@ int  orc_net_num_layers(const orc_net* net);
 void orc_net_layer_desc(const orc_net* net, int l, orc_layer_desc* out);
 /* He-normal filters (std sqrt(2/fan_in)), zero biases, N(0,1) input, integer labels */
 void orc_net_init_seeded(orc_net* net, uint64_t seed);
+/* bfloat16 activation storage: the input, every layer's output, the first difference and every
+ * layer's input gradient are rounded to bfloat16 once; parameters and their updates stay float */
+void orc_net_set_bf16(orc_net* net, int on);
 size_t orc_net_filter_count(const orc_net* net, int l);
 size_t orc_net_bias_count(const orc_net* net, int l);
 float* orc_net_filter(orc_net* net, int l);

@@ -21,6 +21,7 @@ struct orc_net {
     float* input;
     float* label;
     float* diff_last;
+    int bf16; /* activations are stored as bfloat16: every layer output and gradient is rounded once */
 };
 
 static size_t src_count(const orc_layer_desc* d) { return (size_t)d->g.n * d->g.c * d->g.h * d->g.w; }
@@ -197,7 +198,10 @@ void orc_net_init_seeded(orc_net* net, uint64_t seed) {
 
 /* forwardPropagation (network.cu:1056-1110): src[l] = dst[l-1] (:1080-1083), Layer::forward
  * dispatch (layer.cu:489-512) */
+void orc_net_set_bf16(orc_net* net, int on) { net->bf16 = on != 0; }
+
 float orc_net_forward(orc_net* net) {
+    if (net->bf16) orc_round_bf16(src_count(&net->L[0]), net->input, net->input);
     for (int l = 0; l < net->num_layers; l++) {
         const orc_layer_desc* d = &net->L[l];
         const float* src = l == 0 ? net->input : net->dst[l - 1];
@@ -213,8 +217,10 @@ float orc_net_forward(orc_net* net) {
         case T_SOFTMAX: orc_softmax_fwd(d->g.n, d->g.c * d->g.h * d->g.w, src, dst); break;
         default: break;
         }
+        if (net->bf16) orc_round_bf16(dst_count(d), dst, dst);
     }
     const orc_layer_desc* last = &net->L[net->num_layers - 1];
+    (void)last;
     return orc_cross_entropy_dense(last->n_out, last->c_out * last->h_out * last->w_out,
                                    net->dst[net->num_layers - 1], net->label);
 }
@@ -228,6 +234,7 @@ void orc_net_backward(orc_net* net) {
     const int L = net->num_layers;
     const orc_layer_desc* last = &net->L[L - 1];
     orc_sub(dst_count(last), net->dst[L - 1], net->label, net->diff_last);
+    if (net->bf16) orc_round_bf16(dst_count(last), net->diff_last, net->diff_last);
     for (int l = L - 1; l >= 0; l--) {
         const orc_layer_desc* d = &net->L[l];
         const float* src = l == 0 ? net->input : net->dst[l - 1];
@@ -253,5 +260,6 @@ void orc_net_backward(orc_net* net) {
         case T_SOFTMAX: orc_softmax_bwd(d->g.n, d->g.c * d->g.h * d->g.w, dst, diff, grad); break;
         default: break;
         }
+        if (net->bf16) orc_round_bf16(src_count(d), grad, grad);
     }
 }

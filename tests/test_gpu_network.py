@@ -15,7 +15,7 @@ import pytest
 import oracle
 from gpu_util import announce
 from test_oracle_net import load_small_net, small_net_layers
-from util import assert_close, golden, rel_err
+from util import assert_close, assert_close_bf16, golden, rel_err
 from vdnn_implementation_amd import (ALEXNET, ALEXNET_LRN, BASELINE, OVERFEAT, VDNN_ALL, VDNN_CONV, VDNN_MEMORY_OPT_ALGO,
                                      VDNN_NONE, VDNN_PERF_OPT_ALGO, VGG16_128, enums)
 from vdnn_implementation_amd.network import Network, layer_spec
@@ -83,13 +83,14 @@ def assert_bit_identical(a, b, what):
     assert np.array_equal(a["input"].view(np.uint32), b["input"].view(np.uint32)), what + ": input after the step"
 
 
-@pytest.mark.parametrize("cnn,batch,algo", [(None, 4, VDNN_MEMORY_OPT_ALGO), (ALEXNET_LRN, 4, VDNN_MEMORY_OPT_ALGO),
-                                            (OVERFEAT, 3, VDNN_MEMORY_OPT_ALGO), (VGG16_128, 2, VDNN_PERF_OPT_ALGO)])
-def test_policies_are_bit_identical_to_baseline(cnn, batch, algo):
+@pytest.mark.parametrize("cnn,batch,algo,bf16", [(None, 4, VDNN_MEMORY_OPT_ALGO, False), (ALEXNET_LRN, 4, VDNN_MEMORY_OPT_ALGO, False),
+                                                 (OVERFEAT, 3, VDNN_MEMORY_OPT_ALGO, False), (VGG16_128, 2, VDNN_PERF_OPT_ALGO, False),
+                                                 (None, 4, VDNN_MEMORY_OPT_ALGO, True), (VGG16_128, 2, VDNN_MEMORY_OPT_ALGO, True)])
+def test_policies_are_bit_identical_to_baseline(cnn, batch, algo, bf16):
     def make(policy, host_sync=False, refined=False):
         if cnn is None:
-            return Network(layers=small_specs(batch), policy=policy, algo=algo, capture=True, seed=3, host_sync=host_sync, refined=refined)
-        return Network(cnn, policy, algo, batch, capture=True, seed=3, host_sync=host_sync, refined=refined)
+            return Network(layers=small_specs(batch), policy=policy, algo=algo, capture=True, seed=3, host_sync=host_sync, refined=refined, bf16=bf16)
+        return Network(cnn, policy, algo, batch, capture=True, seed=3, host_sync=host_sync, refined=refined, bf16=bf16)
 
     announce("policies bit-identical", cnn, batch, "BASELINE")
     with make(BASELINE) as net:
@@ -169,6 +170,17 @@ def test_reference_networks_against_the_checker(cnn, batch, policy, algo):
     check_network_against_the_checker(cnn, batch, policy, algo)
 
 
+@pytest.mark.parametrize("cnn,batch,policy,algo", [
+    (ALEXNET_LRN, 2, VDNN_ALL, VDNN_MEMORY_OPT_ALGO),
+    (VGG16_128, 1, VDNN_ALL, VDNN_PERF_OPT_ALGO),
+    (OVERFEAT, 2, BASELINE, VDNN_MEMORY_OPT_ALGO),
+])
+def test_reference_networks_bf16_against_the_checker(cnn, batch, policy, algo):
+    """bfloat16 activation storage: every layer within one bfloat16 unit in the last place of the checker's
+    double-precision result on identical (bfloat16) inputs; ReLU and max-pool forward bit-exact."""
+    check_network_against_the_checker(cnn, batch, policy, algo, bf16=True)
+
+
 def smooth_specs(n=3):
     """A table with the two activation modes none of the reference's networks uses (layer.cu:362-369)."""
     return [layer_spec(enums.FC_CONV, n, 3, 16, 16, 1, 1, 8, 3), layer_spec(enums.TANH, n, 8, 16, 16),
@@ -183,7 +195,7 @@ def test_tanh_and_sigmoid_layers_against_the_checker(policy, refined):
     check_network_against_the_checker(None, 3, policy, VDNN_MEMORY_OPT_ALGO, layers=smooth_specs(3), refined=refined)
 
 
-def check_network_against_the_checker(cnn, batch, policy, algo, layers=None, refined=False):
+def check_network_against_the_checker(cnn, batch, policy, algo, layers=None, refined=False, bf16=False):
     """Layer by layer on identical inputs: each layer's output and gradients, computed by the checker
     from the tensors the GPU run fed that layer, within 1e-4 relative (max norm); exact for ReLU and
     max-pool. End to end (where a ReLU or pooling decision that flips on a last-bit difference moves
@@ -193,14 +205,15 @@ def check_network_against_the_checker(cnn, batch, policy, algo, layers=None, ref
         oracle.LayerDesc(s.type, oracle.Shape(s.n, s.c, s.h, s.w, s.k, s.r, s.s, s.pad_h, s.pad_w, s.stride_h, s.stride_w), 0, 0, 0, 0)
         for s in layers])
     o.init_seeded(seed)
+    o.set_bf16(bf16)
     oracle.set_accumulate_double(True)
     try:
         announce("network vs checker", cnn, batch, policy, algo)
-        with (Network(cnn, policy, algo, batch, capture=True, seed=seed) if layers is None else
-              Network(layers=layers, policy=policy, algo=algo, capture=True, seed=seed, refined=refined)) as net:
-            # the product's own seeded draw equals the checker's, bit for bit
+        with (Network(cnn, policy, algo, batch, capture=True, seed=seed, bf16=bf16) if layers is None else
+              Network(layers=layers, policy=policy, algo=algo, capture=True, seed=seed, refined=refined, bf16=bf16)) as net:
+            # the product's own seeded draw equals the checker's, bit for bit (rounded to bfloat16 at upload)
             x0 = net.get_input()
-            assert np.array_equal(x0.view(np.uint32), o.input().view(np.uint32))
+            assert np.array_equal(x0.view(np.uint32), (oracle.round_bf16(o.input()) if bf16 else o.input()).view(np.uint32))
             before = {}
             for l in range(net.num_layers):
                 if net.has_params(l):
@@ -209,7 +222,7 @@ def check_network_against_the_checker(cnn, batch, policy, algo, layers=None, ref
                     before[l] = (w, b)
             want_loss = o.forward()
             assert net.forwardPropagation() == 0
-            assert abs(net.loss() - want_loss) <= 1e-4 * abs(want_loss)
+            assert abs(net.loss() - want_loss) <= (3e-2 if bf16 else 1e-4) * abs(want_loss)
             o.backward()
             assert net.backwardPropagation() == 0
             L = net.num_layers
@@ -224,12 +237,18 @@ def check_network_against_the_checker(cnn, batch, policy, algo, layers=None, ref
                 exact = spec.type in (enums.RELU, enums.POOL)
                 if exact:
                     assert np.array_equal(dst[l], want), "output of layer %d" % l
+                elif bf16:
+                    assert_close_bf16(dst[l], want, "output of layer %d" % l)
                 else:
                     assert_close(dst[l], want, 1e-4, "output of layer %d" % l)
                 dy = (dst[-1] - target) if l == L - 1 else grad[l + 1].reshape(net.dst_shape(l))
+                if bf16 and l == L - 1:
+                    dy = oracle.round_bf16(dy)
                 want_dx, want_w, want_b = layer_backward_on_checker(spec, src, dst[l], dy, w, b)
-                if exact:
+                if exact and not (bf16 and spec.type == enums.POOL):
                     assert np.array_equal(grad[l], want_dx), "gradient of layer %d" % l
+                elif bf16:
+                    assert_close_bf16(grad[l], want_dx, "gradient of layer %d" % l)
                 else:
                     assert_close(grad[l], want_dx, 1e-4, "gradient of layer %d" % l)
                 if want_w is not None:
@@ -242,9 +261,11 @@ def check_network_against_the_checker(cnn, batch, policy, algo, layers=None, ref
                         l2 = np.linalg.norm(dw_got - dw_want) / np.linalg.norm(dw_want)
                         assert l2 <= 5e-2, "dW of layer %d: %.3e" % (l, l2)
             # end to end against the checker's own run
-            assert_close(dst[-1], o.dst(L - 1), 1e-4, "network output")
+            assert_close(dst[-1], o.dst(L - 1), 5e-2 if bf16 else 1e-4, "network output")
             g0, w0 = grad[0].astype(np.float64).ravel(), o.grad(0).astype(np.float64).ravel()
-            assert np.linalg.norm(g0 - w0) <= 2e-2 * np.linalg.norm(w0), "input gradient, end to end"
+            # bfloat16: one unit in the last place is 0.4-0.8 %, so ReLU / pooling decisions flip far more often
+            # through 37 layers; the end-to-end gradient is only required to point the same way
+            assert np.linalg.norm(g0 - w0) <= (0.5 if bf16 else 2e-2) * np.linalg.norm(w0), "input gradient, end to end"
             # offloaded then prefetched: the input block went to the host and back
             assert np.array_equal(net.get_input().view(np.uint32), x0.view(np.uint32))
             st = net.stats()

@@ -215,6 +215,41 @@ def test_refined_lifetimes_cut_peak_memory_threefold():
         assert net.stats()["peak_bytes_in_use"] == base
 
 
+def test_bf16_storage_halves_activations_and_offload_vgg16_512_under_48gb():
+    """VGG16 batch 512 with bfloat16 activations under a 48 GB limit on bytes in use. By the reference's
+    own allocation rule BASELINE needs 72.7 GB in float but 36.7 GB with 2-byte activations, so it
+    fits under 48 GB; a limit it cannot meet is shown with 24 GB, where VDNN_NONE's forward returns -1 in
+    dynamic mode and VDNN_ALL still fits. VDNN_ALL moves half the bytes of the float run."""
+    cap = 48 * GB
+    with plan(enums.VGG16_512, BASELINE, bf16=True, cap_bytes=cap, pool_bytes=120 * GB) as net:
+        assert net.batch == 512
+        assert net.forwardPropagation(True) == 0 and net.backwardPropagation(True) == 0
+        base = net.stats()["peak_bytes_in_use"]
+        assert abs(base / GB - 36.7) < 0.3
+    with plan(enums.VGG16_512, BASELINE, pool_bytes=120 * GB) as net:  # float activations: 72.7 GB, over the limit
+        step(net)
+        assert abs(net.stats()["peak_bytes_in_use"] / GB - 72.7) < 0.3
+    # BASELINE takes its buffers when it is built (network.cu:897-904), where a failed request is fatal as in
+    # the reference; the policy that allocates per layer shows the clean failure under the same 24 GB limit
+    with plan(enums.VGG16_512, VDNN_NONE, bf16=True, cap_bytes=24 * GB, pool_bytes=120 * GB) as net:
+        assert net.forwardPropagation(True) == -1
+    assert base > 24 * GB
+    with plan(enums.VGG16_512, VDNN_ALL, bf16=True, cap_bytes=cap, pool_bytes=120 * GB) as net:
+        assert net.forwardPropagation(True) == 0 and net.backwardPropagation(True) == 0
+        st = net.stats()
+        assert st["offload_bytes"] == st["prefetch_bytes"] == 14741667840 * 4 // 2  # batch x4, 2-byte elements
+        assert st["peak_bytes_in_use"] < 24 * GB
+        assert abs(st["weight_bytes"] / GB - 0.553) < 0.001  # float master parameters
+    with plan(enums.VGG16_512, VDNN_ALL, bf16=True, cap_bytes=24 * GB, pool_bytes=120 * GB) as net:
+        assert net.forwardPropagation(True) == 0 and net.backwardPropagation(True) == 0
+    with plan(VGG16_128, VDNN_ALL) as f32, plan(VGG16_128, VDNN_ALL, bf16=True) as b16:
+        step(f32)
+        step(b16)
+        acts32 = f32.stats()["peak_bytes_in_use"] - f32.stats()["weight_bytes"] - STAGING
+        acts16 = b16.stats()["peak_bytes_in_use"] - b16.stats()["weight_bytes"] - STAGING
+        assert abs(acts16 / acts32 - 0.5) < 0.01
+
+
 def test_unfused_optimizer_costs_one_more_copy_of_the_parameters():
     for policy in (BASELINE, VDNN_ALL):
         with plan(VGG16_128, policy) as net:

@@ -15,6 +15,7 @@ static NetworkOptions to_options(const vdnn_network_options* o) {
     n.planOnly = o->plan_only != 0; n.hostSync = o->host_sync != 0; n.capture = o->capture != 0;
     n.verbose = o->verbose != 0; n.device = o->device;
     n.refinedLifetimes = o->refined_lifetimes != 0;
+    n.dataType = o->data_type;
     n.unfusedOptimizer = o->unfused_optimizer != 0;
     n.deferOptimizer = o->defer_optimizer != 0;
     return n;
@@ -26,7 +27,7 @@ void vdnn_network_default_options(vdnn_network_options* o) {
     if (!o) return;
     NetworkOptions d;
     o->seed = d.seed; o->pool_bytes = 0; o->cap_bytes = 0; o->plan_only = 0; o->host_sync = 0;
-    o->capture = 0; o->verbose = 0; o->device = d.device; o->refined_lifetimes = 0; o->unfused_optimizer = 0; o->defer_optimizer = 0;
+    o->capture = 0; o->verbose = 0; o->device = d.device; o->refined_lifetimes = 0; o->unfused_optimizer = 0; o->defer_optimizer = 0; o->data_type = VDNN_DTYPE_F32;
 }
 
 vdnn_network* vdnn_network_create(int cnn, int policy, int algo, int batch, const vdnn_network_options* o) {

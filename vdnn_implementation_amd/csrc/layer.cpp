@@ -64,6 +64,7 @@ void Layer::construct(vdnn_ctx* _ctx) {
     refCntFwd = refCntBwd = 0;
     srcData = filterData = biasData = dstData = diffData = gradData = nullptr;
     filterGrad = biasGrad = nullptr;
+    actBytes = vdnn_ctx_activation_dtype(ctx) == VDNN_DTYPE_BF16 ? 2 : 4;
     fwdWorkSpaceSize = bwdDataWorkSpaceSize = bwdFilterWorkSpaceSize = 0;
     srcReadyEvent = offloadDoneEvent = nullptr;
     prefetchBlockFreeEvent = prefetchHostReadyEvent = prefetchDoneEvent = nullptr;
@@ -446,7 +447,7 @@ void Layer::initializeFullyConnectedFilterAndBias() {
  * the driver waits on before the block is recycled. */
 void Layer::offloadSrcData(bool*, DATATYPE** _offloadedSrcData_h) {
     if (srcReadyEvent) checkVDNN(vdnn_stream_wait_event(ctx, *stream_memory, srcReadyEvent));
-    checkVDNN(vdnn_memcpy_d2h_async(ctx, _offloadedSrcData_h[layerId], srcData, SrcDataSize() * sizeof(DATATYPE), *stream_memory));
+    checkVDNN(vdnn_memcpy_d2h_async(ctx, _offloadedSrcData_h[layerId], srcData, SrcDataSize() * actBytes, *stream_memory));
     if (offloadDoneEvent) checkVDNN(vdnn_event_record(ctx, offloadDoneEvent, *stream_memory));
 }
 
@@ -466,28 +467,34 @@ void Layer::prefetchPreviousSrcData(DATATYPE* _prefetchedSrcData_h, void* _srcDa
 
 /* layer.cu:989-1011 */
 int Layer::cnmemMallocSrcData(bool isDynamic) {
-    if (ASSERT_EQ(vdnn_pool_malloc(ctx, &srcData, sizeof(DATATYPE) * SrcDataSize()), isDynamic) < 0) return -1;
+    if (ASSERT_EQ(vdnn_pool_malloc(ctx, &srcData, actBytes * SrcDataSize()), isDynamic) < 0) return -1;
     return 0;
 }
 int Layer::cnmemMallocDstData(bool isDynamic) {
-    if (ASSERT_EQ(vdnn_pool_malloc(ctx, &dstData, sizeof(DATATYPE) * DstDataSize()), isDynamic) < 0) return -1;
+    if (ASSERT_EQ(vdnn_pool_malloc(ctx, &dstData, actBytes * DstDataSize()), isDynamic) < 0) return -1;
     return 0;
 }
 /* the reference sizes diffData by SrcDataSize (layer.cu:1001-1005); it is only called for the last
  * layer, a softmax, where input and output extents agree */
 int Layer::cnmemMallocDiffData(bool isDynamic) {
-    if (ASSERT_EQ(vdnn_pool_malloc(ctx, &diffData, sizeof(DATATYPE) * (SrcDataSize() > DstDataSize() ? SrcDataSize() : DstDataSize())), isDynamic) < 0) return -1;
+    if (ASSERT_EQ(vdnn_pool_malloc(ctx, &diffData, actBytes * (SrcDataSize() > DstDataSize() ? SrcDataSize() : DstDataSize())), isDynamic) < 0) return -1;
     return 0;
 }
 int Layer::cnmemMallocGradData(bool isDynamic) {
-    if (ASSERT_EQ(vdnn_pool_malloc(ctx, &gradData, sizeof(DATATYPE) * SrcDataSize()), isDynamic) < 0) return -1;
+    if (ASSERT_EQ(vdnn_pool_malloc(ctx, &gradData, actBytes * SrcDataSize()), isDynamic) < 0) return -1;
     return 0;
 }
 
 /* layer.cu:1149-1185 (debug dumps; the reference indexes rows with h*h_out+w, here h*w_out+w) */
 void Layer::printDstData() {
     std::vector<DATATYPE> h(DstDataSize());
-    checkVDNN(vdnn_memcpy_d2h(ctx, h.data(), dstData, h.size() * sizeof(DATATYPE)));
+    if (actBytes == 2) {
+        std::vector<uint16_t> raw(h.size());
+        checkVDNN(vdnn_memcpy_d2h(ctx, raw.data(), dstData, raw.size() * sizeof(uint16_t)));
+        for (size_t i = 0; i < h.size(); i++) h[i] = vdnn::bf16_to_float_host(raw[i]);
+    } else {
+        checkVDNN(vdnn_memcpy_d2h(ctx, h.data(), dstData, h.size() * sizeof(DATATYPE)));
+    }
     printf("Layer %d dstData:\n", layerId);
     for (int n = 0; n < n_out; n++) for (int c = 0; c < c_out; c++) {
         for (int y = 0; y < h_out; y++) {

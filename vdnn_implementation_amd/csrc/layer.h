@@ -254,6 +254,7 @@ private:
     void* srcData;    // x
     void* filterData; // w
     void* biasData;   // bias
+    size_t actBytes;  // bytes per activation element (the context's activation dtype)
     void* filterGrad; // dW (only with keepGradients)
     void* biasGrad;   // db
     void* dstData;    // y

@@ -136,6 +136,7 @@ void Network::construct(vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) {
     /* context = handles + streams (network.cu:39-42) */
     ctx = nullptr;
     checkVDNN(vdnn_ctx_create(&ctx, options.device, options.planOnly ? VDNN_CTX_PLAN_ONLY : 0));
+    checkVDNN(vdnn_ctx_set_activation_dtype(ctx, options.dataType));
     convHandle.ctx = ctx;
     gemmHandle.ctx = ctx;
     stream_compute = vdnn_ctx_stream_compute(ctx);
@@ -214,15 +215,15 @@ void Network::reset(CNN_t _cnnType, vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) 
 void Network::initPool() {
     size_t bytes = options.poolBytes;
     if (bytes == 0) {
-        size_t sum = 0, maxAct = 0;
+        size_t sum = 0, maxAct = 0, params = 0;
         for (const LayerSpec& s : specs) {
             const size_t src = spec_src_count(s), dst = spec_dst_count(s);
             sum += dst;
             maxAct = std::max(maxAct, std::max(src, dst));
-            if (s.type == FC_GEMM || is_conv(s.type)) sum += ((size_t)s.k * s.c * s.r * s.s + s.k) * (options.unfusedOptimizer ? 2 : 1);
+            if (s.type == FC_GEMM || is_conv(s.type)) params += ((size_t)s.k * s.c * s.r * s.s + s.k) * (options.unfusedOptimizer ? 2 : 1);
         }
         sum += spec_src_count(specs[0]) * 2 + spec_dst_count(specs.back()) * 2 + 3 * maxAct;
-        bytes = sum * sizeof(DATATYPE);
+        bytes = sum * actBytes() + params * sizeof(float);
         bytes += bytes / 8 + (size_t(384) << 20); // rounding of ~100 blocks, staging area, headroom
         size_t freeB = 0, totalB = 0;
         checkVDNN(vdnn_device_mem_info(ctx, &freeB, &totalB));
@@ -304,7 +305,7 @@ void Network::buildLayers() {
 void Network::randomInitializeData(void* data, size_t size) {
     std::vector<DATATYPE> data_h(size);
     vdnn::seeded_fill_normal(data_h.data(), size, options.seed, 1, 0.0f, 1.0f);
-    checkVDNN(vdnn_memcpy_h2d(ctx, data, data_h.data(), sizeof(DATATYPE) * size));
+    uploadActivations(data, data_h.data(), size);
 }
 
 /* network.cu:831-873 */
@@ -363,7 +364,7 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
     auto offload = [&](int l) {
         if (dropSrcAfterFwd[l]) return; /* released, not moved: nothing reads it again */
         isOffload[l] = true;
-        const size_t bytes = layer[l]->SrcDataSize() * sizeof(DATATYPE);
+        const size_t bytes = layer[l]->SrcDataSize() * actBytes();
         checkVDNN(vdnn_host_alloc_pinned(ctx, (void**)&offloadedSrcData_h[l], bytes));
         lastStats.pinnedBytes += bytes;
     };
@@ -404,13 +405,13 @@ void Network::setAlgoType(vdnnAlgoMode_t newAlgoMode) {
 
 /* network.cu:87-90: input and label tensors; plus the loss scalar and the seeded contents */
 void Network::allocIoBuffers() {
-    ASSERT_EQ(vdnn_pool_malloc(ctx, &inputData, sizeof(DATATYPE) * getInputSize()));
-    ASSERT_EQ(vdnn_pool_malloc(ctx, &labelData, sizeof(DATATYPE) * getOutputSize()));
+    ASSERT_EQ(vdnn_pool_malloc(ctx, &inputData, actBytes() * getInputSize()));
+    ASSERT_EQ(vdnn_pool_malloc(ctx, &labelData, actBytes() * getOutputSize()));
     ASSERT_EQ(vdnn_pool_malloc(ctx, (void**)&lossData, sizeof(DATATYPE)));
     if (!options.planOnly) {
         inputHost.resize(getInputSize());
         vdnn::seeded_fill_normal(inputHost.data(), inputHost.size(), options.seed, 1, 0.0f, 1.0f);
-        checkVDNN(vdnn_memcpy_h2d(ctx, inputData, inputHost.data(), sizeof(DATATYPE) * inputHost.size()));
+        uploadActivations(inputData, inputHost.data(), inputHost.size());
         const int classes = c_out * h_out * w_out;
         std::vector<int32_t> lab((size_t)n_out);
         vdnn::seeded_fill_labels(lab.data(), lab.size(), options.seed, 2, classes);
@@ -453,7 +454,7 @@ size_t Network::findMaxDxDySize() {
     size_t ret = 0;
     for (int i = 0; i < numLayers; i++) ret = std::max(ret, layer[i]->SrcDataSize());
     ret = std::max(ret, layer[numLayers - 1]->DstDataSize());
-    return ret * sizeof(DATATYPE);
+    return ret * actBytes();
 }
 
 /* network.cu:1025-1040 */
@@ -487,7 +488,7 @@ void Network::captureLayer(int l, bool grad) {
     std::vector<float>& dstv = grad ? capGrad[l] : capDst[l];
     const size_t count = grad ? layer[l]->SrcDataSize() : layer[l]->DstDataSize();
     dstv.resize(count);
-    checkVDNN(vdnn_memcpy_d2h(ctx, dstv.data(), grad ? layer[l]->GradData() : layer[l]->DstData(), count * sizeof(float)));
+    downloadActivations(dstv.data(), grad ? layer[l]->GradData() : layer[l]->DstData(), count);
 }
 
 /* network.cu:1090-1091, 1168-1169 */
@@ -532,7 +533,7 @@ int Network::forwardPropagation(bool isDynamic) {
             /* Release srcData of this layer. The reference keeps layer 0's block and later allocates
                a second one for its prefetch; releasing it here avoids that leak. */
             if (isOffload[l]) {
-                lastStats.offloadBytes += layer[l]->SrcDataSize() * sizeof(DATATYPE);
+                lastStats.offloadBytes += layer[l]->SrcDataSize() * actBytes();
                 ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->SrcData()), isDynamic);
                 if (l == 0) { inputData = nullptr; inputResident = false; }
             } else if (dropSrcAfterFwd[l]) {
@@ -596,7 +597,7 @@ int Network::backwardPropagation(bool isDynamic) {
             if (prefId >= 0) {
                 if (layer[prefId]->cnmemMallocSrcData(isDynamic) < 0) return -1;
                 layer[l]->setPrefetchEvents(evBlockFree[prefId], evOffloadDone[prefId], evPrefetchDone[prefId]);
-                const size_t bytes = sizeof(DATATYPE) * layer[prefId]->SrcDataSize();
+                const size_t bytes = actBytes() * layer[prefId]->SrcDataSize();
                 if (layer[l]->backward(prefId, offloadedSrcData_h[prefId], layer[prefId]->SrcData(), bytes, workSpace, isDynamic) < 0) return -1;
                 lastStats.prefetchBytes += bytes;
                 prefetchLog.emplace_back(l, prefId);
@@ -670,16 +671,37 @@ int Network::findPrefetchLayer(int currLayerId) {
 }
 
 /* ---- additions ------------------------------------------------------------------------------ */
+/* Host tensors are float; a bfloat16 network converts at the boundary (round to nearest even). */
+void Network::uploadActivations(void* dev, const float* host, size_t count) {
+    if (options.dataType == VDNN_DTYPE_BF16) {
+        std::vector<uint16_t> h(count);
+        for (size_t i = 0; i < count; i++) h[i] = vdnn::float_to_bf16_host(host[i]);
+        checkVDNN(vdnn_memcpy_h2d(ctx, dev, h.data(), count * sizeof(uint16_t)));
+    } else {
+        checkVDNN(vdnn_memcpy_h2d(ctx, dev, host, count * sizeof(float)));
+    }
+}
+
+void Network::downloadActivations(float* host, const void* dev, size_t count) {
+    if (options.dataType == VDNN_DTYPE_BF16) {
+        std::vector<uint16_t> h(count);
+        checkVDNN(vdnn_memcpy_d2h(ctx, h.data(), dev, count * sizeof(uint16_t)));
+        for (size_t i = 0; i < count; i++) host[i] = vdnn::bf16_to_float_host(h[i]);
+    } else {
+        checkVDNN(vdnn_memcpy_d2h(ctx, host, dev, count * sizeof(float)));
+    }
+}
+
 void Network::setInput(const float* host) {
     M_ASSERT(inputResident && inputData, "input block is not resident");
     if (options.planOnly) return;
     inputHost.assign(host, host + getInputSize());
-    checkVDNN(vdnn_memcpy_h2d(ctx, inputData, host, sizeof(DATATYPE) * getInputSize()));
+    uploadActivations(inputData, host, getInputSize());
 }
 
 void Network::getInput(float* host) {
     M_ASSERT(inputResident && inputData, "input block is not resident");
-    checkVDNN(vdnn_memcpy_d2h(ctx, host, inputData, sizeof(DATATYPE) * getInputSize()));
+    downloadActivations(host, inputData, getInputSize());
 }
 
 void Network::setLabels(const int32_t* labels) {
@@ -694,7 +716,7 @@ void Network::setLabels(const int32_t* labels) {
 
 void Network::setLabelTensor(const float* host) {
     if (options.planOnly) return;
-    checkVDNN(vdnn_memcpy_h2d(ctx, labelData, host, sizeof(DATATYPE) * getOutputSize()));
+    uploadActivations(labelData, host, getOutputSize());
 }
 
 int Network::setLayerParams(int l, const float* filter, const float* bias) {

@@ -30,6 +30,11 @@ struct NetworkOptions {
     // backward layer (applyGradients) instead of inside the backward kernels as the reference does
     // (layer.cu:651-660, 736-761). Same bits as the fused step; what a data-parallel exchange or
     // another optimizer needs. deferOptimizer leaves the step to the caller.
+    // Element type of activation tensors (layer inputs, outputs, their gradients, the network input and
+    // target): VDNN_DTYPE_F32 as in the reference (vdnn.h:11-12) or VDNN_DTYPE_BF16, which halves device
+    // memory and offload traffic. Parameters and their gradients stay float (the master copy is what the
+    // kernels read), arithmetic and accumulation are float, results are rounded once when stored.
+    int      dataType = VDNN_DTYPE_F32;
     bool     unfusedOptimizer = false;
     bool     deferOptimizer = false;
     int      device = DEFAULT_DEVICE;
@@ -145,6 +150,9 @@ private:
     void            releasePolicyBuffers();
     void            allocIoBuffers();
     void            captureLayer(int l, bool grad);
+    size_t          actBytes() const { return options.dataType == VDNN_DTYPE_BF16 ? 2 : 4; }
+    void            uploadActivations(void* dev, const float* host, size_t count);
+    void            downloadActivations(float* host, const void* dev, size_t count);
     void            afterLayerSync();
     void            printUsage(const char* tag, int l, size_t workspace);
 

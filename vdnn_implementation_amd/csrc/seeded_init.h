@@ -7,6 +7,7 @@
 #include <cmath>
 #include <cstddef>
 #include <cstdint>
+#include <cstring>
 #include <thread>
 #include <vector>
 
@@ -60,6 +61,23 @@ inline void seeded_fill_uniform(float* p, size_t count, uint64_t seed, uint64_t 
 inline void seeded_fill_labels(int32_t* p, size_t count, uint64_t seed, uint64_t stream, int classes) {
     for (size_t i = 0; i < count; i++)
         p[i] = (int32_t)(((seeded_u64(seed, stream, i) >> 32) * (uint64_t)classes) >> 32);
+}
+
+
+// bfloat16 <-> float on the host (round to nearest, ties to even; NaN stays NaN): the conversion
+// the kernels apply when they store an activation
+inline uint16_t float_to_bf16_host(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+inline float bf16_to_float_host(uint16_t b) {
+    const uint32_t u = (uint32_t)b << 16;
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
 }
 
 } // namespace vdnn

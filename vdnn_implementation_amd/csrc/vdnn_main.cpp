@@ -56,6 +56,7 @@ int main(int argc, char** argv) {
         else if (!strcmp(argv[i], "--plan")) opt.planOnly = true;
         else if (!strcmp(argv[i], "--refined")) opt.refinedLifetimes = true;
         else if (!strcmp(argv[i], "--unfused")) opt.unfusedOptimizer = true;
+        else if (!strcmp(argv[i], "--bf16")) opt.dataType = VDNN_DTYPE_BF16;
         else if (!strcmp(argv[i], "--verbose")) opt.verbose = true;
         else M_ASSERT(0, "unknown flag");
     }
