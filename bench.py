@@ -39,8 +39,9 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0, bf16=False):
-    net = Network(cnn, policy, algo, batch, seed=seed, refined=refined, cap_bytes=cap_bytes, bf16=bf16)
+def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0, bf16=False, offload_lag=0, prefetch_depth=1):
+    net = Network(cnn, policy, algo, batch, seed=seed, refined=refined, cap_bytes=cap_bytes, bf16=bf16,
+                  offload_lag=offload_lag, prefetch_depth=prefetch_depth)
     try:
         for _ in range(warmup):
             assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
@@ -102,6 +103,8 @@ def main():
     ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined")
     ap.add_argument("--cap-gb", type=float, default=0.0, help="artificial limit on pool bytes in use (0 = none)")
     ap.add_argument("--bf16", action="store_true", help="bfloat16 activation storage (float parameters and arithmetic)")
+    ap.add_argument("--offload-lag", type=int, default=0, help="layers enqueued before an offloaded block is recycled (0 = reference schedule)")
+    ap.add_argument("--prefetch-depth", type=int, default=1, help="offloaded tensors fetched ahead in backward (1 = reference schedule)")
     ap.add_argument("--cpu-batch", type=int, default=24)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -121,7 +124,8 @@ def main():
         _, policy, algo = parse("VGG16_128", word, args.algo)
         log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
         results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1,
-                                                   refined=(suffix == "refined"), cap_bytes=int(args.cap_gb * 1e9), bf16=args.bf16)
+                                                   refined=(suffix == "refined"), cap_bytes=int(args.cap_gb * 1e9), bf16=args.bf16,
+                                                   offload_lag=args.offload_lag, prefetch_depth=args.prefetch_depth)
         log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
             results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))
 

@@ -27,6 +27,8 @@ typedef struct {
     int      refined_lifetimes; /* value-preserving lifetime refinements of the vDNN policies (0 = literal schedule) */
     int      unfused_optimizer; /* keep dW / db per layer and step after backward instead of inside it (same bits) */
     int      defer_optimizer;   /* with unfused_optimizer: backward leaves the step to vdnn_network_apply_gradients */
+    int      offload_lag;       /* layers enqueued before an offloaded block is recycled (0 = the reference's schedule) */
+    int      prefetch_depth;    /* offloaded tensors fetched ahead of their backward (1 = the reference's schedule) */
     int      data_type;         /* element type of activation tensors: VDNN_DTYPE_F32 (the reference, vdnn.h:11-12) or VDNN_DTYPE_BF16 */
 } vdnn_network_options;
 

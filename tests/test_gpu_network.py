@@ -87,10 +87,10 @@ def assert_bit_identical(a, b, what):
                                                  (OVERFEAT, 3, VDNN_MEMORY_OPT_ALGO, False), (VGG16_128, 2, VDNN_PERF_OPT_ALGO, False),
                                                  (None, 4, VDNN_MEMORY_OPT_ALGO, True), (VGG16_128, 2, VDNN_MEMORY_OPT_ALGO, True)])
 def test_policies_are_bit_identical_to_baseline(cnn, batch, algo, bf16):
-    def make(policy, host_sync=False, refined=False):
+    def make(policy, host_sync=False, refined=False, **kw):
         if cnn is None:
-            return Network(layers=small_specs(batch), policy=policy, algo=algo, capture=True, seed=3, host_sync=host_sync, refined=refined, bf16=bf16)
-        return Network(cnn, policy, algo, batch, capture=True, seed=3, host_sync=host_sync, refined=refined, bf16=bf16)
+            return Network(layers=small_specs(batch), policy=policy, algo=algo, capture=True, seed=3, host_sync=host_sync, refined=refined, bf16=bf16, **kw)
+        return Network(cnn, policy, algo, batch, capture=True, seed=3, host_sync=host_sync, refined=refined, bf16=bf16, **kw)
 
     announce("policies bit-identical", cnn, batch, "BASELINE")
     with make(BASELINE) as net:
@@ -109,6 +109,13 @@ def test_policies_are_bit_identical_to_baseline(cnn, batch, algo, bf16):
         with make(policy, refined=True) as net:
             got = run_steps(net, 2)
         assert_bit_identical(got, base, "policy %d refined" % policy)
+        # scheduling slack (blocks recycled some layers after their offload, several tensors fetched ahead)
+        # changes when things are copied, never what is computed
+        for refined, lag, depth in ((False, 3, 2), (True, 6, 3), (False, 40, 1)):
+            announce("policies bit-identical", cnn, batch, "policy", policy, "lag", lag, "depth", depth, "refined", refined)
+            with make(policy, refined=refined, offload_lag=lag, prefetch_depth=depth) as net:
+                got = run_steps(net, 2)
+            assert_bit_identical(got, base, "policy %d lag %d depth %d" % (policy, lag, depth))
 
 
 def layer_forward_on_checker(spec, src, w, b):

@@ -250,6 +250,32 @@ def test_bf16_storage_halves_activations_and_offload_vgg16_512_under_48gb():
         assert abs(acts16 / acts32 - 0.5) < 0.01
 
 
+def test_scheduling_slack_moves_the_same_bytes_and_leaks_nothing():
+    """offloadLag / prefetchDepth change lifetimes only: same offload set, every block returned, and the
+    extra memory is bounded and reproducible (VGG16 batch 128, refined VDNN_CONV: 5.96 GB up to a lag of four
+    layers, 6.79 GB at six, 8.46 GB when nothing is recycled before the end of forward)."""
+    with plan(VGG16_128, VDNN_CONV, refined=True) as net:
+        step(net)
+        ref = net.stats()
+    for lag, depth, peak_gb in ((4, 1, 5.96), (6, 2, 6.79), (40, 3, 8.46)):
+        with plan(VGG16_128, VDNN_CONV, refined=True, offload_lag=lag, prefetch_depth=depth) as net:
+            n0 = C.c_size_t()
+            lib.vdnn_pool_live_blocks(net.context, C.byref(n0))
+            step(net)
+            step(net)
+            st = net.stats()
+            n1 = C.c_size_t()
+            lib.vdnn_pool_live_blocks(net.context, C.byref(n1))
+            assert n1.value == n0.value
+            assert st["offload_bytes"] == st["prefetch_bytes"] == ref["offload_bytes"]
+            assert abs(st["peak_bytes_in_use"] / GB - peak_gb) < 0.02
+            fetched = [p for _, p in net.prefetch_trace()]
+            assert sorted(fetched, reverse=True) == fetched and len(set(fetched)) == len(fetched)  # top down, once each
+    with plan(VGG16_128, VDNN_ALL, offload_lag=2, prefetch_depth=4) as net:
+        step(net)
+        assert [p for _, p in net.prefetch_trace()] == list(range(35, -1, -1))
+
+
 def test_unfused_optimizer_costs_one_more_copy_of_the_parameters():
     for policy in (BASELINE, VDNN_ALL):
         with plan(VGG16_128, policy) as net:

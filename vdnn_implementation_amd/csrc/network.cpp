@@ -502,6 +502,7 @@ void Network::afterLayerSync() {
 int Network::forwardPropagation(bool isDynamic) {
     M_ASSERT(inputResident && inputData, "forwardPropagation needs the input on the device (run backwardPropagation after a forward)");
     lastStats.offloadBytes = 0;
+    pendingOffload.clear();
     if (vdnnType == BASELINE) {
         for (int l = 0; l < numLayers; l++) {
             layer[l]->copySrcData(l == 0 ? inputData : layer[l - 1]->DstData());
@@ -528,18 +529,25 @@ int Network::forwardPropagation(bool isDynamic) {
                the block may be recycled once this layer's kernels (stream order) and its offload
                copy (event) are done with it. */
             if (options.hostSync) afterLayerSync();
-            else if (isOffload[l]) checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evOffloadDone[l]));
 
             /* Release srcData of this layer. The reference keeps layer 0's block and later allocates
-               a second one for its prefetch; releasing it here avoids that leak. */
+               a second one for its prefetch; releasing it here avoids that leak. With offloadLag the
+               wait for the copy and the release move behind the next `offloadLag` layers. */
             if (isOffload[l]) {
                 lastStats.offloadBytes += layer[l]->SrcDataSize() * actBytes();
-                ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->SrcData()), isDynamic);
-                if (l == 0) { inputData = nullptr; inputResident = false; }
+                pendingOffload.push_back(l);
             } else if (dropSrcAfterFwd[l]) {
                 /* refined lifetimes: every reader (this layer's forward) is already enqueued */
                 ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->SrcData()), isDynamic);
                 layer[l]->copySrcData(nullptr);
+            }
+            const int lag = options.hostSync ? 0 : options.offloadLag;
+            while (!pendingOffload.empty() && (pendingOffload.front() + lag <= l || l == numLayers - 1)) {
+                const int j = pendingOffload.front();
+                pendingOffload.erase(pendingOffload.begin());
+                if (!options.hostSync) checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evOffloadDone[j]));
+                ASSERT_EQ(vdnn_pool_free(ctx, layer[j]->SrcData()), isDynamic);
+                if (j == 0) { inputData = nullptr; inputResident = false; }
             }
             printUsage("Fwd", l, layer[l]->FwdWorkSpaceSize());
         }
@@ -593,7 +601,7 @@ int Network::backwardPropagation(bool isDynamic) {
             /* this layer reads its own srcData: if that was prefetched, the copy must have landed */
             if (!options.hostSync && isPrefetched[l]) checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evPrefetchDone[l]));
 
-            int prefId = l == 0 ? -1 : findPrefetchLayer(l);
+            int prefId = l == 0 ? -1 : (options.prefetchDepth > 1 ? findPrefetchLayerDeep(l) : findPrefetchLayer(l));
             if (prefId >= 0) {
                 if (layer[prefId]->cnmemMallocSrcData(isDynamic) < 0) return -1;
                 layer[l]->setPrefetchEvents(evBlockFree[prefId], evOffloadDone[prefId], evPrefetchDone[prefId]);
@@ -604,6 +612,18 @@ int Network::backwardPropagation(bool isDynamic) {
                 if (prefId == 0) { inputData = layer[0]->SrcData(); inputResident = true; }
             } else {
                 if (layer[l]->backward(-1, NULL, NULL, 0, workSpace, isDynamic) < 0) return -1;
+            }
+            /* deeper prefetch: further tensors below, enqueued behind this layer's kernels */
+            while (options.prefetchDepth > 1 && l > 0) {
+                const int extra = findPrefetchLayerDeep(l);
+                if (extra < 0) break;
+                if (layer[extra]->cnmemMallocSrcData(isDynamic) < 0) return -1;
+                layer[l]->setPrefetchEvents(evBlockFree[extra], evOffloadDone[extra], evPrefetchDone[extra]);
+                const size_t bytes = actBytes() * layer[extra]->SrcDataSize();
+                layer[l]->prefetchPreviousSrcData(offloadedSrcData_h[extra], layer[extra]->SrcData(), bytes);
+                lastStats.prefetchBytes += bytes;
+                prefetchLog.emplace_back(l, extra);
+                if (extra == 0) { inputData = layer[0]->SrcData(); inputResident = true; }
             }
             captureLayer(l, true);
 
@@ -654,6 +674,22 @@ std::vector<float> Network::train(int steps, bool isDynamic) {
 /* network.cu:1193-1196 */
 void Network::resetIsPrefetchedArray() {
     for (int i = 0; i < DEFAULT_NUM_LAYER; i++) isPrefetched[i] = false;
+}
+
+/* addition (prefetchDepth > 1): the nearest offloaded, not yet fetched layer below currLayerId, as long
+ * as fewer than prefetchDepth fetched tensors below currLayerId are still waiting for their backward */
+int Network::findPrefetchLayerDeep(int currLayerId) {
+    int outstanding = 0;
+    for (int id = currLayerId - 1; id >= 0; id--)
+        if (isOffload[id] && isPrefetched[id]) outstanding++;
+    if (outstanding >= options.prefetchDepth) return -1;
+    for (int id = currLayerId - 1; id >= 0; id--) {
+        if (isOffload[id] && !isPrefetched[id]) {
+            isPrefetched[id] = true;
+            return id;
+        }
+    }
+    return -1;
 }
 
 /* network.cu:1198-1208: scan downward from currLayerId-1; the first layer that is offloaded and not

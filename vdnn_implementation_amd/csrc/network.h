@@ -35,6 +35,14 @@ struct NetworkOptions {
     // memory and offload traffic. Parameters and their gradients stay float (the master copy is what the
     // kernels read), arithmetic and accumulation are float, results are rounded once when stored.
     int      dataType = VDNN_DTYPE_F32;
+    // Scheduling slack of the offloading policies (0 / 1 = the reference's schedule; values unchanged, only
+    // lifetimes). offloadLag: the block of an offloaded srcData is recycled - and the compute stream made to
+    // wait for its device-to-host copy - only after `offloadLag` further layers have been enqueued, so a
+    // copy that is longer than its own layer's kernels overlaps the following layers instead of stalling
+    // them. prefetchDepth: up to that many offloaded tensors below the current layer are in flight or
+    // resident ahead of their backward (the reference fetches one, network.cu:1193-1208).
+    int      offloadLag = 0;
+    int      prefetchDepth = 1;
     bool     unfusedOptimizer = false;
     bool     deferOptimizer = false;
     int      device = DEFAULT_DEVICE;
@@ -103,6 +111,7 @@ public:
     /* Find prefetch layer */
     void            resetIsPrefetchedArray();
     int             findPrefetchLayer(int currLayerId);
+    int             findPrefetchLayerDeep(int currLayerId); /* addition: see NetworkOptions::prefetchDepth */
 
     /* Get functions */
     Layer**         layerArray()            { return layer;              }
@@ -195,6 +204,7 @@ private:
     vdnn_event_t        evOffloadDone[DEFAULT_NUM_LAYER]; // d2h: srcData of layer l is in pinned memory
     vdnn_event_t        evBlockFree[DEFAULT_NUM_LAYER];   // compute: everything enqueued before the prefetch of l
     vdnn_event_t        evPrefetchDone[DEFAULT_NUM_LAYER];// h2d: srcData of layer l is back on the device
+    std::vector<int>    pendingOffload;                    // offloaded layers whose block is not yet recycled (offloadLag)
     bool                inputResident;                     // inputData currently holds the input (addition)
 
     NetworkStats        lastStats;

@@ -57,6 +57,8 @@ int main(int argc, char** argv) {
         else if (!strcmp(argv[i], "--refined")) opt.refinedLifetimes = true;
         else if (!strcmp(argv[i], "--unfused")) opt.unfusedOptimizer = true;
         else if (!strcmp(argv[i], "--bf16")) opt.dataType = VDNN_DTYPE_BF16;
+        else if (!strcmp(argv[i], "--offload-lag")) opt.offloadLag = atoi(need("--offload-lag needs a value"));
+        else if (!strcmp(argv[i], "--prefetch-depth")) opt.prefetchDepth = atoi(need("--prefetch-depth needs a value"));
         else if (!strcmp(argv[i], "--verbose")) opt.verbose = true;
         else M_ASSERT(0, "unknown flag");
     }
