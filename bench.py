@@ -77,6 +77,19 @@ def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refin
     return res, prof
 
 
+def best_offloading(results, base):
+    """The offloading run that is fastest among those holding at least 3x less device memory than the fp32 BASELINE."""
+    if not base:
+        return None
+    ok = {k: v for k, v in results.items() if v["offload_gb_per_step"] > 0 and base["peak_hbm_gb"] / v["peak_hbm_gb"] >= 3.0}
+    if not ok:
+        return None
+    k = max(ok, key=lambda n: ok[n]["images_per_s"])
+    return {"policy": k, "speed_vs_baseline": ok[k]["images_per_s"] / base["images_per_s"],
+            "peak_hbm_reduction": base["peak_hbm_gb"] / ok[k]["peak_hbm_gb"], "images_per_s": ok[k]["images_per_s"],
+            "peak_hbm_gb": ok[k]["peak_hbm_gb"]}
+
+
 def cpu_baseline(batch):
     """The checker's training step on the host cores, VGG16 at a reduced batch."""
     import oracle
@@ -100,7 +113,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--algo", default="VDNN_MEMORY_OPT_ALGO")
-    ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined")
+    ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined,VDNN_CONV+refined+slack,"
+                    "BASELINE+bf16,VDNN_ALL+bf16,VDNN_CONV+refined+slack+bf16,VDNN_ALL+refined+slack+bf16")
     ap.add_argument("--cap-gb", type=float, default=0.0, help="artificial limit on pool bytes in use (0 = none)")
     ap.add_argument("--bf16", action="store_true", help="bfloat16 activation storage (float parameters and arithmetic)")
     ap.add_argument("--offload-lag", type=int, default=0, help="layers enqueued before an offloaded block is recycled (0 = reference schedule)")
@@ -119,13 +133,16 @@ def main():
     cnn = enums.VGG16_128
     results, profiles = {}, {}
     for name in args.policies.split(","):
-        # "+refined": the same policy with the value-preserving lifetime refinements switched on
-        word, _, suffix = name.partition("+")
+        # suffixes: "+refined" = the value-preserving lifetime refinements; "+slack" = blocks recycled six layers
+        # after their offload and two tensors fetched ahead; "+bf16" = bfloat16 activation storage
+        word, *mods = name.split("+")
+        assert set(mods) <= {"refined", "slack", "bf16"}, name
         _, policy, algo = parse("VGG16_128", word, args.algo)
+        lag, depth = (6, 2) if "slack" in mods else (args.offload_lag, args.prefetch_depth)
         log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
         results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1,
-                                                   refined=(suffix == "refined"), cap_bytes=int(args.cap_gb * 1e9), bf16=args.bf16,
-                                                   offload_lag=args.offload_lag, prefetch_depth=args.prefetch_depth)
+                                                   refined=("refined" in mods), cap_bytes=int(args.cap_gb * 1e9),
+                                                   bf16=(args.bf16 or "bf16" in mods), offload_lag=lag, prefetch_depth=depth)
         log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
             results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))
 
@@ -134,7 +151,9 @@ def main():
     # dominant kernel: the convolution class with the most device time over the timed steps of all
     # policies of this run (the same launches a kernel trace of this command sees, warm-up aside)
     prof = {}
-    for p in profiles.values():
+    for pname, p in profiles.items():
+        if pname.endswith("+bf16") != args.bf16:
+            continue  # the roofline entry is taken over the runs of the headline element type
         for k, v in p.items():
             acc = prof.setdefault(k, {"launches": 0, "ms": 0.0, "flops": 0.0, "bytes": 0.0})
             for field in acc:
@@ -163,7 +182,9 @@ def main():
         if base and "VDNN_ALL+refined" in results else None,
         "refined_peak_hbm_reduction_vs_baseline": (base["peak_hbm_gb"] / results["VDNN_ALL+refined"]["peak_hbm_gb"])
         if base and "VDNN_ALL+refined" in results else None,
-        "losses_bit_identical": len({results[k]["loss"] for k in results}) == 1,
+        "losses_bit_identical": len({results[k]["loss"] for k in results if not k.endswith("+bf16")}) <= 1
+        and len({results[k]["loss"] for k in results if k.endswith("+bf16")}) <= 1,
+        "best_offloading_vs_fp32_baseline": best_offloading(results, base),
         "conv_mfma_util": conv_all_tf / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
