@@ -72,11 +72,33 @@ static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, con
     return VDNN_OK;
 }
 
-// Tile shape by output-row count: 64-row tiles for narrow layers, 128 otherwise.
-template <class AL, class BL, class EP>
-static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names, const AL& al, const BL& bl, const EP& ep, int M, int N, int K) {
-    if (M <= 64) return launch_igemm<64, 256>(ctx, stream, names.t64, al, bl, ep, make_dims(M, N, K, 64, 256, 1));
-    return launch_igemm<128, 128>(ctx, stream, names.t128, al, bl, ep, make_dims(M, N, K, 128, 128, 1));
+int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
+                              const float* bias, int opix, int channels);
+int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, size_t count, int splits,
+                              const float* bias, int opix, int channels);
+
+// Forward / backward data. Tile shape by output-row count: 64-row tiles for narrow layers, 128
+// otherwise. A grid that cannot fill the chip (few output pixels: the fully connected layers written
+// as convolutions) splits its reduction; the partial sums go to the staging area and are added in split
+// order, with the bias, by a second kernel. The split count depends on the shape only.
+template <class AL, class BL, class E>
+static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names, const AL& al, const BL& bl, const StoreNCHW<E>& ep, int M, int N, int K) {
+    const bool narrow = M <= 64;
+    const int TM = narrow ? 64 : 128, TN = narrow ? 256 : 128;
+    const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
+    int splits = 1;
+    const size_t out_bytes = (size_t)M * N * sizeof(float);
+    if (tiles < 2l * ctx->num_cu && ctx->reduce_scratch) {
+        long cap = ((long)K + 8 * KB - 1) / (8 * KB); // at least eight slices per split
+        const long by_mem = (long)(ctx->reduce_scratch_bytes / out_bytes);
+        if (cap > by_mem) cap = by_mem;
+        splits = choose_splits(tiles, K, cap, ctx->num_cu, out_bytes, 2.0 * TM * TN * KB);
+    }
+    const GemmDims d = make_dims(M, N, K, TM, TN, splits);
+    const int rc = narrow ? launch_igemm<64, 256>(ctx, stream, names.t64, al, bl, ep, d)
+                          : launch_igemm<128, 128>(ctx, stream, names.t128, al, bl, ep, d);
+    if (rc != VDNN_OK || d.splits == 1) return rc;
+    return launch_reduce_splits_nchw(ctx, stream, ep.out, ep.partial, (size_t)M * N, d.splits, ep.bias, ep.opix, M);
 }
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
@@ -87,7 +109,7 @@ int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const fl
 // forward with the given A loader (128-bit or 32-bit filter loads)
 template <class AL, class E>
 static int conv_fwd_with(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const AL& al, const E* x, const float* bias, E* y) {
-    StoreNCHW<E> ep{y, bias, g.P * g.Q};
+    StoreNCHW<E> ep{y, bias, g.P * g.Q, ctx->reduce_scratch};
     const int M = g.K, N = g.N * g.P * g.Q, K = g.C * g.R * g.S;
     const FastDiv dRS = FastDiv::make(g.R * g.S), dS = FastDiv::make(g.S);
     if (g.R * g.S <= 32) {
@@ -145,7 +167,7 @@ static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
         const int RS = g.R * g.S;
         LoadIm2colPixTap<0, E> bl{{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N,
                                 FastDiv::make(RS), FastDiv::make(g.S)}};
-        StoreNCHW<E> ep{y, bias, g.P * g.Q};
+        StoreNCHW<E> ep{y, bias, g.P * g.Q, ctx->reduce_scratch};
         if (algo_mode == 1 && workspace && workspace_bytes >= wbytes && aligned16(workspace)) {
             // perf-optimal: the filter bank, re-laid-out in the workspace, is a dense 128-bit operand
             float* packed = (float*)workspace;
@@ -190,7 +212,7 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
     VDNN_REQUIRE(pixel_tile_span_ok((long)g.K * g.P * g.Q, g.H * g.W, 256, (int)sizeof(E)), "output-gradient samples too large for one tile's descriptor");
     const int RS = g.R * g.S;
     LoadFilterT al{w, g.C, RS, (unsigned)((long)g.K * g.C * RS * 4), FastDiv::make(RS)};
-    StoreNCHW<E> ep{dx, nullptr, g.H * g.W};
+    StoreNCHW<E> ep{dx, nullptr, g.H * g.W, ctx->reduce_scratch};
     const int M = g.C, N = g.N * g.H * g.W, K = g.K * RS;
     const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S);
     const long sample = (long)g.K * g.P * g.Q;

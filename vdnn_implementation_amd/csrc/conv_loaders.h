@@ -315,14 +315,17 @@ struct StoreNCHW {
     E* out;
     const float* bias; // optional, per output channel
     int opix;          // pixels of one output plane
-    __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int, const GemmDims& d) const {
+    float* partial;    // split reductions: split ks writes its sums to partial[ks][same index], bias added by the reduction
+    __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int ks, const GemmDims& d) const {
         const int l32 = lane & 31, lk = lane >> 5;
 #pragma unroll
         for (int jt = 0; jt < 2; jt++) {
             const int j = j0 + jt * 32 + l32;
             if (j >= d.N) continue;
             const int n = j / opix, pix = j - n * opix;
-            E* o = out + (size_t)n * d.M * opix + pix;
+            const size_t base = (size_t)n * d.M * opix + pix;
+            E* o = out + base;
+            float* po = partial + (size_t)ks * d.M * d.N + base;
 #pragma unroll
             for (int it = 0; it < 2; it++)
 #pragma unroll
@@ -330,8 +333,12 @@ struct StoreNCHW {
                     const int m = m0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
                     if (m >= d.M) continue;
                     float r = acc[it][jt][v];
-                    if (bias) r += bias[m];
-                    store_elem(o + (size_t)m * opix, r);
+                    if (d.splits > 1) {
+                        po[(size_t)m * opix] = r;
+                    } else {
+                        if (bias) r += bias[m];
+                        store_elem(o + (size_t)m * opix, r);
+                    }
                 }
         }
     }

@@ -189,6 +189,36 @@ int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const f
     return launch_reduce_splits_t(ctx, stream, out, partial, count, splits, alpha, accumulate, bias_j, ncols);
 }
 
+// NCHW result of a split convolution: out[i] = p[0][i] + p[1][i] + ... (+ bias[channel of i]); split order fixed
+template <class E>
+__global__ void __launch_bounds__(EB) reduce_splits_nchw_kernel(E* __restrict__ out, const float* __restrict__ partial, size_t count,
+                                                                int splits, const float* __restrict__ bias, int opix, int channels) {
+    const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
+    if (i >= count) return;
+    float s = partial[i];
+    for (int k = 1; k < splits; k++) s += partial[(size_t)k * count + i];
+    if (bias) s += bias[(i / opix) % channels];
+    store_elem(out + i, s);
+}
+
+template <class E>
+static int launch_reduce_splits_nchw_t(vdnn_ctx* ctx, hipStream_t stream, E* out, const float* partial, size_t count, int splits,
+                                       const float* bias, int opix, int channels) {
+    ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)count * (splits + 1));
+    hipLaunchKernelGGL(reduce_splits_nchw_kernel<E>, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
+                       out, partial, count, splits, bias, opix, channels);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
+                              const float* bias, int opix, int channels) {
+    return launch_reduce_splits_nchw_t(ctx, stream, out, partial, count, splits, bias, opix, channels);
+}
+int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, size_t count, int splits,
+                              const float* bias, int opix, int channels) {
+    return launch_reduce_splits_nchw_t(ctx, stream, out, partial, count, splits, bias, opix, channels);
+}
+
 // param[i] = fma(alpha, grad[i], param[i]), the expression the fused updates evaluate
 __global__ void __launch_bounds__(EB) sgd_apply_kernel(const float* __restrict__ grad, float* __restrict__ param, float alpha, size_t count) {
     const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
