@@ -205,7 +205,14 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
         if (s1_3x3 && g.C == 3) hipLaunchKernelGGL((conv_bwd_data_smallc_s1_kernel<3, 3, 3, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
         else if (s1_3x3 && g.C == 4) hipLaunchKernelGGL((conv_bwd_data_smallc_s1_kernel<3, 3, 4, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
         else if (g.sh == 1 && g.sw == 1) hipLaunchKernelGGL((conv_bwd_data_smallc_kernel<true, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
-        else hipLaunchKernelGGL((conv_bwd_data_smallc_kernel<false, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
+        else {
+            // one workgroup per 256 pixels of one (sample, residue class modulo the stride)
+            const int Ht = (g.H + g.ph + g.sh - 1) / g.sh, Wt = (g.W + g.pw + g.sw - 1) / g.sw;
+            const long per_class = ((long)Ht * Wt + 255) / 256;
+            const long sblocks = per_class * g.sh * g.sw * g.N;
+            VDNN_REQUIRE(sblocks < (1l << 31), "grid too large");
+            hipLaunchKernelGGL(conv_bwd_data_smallc_strided_kernel<E>, dim3((unsigned)sblocks), dim3(256), 0, st, dy, w, dx, g, Ht, Wt, (int)per_class);
+        }
         VDNN_LAUNCH_CHECK();
         return VDNN_OK;
     }

@@ -84,6 +84,63 @@ __global__ void __launch_bounds__(256) conv_bwd_data_smallc_kernel(const E* __re
     if (g.C > 3) store_elem(o + 3 * plane, acc.w);
 }
 
+// Strided layers (AlexNet / OverFeat conv1: 11x11, stride 4). An input pixel only receives the taps
+// congruent to its position modulo the stride, so pixels are grouped by residue class (th mod sh,
+// tw mod sw): within a class every pixel uses the same taps, the filter reads are wavefront-uniform
+// and consecutive lanes read consecutive dy columns. One workgroup = 256 pixels of one class of one
+// sample; summation order per pixel is (k, r, s) ascending as in the kernels above.
+template <class E>
+__global__ void __launch_bounds__(256) conv_bwd_data_smallc_strided_kernel(const E* __restrict__ dy, const float* __restrict__ w,
+                                                                           E* __restrict__ dx, const ConvGeo g, int Ht, int Wt, int blocks_per_class) {
+    __shared__ float4 ws[SMALLC_KC][SMALLC_MAXTAPS];
+    const int tid = threadIdx.x;
+    const int RS = g.R * g.S;
+    const int classes = g.sh * g.sw;
+    const int blk = blockIdx.x % blocks_per_class;
+    const int rest = blockIdx.x / blocks_per_class;
+    const int cls = rest % classes, n = rest / classes;
+    const int rh = cls / g.sw, rw = cls - rh * g.sw;
+    const int idx = blk * 256 + tid;
+    const int i = idx / Wt, j = idx - i * Wt;
+    const int th = i * g.sh + rh, tw = j * g.sw + rw;
+    const int h = th - g.ph, x = tw - g.pw;
+    const bool live = i < Ht && h >= 0 && h < g.H && x >= 0 && x < g.W;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k0 = 0; k0 < g.K; k0 += SMALLC_KC) {
+        __syncthreads();
+        for (int t = tid; t < SMALLC_KC * RS; t += 256) {
+            const int kk = t / RS, tap = t - kk * RS;
+            float v[4] = {0.f, 0.f, 0.f, 0.f};
+            if (k0 + kk < g.K)
+                for (int c = 0; c < g.C; c++) v[c] = w[((long)(k0 + kk) * g.C + c) * RS + tap];
+            ws[kk][tap] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+        __syncthreads();
+        if (!live) continue;
+        const int kmax = min(SMALLC_KC, g.K - k0);
+        for (int kk = 0; kk < kmax; kk++) {
+            const E* dyp = dy + ((long)n * g.K + k0 + kk) * g.P * g.Q;
+            for (int r = rh, p = i; r < g.R && p >= 0; r += g.sh, p--) {
+                if (p >= g.P) continue;
+                const E* row = dyp + (long)p * g.Q;
+                for (int s = rw, q = j; s < g.S && q >= 0; s += g.sw, q--) {
+                    if (q >= g.Q) continue;
+                    const float d = load_elem(row + q);
+                    const float4 f = ws[kk][r * g.S + s];
+                    acc.x += d * f.x; acc.y += d * f.y; acc.z += d * f.z; acc.w += d * f.w;
+                }
+            }
+        }
+    }
+    if (!live) return;
+    E* o = dx + ((long)n * g.C * g.H + h) * g.W + x;
+    const long plane = (long)g.H * g.W;
+    store_elem(o, acc.x);
+    if (g.C > 1) store_elem(o + plane, acc.y);
+    if (g.C > 2) store_elem(o + 2 * plane, acc.z);
+    if (g.C > 3) store_elem(o + 3 * plane, acc.w);
+}
+
 // The same, for a compile-time window at stride 1 (VGG's 3x3): fully unrolled and branch-free. Taps
 // outside dy are read from a clamped position and replaced by zero. The filter values of one output
 // channel are wave-uniform, so they are fetched with scalar loads straight from global memory.
