@@ -63,10 +63,12 @@ static const PassNames kFwdPackedNames{"conv_fwd_packed_64x256", "conv_fwd_packe
 static const PassNames kBwdDataPackedNames{"conv_bwd_data_packed_64x256", "conv_bwd_data_packed_128x128"};
 
 template <int TM, int TN, class AL, class BL, class EP>
-static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, const AL& al, const BL& bl, const EP& ep, const GemmDims& d) {
+static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, const AL& al, const BL& bl, const EP& ep, const GemmDims& d, double flops = 0.0) {
     const long blocks = (long)d.mtiles * d.ntiles * d.splits;
     if (blocks <= 0 || blocks >= (1l << 31)) { set_error("igemm: grid of %ld workgroups out of range", blocks); return VDNN_EINVAL; }
-    ProfScope prof(ctx, stream, name, 2.0 * d.M * (double)d.N * d.K, 0.0);
+    // reported work is the algorithmic count where the caller gives one (backward data of a strided or
+    // unpadded layer multiplies taps that fall outside the output; they are not counted)
+    ProfScope prof(ctx, stream, name, flops > 0.0 ? flops : 2.0 * d.M * (double)d.N * d.K, 0.0);
     hipLaunchKernelGGL((igemm_kernel<TM, TN, AL, BL, EP>), dim3((unsigned)blocks), dim3(NT), 0, stream, al, bl, ep, d);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
@@ -82,7 +84,7 @@ int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, co
 // as convolutions) splits its reduction; the partial sums go to the staging area and are added in split
 // order, with the bias, by a second kernel. The split count depends on the shape only.
 template <class AL, class BL, class E>
-static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names, const AL& al, const BL& bl, const StoreNCHW<E>& ep, int M, int N, int K) {
+static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names, const AL& al, const BL& bl, const StoreNCHW<E>& ep, int M, int N, int K, double flops = 0.0) {
     const bool narrow = M <= 64;
     const int TM = narrow ? 64 : 128, TN = narrow ? 256 : 128;
     const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
@@ -95,8 +97,8 @@ static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names
         splits = choose_splits(tiles, K, cap, ctx->num_cu, out_bytes, 2.0 * TM * TN * KB);
     }
     const GemmDims d = make_dims(M, N, K, TM, TN, splits);
-    const int rc = narrow ? launch_igemm<64, 256>(ctx, stream, names.t64, al, bl, ep, d)
-                          : launch_igemm<128, 128>(ctx, stream, names.t128, al, bl, ep, d);
+    const int rc = narrow ? launch_igemm<64, 256>(ctx, stream, names.t64, al, bl, ep, d, flops)
+                          : launch_igemm<128, 128>(ctx, stream, names.t128, al, bl, ep, d, flops);
     if (rc != VDNN_OK || d.splits == 1) return rc;
     return launch_reduce_splits_nchw(ctx, stream, ep.out, ep.partial, (size_t)M * N, d.splits, ep.bias, ep.opix, M);
 }
@@ -131,6 +133,11 @@ constexpr int kPlanningCUs = 256;
 constexpr size_t kDefaultStagingBytes = (size_t)64 << 20;
 constexpr size_t kMaxWgradWorkspace = (size_t)256 << 20;
 
+// A window that covers the whole unpadded input (the fully connected layers OverFeat writes as
+// convolutions, network.cu:449-481) is a dense GEMM over (c,h,w): the implicit-GEMM backward data would
+// spend R*S times the work on taps that fall outside the single output pixel.
+static bool is_dense(const ConvGeo& g) { return g.P == 1 && g.Q == 1 && g.ph == 0 && g.pw == 0 && g.R == g.H && g.S == g.W; }
+
 static bool packed_fwd_ok(const ConvGeo& g) { return g.R * g.S <= 32 && g.C % KB == 0; }
 static bool packed_bwd_data_ok(const ConvGeo& g) {
     return g.C > 4 && g.sh == 1 && g.sw == 1 && g.R * g.S <= 32 && g.K % KB == 0;
@@ -158,6 +165,7 @@ static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
     ConvGeo g;
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(x && w && y, "null tensor");
+    if (is_dense(g)) return vdnn_fc_fwd(ctx, stream, g.N, g.C * g.H * g.W, g.K, x, w, bias, y);
     VDNN_REQUIRE(pixel_tile_span_ok((long)g.C * g.H * g.W, g.P * g.Q, 256, (int)sizeof(E)), "input samples too large for one tile's descriptor");
     hipStream_t st = stream_of(ctx, stream);
     const int K = g.C * g.R * g.S;
@@ -195,6 +203,7 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
     ConvGeo g;
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(dy && w && dx, "null tensor");
+    if (is_dense(g)) return vdnn_fc_bwd_data(ctx, stream, g.N, g.C * g.H * g.W, g.K, dy, w, dx);
     hipStream_t st = stream_of(ctx, stream);
     if (g.C <= 4 && g.R * g.S <= SMALLC_MAXTAPS) {
         const long total = (long)g.N * g.H * g.W;
@@ -223,6 +232,7 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
     const int M = g.C, N = g.N * g.H * g.W, K = g.K * RS;
     const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S);
     const long sample = (long)g.K * g.P * g.Q;
+    const double flops = 2.0 * g.N * (double)g.K * g.C * RS * g.P * g.Q;
     if (g.sh == 1 && g.sw == 1) {
         if (RS <= 32 && g.K % KB == 0) {
             // blocked tap-major reduction: one slice = one tap x 16 output channels
@@ -233,20 +243,20 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
                 const int rc = launch_pack_filter(ctx, st, w, packed, g.C, g.K, RS, RS, g.C * RS);
                 if (rc != VDNN_OK) return rc;
                 LoadDenseRed<true> alp{packed, (long)K, g.C, wbytes};
-                return launch_by_m(ctx, st, kBwdDataPackedNames, alp, bl, ep, M, N, K);
+                return launch_by_m(ctx, st, kBwdDataPackedNames, alp, bl, ep, M, N, K, flops);
             }
             LoadFilterTap<true> alt{w, RS, g.C * RS, g.C, RS, wbytes, dRS};
-            return launch_by_m(ctx, st, kBwdDataNames, alt, bl, ep, M, N, K);
+            return launch_by_m(ctx, st, kBwdDataNames, alt, bl, ep, M, N, K, flops);
         }
         if (RS <= 32) {
             LoadIm2colPix<1, false, E> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS};
-            return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K);
+            return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K, flops);
         }
         LoadIm2colPix<1, true, E> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS};
-        return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K);
+        return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K, flops);
     }
     LoadIm2colPix<2, true, E> bl{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, g.sh, g.sw, sample, g.N, dRS, dS};
-    return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K);
+    return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K, flops);
 }
 
 // out = (accumulate ? out : 0) + alpha * dW
@@ -259,6 +269,9 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     ConvGeo g;
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(x && dy && w, "null tensor");
+    if (is_dense(g))
+        return accumulate ? vdnn_fc_bwd_weight_sgd(ctx, stream, g.N, g.C * g.H * g.W, g.K, x, dy, w, alpha)
+                          : vdnn_fc_bwd_weight(ctx, stream, g.N, g.C * g.H * g.W, g.K, x, dy, w);
     hipStream_t st = stream_of(ctx, stream);
     const int M = g.K, N = g.C * g.R * g.S, PQ = g.P * g.Q, RS = g.R * g.S;
     const long Kred = (long)g.N * PQ;
@@ -334,7 +347,7 @@ extern "C" {
 size_t vdnn_conv_workspace_bytes(const vdnn_shape_t* shape, int algo_mode, int pass) {
     ConvGeo g;
     if (!shape || !geo_from_shape(shape, g)) return 0;
-    if (algo_mode == 0 /* VDNN_MEMORY_OPT_ALGO */) return 0;
+    if (algo_mode == 0 /* VDNN_MEMORY_OPT_ALGO */ || is_dense(g)) return 0;
     // Perf-optimal mode: forward and backward data re-lay the filter bank out for 128-bit operand
     // loads; backward filter takes a staging area large enough for the split count that fills the chip.
     const int RS = g.R * g.S;
