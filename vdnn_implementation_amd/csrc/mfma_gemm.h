@@ -138,9 +138,9 @@ __device__ __forceinline__ floatx4 read_frag(const float* tile, int l32, int lk,
     }
 }
 
-template <int TM, int TN, bool A_RED, bool B_RED>
+template <int TM, int TN, bool A_RED, bool B_RED, class Mid>
 __device__ __forceinline__ void mfma_slice(const float* __restrict__ As, const float* __restrict__ Bs,
-                                           floatx16 (&acc)[2][2], int lane) {
+                                           floatx16 (&acc)[2][2], int lane, Mid&& mid) {
     const int l32 = lane & 31, lk = lane >> 5;
     constexpr int A_TILE = 32 * LdsTile<TM, A_RED>::ROW_STRIDE, B_TILE = 32 * LdsTile<TN, B_RED>::ROW_STRIDE;
     // fragments of group g+1 are read from LDS while the MFMAs of group g execute
@@ -165,6 +165,7 @@ __device__ __forceinline__ void mfma_slice(const float* __restrict__ As, const f
 #pragma unroll
                 for (int j = 0; j < 2; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][e], b[cur][j][e], acc[i][j], 0, 0, 0);
+        if (g == 0) mid(); // work placed between the two halves of the slice's MFMAs
     }
 }
 
@@ -237,27 +238,38 @@ __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, con
     typename AL::template Regs<TM> ra;
     typename BL::template Regs<TN> rb;
 
+    // Software pipeline, one barrier per slice and no branch in the loop: while slice s is multiplied
+    // out of LDS buffer s%2, the registers hold slice s+1 (fetched during slice s-1). Half-way through
+    // the slice's MFMAs they are written to the other LDS buffer (free since the barrier that ended
+    // slice s-1) and the fetch of slice s+2 is issued into the same registers, which gives every
+    // global load a full slice of MFMA time to return. Fetches past the end of the range read as
+    // zero (or are never used): buffer loads cannot fault, so the last two rounds need no guard.
     const int nslices = (k_end - k_begin + KB - 1) / KB;
-    if (nslices > 0) {
-        al.template load<TM>(sa, k_begin, k_end, tid, ra);
-        bl.template load<TN>(sb, k_begin, k_end, tid, rb);
-        AL::template store<TM>(As[0], tid, ra);
-        BL::template store<TN>(Bs[0], tid, rb);
-    }
+    al.template load<TM>(sa, k_begin, k_end, tid, ra);
+    bl.template load<TN>(sb, k_begin, k_end, tid, rb);
+    AL::template store<TM>(As[0], tid, ra);
+    BL::template store<TN>(Bs[0], tid, rb);
+    al.template load<TM>(sa, k_begin + KB, k_end, tid, ra);
+    bl.template load<TN>(sb, k_begin + KB, k_end, tid, rb);
     __syncthreads();
     for (int s = 0; s < nslices; s++) {
         const int cur = s & 1;
-        const bool more = s + 1 < nslices;
-        if (more) {
-            const int kk0 = k_begin + (s + 1) * KB;
-            al.template load<TM>(sa, kk0, k_end, tid, ra);
-            bl.template load<TN>(sb, kk0, k_end, tid, rb);
-        }
-        mfma_slice<TM, TN, AL::RED_MAJOR, BL::RED_MAJOR>(As[cur] + wm0 * LA::ROW_STRIDE, Bs[cur] + wn0 * LB::ROW_STRIDE, acc, lane);
-        if (more) {
+        mfma_slice<TM, TN, AL::RED_MAJOR, BL::RED_MAJOR>(As[cur] + wm0 * LA::ROW_STRIDE, Bs[cur] + wn0 * LB::ROW_STRIDE, acc, lane, [&]() {
             AL::template store<TM>(As[cur ^ 1], tid, ra);
             BL::template store<TN>(Bs[cur ^ 1], tid, rb);
-        }
+            const int kk0 = k_begin + (s + 2) * KB;
+            al.template load<TM>(sa, kk0, k_end, tid, ra);
+            bl.template load<TN>(sb, kk0, k_end, tid, rb);
+        });
+        // Issue order asked of the scheduler: every MFMA is followed by a little of the other work, so the
+        // wavefront keeps the matrix pipe fed instead of stopping for a block of loads and stores:
+        // first quarter fragment reads, second quarter the LDS stores, second half the global loads.
+#pragma unroll
+        for (int i = 0; i < 8; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 3, 0); }
+#pragma unroll
+        for (int i = 0; i < 8; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); }
+#pragma unroll
+        for (int i = 0; i < 16; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
         __syncthreads();
     }
 
