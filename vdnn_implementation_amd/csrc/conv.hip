@@ -324,6 +324,28 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     StoreDense<float> ep{w, staging, nullptr, (long)N, (long)M * N, alpha, accumulate};
     const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S), dQ = FastDiv::make(g.Q);
     const bool vec = PQ % 4 == 0 && aligned16(dy); // bf16: four elements are 8 bytes, covered by the same test
+    // tap-major column order when the tile's columns fall into whole groups of channels with one tap each
+    const int tile_n = narrow ? 256 : 128;
+    const int ntap = g.C % tile_n == 0 ? 1 : (g.C % (tile_n / 2) == 0 ? 2 : (g.C % (tile_n / 4) == 0 ? 4 : 0));
+    if (vec && ntap != 0) {
+        const FastDiv dC = FastDiv::make(g.C);
+        StoreFilterTap ept{w, staging, g.C, RS, (long)M * N, alpha, accumulate, dC};
+        LoadDyRed<true, E> al{dy, g.N, g.K, PQ, d.kchunk, d.K};
+        int rc2;
+#define VDNN_WGRAD_TAP(NTAP)                                                                                                \
+        do {                                                                                                                \
+            LoadIm2colRedTap<NTAP, E> bl{x, g.N, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N, d.kchunk, d.K, dC, dS, dQ}; \
+            rc2 = narrow ? launch_igemm<64, 256>(ctx, st, kBwdFilterNames.t64, al, bl, ept, d)                               \
+                         : launch_igemm<128, 128>(ctx, st, kBwdFilterNames.t128, al, bl, ept, d);                            \
+        } while (0)
+        if (ntap == 1) VDNN_WGRAD_TAP(1);
+        else if (ntap == 2) VDNN_WGRAD_TAP(2);
+        else VDNN_WGRAD_TAP(4);
+#undef VDNN_WGRAD_TAP
+        if (rc2 != VDNN_OK) return rc2;
+        if (d.splits > 1) return launch_reduce_splits(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, accumulate, nullptr, 0);
+        return VDNN_OK;
+    }
     const bool big = RS > 32;
     int rc;
 #define VDNN_WGRAD(VEC, BIG)                                                                                              \

@@ -90,6 +90,113 @@ struct LoadIm2colPixTap {
 
 namespace vdnn {
 
+// ---- im2col operand of backward filter, columns in tap-major order: B[(n,p,q)][tap*C + c] -------------
+// The filter gradient's columns are taken as (tap, channel) instead of (channel, tap), so that the T
+// columns of a tile share one tap (C a multiple of T) or fall into NTAP groups of T/NTAP channels with
+// one tap each (C = T/NTAP). A thread owns pixel t%16 of the slice and columns t/16 + 16*i, as in the
+// channel-major loader, but the tap - its offset and whether it falls outside the image for the
+// thread's pixel - is then a per-slice quantity per group instead of per load: a load costs one vector
+// add. The epilogue StoreFilterTap puts the result back into the filter's (k, c, r, s) layout.
+template <int NTAP, class E = float>
+struct LoadIm2colRedTap {
+    static constexpr bool RED_MAJOR = true;
+    static constexpr int ES = ElemBytes<E>::V;
+    const E* x;
+    int N, C, H, W, R, S, P, Q, ph, pw, sh, sw;
+    int ncols; // C*R*S
+    int kchunk, Ktot;
+    FastDiv divC, divS, divQ;
+    template <int T> struct Regs { float s[T / 16]; };
+    template <int T> struct State {
+        int cconst[T / 16];  // byte offset of the column's channel plane, or SENT outside the matrix
+        int tapoff[NTAP];    // byte offset of the group's tap (r*W + s), wave-uniform
+        int tr[NTAP], ts[NTAP];
+        PixelCursor cur; int kk;
+        __amdgpu_buffer_rsrc_t rsrc;
+    };
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int j0, int tid, int, int k_begin) const {
+        const int PQ = P * Q;
+        const int n_first = k_begin / PQ;
+        const long chw = (long)C * H * W;
+        const long shift = -((long)ph * W + pw);
+        int k_last = k_begin + kchunk; if (k_last > Ktot) k_last = Ktot;
+        const int n_last = k_last > k_begin ? (k_last - 1) / PQ : n_first;
+        st.rsrc = make_rsrc(x + (long)n_first * chw + shift, clamp_range(((long)(n_last - n_first + 1) * chw - shift) * ES));
+        st.kk = k_begin + (tid & 15);
+        st.cur.init(st.kk, PQ, n_first);
+#pragma unroll
+        for (int g = 0; g < NTAP; g++) {
+            const int tap = divC.div(j0 + g * (T / NTAP)); // one tap per group of T/NTAP columns
+            const int r = divS.div(tap), s_ = tap - r * S;
+            st.tr[g] = r; st.ts[g] = s_;
+            st.tapoff[g] = (r * W + s_) * ES;
+        }
+#pragma unroll
+        for (int i = 0; i < T / 16; i++) {
+            const int j = j0 + (tid >> 4) + 16 * i;
+            const int tap = divC.div(j);
+            st.cconst[i] = j < ncols ? (j - tap * C) * H * W * ES : SENT;
+        }
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int, int kend, int, Regs<T>& r) const {
+        const int PQ = P * Q;
+        const int p = divQ.div(st.cur.pq), q = st.cur.pq - p * Q;
+        const int ih0 = p * sh - ph, iw0 = q * sw - pw;
+        const int pixoff = (st.cur.n * C * H * W + p * sh * W + q * sw) * ES;
+        const bool live = st.kk < kend;
+        int base[NTAP];
+#pragma unroll
+        for (int g = 0; g < NTAP; g++) {
+            const bool ok = live & ((unsigned)(ih0 + st.tr[g]) < (unsigned)H) & ((unsigned)(iw0 + st.ts[g]) < (unsigned)W);
+            base[g] = ok ? pixoff + st.tapoff[g] : SENT;
+        }
+#pragma unroll
+        for (int i = 0; i < T / 16; i++) r.s[i] = buf_load_e<E>(st.rsrc, base[i / (T / 16 / NTAP)] + st.cconst[i], 0);
+        st.kk += KB;
+        st.cur.advance(PQ);
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(float* lds, int tid, const Regs<T>& r) {
+#pragma unroll
+        for (int i = 0; i < T / 16; i++) lds[((tid >> 4) + 16 * i) * RED_STRIDE + (tid & 15)] = r.s[i];
+    }
+};
+
+// Result of the tap-major backward filter: GEMM column j = tap*C + c goes to filter element
+// (m, c, tap) at out[m*ncols + c*RS + tap]; a split's partial sums use the same layout.
+struct StoreFilterTap {
+    float* out;
+    float* partial;
+    int C, RS;
+    long partial_stride;
+    float alpha;
+    int accumulate;
+    FastDiv divC;
+    __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int ks, const GemmDims& d) const {
+        const int l32 = lane & 31, lk = lane >> 5;
+#pragma unroll
+        for (int jt = 0; jt < 2; jt++) {
+            const int j = j0 + jt * 32 + l32;
+            if (j >= d.N) continue;
+            const int tap = divC.div(j), c = j - tap * C;
+            const long col = (long)c * RS + tap;
+#pragma unroll
+            for (int it = 0; it < 2; it++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int m = m0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+                    if (m >= d.M) continue;
+                    const long idx = (long)m * d.N + col;
+                    const float a = acc[it][jt][v];
+                    if (d.splits > 1) partial[(long)ks * partial_stride + idx] = a;
+                    else out[idx] = accumulate ? __fmaf_rn(alpha, a, out[idx]) : alpha * a;
+                }
+        }
+    }
+};
+
 // Filter bank re-laid-out for the blocked tap-major order (the workspace of the perf-optimal mode):
 // packed[row][(cb*RS + tap)*16 + l] = w[row*row_stride + (cb*16 + l)*red_stride + tap], so that the A
 // operand becomes a dense reduction-major matrix read with 128-bit loads.
