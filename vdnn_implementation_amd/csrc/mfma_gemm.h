@@ -6,8 +6,8 @@
 // v_mfma_f32_32x32x2_f32 (64 accumulator registers per lane). Operands come from "loader" policies:
 // a loader says how element (row, kk) of its operand is fetched from global memory (a dense matrix,
 // a filter bank, or an im2col view of an NCHW tensor computed on the fly - the im2col matrix only
-// ever exists as LDS tiles). Loads for slice s+1 are issued into registers before slice s is
-// multiplied, then written to the other LDS buffer: one barrier per slice.
+// ever exists as LDS tiles). Global loads run two slices ahead in registers, LDS is double-buffered,
+// and the loop has one barrier per slice and no branch (see igemm_kernel).
 //
 // The matrix pipe and the vector ALU of a SIMD do not overlap well, so every vector instruction in
 // the loop costs MFMA time. The loaders therefore fetch through buffer descriptors: an element that
@@ -138,37 +138,6 @@ __device__ __forceinline__ floatx4 read_frag(const float* tile, int l32, int lk,
     }
 }
 
-template <int TM, int TN, bool A_RED, bool B_RED, class Mid>
-__device__ __forceinline__ void mfma_slice(const float* __restrict__ As, const float* __restrict__ Bs,
-                                           floatx16 (&acc)[2][2], int lane, Mid&& mid) {
-    const int l32 = lane & 31, lk = lane >> 5;
-    constexpr int A_TILE = 32 * LdsTile<TM, A_RED>::ROW_STRIDE, B_TILE = 32 * LdsTile<TN, B_RED>::ROW_STRIDE;
-    // fragments of group g+1 are read from LDS while the MFMAs of group g execute
-    floatx4 a[2][2], b[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) a[0][i] = read_frag<TM, A_RED>(As + i * A_TILE, l32, lk, 0);
-#pragma unroll
-    for (int j = 0; j < 2; j++) b[0][j] = read_frag<TN, B_RED>(Bs + j * B_TILE, l32, lk, 0);
-#pragma unroll
-    for (int g = 0; g < KB / 8; g++) {
-        const int cur = g & 1, nxt = cur ^ 1;
-        if (g + 1 < KB / 8) {
-#pragma unroll
-            for (int i = 0; i < 2; i++) a[nxt][i] = read_frag<TM, A_RED>(As + i * A_TILE, l32, lk, g + 1);
-#pragma unroll
-            for (int j = 0; j < 2; j++) b[nxt][j] = read_frag<TN, B_RED>(Bs + j * B_TILE, l32, lk, g + 1);
-        }
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[cur][i][e], b[cur][j][e], acc[i][j], 0, 0, 0);
-        if (g == 0) mid(); // work placed between the two halves of the slice's MFMAs
-    }
-}
-
 // Launch geometry of one igemm call. Split s covers reduction indices [s*kchunk, min(K, (s+1)*kchunk)).
 struct GemmDims {
     int M, N, K;
@@ -238,13 +207,22 @@ __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, con
     typename AL::template Regs<TM> ra;
     typename BL::template Regs<TN> rb;
 
-    // Software pipeline, one barrier per slice and no branch in the loop: while slice s is multiplied
-    // out of LDS buffer s%2, the registers hold slice s+1 (fetched during slice s-1). Half-way through
-    // the slice's MFMAs they are written to the other LDS buffer (free since the barrier that ended
-    // slice s-1) and the fetch of slice s+2 is issued into the same registers, which gives every
-    // global load a full slice of MFMA time to return. Fetches past the end of the range read as
-    // zero (or are never used): buffer loads cannot fault, so the last two rounds need no guard.
+    // Software pipeline, one barrier per slice - in the middle of it - and no branch in the loop.
+    // A slice's 32 MFMAs per wavefront run as two groups of 16 (reduction indices 0-7 and 8-15).
+    //   first half of slice s:  read the fragments of (s, group 1) from LDS buffer s%2, multiply group 0
+    //                           (fragments already in registers), write the registers holding slice s+1
+    //                           (fetched during slice s-1) to the other LDS buffer;
+    //   barrier;
+    //   second half:            issue the fetch of slice s+2 into the same registers, read the fragments
+    //                           of (s+1, group 0) from the buffer just completed, multiply group 1.
+    // Each group's fragments are thus read while the previous group is multiplied, across the barrier as
+    // well, so no wavefront waits for LDS; a global load has a full slice of MFMA time to return. All
+    // reads of a buffer precede the barrier after which it may be overwritten. Fetches past the end of
+    // the range read as zero or are never used: buffer loads cannot fault, the last rounds need no guard.
     const int nslices = (k_end - k_begin + KB - 1) / KB;
+    const int l32 = lane & 31, lk = lane >> 5;
+    constexpr int A_TILE = 32 * LA::ROW_STRIDE, B_TILE = 32 * LB::ROW_STRIDE;
+    const int a_off = wm0 * LA::ROW_STRIDE, b_off = wn0 * LB::ROW_STRIDE;
     al.template load<TM>(sa, k_begin, k_end, tid, ra);
     bl.template load<TN>(sb, k_begin, k_end, tid, rb);
     AL::template store<TM>(As[0], tid, ra);
@@ -252,25 +230,51 @@ __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, con
     al.template load<TM>(sa, k_begin + KB, k_end, tid, ra);
     bl.template load<TN>(sb, k_begin + KB, k_end, tid, rb);
     __syncthreads();
+    floatx4 a0[2], b0[2], a1[2], b1[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) a0[i] = read_frag<TM, AL::RED_MAJOR>(As[0] + a_off + i * A_TILE, l32, lk, 0);
+#pragma unroll
+    for (int j = 0; j < 2; j++) b0[j] = read_frag<TN, BL::RED_MAJOR>(Bs[0] + b_off + j * B_TILE, l32, lk, 0);
     for (int s = 0; s < nslices; s++) {
-        const int cur = s & 1;
-        mfma_slice<TM, TN, AL::RED_MAJOR, BL::RED_MAJOR>(As[cur] + wm0 * LA::ROW_STRIDE, Bs[cur] + wn0 * LB::ROW_STRIDE, acc, lane, [&]() {
-            AL::template store<TM>(As[cur ^ 1], tid, ra);
-            BL::template store<TN>(Bs[cur ^ 1], tid, rb);
-            const int kk0 = k_begin + (s + 2) * KB;
-            al.template load<TM>(sa, kk0, k_end, tid, ra);
-            bl.template load<TN>(sb, kk0, k_end, tid, rb);
-        });
-        // Issue order asked of the scheduler: every MFMA is followed by a little of the other work, so the
-        // wavefront keeps the matrix pipe fed instead of stopping for a block of loads and stores:
-        // first quarter fragment reads, second quarter the LDS stores, second half the global loads.
+        const int cur = s & 1, nxt = cur ^ 1;
 #pragma unroll
-        for (int i = 0; i < 8; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 3, 0); }
+        for (int i = 0; i < 2; i++) a1[i] = read_frag<TM, AL::RED_MAJOR>(As[cur] + a_off + i * A_TILE, l32, lk, 1);
 #pragma unroll
-        for (int i = 0; i < 8; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); }
+        for (int j = 0; j < 2; j++) b1[j] = read_frag<TN, BL::RED_MAJOR>(Bs[cur] + b_off + j * B_TILE, l32, lk, 1);
 #pragma unroll
-        for (int i = 0; i < 16; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); }
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i][e], b0[j][e], acc[i][j], 0, 0, 0);
+        AL::template store<TM>(As[nxt], tid, ra);
+        BL::template store<TN>(Bs[nxt], tid, rb);
+        // issue order of the first half: every MFMA is followed by one LDS access
+#pragma unroll
+        for (int i = 0; i < 16; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x300, 2, 0); }
         __syncthreads();
+        const int kk0 = k_begin + (s + 2) * KB;
+        al.template load<TM>(sa, kk0, k_end, tid, ra);
+        bl.template load<TN>(sb, kk0, k_end, tid, rb);
+#pragma unroll
+        for (int i = 0; i < 2; i++) a0[i] = read_frag<TM, AL::RED_MAJOR>(As[nxt] + a_off + i * A_TILE, l32, lk, 0);
+#pragma unroll
+        for (int j = 0; j < 2; j++) b0[j] = read_frag<TN, BL::RED_MAJOR>(Bs[nxt] + b_off + j * B_TILE, l32, lk, 0);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i][e], b1[j][e], acc[i][j], 0, 0, 0);
+        // second half: every MFMA is followed by a global load and an LDS read
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
     }
 
     ep.store(acc, m0 + wm0, j0 + wn0, lane, ks, d);
