@@ -74,6 +74,8 @@ static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, con
     return VDNN_OK;
 }
 
+int launch_reduce_splits_tap(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
+                             float alpha, int accumulate, int C, int RS);
 int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
                               const float* bias, int opix, int channels);
 int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, size_t count, int splits,
@@ -343,7 +345,7 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
         else VDNN_WGRAD_TAP(4);
 #undef VDNN_WGRAD_TAP
         if (rc2 != VDNN_OK) return rc2;
-        if (d.splits > 1) return launch_reduce_splits(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, accumulate, nullptr, 0);
+        if (d.splits > 1) return launch_reduce_splits_tap(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, accumulate, g.C, RS);
         return VDNN_OK;
     }
     const bool big = RS > 32;

@@ -164,8 +164,9 @@ struct LoadIm2colRedTap {
     }
 };
 
-// Result of the tap-major backward filter: GEMM column j = tap*C + c goes to filter element
-// (m, c, tap) at out[m*ncols + c*RS + tap]; a split's partial sums use the same layout.
+// Result of the tap-major backward filter: GEMM column j = tap*C + c is filter element (m, c, tap) at
+// out[m*ncols + c*RS + tap]. A split's partial sums stay in GEMM order (coalesced stores); the ordered
+// sum over the splits puts them into the filter's layout.
 struct StoreFilterTap {
     float* out;
     float* partial;
@@ -190,7 +191,7 @@ struct StoreFilterTap {
                     if (m >= d.M) continue;
                     const long idx = (long)m * d.N + col;
                     const float a = acc[it][jt][v];
-                    if (d.splits > 1) partial[(long)ks * partial_stride + idx] = a;
+                    if (d.splits > 1) partial[(long)ks * partial_stride + (long)m * d.N + j] = a;
                     else out[idx] = accumulate ? __fmaf_rn(alpha, a, out[idx]) : alpha * a;
                 }
         }

@@ -189,6 +189,30 @@ int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const f
     return launch_reduce_splits_t(ctx, stream, out, partial, count, splits, alpha, accumulate, bias_j, ncols);
 }
 
+// filter gradient whose partial sums are in tap-major column order: out[m][c][tap] gets partial[.][m][tap*C + c]
+__global__ void __launch_bounds__(EB) reduce_splits_tap_kernel(float* __restrict__ out, const float* __restrict__ partial, size_t count,
+                                                               int splits, float alpha, int accumulate, int C, int RS) {
+    const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
+    if (i >= count) return;
+    const int ncols = C * RS;
+    const size_t m = i / ncols;
+    const int rem = (int)(i - m * ncols);
+    const int c = rem / RS, tap = rem - c * RS;
+    const size_t src = m * ncols + (size_t)tap * C + c;
+    float s = partial[src];
+    for (int k = 1; k < splits; k++) s += partial[(size_t)k * count + src];
+    out[i] = accumulate ? __fmaf_rn(alpha, s, out[i]) : alpha * s;
+}
+
+int launch_reduce_splits_tap(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
+                             float alpha, int accumulate, int C, int RS) {
+    ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)count * (splits + 2));
+    hipLaunchKernelGGL(reduce_splits_tap_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
+                       out, partial, count, splits, alpha, accumulate, C, RS);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
 // NCHW result of a split convolution: out[i] = p[0][i] + p[1][i] + ... (+ bias[channel of i]); split order fixed
 template <class E>
 __global__ void __launch_bounds__(EB) reduce_splits_nchw_kernel(E* __restrict__ out, const float* __restrict__ partial, size_t count,
