@@ -140,6 +140,37 @@ def test_conv_perf_opt_variants(ctx, geom):
         assert_close(got, gpu_conv_bwd_filter(ctx, g, x, dy, zero, np.float32(1.0), algo=0), TOL, "bwd filter, two split counts")
 
 
+def test_conv_tail_round_is_split_and_agrees_with_two_half_batches(ctx):
+    """VGG16's 14x14 layers at batch 128 make 784 output tiles for 768 resident workgroups: the 16 tiles of
+    the last round are split along the reduction. No CPU result is affordable at this size; convolution is
+    independent per sample, so the two half batches (392 tiles each, a different launch geometry) must
+    give the same values to float rounding."""
+    geom = (128, 512, 14, 14, 512, 3, 3, 1, 1, 1, 1)
+    half = (64,) + geom[1:]
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((128, 512, 14, 14)).astype(np.float32)
+    w = (rng.standard_normal((512, 512, 3, 3)) * np.sqrt(2.0 / 4608)).astype(np.float32)
+    b = rng.standard_normal(512).astype(np.float32)
+    announce("tail round", geom, "fwd")
+    y = gpu_conv_fwd(ctx, be.shape(*geom), x, w, b)
+    y2 = np.concatenate([gpu_conv_fwd(ctx, be.shape(*half), x[:64], w, b), gpu_conv_fwd(ctx, be.shape(*half), x[64:], w, b)])
+    assert_close(y, y2, 1e-5, "forward, whole batch against two halves")
+    # a few output elements against the definition, in float64
+    for (n, k, p, q) in ((0, 0, 0, 0), (127, 511, 13, 13), (77, 300, 6, 0), (127, 5, 0, 13)):
+        acc = float(b[k])
+        for r in range(3):
+            for s_ in range(3):
+                ih, iw = p - 1 + r, q - 1 + s_
+                if 0 <= ih < 14 and 0 <= iw < 14:
+                    acc += float(np.dot(x[n, :, ih, iw].astype(np.float64), w[k, :, r, s_].astype(np.float64)))
+        assert abs(y[n, k, p, q] - acc) <= 1e-4 * max(1.0, abs(acc))
+    announce("tail round", geom, "bwd_data")
+    dy = rng.standard_normal(y.shape).astype(np.float32)
+    dx = gpu_conv_bwd_data(ctx, be.shape(*geom), dy, w)
+    dx2 = np.concatenate([gpu_conv_bwd_data(ctx, be.shape(*half), dy[:64], w), gpu_conv_bwd_data(ctx, be.shape(*half), dy[64:], w)])
+    assert_close(dx, dx2, 1e-5, "backward data, whole batch against two halves")
+
+
 def test_conv_results_do_not_depend_on_the_run(ctx):
     """Split reductions are ordered: two runs give identical bits."""
     geom = (4, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1)

@@ -130,8 +130,6 @@ int vdnn_pool_init(vdnn_ctx* ctx, size_t bytes) {
     uintptr_t s = ctx->pool.allocate(kReduceScratchBytes);
     ctx->reduce_scratch = (float*)s;
     ctx->reduce_scratch_bytes = kReduceScratchBytes;
-    ctx->zeros = (const float*)ctx->pool.allocate(vdnn::Pool::kGranularity);
-    if (!ctx->plan_only) VDNN_HIP(hipMemset((void*)ctx->zeros, 0, vdnn::Pool::kGranularity));
     return VDNN_OK;
 }
 
@@ -145,7 +143,6 @@ int vdnn_pool_finalize(vdnn_ctx* ctx) {
     ctx->pool_base = nullptr;
     ctx->reduce_scratch = nullptr;
     ctx->reduce_scratch_bytes = 0;
-    ctx->zeros = nullptr;
     ctx->pool.clear();
     return VDNN_OK;
 }

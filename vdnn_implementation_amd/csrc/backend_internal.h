@@ -19,9 +19,6 @@ struct vdnn_ctx {
     // Taken from the pool at vdnn_pool_init so the usage meter sees it; bounded, shape-independent.
     float* reduce_scratch = nullptr;
     size_t reduce_scratch_bytes = 0;
-    // 512 bytes of zeros (the first block of the pool): out-of-range operand elements of the MFMA
-    // kernels are loaded from here, so their loads need neither a branch nor a select afterwards
-    const float* zeros = nullptr;
     int num_cu = 256;
     int act_dtype = VDNN_DTYPE_F32;   // element type of activation tensors handed to the kernels
     // per-kernel timing (vdnn_profile_*)

@@ -51,6 +51,7 @@ static GemmDims make_dims(int M, int N, int K, int TM, int TN, int splits) {
     kchunk = (kchunk + KB - 1) / KB * KB;
     d.kchunk = kchunk;
     d.splits = (K + kchunk - 1) / kchunk;
+    d.full_tiles = 0;
     return d;
 }
 
@@ -64,7 +65,8 @@ static const PassNames kBwdDataPackedNames{"conv_bwd_data_packed_64x256", "conv_
 
 template <int TM, int TN, class AL, class BL, class EP>
 static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, const AL& al, const BL& bl, const EP& ep, const GemmDims& d, double flops = 0.0) {
-    const long blocks = (long)d.mtiles * d.ntiles * d.splits;
+    const long all_tiles = (long)d.mtiles * d.ntiles;
+    const long blocks = d.full_tiles > 0 ? d.full_tiles + (all_tiles - d.full_tiles) * d.splits : all_tiles * d.splits;
     if (blocks <= 0 || blocks >= (1l << 31)) { set_error("igemm: grid of %ld workgroups out of range", blocks); return VDNN_EINVAL; }
     // reported work is the algorithmic count where the caller gives one (backward data of a strided or
     // unpadded layer multiplies taps that fall outside the output; they are not counted)
@@ -74,6 +76,10 @@ static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, con
     return VDNN_OK;
 }
 
+int launch_reduce_tail_nchw(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, int tail_tiles, int splits, int TM, int TN,
+                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix);
+int launch_reduce_tail_nchw(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, int tail_tiles, int splits, int TM, int TN,
+                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix);
 int launch_reduce_splits_tap(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
                              float alpha, int accumulate, int C, int RS);
 int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
@@ -98,10 +104,30 @@ static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names
         if (cap > by_mem) cap = by_mem;
         splits = choose_splits(tiles, K, cap, ctx->num_cu, out_bytes, 2.0 * TM * TN * KB);
     }
-    const GemmDims d = make_dims(M, N, K, TM, TN, splits);
+    GemmDims d = make_dims(M, N, K, TM, TN, splits);
+    // Tail mode: when the tiles make whole rounds of resident workgroups (three per compute unit) plus a
+    // small remainder, that remainder would run as a nearly empty last round as long as a full one. Its
+    // tiles are split so that together they fill about one round of short workgroups instead.
+    const long slots = 3l * ctx->num_cu;
+    const long rem = tiles % slots;
+    int tail_tiles = 0;
+    if (splits == 1 && tiles > slots && rem > 0 && 2 * rem <= slots && ctx->reduce_scratch) {
+        long s = slots / rem;
+        const long by_depth = (long)K / (8 * KB); // at least eight slices per split
+        const long by_mem = (long)(ctx->reduce_scratch_bytes / ((size_t)rem * TM * TN * sizeof(float)));
+        if (s > by_depth) s = by_depth;
+        if (s > by_mem) s = by_mem;
+        if (s >= 2) {
+            d = make_dims(M, N, K, TM, TN, (int)s);
+            if (d.splits >= 2) { d.full_tiles = (int)(tiles - rem); tail_tiles = (int)rem; }
+            else d = make_dims(M, N, K, TM, TN, 1);
+        }
+    }
     const int rc = narrow ? launch_igemm<64, 256>(ctx, stream, names.t64, al, bl, ep, d, flops)
                           : launch_igemm<128, 128>(ctx, stream, names.t128, al, bl, ep, d, flops);
     if (rc != VDNN_OK || d.splits == 1) return rc;
+    if (tail_tiles > 0)
+        return launch_reduce_tail_nchw(ctx, stream, ep.out, ep.partial, tail_tiles, d.splits, TM, TN, M, N, d.mtiles, d.full_tiles, ep.bias, ep.opix);
     return launch_reduce_splits_nchw(ctx, stream, ep.out, ep.partial, (size_t)M * N, d.splits, ep.bias, ep.opix, M);
 }
 
@@ -215,7 +241,7 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
         const bool s1_3x3 = g.sh == 1 && g.sw == 1 && g.R == 3 && g.S == 3;
         if (s1_3x3 && g.C == 3) hipLaunchKernelGGL((conv_bwd_data_smallc_s1_kernel<3, 3, 3, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
         else if (s1_3x3 && g.C == 4) hipLaunchKernelGGL((conv_bwd_data_smallc_s1_kernel<3, 3, 4, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
-        else if (g.sh == 1 && g.sw == 1) hipLaunchKernelGGL((conv_bwd_data_smallc_kernel<true, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
+        else if (g.sh == 1 && g.sw == 1) hipLaunchKernelGGL(conv_bwd_data_smallc_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
         else {
             // one workgroup per 256 pixels of one (sample, residue class modulo the stride)
             const int Ht = (g.H + g.ph + g.sh - 1) / g.sh, Wt = (g.W + g.pw + g.sw - 1) / g.sw;

@@ -316,7 +316,20 @@ struct StoreNCHW {
     const float* bias; // optional, per output channel
     int opix;          // pixels of one output plane
     float* partial;    // split reductions: split ks writes its sums to partial[ks][same index], bias added by the reduction
-    __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int ks, const GemmDims& d) const {
+    static constexpr bool TAIL = true;
+    // tail mode: a split tile's sums go to partial[slot][row in tile][column in tile], slot = (tile, split)
+    __device__ __forceinline__ void store_tail(const floatx16 (&acc)[2][2], int wm0, int wn0, int lane, long slot, int TM, int TN) const {
+        const int l32 = lane & 31, lk = lane >> 5;
+        float* po = partial + slot * TM * TN;
+#pragma unroll
+        for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+            for (int it = 0; it < 2; it++)
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                    po[(wm0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4)) * TN + wn0 + jt * 32 + l32] = acc[it][jt][v];
+    }
+    __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int ks, const GemmDims& d, bool to_partial) const {
         const int l32 = lane & 31, lk = lane >> 5;
 #pragma unroll
         for (int jt = 0; jt < 2; jt++) {
@@ -333,7 +346,7 @@ struct StoreNCHW {
                     const int m = m0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
                     if (m >= d.M) continue;
                     float r = acc[it][jt][v];
-                    if (d.splits > 1) {
+                    if (to_partial) {
                         po[(size_t)m * opix] = r;
                     } else {
                         if (bias) r += bias[m];

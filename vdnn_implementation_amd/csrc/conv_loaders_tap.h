@@ -175,7 +175,9 @@ struct StoreFilterTap {
     float alpha;
     int accumulate;
     FastDiv divC;
-    __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int ks, const GemmDims& d) const {
+    static constexpr bool TAIL = false;
+    __device__ __forceinline__ void store_tail(const floatx16 (&)[2][2], int, int, int, long, int, int) const {}
+    __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int ks, const GemmDims& d, bool to_partial) const {
         const int l32 = lane & 31, lk = lane >> 5;
 #pragma unroll
         for (int jt = 0; jt < 2; jt++) {
@@ -191,7 +193,7 @@ struct StoreFilterTap {
                     if (m >= d.M) continue;
                     const long idx = (long)m * d.N + col;
                     const float a = acc[it][jt][v];
-                    if (d.splits > 1) partial[(long)ks * partial_stride + (long)m * d.N + j] = a;
+                    if (to_partial) partial[(long)ks * partial_stride + (long)m * d.N + j] = a;
                     else out[idx] = accumulate ? __fmaf_rn(alpha, a, out[idx]) : alpha * a;
                 }
         }

@@ -15,7 +15,8 @@ namespace vdnn {
 constexpr int SMALLC_KC = 8;
 constexpr int SMALLC_MAXTAPS = 128;
 
-template <bool STRIDE1, class E>
+// stride 1, any window
+template <class E>
 __global__ void __launch_bounds__(256) conv_bwd_data_smallc_kernel(const E* __restrict__ dy, const float* __restrict__ w,
                                                                    E* __restrict__ dx, const ConvGeo g) {
     __shared__ float4 ws[SMALLC_KC][SMALLC_MAXTAPS];
@@ -44,33 +45,16 @@ __global__ void __launch_bounds__(256) conv_bwd_data_smallc_kernel(const E* __re
         const int kmax = min(SMALLC_KC, g.K - k0);
         for (int kk = 0; kk < kmax; kk++) {
             const E* dyp = dy + ((long)n * g.K + k0 + kk) * g.P * g.Q;
-            if (STRIDE1) {
-                for (int r = 0; r < g.R; r++) {
-                    const int p = th - r;
-                    if ((unsigned)p >= (unsigned)g.P) continue;
-                    const E* row = dyp + (long)p * g.Q;
-                    for (int s = 0; s < g.S; s++) {
-                        const int q = tw - s;
-                        if ((unsigned)q >= (unsigned)g.Q) continue;
-                        const float d = load_elem(row + q);
-                        const float4 f = ws[kk][r * g.S + s];
-                        acc.x += d * f.x; acc.y += d * f.y; acc.z += d * f.z; acc.w += d * f.w;
-                    }
-                }
-            } else {
-                // only the taps congruent to the pixel's position modulo the stride reach an output:
-                // r = th mod sh, th mod sh + sh, ... (ascending, the order of the full scan)
-                for (int r = th % g.sh; r < g.R && r <= th; r += g.sh) {
-                    const int p = (th - r) / g.sh;
-                    if (p >= g.P) continue;
-                    const E* row = dyp + (long)p * g.Q;
-                    for (int s = tw % g.sw; s < g.S && s <= tw; s += g.sw) {
-                        const int q = (tw - s) / g.sw;
-                        if (q >= g.Q) continue;
-                        const float d = load_elem(row + q);
-                        const float4 f = ws[kk][r * g.S + s];
-                        acc.x += d * f.x; acc.y += d * f.y; acc.z += d * f.z; acc.w += d * f.w;
-                    }
+            for (int r = 0; r < g.R; r++) {
+                const int p = th - r;
+                if ((unsigned)p >= (unsigned)g.P) continue;
+                const E* row = dyp + (long)p * g.Q;
+                for (int s = 0; s < g.S; s++) {
+                    const int q = tw - s;
+                    if ((unsigned)q >= (unsigned)g.Q) continue;
+                    const float d = load_elem(row + q);
+                    const float4 f = ws[kk][r * g.S + s];
+                    acc.x += d * f.x; acc.y += d * f.y; acc.z += d * f.z; acc.w += d * f.w;
                 }
             }
         }

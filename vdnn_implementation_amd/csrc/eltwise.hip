@@ -189,6 +189,46 @@ int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const f
     return launch_reduce_splits_t(ctx, stream, out, partial, count, splits, alpha, accumulate, bias_j, ncols);
 }
 
+// tiles of a convolution result that were split (tail mode): out[n][m][pix] = sum over the tile's splits (+ bias[m]);
+// partial[(t*splits + ks)*TM*TN + row*TN + col] for the t-th split tile, tiles numbered m-tile fastest
+template <class E>
+__global__ void __launch_bounds__(EB) reduce_tail_nchw_kernel(E* __restrict__ out, const float* __restrict__ partial, int splits, int TM, int TN,
+                                                              int M, int N, int mtiles, int full_tiles, const float* __restrict__ bias, int opix, size_t total) {
+    const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
+    if (i >= total) return;
+    const int per = TM * TN;
+    const int t = (int)(i / per), local = (int)(i - (size_t)t * per);
+    const int row = local / TN, col = local - row * TN;
+    const int tile = full_tiles + t;
+    const int m = (tile % mtiles) * TM + row, j = (tile / mtiles) * TN + col;
+    if (m >= M || j >= N) return;
+    const float* p = partial + (size_t)t * splits * per + local;
+    float s = p[0];
+    for (int k = 1; k < splits; k++) s += p[(size_t)k * per];
+    if (bias) s += bias[m];
+    const int n = j / opix, pix = j - n * opix;
+    store_elem(out + ((size_t)n * M + m) * opix + pix, s);
+}
+
+template <class E>
+static int launch_reduce_tail_nchw_t(vdnn_ctx* ctx, hipStream_t stream, E* out, const float* partial, int tail_tiles, int splits, int TM, int TN,
+                                     int M, int N, int mtiles, int full_tiles, const float* bias, int opix) {
+    const size_t total = (size_t)tail_tiles * TM * TN;
+    ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)total * (splits + 1));
+    hipLaunchKernelGGL(reduce_tail_nchw_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
+                       out, partial, splits, TM, TN, M, N, mtiles, full_tiles, bias, opix, total);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+int launch_reduce_tail_nchw(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, int tail_tiles, int splits, int TM, int TN,
+                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix) {
+    return launch_reduce_tail_nchw_t(ctx, stream, out, partial, tail_tiles, splits, TM, TN, M, N, mtiles, full_tiles, bias, opix);
+}
+int launch_reduce_tail_nchw(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, int tail_tiles, int splits, int TM, int TN,
+                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix) {
+    return launch_reduce_tail_nchw_t(ctx, stream, out, partial, tail_tiles, splits, TM, TN, M, N, mtiles, full_tiles, bias, opix);
+}
+
 // filter gradient whose partial sums are in tap-major column order: out[m][c][tap] gets partial[.][m][tap*C + c]
 __global__ void __launch_bounds__(EB) reduce_splits_tap_kernel(float* __restrict__ out, const float* __restrict__ partial, size_t count,
                                                                int splits, float alpha, int accumulate, int C, int RS) {

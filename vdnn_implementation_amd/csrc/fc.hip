@@ -30,6 +30,7 @@ static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const char* name, const AL& al
     kchunk = (kchunk + KB - 1) / KB * KB;
     d.kchunk = kchunk;
     d.splits = (K + kchunk - 1) / kchunk;
+    d.full_tiles = 0;
     StoreDense<EO> ep{out, ctx->reduce_scratch, d.splits > 1 ? nullptr : bias_j, (long)N, (long)M * N, alpha, accumulate};
     const long blocks = (long)d.mtiles * d.ntiles * d.splits;
     ProfScope prof(ctx, st, name, 2.0 * M * (double)N * K, 0.0);

@@ -139,9 +139,12 @@ __device__ __forceinline__ floatx4 read_frag(const float* tile, int l32, int lk,
 }
 
 // Launch geometry of one igemm call. Split s covers reduction indices [s*kchunk, min(K, (s+1)*kchunk)).
+// full_tiles > 0 (tail mode): the first full_tiles tiles are computed whole by one workgroup each, only the
+// remaining tiles - the ones that would start a nearly empty last round - are split.
 struct GemmDims {
     int M, N, K;
     int mtiles, ntiles, splits, kchunk;
+    int full_tiles;
 };
 
 // Number of reduction splits for a grid of `tiles` output tiles over a reduction of K, at most
@@ -180,15 +183,23 @@ __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, con
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int bid = xcd_remap(blockIdx.x, gridDim.x);
     // m-tile fastest: workgroups that share a B tile (the large operand) are neighbours
-    const int mt = bid % d.mtiles;
-    const int rest = bid / d.mtiles;
-    const int nt = rest % d.ntiles;
-    const int ks = rest / d.ntiles;
+    const int ntiles_all = d.mtiles * d.ntiles;
+    int tile, ks;
+    bool whole;
+    if ((int)blockIdx.x < d.full_tiles) {
+        tile = xcd_remap(blockIdx.x, d.full_tiles); ks = 0; whole = true;
+    } else if (d.full_tiles > 0) {
+        const int r = blockIdx.x - d.full_tiles, tl = ntiles_all - d.full_tiles;
+        tile = d.full_tiles + r % tl; ks = r / tl; whole = false;
+    } else {
+        const int bid = xcd_remap(blockIdx.x, gridDim.x);
+        tile = bid % ntiles_all; ks = bid / ntiles_all; whole = d.splits == 1;
+    }
+    const int mt = tile % d.mtiles, nt = tile / d.mtiles;
     const int m0 = mt * TM, j0 = nt * TN;
-    const int k_begin = ks * d.kchunk;
-    const int k_end = min(d.K, k_begin + d.kchunk);
+    const int k_begin = whole ? 0 : ks * d.kchunk;
+    const int k_end = whole ? d.K : min(d.K, k_begin + d.kchunk);
 
     typename AL::template State<TM> sa;
     typename BL::template State<TN> sb;
@@ -277,7 +288,10 @@ __global__ void __launch_bounds__(NT) igemm_kernel(const AL al, const BL bl, con
         }
     }
 
-    ep.store(acc, m0 + wm0, j0 + wn0, lane, ks, d);
+    if (EP::TAIL && d.full_tiles > 0 && !whole)
+        ep.store_tail(acc, wm0, wn0, lane, (long)(tile - d.full_tiles) * d.splits + ks, TM, TN);
+    else
+        ep.store(acc, m0 + wm0, j0 + wn0, lane, ks, d, !whole);
 }
 
 // ---- dense reduction-major operand: element (row, kk) at base[row*ld + kk] -------------------------
@@ -384,7 +398,9 @@ struct StoreDense {
     long partial_stride; // elements per split
     float alpha;
     int accumulate;
-    __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int ks, const GemmDims& d) const {
+    static constexpr bool TAIL = false;
+    __device__ __forceinline__ void store_tail(const floatx16 (&)[2][2], int, int, int, long, int, int) const {}
+    __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int ks, const GemmDims& d, bool to_partial) const {
         const int l32 = lane & 31, lk = lane >> 5;
 #pragma unroll
         for (int jt = 0; jt < 2; jt++) {
@@ -398,7 +414,7 @@ struct StoreDense {
                     if (m >= d.M) continue;
                     const long idx = (long)m * ld_m + j;
                     const float a = acc[it][jt][v];
-                    if (d.splits > 1) {
+                    if (to_partial) {
                         partial[(long)ks * partial_stride + idx] = a;
                     } else {
                         // one fused multiply-add: every route to "out += alpha * sum" rounds the same way
