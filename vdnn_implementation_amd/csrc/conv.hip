@@ -304,6 +304,7 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     const int M = g.K, N = g.C * g.R * g.S, PQ = g.P * g.Q, RS = g.R * g.S;
     const long Kred = (long)g.N * PQ;
     VDNN_REQUIRE(Kred < (1l << 31), "reduction too long");
+    VDNN_REQUIRE((long)(PQ + KB) * PQ < (1l << 32), "output plane too large for the pixel cursor's exact division");
     if (g.C <= 4 && g.R == 3 && g.S == 3 && g.K % 4 == 0 && ctx->reduce_scratch) {
         // few input channels: vector-ALU kernel over chunks of output pixels, then the ordered chunk sum
         const long total = Kred;
@@ -350,19 +351,19 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     VDNN_REQUIRE(nspan * g.K * PQ * (long)sizeof(E) < (long)MAX_SUM_RANGE && nspan * g.C * g.H * g.W * (long)sizeof(E) < (long)MAX_SUM_RANGE,
                  "samples of one reduction split too large for one descriptor");
     StoreDense<float> ep{w, staging, nullptr, (long)N, (long)M * N, alpha, accumulate};
-    const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S), dQ = FastDiv::make(g.Q);
+    const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S), dQ = FastDiv::make(g.Q), dPQ = FastDiv::make(PQ);
     const bool vec = PQ % 4 == 0 && aligned16(dy); // bf16: four elements are 8 bytes, covered by the same test
     // tap-major column order when the tile's columns fall into whole groups of channels with one tap each
     const int tile_n = narrow ? 256 : 128;
     const int ntap = g.C % tile_n == 0 ? 1 : (g.C % (tile_n / 2) == 0 ? 2 : (g.C % (tile_n / 4) == 0 ? 4 : 0));
-    if (vec && ntap != 0) {
+    if (vec && ntap != 0 && PQ >= KB && 2 * g.Q >= KB) {
         const FastDiv dC = FastDiv::make(g.C);
         StoreFilterTap ept{w, staging, g.C, RS, (long)M * N, alpha, accumulate, dC};
-        LoadDyRed<true, E> al{dy, g.N, g.K, PQ, d.kchunk, d.K};
+        LoadDyRedInc<E> al{dy, g.N, g.K, PQ, d.kchunk, d.K};
         int rc2;
 #define VDNN_WGRAD_TAP(NTAP)                                                                                                \
         do {                                                                                                                \
-            LoadIm2colRedTap<NTAP, E> bl{x, g.N, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N, d.kchunk, d.K, dC, dS, dQ}; \
+            LoadIm2colRedTap<NTAP, E> bl{x, g.N, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N, d.kchunk, d.K, dC, dS}; \
             rc2 = narrow ? launch_igemm<64, 256>(ctx, st, kBwdFilterNames.t64, al, bl, ept, d)                               \
                          : launch_igemm<128, 128>(ctx, st, kBwdFilterNames.t128, al, bl, ept, d);                            \
         } while (0)
@@ -378,8 +379,8 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     int rc;
 #define VDNN_WGRAD(VEC, BIG)                                                                                              \
     do {                                                                                                                  \
-        LoadDyRed<VEC, E> al{dy, g.N, g.K, PQ, d.kchunk, d.K};                                                               \
-        LoadIm2colRed<BIG, E> bl{x, g.N, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N, d.kchunk, d.K, dRS, dS, dQ}; \
+        LoadDyRed<VEC, E> al{dy, g.N, g.K, PQ, d.kchunk, d.K, dPQ};                                                               \
+        LoadIm2colRed<BIG, E> bl{x, g.N, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N, d.kchunk, d.K, dRS, dS, dQ, dPQ}; \
         rc = conv_wgrad_with(ctx, st, al, bl, ep, d, narrow);                                                             \
     } while (0)
     if (vec && !big) VDNN_WGRAD(true, false);

@@ -162,20 +162,16 @@ struct LoadFilterT {
     }
 };
 
-// (n, pq) of a reduction index that advances by KB per slice
+// (n, pq) of a reduction index that advances by KB per slice. Branch-free for any plane size (a plane may
+// be smaller than a slice): the quotient comes from a multiply-high, so the tile loop stays one basic block.
 struct PixelCursor {
     int n, pq;
     __device__ __forceinline__ void init(int kk, int PQ, int n_first) { n = kk / PQ; pq = kk - n * PQ; n -= n_first; }
-    __device__ __forceinline__ void advance(int PQ) {
+    __device__ __forceinline__ void advance(int PQ, FastDiv divPQ) {
         pq += KB;
-        if (PQ >= KB) {
-            const bool wrap = pq >= PQ;
-            pq = wrap ? pq - PQ : pq;
-            n += wrap ? 1 : 0;
-        } else {
-            const int q = pq / PQ;
-            n += q; pq -= q * PQ;
-        }
+        const int q = divPQ.div(pq);
+        n += q;
+        pq -= q * PQ;
     }
 };
 
@@ -189,6 +185,7 @@ struct LoadDyRed {
     const E* dy;
     int N, K, PQ;
     int kchunk, Ktot; // reduction indices per split and in total
+    FastDiv divPQ;
     template <int T> struct Regs { floatx4 v[T / 64]; float s[VEC4 ? 1 : T / 16]; };
     template <int T> struct State { int mrow[VEC4 ? T / 64 : T / 16]; PixelCursor cur; int kk; __amdgpu_buffer_rsrc_t rsrc; };
     template <int T>
@@ -210,7 +207,8 @@ struct LoadDyRed {
     }
     template <int T>
     __device__ __forceinline__ void load(State<T>& st, int, int kend, int, Regs<T>& r) const {
-        const int npart = st.kk < kend ? (st.cur.n * K * PQ + st.cur.pq) * ES : SENT;
+        // the marker is OR-ed in (offsets stay below SENT) so that nothing here tempts the compiler into a branch
+        const int npart = ((st.cur.n * K * PQ + st.cur.pq) * ES) | (st.kk < kend ? 0 : SENT);
         if (VEC4) {
 #pragma unroll
             for (int i = 0; i < T / 64; i++) r.v[i] = buf_load4_e<E>(st.rsrc, st.mrow[i] + npart, 0);
@@ -219,7 +217,7 @@ struct LoadDyRed {
             for (int i = 0; i < T / 16; i++) r.s[i] = buf_load_e<E>(st.rsrc, st.mrow[i] + npart, 0);
         }
         st.kk += KB;
-        st.cur.advance(PQ);
+        st.cur.advance(PQ, divPQ);
     }
     template <int T>
     __device__ static __forceinline__ void store(float* lds, int tid, const Regs<T>& r) {
@@ -230,6 +228,48 @@ struct LoadDyRed {
 #pragma unroll
             for (int i = 0; i < T / 16; i++) lds[((tid >> 4) + 16 * i) * RED_STRIDE + (tid & 15)] = r.s[i];
         }
+    }
+};
+
+// The same operand with 128-bit chunks and a byte offset that is carried from slice to slice with adds and
+// selects (no integer multiply in the loop). Needs P*Q >= KB (at most one sample wrap per step), P*Q a
+// multiple of four and 16-byte aligned planes.
+template <class E = float>
+struct LoadDyRedInc {
+    static constexpr bool RED_MAJOR = true;
+    static constexpr int ES = ElemBytes<E>::V;
+    const E* dy;
+    int N, K, PQ;
+    int kchunk, Ktot;
+    template <int T> struct Regs { floatx4 v[T / 64]; };
+    // Pixels past the end of the reduction lie in the sample after the descriptor's range and read as zero.
+    template <int T> struct State { int mrow[T / 64]; int pq, off; __amdgpu_buffer_rsrc_t rsrc; };
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int row0, int tid, int, int k_begin) const {
+        const int n_first = k_begin / PQ;
+        int k_last = k_begin + kchunk; if (k_last > Ktot) k_last = Ktot;
+        const int n_last = k_last > k_begin ? (k_last - 1) / PQ : n_first;
+        st.rsrc = make_rsrc(dy + (long)n_first * K * PQ, clamp_range((long)(n_last - n_first + 1) * K * PQ * ES));
+        const int kk = k_begin + 4 * (tid & 3);
+        const int n = kk / PQ;
+        st.pq = kk - n * PQ;
+        st.off = (int)(((long)(n - n_first) * K * PQ + st.pq) * ES);
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) { const int m = row0 + (tid >> 2) + 64 * i; st.mrow[i] = m < K ? m * PQ * ES : SENT; }
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int, int, int, Regs<T>& r) const {
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) r.v[i] = buf_load4_e<E>(st.rsrc, st.mrow[i] + st.off, 0);
+        st.pq += KB;
+        const bool wrap = st.pq >= PQ;
+        st.pq -= wrap ? PQ : 0;
+        st.off += wrap ? (KB + (K - 1) * PQ) * ES : KB * ES;
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(float* lds, int tid, const Regs<T>& r) {
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) *(floatx4*)(lds + ((tid >> 2) + 64 * i) * RED_STRIDE + 4 * (tid & 3)) = r.v[i];
     }
 };
 
@@ -244,7 +284,7 @@ struct LoadIm2colRed {
     int N, C, H, W, R, S, P, Q, ph, pw, sh, sw;
     int ncols; // C*R*S
     int kchunk, Ktot; // reduction indices per split and in total
-    FastDiv divRS, divS, divQ;
+    FastDiv divRS, divS, divQ, divPQ;
     template <int T> struct Regs { float s[T / 16]; };
     template <int T> struct State {
         int jconst[T / 16]; // byte offset of (c*H*W + r*W + s), or SENT for a column outside the matrix
@@ -282,7 +322,7 @@ struct LoadIm2colRed {
         const int PQ = P * Q;
         const int p = divQ.div(st.cur.pq), q = st.cur.pq - p * Q;
         const int ih0 = p * sh - ph, iw0 = q * sw - pw;
-        const int pixbase = st.kk < kend ? (st.cur.n * C * H * W + p * sh * W + q * sw) * ES : SENT;
+        const int pixbase = ((st.cur.n * C * H * W + p * sh * W + q * sw) * ES) | (st.kk < kend ? 0 : SENT);
         const unsigned vrow = valid_window_bits(ih0, R, H), vcol = valid_window_bits(iw0, S, W);
         if (BIGWIN) {
             const unsigned invrow = ~vrow, invcol = ~vcol;
@@ -300,7 +340,7 @@ struct LoadIm2colRed {
                 r.s[i] = buf_load_e<E>(st.rsrc, (pixbase + st.jconst[i]) | bit_to_all_ones(inv, st.tap[i]), 0);
         }
         st.kk += KB;
-        st.cur.advance(PQ);
+        st.cur.advance(PQ, divPQ);
     }
     template <int T>
     __device__ static __forceinline__ void store(float* lds, int tid, const Regs<T>& r) {

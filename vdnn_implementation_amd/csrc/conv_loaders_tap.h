@@ -105,13 +105,21 @@ struct LoadIm2colRedTap {
     int N, C, H, W, R, S, P, Q, ph, pw, sh, sw;
     int ncols; // C*R*S
     int kchunk, Ktot;
-    FastDiv divC, divS, divQ;
+    FastDiv divC, divS;
     template <int T> struct Regs { float s[T / 16]; };
+    // The vector unit is shared with the MFMAs, so the per-slice address work is kept to adds, compares
+    // and selects on three carried quantities: the input row and column the thread's pixel reads through
+    // the first group's tap, and the byte offset of that element in the thread's first channel plane.
+    // A slice moves the pixel KB places along (n, p, q); up to two row wraps (Q >= KB/2) and one sample
+    // wrap (P*Q >= KB) are applied without branches. Pixels past the end of the reduction lie in the
+    // sample after the descriptor's range and read as zero, as do the matching values of the other
+    // operand, so no liveness test is needed; the columns of a group are whole channel planes apart
+    // (scalar offsets of the load instructions).
     template <int T> struct State {
-        int cconst[T / 16];  // byte offset of the column's channel plane, or SENT outside the matrix
-        int tapoff[NTAP];    // byte offset of the group's tap (r*W + s), wave-uniform
-        int tr[NTAP], ts[NTAP];
-        PixelCursor cur; int kk;
+        int ih, iw;          // p*sh - ph + r0, q*sw - pw + s0 for the first group's tap (r0, s0)
+        int off;             // byte offset of (n, c_thread, ih, iw) from the descriptor base
+        int dih[NTAP], diw[NTAP], doff[NTAP]; // further groups relative to the first (wave-uniform)
+        int iw_wrap, ih_wrap; // values of iw / ih at which the row / the sample ends
         __amdgpu_buffer_rsrc_t rsrc;
     };
     template <int T>
@@ -123,39 +131,50 @@ struct LoadIm2colRedTap {
         int k_last = k_begin + kchunk; if (k_last > Ktot) k_last = Ktot;
         const int n_last = k_last > k_begin ? (k_last - 1) / PQ : n_first;
         st.rsrc = make_rsrc(x + (long)n_first * chw + shift, clamp_range(((long)(n_last - n_first + 1) * chw - shift) * ES));
-        st.kk = k_begin + (tid & 15);
-        st.cur.init(st.kk, PQ, n_first);
+        const int kk = k_begin + (tid & 15);
+        const int n = kk / PQ, pq = kk - n * PQ;
+        const int p = pq / Q, q = pq - p * Q;
+        int r0 = 0, s0 = 0, c0 = 0;
 #pragma unroll
         for (int g = 0; g < NTAP; g++) {
-            const int tap = divC.div(j0 + g * (T / NTAP)); // one tap per group of T/NTAP columns
+            const int jg = j0 + g * (T / NTAP);           // one tap per group of T/NTAP columns
+            const int tap = divC.div(jg);
             const int r = divS.div(tap), s_ = tap - r * S;
-            st.tr[g] = r; st.ts[g] = s_;
-            st.tapoff[g] = (r * W + s_) * ES;
+            const int c = jg - tap * C;
+            if (g == 0) { r0 = r; s0 = s_; c0 = c; st.dih[0] = 0; st.diw[0] = 0; st.doff[0] = 0; }
+            else {
+                st.dih[g] = jg < ncols ? r - r0 : 0x20000000; // a group past the last tap never passes the row test
+                st.diw[g] = s_ - s0;
+                st.doff[g] = (((r - r0) * W + (s_ - s0)) + (c - c0) * H * W) * ES;
+            }
         }
-#pragma unroll
-        for (int i = 0; i < T / 16; i++) {
-            const int j = j0 + (tid >> 4) + 16 * i;
-            const int tap = divC.div(j);
-            st.cconst[i] = j < ncols ? (j - tap * C) * H * W * ES : SENT;
-        }
+        st.ih = p * sh - ph + r0; st.iw = q * sw - pw + s0;
+        st.iw_wrap = Q * sw - pw + s0; st.ih_wrap = P * sh - ph + r0;
+        st.off = (int)(((long)(n - n_first) * chw + (long)(c0 + (tid >> 4)) * H * W + (long)(p * sh + r0) * W + q * sw + s0) * ES);
     }
     template <int T>
-    __device__ __forceinline__ void load(State<T>& st, int, int kend, int, Regs<T>& r) const {
-        const int PQ = P * Q;
-        const int p = divQ.div(st.cur.pq), q = st.cur.pq - p * Q;
-        const int ih0 = p * sh - ph, iw0 = q * sw - pw;
-        const int pixoff = (st.cur.n * C * H * W + p * sh * W + q * sw) * ES;
-        const bool live = st.kk < kend;
+    __device__ __forceinline__ void load(State<T>& st, int, int, int, Regs<T>& r) const {
         int base[NTAP];
 #pragma unroll
         for (int g = 0; g < NTAP; g++) {
-            const bool ok = live & ((unsigned)(ih0 + st.tr[g]) < (unsigned)H) & ((unsigned)(iw0 + st.ts[g]) < (unsigned)W);
-            base[g] = ok ? pixoff + st.tapoff[g] : SENT;
+            const bool ok = g == 0 ? ((unsigned)st.ih < (unsigned)H) & ((unsigned)st.iw < (unsigned)W)
+                                   : ((unsigned)(st.ih + st.dih[g]) < (unsigned)H) & ((unsigned)(st.iw + st.diw[g]) < (unsigned)W);
+            base[g] = (g == 0 ? st.off : st.off + st.doff[g]) | (ok ? 0 : SENT);
         }
+        constexpr int PERG = T / 16 / NTAP;
+        const int plane16 = 16 * H * W * ES;
 #pragma unroll
-        for (int i = 0; i < T / 16; i++) r.s[i] = buf_load_e<E>(st.rsrc, base[i / (T / 16 / NTAP)] + st.cconst[i], 0);
-        st.kk += KB;
-        st.cur.advance(PQ);
+        for (int i = 0; i < T / 16; i++) r.s[i] = buf_load_e<E>(st.rsrc, base[i / PERG], (i % PERG) * plane16);
+        // next slice: KB pixels further
+        st.iw += KB * sw; st.off += KB * sw * ES;
+        const int qsw = Q * sw;
+        const int wraps = (st.iw >= st.iw_wrap ? 1 : 0) + (st.iw >= st.iw_wrap + qsw ? 1 : 0);
+        st.iw -= __mul24(wraps, qsw);
+        st.ih += __mul24(wraps, sh);
+        st.off += __mul24(wraps, (sh * W - qsw) * ES);
+        const bool next = st.ih >= st.ih_wrap;                // into the next sample
+        st.ih -= next ? P * sh : 0;
+        st.off += next ? (C * H * W - P * sh * W) * ES : 0;
     }
     template <int T>
     __device__ static __forceinline__ void store(float* lds, int tid, const Regs<T>& r) {
