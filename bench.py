@@ -39,9 +39,10 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0, bf16=False, offload_lag=0, prefetch_depth=1):
+def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0, bf16=False, offload_lag=0, prefetch_depth=1,
+               fuse=False):
     net = Network(cnn, policy, algo, batch, seed=seed, refined=refined, cap_bytes=cap_bytes, bf16=bf16,
-                  offload_lag=offload_lag, prefetch_depth=prefetch_depth)
+                  offload_lag=offload_lag, prefetch_depth=prefetch_depth, fuse=fuse)
     try:
         for _ in range(warmup):
             assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
@@ -75,6 +76,10 @@ def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refin
         # step = kernels + copies - overlap + idle  =>  overlap >= kernels + copies - step
         res["overlap_fraction_lower_bound"] = max(0.0, min(1.0, (kernel_ms + copy_ms - dt * 1e3) / copy_ms))
     return res, prof
+
+
+def is_bf16(policy_name):
+    return "bf16" in policy_name.split("+")[1:]
 
 
 def best_offloading(results, base):
@@ -114,7 +119,9 @@ def main():
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--algo", default="VDNN_MEMORY_OPT_ALGO")
     ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined,VDNN_CONV+refined+slack,"
-                    "BASELINE+bf16,VDNN_ALL+bf16,VDNN_CONV+refined+slack+bf16,VDNN_ALL+refined+slack+bf16")
+                    "BASELINE+fused,VDNN_CONV+refined+slack+fused,"
+                    "BASELINE+bf16,VDNN_ALL+bf16,VDNN_CONV+refined+slack+bf16,VDNN_ALL+refined+slack+bf16,"
+                    "BASELINE+bf16+fused,VDNN_CONV+refined+slack+bf16+fused")
     ap.add_argument("--cap-gb", type=float, default=0.0, help="artificial limit on pool bytes in use (0 = none)")
     ap.add_argument("--bf16", action="store_true", help="bfloat16 activation storage (float parameters and arithmetic)")
     ap.add_argument("--offload-lag", type=int, default=0, help="layers enqueued before an offloaded block is recycled (0 = reference schedule)")
@@ -134,15 +141,17 @@ def main():
     results, profiles = {}, {}
     for name in args.policies.split(","):
         # suffixes: "+refined" = the value-preserving lifetime refinements; "+slack" = blocks recycled six layers
-        # after their offload and two tensors fetched ahead; "+bf16" = bfloat16 activation storage
+        # after their offload and two tensors fetched ahead; "+bf16" = bfloat16 activation storage; "+fused" = ReLU
+        # layers run inside the neighbouring layers' kernels
         word, *mods = name.split("+")
-        assert set(mods) <= {"refined", "slack", "bf16"}, name
+        assert set(mods) <= {"refined", "slack", "bf16", "fused"}, name
         _, policy, algo = parse("VGG16_128", word, args.algo)
         lag, depth = (6, 2) if "slack" in mods else (args.offload_lag, args.prefetch_depth)
         log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
         results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1,
                                                    refined=("refined" in mods), cap_bytes=int(args.cap_gb * 1e9),
-                                                   bf16=(args.bf16 or "bf16" in mods), offload_lag=lag, prefetch_depth=depth)
+                                                   bf16=(args.bf16 or "bf16" in mods), offload_lag=lag, prefetch_depth=depth,
+                                                   fuse=("fused" in mods))
         log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
             results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))
 
@@ -152,7 +161,7 @@ def main():
     # policies of this run (the same launches a kernel trace of this command sees, warm-up aside)
     prof = {}
     for pname, p in profiles.items():
-        if pname.endswith("+bf16") != args.bf16:
+        if is_bf16(pname) != args.bf16:
             continue  # the roofline entry is taken over the runs of the headline element type
         for k, v in p.items():
             acc = prof.setdefault(k, {"launches": 0, "ms": 0.0, "flops": 0.0, "bytes": 0.0})
@@ -182,8 +191,8 @@ def main():
         if base and "VDNN_ALL+refined" in results else None,
         "refined_peak_hbm_reduction_vs_baseline": (base["peak_hbm_gb"] / results["VDNN_ALL+refined"]["peak_hbm_gb"])
         if base and "VDNN_ALL+refined" in results else None,
-        "losses_bit_identical": len({results[k]["loss"] for k in results if not k.endswith("+bf16")}) <= 1
-        and len({results[k]["loss"] for k in results if k.endswith("+bf16")}) <= 1,
+        "losses_bit_identical": len({results[k]["loss"] for k in results if not is_bf16(k)}) <= 1
+        and len({results[k]["loss"] for k in results if is_bf16(k)}) <= 1,
         "best_offloading_vs_fp32_baseline": best_offloading(results, base),
         "conv_mfma_util": conv_all_tf / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",

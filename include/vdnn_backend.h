@@ -159,6 +159,27 @@ int vdnn_conv_bwd_filter(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
                          const void* x, const void* dy, float* dw, void* workspace, size_t workspace_bytes);
 int vdnn_sgd_apply(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float alpha, const float* grad, float* param);
 
+/* ---- layers fused with the rectifier next to them ------------------------------------------------
+ * The reference runs every ReLU as a layer of its own (cudnnActivationForward / Backward, layer.cu:766-814),
+ * which reads and writes the whole tensor once more. These entry points apply it where the tensor is
+ * produced instead; each gives the bits of the two separate calls it stands for.
+ *   vdnn_conv_fwd_relu / vdnn_fc_fwd_relu:  y = relu(layer(x))            = vdnn_conv_fwd, then vdnn_relu_fwd
+ *   vdnn_conv_bwd_data_relu / vdnn_fc_bwd_data_relu / vdnn_maxpool_bwd_relu:
+ *       dx = (x > 0) ? layer_backward(dy) : 0, where x is the layer's own input and the output of a ReLU
+ *                                                                         = the layer's backward, then vdnn_relu_bwd */
+int vdnn_conv_fwd_relu(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                       const void* x, const float* w, const float* bias, void* y,
+                       void* workspace, size_t workspace_bytes);
+int vdnn_conv_bwd_data_relu(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                            const void* dy, const float* w, const void* x, void* dx,
+                            void* workspace, size_t workspace_bytes);
+int vdnn_fc_fwd_relu(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                     const void* x, const float* w, const float* bias, void* y);
+int vdnn_fc_bwd_data_relu(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                          const void* dy, const float* w, const void* x, void* dx);
+int vdnn_maxpool_bwd_relu(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape,
+                          const void* x, const void* y, const void* dy, void* dx);
+
 /* ---- fully connected (replaces cuBLAS: layer.cu:667-764) ------------------------------------- */
 /* Sgemm(T,N) + rank-1 bias broadcast (layer.cu:677-706): y[n,o] = sum_i w[o,i] x[n,i] + bias[o].
  * w is [c_out][c_in] row-major. */

@@ -30,6 +30,7 @@ typedef struct {
     int      offload_lag;       /* layers enqueued before an offloaded block is recycled (0 = the reference's schedule) */
     int      prefetch_depth;    /* offloaded tensors fetched ahead of their backward (1 = the reference's schedule) */
     int      data_type;         /* element type of activation tensors: VDNN_DTYPE_F32 (the reference, vdnn.h:11-12) or VDNN_DTYPE_BF16 */
+    int      fuse_activations;  /* a ReLU after a CONV / FC layer runs inside the neighbouring layers' kernels (same bits, layer.cu:766-814) */
 } vdnn_network_options;
 
 typedef struct {

@@ -386,3 +386,36 @@ def test_tables_agree_with_the_checker():
                 assert net.specs[l].type == o.desc[l].type
                 assert net.src_shape(l) == o.src_shape(l) and net.dst_shape(l) == o.dst_shape(l)
         o.close()
+
+
+def test_fused_rectifiers_own_no_tensor_and_leak_nothing():
+    """fuse: a ReLU behind a CONV / FC layer has no output block (its layer is elided), is never offloaded, and
+    every policy still returns all blocks. VGG16 batch 128: BASELINE keeps 6.94 GB less (the 15 ReLU outputs),
+    VDNN_ALL moves the bytes of the refined schedule (the ReLU inputs are not tensors of their own)."""
+    with plan(VGG16_128, BASELINE) as net:
+        step(net)
+        base = net.stats()["peak_bytes_in_use"]
+    with plan(VGG16_128, BASELINE, fuse=True) as net:
+        step(net)
+        relu_out = sum(int(np.prod(net.dst_shape(l))) * 4 for l, s in enumerate(net.specs) if s.type == enums.RELU)
+        assert net.stats()["peak_bytes_in_use"] == base - relu_out
+        assert abs(relu_out / GB - 6.94) < 0.01
+    with plan(VGG16_128, VDNN_ALL, refined=True) as net:
+        step(net)
+        ref = net.stats()
+    for policy, kw in ((VDNN_NONE, {}), (VDNN_CONV, {}), (VDNN_ALL, {}), (VDNN_ALL, {"refined": True}),
+                       (VDNN_CONV, {"refined": True, "offload_lag": 6, "prefetch_depth": 2})):
+        with plan(VGG16_128, policy, fuse=True, **kw) as net:
+            n0 = C.c_size_t()
+            lib.vdnn_pool_live_blocks(net.context, C.byref(n0))
+            step(net)
+            step(net)
+            n1 = C.c_size_t()
+            lib.vdnn_pool_live_blocks(net.context, C.byref(n1))
+            assert n1.value == n0.value
+            st = net.stats()
+            assert not any(net.is_offloaded(l) for l, s in enumerate(net.specs) if s.type == enums.RELU)
+            if policy == VDNN_ALL:
+                assert st["offload_bytes"] == st["prefetch_bytes"] == ref["offload_bytes"]
+                if kw.get("refined"):
+                    assert st["peak_bytes_in_use"] <= ref["peak_bytes_in_use"]

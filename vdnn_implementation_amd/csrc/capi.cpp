@@ -20,6 +20,7 @@ static NetworkOptions to_options(const vdnn_network_options* o) {
     n.prefetchDepth = o->prefetch_depth < 1 ? 1 : o->prefetch_depth;
     n.unfusedOptimizer = o->unfused_optimizer != 0;
     n.deferOptimizer = o->defer_optimizer != 0;
+    n.fuseActivations = o->fuse_activations != 0;
     return n;
 }
 
@@ -29,7 +30,7 @@ void vdnn_network_default_options(vdnn_network_options* o) {
     if (!o) return;
     NetworkOptions d;
     o->seed = d.seed; o->pool_bytes = 0; o->cap_bytes = 0; o->plan_only = 0; o->host_sync = 0;
-    o->capture = 0; o->verbose = 0; o->device = d.device; o->refined_lifetimes = 0; o->unfused_optimizer = 0; o->defer_optimizer = 0; o->data_type = VDNN_DTYPE_F32; o->offload_lag = 0; o->prefetch_depth = 1;
+    o->capture = 0; o->verbose = 0; o->device = d.device; o->refined_lifetimes = 0; o->unfused_optimizer = 0; o->defer_optimizer = 0; o->data_type = VDNN_DTYPE_F32; o->offload_lag = 0; o->prefetch_depth = 1; o->fuse_activations = 0;
 }
 
 vdnn_network* vdnn_network_create(int cnn, int policy, int algo, int batch, const vdnn_network_options* o) {

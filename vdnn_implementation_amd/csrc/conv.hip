@@ -77,15 +77,15 @@ static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, con
 }
 
 int launch_reduce_tail_nchw(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, int tail_tiles, int splits, int TM, int TN,
-                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix);
+                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix, int relu, const float* gate);
 int launch_reduce_tail_nchw(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, int tail_tiles, int splits, int TM, int TN,
-                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix);
+                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix, int relu, const bf16_t* gate);
 int launch_reduce_splits_tap(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
                              float alpha, int accumulate, int C, int RS);
 int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
-                              const float* bias, int opix, int channels);
+                              const float* bias, int opix, int channels, int relu, const float* gate);
 int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, size_t count, int splits,
-                              const float* bias, int opix, int channels);
+                              const float* bias, int opix, int channels, int relu, const bf16_t* gate);
 
 // Forward / backward data. Tile shape by output-row count: 64-row tiles for narrow layers, 128
 // otherwise. A grid that cannot fill the chip (few output pixels: the fully connected layers written
@@ -127,19 +127,19 @@ static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names
                           : launch_igemm<128, 128>(ctx, stream, names.t128, al, bl, ep, d, flops);
     if (rc != VDNN_OK || d.splits == 1) return rc;
     if (tail_tiles > 0)
-        return launch_reduce_tail_nchw(ctx, stream, ep.out, ep.partial, tail_tiles, d.splits, TM, TN, M, N, d.mtiles, d.full_tiles, ep.bias, ep.opix);
-    return launch_reduce_splits_nchw(ctx, stream, ep.out, ep.partial, (size_t)M * N, d.splits, ep.bias, ep.opix, M);
+        return launch_reduce_tail_nchw(ctx, stream, ep.out, ep.partial, tail_tiles, d.splits, TM, TN, M, N, d.mtiles, d.full_tiles, ep.bias, ep.opix, ep.relu, ep.gate);
+    return launch_reduce_splits_nchw(ctx, stream, ep.out, ep.partial, (size_t)M * N, d.splits, ep.bias, ep.opix, M, ep.relu, ep.gate);
 }
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
-                         int splits, float alpha, int accumulate, const float* bias_j, int ncols);
+                         int splits, float alpha, int accumulate, const float* bias_j, int ncols, int relu = 0, const float* gate = nullptr);
 
 // forward with the given A loader (128-bit or 32-bit filter loads)
 template <class AL, class E>
-static int conv_fwd_with(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const AL& al, const E* x, const float* bias, E* y) {
-    StoreNCHW<E> ep{y, bias, g.P * g.Q, ctx->reduce_scratch};
+static int conv_fwd_with(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const AL& al, const E* x, const float* bias, E* y, int relu) {
+    StoreNCHW<E> ep{y, bias, g.P * g.Q, ctx->reduce_scratch, relu, nullptr};
     const int M = g.K, N = g.N * g.P * g.Q, K = g.C * g.R * g.S;
     const FastDiv dRS = FastDiv::make(g.R * g.S), dS = FastDiv::make(g.S);
     if (g.R * g.S <= 32) {
@@ -188,12 +188,14 @@ using namespace vdnn;
 template <class E>
 static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
                          const E* x, const float* w, const float* bias, E* y,
-                         void* workspace, size_t workspace_bytes) {
+                         void* workspace, size_t workspace_bytes, int relu) {
     VDNN_KERNEL_PROLOGUE(ctx);
     ConvGeo g;
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(x && w && y, "null tensor");
-    if (is_dense(g)) return vdnn_fc_fwd(ctx, stream, g.N, g.C * g.H * g.W, g.K, x, w, bias, y);
+    if (is_dense(g))
+        return relu ? vdnn_fc_fwd_relu(ctx, stream, g.N, g.C * g.H * g.W, g.K, x, w, bias, y)
+                    : vdnn_fc_fwd(ctx, stream, g.N, g.C * g.H * g.W, g.K, x, w, bias, y);
     VDNN_REQUIRE(pixel_tile_span_ok((long)g.C * g.H * g.W, g.P * g.Q, 256, (int)sizeof(E)), "input samples too large for one tile's descriptor");
     hipStream_t st = stream_of(ctx, stream);
     const int K = g.C * g.R * g.S;
@@ -203,7 +205,7 @@ static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
         const int RS = g.R * g.S;
         LoadIm2colPixTap<0, E> bl{{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N,
                                 FastDiv::make(RS), FastDiv::make(g.S)}};
-        StoreNCHW<E> ep{y, bias, g.P * g.Q, ctx->reduce_scratch};
+        StoreNCHW<E> ep{y, bias, g.P * g.Q, ctx->reduce_scratch, relu, nullptr};
         if (algo_mode == 1 && workspace && workspace_bytes >= wbytes && aligned16(workspace)) {
             // perf-optimal: the filter bank, re-laid-out in the workspace, is a dense 128-bit operand
             float* packed = (float*)workspace;
@@ -217,23 +219,25 @@ static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
     }
     if (K % 4 == 0 && aligned16(w)) {
         LoadDenseRed<true> al{w, (long)K, g.K, wbytes};
-        return conv_fwd_with(ctx, st, g, al, x, bias, y);
+        return conv_fwd_with(ctx, st, g, al, x, bias, y, relu);
     }
     LoadDenseRed<false> al{w, (long)K, g.K, wbytes};
-    return conv_fwd_with(ctx, st, g, al, x, bias, y);
+    return conv_fwd_with(ctx, st, g, al, x, bias, y, relu);
 }
 
 template <class E>
 static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
                               const E* dy, const float* w, E* dx,
-                              void* workspace, size_t workspace_bytes) {
+                              void* workspace, size_t workspace_bytes, const E* gate) {
     VDNN_KERNEL_PROLOGUE(ctx);
     ConvGeo g;
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(dy && w && dx, "null tensor");
-    if (is_dense(g)) return vdnn_fc_bwd_data(ctx, stream, g.N, g.C * g.H * g.W, g.K, dy, w, dx);
+    if (is_dense(g))
+        return gate ? vdnn_fc_bwd_data_relu(ctx, stream, g.N, g.C * g.H * g.W, g.K, dy, w, gate, dx)
+                    : vdnn_fc_bwd_data(ctx, stream, g.N, g.C * g.H * g.W, g.K, dy, w, dx);
     hipStream_t st = stream_of(ctx, stream);
-    if (g.C <= 4 && g.R * g.S <= SMALLC_MAXTAPS) {
+    if (g.C <= 4 && g.R * g.S <= SMALLC_MAXTAPS && !gate) { // the vector-ALU kernels have no gated store
         const long total = (long)g.N * g.H * g.W;
         const long blocks = (total + 255) / 256;
         VDNN_REQUIRE(blocks < (1l << 31), "grid too large");
@@ -256,7 +260,7 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
     VDNN_REQUIRE(pixel_tile_span_ok((long)g.K * g.P * g.Q, g.H * g.W, 256, (int)sizeof(E)), "output-gradient samples too large for one tile's descriptor");
     const int RS = g.R * g.S;
     LoadFilterT al{w, g.C, RS, (unsigned)((long)g.K * g.C * RS * 4), FastDiv::make(RS)};
-    StoreNCHW<E> ep{dx, nullptr, g.H * g.W, ctx->reduce_scratch};
+    StoreNCHW<E> ep{dx, nullptr, g.H * g.W, ctx->reduce_scratch, 0, gate};
     const int M = g.C, N = g.N * g.H * g.W, K = g.K * RS;
     const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S);
     const long sample = (long)g.K * g.P * g.Q;
@@ -422,15 +426,30 @@ size_t vdnn_conv_workspace_bytes(const vdnn_shape_t* shape, int algo_mode, int p
 int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
                   const void* x, const float* w, const float* bias, void* y,
                   void* workspace, size_t workspace_bytes) {
-    return VDNN_BY_ACT(ctx, conv_fwd_impl<float>(ctx, stream, shape, algo_mode, (const float*)x, w, bias, (float*)y, workspace, workspace_bytes),
-                       conv_fwd_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)x, w, bias, (bf16_t*)y, workspace, workspace_bytes));
+    return VDNN_BY_ACT(ctx, conv_fwd_impl<float>(ctx, stream, shape, algo_mode, (const float*)x, w, bias, (float*)y, workspace, workspace_bytes, 0),
+                       conv_fwd_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)x, w, bias, (bf16_t*)y, workspace, workspace_bytes, 0));
+}
+
+int vdnn_conv_fwd_relu(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                       const void* x, const float* w, const float* bias, void* y,
+                       void* workspace, size_t workspace_bytes) {
+    return VDNN_BY_ACT(ctx, conv_fwd_impl<float>(ctx, stream, shape, algo_mode, (const float*)x, w, bias, (float*)y, workspace, workspace_bytes, 1),
+                       conv_fwd_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)x, w, bias, (bf16_t*)y, workspace, workspace_bytes, 1));
 }
 
 int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
                        const void* dy, const float* w, void* dx,
                        void* workspace, size_t workspace_bytes) {
-    return VDNN_BY_ACT(ctx, conv_bwd_data_impl<float>(ctx, stream, shape, algo_mode, (const float*)dy, w, (float*)dx, workspace, workspace_bytes),
-                       conv_bwd_data_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)dy, w, (bf16_t*)dx, workspace, workspace_bytes));
+    return VDNN_BY_ACT(ctx, conv_bwd_data_impl<float>(ctx, stream, shape, algo_mode, (const float*)dy, w, (float*)dx, workspace, workspace_bytes, nullptr),
+                       conv_bwd_data_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)dy, w, (bf16_t*)dx, workspace, workspace_bytes, nullptr));
+}
+
+int vdnn_conv_bwd_data_relu(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                            const void* dy, const float* w, const void* x, void* dx,
+                            void* workspace, size_t workspace_bytes) {
+    VDNN_REQUIRE(x != nullptr, "null input tensor");
+    return VDNN_BY_ACT(ctx, conv_bwd_data_impl<float>(ctx, stream, shape, algo_mode, (const float*)dy, w, (float*)dx, workspace, workspace_bytes, (const float*)x),
+                       conv_bwd_data_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)dy, w, (bf16_t*)dx, workspace, workspace_bytes, (const bf16_t*)x));
 }
 
 int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,

@@ -356,6 +356,8 @@ struct StoreNCHW {
     const float* bias; // optional, per output channel
     int opix;          // pixels of one output plane
     float* partial;    // split reductions: split ks writes its sums to partial[ks][same index], bias added by the reduction
+    int relu;          // rectify the result (after the bias)
+    const E* gate;     // optional, same layout as out: the result is kept where gate > 0 and zero elsewhere
     static constexpr bool TAIL = true;
     // tail mode: a split tile's sums go to partial[slot][row in tile][column in tile], slot = (tile, split)
     __device__ __forceinline__ void store_tail(const floatx16 (&acc)[2][2], int wm0, int wn0, int lane, long slot, int TM, int TN) const {
@@ -390,6 +392,8 @@ struct StoreNCHW {
                         po[(size_t)m * opix] = r;
                     } else {
                         if (bias) r += bias[m];
+                        if (relu) r = relu_value(r);
+                        if (gate) r = load_elem(gate + base + (size_t)m * opix) > 0.0f ? r : 0.0f;
                         store_elem(o + (size_t)m * opix, r);
                     }
                 }

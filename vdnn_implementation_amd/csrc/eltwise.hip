@@ -73,17 +73,16 @@ __device__ __forceinline__ void st2(bf16_t* p, float2 v) {
 }
 
 // ---- ReLU ---------------------------------------------------------------------------------------
-__device__ __forceinline__ float relu1(float v) { return v > 0.0f ? v : (v != v ? v : 0.0f); }
 
 template <class E>
 __global__ void __launch_bounds__(EB) relu_fwd_kernel(const E* __restrict__ x, E* __restrict__ y, size_t n4, size_t n) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < n4; i += stride) {
         float4 v = ld4(x + 4 * i);
-        v.x = relu1(v.x); v.y = relu1(v.y); v.z = relu1(v.z); v.w = relu1(v.w);
+        v.x = relu_value(v.x); v.y = relu_value(v.y); v.z = relu_value(v.z); v.w = relu_value(v.w);
         st4(y + 4 * i, v);
     }
-    for (size_t i = n4 * 4 + (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) store_elem(y + i, relu1(load_elem(x + i)));
+    for (size_t i = n4 * 4 + (size_t)blockIdx.x * EB + threadIdx.x; i < n; i += stride) store_elem(y + i, relu_value(load_elem(x + i)));
 }
 
 template <class E>
@@ -160,40 +159,44 @@ __global__ void __launch_bounds__(EB) bias_add_kernel(E* __restrict__ y, const f
 // out[i] = (accumulate ? out[i] : 0) + alpha * (p[0][i] + p[1][i] + ...) (+ bias[i % ncols]); split order fixed
 template <class E>
 __global__ void __launch_bounds__(EB) reduce_splits_kernel(E* __restrict__ out, const float* __restrict__ partial, size_t count,
-                                                           int splits, float alpha, int accumulate, const float* __restrict__ bias_j, int ncols) {
+                                                           int splits, float alpha, int accumulate, const float* __restrict__ bias_j, int ncols,
+                                                           int relu, const E* __restrict__ gate) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < count; i += stride) {
         float s = partial[i];
         for (int k = 1; k < splits; k++) s += partial[(size_t)k * count + i];
         float r = accumulate ? __fmaf_rn(alpha, s, load_elem(out + i)) : alpha * s; // one fused multiply-add on every route
         if (bias_j) r += bias_j[i % ncols];
+        if (relu) r = relu_value(r);
+        if (gate) r = load_elem(gate + i) > 0.0f ? r : 0.0f;
         store_elem(out + i, r);
     }
 }
 
 template <class E>
 static int launch_reduce_splits_t(vdnn_ctx* ctx, hipStream_t stream, E* out, const float* partial, size_t count,
-                                  int splits, float alpha, int accumulate, const float* bias_j, int ncols) {
+                                  int splits, float alpha, int accumulate, const float* bias_j, int ncols, int relu, const E* gate) {
     ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)count * (splits + 2));
     hipLaunchKernelGGL(reduce_splits_kernel<E>, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
-                       out, partial, count, splits, alpha, accumulate, bias_j, ncols);
+                       out, partial, count, splits, alpha, accumulate, bias_j, ncols, relu, gate);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
-                         int splits, float alpha, int accumulate, const float* bias_j, int ncols) {
-    return launch_reduce_splits_t(ctx, stream, out, partial, count, splits, alpha, accumulate, bias_j, ncols);
+                         int splits, float alpha, int accumulate, const float* bias_j, int ncols, int relu, const float* gate) {
+    return launch_reduce_splits_t(ctx, stream, out, partial, count, splits, alpha, accumulate, bias_j, ncols, relu, gate);
 }
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, size_t count,
-                         int splits, float alpha, int accumulate, const float* bias_j, int ncols) {
-    return launch_reduce_splits_t(ctx, stream, out, partial, count, splits, alpha, accumulate, bias_j, ncols);
+                         int splits, float alpha, int accumulate, const float* bias_j, int ncols, int relu, const bf16_t* gate) {
+    return launch_reduce_splits_t(ctx, stream, out, partial, count, splits, alpha, accumulate, bias_j, ncols, relu, gate);
 }
 
 // tiles of a convolution result that were split (tail mode): out[n][m][pix] = sum over the tile's splits (+ bias[m]);
 // partial[(t*splits + ks)*TM*TN + row*TN + col] for the t-th split tile, tiles numbered m-tile fastest
 template <class E>
 __global__ void __launch_bounds__(EB) reduce_tail_nchw_kernel(E* __restrict__ out, const float* __restrict__ partial, int splits, int TM, int TN,
-                                                              int M, int N, int mtiles, int full_tiles, const float* __restrict__ bias, int opix, size_t total) {
+                                                              int M, int N, int mtiles, int full_tiles, const float* __restrict__ bias, int opix, size_t total,
+                                                              int relu, const E* __restrict__ gate) {
     const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
     if (i >= total) return;
     const int per = TM * TN;
@@ -206,27 +209,30 @@ __global__ void __launch_bounds__(EB) reduce_tail_nchw_kernel(E* __restrict__ ou
     float s = p[0];
     for (int k = 1; k < splits; k++) s += p[(size_t)k * per];
     if (bias) s += bias[m];
+    if (relu) s = relu_value(s);
     const int n = j / opix, pix = j - n * opix;
-    store_elem(out + ((size_t)n * M + m) * opix + pix, s);
+    const size_t o = ((size_t)n * M + m) * opix + pix;
+    if (gate) s = load_elem(gate + o) > 0.0f ? s : 0.0f;
+    store_elem(out + o, s);
 }
 
 template <class E>
 static int launch_reduce_tail_nchw_t(vdnn_ctx* ctx, hipStream_t stream, E* out, const float* partial, int tail_tiles, int splits, int TM, int TN,
-                                     int M, int N, int mtiles, int full_tiles, const float* bias, int opix) {
+                                     int M, int N, int mtiles, int full_tiles, const float* bias, int opix, int relu, const E* gate) {
     const size_t total = (size_t)tail_tiles * TM * TN;
     ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)total * (splits + 1));
     hipLaunchKernelGGL(reduce_tail_nchw_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
-                       out, partial, splits, TM, TN, M, N, mtiles, full_tiles, bias, opix, total);
+                       out, partial, splits, TM, TN, M, N, mtiles, full_tiles, bias, opix, total, relu, gate);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 int launch_reduce_tail_nchw(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, int tail_tiles, int splits, int TM, int TN,
-                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix) {
-    return launch_reduce_tail_nchw_t(ctx, stream, out, partial, tail_tiles, splits, TM, TN, M, N, mtiles, full_tiles, bias, opix);
+                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix, int relu, const float* gate) {
+    return launch_reduce_tail_nchw_t(ctx, stream, out, partial, tail_tiles, splits, TM, TN, M, N, mtiles, full_tiles, bias, opix, relu, gate);
 }
 int launch_reduce_tail_nchw(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, int tail_tiles, int splits, int TM, int TN,
-                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix) {
-    return launch_reduce_tail_nchw_t(ctx, stream, out, partial, tail_tiles, splits, TM, TN, M, N, mtiles, full_tiles, bias, opix);
+                            int M, int N, int mtiles, int full_tiles, const float* bias, int opix, int relu, const bf16_t* gate) {
+    return launch_reduce_tail_nchw_t(ctx, stream, out, partial, tail_tiles, splits, TM, TN, M, N, mtiles, full_tiles, bias, opix, relu, gate);
 }
 
 // filter gradient whose partial sums are in tap-major column order: out[m][c][tap] gets partial[.][m][tap*C + c]
@@ -256,31 +262,34 @@ int launch_reduce_splits_tap(vdnn_ctx* ctx, hipStream_t stream, float* out, cons
 // NCHW result of a split convolution: out[i] = p[0][i] + p[1][i] + ... (+ bias[channel of i]); split order fixed
 template <class E>
 __global__ void __launch_bounds__(EB) reduce_splits_nchw_kernel(E* __restrict__ out, const float* __restrict__ partial, size_t count,
-                                                                int splits, const float* __restrict__ bias, int opix, int channels) {
+                                                                int splits, const float* __restrict__ bias, int opix, int channels,
+                                                                int relu, const E* __restrict__ gate) {
     const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
     if (i >= count) return;
     float s = partial[i];
     for (int k = 1; k < splits; k++) s += partial[(size_t)k * count + i];
     if (bias) s += bias[(i / opix) % channels];
+    if (relu) s = relu_value(s);
+    if (gate) s = load_elem(gate + i) > 0.0f ? s : 0.0f;
     store_elem(out + i, s);
 }
 
 template <class E>
 static int launch_reduce_splits_nchw_t(vdnn_ctx* ctx, hipStream_t stream, E* out, const float* partial, size_t count, int splits,
-                                       const float* bias, int opix, int channels) {
+                                       const float* bias, int opix, int channels, int relu, const E* gate) {
     ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)count * (splits + 1));
     hipLaunchKernelGGL(reduce_splits_nchw_kernel<E>, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
-                       out, partial, count, splits, bias, opix, channels);
+                       out, partial, count, splits, bias, opix, channels, relu, gate);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
 int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
-                              const float* bias, int opix, int channels) {
-    return launch_reduce_splits_nchw_t(ctx, stream, out, partial, count, splits, bias, opix, channels);
+                              const float* bias, int opix, int channels, int relu, const float* gate) {
+    return launch_reduce_splits_nchw_t(ctx, stream, out, partial, count, splits, bias, opix, channels, relu, gate);
 }
 int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, size_t count, int splits,
-                              const float* bias, int opix, int channels) {
-    return launch_reduce_splits_nchw_t(ctx, stream, out, partial, count, splits, bias, opix, channels);
+                              const float* bias, int opix, int channels, int relu, const bf16_t* gate) {
+    return launch_reduce_splits_nchw_t(ctx, stream, out, partial, count, splits, bias, opix, channels, relu, gate);
 }
 
 // param[i] = fma(alpha, grad[i], param[i]), the expression the fused updates evaluate
@@ -410,7 +419,7 @@ __device__ __forceinline__ int window_argmax(const E* __restrict__ xp, const Poo
 // gather form: one thread per input element, windows visited in row-major order
 template <class E>
 __global__ void __launch_bounds__(EB) maxpool_bwd_kernel(const E* __restrict__ x, const E* __restrict__ dy, E* __restrict__ dx,
-                                                         PoolGeo g, size_t total) {
+                                                         PoolGeo g, size_t total, int gate) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
         const int w = (int)(i % g.W);
@@ -429,6 +438,7 @@ __global__ void __launch_bounds__(EB) maxpool_bwd_kernel(const E* __restrict__ x
         for (int p = p_lo; p <= p_hi; p++)
             for (int q = q_lo; q <= q_hi; q++)
                 if (window_argmax(xp, g, p, q) == self) acc += load_elem(dyp + (size_t)p * g.Q + q);
+        if (gate && !(load_elem(x + i) > 0.0f)) acc = 0.0f; // x is a rectifier's output: its gradient passes only where x > 0
         store_elem(dx + i, acc);
     }
 }
@@ -436,7 +446,7 @@ __global__ void __launch_bounds__(EB) maxpool_bwd_kernel(const E* __restrict__ x
 // 2x2 stride 2 exact cover: one thread per pair of windows, writes all eight inputs
 template <class E>
 __global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const E* __restrict__ x, const E* __restrict__ dy, E* __restrict__ dx,
-                                                            int H, int W, size_t total_pairs) {
+                                                            int H, int W, size_t total_pairs, int gate) {
     const int Q2 = W / 4, P = H / 2;
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total_pairs; i += stride) {
@@ -446,7 +456,7 @@ __global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const E* __restrict_
         const size_t nc = t / P;
         const size_t off = (nc * H + 2 * (size_t)p) * W + 4 * (size_t)q2;
         const float4 a = ld4(x + off), b = ld4(x + off + W);
-        const float2 d = ld2(dy + (nc * P + p) * (size_t)(W / 2) + 2 * (size_t)q2);
+        float2 d = ld2(dy + (nc * P + p) * (size_t)(W / 2) + 2 * (size_t)q2);
         // window 0: a.x a.y / b.x b.y ; window 1: a.z a.w / b.z b.w ; first strict maximum wins
         int s0 = 0; float m0 = -FLT_MAX;
         if (a.x > m0) { m0 = a.x; s0 = 0; } if (a.y > m0) { m0 = a.y; s0 = 1; }
@@ -454,6 +464,8 @@ __global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const E* __restrict_
         int s1 = 0; float m1 = -FLT_MAX;
         if (a.z > m1) { m1 = a.z; s1 = 0; } if (a.w > m1) { m1 = a.w; s1 = 1; }
         if (b.z > m1) { m1 = b.z; s1 = 2; } if (b.w > m1) { m1 = b.w; s1 = 3; }
+        // gated: the winner receives the gradient only where it is positive (the rectifier that produced x)
+        if (gate) { d.x = m0 > 0.0f ? d.x : 0.0f; d.y = m1 > 0.0f ? d.y : 0.0f; }
         float4 oa, ob;
         oa.x = s0 == 0 ? d.x : 0.0f; oa.y = s0 == 1 ? d.x : 0.0f; ob.x = s0 == 2 ? d.x : 0.0f; ob.y = s0 == 3 ? d.x : 0.0f;
         oa.z = s1 == 0 ? d.y : 0.0f; oa.w = s1 == 1 ? d.y : 0.0f; ob.z = s1 == 2 ? d.y : 0.0f; ob.w = s1 == 3 ? d.y : 0.0f;
@@ -743,7 +755,7 @@ static int maxpool_fwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
 
 template <class E>
 static int maxpool_bwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape,
-                         const void* xv, const void* yv, const void* dyv, void* dxv) {
+                         const void* xv, const void* yv, const void* dyv, void* dxv, int gate) {
     VDNN_KERNEL_PROLOGUE(ctx);
     (void)yv; // the winner of each window is recomputed from x with the forward's comparison
     const E* x = (const E*)xv; const E* dy = (const E*)dyv; E* dx = (E*)dxv;
@@ -754,10 +766,10 @@ static int maxpool_bwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
     ProfScope prof(ctx, st, "maxpool_bwd", 0.0, (double)sizeof(E) * (2.0 * g.N * g.C * g.H * g.W + (double)g.N * g.C * g.P * g.Q));
     if (pool_is_2x2_exact(g, x, dx, dy) && (g.W / 2) % 2 == 0) {
         const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
-        hipLaunchKernelGGL(maxpool2x2_bwd_kernel<E>, dim3(grid_for(pairs, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g.H, g.W, pairs);
+        hipLaunchKernelGGL(maxpool2x2_bwd_kernel<E>, dim3(grid_for(pairs, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g.H, g.W, pairs, gate);
     } else {
         const size_t total = (size_t)g.N * g.C * g.H * g.W;
-        hipLaunchKernelGGL(maxpool_bwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g, total);
+        hipLaunchKernelGGL(maxpool_bwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g, total, gate);
     }
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
@@ -902,7 +914,10 @@ int vdnn_sgd_apply(vdnn_ctx* ctx, vdnn_stream_t stream, size_t count, float alph
 
 int vdnn_maxpool_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* x, void* y) { return ACT_CALL(maxpool_fwd_t, ctx, stream, shape, x, y); }
 int vdnn_maxpool_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* x, const void* y, const void* dy, void* dx) {
-    return ACT_CALL(maxpool_bwd_t, ctx, stream, shape, x, y, dy, dx);
+    return ACT_CALL(maxpool_bwd_t, ctx, stream, shape, x, y, dy, dx, 0);
+}
+int vdnn_maxpool_bwd_relu(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* x, const void* y, const void* dy, void* dx) {
+    return ACT_CALL(maxpool_bwd_t, ctx, stream, shape, x, y, dy, dx, 1);
 }
 int vdnn_lrn_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const void* x, void* y) { return ACT_CALL(lrn_fwd_t, ctx, stream, n, c, hw, x, y); }
 int vdnn_lrn_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const void* x, const void* y, const void* dy, void* dx) {

@@ -6,9 +6,9 @@
 namespace vdnn {
 
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
-                         int splits, float alpha, int accumulate, const float* bias_j, int ncols);
+                         int splits, float alpha, int accumulate, const float* bias_j, int ncols, int relu, const float* gate);
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const float* partial, size_t count,
-                         int splits, float alpha, int accumulate, const float* bias_j, int ncols);
+                         int splits, float alpha, int accumulate, const float* bias_j, int ncols, int relu, const bf16_t* gate);
 
 static inline bool fc_aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
@@ -16,7 +16,7 @@ static inline bool fc_aligned16(const void* p) { return ((uintptr_t)p & 15) == 0
 // ordered partial sums when the tile grid alone cannot fill the chip.
 template <class AL, class BL, class EO>
 static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const char* name, const AL& al, const BL& bl, int M, int N, int K,
-                   EO* out, float alpha, int accumulate, const float* bias_j) {
+                   EO* out, float alpha, int accumulate, const float* bias_j, int relu = 0, const EO* gate = nullptr) {
     const int TM = M <= 64 ? 64 : 128, TN = M <= 64 ? 256 : 128;
     const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
     long cap = ((long)K + 8 * KB - 1) / (8 * KB); // at least eight slices per split
@@ -31,13 +31,13 @@ static int fc_gemm(vdnn_ctx* ctx, hipStream_t st, const char* name, const AL& al
     d.kchunk = kchunk;
     d.splits = (K + kchunk - 1) / kchunk;
     d.full_tiles = 0;
-    StoreDense<EO> ep{out, ctx->reduce_scratch, d.splits > 1 ? nullptr : bias_j, (long)N, (long)M * N, alpha, accumulate};
+    StoreDense<EO> ep{out, ctx->reduce_scratch, d.splits > 1 ? nullptr : bias_j, (long)N, (long)M * N, alpha, accumulate, relu, gate};
     const long blocks = (long)d.mtiles * d.ntiles * d.splits;
     ProfScope prof(ctx, st, name, 2.0 * M * (double)N * K, 0.0);
     if (TM == 64) hipLaunchKernelGGL((igemm_kernel<64, 256, AL, BL, StoreDense<EO>>), dim3((unsigned)blocks), dim3(NT), 0, st, al, bl, ep, d);
     else hipLaunchKernelGGL((igemm_kernel<128, 128, AL, BL, StoreDense<EO>>), dim3((unsigned)blocks), dim3(NT), 0, st, al, bl, ep, d);
     VDNN_LAUNCH_CHECK();
-    if (d.splits > 1) return launch_reduce_splits(ctx, st, out, ctx->reduce_scratch, (size_t)M * N, d.splits, alpha, accumulate, bias_j, N);
+    if (d.splits > 1) return launch_reduce_splits(ctx, st, out, ctx->reduce_scratch, (size_t)M * N, d.splits, alpha, accumulate, bias_j, N, relu, gate);
     return VDNN_OK;
 }
 
@@ -50,7 +50,7 @@ using namespace vdnn;
 // y[n][o] = sum_i x[n][i] * w[o][i] + bias[o]        (Sgemm(T,N) + bias broadcast, layer.cu:677-706)
 template <class E>
 static int fc_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
-                       const E* x, const float* w, const float* bias, E* y) {
+                       const E* x, const float* w, const float* bias, E* y, int relu) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && w && y && n > 0 && c_in > 0 && c_out > 0, "bad argument");
     FC_REQUIRE_SMALL((long)n * c_in); FC_REQUIRE_SMALL((long)c_out * c_in);
@@ -59,17 +59,17 @@ static int fc_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int
     if (c_in % 4 == 0 && fc_aligned16(x) && fc_aligned16(w)) {
         LoadDenseRed<true, E> al{x, (long)c_in, n, xb};
         LoadDenseRed<true> bl{w, (long)c_in, c_out, wb};
-        return fc_gemm(ctx, st, "fc_fwd", al, bl, n, c_out, c_in, y, 1.0f, 0, bias);
+        return fc_gemm(ctx, st, "fc_fwd", al, bl, n, c_out, c_in, y, 1.0f, 0, bias, relu);
     }
     LoadDenseRed<false, E> al{x, (long)c_in, n, xb};
     LoadDenseRed<false> bl{w, (long)c_in, c_out, wb};
-    return fc_gemm(ctx, st, "fc_fwd", al, bl, n, c_out, c_in, y, 1.0f, 0, bias);
+    return fc_gemm(ctx, st, "fc_fwd", al, bl, n, c_out, c_in, y, 1.0f, 0, bias, relu);
 }
 
 // dx[n][i] = sum_o dy[n][o] * w[o][i]                 (Sgemm(N,N), layer.cu:725-733)
 template <class E>
 static int fc_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
-                            const E* dy, const float* w, E* dx) {
+                            const E* dy, const float* w, E* dx, const E* gate) {
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(dy && w && dx && n > 0 && c_in > 0 && c_out > 0, "bad argument");
     FC_REQUIRE_SMALL((long)n * c_out); FC_REQUIRE_SMALL((long)c_out * c_in);
@@ -78,10 +78,10 @@ static int fc_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in
     LoadDenseRow<float> bl{w, (long)c_in, c_in, wb};
     if (c_out % 4 == 0 && fc_aligned16(dy)) {
         LoadDenseRed<true, E> al{dy, (long)c_out, n, db};
-        return fc_gemm(ctx, st, "fc_bwd_data", al, bl, n, c_in, c_out, dx, 1.0f, 0, nullptr);
+        return fc_gemm(ctx, st, "fc_bwd_data", al, bl, n, c_in, c_out, dx, 1.0f, 0, nullptr, 0, gate);
     }
     LoadDenseRed<false, E> al{dy, (long)c_out, n, db};
-    return fc_gemm(ctx, st, "fc_bwd_data", al, bl, n, c_in, c_out, dx, 1.0f, 0, nullptr);
+    return fc_gemm(ctx, st, "fc_bwd_data", al, bl, n, c_in, c_out, dx, 1.0f, 0, nullptr, 0, gate);
 }
 
 // out[o][i] = (accumulate ? out : 0) + alpha * sum_n dy[n][o] * x[n][i]   (Sgemm(N,T), layer.cu:736-744)
@@ -100,14 +100,27 @@ extern "C" {
 
 int vdnn_fc_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
                 const void* x, const float* w, const float* bias, void* y) {
-    return VDNN_BY_ACT(ctx, fc_fwd_impl<float>(ctx, stream, n, c_in, c_out, (const float*)x, w, bias, (float*)y),
-                       fc_fwd_impl<bf16_t>(ctx, stream, n, c_in, c_out, (const bf16_t*)x, w, bias, (bf16_t*)y));
+    return VDNN_BY_ACT(ctx, fc_fwd_impl<float>(ctx, stream, n, c_in, c_out, (const float*)x, w, bias, (float*)y, 0),
+                       fc_fwd_impl<bf16_t>(ctx, stream, n, c_in, c_out, (const bf16_t*)x, w, bias, (bf16_t*)y, 0));
+}
+
+int vdnn_fc_fwd_relu(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                     const void* x, const float* w, const float* bias, void* y) {
+    return VDNN_BY_ACT(ctx, fc_fwd_impl<float>(ctx, stream, n, c_in, c_out, (const float*)x, w, bias, (float*)y, 1),
+                       fc_fwd_impl<bf16_t>(ctx, stream, n, c_in, c_out, (const bf16_t*)x, w, bias, (bf16_t*)y, 1));
 }
 
 int vdnn_fc_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
                      const void* dy, const float* w, void* dx) {
-    return VDNN_BY_ACT(ctx, fc_bwd_data_impl<float>(ctx, stream, n, c_in, c_out, (const float*)dy, w, (float*)dx),
-                       fc_bwd_data_impl<bf16_t>(ctx, stream, n, c_in, c_out, (const bf16_t*)dy, w, (bf16_t*)dx));
+    return VDNN_BY_ACT(ctx, fc_bwd_data_impl<float>(ctx, stream, n, c_in, c_out, (const float*)dy, w, (float*)dx, nullptr),
+                       fc_bwd_data_impl<bf16_t>(ctx, stream, n, c_in, c_out, (const bf16_t*)dy, w, (bf16_t*)dx, nullptr));
+}
+
+int vdnn_fc_bwd_data_relu(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,
+                          const void* dy, const float* w, const void* x, void* dx) {
+    VDNN_REQUIRE(x != nullptr, "null input tensor");
+    return VDNN_BY_ACT(ctx, fc_bwd_data_impl<float>(ctx, stream, n, c_in, c_out, (const float*)dy, w, (float*)dx, (const float*)x),
+                       fc_bwd_data_impl<bf16_t>(ctx, stream, n, c_in, c_out, (const bf16_t*)dy, w, (bf16_t*)dx, (const bf16_t*)x));
 }
 
 int vdnn_fc_bwd_weight_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int c_out,

@@ -59,6 +59,7 @@ void Layer::construct(vdnn_ctx* _ctx) {
     ctx = _ctx;
     /* Basic settings (layer.cu:58-77, 122-142) */
     insideInceptionModule = headOfFork = tailOfFork = inPlaceOp = false;
+    fuseRelu = elided = elidedBackward = gateGrad = false;
     forkId = -1;
     concatenateChannelOffset = 0;
     refCntFwd = refCntBwd = 0;
@@ -127,7 +128,16 @@ Layer::~Layer() {
     if (biasData) vdnn_pool_free(ctx, biasData);
     if (filterGrad) vdnn_pool_free(ctx, filterGrad);
     if (biasGrad) vdnn_pool_free(ctx, biasGrad);
-    if (vdnnMode == BASELINE && dstData) vdnn_pool_free(ctx, dstData);
+    if (vdnnMode == BASELINE && dstData && !elided) vdnn_pool_free(ctx, dstData);
+}
+
+/* an elided ReLU has no output block of its own: under BASELINE the one taken at construction goes back */
+void Layer::setElided(bool v) {
+    if (v == elided) return;
+    if (v && vdnnMode == BASELINE && dstData) { vdnn_pool_free(ctx, dstData); dstData = nullptr; }
+    if (!v && vdnnMode == BASELINE) { dstData = nullptr; cnmemMallocDstData(false); }
+    elided = v;
+    if (!v) elidedBackward = false;
 }
 
 void Layer::setAlgoMode(vdnnAlgoMode_t m) {
@@ -231,8 +241,12 @@ int Layer::convolutionForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, 
         }
     }
 
-    checkVDNN(vdnn_conv_fwd(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)filterData,
-                            (const float*)biasData, (float*)dstData, curWorkSpace, fwdWorkSpaceSize));
+    if (fuseRelu)
+        checkVDNN(vdnn_conv_fwd_relu(ctx, *stream_compute, &shape, vdnnAlgoMode, srcData, (const float*)filterData,
+                                     (const float*)biasData, dstData, curWorkSpace, fwdWorkSpaceSize));
+    else
+        checkVDNN(vdnn_conv_fwd(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)filterData,
+                                (const float*)biasData, (float*)dstData, curWorkSpace, fwdWorkSpaceSize));
 
     /* Offload srcData to host */
     if (_offloaded[layerId]) offloadSrcData(_offloaded, _offloadedSrcData_h);
@@ -256,8 +270,12 @@ int Layer::convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedS
         prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);
 
     if (mallocWorkSpace(workSpace, bwdDataWorkSpaceSize, &curWorkSpace, isDynamic) < 0) return -1;
-    checkVDNN(vdnn_conv_bwd_data(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)diffData, (const float*)filterData,
-                                 (float*)gradData, curWorkSpace, bwdDataWorkSpaceSize));
+    if (gateGrad)
+        checkVDNN(vdnn_conv_bwd_data_relu(ctx, *stream_compute, &shape, vdnnAlgoMode, diffData, (const float*)filterData,
+                                          srcData, gradData, curWorkSpace, bwdDataWorkSpaceSize));
+    else
+        checkVDNN(vdnn_conv_bwd_data(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)diffData, (const float*)filterData,
+                                     (float*)gradData, curWorkSpace, bwdDataWorkSpaceSize));
     freeWorkSpace(workSpace, bwdDataWorkSpaceSize, curWorkSpace, isDynamic);
 
     /* Backward Bias Propagation: the learning rate is folded into the update */
@@ -281,8 +299,12 @@ int Layer::fullyConnectedForward(bool* _offloaded, DATATYPE** _offloadedSrcData_
     if (vdnnMode != BASELINE) {
         if (cnmemMallocDstData(isDynamic) < 0) return -1;
     }
-    checkVDNN(vdnn_fc_fwd(ctx, *stream_compute, n_out, c_in, c_out, (const float*)srcData, (const float*)filterData,
-                          (const float*)biasData, (float*)dstData));
+    if (fuseRelu)
+        checkVDNN(vdnn_fc_fwd_relu(ctx, *stream_compute, n_out, c_in, c_out, srcData, (const float*)filterData,
+                                   (const float*)biasData, dstData));
+    else
+        checkVDNN(vdnn_fc_fwd(ctx, *stream_compute, n_out, c_in, c_out, (const float*)srcData, (const float*)filterData,
+                              (const float*)biasData, (float*)dstData));
     if (_offloaded[layerId]) offloadSrcData(_offloaded, _offloadedSrcData_h);
     return 0;
 }
@@ -296,7 +318,10 @@ int Layer::fullyConnectedBackward(int _layer_id_to_prefetch, DATATYPE* _prefetch
     }
     if (vdnnMode != BASELINE && _layer_id_to_prefetch >= 0)
         prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);
-    checkVDNN(vdnn_fc_bwd_data(ctx, *stream_compute, n_out, c_in, c_out, (const float*)diffData, (const float*)filterData, (float*)gradData));
+    if (gateGrad)
+        checkVDNN(vdnn_fc_bwd_data_relu(ctx, *stream_compute, n_out, c_in, c_out, diffData, (const float*)filterData, srcData, gradData));
+    else
+        checkVDNN(vdnn_fc_bwd_data(ctx, *stream_compute, n_out, c_in, c_out, (const float*)diffData, (const float*)filterData, (float*)gradData));
     if (filterGrad) {
         checkVDNN(vdnn_fc_bwd_weight(ctx, *stream_compute, n_out, c_in, c_out, (const float*)srcData, (const float*)diffData, (float*)filterGrad));
         checkVDNN(vdnn_fc_bwd_bias(ctx, *stream_compute, n_out, c_out, (const float*)diffData, (float*)biasGrad));
@@ -309,6 +334,10 @@ int Layer::fullyConnectedBackward(int _layer_id_to_prefetch, DATATYPE* _prefetch
 
 /* layer.cu:766-788 */
 int Layer::activationForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void*, bool isDynamic) {
+    if (elided) { /* the producer has rectified already: the output is the input block */
+        dstData = srcData;
+        return 0;
+    }
     if (vdnnMode != BASELINE) {
         if (cnmemMallocDstData(isDynamic) < 0) return -1;
     }
@@ -324,11 +353,12 @@ int Layer::activationForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, v
 int Layer::activationBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h, void* _srcDataToPrefetch,
                               unsigned long _prefetch_bytes, void*, bool isDynamic) {
     if (vdnnMode != BASELINE) {
-        if (inPlaceOp) gradData = diffData; /* elementwise: dx may overwrite dy */
+        if (inPlaceOp || elidedBackward) gradData = diffData; /* elementwise: dx may overwrite dy */
         else if (cnmemMallocGradData(isDynamic) < 0) return -1;
     }
     if (vdnnMode != BASELINE && _layer_id_to_prefetch >= 0)
         prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);
+    if (elidedBackward) return 0; /* the consumer's backward has applied the mask */
     if (layerType == TANH)
         checkVDNN(vdnn_tanh_bwd(ctx, *stream_compute, SrcDataSize(), (const float*)dstData, (const float*)diffData, (float*)gradData));
     else if (layerType == SIGMOID)
@@ -379,8 +409,11 @@ int Layer::poolingBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcDa
     }
     if (vdnnMode != BASELINE && _layer_id_to_prefetch >= 0)
         prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);
-    checkVDNN(vdnn_maxpool_bwd(ctx, *stream_compute, &shape, (const float*)srcData, (const float*)dstData,
-                               (const float*)diffData, (float*)gradData));
+    if (gateGrad)
+        checkVDNN(vdnn_maxpool_bwd_relu(ctx, *stream_compute, &shape, srcData, dstData, diffData, gradData));
+    else
+        checkVDNN(vdnn_maxpool_bwd(ctx, *stream_compute, &shape, (const float*)srcData, (const float*)dstData,
+                                   (const float*)diffData, (float*)gradData));
     return 0;
 }
 

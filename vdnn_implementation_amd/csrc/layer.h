@@ -170,6 +170,18 @@ public:
     void    setVdnnMode(vdnn_t _vdnnMode) { vdnnMode = _vdnnMode; }
     // ReLU only: backward writes dx over dy instead of into a freshly allocated gradData
     void    setInPlaceOp(bool v) { inPlaceOp = v; }
+    /* Addition: a ReLU fused into its neighbours. The producing CONV / FC layer rectifies in its own
+       kernel (setFuseRelu); the RELU layer then launches nothing in forward and its dstData is its
+       srcData (setElided). Where the consumer's backward zeroes its gradData at non-positive inputs
+       (setGateGrad), the RELU layer launches nothing in backward either (setElidedBackward). */
+    void    setFuseRelu(bool v) { fuseRelu = v; }
+    bool    FuseRelu() const { return fuseRelu; }
+    void    setElided(bool v);
+    bool    Elided() const { return elided; }
+    void    setElidedBackward(bool v) { elidedBackward = v; }
+    bool    ElidedBackward() const { return elidedBackward; }
+    void    setGateGrad(bool v) { gateGrad = v; }
+    bool    GateGrad() const { return gateGrad; }
     bool    InPlaceOp() const { return inPlaceOp; }
     void    setAlgoMode(vdnnAlgoMode_t m);
     // Event the offload copy waits for (srcData fully written) and the events this layer's copies
@@ -269,6 +281,7 @@ private:
     std::vector<int> producerLayerId, consumerLayerId;
     int  refCntFwd, refCntBwd;
     bool inPlaceOp, insideInceptionModule, headOfFork, tailOfFork;
+    bool fuseRelu, elided, elidedBackward, gateGrad;
     int  forkId, concatenateChannelOffset;
 
     vdnnConvHandle_t* convHandle;

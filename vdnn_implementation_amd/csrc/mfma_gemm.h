@@ -102,6 +102,9 @@ __device__ __forceinline__ void store_elem(float* p, float v) { *p = v; }
 __device__ __forceinline__ void store_elem(bf16_t* p, float v) { p->bits = float_to_bf16_bits(v); }
 
 // one element / four consecutive elements through a descriptor, as float (offsets in bytes)
+// max(v, 0) that lets NaN through
+__device__ __forceinline__ float relu_value(float v) { return v > 0.0f ? v : (v != v ? v : 0.0f); }
+
 template <class E> __device__ __forceinline__ float buf_load_e(__amdgpu_buffer_rsrc_t r, int voff, int soff);
 template <> __device__ __forceinline__ float buf_load_e<float>(__amdgpu_buffer_rsrc_t r, int voff, int soff) { return buf_load(r, voff, soff); }
 template <> __device__ __forceinline__ float buf_load_e<bf16_t>(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
@@ -398,6 +401,8 @@ struct StoreDense {
     long partial_stride; // elements per split
     float alpha;
     int accumulate;
+    int relu;      // rectify the result (after the bias)
+    const E* gate; // optional, same layout as out: the result is kept where gate > 0 and zero elsewhere
     static constexpr bool TAIL = false;
     __device__ __forceinline__ void store_tail(const floatx16 (&)[2][2], int, int, int, long, int, int) const {}
     __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int ks, const GemmDims& d, bool to_partial) const {
@@ -420,6 +425,8 @@ struct StoreDense {
                         // one fused multiply-add: every route to "out += alpha * sum" rounds the same way
                         float r = accumulate ? __fmaf_rn(alpha, a, load_elem(out + idx)) : alpha * a;
                         if (bias_j) r += bias_j[j];
+                        if (relu) r = relu_value(r);
+                        if (gate) r = load_elem(gate + idx) > 0.0f ? r : 0.0f;
                         store_elem(out + idx, r);
                     }
                 }

@@ -295,9 +295,17 @@ void Network::buildLayers() {
             layer[l] = new Layer(vdnnType, mode, s.type, &convHandle, &stream_compute, &stream_memory, l,
                                  s.n, s.c, s.h, s.w, s.pad_h, s.pad_w, s.stride_h, s.stride_w, s.k, s.r, s.s);
         if (options.unfusedOptimizer) layer[l]->keepGradients();
+        /* before the next layer takes its blocks: an elided ReLU hands its BASELINE output block back */
+        if (fusesRelu(l)) layer[l]->setElided(true);
     }
     capDst.assign(numLayers, {});
     capGrad.assign(numLayers, {});
+}
+
+/* addition (fuseActivations): layer l is a ReLU that the CONV / FC layer before it applies */
+bool Network::fusesRelu(int l) const {
+    if (!options.fuseActivations || l <= 0 || l >= (int)specs.size() || specs[l].type != RELU) return false;
+    return is_conv(specs[l - 1].type) || specs[l - 1].type == FC_GEMM;
 }
 
 /* network.cu:819-829: the reference draws U(-0.01, 0.01) from an unseeded generator on every call;
@@ -346,6 +354,28 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         if (layer[i] != NULL) {
             layer[i]->setVdnnMode(newVdnnType);
             layer[i]->setInPlaceOp(false);
+            layer[i]->setFuseRelu(false);
+            layer[i]->setElidedBackward(false);
+            layer[i]->setGateGrad(false);
+        }
+    }
+    /* fused rectifiers: producer l-1 rectifies, consumer l+1 masks its gradient */
+    if (options.fuseActivations) {
+        for (int l = 1; l < numLayers; l++) {
+            if (!fusesRelu(l)) continue;
+            layer[l - 1]->setFuseRelu(true);
+            layer[l]->setElided(true);
+            layer[l]->setInPlaceOp(true);
+            if (l + 1 < numLayers) {
+                const Layer_t next = layer[l + 1]->LayerType();
+                /* a convolution over at most four channels computes its input gradient with a kernel of
+                   its own that has no masked store: the ReLU's backward stays a launch there */
+                const bool few_channels = is_conv(next) && layer[l + 1]->InputC() <= 4;
+                if ((is_conv(next) || next == FC_GEMM || next == POOL) && !few_channels) {
+                    layer[l + 1]->setGateGrad(true);
+                    layer[l]->setElidedBackward(true);
+                }
+            }
         }
     }
     lastStats.pinnedBytes = 0;
@@ -357,12 +387,13 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
             const Layer_t kind = layer[l]->LayerType(); /* all three activations differentiate from y alone */
             if (kind != RELU && kind != TANH && kind != SIGMOID) continue;
             layer[l]->setInPlaceOp(true);
-            if (l > 0) dropSrcAfterFwd[l] = true;
+            if (l > 0 && !layer[l]->Elided()) dropSrcAfterFwd[l] = true;
         }
     }
 
     auto offload = [&](int l) {
         if (dropSrcAfterFwd[l]) return; /* released, not moved: nothing reads it again */
+        if (layer[l]->Elided()) return;  /* its input is the next layer's srcData, which has its own turn */
         isOffload[l] = true;
         const size_t bytes = layer[l]->SrcDataSize() * actBytes();
         checkVDNN(vdnn_host_alloc_pinned(ctx, (void**)&offloadedSrcData_h[l], bytes));
@@ -572,6 +603,15 @@ int Network::backwardPropagation(bool isDynamic) {
                 layer[l]->copyDiffData(layer[l + 1]->GradData());
                 layer[l]->copyGradData(layer[l + 1]->DiffData());
             }
+            if (layer[l]->ElidedBackward()) {
+                /* the masked gradient is already in place: it is this layer's gradData, and the other
+                   buffer of the pair stays free for the layer below */
+                void* masked = layer[l]->DiffData();
+                layer[l]->copyDiffData(layer[l]->GradData());
+                layer[l]->copyGradData(masked);
+                captureLayer(l, true);
+                continue;
+            }
             if (layer[l]->backward(-1, NULL, NULL, 0, workSpace, isDynamic) < 0) return -1;
             captureLayer(l, true);
             printUsage("Bwd", l, layer[l]->BwdDataWorkSpaceSize() + layer[l]->BwdFilterWorkSpaceSize());
@@ -585,6 +625,9 @@ int Network::backwardPropagation(bool isDynamic) {
             if (l != numLayers - 1) {
                 layer[l]->copyDiffData(layer[l + 1]->GradData());
                 layer[l]->copyDstData(layer[l + 1]->SrcData());
+                /* an elided ReLU's input and output are one block: the next layer's srcData, by now
+                   possibly a prefetched copy at another address */
+                if (layer[l]->Elided()) layer[l]->copySrcData(layer[l]->DstData());
             }
             /* refined lifetimes: convolution, FC and pooling backward never read their output, so
                its block (the next layer's srcData) goes back to the pool before anything is
@@ -631,7 +674,8 @@ int Network::backwardPropagation(bool isDynamic) {
 
             /* Release dstData and diffData: every reader is already enqueued on the compute stream.
                An in-place ReLU's diffData is its gradData and lives on as the next layer's diffData. */
-            if (!dstReleased) ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DstData()), isDynamic);
+            /* an elided ReLU's block is released by the layer below, as its dstData */
+            if (!dstReleased && !layer[l]->Elided()) ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DstData()), isDynamic);
             if (!(layer[l]->InPlaceOp() && layer[l]->GradData() == layer[l]->DiffData()))
                 ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DiffData()), isDynamic);
             printUsage("Bwd", l, layer[l]->BwdDataWorkSpaceSize() + layer[l]->BwdFilterWorkSpaceSize());

@@ -45,6 +45,12 @@ struct NetworkOptions {
     int      prefetchDepth = 1;
     bool     unfusedOptimizer = false;
     bool     deferOptimizer = false;
+    // A ReLU layer that follows a CONV / FC layer is applied by that layer's own kernel, and its backward
+    // by the backward of the CONV / FC / POOL layer that consumes it (where one does); the ReLU layer then
+    // launches nothing and owns no tensor: its dstData is its srcData and its gradData its diffData. Same
+    // bits as the separate layers of the reference (layer.cu:766-814); two passes over the tensor fewer.
+    // Such a ReLU layer is never offloaded (its input is not a tensor of its own any more).
+    bool     fuseActivations = false;
     int      device = DEFAULT_DEVICE;
 };
 
@@ -91,6 +97,7 @@ public:
     void            setLayersAlexnet();
     void            setLayersOverfeat();
     void            setLayersGooglenet();
+    bool            fusesRelu(int l) const;
     void            setLayersVgg16(int givenBatch);
     void            setLayersCustomCNN();
     void            randomInitializeData(void* data, size_t size);

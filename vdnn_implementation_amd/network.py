@@ -15,7 +15,8 @@ _ip = C.POINTER(C.c_int32)
 class Options(C.Structure):
     _fields_ = [("seed", C.c_uint64), ("pool_bytes", _sz), ("cap_bytes", _sz), ("plan_only", _i), ("host_sync", _i),
                 ("capture", _i), ("verbose", _i), ("device", _i), ("refined_lifetimes", _i),
-                ("unfused_optimizer", _i), ("defer_optimizer", _i), ("offload_lag", _i), ("prefetch_depth", _i), ("data_type", _i)]
+                ("unfused_optimizer", _i), ("defer_optimizer", _i), ("offload_lag", _i), ("prefetch_depth", _i), ("data_type", _i),
+                ("fuse_activations", _i)]
 
 
 class LayerSpec(C.Structure):
@@ -91,7 +92,8 @@ class Network:
 
     def __init__(self, cnn=None, policy=enums.BASELINE, algo=enums.VDNN_MEMORY_OPT_ALGO, batch=0, layers=None, seed=1,
                  pool_bytes=0, cap_bytes=0, plan_only=False, host_sync=False, capture=False, verbose=False, device=0,
-                 refined=False, unfused_optimizer=False, defer_optimizer=False, bf16=False, offload_lag=0, prefetch_depth=1):
+                 refined=False, unfused_optimizer=False, defer_optimizer=False, bf16=False, offload_lag=0, prefetch_depth=1,
+                 fuse=False):
         o = Options()
         lib.vdnn_network_default_options(C.byref(o))
         o.seed, o.pool_bytes, o.cap_bytes = seed, int(pool_bytes), int(cap_bytes)
@@ -100,6 +102,7 @@ class Network:
         o.unfused_optimizer, o.defer_optimizer = int(unfused_optimizer), int(defer_optimizer)
         o.data_type = 1 if bf16 else 0  # VDNN_DTYPE_BF16 / VDNN_DTYPE_F32
         o.offload_lag, o.prefetch_depth = int(offload_lag), int(prefetch_depth)
+        o.fuse_activations = int(fuse)
         if layers is not None:
             arr = (LayerSpec * len(layers))(*layers)
             self._h = lib.vdnn_network_create_custom(arr, len(layers), policy, algo, C.byref(o))
