@@ -127,7 +127,8 @@ def test_fc_fused_rectifier_gives_the_bits_of_the_separate_calls(ctx, n, cin, co
         assert_close(gxf, oracle.fc_bwd_data(dy, w) * (x > 0), 2e-5, "masked fc backward data against the checker")
 
 
-@pytest.mark.parametrize("n,c,h,w,win,stride", [(2, 8, 16, 16, 2, 2), (3, 5, 13, 13, 3, 2), (2, 4, 12, 20, 2, 2), (1, 3, 9, 9, 3, 3)])
+@pytest.mark.parametrize("n,c,h,w,win,stride", [(2, 8, 16, 16, 2, 2), (3, 5, 13, 13, 3, 2), (2, 4, 12, 20, 2, 2), (1, 3, 9, 9, 3, 3),
+                                                (1, 2, 130, 121, 3, 2)])
 def test_maxpool_backward_masked_by_its_input(ctx, n, c, h, w, win, stride):
     rng = np.random.default_rng(h * 100 + win)
     x = relu(rng.standard_normal((n, c, h, w)).astype(np.float32))  # about half zeros: windows of zeros have ties

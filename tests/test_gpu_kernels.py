@@ -269,7 +269,11 @@ def test_tanh_and_sigmoid(ctx, count):
         assert_close(got_dx, bwd(got_y, dy), 1e-6, name + " backward")
 
 
-POOLS = [(2, 3, 13, 15, 3, 2), (2, 3, 12, 12, 2, 2), (1, 2, 7, 9, 2, 2), (3, 5, 8, 16, 2, 2), (2, 4, 27, 27, 3, 2), (1, 2, 6, 10, 2, 2)]
+POOLS = [(2, 3, 13, 15, 3, 2), (2, 3, 12, 12, 2, 2), (1, 2, 7, 9, 2, 2), (3, 5, 8, 16, 2, 2), (2, 4, 27, 27, 3, 2), (1, 2, 6, 10, 2, 2),
+         (3, 7, 55, 55, 3, 2),     # AlexNet's first pool: one plane per workgroup in LDS
+         (2, 37, 13, 13, 3, 2),    # several planes per workgroup, the last group short
+         (1, 2, 130, 121, 3, 2),   # planes too large for LDS: the gather kernel
+         (2, 3, 20, 20, 3, 1)]     # stride 1: every input in up to nine windows
 
 
 @pytest.mark.parametrize("n,c,h,w,win,stride", POOLS)

@@ -98,7 +98,7 @@ static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names
     const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
     int splits = 1;
     const size_t out_bytes = (size_t)M * N * sizeof(float);
-    if (tiles < 2l * ctx->num_cu && ctx->reduce_scratch) {
+    if (tiles < 2l * ctx->num_cu && ctx->reduce_scratch && ep.partial) {
         long cap = ((long)K + 8 * KB - 1) / (8 * KB); // at least eight slices per split
         const long by_mem = (long)(ctx->reduce_scratch_bytes / out_bytes);
         if (cap > by_mem) cap = by_mem;
@@ -111,7 +111,7 @@ static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names
     const long slots = 3l * ctx->num_cu;
     const long rem = tiles % slots;
     int tail_tiles = 0;
-    if (splits == 1 && tiles > slots && rem > 0 && 2 * rem <= slots && ctx->reduce_scratch) {
+    if (splits == 1 && tiles > slots && rem > 0 && 2 * rem <= slots && ctx->reduce_scratch && ep.partial) {
         long s = slots / rem;
         const long by_depth = (long)K / (8 * KB); // at least eight slices per split
         const long by_mem = (long)(ctx->reduce_scratch_bytes / ((size_t)rem * TM * TN * sizeof(float)));
@@ -238,6 +238,34 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
                     : vdnn_fc_bwd_data(ctx, stream, g.N, g.C * g.H * g.W, g.K, dy, w, dx);
     hipStream_t st = stream_of(ctx, stream);
     if (g.C <= 4 && g.R * g.S <= SMALLC_MAXTAPS && !gate) { // the vector-ALU kernels have no gated store
+        if ((g.sh != 1 || g.sw != 1) && ctx->reduce_scratch && ctx->reduce_scratch_bytes >= (size_t)g.C * g.R * g.S * g.P * g.Q * sizeof(float) &&
+                 pixel_tile_span_ok((long)g.K * g.P * g.Q, g.P * g.Q, 256, (int)sizeof(E))) {
+            // Strided layer with few input channels (the 11x11 stride-4 first layers): its three or four
+            // output rows cannot fill a matrix tile, so the products are formed once, as a 1x1 convolution
+            // with C*R*S output channels over dy on the matrix cores, into the staging area, and gathered
+            // into dx by a second kernel; as many samples at a time as the staging area holds.
+            const int RS = g.R * g.S, CRS = g.C * RS, PQ = g.P * g.Q;
+            const size_t per_sample = (size_t)CRS * PQ * sizeof(float);
+            int nb = (int)(ctx->reduce_scratch_bytes / per_sample);
+            if (nb > g.N) nb = g.N;
+            float* T = ctx->reduce_scratch;
+            LoadFilterT alt{w, CRS, 1, (unsigned)((long)g.K * CRS * 4), FastDiv::make(1)};
+            for (int n0 = 0; n0 < g.N; n0 += nb) {
+                const int nc = g.N - n0 < nb ? g.N - n0 : nb;
+                LoadIm2colPix<0, false, E> bl{dy + (long)n0 * g.K * PQ, g.P, g.Q, g.P, g.Q, 1, 1, 0, 0, 1, 1, (long)g.K * PQ, nc,
+                                              FastDiv::make(1), FastDiv::make(1)};
+                StoreNCHW<float> ept{T, nullptr, PQ, nullptr, 0, nullptr};
+                const int rc = launch_by_m(ctx, st, kBwdDataNames, alt, bl, ept, CRS, nc * PQ, g.K, 2.0 * nc * (double)g.K * CRS * PQ);
+                if (rc != VDNN_OK) return rc;
+                ConvGeo gc = g; gc.N = nc;
+                const long total = (long)nc * g.C * g.H * g.W;
+                ProfScope gather(ctx, st, "conv_bwd_data_gather", 0.0, (double)per_sample * nc + (double)total * sizeof(E));
+                hipLaunchKernelGGL(conv_bwd_data_gather_taps_kernel<E>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                                   T, dx + (long)n0 * g.C * g.H * g.W, gc, total);
+                VDNN_LAUNCH_CHECK();
+            }
+            return VDNN_OK;
+        }
         const long total = (long)g.N * g.H * g.W;
         const long blocks = (total + 255) / 256;
         VDNN_REQUIRE(blocks < (1l << 31), "grid too large");

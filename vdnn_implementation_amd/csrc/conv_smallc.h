@@ -125,6 +125,36 @@ __global__ void __launch_bounds__(256) conv_bwd_data_smallc_strided_kernel(const
     if (g.C > 3) store_elem(o + 3 * plane, acc.w);
 }
 
+// Second stage of the strided few-channel backward data on the matrix cores. The first stage is a 1x1
+// convolution T[n][(c,r,s)][p][q] = sum_k w[k,c,r,s] * dy[n,k,p,q] (every product the layer needs, once);
+// here an input pixel adds up the entries whose tap lands on it: dx[n,c,h,x] = sum over taps (r,s) with
+// (h+ph-r) = p*sh and (x+pw-s) = q*sw of T[n][(c,r,s)][p][q], taps in ascending (r,s) order.
+template <class E>
+__global__ void __launch_bounds__(256) conv_bwd_data_gather_taps_kernel(const float* __restrict__ T, E* __restrict__ dx, const ConvGeo g, long total) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int x = (int)(i % g.W);
+    long t = i / g.W;
+    const int h = (int)(t % g.H); t /= g.H;
+    const int c = (int)(t % g.C);
+    const long n = t / g.C;
+    const int PQ = g.P * g.Q;
+    const float* Tc = T + (n * g.C + c) * (long)g.R * g.S * PQ;
+    float acc = 0.0f;
+    for (int r = (h + g.ph) % g.sh; r < g.R; r += g.sh) {
+        const int p = (h + g.ph - r) / g.sh;
+        if (h + g.ph - r < 0) break;
+        if (p >= g.P) continue;
+        for (int s = (x + g.pw) % g.sw; s < g.S; s += g.sw) {
+            const int q = (x + g.pw - s) / g.sw;
+            if (x + g.pw - s < 0) break;
+            if (q >= g.Q) continue;
+            acc += Tc[(long)(r * g.S + s) * PQ + p * g.Q + q];
+        }
+    }
+    store_elem(dx + i, acc);
+}
+
 // The same, for a compile-time window at stride 1 (VGG's 3x3): fully unrolled and branch-free. Taps
 // outside dy are read from a clamped position and replaced by zero. The filter values of one output
 // channel are wave-uniform, so they are fetched with scalar loads straight from global memory.

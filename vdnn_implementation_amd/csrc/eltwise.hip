@@ -443,6 +443,62 @@ __global__ void __launch_bounds__(EB) maxpool_bwd_kernel(const E* __restrict__ x
     }
 }
 
+// Overlapping windows on planes that fit LDS (AlexNet's 3x3 stride 2): a workgroup stages `group` whole
+// (n,c) planes and their dy, finds every window's winner once, and each input element then asks the few
+// windows that contain it. Same winner rule and the same summation order as the gather kernel above, so the
+// same bits; x, dy and dx cross HBM once.
+template <class E>
+__global__ void __launch_bounds__(EB) maxpool_bwd_planes_kernel(const E* __restrict__ x, const E* __restrict__ dy, E* __restrict__ dx,
+                                                                PoolGeo g, long planes, int group, int gate) {
+    extern __shared__ float pool_lds[];
+    const int HW = g.H * g.W, PQ = g.P * g.Q;
+    float* xs = pool_lds;                      // [group][HW]
+    float* dys = xs + group * HW;              // [group][PQ]
+    int* arg = (int*)(dys + group * PQ);       // [group][PQ] winner's index in its plane
+    const long plane0 = (long)blockIdx.x * group;
+    const int here = (int)(planes - plane0 < group ? planes - plane0 : group);
+    const E* xp = x + plane0 * HW;
+    const E* dyp = dy + plane0 * PQ;
+    for (int i = threadIdx.x; i < here * HW; i += EB) xs[i] = load_elem(xp + i);
+    for (int i = threadIdx.x; i < here * PQ; i += EB) dys[i] = load_elem(dyp + i);
+    __syncthreads();
+    for (int o = threadIdx.x; o < here * PQ; o += EB) {
+        const int pl = o / PQ, pq = o - pl * PQ;
+        const int p = pq / g.Q, q = pq - p * g.Q;
+        const float* xpl = xs + pl * HW;
+        float m = -FLT_MAX;
+        int a = -1;
+        for (int r = 0; r < g.R; r++) {
+            const int ih = p * g.sh - g.ph + r;
+            if (ih < 0 || ih >= g.H) continue;
+            for (int s_ = 0; s_ < g.S; s_++) {
+                const int iw = q * g.sw - g.pw + s_;
+                if (iw < 0 || iw >= g.W) continue;
+                const float v = xpl[ih * g.W + iw];
+                if (a < 0) a = ih * g.W + iw;
+                if (v > m) { m = v; a = ih * g.W + iw; }
+            }
+        }
+        arg[o] = a;
+    }
+    __syncthreads();
+    E* dxp = dx + plane0 * HW;
+    for (int i = threadIdx.x; i < here * HW; i += EB) {
+        const int pl = i / HW, self = i - pl * HW;
+        const int h = self / g.W, w = self - h * g.W;
+        int p_lo = h + g.ph - g.R + 1; p_lo = p_lo <= 0 ? 0 : (p_lo + g.sh - 1) / g.sh;
+        int p_hi = (h + g.ph) / g.sh; if (p_hi > g.P - 1) p_hi = g.P - 1;
+        int q_lo = w + g.pw - g.S + 1; q_lo = q_lo <= 0 ? 0 : (q_lo + g.sw - 1) / g.sw;
+        int q_hi = (w + g.pw) / g.sw; if (q_hi > g.Q - 1) q_hi = g.Q - 1;
+        float acc = 0.0f;
+        for (int p = p_lo; p <= p_hi; p++)
+            for (int q = q_lo; q <= q_hi; q++)
+                if (arg[pl * PQ + p * g.Q + q] == self) acc += dys[pl * PQ + p * g.Q + q];
+        if (gate && !(xs[i] > 0.0f)) acc = 0.0f;
+        store_elem(dxp + i, acc);
+    }
+}
+
 // 2x2 stride 2 exact cover: one thread per pair of windows, writes all eight inputs
 template <class E>
 __global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const E* __restrict__ x, const E* __restrict__ dy, E* __restrict__ dx,
@@ -767,6 +823,16 @@ static int maxpool_bwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
     if (pool_is_2x2_exact(g, x, dx, dy) && (g.W / 2) % 2 == 0) {
         const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
         hipLaunchKernelGGL(maxpool2x2_bwd_kernel<E>, dim3(grid_for(pairs, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g.H, g.W, pairs, gate);
+    } else if ((size_t)g.H * g.W * 4 + (size_t)g.P * g.Q * 8 <= 48 * 1024) {
+        // whole planes in LDS: as many per workgroup as give every thread a few elements
+        const size_t per_plane = (size_t)g.H * g.W * 4 + (size_t)g.P * g.Q * 8;
+        int group = (int)((4 * EB + g.H * g.W - 1) / (g.H * g.W));
+        if ((size_t)group * per_plane > 48 * 1024) group = (int)(48 * 1024 / per_plane);
+        if (group < 1) group = 1;
+        const long planes = (long)g.N * g.C;
+        const long blocks = (planes + group - 1) / group;
+        VDNN_REQUIRE(blocks < (1l << 31), "grid too large");
+        hipLaunchKernelGGL(maxpool_bwd_planes_kernel<E>, dim3((unsigned)blocks), dim3(EB), group * per_plane, st, x, dy, dx, g, planes, group, gate);
     } else {
         const size_t total = (size_t)g.N * g.C * g.H * g.W;
         hipLaunchKernelGGL(maxpool_bwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g, total, gate);
