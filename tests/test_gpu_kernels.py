@@ -311,7 +311,8 @@ def test_maxpool_golden(ctx):
             assert_close(dx.download(f["x"].shape), f["dx"], 1e-7)
 
 
-@pytest.mark.parametrize("shape,scale", [((2, 9, 4, 5), 1.0), ((2, 9, 4, 5), 60.0), ((3, 96, 11, 13), 30.0), ((1, 3, 5, 5), 10.0)])
+@pytest.mark.parametrize("shape,scale", [((2, 9, 4, 5), 1.0), ((2, 9, 4, 5), 60.0), ((3, 96, 11, 13), 30.0), ((1, 3, 5, 5), 10.0),
+                                         ((2, 37, 7, 9), 20.0), ((1, 16, 3, 3), 5.0), ((2, 17, 3, 3), 5.0), ((1, 1, 4, 4), 50.0)])
 def test_lrn(ctx, shape, scale):
     rng = np.random.default_rng(int(scale) + shape[1])
     x = (rng.standard_normal(shape) * scale).astype(np.float32)

@@ -535,53 +535,77 @@ __global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const E* __restrict_
 #define LRN_BETA 0.75f
 #define LRN_KC 2.0f
 
+// One thread = LRN_CH consecutive channels of one (sample, pixel), lanes along pixels: the channels it needs
+// (its own and the halo of the windows) are fetched up front, each window sum is taken in ascending channel
+// order, and a value crosses HBM once apart from the halo.
+constexpr int LRN_CH = 16;
+
 template <class E>
-__global__ void __launch_bounds__(EB) lrn_fwd_kernel(const E* __restrict__ x, E* __restrict__ y, int C, int hw, size_t total) {
-    const size_t stride = (size_t)gridDim.x * EB;
-    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
-        const int c = (int)((i / hw) % C);
+__global__ void __launch_bounds__(EB) lrn_fwd_kernel(const E* __restrict__ x, E* __restrict__ y, int C, int hw, int chunks, size_t total) {
+    const size_t i = (size_t)blockIdx.x * EB + threadIdx.x; // (sample, chunk, pixel), pixel fastest
+    if (i >= total) return;
+    const int pix = (int)(i % hw);
+    const size_t t = i / hw;
+    const int chunk = (int)(t % chunks);
+    const size_t n = t / chunks;
+    const int c0 = chunk * LRN_CH;
+    const E* xp = x + (n * C) * hw + pix;
+    E* yp = y + (n * C) * hw + pix;
+    float v[LRN_CH + 4]; // channels c0-2 .. c0+LRN_CH+1, zero outside the tensor
+#pragma unroll
+    for (int k = 0; k < LRN_CH + 4; k++) {
+        const int c = c0 - 2 + k;
+        v[k] = (c >= 0 && c < C) ? load_elem(xp + (size_t)c * hw) : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < LRN_CH; k++) {
+        if (c0 + k >= C) break;
         float ss = 0.0f;
 #pragma unroll
-        for (int d = -2; d <= 2; d++) {
-            const int cc = c + d;
-            if (cc < 0 || cc >= C) continue;
-            const float v = load_elem(x + ((long)i + (long)d * hw));
-            ss += v * v;
-        }
+        for (int d = 0; d < 5; d++) ss += v[k + d] * v[k + d];
         const float scale = LRN_KC + LRN_A5 * ss;
-        store_elem(y + i, load_elem(x + i) * powf(scale, -LRN_BETA));
+        store_elem(yp + (size_t)(c0 + k) * hw, v[k + 2] * powf(scale, -LRN_BETA));
     }
 }
 
 template <class E>
 __global__ void __launch_bounds__(EB) lrn_bwd_kernel(const E* __restrict__ x, const E* __restrict__ y, const E* __restrict__ dy,
-                                                     E* __restrict__ dx, int C, int hw, size_t total) {
-    const size_t stride = (size_t)gridDim.x * EB;
-    for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < total; i += stride) {
-        const int c = (int)((i / hw) % C);
-        float xs[9]; // x^2 of channels c-4 .. c+4
+                                                     E* __restrict__ dx, int C, int hw, int chunks, size_t total) {
+    const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
+    if (i >= total) return;
+    const int pix = (int)(i % hw);
+    const size_t t_ = i / hw;
+    const int chunk = (int)(t_ % chunks);
+    const size_t n = t_ / chunks;
+    const int c0 = chunk * LRN_CH;
+    const size_t base = (n * C) * hw + pix;
+    float xv[LRN_CH + 8];  // channels c0-4 .. c0+LRN_CH+3
+    float term[LRN_CH + 4]; // dy*y/scale of channels c0-2 .. c0+LRN_CH+1
+    float scale_own[LRN_CH];
 #pragma unroll
-        for (int d = -4; d <= 4; d++) {
-            const int cc = c + d;
-            float v = 0.0f;
-            if (cc >= 0 && cc < C) v = load_elem(x + ((long)i + (long)d * hw));
-            xs[d + 4] = v * v;
-        }
-        float t = 0.0f, scale_c = 1.0f;
+    for (int k = 0; k < LRN_CH + 8; k++) {
+        const int c = c0 - 4 + k;
+        xv[k] = (c >= 0 && c < C) ? load_elem(x + base + (size_t)c * hw) : 0.0f;
+    }
 #pragma unroll
-        for (int d = -2; d <= 2; d++) {
-            const int cc = c + d;
-            // scale of channel cc: its own window, taken in ascending channel order
-            float ss = 0.0f;
+    for (int k = 0; k < LRN_CH + 4; k++) {
+        const int c = c0 - 2 + k;
+        float ss = 0.0f; // the window of channel c, ascending
 #pragma unroll
-            for (int e = -2; e <= 2; e++) ss += xs[d + e + 4];
-            const float scale = LRN_KC + LRN_A5 * ss;
-            if (d == 0) scale_c = scale;
-            if (cc < 0 || cc >= C) continue;
-            const long o = (long)i + (long)d * hw;
-            t += load_elem(dy + o) * load_elem(y + o) / scale;
-        }
-        store_elem(dx + i, load_elem(dy + i) * powf(scale_c, -LRN_BETA) - (2.0f * 1e-4f * LRN_BETA / 5.0f) * load_elem(x + i) * t);
+        for (int e = 0; e < 5; e++) ss += xv[k + e] * xv[k + e];
+        const float scale = LRN_KC + LRN_A5 * ss;
+        if (k >= 2 && k < LRN_CH + 2) scale_own[k - 2] = scale;
+        term[k] = (c >= 0 && c < C) ? load_elem(dy + base + (size_t)c * hw) * load_elem(y + base + (size_t)c * hw) / scale : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < LRN_CH; k++) {
+        const int c = c0 + k;
+        if (c >= C) break;
+        float tsum = 0.0f;
+#pragma unroll
+        for (int d = 0; d < 5; d++) tsum += term[k + d];
+        const float dyc = load_elem(dy + base + (size_t)c * hw);
+        store_elem(dx + base + (size_t)c * hw, dyc * powf(scale_own[k], -LRN_BETA) - (2.0f * 1e-4f * LRN_BETA / 5.0f) * xv[k + 4] * tsum);
     }
 }
 
@@ -846,8 +870,11 @@ static int lrn_fwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, 
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && y && n > 0 && c > 0 && hw > 0, "bad argument");
     const size_t total = (size_t)n * c * hw;
+    const int chunks = (c + LRN_CH - 1) / LRN_CH;
+    const size_t threads = (size_t)n * chunks * hw;
+    VDNN_REQUIRE((threads + EB - 1) / EB < (1ul << 31), "grid too large");
     ProfScope prof(ctx, stream_of(ctx, stream), "lrn_fwd", 0.0, 2.0 * sizeof(E) * (double)total);
-    hipLaunchKernelGGL(lrn_fwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), (const E*)x, (E*)y, c, hw, total);
+    hipLaunchKernelGGL(lrn_fwd_kernel<E>, dim3(grid_for(threads, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream), (const E*)x, (E*)y, c, hw, chunks, threads);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
@@ -857,9 +884,12 @@ static int lrn_bwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, 
     VDNN_KERNEL_PROLOGUE(ctx);
     VDNN_REQUIRE(x && y && dy && dx && n > 0 && c > 0 && hw > 0, "bad argument");
     const size_t total = (size_t)n * c * hw;
+    const int chunks = (c + LRN_CH - 1) / LRN_CH;
+    const size_t threads = (size_t)n * chunks * hw;
+    VDNN_REQUIRE((threads + EB - 1) / EB < (1ul << 31), "grid too large");
     ProfScope prof(ctx, stream_of(ctx, stream), "lrn_bwd", 0.0, 4.0 * sizeof(E) * (double)total);
-    hipLaunchKernelGGL(lrn_bwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream),
-                       (const E*)x, (const E*)y, (const E*)dy, (E*)dx, c, hw, total);
+    hipLaunchKernelGGL(lrn_bwd_kernel<E>, dim3(grid_for(threads, EB, 0x7FFFFFFF)), dim3(EB), 0, stream_of(ctx, stream),
+                       (const E*)x, (const E*)y, (const E*)dy, (E*)dx, c, hw, chunks, threads);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
