@@ -29,9 +29,9 @@ FLOP_PER_IMAGE = 92.82e9  # 3 passes over 13 convolutions and 3 FC layers
 # kept under profiles/. FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0: what the same counters
 # read for the ReLU kernels of the same run, which move a known number of bytes.
 MEASURED_TRAFFIC_BYTES = {
-    "conv_fwd_128x128": 960.7e6,
-    "conv_bwd_data_128x128": 912.1e6,
-    "conv_bwd_filter_128x128": 1813.8e6,
+    "conv_fwd_128x128": 984.8e6,
+    "conv_bwd_data_128x128": 940.3e6,
+    "conv_bwd_filter_128x128": 1724.8e6,
 }
 
 
