@@ -21,7 +21,9 @@ struct orc_net {
     float* input;
     float* label;
     float* diff_last;
-    int bf16; /* activations are stored as bfloat16: every layer output and gradient is rounded once */
+    int bf16; /* activations are stored as bfloat16: every layer output and gradient is rounded once, and the
+                 products of forward and backward data take the filter rounded to bfloat16 (the update acts
+                 on the float master copy) */
 };
 
 static size_t src_count(const orc_layer_desc* d) { return (size_t)d->g.n * d->g.c * d->g.h * d->g.w; }
@@ -200,6 +202,16 @@ void orc_net_init_seeded(orc_net* net, uint64_t seed) {
  * dispatch (layer.cu:489-512) */
 void orc_net_set_bf16(orc_net* net, int on) { net->bf16 = on != 0; }
 
+/* the filter as forward / backward data multiply it: the master copy, or its bfloat16 rounding in a scratch copy */
+static const float* product_filter(const orc_net* net, int l, float** scratch) {
+    *scratch = NULL;
+    if (!net->bf16) return net->filter[l];
+    const size_t count = orc_net_filter_count(net, l);
+    *scratch = (float*)malloc(sizeof(float) * count);
+    orc_round_bf16(count, net->filter[l], *scratch);
+    return *scratch;
+}
+
 float orc_net_forward(orc_net* net) {
     if (net->bf16) orc_round_bf16(src_count(&net->L[0]), net->input, net->input);
     for (int l = 0; l < net->num_layers; l++) {
@@ -207,8 +219,8 @@ float orc_net_forward(orc_net* net) {
         const float* src = l == 0 ? net->input : net->dst[l - 1];
         float* dst = net->dst[l];
         switch (d->type) {
-        case T_FC_GEMM: orc_fc_fwd(d->g.n, d->g.c, d->g.k, src, net->filter[l], net->bias[l], dst); break;
-        case T_CONV: case T_FC_CONV: orc_conv_fwd(&d->g, src, net->filter[l], net->bias[l], dst); break;
+        case T_FC_GEMM: { float* tmp; const float* w = product_filter(net, l, &tmp); orc_fc_fwd(d->g.n, d->g.c, d->g.k, src, w, net->bias[l], dst); free(tmp); } break;
+        case T_CONV: case T_FC_CONV: { float* tmp; const float* w = product_filter(net, l, &tmp); orc_conv_fwd(&d->g, src, w, net->bias[l], dst); free(tmp); } break;
         case T_RELU: orc_relu_fwd(src_count(d), src, dst); break;
         case T_TANH: orc_tanh_fwd(src_count(d), src, dst); break;
         case T_SIGMOID: orc_sigmoid_fwd(src_count(d), src, dst); break;
@@ -243,12 +255,12 @@ void orc_net_backward(orc_net* net) {
         float* grad = net->grad[l];
         switch (d->type) {
         case T_FC_GEMM:
-            orc_fc_bwd_data(d->g.n, d->g.c, d->g.k, diff, net->filter[l], grad);
+            { float* tmp; const float* w = product_filter(net, l, &tmp); orc_fc_bwd_data(d->g.n, d->g.c, d->g.k, diff, w, grad); free(tmp); }
             orc_fc_bwd_weight_sgd(d->g.n, d->g.c, d->g.k, src, diff, net->filter[l], alpha);
             orc_fc_bwd_bias_sgd(d->g.n, d->g.k, diff, net->bias[l], alpha);
             break;
         case T_CONV: case T_FC_CONV:
-            orc_conv_bwd_data(&d->g, diff, net->filter[l], grad);
+            { float* tmp; const float* w = product_filter(net, l, &tmp); orc_conv_bwd_data(&d->g, diff, w, grad); free(tmp); }
             orc_conv_bwd_bias_sgd(&d->g, diff, net->bias[l], alpha);
             orc_conv_bwd_filter_sgd(&d->g, src, diff, net->filter[l], alpha);
             break;

@@ -1,7 +1,8 @@
 """GPU parity with bfloat16 activation storage, through the C ABI.
 
-Activation tensors are bfloat16 in memory, parameters float, arithmetic float with float accumulation;
-a result is rounded once when stored. The checker computes the same layer on the same (bfloat16-valued)
+Activation tensors are bfloat16 in memory, parameters float, accumulation float; a result is rounded once when
+stored. Forward and backward data multiply the filter rounded to bfloat16 (nearest even), so that every product
+has two bfloat16 factors and can run on the bfloat16 matrix cores; the update acts on the float master copy. The checker computes the same layer on the same (bfloat16-valued)
 inputs in double and the GPU result must lie within one bfloat16 unit in the last place of it
 (util.assert_close_bf16). ReLU, max-pool and subtraction have exactly representable results: bit-exact.
 """
@@ -100,7 +101,8 @@ def test_conv_bf16(ctx, geom, algo):
     x = rnd(rng, (g.n, g.c, g.h, g.w))
     w = (rng.standard_normal((g.k, g.c, g.r, g.s)) * np.sqrt(2.0 / (g.c * g.r * g.s))).astype(np.float32)
     b = rng.standard_normal(g.k).astype(np.float32)
-    want_y = oracle.conv_fwd(og, x, w, b)
+    wr = oracle.round_bf16(w)  # forward and backward data multiply the filter rounded to bfloat16
+    want_y = oracle.conv_fwd(og, x, wr, b)
     dy = rnd(rng, want_y.shape)
     with Dev(ctx) as d:
         dx_, ddy, dw, db = d.act(x), d.act(dy), d.f32(w), d.f32(b)
@@ -112,7 +114,7 @@ def test_conv_bf16(ctx, geom, algo):
         announce("conv bf16", geom, "algo", algo, "bwd_data")
         p, n = ws(d, g, algo, 1)
         check(lib.vdnn_conv_bwd_data(ctx.handle, None, g, algo, ddy.ptr, dw.ptr, gx.ptr, p, n))
-        assert_close_bf16(get_act(gx, x.shape), oracle.conv_bwd_data(og, dy, w), "bwd data")
+        assert_close_bf16(get_act(gx, x.shape), oracle.conv_bwd_data(og, dy, wr), "bwd data")
         # parameter gradients stay float: the float tolerance applies
         announce("conv bf16", geom, "algo", algo, "bwd_filter")
         gw = d.f32(np.zeros_like(w))
@@ -139,8 +141,8 @@ def test_fc_bf16(ctx, n, cin, cout):
         check(lib.vdnn_fc_bwd_data(ctx.handle, None, n, cin, cout, ddy.ptr, dw.ptr, gx.ptr))
         check(lib.vdnn_fc_bwd_weight(ctx.handle, None, n, cin, cout, dx_.ptr, ddy.ptr, gw.ptr))
         check(lib.vdnn_fc_bwd_bias(ctx.handle, None, n, cout, ddy.ptr, gb.ptr))
-        assert_close_bf16(get_act(y, (n, cout)), oracle.fc_fwd(x, w, b), "fc fwd")
-        assert_close_bf16(get_act(gx, (n, cin)), oracle.fc_bwd_data(dy, w), "fc bwd data")
+        assert_close_bf16(get_act(y, (n, cout)), oracle.fc_fwd(x, oracle.round_bf16(w), b), "fc fwd")
+        assert_close_bf16(get_act(gx, (n, cin)), oracle.fc_bwd_data(dy, oracle.round_bf16(w)), "fc bwd data")
         assert_close(gw.download(w.shape), oracle.fc_bwd_weight_sgd(x, dy, np.zeros_like(w), 1.0), 1e-4, "fc dW")
         assert_close(gb.download(b.shape), oracle.fc_bwd_bias_sgd(dy, np.zeros_like(b), 1.0), 1e-4, "fc db")
 

@@ -118,8 +118,11 @@ def test_policies_are_bit_identical_to_baseline(cnn, batch, algo, bf16):
             assert_bit_identical(got, base, "policy %d lag %d depth %d" % (policy, lag, depth))
 
 
-def layer_forward_on_checker(spec, src, w, b):
-    """The checker's math for one layer on the given input (identical inputs, layer by layer)."""
+def layer_forward_on_checker(spec, src, w, b, bf16=False):
+    """The checker's math for one layer on the given input (identical inputs, layer by layer). With bfloat16
+    activations the products of forward and backward data take the filter rounded to bfloat16."""
+    if bf16 and w is not None:
+        w = oracle.round_bf16(w)
     g = oracle.shape(spec.n, spec.c, spec.h, spec.w, spec.k, spec.r, spec.s, spec.pad_h, spec.pad_w, spec.stride_h, spec.stride_w)
     t = spec.type
     if t in (enums.FC_CONV, enums.CONV):
@@ -141,16 +144,17 @@ def layer_forward_on_checker(spec, src, w, b):
     raise AssertionError(t)
 
 
-def layer_backward_on_checker(spec, src, dst, dy, w, b):
+def layer_backward_on_checker(spec, src, dst, dy, w, b, bf16=False):
     """(dx, w_after, b_after) of one layer from the checker, lr = 1e-5 fused as in layer.cu:593."""
+    wp = oracle.round_bf16(w) if bf16 and w is not None else w  # the filter as backward data multiplies it
     g = oracle.shape(spec.n, spec.c, spec.h, spec.w, spec.k, spec.r, spec.s, spec.pad_h, spec.pad_w, spec.stride_h, spec.stride_w)
     t = spec.type
     alpha = np.float32(1e-5 * -1.0)
     if t in (enums.FC_CONV, enums.CONV):
-        return oracle.conv_bwd_data(g, dy, w), oracle.conv_bwd_filter_sgd(g, src, dy, w, alpha), oracle.conv_bwd_bias_sgd(g, dy, b, alpha)
+        return oracle.conv_bwd_data(g, dy, wp), oracle.conv_bwd_filter_sgd(g, src, dy, w, alpha), oracle.conv_bwd_bias_sgd(g, dy, b, alpha)
     if t == enums.FC_GEMM:
         x2, dy2, w2 = src.reshape(spec.n, -1), dy.reshape(spec.n, -1), w.reshape(spec.k, -1)
-        return (oracle.fc_bwd_data(dy2, w2).reshape(src.shape), oracle.fc_bwd_weight_sgd(x2, dy2, w2, alpha).reshape(w.shape),
+        return (oracle.fc_bwd_data(dy2, wp.reshape(spec.k, -1)).reshape(src.shape), oracle.fc_bwd_weight_sgd(x2, dy2, w2, alpha).reshape(w.shape),
                 oracle.fc_bwd_bias_sgd(dy2, b, alpha))
     if t == enums.RELU:
         return oracle.relu_bwd(src, dst, dy), None, None
@@ -240,7 +244,7 @@ def check_network_against_the_checker(cnn, batch, policy, algo, layers=None, ref
                 spec = net.specs[l]
                 src = (x0 if l == 0 else dst[l - 1]).reshape(net.src_shape(l))
                 w, b = before.get(l, (None, None))
-                want = layer_forward_on_checker(spec, src, w, b)
+                want = layer_forward_on_checker(spec, src, w, b, bf16)
                 exact = spec.type in (enums.RELU, enums.POOL)
                 if exact:
                     assert np.array_equal(dst[l], want), "output of layer %d" % l
@@ -251,7 +255,7 @@ def check_network_against_the_checker(cnn, batch, policy, algo, layers=None, ref
                 dy = (dst[-1] - target) if l == L - 1 else grad[l + 1].reshape(net.dst_shape(l))
                 if bf16 and l == L - 1:
                     dy = oracle.round_bf16(dy)
-                want_dx, want_w, want_b = layer_backward_on_checker(spec, src, dst[l], dy, w, b)
+                want_dx, want_w, want_b = layer_backward_on_checker(spec, src, dst[l], dy, w, b, bf16)
                 if exact and not (bf16 and spec.type == enums.POOL):
                     assert np.array_equal(grad[l], want_dx), "gradient of layer %d" % l
                 elif bf16:

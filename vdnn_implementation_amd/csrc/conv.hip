@@ -10,6 +10,7 @@
 #include "backend_internal.h"
 #include "conv_loaders.h"
 #include "conv_loaders_tap.h"
+#include "mfma_bf16.h"
 #include "conv_smallc.h"
 
 namespace vdnn {
@@ -41,14 +42,14 @@ static bool pixel_tile_span_ok(long sample_elems, int opix, int tile, int elem_b
     return span < 0x7FFF0000l;
 }
 
-static GemmDims make_dims(int M, int N, int K, int TM, int TN, int splits) {
+static GemmDims make_dims(int M, int N, int K, int TM, int TN, int splits, int depth = KB) {
     GemmDims d;
     d.M = M; d.N = N; d.K = K;
     d.mtiles = (M + TM - 1) / TM;
     d.ntiles = (N + TN - 1) / TN;
     if (splits < 1) splits = 1;
     int kchunk = (K + splits - 1) / splits;
-    kchunk = (kchunk + KB - 1) / KB * KB;
+    kchunk = (kchunk + depth - 1) / depth * depth;
     d.kchunk = kchunk;
     d.splits = (K + kchunk - 1) / kchunk;
     d.full_tiles = 0;
@@ -62,8 +63,10 @@ static const PassNames kBwdDataNames{"conv_bwd_data_64x256", "conv_bwd_data_128x
 static const PassNames kBwdFilterNames{"conv_bwd_filter_64x256", "conv_bwd_filter_128x128"};
 static const PassNames kFwdPackedNames{"conv_fwd_packed_64x256", "conv_fwd_packed_128x128"};
 static const PassNames kBwdDataPackedNames{"conv_bwd_data_packed_64x256", "conv_bwd_data_packed_128x128"};
+static const PassNames kFwdHalfNames{"conv_fwd_bf16mfma_64x256", "conv_fwd_bf16mfma_128x128"};
+static const PassNames kBwdDataHalfNames{"conv_bwd_data_bf16mfma_64x256", "conv_bwd_data_bf16mfma_128x128"};
 
-template <int TM, int TN, class AL, class BL, class EP>
+template <int TM, int TN, class AL, class BL, class EP, bool HALF = false>
 static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, const AL& al, const BL& bl, const EP& ep, const GemmDims& d, double flops = 0.0) {
     const long all_tiles = (long)d.mtiles * d.ntiles;
     const long blocks = d.full_tiles > 0 ? d.full_tiles + (all_tiles - d.full_tiles) * d.splits : all_tiles * d.splits;
@@ -71,7 +74,8 @@ static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, con
     // reported work is the algorithmic count where the caller gives one (backward data of a strided or
     // unpadded layer multiplies taps that fall outside the output; they are not counted)
     ProfScope prof(ctx, stream, name, flops > 0.0 ? flops : 2.0 * d.M * (double)d.N * d.K, 0.0);
-    hipLaunchKernelGGL((igemm_kernel<TM, TN, AL, BL, EP>), dim3((unsigned)blocks), dim3(NT), 0, stream, al, bl, ep, d);
+    if constexpr (HALF) hipLaunchKernelGGL((igemm_bf16_kernel<TM, TN, AL, BL, EP>), dim3((unsigned)blocks), dim3(NT), 0, stream, al, bl, ep, d);
+    else hipLaunchKernelGGL((igemm_kernel<TM, TN, AL, BL, EP>), dim3((unsigned)blocks), dim3(NT), 0, stream, al, bl, ep, d);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
@@ -91,20 +95,25 @@ int launch_reduce_splits_nchw(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, co
 // otherwise. A grid that cannot fill the chip (few output pixels: the fully connected layers written
 // as convolutions) splits its reduction; the partial sums go to the staging area and are added in split
 // order, with the bias, by a second kernel. The split count depends on the shape only.
-template <class AL, class BL, class E>
-static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names, const AL& al, const BL& bl, const StoreNCHW<E>& ep, int M, int N, int K, double flops = 0.0) {
+// HALF: the bfloat16 engine (32-deep slices); partial_bytes: room behind ep.partial (the context's staging
+// area unless part of it is taken by something else).
+template <class AL, class BL, class E, bool HALF = false>
+static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names, const AL& al, const BL& bl, const StoreNCHW<E>& ep, int M, int N, int K, double flops = 0.0,
+                       size_t partial_bytes = ~(size_t)0) {
+    constexpr int DEPTH = HALF ? KH : KB;
+    if (partial_bytes == ~(size_t)0) partial_bytes = ctx->reduce_scratch_bytes;
     const bool narrow = M <= 64;
     const int TM = narrow ? 64 : 128, TN = narrow ? 256 : 128;
     const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
     int splits = 1;
     const size_t out_bytes = (size_t)M * N * sizeof(float);
     if (tiles < 2l * ctx->num_cu && ctx->reduce_scratch && ep.partial) {
-        long cap = ((long)K + 8 * KB - 1) / (8 * KB); // at least eight slices per split
-        const long by_mem = (long)(ctx->reduce_scratch_bytes / out_bytes);
+        long cap = ((long)K + 8 * DEPTH - 1) / (8 * DEPTH); // at least eight slices per split
+        const long by_mem = (long)(partial_bytes / out_bytes);
         if (cap > by_mem) cap = by_mem;
         splits = choose_splits(tiles, K, cap, ctx->num_cu, out_bytes, 2.0 * TM * TN * KB);
     }
-    GemmDims d = make_dims(M, N, K, TM, TN, splits);
+    GemmDims d = make_dims(M, N, K, TM, TN, splits, DEPTH);
     // Tail mode: when the tiles make whole rounds of resident workgroups (three per compute unit) plus a
     // small remainder, that remainder would run as a nearly empty last round as long as a full one. Its
     // tiles are split so that together they fill about one round of short workgroups instead.
@@ -113,18 +122,18 @@ static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names
     int tail_tiles = 0;
     if (splits == 1 && tiles > slots && rem > 0 && 2 * rem <= slots && ctx->reduce_scratch && ep.partial) {
         long s = slots / rem;
-        const long by_depth = (long)K / (8 * KB); // at least eight slices per split
-        const long by_mem = (long)(ctx->reduce_scratch_bytes / ((size_t)rem * TM * TN * sizeof(float)));
+        const long by_depth = (long)K / (8 * DEPTH); // at least eight slices per split
+        const long by_mem = (long)(partial_bytes / ((size_t)rem * TM * TN * sizeof(float)));
         if (s > by_depth) s = by_depth;
         if (s > by_mem) s = by_mem;
         if (s >= 2) {
-            d = make_dims(M, N, K, TM, TN, (int)s);
+            d = make_dims(M, N, K, TM, TN, (int)s, DEPTH);
             if (d.splits >= 2) { d.full_tiles = (int)(tiles - rem); tail_tiles = (int)rem; }
-            else d = make_dims(M, N, K, TM, TN, 1);
+            else d = make_dims(M, N, K, TM, TN, 1, DEPTH);
         }
     }
-    const int rc = narrow ? launch_igemm<64, 256>(ctx, stream, names.t64, al, bl, ep, d, flops)
-                          : launch_igemm<128, 128>(ctx, stream, names.t128, al, bl, ep, d, flops);
+    const int rc = narrow ? launch_igemm<64, 256, AL, BL, StoreNCHW<E>, HALF>(ctx, stream, names.t64, al, bl, ep, d, flops)
+                          : launch_igemm<128, 128, AL, BL, StoreNCHW<E>, HALF>(ctx, stream, names.t128, al, bl, ep, d, flops);
     if (rc != VDNN_OK || d.splits == 1) return rc;
     if (tail_tiles > 0)
         return launch_reduce_tail_nchw(ctx, stream, ep.out, ep.partial, tail_tiles, d.splits, TM, TN, M, N, d.mtiles, d.full_tiles, ep.bias, ep.opix, ep.relu, ep.gate);
@@ -171,6 +180,70 @@ static bool packed_bwd_data_ok(const ConvGeo& g) {
     return g.C > 4 && g.sh == 1 && g.sw == 1 && g.R * g.S <= 32 && g.K % KB == 0;
 }
 
+// The bfloat16 engine's filter operand lives at the front of the staging area (rounded and re-laid-out by a
+// small kernel before every use: the master copy changes every step); what is left holds partial sums.
+static bool half_engine_ok(const vdnn_ctx* ctx, int reduced_channels, int RS, size_t filter_elems) {
+    return reduced_channels % KH == 0 && RS <= 32 && ctx->reduce_scratch && filter_elems * 2 + (16u << 20) <= ctx->reduce_scratch_bytes;
+}
+
+static int launch_pack_filter_bf16(vdnn_ctx* ctx, hipStream_t st, const float* w, unsigned short* packed, int rows, int Cred, int RS,
+                                   int row_stride, int red_stride) {
+    const long total = (long)rows * Cred * RS;
+    ProfScope prof(ctx, st, "conv_pack_filter", 0.0, 6.0 * (double)total);
+    hipLaunchKernelGGL(pack_filter_tap_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, packed, rows, Cred, RS,
+                       row_stride, red_stride, total);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
+// Takes bytes from the front of the context's staging area for as long as the object lives; everything that
+// uses the staging area meanwhile (partial sums, intermediate products) sees the remainder.
+struct StagingCarve {
+    vdnn_ctx* ctx;
+    float* base = nullptr;
+    size_t total = 0;
+    bool taken = false;
+    explicit StagingCarve(vdnn_ctx* c) : ctx(c) {}
+    void* take(size_t bytes) {
+        base = ctx->reduce_scratch; total = ctx->reduce_scratch_bytes; taken = true;
+        const size_t t = (bytes + 255) / 256 * 256;
+        ctx->reduce_scratch = (float*)((char*)base + t);
+        ctx->reduce_scratch_bytes = total - t;
+        return base;
+    }
+    ~StagingCarve() { if (taken) { ctx->reduce_scratch = base; ctx->reduce_scratch_bytes = total; } }
+};
+
+__global__ void __launch_bounds__(256) round_filter_bf16_kernel(const float* __restrict__ w, float* __restrict__ out, long count) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) out[i] = round_to_bf16_value(w[i]);
+}
+
+// Layers with bfloat16 activations multiply the filter rounded to bfloat16 (two bfloat16 factors per product)
+// on every route. Routes outside the bfloat16 engine read a rounded float copy, made here at the front of the
+// staging area. Returns null when it does not fit.
+static const float* rounded_filter_copy(vdnn_ctx* ctx, hipStream_t st, StagingCarve& carve, const float* w, size_t count) {
+    if (!ctx->reduce_scratch || count * sizeof(float) + (8u << 20) > ctx->reduce_scratch_bytes) return nullptr;
+    float* wr = (float*)carve.take(count * sizeof(float));
+    hipLaunchKernelGGL(round_filter_bf16_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st, w, wr, (long)count);
+    return wr;
+}
+
+// forward / backward data of a bfloat16 layer on the bfloat16 matrix cores; MODE as in LoadIm2colPixTapH
+template <int MODE>
+static int conv_half_engine(vdnn_ctx* ctx, hipStream_t st, const PassNames& names, const float* w, int rows, int Cred, int RS, int row_stride, int red_stride,
+                            const LoadIm2colPix<MODE, false, bf16_t>& pix, StoreNCHW<bf16_t> ep, int N, double flops) {
+    const size_t filter_elems = (size_t)rows * Cred * RS;
+    unsigned short* packed = (unsigned short*)ctx->reduce_scratch;
+    const size_t taken = (filter_elems * 2 + 255) / 256 * 256;
+    const int rc = launch_pack_filter_bf16(ctx, st, w, packed, rows, Cred, RS, row_stride, red_stride);
+    if (rc != VDNN_OK) return rc;
+    ep.partial = (float*)((char*)ctx->reduce_scratch + taken);
+    LoadPackedH al{packed, (long)Cred * RS, rows, (unsigned)(filter_elems * 2)};
+    LoadIm2colPixTapH<MODE> bl{pix};
+    return launch_by_m<LoadPackedH, LoadIm2colPixTapH<MODE>, bf16_t, true>(ctx, st, names, al, bl, ep, rows, N, Cred * RS, flops, ctx->reduce_scratch_bytes - taken);
+}
+
 static int launch_pack_filter(vdnn_ctx* ctx, hipStream_t st, const float* w, float* packed, int rows, int Cred, int RS,
                               int row_stride, int red_stride) {
     const long total = (long)rows * Cred * RS;
@@ -200,6 +273,22 @@ static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
     hipStream_t st = stream_of(ctx, stream);
     const int K = g.C * g.R * g.S;
     const unsigned wbytes = (unsigned)((long)g.K * K * 4);
+    if constexpr (sizeof(E) == 2) {
+        if (half_engine_ok(ctx, g.C, g.R * g.S, (size_t)g.K * K)) {
+            const int RS = g.R * g.S;
+            LoadIm2colPix<0, false, bf16_t> pix{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N,
+                                               FastDiv::make(RS), FastDiv::make(g.S)};
+            StoreNCHW<bf16_t> ep{y, bias, g.P * g.Q, nullptr, relu, nullptr};
+            return conv_half_engine<0>(ctx, st, kFwdHalfNames, w, g.K, g.C, RS, g.C * RS, RS, pix, ep, g.N * g.P * g.Q,
+                                       2.0 * g.N * (double)g.K * K * g.P * g.Q);
+        }
+    }
+    StagingCarve carve(ctx);
+    if constexpr (sizeof(E) == 2) {
+        w = rounded_filter_copy(ctx, st, carve, w, (size_t)g.K * K);
+        VDNN_REQUIRE(w != nullptr, "filter too large for the staging area (bfloat16 layer outside the bfloat16 engine)");
+        VDNN_LAUNCH_CHECK();
+    }
     if (g.R * g.S <= 32 && g.C % KB == 0) {
         // blocked tap-major reduction: one slice = one tap x 16 input channels
         const int RS = g.R * g.S;
@@ -237,7 +326,18 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
         return gate ? vdnn_fc_bwd_data_relu(ctx, stream, g.N, g.C * g.H * g.W, g.K, dy, w, gate, dx)
                     : vdnn_fc_bwd_data(ctx, stream, g.N, g.C * g.H * g.W, g.K, dy, w, dx);
     hipStream_t st = stream_of(ctx, stream);
-    if (g.C <= 4 && g.R * g.S <= SMALLC_MAXTAPS && !gate) { // the vector-ALU kernels have no gated store
+    StagingCarve carve(ctx);
+    const bool few_channels = g.C <= 4 && g.R * g.S <= SMALLC_MAXTAPS && !gate; // the vector-ALU kernels have no gated store
+    bool half_engine = false;
+    if constexpr (sizeof(E) == 2) {
+        half_engine = !few_channels && g.sh == 1 && g.sw == 1 && half_engine_ok(ctx, g.K, g.R * g.S, (size_t)g.K * g.C * g.R * g.S);
+        if (!half_engine) {
+            w = rounded_filter_copy(ctx, st, carve, w, (size_t)g.K * g.C * g.R * g.S);
+            VDNN_REQUIRE(w != nullptr, "filter too large for the staging area (bfloat16 layer outside the bfloat16 engine)");
+            VDNN_LAUNCH_CHECK();
+        }
+    }
+    if (few_channels) {
         if ((g.sh != 1 || g.sw != 1) && ctx->reduce_scratch && ctx->reduce_scratch_bytes >= (size_t)g.C * g.R * g.S * g.P * g.Q * sizeof(float) &&
                  pixel_tile_span_ok((long)g.K * g.P * g.Q, g.P * g.Q, 256, (int)sizeof(E))) {
             // Strided layer with few input channels (the 11x11 stride-4 first layers): its three or four
@@ -293,6 +393,12 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
     const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S);
     const long sample = (long)g.K * g.P * g.Q;
     const double flops = 2.0 * g.N * (double)g.K * g.C * RS * g.P * g.Q;
+    if constexpr (sizeof(E) == 2) {
+        if (half_engine) {
+            LoadIm2colPix<1, false, bf16_t> pix{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS};
+            return conv_half_engine<1>(ctx, st, kBwdDataHalfNames, w, g.C, g.K, RS, RS, g.C * RS, pix, ep, N, flops);
+        }
+    }
     if (g.sh == 1 && g.sw == 1) {
         if (RS <= 32 && g.K % KB == 0) {
             // blocked tap-major reduction: one slice = one tap x 16 output channels

@@ -12,6 +12,11 @@ int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const f
 
 static inline bool fc_aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
+// The filter operand of forward and backward data: as stored for float activations; rounded to bfloat16 on
+// its way into LDS when the activations are bfloat16 (the products then have two bfloat16 factors).
+template <class L, class E> struct FilterOperand { struct type : L {}; };
+template <class L> struct FilterOperand<L, bf16_t> { typedef RoundedToBf16<L> type; };
+
 // Out[M][N] (dense, row stride N) = alpha * A*B (+ Out) (+ bias per column); the reduction is split into
 // ordered partial sums when the tile grid alone cannot fill the chip.
 template <class AL, class BL, class EO>
@@ -58,11 +63,11 @@ static int fc_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, int
     hipStream_t st = stream_of(ctx, stream);
     if (c_in % 4 == 0 && fc_aligned16(x) && fc_aligned16(w)) {
         LoadDenseRed<true, E> al{x, (long)c_in, n, xb};
-        LoadDenseRed<true> bl{w, (long)c_in, c_out, wb};
+        typename FilterOperand<LoadDenseRed<true>, E>::type bl{{w, (long)c_in, c_out, wb}};
         return fc_gemm(ctx, st, "fc_fwd", al, bl, n, c_out, c_in, y, 1.0f, 0, bias, relu);
     }
     LoadDenseRed<false, E> al{x, (long)c_in, n, xb};
-    LoadDenseRed<false> bl{w, (long)c_in, c_out, wb};
+    typename FilterOperand<LoadDenseRed<false>, E>::type bl{{w, (long)c_in, c_out, wb}};
     return fc_gemm(ctx, st, "fc_fwd", al, bl, n, c_out, c_in, y, 1.0f, 0, bias, relu);
 }
 
@@ -75,7 +80,7 @@ static int fc_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in
     FC_REQUIRE_SMALL((long)n * c_out); FC_REQUIRE_SMALL((long)c_out * c_in);
     const unsigned db = (unsigned)((long)n * c_out * sizeof(E)), wb = (unsigned)((long)c_out * c_in * 4);
     hipStream_t st = stream_of(ctx, stream);
-    LoadDenseRow<float> bl{w, (long)c_in, c_in, wb};
+    typename FilterOperand<LoadDenseRow<float>, E>::type bl{{w, (long)c_in, c_in, wb}};
     if (c_out % 4 == 0 && fc_aligned16(dy)) {
         LoadDenseRed<true, E> al{dy, (long)c_out, n, db};
         return fc_gemm(ctx, st, "fc_bwd_data", al, bl, n, c_in, c_out, dx, 1.0f, 0, nullptr, 0, gate);

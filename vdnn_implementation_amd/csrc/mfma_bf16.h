@@ -1,0 +1,197 @@
+// Tile engine on the bfloat16 matrix cores (v_mfma_f32_32x32x16_bf16: 16x the multiply rate of the float
+// instruction). Used when activations are stored as bfloat16: products of two bfloat16 values are exact in
+// float and the accumulators are float, so against the float engine on the same (bfloat16-valued) operands
+// only the order of summation differs. The filter operand is the float master copy rounded to bfloat16
+// (nearest even) by the packing kernel below.
+//
+// Same tiling as the float engine (256 threads, four 64x64 wave tiles, two LDS buffers) with 32-deep slices.
+// Both operands sit in LDS reduction-major, 32 values (64 bytes) + 16 bytes of padding per row, so that the
+// 128-bit store of eight consecutive reduction values by eight consecutive lanes and the 128-bit fragment
+// read of a 32-row block are both free of bank conflicts. The instruction takes eight reduction values per
+// lane for both operands, so any order of the reduction inside a slice works as long as both sides agree.
+#pragma once
+#include "conv_loaders.h"
+
+namespace vdnn {
+
+constexpr int KH = 32;      // reduction depth of one slice
+constexpr int HSTRIDE = 40; // LDS row stride in 16-bit units
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+
+// ---- dense bfloat16 reduction-major operand: element (row, kk) at base[row*ld + kk] --------------------
+// thread t: values 8*(t%4) .. +7 of rows t/4 + 64*i, one 128-bit load each
+struct LoadPackedH {
+    const unsigned short* base;
+    long ld;        // elements between rows (a multiple of 8)
+    int rows;
+    unsigned bytes; // below 2 GiB
+    template <int T> struct Regs { uintx4 v[T / 64]; };
+    template <int T> struct State { int vrow[T / 64]; __amdgpu_buffer_rsrc_t rsrc; };
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int row0, int tid, int, int) const {
+        st.rsrc = make_rsrc(base, bytes);
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) {
+            const int row = row0 + (tid >> 2) + 64 * i;
+            st.vrow[i] = row < rows ? (int)(((long)row * ld + 8 * (tid & 3)) * 2) : OOB;
+        }
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int kk0, int, int, Regs<T>& r) const {
+        const int soff = kk0 * 2;
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) r.v[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(st.rsrc, st.vrow[i], soff, 0));
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(unsigned short* lds, int tid, const Regs<T>& r) {
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) *(uintx4*)(lds + ((tid >> 2) + 64 * i) * HSTRIDE + 8 * (tid & 3)) = r.v[i];
+    }
+};
+
+// ---- im2col operand, columns = output pixels, blocked tap-major reduction (32 channels per tap) ------
+// MODE 0: forward gather from x; MODE 1: backward data at stride 1 (src = dy). A lane owns one pixel
+// (consecutive lanes, consecutive pixels: every 16-bit load of a wavefront covers one run of a plane) and
+// fetches eight consecutive channels of it per item, packed into one 128-bit LDS store.
+template <int MODE>
+struct LoadIm2colPixTapH {
+    LoadIm2colPix<MODE, false, bf16_t> base; // geometry and per-pixel state of the float engine's loader
+    template <int T> struct Regs { uintx4 v[T / 64]; };
+    template <int T> using State = typename LoadIm2colPix<MODE, false, bf16_t>::template State<T>;
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int j0, int tid, int ncols, int k_begin) const {
+        base.template init<T>(st, j0, tid, ncols, k_begin);
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int kk0, int, int tid, Regs<T>& r) const {
+        const int plane = base.Hs * base.Ws;
+        const int slice = kk0 / KH;
+        const int cb = base.divRS.div(slice), tap = slice - cb * (base.R * base.S);
+        const int tr = base.divS.div(tap), ts = tap - tr * base.S;
+        const int tapoff = MODE == 0 ? tr * base.Ws + ts : (base.R - 1 - tr) * base.Ws + (base.S - 1 - ts);
+        const int voff = st.vbase | bit_to_all_ones(st.inv, tap);
+        const int g0 = __builtin_amdgcn_readfirstlane(tid / T);
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) {
+            const int ch = cb * KH + 8 * (g0 + (NT / T) * i);
+            const int soff = (ch * plane + tapoff) * 2, step = plane * 2;
+            unsigned h[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) h[e] = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(st.rsrc, voff, soff + e * step, 0);
+            r.v[i].x = h[0] | (h[1] << 16); r.v[i].y = h[2] | (h[3] << 16);
+            r.v[i].z = h[4] | (h[5] << 16); r.v[i].w = h[6] | (h[7] << 16);
+        }
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(unsigned short* lds, int tid, const Regs<T>& r) {
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) *(uintx4*)(lds + (tid % T) * HSTRIDE + 8 * (tid / T + (NT / T) * i)) = r.v[i];
+    }
+};
+
+// Filter bank rounded to bfloat16 and re-laid-out for the blocked tap-major order:
+// packed[row][(cb*RS + tap)*32 + l] = bf16(w[row*row_stride + (cb*32 + l)*red_stride + tap])
+//   forward:       rows = output channels, reduced channels = input channels:  row_stride = C*RS, red_stride = RS
+//   backward data: rows = input channels,  reduced channels = output channels: row_stride = RS,   red_stride = C*RS
+__global__ void __launch_bounds__(256) pack_filter_tap_bf16_kernel(const float* __restrict__ w, unsigned short* __restrict__ packed,
+                                                                   int rows, int Cred, int RS, int row_stride, int red_stride, long total) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int per_row = Cred * RS;
+    const int row = (int)(i / per_row), kk = (int)(i - (long)row * per_row);
+    const int l = kk & 31, slice = kk >> 5;
+    const int cb = slice / RS, tap = slice - cb * RS;
+    packed[i] = float_to_bf16_bits(w[(long)row * row_stride + (long)(cb * 32 + l) * red_stride + tap]);
+}
+
+// Out tile = A tile x B tile over this workgroup's share of the reduction; tile decoding and epilogues are
+// those of the float engine (igemm_kernel), slices are KH deep.
+template <int TM, int TN, class AL, class BL, class EP>
+__global__ void __launch_bounds__(NT) igemm_bf16_kernel(const AL al, const BL bl, const EP ep, const GemmDims d) {
+    static_assert(TM % 64 == 0 && TN % 64 == 0 && (TM / 64) * (TN / 64) == 4, "four 64x64 wave tiles");
+    __shared__ __attribute__((aligned(16))) unsigned short As[2][TM * HSTRIDE];
+    __shared__ __attribute__((aligned(16))) unsigned short Bs[2][TN * HSTRIDE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int ntiles_all = d.mtiles * d.ntiles;
+    int tile, ks;
+    bool whole;
+    if ((int)blockIdx.x < d.full_tiles) {
+        tile = xcd_remap(blockIdx.x, d.full_tiles); ks = 0; whole = true;
+    } else if (d.full_tiles > 0) {
+        const int r = blockIdx.x - d.full_tiles, tl = ntiles_all - d.full_tiles;
+        tile = d.full_tiles + r % tl; ks = r / tl; whole = false;
+    } else {
+        const int bid = xcd_remap(blockIdx.x, gridDim.x);
+        tile = bid % ntiles_all; ks = bid / ntiles_all; whole = d.splits == 1;
+    }
+    const int mt = tile % d.mtiles, nt = tile / d.mtiles;
+    const int m0 = mt * TM, j0 = nt * TN;
+    const int k_begin = whole ? 0 : ks * d.kchunk;
+    const int k_end = whole ? d.K : min(d.K, k_begin + d.kchunk);
+
+    typename AL::template State<TM> sa;
+    typename BL::template State<TN> sb;
+    al.template init<TM>(sa, m0, tid, d.M, k_begin);
+    bl.template init<TN>(sb, j0, tid, d.N, k_begin);
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    const int wm0 = (wave % (TM / 64)) * 64, wn0 = (wave / (TM / 64)) * 64;
+    const int l32 = lane & 31, lk = lane >> 5;
+    typename AL::template Regs<TM> ra;
+    typename BL::template Regs<TN> rb;
+
+    // slice s is multiplied from LDS buffer s%2 while slice s+1 (fetched during slice s-1) is written to the
+    // other buffer and slice s+2 is fetched; one barrier per slice. Fetches past the end of the range are
+    // never used (buffer loads cannot fault).
+    const int nslices = (k_end - k_begin + KH - 1) / KH;
+    al.template load<TM>(sa, k_begin, k_end, tid, ra);
+    bl.template load<TN>(sb, k_begin, k_end, tid, rb);
+    AL::template store<TM>(As[0], tid, ra);
+    BL::template store<TN>(Bs[0], tid, rb);
+    al.template load<TM>(sa, k_begin + KH, k_end, tid, ra);
+    bl.template load<TN>(sb, k_begin + KH, k_end, tid, rb);
+    __syncthreads();
+    for (int s = 0; s < nslices; s++) {
+        const int cur = s & 1, nxt = cur ^ 1;
+        const unsigned short* ap = As[cur] + (wm0 + l32) * HSTRIDE + 8 * lk;
+        const unsigned short* bp = Bs[cur] + (wn0 + l32) * HSTRIDE + 8 * lk;
+        bf16x8 a[2][2], b[2][2];
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                a[h][i] = *(const bf16x8*)(ap + i * 32 * HSTRIDE + 16 * h);
+                b[h][i] = *(const bf16x8*)(bp + i * 32 * HSTRIDE + 16 * h);
+            }
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[h][i], b[h][j], acc[i][j], 0, 0, 0);
+        AL::template store<TM>(As[nxt], tid, ra);
+        BL::template store<TN>(Bs[nxt], tid, rb);
+        __syncthreads();
+        const int kk0 = k_begin + (s + 2) * KH;
+        al.template load<TM>(sa, kk0, k_end, tid, ra);
+        bl.template load<TN>(sb, kk0, k_end, tid, rb);
+    }
+
+    if (EP::TAIL && d.full_tiles > 0 && !whole)
+        ep.store_tail(acc, wm0, wn0, lane, (long)(tile - d.full_tiles) * d.splits + ks, TM, TN);
+    else
+        ep.store(acc, m0 + wm0, j0 + wn0, lane, ks, d, !whole);
+}
+
+} // namespace vdnn

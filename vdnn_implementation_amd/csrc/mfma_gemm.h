@@ -390,6 +390,23 @@ struct LoadDenseRow {
     }
 };
 
+// the float nearest to v among those exactly representable in bfloat16 (ties to even, NaN stays NaN)
+__device__ __forceinline__ float round_to_bf16_value(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
+
+// An operand whose values are rounded to bfloat16 on their way into LDS: the filter operands of layers whose
+// activations are stored as bfloat16 (the filter itself stays a float master copy in memory).
+template <class L>
+struct RoundedToBf16 : L {
+    template <int T>
+    __device__ static __forceinline__ void store(float* lds, int tid, const typename L::template Regs<T>& r) {
+        typename L::template Regs<T> q = r;
+        float* f = (float*)&q;
+#pragma unroll
+        for (int i = 0; i < (int)(sizeof(q) / sizeof(float)); i++) f[i] = round_to_bf16_value(f[i]);
+        L::template store<T>(lds, tid, q);
+    }
+};
+
 // ---- dense result: out[m*ld_m + j] = alpha*acc (+ old if accumulate) (+ bias[j]); or a split's
 //      partial sums to scratch[ks][m*ld_m + j] ------------------------------------------------------
 template <class E = float>
