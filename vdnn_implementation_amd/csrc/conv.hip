@@ -65,6 +65,7 @@ static const PassNames kFwdPackedNames{"conv_fwd_packed_64x256", "conv_fwd_packe
 static const PassNames kBwdDataPackedNames{"conv_bwd_data_packed_64x256", "conv_bwd_data_packed_128x128"};
 static const PassNames kFwdHalfNames{"conv_fwd_bf16mfma_64x256", "conv_fwd_bf16mfma_128x128"};
 static const PassNames kBwdDataHalfNames{"conv_bwd_data_bf16mfma_64x256", "conv_bwd_data_bf16mfma_128x128"};
+static const PassNames kBwdFilterHalfNames{"conv_bwd_filter_bf16mfma_64x256", "conv_bwd_filter_bf16mfma_128x128"};
 
 template <int TM, int TN, class AL, class BL, class EP, bool HALF = false>
 static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, const AL& al, const BL& bl, const EP& ep, const GemmDims& d, double flops = 0.0) {
@@ -494,6 +495,35 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     // tap-major column order when the tile's columns fall into whole groups of channels with one tap each
     const int tile_n = narrow ? 256 : 128;
     const int ntap = g.C % tile_n == 0 ? 1 : (g.C % (tile_n / 2) == 0 ? 2 : (g.C % (tile_n / 4) == 0 ? 4 : 0));
+    if constexpr (sizeof(E) == 2) {
+        // bfloat16 activations: both factors of every product are bfloat16 already
+        if (vec && ntap != 0 && PQ >= KH && 3 * g.Q >= KH && g.Q % 2 == 0 && ((uintptr_t)x & 3) == 0 && staging) {
+            long caph = (Kred + 4 * KH - 1) / (4 * KH);
+            if (caph > by_mem) caph = by_mem;
+            const int wanth = choose_splits(tiles, Kred, caph, ctx->num_cu, out_bytes, 2.0 * TM * TN * KB);
+            GemmDims dh = make_dims(M, N, (int)Kred, TM, TN, wanth, KH);
+            const long nspanh = dh.kchunk / PQ + 2;
+            if (nspanh * g.K * PQ * 2 < (long)MAX_SUM_RANGE && nspanh * g.C * g.H * g.W * 2 < (long)MAX_SUM_RANGE) {
+                const FastDiv dC = FastDiv::make(g.C);
+                StoreFilterTap ept{w, staging, g.C, RS, (long)M * N, alpha, accumulate, dC};
+                LoadDyRedIncH al{dy, g.N, g.K, PQ, dh.kchunk, dh.K};
+                int rch;
+#define VDNN_WGRAD_TAP_H(NTAP)                                                                                              \
+                do {                                                                                                        \
+                    LoadIm2colRedTapH<NTAP> bl{x, g.N, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N, dh.kchunk, dh.K, dC, dS}; \
+                    rch = narrow ? launch_igemm<64, 256, LoadDyRedIncH, LoadIm2colRedTapH<NTAP>, StoreFilterTap, true>(ctx, st, kBwdFilterHalfNames.t64, al, bl, ept, dh) \
+                                 : launch_igemm<128, 128, LoadDyRedIncH, LoadIm2colRedTapH<NTAP>, StoreFilterTap, true>(ctx, st, kBwdFilterHalfNames.t128, al, bl, ept, dh); \
+                } while (0)
+                if (ntap == 1) VDNN_WGRAD_TAP_H(1);
+                else if (ntap == 2) VDNN_WGRAD_TAP_H(2);
+                else VDNN_WGRAD_TAP_H(4);
+#undef VDNN_WGRAD_TAP_H
+                if (rch != VDNN_OK) return rch;
+                if (dh.splits > 1) return launch_reduce_splits_tap(ctx, st, w, staging, (size_t)M * N, dh.splits, alpha, accumulate, g.C, RS);
+                return VDNN_OK;
+            }
+        }
+    }
     if (vec && ntap != 0 && PQ >= KB && 2 * g.Q >= KB) {
         const FastDiv dC = FastDiv::make(g.C);
         StoreFilterTap ept{w, staging, g.C, RS, (long)M * N, alpha, accumulate, dC};

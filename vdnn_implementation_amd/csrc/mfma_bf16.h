@@ -195,3 +195,134 @@ __global__ void __launch_bounds__(NT) igemm_bf16_kernel(const AL al, const BL bl
 }
 
 } // namespace vdnn
+
+namespace vdnn {
+
+typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
+
+// ---- backward filter on the bfloat16 matrix cores: the reduction runs over output pixels (n, p, q) ----
+// dy as A[k][(n,p,q)]: thread t fetches pixels 4*(t%8) .. +3 (64 bits) of rows t/8 + 32*i. The byte offset is
+// carried from slice to slice with adds and selects (P*Q >= 32: at most one sample wrap per step; P*Q a
+// multiple of four). Pixels past the end of the reduction lie beyond the descriptor's range: zero.
+struct LoadDyRedIncH {
+    const bf16_t* dy;
+    int N, K, PQ;
+    int kchunk, Ktot;
+    template <int T> struct Regs { uintx2 v[T / 32]; };
+    template <int T> struct State { int mrow[T / 32]; int pq, off; __amdgpu_buffer_rsrc_t rsrc; };
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int row0, int tid, int, int k_begin) const {
+        const int n_first = k_begin / PQ;
+        int k_last = k_begin + kchunk; if (k_last > Ktot) k_last = Ktot;
+        const int n_last = k_last > k_begin ? (k_last - 1) / PQ : n_first;
+        st.rsrc = make_rsrc(dy + (long)n_first * K * PQ, clamp_range((long)(n_last - n_first + 1) * K * PQ * 2));
+        const int kk = k_begin + 4 * (tid & 7);
+        const int n = kk / PQ;
+        st.pq = kk - n * PQ;
+        st.off = (int)(((long)(n - n_first) * K * PQ + st.pq) * 2);
+#pragma unroll
+        for (int i = 0; i < T / 32; i++) { const int m = row0 + (tid >> 3) + 32 * i; st.mrow[i] = m < K ? m * PQ * 2 : SENT; }
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int, int, int, Regs<T>& r) const {
+#pragma unroll
+        for (int i = 0; i < T / 32; i++) r.v[i] = __builtin_bit_cast(uintx2, __builtin_amdgcn_raw_buffer_load_b64(st.rsrc, st.mrow[i] + st.off, 0, 0));
+        st.pq += KH;
+        const bool wrap = st.pq >= PQ;
+        st.pq -= wrap ? PQ : 0;
+        st.off += wrap ? (KH + (K - 1) * PQ) * 2 : KH * 2;
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(unsigned short* lds, int tid, const Regs<T>& r) {
+#pragma unroll
+        for (int i = 0; i < T / 32; i++) *(uintx2*)(lds + ((tid >> 3) + 32 * i) * HSTRIDE + 4 * (tid & 7)) = r.v[i];
+    }
+};
+
+// im2col operand in tap-major column order (as LoadIm2colRedTap): B[(tap, c)][(n,p,q)]. Thread t owns the
+// pixel pair 2*(t%16), +1 of the slice (both in one output row: Q is even) and the columns t/16 + 16*i; the two
+// 16-bit values of a column are packed into one LDS word. The pair's input row / column / byte offset are
+// carried from slice to slice (Q >= 11: at most three row wraps per 32 pixels; P*Q >= 32: one sample wrap).
+template <int NTAP>
+struct LoadIm2colRedTapH {
+    const bf16_t* x;
+    int N, C, H, W, R, S, P, Q, ph, pw, sh, sw;
+    int ncols; // C*R*S
+    int kchunk, Ktot;
+    FastDiv divC, divS;
+    template <int T> struct Regs { unsigned s[T / 16]; };
+    template <int T> struct State {
+        int ih, iw;   // input row / column of the pair's first pixel through the first group's tap
+        int off;      // byte offset of that element in the thread's first channel plane
+        int dih[NTAP], diw[NTAP], doff[NTAP];
+        int iw_wrap, ih_wrap;
+        __amdgpu_buffer_rsrc_t rsrc;
+    };
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int j0, int tid, int, int k_begin) const {
+        const int PQ = P * Q;
+        const int n_first = k_begin / PQ;
+        const long chw = (long)C * H * W;
+        const long shift = -((long)ph * W + pw);
+        int k_last = k_begin + kchunk; if (k_last > Ktot) k_last = Ktot;
+        const int n_last = k_last > k_begin ? (k_last - 1) / PQ : n_first;
+        st.rsrc = make_rsrc(x + (long)n_first * chw + shift, clamp_range(((long)(n_last - n_first + 1) * chw - shift) * 2));
+        const int kk = k_begin + 2 * (tid & 15);
+        const int n = kk / PQ, pq = kk - n * PQ;
+        const int p = pq / Q, q = pq - p * Q;
+        int r0 = 0, s0 = 0, c0 = 0;
+#pragma unroll
+        for (int g = 0; g < NTAP; g++) {
+            const int jg = j0 + g * (T / NTAP);
+            const int tap = divC.div(jg);
+            const int r = divS.div(tap), s_ = tap - r * S;
+            const int c = jg - tap * C;
+            if (g == 0) { r0 = r; s0 = s_; c0 = c; st.dih[0] = 0; st.diw[0] = 0; st.doff[0] = 0; }
+            else {
+                st.dih[g] = jg < ncols ? r - r0 : 0x20000000;
+                st.diw[g] = s_ - s0;
+                st.doff[g] = (((r - r0) * W + (s_ - s0)) + (c - c0) * H * W) * 2;
+            }
+        }
+        st.ih = p * sh - ph + r0; st.iw = q * sw - pw + s0;
+        st.iw_wrap = Q * sw - pw + s0; st.ih_wrap = P * sh - ph + r0;
+        st.off = (int)(((long)(n - n_first) * chw + (long)(c0 + (tid >> 4)) * H * W + (long)(p * sh + r0) * W + q * sw + s0) * 2);
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int, int, int, Regs<T>& r) const {
+        int base0[NTAP], base1[NTAP];
+#pragma unroll
+        for (int g = 0; g < NTAP; g++) {
+            const int ih = g == 0 ? st.ih : st.ih + st.dih[g], iw = g == 0 ? st.iw : st.iw + st.diw[g];
+            const int o = g == 0 ? st.off : st.off + st.doff[g];
+            const bool row_ok = (unsigned)ih < (unsigned)H;
+            base0[g] = o | ((row_ok & ((unsigned)iw < (unsigned)W)) ? 0 : SENT);
+            base1[g] = (o + sw * 2) | ((row_ok & ((unsigned)(iw + sw) < (unsigned)W)) ? 0 : SENT);
+        }
+        constexpr int PERG = T / 16 / NTAP;
+        const int plane16 = 16 * H * W * 2;
+#pragma unroll
+        for (int i = 0; i < T / 16; i++) {
+            const unsigned lo = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(st.rsrc, base0[i / PERG], (i % PERG) * plane16, 0);
+            const unsigned hi = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(st.rsrc, base1[i / PERG], (i % PERG) * plane16, 0);
+            r.s[i] = lo | (hi << 16);
+        }
+        // next slice: KH pixels further
+        st.iw += KH * sw; st.off += KH * sw * 2;
+        const int qsw = Q * sw;
+        const int wraps = (st.iw >= st.iw_wrap ? 1 : 0) + (st.iw >= st.iw_wrap + qsw ? 1 : 0) + (st.iw >= st.iw_wrap + 2 * qsw ? 1 : 0);
+        st.iw -= __mul24(wraps, qsw);
+        st.ih += __mul24(wraps, sh);
+        st.off += __mul24(wraps, (sh * W - qsw) * 2);
+        const bool next = st.ih >= st.ih_wrap;
+        st.ih -= next ? P * sh : 0;
+        st.off += next ? (C * H * W - P * sh * W) * 2 : 0;
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(unsigned short* lds, int tid, const Regs<T>& r) {
+#pragma unroll
+        for (int i = 0; i < T / 16; i++) *(unsigned*)(lds + ((tid >> 4) + 16 * i) * HSTRIDE + 2 * (tid & 15)) = r.s[i];
+    }
+};
+
+} // namespace vdnn
