@@ -66,7 +66,11 @@ typedef struct {
 int vdnn_ctx_create(vdnn_ctx** out, int device, int flags);
 int vdnn_ctx_destroy(vdnn_ctx* ctx);
 /* Element type of the activation tensors handed to later kernel calls on this context (default
- * VDNN_DTYPE_F32). No counterpart in the reference (CUDNN_DATA_FLOAT is fixed, vdnn.h:12). */
+ * VDNN_DTYPE_F32). No counterpart in the reference (CUDNN_DATA_FLOAT is fixed, vdnn.h:12).
+ * With VDNN_DTYPE_BF16 the products of forward and backward data (convolution and FC) take the filter
+ * rounded to bfloat16, nearest even, so that both factors are bfloat16 and the bfloat16 matrix cores can form
+ * them exactly; accumulation, biases, parameter gradients and the parameters in memory stay float, and the
+ * update acts on the float values. Backward filter multiplies two activation tensors and rounds nothing. */
 int vdnn_ctx_set_activation_dtype(vdnn_ctx* ctx, int dtype);
 int vdnn_ctx_activation_dtype(vdnn_ctx* ctx);
 const char* vdnn_last_error(void);

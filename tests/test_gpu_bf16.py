@@ -90,6 +90,12 @@ CONV = [
     (2, 48, 27, 27, 96, 5, 5, 2, 2, 1, 1),     # AlexNet conv2
     (5, 64, 6, 6, 200, 6, 6, 0, 0, 1, 1),      # OverFeat 6x6 -> 1x1
     (1, 16, 20, 24, 32, 3, 5, 1, 2, 2, 1),     # asymmetric, strided backward data
+    # the bfloat16 matrix-core engine (reduced channels a multiple of 32):
+    (6, 96, 27, 27, 160, 5, 5, 2, 2, 1, 1),    # 25 taps, three channel blocks, ragged row and column tiles
+    (4, 32, 12, 20, 64, 3, 3, 1, 1, 2, 2),     # strided: the engine in forward and backward filter only
+    (3, 64, 16, 22, 96, 3, 3, 0, 0, 1, 1),     # no padding, plane not a multiple of the slice
+    (9, 256, 14, 14, 64, 3, 3, 1, 1, 1, 1),    # 14x14: three row wraps per slice in backward filter; forward splits its reduction
+    (2, 64, 40, 36, 64, 1, 1, 0, 0, 1, 1),     # 1x1 window
 ]
 
 
@@ -223,3 +229,44 @@ def test_lrn_softmax_and_loss_bf16(ctx):
         check(lib.vdnn_cross_entropy_dense(ctx.handle, None, n, classes, prob.ptr, dt.ptr, loss.ptr))
         want = float(np.mean(-np.log(gp[np.arange(n), labels].astype(np.float64))))
         assert abs(loss.download((1,))[0] - want) <= 1e-5 * abs(want)
+
+
+def test_bf16_engine_in_a_split_last_round_agrees_with_two_half_batches(ctx):
+    """VGG16's 14x14 layers at batch 128 on the bfloat16 engine: 784 tiles for 768 resident workgroups, the last 16
+    split along the reduction. No CPU result is affordable at this size; convolution is independent per sample,
+    so the two half batches (another launch geometry) must give the same values up to one rounding of the
+    differently ordered float sums."""
+    geom, half = (128, 512, 14, 14, 512, 3, 3, 1, 1, 1, 1), (64, 512, 14, 14, 512, 3, 3, 1, 1, 1, 1)
+    g, gh = be.shape(*geom), be.shape(*half)
+    rng = np.random.default_rng(31)
+    x = rnd(rng, (128, 512, 14, 14))
+    w = (rng.standard_normal((512, 512, 3, 3)) * np.sqrt(2.0 / 4608)).astype(np.float32)
+    b = rng.standard_normal(512).astype(np.float32)
+    dy = rnd(rng, (128, 512, 14, 14))
+    with Dev(ctx) as d:
+        dx_, ddy, dw, db = d.act(x), d.act(dy), d.f32(w), d.f32(b)
+        y, gx = d.empty_act(x.shape), d.empty_act(x.shape)
+        announce("bf16 engine, split last round, whole batch")
+        check(lib.vdnn_conv_fwd(ctx.handle, None, g, 0, dx_.ptr, dw.ptr, db.ptr, y.ptr, None, 0))
+        check(lib.vdnn_conv_bwd_data(ctx.handle, None, g, 0, ddy.ptr, dw.ptr, gx.ptr, None, 0))
+        whole_y, whole_gx = get_act(y, x.shape), get_act(gx, x.shape)
+        halves_y, halves_gx = [], []
+        for i in range(2):
+            hx, hdy = d.act(x[64 * i:64 * i + 64]), d.act(dy[64 * i:64 * i + 64])
+            hy, hgx = d.empty_act((64, 512, 14, 14)), d.empty_act((64, 512, 14, 14))
+            announce("bf16 engine, split last round, half", i)
+            check(lib.vdnn_conv_fwd(ctx.handle, None, gh, 0, hx.ptr, dw.ptr, db.ptr, hy.ptr, None, 0))
+            check(lib.vdnn_conv_bwd_data(ctx.handle, None, gh, 0, hdy.ptr, dw.ptr, hgx.ptr, None, 0))
+            halves_y.append(get_act(hy, (64, 512, 14, 14))); halves_gx.append(get_act(hgx, (64, 512, 14, 14)))
+    assert_close_bf16(whole_y, np.concatenate(halves_y), "forward, whole batch against two halves")
+    assert_close_bf16(whole_gx, np.concatenate(halves_gx), "backward data, whole batch against two halves")
+    # a few output elements against the definition in double, with the filter rounded to bfloat16
+    wr = oracle.round_bf16(w).astype(np.float64)
+    for (n, k, p, q) in ((0, 0, 0, 0), (127, 511, 13, 13), (77, 300, 6, 0), (127, 5, 0, 13)):
+        acc = float(b[k])
+        for r in range(3):
+            for s_ in range(3):
+                ih, iw = p - 1 + r, q - 1 + s_
+                if 0 <= ih < 14 and 0 <= iw < 14:
+                    acc += float(np.dot(x[n, :, ih, iw].astype(np.float64), wr[k, :, r, s_]))
+        assert abs(whole_y[n, k, p, q] - acc) <= 2.0 ** -7 * max(abs(acc), 1e-3)
