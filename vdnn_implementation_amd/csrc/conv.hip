@@ -241,6 +241,11 @@ static int conv_half_engine(vdnn_ctx* ctx, hipStream_t st, const PassNames& name
     if (rc != VDNN_OK) return rc;
     ep.partial = (float*)((char*)ctx->reduce_scratch + taken);
     LoadPackedH al{packed, (long)Cred * RS, rows, (unsigned)(filter_elems * 2)};
+    // a pixel pair per lane where the pairs of an output row are contiguous in the input
+    if (pix.OW % 2 == 0 && pix.S <= 16 && pix.Ws >= pix.S && pix.Ws > pix.pw + 1 && (MODE == 1 || pix.sw == 1)) {
+        LoadIm2colPixTapH2<MODE> bl2{pix};
+        return launch_by_m<LoadPackedH, LoadIm2colPixTapH2<MODE>, bf16_t, true>(ctx, st, names, al, bl2, ep, rows, N, Cred * RS, flops, ctx->reduce_scratch_bytes - taken);
+    }
     LoadIm2colPixTapH<MODE> bl{pix};
     return launch_by_m<LoadPackedH, LoadIm2colPixTapH<MODE>, bf16_t, true>(ctx, st, names, al, bl, ep, rows, N, Cred * RS, flops, ctx->reduce_scratch_bytes - taken);
 }
@@ -510,6 +515,12 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
                 int rch;
 #define VDNN_WGRAD_TAP_H(NTAP)                                                                                              \
                 do {                                                                                                        \
+                    if (g.sw == 1) {                                                                                        \
+                        LoadIm2colRedTapH<NTAP, true> bl{x, g.N, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N, dh.kchunk, dh.K, dC, dS}; \
+                        rch = narrow ? launch_igemm<64, 256, LoadDyRedIncH, LoadIm2colRedTapH<NTAP, true>, StoreFilterTap, true>(ctx, st, kBwdFilterHalfNames.t64, al, bl, ept, dh) \
+                                     : launch_igemm<128, 128, LoadDyRedIncH, LoadIm2colRedTapH<NTAP, true>, StoreFilterTap, true>(ctx, st, kBwdFilterHalfNames.t128, al, bl, ept, dh); \
+                        break;                                                                                              \
+                    }                                                                                                       \
                     LoadIm2colRedTapH<NTAP> bl{x, g.N, g.C, g.H, g.W, g.R, g.S, g.P, g.Q, g.ph, g.pw, g.sh, g.sw, N, dh.kchunk, dh.K, dC, dS}; \
                     rch = narrow ? launch_igemm<64, 256, LoadDyRedIncH, LoadIm2colRedTapH<NTAP>, StoreFilterTap, true>(ctx, st, kBwdFilterHalfNames.t64, al, bl, ept, dh) \
                                  : launch_igemm<128, 128, LoadDyRedIncH, LoadIm2colRedTapH<NTAP>, StoreFilterTap, true>(ctx, st, kBwdFilterHalfNames.t128, al, bl, ept, dh); \

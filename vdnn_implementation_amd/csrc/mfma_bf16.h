@@ -243,7 +243,7 @@ struct LoadDyRedIncH {
 // pixel pair 2*(t%16), +1 of the slice (both in one output row: Q is even) and the columns t/16 + 16*i; the two
 // 16-bit values of a column are packed into one LDS word. The pair's input row / column / byte offset are
 // carried from slice to slice (Q >= 11: at most three row wraps per 32 pixels; P*Q >= 32: one sample wrap).
-template <int NTAP>
+template <int NTAP, bool PAIR32 = false>
 struct LoadIm2colRedTapH {
     const bf16_t* x;
     int N, C, H, W, R, S, P, Q, ph, pw, sh, sw;
@@ -266,7 +266,10 @@ struct LoadIm2colRedTapH {
         const long shift = -((long)ph * W + pw);
         int k_last = k_begin + kchunk; if (k_last > Ktot) k_last = Ktot;
         const int n_last = k_last > k_begin ? (k_last - 1) / PQ : n_first;
-        st.rsrc = make_rsrc(x + (long)n_first * chw + shift, clamp_range(((long)(n_last - n_first + 1) * chw - shift) * 2));
+        // the descriptor's base is kept four-byte aligned (x is): the 32-bit pair loads rely on it
+        const long base_e = (long)n_first * chw + shift;
+        const int odd = (int)(base_e & 1);
+        st.rsrc = make_rsrc(x + base_e - odd, clamp_range(((long)(n_last - n_first + 1) * chw - shift + odd) * 2));
         const int kk = k_begin + 2 * (tid & 15);
         const int n = kk / PQ, pq = kk - n * PQ;
         const int p = pq / Q, q = pq - p * Q;
@@ -286,26 +289,46 @@ struct LoadIm2colRedTapH {
         }
         st.ih = p * sh - ph + r0; st.iw = q * sw - pw + s0;
         st.iw_wrap = Q * sw - pw + s0; st.ih_wrap = P * sh - ph + r0;
-        st.off = (int)(((long)(n - n_first) * chw + (long)(c0 + (tid >> 4)) * H * W + (long)(p * sh + r0) * W + q * sw + s0) * 2);
+        st.off = (int)(((long)(n - n_first) * chw + (long)(c0 + (tid >> 4)) * H * W + (long)(p * sh + r0) * W + q * sw + s0 + odd) * 2);
     }
     template <int T>
     __device__ __forceinline__ void load(State<T>& st, int, int, int, Regs<T>& r) const {
         int base0[NTAP], base1[NTAP];
+        unsigned keep[NTAP]; // PAIR32: which halves of the loaded word lie inside the image
+        int down[NTAP];      // PAIR32: 16 when the word was fetched one element lower
 #pragma unroll
         for (int g = 0; g < NTAP; g++) {
             const int ih = g == 0 ? st.ih : st.ih + st.dih[g], iw = g == 0 ? st.iw : st.iw + st.diw[g];
             const int o = g == 0 ? st.off : st.off + st.doff[g];
             const bool row_ok = (unsigned)ih < (unsigned)H;
-            base0[g] = o | ((row_ok & ((unsigned)iw < (unsigned)W)) ? 0 : SENT);
-            base1[g] = (o + sw * 2) | ((row_ok & ((unsigned)(iw + sw) < (unsigned)W)) ? 0 : SENT);
+            const bool ok0 = (unsigned)iw < (unsigned)W, ok1 = (unsigned)(iw + sw) < (unsigned)W;
+            if (PAIR32) {
+                // A pair whose second pixel reads past the right edge is fetched one element lower and shifted
+                // down afterwards: its first element may be the last one of the descriptor's range, and a
+                // 32-bit load that crosses the end of the range returns zero.
+                base0[g] = (ok1 ? o : o - 2) | (row_ok ? 0 : SENT);
+                base1[g] = 0;
+                down[g] = ok1 ? 0 : 16;
+                keep[g] = (ok0 ? 0x0000FFFFu : 0u) | (ok1 ? 0xFFFF0000u : 0u);
+            } else {
+                base0[g] = o | ((row_ok & ok0) ? 0 : SENT);
+                base1[g] = (o + sw * 2) | ((row_ok & ok1) ? 0 : SENT);
+                keep[g] = 0; down[g] = 0;
+            }
         }
         constexpr int PERG = T / 16 / NTAP;
         const int plane16 = 16 * H * W * 2;
 #pragma unroll
         for (int i = 0; i < T / 16; i++) {
-            const unsigned lo = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(st.rsrc, base0[i / PERG], (i % PERG) * plane16, 0);
-            const unsigned hi = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(st.rsrc, base1[i / PERG], (i % PERG) * plane16, 0);
-            r.s[i] = lo | (hi << 16);
+            if (PAIR32) {
+                // the pair is two neighbouring elements of an input row: one load (two-byte alignment suffices)
+                const unsigned word = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(st.rsrc, base0[i / PERG], (i % PERG) * plane16, 0);
+                r.s[i] = __builtin_amdgcn_alignbit(0u, word, (unsigned)down[i / PERG]) & keep[i / PERG];
+            } else {
+                const unsigned lo = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(st.rsrc, base0[i / PERG], (i % PERG) * plane16, 0);
+                const unsigned hi = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(st.rsrc, base1[i / PERG], (i % PERG) * plane16, 0);
+                r.s[i] = lo | (hi << 16);
+            }
         }
         // next slice: KH pixels further
         st.iw += KH * sw; st.off += KH * sw * 2;
@@ -322,6 +345,96 @@ struct LoadIm2colRedTapH {
     __device__ static __forceinline__ void store(unsigned short* lds, int tid, const Regs<T>& r) {
 #pragma unroll
         for (int i = 0; i < T / 16; i++) *(unsigned*)(lds + ((tid >> 4) + 16 * i) * HSTRIDE + 2 * (tid & 15)) = r.s[i];
+    }
+};
+
+} // namespace vdnn
+
+namespace vdnn {
+
+// ---- im2col operand of forward (unit column stride) / backward data, a pixel pair per lane --------------
+// The engine is bound by the number of load instructions. Two neighbouring output pixels of a row read two
+// neighbouring elements of an input row through any tap: one 32-bit load (two-byte alignment suffices for
+// buffer loads, and with consecutive lanes on consecutive pairs a wavefront's load still covers one run of
+// a plane). Item = (pixel pair, eight consecutive channels): eight loads, a 2x8 transpose of 16-bit values
+// (v_perm_b32), two 128-bit LDS stores. A pixel left or right of the image is read from the neighbouring row
+// and masked; a pair whose second pixel is past the right edge is fetched one element lower (the last element
+// of the descriptor's range must not be the first half of a word) and unpacked from the upper halves.
+// Needs an even output row length, unit column stride in forward, at most 16 taps per filter row.
+template <int MODE>
+struct LoadIm2colPixTapH2 {
+    LoadIm2colPix<MODE, false, bf16_t> base; // geometry only
+    template <int T> struct Regs { uintx4 v[T / 128][2]; }; // [item][pixel of the pair]
+    template <int T> struct State {
+        int vbase[T / 128];       // byte offset of the pair's first pixel from the descriptor base
+        unsigned invrow[T / 128]; // bit r set: filter row r reads outside the image
+        unsigned colbad[T / 128]; // bit 2*s + e set: pixel e of the pair reads outside the image through filter column s
+        __amdgpu_buffer_rsrc_t rsrc;
+    };
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int j0, int tid, int ncols, int) const {
+        constexpr int PAIRS = T / 2;
+        const int opix = base.OH * base.OW;
+        const int n_first = j0 / opix;
+        const long first = (long)n_first * base.sample_elems;
+        const long shift = MODE == 0 ? -((long)base.ph * base.Ws + base.pw) : (long)(base.ph - base.R + 1) * base.Ws + (base.pw - base.S + 1);
+        int n_last = (j0 + T - 1) / opix;
+        if (n_last > base.nsamples - 1) n_last = base.nsamples - 1;
+        st.rsrc = make_rsrc(base.src + first + shift, clamp_range(((long)(n_last - n_first + 1) * base.sample_elems - shift) * 2));
+        const int j = j0 + 2 * (tid % PAIRS);
+        const bool valid = j < ncols;
+        const int jj = valid ? j : j0;
+        const int n = jj / opix, pix = jj - n * opix;
+        const int oh = pix / base.OW, ow = pix - oh * base.OW;
+        const int ih0 = MODE == 0 ? oh * base.sh - base.ph : oh + base.ph;
+        const int iw0 = MODE == 0 ? ow - base.pw : ow + base.pw;
+        unsigned vrow = 0, bad = 0;
+        for (int r = 0; r < base.R; r++)
+            if ((unsigned)(MODE == 0 ? ih0 + r : ih0 - r) < (unsigned)base.Hs) vrow |= 1u << r;
+        for (int s = 0; s < base.S; s++)
+            for (int e = 0; e < 2; e++)
+                if (!((unsigned)(MODE == 0 ? iw0 + e + s : iw0 + e - s) < (unsigned)base.Ws)) bad |= 1u << (2 * s + e);
+        if (!valid) { vrow = 0; bad = ~0u; }
+#pragma unroll
+        for (int i = 0; i < T / 128; i++) { // the items of a thread differ in their channels only
+            st.vbase[i] = (int)(((long)(n - n_first) * base.sample_elems + (long)(MODE == 0 ? oh * base.sh : oh) * base.Ws + ow) * 2);
+            st.invrow[i] = ~vrow; st.colbad[i] = bad;
+        }
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int kk0, int, int tid, Regs<T>& r) const {
+        constexpr int PAIRS = T / 2;
+        const int plane = base.Hs * base.Ws;
+        const int slice = kk0 / KH;
+        const int cb = base.divRS.div(slice), tap = slice - cb * (base.R * base.S);
+        const int tr = base.divS.div(tap), ts = tap - tr * base.S;
+        const int tapoff = MODE == 0 ? tr * base.Ws + ts : (base.R - 1 - tr) * base.Ws + (base.S - 1 - ts);
+        const int g0 = __builtin_amdgcn_readfirstlane(tid / PAIRS);
+#pragma unroll
+        for (int i = 0; i < T / 128; i++) {
+            const unsigned m0 = (unsigned)bit_to_all_ones(st.colbad[i], 2 * ts), m1 = (unsigned)bit_to_all_ones(st.colbad[i], 2 * ts + 1);
+            // second pixel outside: fetch one element lower, the first pixel is then the upper half of each word
+            const int voff = (st.vbase[i] + (int)(m1 & 0xFFFFFFFEu)) | bit_to_all_ones(st.invrow[i], tr); // m1 is 0 or -1: adds -2
+            const unsigned sel0 = m1 ? 0x07060302u : 0x05040100u;
+            const int ch = cb * KH + 8 * (g0 + (NT / PAIRS) * i);
+            const int soff = (ch * plane + tapoff) * 2, step = plane * 2;
+            unsigned c[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) c[e] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(st.rsrc, voff, soff + e * step, 0);
+            r.v[i][0].x = __builtin_amdgcn_perm(c[1], c[0], sel0) & ~m0; r.v[i][0].y = __builtin_amdgcn_perm(c[3], c[2], sel0) & ~m0;
+            r.v[i][0].z = __builtin_amdgcn_perm(c[5], c[4], sel0) & ~m0; r.v[i][0].w = __builtin_amdgcn_perm(c[7], c[6], sel0) & ~m0;
+            r.v[i][1].x = __builtin_amdgcn_perm(c[1], c[0], 0x07060302u) & ~m1; r.v[i][1].y = __builtin_amdgcn_perm(c[3], c[2], 0x07060302u) & ~m1;
+            r.v[i][1].z = __builtin_amdgcn_perm(c[5], c[4], 0x07060302u) & ~m1; r.v[i][1].w = __builtin_amdgcn_perm(c[7], c[6], 0x07060302u) & ~m1;
+        }
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(unsigned short* lds, int tid, const Regs<T>& r) {
+        constexpr int PAIRS = T / 2;
+#pragma unroll
+        for (int i = 0; i < T / 128; i++)
+#pragma unroll
+            for (int e = 0; e < 2; e++)
+                *(uintx4*)(lds + (2 * (tid % PAIRS) + e) * HSTRIDE + 8 * (tid / PAIRS + (NT / PAIRS) * i)) = r.v[i][e];
     }
 };
 
