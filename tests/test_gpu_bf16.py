@@ -270,3 +270,37 @@ def test_bf16_engine_in_a_split_last_round_agrees_with_two_half_batches(ctx):
                 if 0 <= ih < 14 and 0 <= iw < 14:
                     acc += float(np.dot(x[n, :, ih, iw].astype(np.float64), wr[k, :, r, s_]))
         assert abs(whole_y[n, k, p, q] - acc) <= 2.0 ** -7 * max(abs(acc), 1e-3)
+
+
+def test_conv_bf16_tensors_at_odd_element_offsets(ctx):
+    """Activation tensors that start two bytes off a four-byte boundary (a view into a larger buffer): the pixel-pair
+    loads of the bfloat16 engine do not depend on the alignment of the tensor, and backward filter leaves the engine."""
+    geom = (3, 64, 12, 16, 96, 3, 3, 1, 1, 1, 1)
+    g, og = be.shape(*geom), oracle.shape(*geom)
+    rng = np.random.default_rng(77)
+    x = rnd(rng, (3, 64, 12, 16))
+    w = (rng.standard_normal((96, 64, 3, 3)) * np.sqrt(2.0 / 576)).astype(np.float32)
+    b = rng.standard_normal(96).astype(np.float32)
+    dy = rnd(rng, (3, 96, 12, 16))
+    wr = oracle.round_bf16(w)
+
+    def shifted(d, a):
+        """uploads `a` one element into a buffer that is one element longer"""
+        bits = np.concatenate([np.zeros(1, np.uint16), to_bf16_bits(a).ravel()])
+        buf = d.ctx.to_device(bits, np.uint16)
+        d.bufs.append(buf)
+        return buf.ptr + 2
+
+    with Dev(ctx) as d:
+        px, pdy, dw, db = shifted(d, x), shifted(d, dy), d.f32(w), d.f32(b)
+        y, gx = d.raw(dy.size * 2 + 2), d.raw(x.size * 2 + 2)
+        announce("conv bf16, tensors at odd element offsets")
+        check(lib.vdnn_conv_fwd(ctx.handle, None, g, 0, px, dw.ptr, db.ptr, y.ptr + 2, None, 0))
+        check(lib.vdnn_conv_bwd_data(ctx.handle, None, g, 0, pdy, dw.ptr, gx.ptr + 2, None, 0))
+        gw = d.f32(np.zeros_like(w))
+        check(lib.vdnn_conv_bwd_filter(ctx.handle, None, g, 0, px, pdy, gw.ptr, None, 0))
+        got_y = from_bf16_bits(y.download((dy.size + 1,), np.uint16)[1:]).reshape(dy.shape)
+        got_gx = from_bf16_bits(gx.download((x.size + 1,), np.uint16)[1:]).reshape(x.shape)
+        assert_close_bf16(got_y, oracle.conv_fwd(og, x, wr, b), "fwd")
+        assert_close_bf16(got_gx, oracle.conv_bwd_data(og, dy, wr), "bwd data")
+        assert_close(gw.download(w.shape), oracle.conv_bwd_filter_sgd(og, x, dy, np.zeros_like(w), 1.0), 1e-4, "bwd filter")
