@@ -41,9 +41,9 @@ def log(*a):
 
 
 def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0, bf16=False, offload_lag=0, prefetch_depth=1,
-               fuse=False):
+               fuse=False, compress=False):
     net = Network(cnn, policy, algo, batch, seed=seed, refined=refined, cap_bytes=cap_bytes, bf16=bf16,
-                  offload_lag=offload_lag, prefetch_depth=prefetch_depth, fuse=fuse)
+                  offload_lag=offload_lag, prefetch_depth=prefetch_depth, fuse=fuse, compress=compress)
     try:
         for _ in range(warmup):
             assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
@@ -60,18 +60,25 @@ def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refin
         be.profile_enable(net.context, False)
         st = net.stats()
         loss = net.loss()
+        tensor_bytes, link_bytes = be.zvc_traffic(net.context)
     finally:
         net.close()
     res = {"ms_per_step": dt * 1e3 / steps, "images_per_s": batch * steps / dt, "loss": loss,
            "peak_hbm_gb": st["peak_bytes_in_use"] / 1e9, "offload_gb_per_step": st["offload_bytes"] / 1e9,
            "prefetch_gb_per_step": st["prefetch_bytes"] / 1e9, "pinned_gb": st["pinned_bytes"] / 1e9}
     # host link: busy time and rate of the copies, and how much of the copy time ran under compute
-    copies = [prof[k] for k in ("offload_d2h", "prefetch_h2d") if k in prof]
+    # (the *_zvc entries are the compacting copies: their bytes are the tensors', not what crossed the link)
+    link = ("offload_d2h", "prefetch_h2d", "offload_zvc", "prefetch_zvc")
+    copies = [prof[k] for k in link if k in prof]
+    if tensor_bytes:
+        res["zvc_link_bytes_per_tensor_byte"] = link_bytes / tensor_bytes
     if copies:
         copy_ms = sum(c["ms"] for c in copies)
-        kernel_ms = sum(v["ms"] for k, v in prof.items() if k not in ("offload_d2h", "prefetch_h2d"))
-        res["d2h_gbs"] = prof["offload_d2h"]["bytes"] / (prof["offload_d2h"]["ms"] * 1e-3) / 1e9
-        res["h2d_gbs"] = prof["prefetch_h2d"]["bytes"] / (prof["prefetch_h2d"]["ms"] * 1e-3) / 1e9
+        kernel_ms = sum(v["ms"] for k, v in prof.items() if k not in link)
+        rate = lambda keys: (sum(prof[k]["bytes"] for k in keys if k in prof) /
+                             max(sum(prof[k]["ms"] for k in keys if k in prof), 1e-9) * 1e3 / 1e9)
+        res["d2h_gbs"] = rate(("offload_d2h", "offload_zvc"))
+        res["h2d_gbs"] = rate(("prefetch_h2d", "prefetch_zvc"))
         res["copy_busy_ms_per_step"] = copy_ms / steps
         res["kernel_busy_ms_per_step"] = kernel_ms / steps
         # step = kernels + copies - overlap + idle  =>  overlap >= kernels + copies - step
@@ -143,16 +150,17 @@ def main():
     for name in args.policies.split(","):
         # suffixes: "+refined" = the value-preserving lifetime refinements; "+slack" = blocks recycled six layers
         # after their offload and two tensors fetched ahead; "+bf16" = bfloat16 activation storage; "+fused" = ReLU
-        # layers run inside the neighbouring layers' kernels
+        # layers run inside the neighbouring layers' kernels; "+zvc" = offloaded rectified tensors cross the link
+        # without their zero elements (lossless)
         word, *mods = name.split("+")
-        assert set(mods) <= {"refined", "slack", "bf16", "fused"}, name
+        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc"}, name
         _, policy, algo = parse("VGG16_128", word, args.algo)
         lag, depth = (6, 2) if "slack" in mods else (args.offload_lag, args.prefetch_depth)
         log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
         results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1,
                                                    refined=("refined" in mods), cap_bytes=int(args.cap_gb * 1e9),
                                                    bf16=(args.bf16 or "bf16" in mods), offload_lag=lag, prefetch_depth=depth,
-                                                   fuse=("fused" in mods))
+                                                   fuse=("fused" in mods), compress=("zvc" in mods))
         log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
             results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))
 

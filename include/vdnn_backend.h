@@ -118,6 +118,19 @@ int vdnn_host_free_pinned(vdnn_ctx* ctx, void* ptr);
  * layer.cu:979-987). */
 int vdnn_memcpy_d2h_async(vdnn_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes, vdnn_stream_t stream);
 int vdnn_memcpy_h2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes, vdnn_stream_t stream);
+/* The same two copies (layer.cu:969-987) with zero-value compression: a kernel on `stream` compacts the
+ * tensor of `count` elements (elem_bytes 4: float, 2: bfloat16) while it writes it into pinned host memory,
+ * and a second one expands it while it reads it back; elements whose bits are all zero do not cross the
+ * link. Lossless. The reference copies every tensor whole; a rectified tensor is about half zeros.
+ * The host buffer must come from vdnn_host_alloc_pinned and hold vdnn_zvc_buffer_bytes(count, elem_bytes):
+ * slots of 4096 elements, each a 512-byte map (bit l of 64-bit word g: element 64 g + l is kept) followed
+ * by the kept elements in order. */
+size_t vdnn_zvc_buffer_bytes(size_t count, int elem_bytes);
+int vdnn_zvc_offload_async(vdnn_ctx* ctx, void* dst_host, const void* src_dev, size_t count, int elem_bytes, vdnn_stream_t stream);
+int vdnn_zvc_prefetch_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t count, int elem_bytes, vdnn_stream_t stream);
+/* Bytes of the tensors offloaded this way since the context was made, and bytes that crossed the link for
+ * them (waits for the device). */
+int vdnn_zvc_traffic(vdnn_ctx* ctx, unsigned long long* tensor_bytes, unsigned long long* link_bytes);
 /* Blocking copies (cudaMemcpy: layer.cu:940-942, network.cu:827). */
 int vdnn_memcpy_d2h(vdnn_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);
 int vdnn_memcpy_h2d(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);

@@ -1,0 +1,170 @@
+"""Zero-value compression of offloaded tensors, through the C ABI.
+
+The reference moves an offloaded tensor whole (layer.cu:969-987); this library can compact it on the way to pinned
+host memory. The code is lossless, so the bar is bit equality: what comes back is the tensor that left, for every
+size (whole slots, ragged tails, one element), both element widths and every bit pattern (negative zero, NaN and
+denormals are kept; only all-zero bits are dropped). The host bytes are also decoded here in numpy from the
+documented format, which pins the format itself: a slot of 4096 elements is a 512-byte map followed by the kept
+elements in order.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import vdnn_implementation_amd.backend as be
+from gpu_util import announce
+from vdnn_implementation_amd.backend import check, lib
+
+pytestmark = pytest.mark.gpu
+CHUNK, MAP = 4096, 512
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = be.Context(pool_bytes=2 << 30)
+    yield c
+    c.close()
+
+
+class Pinned:
+    def __init__(self, ctx, nbytes):
+        self.ctx, self.nbytes = ctx, nbytes
+        p = C.c_void_p()
+        check(lib.vdnn_host_alloc_pinned(ctx.handle, C.byref(p), nbytes))
+        self.ptr = p.value
+        self.view = np.ctypeslib.as_array(C.cast(self.ptr, C.POINTER(C.c_ubyte)), shape=(nbytes,))
+
+    def free(self):
+        self.view = None
+        check(lib.vdnn_host_free_pinned(self.ctx.handle, self.ptr))
+
+
+def decode(host, count, dtype):
+    """numpy restatement of the host format: returns the tensor and the bytes that had to cross the link"""
+    es = np.dtype(dtype).itemsize
+    slot = MAP + CHUNK * es
+    out = np.zeros(count, dtype)
+    link = 0
+    for c in range((count + CHUNK - 1) // CHUNK):
+        raw = host[c * slot:(c + 1) * slot]
+        bits = np.unpackbits(raw[:MAP], bitorder="little").astype(bool)   # bit l of word g = element 64 g + l
+        kept = int(bits.sum())
+        values = raw[MAP:MAP + kept * es].view(dtype)
+        piece = np.zeros(CHUNK, dtype)
+        piece[bits] = values
+        n = min(CHUNK, count - c * CHUNK)
+        assert not bits[n:].any(), "elements past the end of the tensor are never kept"
+        out[c * CHUNK:c * CHUNK + n] = piece[:n]
+        link += MAP + (kept * es + 15) // 16 * 16
+    return out, link
+
+
+def tensor(rng, count, dtype, zero_fraction):
+    info = np.iinfo(dtype)
+    a = rng.integers(1, int(info.max) + 1, size=count, dtype=np.uint64).astype(dtype)   # any non-zero bit pattern
+    a[rng.random(count) < zero_fraction] = 0
+    return a
+
+
+CASES = [
+    (1, 0.5), (63, 0.5), (64, 0.0), (4095, 0.5), (4096, 0.5), (4097, 0.5), (3 * 4096, 1.0), (3 * 4096, 0.0),
+    (10 * 4096 + 777, 0.5), (1 << 20, 0.9), ((1 << 22) + 12345, 0.47),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.uint32, np.uint16])
+@pytest.mark.parametrize("count,zero_fraction", CASES)
+def test_round_trip_and_host_format(ctx, dtype, count, zero_fraction):
+    es = np.dtype(dtype).itemsize
+    rng = np.random.default_rng(count * 7 + es)
+    a = tensor(rng, count, dtype, zero_fraction)
+    if count > 200:   # special values of the float formats, placed by hand
+        a[5] = 0x80000000 if es == 4 else 0x8000        # negative zero has a bit set: kept
+        a[6] = 0x7FC00000 if es == 4 else 0x7FC0        # NaN
+        a[7] = 1                                        # smallest denormal
+    need = lib.vdnn_zvc_buffer_bytes(count, es)
+    assert need == (count + CHUNK - 1) // CHUNK * (MAP + CHUNK * es)
+    host = Pinned(ctx, need)
+    host.view[:] = 0xA5   # stale bytes of an earlier tensor must not matter
+    src = ctx.to_device(a, dtype)
+    dst = ctx.alloc(count * es + 64)
+    dst.upload(np.full(count * es + 64, 0xEE, np.uint8))
+    t0, l0 = C.c_ulonglong(), C.c_ulonglong()
+    check(lib.vdnn_zvc_traffic(ctx.handle, C.byref(t0), C.byref(l0)))
+    announce(f"zvc round trip count={count} bytes={es} zeros={zero_fraction}")
+    check(lib.vdnn_zvc_offload_async(ctx.handle, host.ptr, src.ptr, count, es, None))
+    ctx.synchronize()
+    decoded, link = decode(host.view, count, dtype)
+    assert np.array_equal(decoded, a), "host bytes decode to the tensor"
+    t1, l1 = C.c_ulonglong(), C.c_ulonglong()
+    check(lib.vdnn_zvc_traffic(ctx.handle, C.byref(t1), C.byref(l1)))
+    assert t1.value - t0.value == count * es
+    assert l1.value - l0.value == link
+    check(lib.vdnn_zvc_prefetch_async(ctx.handle, dst.ptr, host.ptr, count, es, None))
+    ctx.synchronize()
+    back = dst.download((count * es + 64,), np.uint8)
+    assert np.array_equal(back[:count * es].view(dtype), a), "round trip"
+    assert (back[count * es:] == 0xEE).all(), "nothing is written past the tensor"
+    host.free(); src.free(); dst.free()
+
+
+def test_rejects_bad_arguments(ctx):
+    host = Pinned(ctx, lib.vdnn_zvc_buffer_bytes(100, 4))
+    buf = ctx.alloc(400)
+    assert lib.vdnn_zvc_buffer_bytes(100, 3) == 0
+    assert lib.vdnn_zvc_offload_async(ctx.handle, host.ptr, buf.ptr, 100, 3, None) != 0
+    assert lib.vdnn_zvc_offload_async(ctx.handle, None, buf.ptr, 100, 4, None) != 0
+    assert lib.vdnn_zvc_prefetch_async(ctx.handle, buf.ptr, None, 100, 4, None) != 0
+    assert lib.vdnn_zvc_offload_async(ctx.handle, host.ptr + 4, buf.ptr, 100, 4, None) != 0
+    check(lib.vdnn_zvc_offload_async(ctx.handle, host.ptr, buf.ptr, 0, 4, None))   # empty tensor: nothing to do
+    host.free(); buf.free()
+
+
+from test_gpu_network import assert_bit_identical, run_steps, small_specs   # noqa: E402
+from vdnn_implementation_amd import (ALEXNET_LRN, BASELINE, OVERFEAT, VDNN_ALL, VDNN_CONV, VDNN_MEMORY_OPT_ALGO,   # noqa: E402
+                                     VDNN_PERF_OPT_ALGO, VGG16_128)
+from vdnn_implementation_amd.network import Network   # noqa: E402
+
+
+@pytest.mark.parametrize("cnn,batch,algo,bf16", [(None, 4, VDNN_MEMORY_OPT_ALGO, False), (ALEXNET_LRN, 4, VDNN_MEMORY_OPT_ALGO, False),
+                                                 (OVERFEAT, 3, VDNN_MEMORY_OPT_ALGO, False), (VGG16_128, 2, VDNN_PERF_OPT_ALGO, False),
+                                                 (VGG16_128, 2, VDNN_MEMORY_OPT_ALGO, True)])
+def test_networks_with_compressed_offload_keep_every_bit(cnn, batch, algo, bf16):
+    """Two training steps under the offloading policies: with compression every loss, captured output and gradient,
+    parameter and the input after the step have the bits of BASELINE, and less than the tensors crosses the link."""
+    def make(policy, **kw):
+        if cnn is None:
+            return Network(layers=small_specs(batch), policy=policy, algo=algo, capture=True, seed=3, bf16=bf16, **kw)
+        return Network(cnn, policy, algo, batch, capture=True, seed=3, bf16=bf16, **kw)
+
+    announce("compressed offload", cnn, batch, "BASELINE")
+    with make(BASELINE) as net:
+        want = run_steps(net, 2)
+    assert all(np.isfinite(v) for v in want["loss"])
+    with make(BASELINE, fuse=True) as net:
+        want_fused = run_steps(net, 2)
+    for policy, kw in ((VDNN_CONV, {}), (VDNN_ALL, {}), (VDNN_ALL, {"host_sync": True}), (VDNN_CONV, {"refined": True}),
+                       (VDNN_ALL, {"refined": True, "offload_lag": 6, "prefetch_depth": 3}),
+                       (VDNN_CONV, {"refined": True, "offload_lag": 6, "prefetch_depth": 2, "fuse": True}),
+                       (VDNN_ALL, {"fuse": True})):
+        announce("compressed offload", cnn, batch, "policy", policy, kw)
+        with make(policy, compress=True, **kw) as net:
+            got = run_steps(net, 2)
+            tensor_bytes, link_bytes = be.zvc_traffic(net.context)
+            packed = [l for l in range(net.num_layers) if net.is_offloaded(l)]
+        assert_bit_identical(got, want_fused if kw.get("fuse") else want, "policy %d %s" % (policy, kw))
+        assert packed, "the policy offloads something"
+        assert tensor_bytes > 0, "some offloaded tensor is a rectified one"
+        if cnn is not None:   # (the tensors of the small table are a slot or two: the map can outweigh their few zeros)
+            assert link_bytes < tensor_bytes, "zeros stayed behind"
+
+
+def test_plan_only_counts_the_larger_host_buffers():
+    """Planning without a device: a compacted tensor's host buffer holds the worst case, a map on top of every element."""
+    kw = dict(plan_only=True, refined=True)
+    with Network(VGG16_128, VDNN_CONV, VDNN_MEMORY_OPT_ALGO, 128, **kw) as plain, \
+         Network(VGG16_128, VDNN_CONV, VDNN_MEMORY_OPT_ALGO, 128, compress=True, **kw) as packed:
+        a, b = plain.stats(), packed.stats()
+    assert a["peak_bytes_in_use"] == b["peak_bytes_in_use"]
+    assert a["pinned_bytes"] < b["pinned_bytes"] <= a["pinned_bytes"] * (1 + 1 / 32) + 13 * (512 + 4096 * 4)

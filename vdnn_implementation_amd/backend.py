@@ -81,6 +81,10 @@ BACKEND_SYMBOLS = {
     "vdnn_host_free_pinned": (_i, [_vp, _vp]),
     "vdnn_memcpy_d2h_async": (_i, [_vp, _vp, _vp, _sz, _vp]),
     "vdnn_memcpy_h2d_async": (_i, [_vp, _vp, _vp, _sz, _vp]),
+    "vdnn_zvc_buffer_bytes": (_sz, [_sz, _i]),
+    "vdnn_zvc_offload_async": (_i, [_vp, _vp, _vp, _sz, _i, _vp]),
+    "vdnn_zvc_prefetch_async": (_i, [_vp, _vp, _vp, _sz, _i, _vp]),
+    "vdnn_zvc_traffic": (_i, [_vp, C.POINTER(C.c_ulonglong), C.POINTER(C.c_ulonglong)]),
     "vdnn_memcpy_d2h": (_i, [_vp, _vp, _vp, _sz]),
     "vdnn_memcpy_h2d": (_i, [_vp, _vp, _vp, _sz]),
     "vdnn_memcpy_d2d_async": (_i, [_vp, _vp, _vp, _sz, _vp]),
@@ -152,6 +156,13 @@ def profile_collect(ctx_handle):
     check(lib.vdnn_profile_collect(ctx_handle, arr, 64, C.byref(n)))
     return {arr[i].name.decode(): {"launches": int(arr[i].launches), "ms": arr[i].ms, "flops": arr[i].flops, "bytes": arr[i].bytes}
             for i in range(min(n.value, 64))}
+
+
+def zvc_traffic(ctx_handle):
+    """(bytes of the tensors offloaded with zero-value compression, bytes that crossed the link for them)"""
+    t, l = C.c_ulonglong(), C.c_ulonglong()
+    check(lib.vdnn_zvc_traffic(ctx_handle, C.byref(t), C.byref(l)))
+    return t.value, l.value
 
 
 class DeviceBuffer:

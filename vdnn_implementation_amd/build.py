@@ -23,7 +23,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
 
-DEVICE_SOURCES = ["backend.hip", "eltwise.hip", "conv.hip", "fc.hip"]
+DEVICE_SOURCES = ["backend.hip", "eltwise.hip", "conv.hip", "fc.hip", "zvc.hip"]
 HOST_SOURCES = ["pool.cpp", "layer.cpp", "network.cpp", "capi.cpp"]
 CLI_SOURCE = "vdnn_main.cpp"
 

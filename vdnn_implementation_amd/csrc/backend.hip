@@ -80,6 +80,7 @@ int vdnn_ctx_destroy(vdnn_ctx* ctx) {
         (void)hipDeviceSynchronize();
         for (auto& r : ctx->prof_records) { (void)hipEventDestroy(r.start); (void)hipEventDestroy(r.stop); }
         for (auto e : ctx->prof_free_events) (void)hipEventDestroy(e);
+        if (ctx->zvc_wire_bytes) (void)hipFree(ctx->zvc_wire_bytes);
         if (ctx->compute) (void)hipStreamDestroy(ctx->compute);
         if (ctx->d2h) (void)hipStreamDestroy(ctx->d2h);
         if (ctx->h2d) (void)hipStreamDestroy(ctx->h2d);

@@ -26,6 +26,10 @@ struct vdnn_ctx {
     bool profiling = false;
     std::vector<ProfRecord> prof_records;
     std::vector<hipEvent_t> prof_free_events;
+    // zero-value compression of offloaded tensors: bytes sent over the link (counted on the device) and
+    // bytes of the tensors they stood for
+    unsigned long long* zvc_wire_bytes = nullptr;
+    unsigned long long zvc_raw_bytes = 0;
 };
 
 namespace vdnn {

@@ -21,6 +21,7 @@ static NetworkOptions to_options(const vdnn_network_options* o) {
     n.unfusedOptimizer = o->unfused_optimizer != 0;
     n.deferOptimizer = o->defer_optimizer != 0;
     n.fuseActivations = o->fuse_activations != 0;
+    n.compressOffload = o->compress_offload != 0;
     return n;
 }
 

@@ -480,7 +480,10 @@ void Layer::initializeFullyConnectedFilterAndBias() {
  * the driver waits on before the block is recycled. */
 void Layer::offloadSrcData(bool*, DATATYPE** _offloadedSrcData_h) {
     if (srcReadyEvent) checkVDNN(vdnn_stream_wait_event(ctx, *stream_memory, srcReadyEvent));
-    checkVDNN(vdnn_memcpy_d2h_async(ctx, _offloadedSrcData_h[layerId], srcData, SrcDataSize() * actBytes, *stream_memory));
+    if (srcPacked)
+        checkVDNN(vdnn_zvc_offload_async(ctx, _offloadedSrcData_h[layerId], srcData, SrcDataSize(), actBytes, *stream_memory));
+    else
+        checkVDNN(vdnn_memcpy_d2h_async(ctx, _offloadedSrcData_h[layerId], srcData, SrcDataSize() * actBytes, *stream_memory));
     if (offloadDoneEvent) checkVDNN(vdnn_event_record(ctx, offloadDoneEvent, *stream_memory));
 }
 
@@ -494,7 +497,10 @@ void Layer::prefetchPreviousSrcData(DATATYPE* _prefetchedSrcData_h, void* _srcDa
         checkVDNN(vdnn_stream_wait_event(ctx, h2d, prefetchBlockFreeEvent));
     }
     if (prefetchHostReadyEvent) checkVDNN(vdnn_stream_wait_event(ctx, h2d, prefetchHostReadyEvent));
-    checkVDNN(vdnn_memcpy_h2d_async(ctx, _srcDataToPrefetch, _prefetchedSrcData_h, _prefetch_bytes, h2d));
+    if (prefetchPacked)
+        checkVDNN(vdnn_zvc_prefetch_async(ctx, _srcDataToPrefetch, _prefetchedSrcData_h, _prefetch_bytes / actBytes, actBytes, h2d));
+    else
+        checkVDNN(vdnn_memcpy_h2d_async(ctx, _srcDataToPrefetch, _prefetchedSrcData_h, _prefetch_bytes, h2d));
     if (prefetchDoneEvent) checkVDNN(vdnn_event_record(ctx, prefetchDoneEvent, h2d));
 }
 

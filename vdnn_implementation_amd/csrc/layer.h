@@ -191,6 +191,10 @@ public:
     void    setPrefetchEvents(vdnn_event_t blockFree, vdnn_event_t hostReady, vdnn_event_t done) {
         prefetchBlockFreeEvent = blockFree; prefetchHostReadyEvent = hostReady; prefetchDoneEvent = done;
     }
+    // This layer's offloaded input / the tensor this layer fetches next crosses the link without its zeros.
+    void    setSrcPacked(bool on)                { srcPacked = on; }
+    bool    SrcPacked() const                    { return srcPacked; }
+    void    setPrefetchPacked(bool on)           { prefetchPacked = on; }
 
     /* Get functions */
     Layer_t LayerType()              { return layerType; }
@@ -276,6 +280,7 @@ private:
     /* Ordering of the copies */
     vdnn_event_t srcReadyEvent, offloadDoneEvent;
     vdnn_event_t prefetchBlockFreeEvent, prefetchHostReadyEvent, prefetchDoneEvent;
+    bool    srcPacked = false, prefetchPacked = false;
 
     /* Connection to other layers (GoogLeNet plumbing of the reference, unused) */
     std::vector<int> producerLayerId, consumerLayerId;

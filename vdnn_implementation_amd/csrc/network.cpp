@@ -308,6 +308,14 @@ bool Network::fusesRelu(int l) const {
     return is_conv(specs[l - 1].type) || specs[l - 1].type == FC_GEMM;
 }
 
+/* addition (compressOffload): the input of layer l holds rectified values - it is the output of a ReLU,
+ * directly or behind max-pool / LRN layers, which map zero to zero and keep a tensor of many zeros one */
+bool Network::srcIsRectified(int l) const {
+    int p = l - 1;
+    while (p >= 0 && (specs[p].type == POOL || specs[p].type == LRN)) p--;
+    return p >= 0 && specs[p].type == RELU;
+}
+
 /* network.cu:819-829: the reference draws U(-0.01, 0.01) from an unseeded generator on every call;
  * here the draw is seeded (stream 1) and N(0,1) */
 void Network::randomInitializeData(void* data, size_t size) {
@@ -354,6 +362,7 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         if (layer[i] != NULL) {
             layer[i]->setVdnnMode(newVdnnType);
             layer[i]->setInPlaceOp(false);
+            layer[i]->setSrcPacked(false);
             layer[i]->setFuseRelu(false);
             layer[i]->setElidedBackward(false);
             layer[i]->setGateGrad(false);
@@ -395,7 +404,10 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         if (dropSrcAfterFwd[l]) return; /* released, not moved: nothing reads it again */
         if (layer[l]->Elided()) return;  /* its input is the next layer's srcData, which has its own turn */
         isOffload[l] = true;
-        const size_t bytes = layer[l]->SrcDataSize() * actBytes();
+        const bool packed = options.compressOffload && srcIsRectified(l);
+        layer[l]->setSrcPacked(packed);
+        const size_t bytes = packed ? vdnn_zvc_buffer_bytes(layer[l]->SrcDataSize(), (int)actBytes())
+                                    : layer[l]->SrcDataSize() * actBytes();
         checkVDNN(vdnn_host_alloc_pinned(ctx, (void**)&offloadedSrcData_h[l], bytes));
         lastStats.pinnedBytes += bytes;
     };
@@ -648,6 +660,7 @@ int Network::backwardPropagation(bool isDynamic) {
             if (prefId >= 0) {
                 if (layer[prefId]->cnmemMallocSrcData(isDynamic) < 0) return -1;
                 layer[l]->setPrefetchEvents(evBlockFree[prefId], evOffloadDone[prefId], evPrefetchDone[prefId]);
+                layer[l]->setPrefetchPacked(layer[prefId]->SrcPacked());
                 const size_t bytes = actBytes() * layer[prefId]->SrcDataSize();
                 if (layer[l]->backward(prefId, offloadedSrcData_h[prefId], layer[prefId]->SrcData(), bytes, workSpace, isDynamic) < 0) return -1;
                 lastStats.prefetchBytes += bytes;
@@ -662,6 +675,7 @@ int Network::backwardPropagation(bool isDynamic) {
                 if (extra < 0) break;
                 if (layer[extra]->cnmemMallocSrcData(isDynamic) < 0) return -1;
                 layer[l]->setPrefetchEvents(evBlockFree[extra], evOffloadDone[extra], evPrefetchDone[extra]);
+                layer[l]->setPrefetchPacked(layer[extra]->SrcPacked());
                 const size_t bytes = actBytes() * layer[extra]->SrcDataSize();
                 layer[l]->prefetchPreviousSrcData(offloadedSrcData_h[extra], layer[extra]->SrcData(), bytes);
                 lastStats.prefetchBytes += bytes;

@@ -51,6 +51,11 @@ struct NetworkOptions {
     // bits as the separate layers of the reference (layer.cu:766-814); two passes over the tensor fewer.
     // Such a ReLU layer is never offloaded (its input is not a tensor of its own any more).
     bool     fuseActivations = false;
+    // Offloaded tensors that hold rectified values (the output of a ReLU, also behind max-pool and LRN
+    // layers, which keep zeros zero) cross the link to host memory without their zero elements: a kernel on
+    // the copy stream compacts the tensor into the pinned buffer and another expands it on the way back.
+    // Lossless; the reference copies every tensor whole (layer.cu:969-987). Other tensors are copied as before.
+    bool     compressOffload = false;
     int      device = DEFAULT_DEVICE;
 };
 
@@ -98,6 +103,7 @@ public:
     void            setLayersOverfeat();
     void            setLayersGooglenet();
     bool            fusesRelu(int l) const;
+    bool            srcIsRectified(int l) const;
     void            setLayersVgg16(int givenBatch);
     void            setLayersCustomCNN();
     void            randomInitializeData(void* data, size_t size);

@@ -56,6 +56,7 @@ int main(int argc, char** argv) {
         else if (!strcmp(argv[i], "--plan")) opt.planOnly = true;
         else if (!strcmp(argv[i], "--refined")) opt.refinedLifetimes = true;
         else if (!strcmp(argv[i], "--fuse")) opt.fuseActivations = true;
+        else if (!strcmp(argv[i], "--zvc")) opt.compressOffload = true;
         else if (!strcmp(argv[i], "--unfused")) opt.unfusedOptimizer = true;
         else if (!strcmp(argv[i], "--bf16")) opt.dataType = VDNN_DTYPE_BF16;
         else if (!strcmp(argv[i], "--offload-lag")) opt.offloadLag = atoi(need("--offload-lag needs a value"));
