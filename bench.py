@@ -41,9 +41,9 @@ def log(*a):
 
 
 def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0, bf16=False, offload_lag=0, prefetch_depth=1,
-               fuse=False, compress=False):
+               fuse=False, compress=False, keep_tail_bytes=0):
     net = Network(cnn, policy, algo, batch, seed=seed, refined=refined, cap_bytes=cap_bytes, bf16=bf16,
-                  offload_lag=offload_lag, prefetch_depth=prefetch_depth, fuse=fuse, compress=compress)
+                  offload_lag=offload_lag, prefetch_depth=prefetch_depth, fuse=fuse, compress=compress, keep_tail_bytes=keep_tail_bytes)
     try:
         for _ in range(warmup):
             assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
@@ -68,7 +68,7 @@ def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refin
            "prefetch_gb_per_step": st["prefetch_bytes"] / 1e9, "pinned_gb": st["pinned_bytes"] / 1e9}
     # host link: busy time and rate of the copies, and how much of the copy time ran under compute
     # (the *_zvc entries are the compacting copies: their bytes are the tensors', not what crossed the link)
-    link = ("offload_d2h", "prefetch_h2d", "offload_zvc", "prefetch_zvc")
+    link = ("offload_d2h", "prefetch_h2d", "offload_zvc", "offload_zvc_copy", "prefetch_zvc")
     copies = [prof[k] for k in link if k in prof]
     if tensor_bytes:
         res["zvc_link_bytes_per_tensor_byte"] = link_bytes / tensor_bytes
@@ -77,7 +77,7 @@ def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refin
         kernel_ms = sum(v["ms"] for k, v in prof.items() if k not in link)
         rate = lambda keys: (sum(prof[k]["bytes"] for k in keys if k in prof) /
                              max(sum(prof[k]["ms"] for k in keys if k in prof), 1e-9) * 1e3 / 1e9)
-        res["d2h_gbs"] = rate(("offload_d2h", "offload_zvc"))
+        res["d2h_gbs"] = rate(("offload_d2h", "offload_zvc", "offload_zvc_copy"))
         res["h2d_gbs"] = rate(("prefetch_h2d", "prefetch_zvc"))
         res["copy_busy_ms_per_step"] = copy_ms / steps
         res["kernel_busy_ms_per_step"] = kernel_ms / steps
@@ -127,13 +127,16 @@ def main():
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--algo", default="VDNN_MEMORY_OPT_ALGO")
     ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined,VDNN_CONV+refined+slack,"
-                    "BASELINE+fused,VDNN_CONV+refined+slack+fused,"
+                    "BASELINE+fused,VDNN_CONV+refined+slack+fused,VDNN_CONV+refined+slack+zvc,VDNN_CONV+refined+slack+fused+zvc+tail,"
+                    "VDNN_ALL+refined+slack+fused+zvc,"
                     "BASELINE+bf16,VDNN_ALL+bf16,VDNN_CONV+refined+slack+bf16,VDNN_ALL+refined+slack+bf16,"
-                    "BASELINE+bf16+fused,VDNN_CONV+refined+slack+bf16+fused")
+                    "BASELINE+bf16+fused,VDNN_CONV+refined+slack+bf16+fused,VDNN_CONV+refined+slack+bf16+fused+zvc+tail,"
+                    "VDNN_ALL+refined+slack+bf16+fused+zvc")
     ap.add_argument("--cap-gb", type=float, default=0.0, help="artificial limit on pool bytes in use (0 = none)")
     ap.add_argument("--bf16", action="store_true", help="bfloat16 activation storage (products on the bfloat16 matrix cores, float accumulation and parameters)")
     ap.add_argument("--offload-lag", type=int, default=0, help="layers enqueued before an offloaded block is recycled (0 = reference schedule)")
     ap.add_argument("--prefetch-depth", type=int, default=1, help="offloaded tensors fetched ahead in backward (1 = reference schedule)")
+    ap.add_argument("--keep-tail-gb", type=float, default=0.0, help="the deepest offloaded tensors stay on the device, up to this many GB")
     ap.add_argument("--cpu-batch", type=int, default=24)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -153,14 +156,16 @@ def main():
         # layers run inside the neighbouring layers' kernels; "+zvc" = offloaded rectified tensors cross the link
         # without their zero elements (lossless)
         word, *mods = name.split("+")
-        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc"}, name
+        # "+tail" = the deepest offloaded tensors, 0.3 G elements of them, stay on the device
+        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail"}, name
         _, policy, algo = parse("VGG16_128", word, args.algo)
         lag, depth = (6, 2) if "slack" in mods else (args.offload_lag, args.prefetch_depth)
         log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
         results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1,
                                                    refined=("refined" in mods), cap_bytes=int(args.cap_gb * 1e9),
                                                    bf16=(args.bf16 or "bf16" in mods), offload_lag=lag, prefetch_depth=depth,
-                                                   fuse=("fused" in mods), compress=("zvc" in mods))
+                                                   fuse=("fused" in mods), compress=("zvc" in mods), keep_tail_bytes=(int(0.3e9) * (2 if (args.bf16 or "bf16" in mods) else 4) if "tail" in mods
+                                                                    else int(args.keep_tail_gb * 1e9)))
         log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
             results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))
 

@@ -82,6 +82,9 @@ int vdnn_device_synchronize(vdnn_ctx* ctx);
 vdnn_stream_t vdnn_ctx_stream_compute(vdnn_ctx* ctx);
 vdnn_stream_t vdnn_ctx_stream_d2h(vdnn_ctx* ctx);
 vdnn_stream_t vdnn_ctx_stream_h2d(vdnn_ctx* ctx);
+/* A fourth stream, for the kernels that pack offloaded tensors (vdnn_zvc_offload_staged_async): the next tensor
+ * is packed while the copy engine still moves the one before on the device-to-host stream. */
+vdnn_stream_t vdnn_ctx_stream_pack(vdnn_ctx* ctx);
 
 /* ---- pooled device memory (replaces cnmem: network.cu:47-53, layer.cu:989-1011) --------------- */
 /* cnmemInit: reserve `bytes` of device memory once; all later requests are carved from it. */
@@ -118,15 +121,29 @@ int vdnn_host_free_pinned(vdnn_ctx* ctx, void* ptr);
  * layer.cu:979-987). */
 int vdnn_memcpy_d2h_async(vdnn_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes, vdnn_stream_t stream);
 int vdnn_memcpy_h2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes, vdnn_stream_t stream);
-/* The same two copies (layer.cu:969-987) with zero-value compression: a kernel on `stream` compacts the
- * tensor of `count` elements (elem_bytes 4: float, 2: bfloat16) while it writes it into pinned host memory,
- * and a second one expands it while it reads it back; elements whose bits are all zero do not cross the
- * link. Lossless. The reference copies every tensor whole; a rectified tensor is about half zeros.
- * The host buffer must come from vdnn_host_alloc_pinned and hold vdnn_zvc_buffer_bytes(count, elem_bytes):
- * slots of 4096 elements, each a 512-byte map (bit l of 64-bit word g: element 64 g + l is kept) followed
- * by the kept elements in order. */
+/* The same two copies (layer.cu:969-987) with zero-value compression: the tensor of `count` elements
+ * (elem_bytes 4: float, 2: bfloat16) crosses the link without the elements whose bits are all zero, and comes
+ * back with every bit it had. The reference copies every tensor whole; a rectified tensor is about half zeros.
+ * The host buffer must come from vdnn_host_alloc_pinned and hold vdnn_zvc_buffer_bytes(count, elem_bytes).
+ * It receives a packed stream: a table of one 32-bit word per chunk of 4096 elements (padded to 16 bytes), the
+ * offset of the chunk's record in units of 16 bytes; a record is a 512-byte map (bit l of 64-bit word g: element
+ * 64 g + l is kept) followed by the kept elements in order, zero filled to 16 bytes. Records lie without gaps in
+ * no particular order, so the stream is as long as its content.
+ *   vdnn_zvc_offload_async: a kernel on `stream` packs the tensor straight into the host buffer.
+ *   vdnn_zvc_offload_staged_async: the kernel packs into `staging_dev` (device memory, 16-byte aligned,
+ *     staging_bytes a multiple of 16) at HBM speed and the copy engine moves staging_bytes to the host buffer;
+ *     what the stream has beyond staging_bytes the kernel stores into the host buffer itself, so any size is
+ *     correct and the stream's length of the step before is the one to pass. total_host (pinned, may be NULL)
+ *     receives the stream's length in bytes when the kernel is done. The kernel runs on pack_stream (NULL: the
+ *     context's packing stream) behind what that stream holds, `packed` is recorded there when src_dev has been
+ *     read, and the copy runs on copy_stream (NULL: the device-to-host stream) behind `packed`; with `packed`
+ *     NULL everything runs on copy_stream. staging_dev must stay until the work on copy_stream is done.
+ *   vdnn_zvc_prefetch_async: a kernel on `stream` reads the host buffer and expands it into dst_dev. */
 size_t vdnn_zvc_buffer_bytes(size_t count, int elem_bytes);
 int vdnn_zvc_offload_async(vdnn_ctx* ctx, void* dst_host, const void* src_dev, size_t count, int elem_bytes, vdnn_stream_t stream);
+int vdnn_zvc_offload_staged_async(vdnn_ctx* ctx, void* dst_host, void* staging_dev, size_t staging_bytes, const void* src_dev, size_t count,
+                                  int elem_bytes, unsigned long long* total_host, vdnn_stream_t pack_stream, vdnn_stream_t copy_stream,
+                                  vdnn_event_t packed);
 int vdnn_zvc_prefetch_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t count, int elem_bytes, vdnn_stream_t stream);
 /* Bytes of the tensors offloaded this way since the context was made, and bytes that crossed the link for
  * them (waits for the device). */

@@ -1,11 +1,12 @@
 """Zero-value compression of offloaded tensors, through the C ABI.
 
-The reference moves an offloaded tensor whole (layer.cu:969-987); this library can compact it on the way to pinned
-host memory. The code is lossless, so the bar is bit equality: what comes back is the tensor that left, for every
-size (whole slots, ragged tails, one element), both element widths and every bit pattern (negative zero, NaN and
-denormals are kept; only all-zero bits are dropped). The host bytes are also decoded here in numpy from the
-documented format, which pins the format itself: a slot of 4096 elements is a 512-byte map followed by the kept
-elements in order.
+The reference moves an offloaded tensor whole (layer.cu:969-987); this library can send it without its zero
+elements. The code is lossless, so the bar is bit equality: what comes back is the tensor that left, for every
+size (whole chunks, ragged tails, one element), both element widths and every bit pattern (negative zero, NaN and
+denormals are kept; only all-zero bits are dropped), whether the stream goes to host memory through a staging
+buffer of any size or straight from the kernel. The host bytes are also decoded here in numpy from the documented
+format, which pins the format itself: a table of record offsets, then per chunk of 4096 elements a 512-byte map
+followed by the kept elements in order.
 """
 import ctypes as C
 
@@ -41,23 +42,32 @@ class Pinned:
 
 
 def decode(host, count, dtype):
-    """numpy restatement of the host format: returns the tensor and the bytes that had to cross the link"""
+    """numpy restatement of the stream format: returns the tensor and the length of the stream"""
     es = np.dtype(dtype).itemsize
-    slot = MAP + CHUNK * es
+    chunks = (count + CHUNK - 1) // CHUNK
+    table_bytes = (chunks * 4 + 15) // 16 * 16
+    table = host[:chunks * 4].view(np.uint32)
     out = np.zeros(count, dtype)
-    link = 0
-    for c in range((count + CHUNK - 1) // CHUNK):
-        raw = host[c * slot:(c + 1) * slot]
-        bits = np.unpackbits(raw[:MAP], bitorder="little").astype(bool)   # bit l of word g = element 64 g + l
+    spans = []
+    for c in range(chunks):
+        at = int(table[c]) * 16
+        bits = np.unpackbits(host[at:at + MAP], bitorder="little").astype(bool)   # bit l of word g = element 64 g + l
         kept = int(bits.sum())
-        values = raw[MAP:MAP + kept * es].view(dtype)
+        values = host[at + MAP:at + MAP + kept * es].view(dtype)
+        padded = (kept * es + 15) // 16 * 16
+        assert not host[at + MAP + kept * es:at + MAP + padded].any(), "zero fill behind the kept elements"
         piece = np.zeros(CHUNK, dtype)
         piece[bits] = values
         n = min(CHUNK, count - c * CHUNK)
         assert not bits[n:].any(), "elements past the end of the tensor are never kept"
         out[c * CHUNK:c * CHUNK + n] = piece[:n]
-        link += MAP + (kept * es + 15) // 16 * 16
-    return out, link
+        spans.append((at, at + MAP + padded))
+    spans.sort()
+    edge = table_bytes
+    for lo, hi in spans:   # records follow the table without gaps or overlap
+        assert lo == edge
+        edge = hi
+    return out, edge
 
 
 def tensor(rng, count, dtype, zero_fraction):
@@ -73,9 +83,15 @@ CASES = [
 ]
 
 
+# staging buffer as a fraction of the stream's length: none (the kernel stores everything itself), too short by a
+# lot and by a little (the rest goes straight to host memory), exact, longer
+STAGING = [None, 0.0, 0.37, 0.999, 1.0, 1.5]
+
+
 @pytest.mark.parametrize("dtype", [np.uint32, np.uint16])
+@pytest.mark.parametrize("staging", STAGING)
 @pytest.mark.parametrize("count,zero_fraction", CASES)
-def test_round_trip_and_host_format(ctx, dtype, count, zero_fraction):
+def test_round_trip_and_host_format(ctx, dtype, count, zero_fraction, staging):
     es = np.dtype(dtype).itemsize
     rng = np.random.default_rng(count * 7 + es)
     a = tensor(rng, count, dtype, zero_fraction)
@@ -84,7 +100,8 @@ def test_round_trip_and_host_format(ctx, dtype, count, zero_fraction):
         a[6] = 0x7FC00000 if es == 4 else 0x7FC0        # NaN
         a[7] = 1                                        # smallest denormal
     need = lib.vdnn_zvc_buffer_bytes(count, es)
-    assert need == (count + CHUNK - 1) // CHUNK * (MAP + CHUNK * es)
+    chunks = (count + CHUNK - 1) // CHUNK
+    assert need == (chunks * 4 + 15) // 16 * 16 + chunks * (MAP + CHUNK * es)
     host = Pinned(ctx, need)
     host.view[:] = 0xA5   # stale bytes of an earlier tensor must not matter
     src = ctx.to_device(a, dtype)
@@ -92,15 +109,36 @@ def test_round_trip_and_host_format(ctx, dtype, count, zero_fraction):
     dst.upload(np.full(count * es + 64, 0xEE, np.uint8))
     t0, l0 = C.c_ulonglong(), C.c_ulonglong()
     check(lib.vdnn_zvc_traffic(ctx.handle, C.byref(t0), C.byref(l0)))
-    announce(f"zvc round trip count={count} bytes={es} zeros={zero_fraction}")
-    check(lib.vdnn_zvc_offload_async(ctx.handle, host.ptr, src.ptr, count, es, None))
+    announce(f"zvc round trip count={count} bytes={es} zeros={zero_fraction} staging={staging}")
+    stage_bytes, stage, word = 0, None, None
+    if staging is None:
+        check(lib.vdnn_zvc_offload_async(ctx.handle, host.ptr, src.ptr, count, es, None))
+    else:
+        kept = int(np.count_nonzero(a))   # the stream's length follows from the tensor: table, maps, kept elements
+        per_chunk = [int(np.count_nonzero(a[c * CHUNK:(c + 1) * CHUNK])) for c in range(chunks)]
+        length = (chunks * 4 + 15) // 16 * 16 + sum(MAP + (k * es + 15) // 16 * 16 for k in per_chunk)
+        stage_bytes = min(int(length * staging) // 16 * 16, need)
+        stage = ctx.alloc(max(stage_bytes, 16))
+        word = Pinned(ctx, 8)
+        word.view[:] = 0xFF
+        packed = None
+        if count % 2:   # with an event the kernel runs on the packing stream and the copy behind it on the copy stream
+            packed = C.c_void_p()
+            check(lib.vdnn_event_create(ctx.handle, C.byref(packed), 0))
+        check(lib.vdnn_zvc_offload_staged_async(ctx.handle, host.ptr, stage.ptr, stage_bytes, src.ptr, count, es, word.ptr, None, None, packed))
     ctx.synchronize()
-    decoded, link = decode(host.view, count, dtype)
+    decoded, length_seen = decode(host.view, count, dtype)
     assert np.array_equal(decoded, a), "host bytes decode to the tensor"
     t1, l1 = C.c_ulonglong(), C.c_ulonglong()
     check(lib.vdnn_zvc_traffic(ctx.handle, C.byref(t1), C.byref(l1)))
     assert t1.value - t0.value == count * es
-    assert l1.value - l0.value == link
+    assert l1.value - l0.value == max(length_seen, stage_bytes)
+    if staging is not None:
+        assert length_seen == length
+        assert int(word.view.view(np.uint64)[0]) == length, "the kernel reports the stream's length"
+        stage.free(); word.free()
+        if packed:
+            check(lib.vdnn_event_destroy(ctx.handle, packed))
     check(lib.vdnn_zvc_prefetch_async(ctx.handle, dst.ptr, host.ptr, count, es, None))
     ctx.synchronize()
     back = dst.download((count * es + 64,), np.uint8)
@@ -112,6 +150,15 @@ def test_round_trip_and_host_format(ctx, dtype, count, zero_fraction):
 def test_rejects_bad_arguments(ctx):
     host = Pinned(ctx, lib.vdnn_zvc_buffer_bytes(100, 4))
     buf = ctx.alloc(400)
+    stage = ctx.alloc(1 << 20)
+    staged = lambda ptr, nbytes: lib.vdnn_zvc_offload_staged_async(ctx.handle, host.ptr, ptr, nbytes, buf.ptr, 100, 4, None, None, None, None)
+    assert staged(None, 64) != 0              # bytes without a buffer
+    assert staged(stage.ptr, 24) != 0         # not a multiple of 16
+    assert staged(stage.ptr + 4, 64) != 0     # misaligned
+    assert staged(stage.ptr, 1 << 20) != 0    # longer than the longest stream of 100 elements
+    check(staged(stage.ptr, 64))
+    ctx.synchronize()
+    stage.free()
     assert lib.vdnn_zvc_buffer_bytes(100, 3) == 0
     assert lib.vdnn_zvc_offload_async(ctx.handle, host.ptr, buf.ptr, 100, 3, None) != 0
     assert lib.vdnn_zvc_offload_async(ctx.handle, None, buf.ptr, 100, 4, None) != 0
@@ -141,19 +188,24 @@ def test_networks_with_compressed_offload_keep_every_bit(cnn, batch, algo, bf16)
     announce("compressed offload", cnn, batch, "BASELINE")
     with make(BASELINE) as net:
         want = run_steps(net, 2)
+        # a third of the activations, counted from the last layer down, stay on the device where a case says so
+        tail = sum(int(np.prod([s.n, s.c, s.h, s.w])) for s in net.specs) * (2 if bf16 else 4) // 3
     assert all(np.isfinite(v) for v in want["loss"])
     with make(BASELINE, fuse=True) as net:
         want_fused = run_steps(net, 2)
     for policy, kw in ((VDNN_CONV, {}), (VDNN_ALL, {}), (VDNN_ALL, {"host_sync": True}), (VDNN_CONV, {"refined": True}),
                        (VDNN_ALL, {"refined": True, "offload_lag": 6, "prefetch_depth": 3}),
                        (VDNN_CONV, {"refined": True, "offload_lag": 6, "prefetch_depth": 2, "fuse": True}),
-                       (VDNN_ALL, {"fuse": True})):
+                       (VDNN_ALL, {"fuse": True}), (VDNN_CONV, {"fuse": True, "offload_lag": 3, "keep_tail_bytes": tail}),
+                       (VDNN_ALL, {"refined": True, "keep_tail_bytes": tail})):
         announce("compressed offload", cnn, batch, "policy", policy, kw)
         with make(policy, compress=True, **kw) as net:
             got = run_steps(net, 2)
             tensor_bytes, link_bytes = be.zvc_traffic(net.context)
             packed = [l for l in range(net.num_layers) if net.is_offloaded(l)]
         assert_bit_identical(got, want_fused if kw.get("fuse") else want, "policy %d %s" % (policy, kw))
+        if "keep_tail_bytes" in kw:
+            continue   # (a third of the activations can be the whole offload set of the policy)
         assert packed, "the policy offloads something"
         assert tensor_bytes > 0, "some offloaded tensor is a rectified one"
         if cnn is not None:   # (the tensors of the small table are a slot or two: the map can outweigh their few zeros)
@@ -166,5 +218,29 @@ def test_plan_only_counts_the_larger_host_buffers():
     with Network(VGG16_128, VDNN_CONV, VDNN_MEMORY_OPT_ALGO, 128, **kw) as plain, \
          Network(VGG16_128, VDNN_CONV, VDNN_MEMORY_OPT_ALGO, 128, compress=True, **kw) as packed:
         a, b = plain.stats(), packed.stats()
-    assert a["peak_bytes_in_use"] == b["peak_bytes_in_use"]
-    assert a["pinned_bytes"] < b["pinned_bytes"] <= a["pinned_bytes"] * (1 + 1 / 32) + 13 * (512 + 4096 * 4)
+    # (the plan holds a staging block as long as the longest stream beside every packed tensor; a run sizes the
+    # blocks from the streams it has seen, and releases the tensor itself behind its layer's forward)
+    assert a["peak_bytes_in_use"] <= b["peak_bytes_in_use"]
+    assert a["pinned_bytes"] < b["pinned_bytes"] <= a["pinned_bytes"] * (1 + 1 / 32 + 1 / 4096) + 13 * (512 + 4096 * 4 + 16)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_losses_at_a_batch_that_keeps_the_streams_busy(bf16):
+    """VGG16 at batch 32, four steps: with copies of tens of milliseconds in flight on three streams beside the
+    kernels, blocks that are recycled too early show up as a different loss. Steps two to four pack through staging
+    blocks sized from the step before."""
+    def losses(policy, **kw):
+        with Network(VGG16_128, policy, VDNN_MEMORY_OPT_ALGO, 32, seed=5, bf16=bf16, **kw) as net:
+            out = []
+            for _ in range(4):
+                assert net.forwardPropagation() == 0
+                assert net.backwardPropagation() == 0
+                out.append(np.float32(net.loss()).tobytes())
+            return out
+
+    announce("compressed offload at batch 32, BASELINE, bf16", bf16)
+    want = losses(BASELINE, fuse=True)
+    for policy, kw in ((VDNN_CONV, {"refined": True, "offload_lag": 6, "prefetch_depth": 2}), (VDNN_ALL, {"refined": True, "offload_lag": 6, "prefetch_depth": 2}),
+                       (VDNN_CONV, {}), (VDNN_ALL, {"offload_lag": 2})):
+        announce("compressed offload at batch 32, policy", policy, kw, "bf16", bf16)
+        assert losses(policy, fuse=True, compress=True, **kw) == want, "policy %d %s" % (policy, kw)

@@ -419,3 +419,45 @@ def test_fused_rectifiers_own_no_tensor_and_leak_nothing():
                 assert st["offload_bytes"] == st["prefetch_bytes"] == ref["offload_bytes"]
                 if kw.get("refined"):
                     assert st["peak_bytes_in_use"] <= ref["peak_bytes_in_use"]
+
+
+def live_blocks(net):
+    n = C.c_size_t()
+    lib.vdnn_pool_live_blocks(net.context, C.byref(n))
+    return n.value
+
+
+def test_keep_tail_takes_the_deepest_members_out_of_the_offload_set():
+    """keep_tail_bytes walks the policy's offload set from the last layer down and keeps what fits on the device."""
+    with plan(VGG16_128, VDNN_CONV, batch=128) as net:
+        convs = conv_layers(net)
+        size = {l: int(np.prod(net.src_shape(l))) * 4 for l in convs}
+    for keep in (0, 1, size[convs[-1]], size[convs[-1]] + size[convs[-2]] + 5, sum(size.values())):
+        want, left = list(convs), keep
+        while want and size[want[-1]] <= left:
+            left -= size[want.pop()]
+        with plan(VGG16_128, VDNN_CONV, batch=128, keep_tail_bytes=keep) as net:
+            assert [l for l in range(net.num_layers) if net.is_offloaded(l)] == want, keep
+            step(net)
+            assert net.stats()["offload_bytes"] == sum(size[l] for l in want)
+            assert net.stats()["prefetch_bytes"] == sum(size[l] for l in want)
+    # the tail is small and gone before the large tensors come back: the peak of the plan does not move
+    with plan(VGG16_128, VDNN_CONV, batch=128, refined=True) as a, \
+         plan(VGG16_128, VDNN_CONV, batch=128, refined=True, keep_tail_bytes=int(1.2e9)) as b:
+        step(a); step(b)
+        assert len([l for l in range(b.num_layers) if b.is_offloaded(l)]) < len(conv_layers(a))
+        assert b.stats()["peak_bytes_in_use"] == a.stats()["peak_bytes_in_use"]
+        assert live_blocks(b) == live_blocks(a)
+
+
+def test_compressed_offload_plans_for_the_longest_stream_and_leaks_nothing():
+    """Planning has no data: it holds a staging block as long as the longest stream beside each packed tensor."""
+    for policy, kw in ((VDNN_CONV, {}), (VDNN_ALL, {"refined": True, "offload_lag": 6, "prefetch_depth": 2}), (VDNN_ALL, {"fuse": True})):
+        with plan(VGG16_128, policy, batch=16, **kw) as a, plan(VGG16_128, policy, batch=16, compress=True, **kw) as b:
+            for _ in range(2):
+                step(a); step(b)
+            sa, sb = a.stats(), b.stats()
+            assert sb["offload_bytes"] == sa["offload_bytes"] and sb["prefetch_bytes"] == sa["prefetch_bytes"]
+            assert sa["pinned_bytes"] < sb["pinned_bytes"] < sa["pinned_bytes"] * 1.04
+            assert sa["peak_bytes_in_use"] <= sb["peak_bytes_in_use"]
+            assert live_blocks(b) == live_blocks(a)

@@ -54,7 +54,8 @@ int vdnn_ctx_create(vdnn_ctx** out, int device, int flags) {
         // default priority on every stream
         if (hipStreamCreateWithFlags(&ctx->compute, hipStreamNonBlocking) != hipSuccess ||
             hipStreamCreateWithFlags(&ctx->d2h, hipStreamNonBlocking) != hipSuccess ||
-            hipStreamCreateWithFlags(&ctx->h2d, hipStreamNonBlocking) != hipSuccess) {
+            hipStreamCreateWithFlags(&ctx->h2d, hipStreamNonBlocking) != hipSuccess ||
+            hipStreamCreateWithFlags(&ctx->pack, hipStreamNonBlocking) != hipSuccess) {
             set_error("hipStreamCreate failed");
             delete ctx;
             return VDNN_EDEVICE;
@@ -80,10 +81,11 @@ int vdnn_ctx_destroy(vdnn_ctx* ctx) {
         (void)hipDeviceSynchronize();
         for (auto& r : ctx->prof_records) { (void)hipEventDestroy(r.start); (void)hipEventDestroy(r.stop); }
         for (auto e : ctx->prof_free_events) (void)hipEventDestroy(e);
-        if (ctx->zvc_wire_bytes) (void)hipFree(ctx->zvc_wire_bytes);
+        if (ctx->zvc_counters) (void)hipFree(ctx->zvc_counters);
         if (ctx->compute) (void)hipStreamDestroy(ctx->compute);
         if (ctx->d2h) (void)hipStreamDestroy(ctx->d2h);
         if (ctx->h2d) (void)hipStreamDestroy(ctx->h2d);
+        if (ctx->pack) (void)hipStreamDestroy(ctx->pack);
     }
     delete ctx;
     return VDNN_OK;
@@ -110,6 +112,7 @@ int vdnn_device_synchronize(vdnn_ctx* ctx) {
 vdnn_stream_t vdnn_ctx_stream_compute(vdnn_ctx* ctx) { return ctx ? ctx->compute : nullptr; }
 vdnn_stream_t vdnn_ctx_stream_d2h(vdnn_ctx* ctx) { return ctx ? ctx->d2h : nullptr; }
 vdnn_stream_t vdnn_ctx_stream_h2d(vdnn_ctx* ctx) { return ctx ? ctx->h2d : nullptr; }
+vdnn_stream_t vdnn_ctx_stream_pack(vdnn_ctx* ctx) { return ctx ? ctx->pack : nullptr; }
 
 /* ---- pool ----------------------------------------------------------------------------------- */
 int vdnn_pool_init(vdnn_ctx* ctx, size_t bytes) {

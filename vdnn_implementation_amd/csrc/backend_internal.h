@@ -12,7 +12,7 @@
 struct vdnn_ctx {
     int device = 0;
     bool plan_only = false;
-    hipStream_t compute = nullptr, d2h = nullptr, h2d = nullptr;
+    hipStream_t compute = nullptr, d2h = nullptr, h2d = nullptr, pack = nullptr;
     vdnn::Pool pool;
     void* pool_base = nullptr;      // hipMalloc'd reservation (null in plan-only mode)
     // Staging for deterministic split reductions (filter gradients, bias gradients, FC split-K).
@@ -26,10 +26,11 @@ struct vdnn_ctx {
     bool profiling = false;
     std::vector<ProfRecord> prof_records;
     std::vector<hipEvent_t> prof_free_events;
-    // zero-value compression of offloaded tensors: bytes sent over the link (counted on the device) and
-    // bytes of the tensors they stood for
-    unsigned long long* zvc_wire_bytes = nullptr;
+    // zero-value compression of offloaded tensors: device words (bytes sent over the link, then the stream
+    // cursors of the offloads in flight) and bytes of the tensors that were packed
+    unsigned long long* zvc_counters = nullptr;
     unsigned long long zvc_raw_bytes = 0;
+    unsigned zvc_next_cursor = 0;
 };
 
 namespace vdnn {

@@ -22,6 +22,7 @@ static NetworkOptions to_options(const vdnn_network_options* o) {
     n.deferOptimizer = o->defer_optimizer != 0;
     n.fuseActivations = o->fuse_activations != 0;
     n.compressOffload = o->compress_offload != 0;
+    n.keepTailBytes = o->keep_tail_bytes;
     return n;
 }
 

@@ -479,11 +479,16 @@ void Layer::initializeFullyConnectedFilterAndBias() {
  * stream first waits for the event that marks srcData as completely written, and signals an event
  * the driver waits on before the block is recycled. */
 void Layer::offloadSrcData(bool*, DATATYPE** _offloadedSrcData_h) {
-    if (srcReadyEvent) checkVDNN(vdnn_stream_wait_event(ctx, *stream_memory, srcReadyEvent));
-    if (srcPacked)
-        checkVDNN(vdnn_zvc_offload_async(ctx, _offloadedSrcData_h[layerId], srcData, SrcDataSize(), actBytes, *stream_memory));
-    else
+    if (srcPacked) {
+        /* the packing kernel runs on a stream of its own, so that it overlaps the copy of the tensor before */
+        vdnn_stream_t pack = srcPackedEvent ? vdnn_ctx_stream_pack(ctx) : *stream_memory;
+        if (srcReadyEvent) checkVDNN(vdnn_stream_wait_event(ctx, pack, srcReadyEvent));
+        checkVDNN(vdnn_zvc_offload_staged_async(ctx, _offloadedSrcData_h[layerId], offloadStaging, offloadStagingBytes, srcData, SrcDataSize(),
+                                                actBytes, offloadLengthWord, pack, *stream_memory, srcPackedEvent));
+    } else {
+        if (srcReadyEvent) checkVDNN(vdnn_stream_wait_event(ctx, *stream_memory, srcReadyEvent));
         checkVDNN(vdnn_memcpy_d2h_async(ctx, _offloadedSrcData_h[layerId], srcData, SrcDataSize() * actBytes, *stream_memory));
+    }
     if (offloadDoneEvent) checkVDNN(vdnn_event_record(ctx, offloadDoneEvent, *stream_memory));
 }
 

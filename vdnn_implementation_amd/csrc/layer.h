@@ -195,6 +195,12 @@ public:
     void    setSrcPacked(bool on)                { srcPacked = on; }
     bool    SrcPacked() const                    { return srcPacked; }
     void    setPrefetchPacked(bool on)           { prefetchPacked = on; }
+    // Where the packed stream of this layer's input is staged on its way out (bytes may be 0: the kernel stores
+    // all of it into host memory itself), the pinned word that receives its length, and the event recorded when
+    // the packing kernel has read srcData.
+    void    setOffloadStaging(void* staging, size_t bytes, unsigned long long* lengthWord, vdnn_event_t packed) {
+        offloadStaging = staging; offloadStagingBytes = bytes; offloadLengthWord = lengthWord; srcPackedEvent = packed;
+    }
 
     /* Get functions */
     Layer_t LayerType()              { return layerType; }
@@ -281,6 +287,10 @@ private:
     vdnn_event_t srcReadyEvent, offloadDoneEvent;
     vdnn_event_t prefetchBlockFreeEvent, prefetchHostReadyEvent, prefetchDoneEvent;
     bool    srcPacked = false, prefetchPacked = false;
+    void*   offloadStaging = nullptr;
+    size_t  offloadStagingBytes = 0;
+    unsigned long long* offloadLengthWord = nullptr;
+    vdnn_event_t srcPackedEvent = nullptr;
 
     /* Connection to other layers (GoogLeNet plumbing of the reference, unused) */
     std::vector<int> producerLayerId, consumerLayerId;

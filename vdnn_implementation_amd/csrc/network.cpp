@@ -130,8 +130,11 @@ void Network::construct(vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) {
         isOffload[i] = isPrefetched[i] = false;
         dropSrcAfterFwd[i] = false;
         offloadedSrcData_h[i] = nullptr;
-        evFwdDone[i] = evOffloadDone[i] = evBlockFree[i] = evPrefetchDone[i] = nullptr;
+        evFwdDone[i] = evOffloadDone[i] = evBlockFree[i] = evPrefetchDone[i] = evPacked[i] = nullptr;
+        zvcStaging[i] = nullptr;
+        srcReleasedEarly[i] = false;
     }
+    zvcLength_h = nullptr;
 
     /* context = handles + streams (network.cu:39-42) */
     ctx = nullptr;
@@ -165,7 +168,7 @@ Network::~Network() {
     releasePolicyBuffers();
     releaseLayers();
     for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
-        for (vdnn_event_t* e : {&evFwdDone[i], &evOffloadDone[i], &evBlockFree[i], &evPrefetchDone[i]}) {
+        for (vdnn_event_t* e : {&evFwdDone[i], &evOffloadDone[i], &evBlockFree[i], &evPrefetchDone[i], &evPacked[i]}) {
             if (*e) vdnn_event_destroy(ctx, *e);
             *e = nullptr;
         }
@@ -190,6 +193,8 @@ void Network::releasePolicyBuffers() {
         offloadedSrcData_h[i] = nullptr;
         isOffload[i] = isPrefetched[i] = false;
     }
+    if (zvcLength_h) vdnn_host_free_pinned(ctx, zvcLength_h);
+    zvcLength_h = nullptr;
 }
 
 /* network.cu:101-132: drop every allocation, rebuild layers and buffers for a new configuration */
@@ -400,9 +405,25 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         }
     }
 
+    /* keepTailBytes: the deepest members of the offload set stay on the device */
+    int tailStart = numLayers;
+    {
+        size_t tail = 0;
+        for (int l = numLayers - 2; l >= 0 && options.keepTailBytes > 0; l--) {
+            const bool member = (newVdnnType == VDNN_ALL || (newVdnnType == VDNN_CONV && is_conv(layer[l]->LayerType()))) &&
+                                !dropSrcAfterFwd[l] && !layer[l]->Elided();
+            if (!member) continue;
+            const size_t bytes = layer[l]->SrcDataSize() * actBytes();
+            if (tail + bytes > options.keepTailBytes) break;
+            tail += bytes;
+            tailStart = l;
+        }
+    }
+
     auto offload = [&](int l) {
         if (dropSrcAfterFwd[l]) return; /* released, not moved: nothing reads it again */
         if (layer[l]->Elided()) return;  /* its input is the next layer's srcData, which has its own turn */
+        if (l >= tailStart) return;
         isOffload[l] = true;
         const bool packed = options.compressOffload && srcIsRectified(l);
         layer[l]->setSrcPacked(packed);
@@ -434,8 +455,12 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
 
     if (newVdnnType != BASELINE) {
         for (int l = 0; l < numLayers; l++)
-            for (vdnn_event_t* e : {&evFwdDone[l], &evOffloadDone[l], &evBlockFree[l], &evPrefetchDone[l]})
+            for (vdnn_event_t* e : {&evFwdDone[l], &evOffloadDone[l], &evBlockFree[l], &evPrefetchDone[l], &evPacked[l]})
                 if (!*e) checkVDNN(vdnn_event_create(ctx, e, 0));
+        if (options.compressOffload && !options.planOnly && !zvcLength_h) {
+            checkVDNN(vdnn_host_alloc_pinned(ctx, (void**)&zvcLength_h, sizeof(unsigned long long) * DEFAULT_NUM_LAYER));
+            for (int l = 0; l < DEFAULT_NUM_LAYER; l++) zvcLength_h[l] = 0; /* 0: not known yet */
+        }
     }
 }
 
@@ -562,6 +587,26 @@ int Network::forwardPropagation(bool isDynamic) {
                 layer[l]->setSrcReadyEvent(l == 0 ? evBlockFree[0] : evFwdDone[l - 1]);
                 layer[l]->setOffloadDoneEvent(evOffloadDone[l]);
             }
+            /* compressOffload: the stream is packed into a staging block sized from its length one step ago (plus
+               a margin; what does not fit the kernel stores into host memory itself) and the copy engine moves
+               the block. The first step has no length to go by and stores everything from the kernel; planning
+               without a device assumes the longest stream. */
+            zvcStaging[l] = nullptr;
+            srcReleasedEarly[l] = false;
+            if (isOffload[l] && layer[l]->SrcPacked()) {
+                const size_t longest = vdnn_zvc_buffer_bytes(layer[l]->SrcDataSize(), (int)actBytes());
+                const size_t known = options.planOnly ? longest : (size_t)zvcLength_h[l];
+                size_t want = known ? known + known / 32 + 65536 : 0;
+                want = std::min(longest, (want + 15) / 16 * 16);
+                if (want && ASSERT_EQ(vdnn_pool_malloc(ctx, &zvcStaging[l], want), isDynamic) < 0) return -1;
+                if (want) {
+                    /* the packing stream writes a recycled block: whatever the compute stream was told to wait
+                       for before the block went back to the pool (a copy out of it, say) comes first */
+                    checkVDNN(vdnn_event_record(ctx, evBlockFree[l], stream_compute));
+                    layer[l]->setSrcReadyEvent(evBlockFree[l]);
+                }
+                layer[l]->setOffloadStaging(zvcStaging[l], want, options.planOnly ? nullptr : &zvcLength_h[l], evPacked[l]);
+            }
 
             /* Forward propagation */
             if (layer[l]->forward(isOffload, offloadedSrcData_h, workSpace, isDynamic) < 0) return -1;
@@ -579,6 +624,13 @@ int Network::forwardPropagation(bool isDynamic) {
             if (isOffload[l]) {
                 lastStats.offloadBytes += layer[l]->SrcDataSize() * actBytes();
                 pendingOffload.push_back(l);
+                if (zvcStaging[l]) {
+                    /* the staging block has the tensor: srcData goes back behind this layer's kernels and the
+                       packing kernel, which works at HBM speed and started when this layer did */
+                    if (!options.hostSync) checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evPacked[l]));
+                    ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->SrcData()), isDynamic);
+                    srcReleasedEarly[l] = true;
+                }
             } else if (dropSrcAfterFwd[l]) {
                 /* refined lifetimes: every reader (this layer's forward) is already enqueued */
                 ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->SrcData()), isDynamic);
@@ -589,7 +641,9 @@ int Network::forwardPropagation(bool isDynamic) {
                 const int j = pendingOffload.front();
                 pendingOffload.erase(pendingOffload.begin());
                 if (!options.hostSync) checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evOffloadDone[j]));
-                ASSERT_EQ(vdnn_pool_free(ctx, layer[j]->SrcData()), isDynamic);
+                if (zvcStaging[j]) ASSERT_EQ(vdnn_pool_free(ctx, zvcStaging[j]), isDynamic);
+                zvcStaging[j] = nullptr;
+                if (!srcReleasedEarly[j]) ASSERT_EQ(vdnn_pool_free(ctx, layer[j]->SrcData()), isDynamic);
                 if (j == 0) { inputData = nullptr; inputResident = false; }
             }
             printUsage("Fwd", l, layer[l]->FwdWorkSpaceSize());

@@ -56,6 +56,12 @@ struct NetworkOptions {
     // the copy stream compacts the tensor into the pinned buffer and another expands it on the way back.
     // Lossless; the reference copies every tensor whole (layer.cu:969-987). Other tensors are copied as before.
     bool     compressOffload = false;
+    // The deepest tensors that the policy would offload stay on the device instead, as many as fit in this
+    // many bytes counted from the last layer down. They are the last into the copy queue and the first that
+    // backward asks for, so offloading them makes backward wait for the queue to drain, and they are small and
+    // gone before the large tensors of the shallow layers come back: the peak is elsewhere. 0: the reference's
+    // policies (network.cu:898-921).
+    size_t   keepTailBytes = 0;
     int      device = DEFAULT_DEVICE;
 };
 
@@ -217,6 +223,11 @@ private:
     vdnn_event_t        evOffloadDone[DEFAULT_NUM_LAYER]; // d2h: srcData of layer l is in pinned memory
     vdnn_event_t        evBlockFree[DEFAULT_NUM_LAYER];   // compute: everything enqueued before the prefetch of l
     vdnn_event_t        evPrefetchDone[DEFAULT_NUM_LAYER];// h2d: srcData of layer l is back on the device
+    /* compressOffload: the packed stream of an offloaded input waits in device memory for the copy engine */
+    vdnn_event_t        evPacked[DEFAULT_NUM_LAYER];      // d2h: the packing kernel has read srcData of layer l
+    void*               zvcStaging[DEFAULT_NUM_LAYER];    // staging block of layer l's stream (null: none this step)
+    bool                srcReleasedEarly[DEFAULT_NUM_LAYER]; // srcData of layer l went back to the pool behind its forward
+    unsigned long long* zvcLength_h;                       // pinned: length of each layer's stream, reported by the packing kernel
     std::vector<int>    pendingOffload;                    // offloaded layers whose block is not yet recycled (offloadLag)
     bool                inputResident;                     // inputData currently holds the input (addition)
 
