@@ -96,7 +96,22 @@ __global__ __launch_bounds__(kZvcThreads) void zvc_pack_kernel(const E* __restri
 #pragma unroll
         for (int w = 0; w < 4; ++w) { const unsigned t = wave_total[team][w]; pos += w < wave ? t : 0u; total += t; }
         const unsigned units = kZvcMapBytes / 16 + (total * unsigned(sizeof(E)) + 15u) / 16u;   // 16-byte units of the record
-        if (tid == 0 && live) place[team] = atomicAdd(cursor, (unsigned long long)units * 16ull);
+        if (threadIdx.x == 0) {
+            // one claim for the workgroup's records: every claim is an atomic on the same word, and those come one
+            // at a time
+            unsigned bytes[kZvcTeams], all = 0;
+#pragma unroll
+            for (int t = 0; t < kZvcTeams; ++t) {
+                unsigned n = 0;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) n += wave_total[t][w];
+                bytes[t] = first_chunk + t < chunks ? kZvcMapBytes + (n * unsigned(sizeof(E)) + 15u) / 16u * 16u : 0u;
+                all += bytes[t];
+            }
+            unsigned long long at = atomicAdd(cursor, (unsigned long long)all);
+#pragma unroll
+            for (int t = 0; t < kZvcTeams; ++t) { place[t] = at; at += bytes[t]; }
+        }
 #pragma unroll
         for (int i = 0; i < kZvcGroupsPerWave; ++i) {
             if (v[i] != 0) rec[team].kept[pos + __popcll(m[i] & below)] = v[i];
