@@ -41,9 +41,9 @@ def log(*a):
 
 
 def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0, bf16=False, offload_lag=0, prefetch_depth=1,
-               fuse=False, compress=False, keep_tail_bytes=0):
+               fuse=False, compress=False, keep_tail_bytes=0, ahead=False):
     net = Network(cnn, policy, algo, batch, seed=seed, refined=refined, cap_bytes=cap_bytes, bf16=bf16,
-                  offload_lag=offload_lag, prefetch_depth=prefetch_depth, fuse=fuse, compress=compress, keep_tail_bytes=keep_tail_bytes)
+                  offload_lag=offload_lag, prefetch_depth=prefetch_depth, fuse=fuse, compress=compress, keep_tail_bytes=keep_tail_bytes, prefetch_within_peak=ahead)
     try:
         for _ in range(warmup):
             assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
@@ -127,10 +127,10 @@ def main():
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--algo", default="VDNN_MEMORY_OPT_ALGO")
     ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined,VDNN_CONV+refined+slack,"
-                    "BASELINE+fused,VDNN_CONV+refined+slack+fused,VDNN_CONV+refined+slack+zvc,VDNN_CONV+refined+slack+fused+zvc+tail,"
-                    "VDNN_ALL+refined+slack+fused+zvc,"
+                    "BASELINE+fused,VDNN_CONV+refined+slack+fused,VDNN_CONV+refined+slack+zvc,VDNN_CONV+refined+ahead+fused+zvc,"
+                    "VDNN_CONV+refined+ahead+fused+zvc+tail,VDNN_ALL+refined+slack+fused+zvc,"
                     "BASELINE+bf16,VDNN_ALL+bf16,VDNN_CONV+refined+slack+bf16,VDNN_ALL+refined+slack+bf16,"
-                    "BASELINE+bf16+fused,VDNN_CONV+refined+slack+bf16+fused,VDNN_CONV+refined+slack+bf16+fused+zvc+tail,"
+                    "BASELINE+bf16+fused,VDNN_CONV+refined+slack+bf16+fused,VDNN_CONV+refined+ahead+bf16+fused+zvc+tail,"
                     "VDNN_ALL+refined+slack+bf16+fused+zvc")
     ap.add_argument("--cap-gb", type=float, default=0.0, help="artificial limit on pool bytes in use (0 = none)")
     ap.add_argument("--bf16", action="store_true", help="bfloat16 activation storage (products on the bfloat16 matrix cores, float accumulation and parameters)")
@@ -156,15 +156,16 @@ def main():
         # layers run inside the neighbouring layers' kernels; "+zvc" = offloaded rectified tensors cross the link
         # without their zero elements (lossless)
         word, *mods = name.split("+")
-        # "+tail" = the deepest offloaded tensors, 0.3 G elements of them, stay on the device
-        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail"}, name
+        # "+tail" = the deepest offloaded tensors, 0.75 G elements of them, stay on the device
+        # "+ahead" = backward fetches ahead wherever the peak cannot rise, blocks recycled six layers after their offload
+        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead"}, name
         _, policy, algo = parse("VGG16_128", word, args.algo)
-        lag, depth = (6, 2) if "slack" in mods else (args.offload_lag, args.prefetch_depth)
+        lag, depth = (6, 2) if "slack" in mods else (6, 1) if "ahead" in mods else (args.offload_lag, args.prefetch_depth)
         log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
         results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1,
                                                    refined=("refined" in mods), cap_bytes=int(args.cap_gb * 1e9),
                                                    bf16=(args.bf16 or "bf16" in mods), offload_lag=lag, prefetch_depth=depth,
-                                                   fuse=("fused" in mods), compress=("zvc" in mods), keep_tail_bytes=(int(0.3e9) * (2 if (args.bf16 or "bf16" in mods) else 4) if "tail" in mods
+                                                   fuse=("fused" in mods), compress=("zvc" in mods), ahead=("ahead" in mods), keep_tail_bytes=(int(0.75e9) * (2 if (args.bf16 or "bf16" in mods) else 4) if "tail" in mods
                                                                     else int(args.keep_tail_gb * 1e9)))
         log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
             results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))
@@ -174,8 +175,9 @@ def main():
     # dominant kernel: the convolution class with the most device time over the timed steps of all
     # policies of this run (the same launches a kernel trace of this command sees, warm-up aside)
     prof = {}
+    headline_bf16 = args.bf16 or all(is_bf16(n) for n in profiles)   # (a run of bfloat16 configurations only)
     for pname, p in profiles.items():
-        if is_bf16(pname) != args.bf16:
+        if is_bf16(pname) != headline_bf16:
             continue  # the roofline entry is taken over the runs of the headline element type
         for k, v in p.items():
             acc = prof.setdefault(k, {"launches": 0, "ms": 0.0, "flops": 0.0, "bytes": 0.0})
@@ -196,8 +198,8 @@ def main():
         "metric": "VGG16-128 train img/s (VDNN_ALL vs BASELINE); peak HBM GB; conv MFMA util",
         "value": results[head]["images_per_s"], "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": results[head]["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 (bf16 MFMA products, f32 accumulation, f32 master weights)" if args.bf16 else "f32", "data": "synthetic (seeded N(0,1) inputs, integer labels, He-normal filters)",
-        "config": {"workload": "VGG16 %s batch %d, one SGD step (fwd+bwd), policy %s, %s" % ("bf16-storage" if args.bf16 else "fp32", args.batch, head, args.algo),
+        "dtype": "bf16 (bf16 MFMA products, f32 accumulation, f32 master weights)" if headline_bf16 else "f32", "data": "synthetic (seeded N(0,1) inputs, integer labels, He-normal filters)",
+        "config": {"workload": "VGG16 %s batch %d, one SGD step (fwd+bwd), policy %s, %s" % ("bf16-storage" if headline_bf16 else "fp32", args.batch, head, args.algo),
                    "batch": args.batch, "policy": head, "algo": args.algo},
         "policies": results,
         "vdnn_all_vs_baseline_speed": (results[head]["images_per_s"] / base["images_per_s"]) if base else None,
@@ -212,7 +214,7 @@ def main():
         "conv_mfma_util": conv_all_tf / peak,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                      "frac": achieved / peak,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom) if args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" and not args.bf16 else None,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom) if args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" and not headline_bf16 else None,
                      "traffic_unit": "bytes per launch (L2 fetch + write-back, counters scaled by a known-size kernel)",
                      "algorithmic_flop_per_launch": d["flops"] / d["launches"],
                      "avg_launch_ms": d["ms"] / d["launches"], "launches": d["launches"]},

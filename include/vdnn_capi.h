@@ -32,6 +32,7 @@ typedef struct {
     int      data_type;         /* element type of activation tensors: VDNN_DTYPE_F32 (the reference, vdnn.h:11-12) or VDNN_DTYPE_BF16 */
     int      fuse_activations;  /* a ReLU after a CONV / FC layer runs inside the neighbouring layers' kernels (same bits, layer.cu:766-814) */
     size_t   keep_tail_bytes;   /* the deepest tensors of the policy's offload set stay on the device, up to this many bytes (0 = the reference's policies, network.cu:898-921) */
+    int      prefetch_within_peak; /* backward fetches tensors ahead of the reference's schedule (network.cu:1198-1208) wherever a replay of the schedule shows that the peak cannot rise */
     int      compress_offload;  /* offloaded rectified tensors cross the link without their zero elements (lossless; layer.cu:969-987 copies them whole) */
 } vdnn_network_options;
 

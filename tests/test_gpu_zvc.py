@@ -197,7 +197,9 @@ def test_networks_with_compressed_offload_keep_every_bit(cnn, batch, algo, bf16)
                        (VDNN_ALL, {"refined": True, "offload_lag": 6, "prefetch_depth": 3}),
                        (VDNN_CONV, {"refined": True, "offload_lag": 6, "prefetch_depth": 2, "fuse": True}),
                        (VDNN_ALL, {"fuse": True}), (VDNN_CONV, {"fuse": True, "offload_lag": 3, "keep_tail_bytes": tail}),
-                       (VDNN_ALL, {"refined": True, "keep_tail_bytes": tail})):
+                       (VDNN_ALL, {"refined": True, "keep_tail_bytes": tail}),
+                       (VDNN_CONV, {"refined": True, "offload_lag": 6, "prefetch_within_peak": True}),
+                       (VDNN_ALL, {"fuse": True, "offload_lag": 2, "prefetch_within_peak": True, "keep_tail_bytes": tail // 2})):
         announce("compressed offload", cnn, batch, "policy", policy, kw)
         with make(policy, compress=True, **kw) as net:
             got = run_steps(net, 2)
@@ -241,6 +243,8 @@ def test_losses_at_a_batch_that_keeps_the_streams_busy(bf16):
     announce("compressed offload at batch 32, BASELINE, bf16", bf16)
     want = losses(BASELINE, fuse=True)
     for policy, kw in ((VDNN_CONV, {"refined": True, "offload_lag": 6, "prefetch_depth": 2}), (VDNN_ALL, {"refined": True, "offload_lag": 6, "prefetch_depth": 2}),
-                       (VDNN_CONV, {}), (VDNN_ALL, {"offload_lag": 2})):
+                       (VDNN_CONV, {}), (VDNN_ALL, {"offload_lag": 2}),
+                       (VDNN_CONV, {"refined": True, "offload_lag": 6, "prefetch_within_peak": True, "keep_tail_bytes": 40 << 20}),
+                       (VDNN_ALL, {"refined": True, "offload_lag": 6, "prefetch_within_peak": True})):
         announce("compressed offload at batch 32, policy", policy, kw, "bf16", bf16)
         assert losses(policy, fuse=True, compress=True, **kw) == want, "policy %d %s" % (policy, kw)

@@ -461,3 +461,24 @@ def test_compressed_offload_plans_for_the_longest_stream_and_leaks_nothing():
             assert sa["pinned_bytes"] < sb["pinned_bytes"] < sa["pinned_bytes"] * 1.04
             assert sa["peak_bytes_in_use"] <= sb["peak_bytes_in_use"]
             assert live_blocks(b) == live_blocks(a)
+
+
+def test_prefetch_within_peak_fetches_earlier_and_holds_the_peak():
+    """The replay of the schedule tells backward where a tensor may come back early without raising the peak."""
+    for policy, kw in ((VDNN_CONV, {}), (VDNN_CONV, {"refined": True, "offload_lag": 6}), (VDNN_ALL, {"refined": True}),
+                       (VDNN_ALL, {"fuse": True, "offload_lag": 3, "prefetch_depth": 2}), (VDNN_CONV, {"refined": True, "keep_tail_bytes": int(1e9)})):
+        with plan(VGG16_128, policy, batch=128, **kw) as a, plan(VGG16_128, policy, batch=128, prefetch_within_peak=True, **kw) as b:
+            for _ in range(2):
+                step(a); step(b)
+            sa, sb = a.stats(), b.stats()
+            assert sb["peak_bytes_in_use"] == sa["peak_bytes_in_use"], (policy, kw)
+            assert sb["prefetch_bytes"] == sa["prefetch_bytes"] and sb["offload_bytes"] == sa["offload_bytes"]
+            ta, tb = a.prefetch_trace(), b.prefetch_trace()
+            assert [p for _, p in tb] == [p for _, p in ta], "the same tensors in the same order"
+            assert all(lb >= la for (la, _), (lb, _) in zip(ta, tb)), "never later than the plain schedule"
+            assert any(lb > la for (la, _), (lb, _) in zip(ta, tb)), "some of them earlier"
+            assert live_blocks(b) == live_blocks(a)
+    # BASELINE has nothing to fetch: the option is accepted and changes nothing
+    with plan(VGG16_128, BASELINE, batch=128, prefetch_within_peak=True) as net:
+        step(net)
+        assert net.prefetch_trace() == []

@@ -457,6 +457,7 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         for (int l = 0; l < numLayers; l++)
             for (vdnn_event_t* e : {&evFwdDone[l], &evOffloadDone[l], &evBlockFree[l], &evPrefetchDone[l], &evPacked[l]})
                 if (!*e) checkVDNN(vdnn_event_create(ctx, e, 0));
+        if (options.prefetchWithinPeak && !options.tracePeaks) buildPeakPlan(newVdnnType);
         if (options.compressOffload && !options.planOnly && !zvcLength_h) {
             checkVDNN(vdnn_host_alloc_pinned(ctx, (void**)&zvcLength_h, sizeof(unsigned long long) * DEFAULT_NUM_LAYER));
             for (int l = 0; l < DEFAULT_NUM_LAYER; l++) zvcLength_h[l] = 0; /* 0: not known yet */
@@ -687,7 +688,10 @@ int Network::backwardPropagation(bool isDynamic) {
         if (layer[numLayers - 1]->cnmemMallocDiffData(isDynamic) < 0) return -1;
         calculateFirstDiffData(layer[numLayers - 1]->DiffData(), layer[numLayers - 1]->DstData(), labelData);
 
+        if (options.tracePeaks) bwdPeakTrace.assign(numLayers, 0);
+        fetchedAhead.assign(numLayers, 0);
         for (int l = numLayers - 1; l >= 0; l--) {
+            if (options.tracePeaks) vdnn_pool_reset_peak(ctx);
             if (l != numLayers - 1) {
                 layer[l]->copyDiffData(layer[l + 1]->GradData());
                 layer[l]->copyDstData(layer[l + 1]->SrcData());
@@ -724,8 +728,9 @@ int Network::backwardPropagation(bool isDynamic) {
                 if (layer[l]->backward(-1, NULL, NULL, 0, workSpace, isDynamic) < 0) return -1;
             }
             /* deeper prefetch: further tensors below, enqueued behind this layer's kernels */
-            while (options.prefetchDepth > 1 && l > 0) {
-                const int extra = findPrefetchLayerDeep(l);
+            while ((options.prefetchDepth > 1 || options.prefetchWithinPeak) && l > 0) {
+                int extra = options.prefetchDepth > 1 ? findPrefetchLayerDeep(l) : -1;
+                if (extra < 0 && options.prefetchWithinPeak) extra = findPrefetchWithinPeak(l);
                 if (extra < 0) break;
                 if (layer[extra]->cnmemMallocSrcData(isDynamic) < 0) return -1;
                 layer[l]->setPrefetchEvents(evBlockFree[extra], evOffloadDone[extra], evPrefetchDone[extra]);
@@ -747,6 +752,11 @@ int Network::backwardPropagation(bool isDynamic) {
             if (!(layer[l]->InPlaceOp() && layer[l]->GradData() == layer[l]->DiffData()))
                 ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DiffData()), isDynamic);
             printUsage("Bwd", l, layer[l]->BwdDataWorkSpaceSize() + layer[l]->BwdFilterWorkSpaceSize());
+            if (options.tracePeaks) {
+                size_t inUse = 0, extent = 0;
+                vdnn_pool_peak(ctx, &inUse, &extent);
+                bwdPeakTrace[l] = inUse;
+            }
         }
         ASSERT_EQ(vdnn_pool_free(ctx, layer[0]->GradData()), isDynamic);
         inputData = layer[0]->SrcData(); /* network.cu:1185 */
@@ -800,6 +810,42 @@ int Network::findPrefetchLayerDeep(int currLayerId) {
             isPrefetched[id] = true;
             return id;
         }
+    }
+    return -1;
+}
+
+/* addition (prefetchWithinPeak): one step of this network's schedule on a context without a device, with the
+ * bytes in use noted per backward layer */
+void Network::buildPeakPlan(vdnn_t policy) {
+    planBwdPeak.clear();
+    planIssueLayer.assign(numLayers, -1);
+    planPeak = 0;
+    if (policy == BASELINE) return;
+    NetworkOptions o = options;
+    o.planOnly = true; o.tracePeaks = true; o.prefetchWithinPeak = false;
+    o.capture = false; o.verbose = false; o.capBytes = 0;
+    Network replay(specs, policy, algoMode == VDNN_DYNAMIC_ALGO ? VDNN_MEMORY_OPT_ALGO : algoMode, o);
+    if (replay.forwardPropagation(false) < 0 || replay.backwardPropagation(false) < 0) return;
+    planBwdPeak = replay.backwardPeakTrace();
+    for (const auto& p : replay.prefetchTrace()) planIssueLayer[p.second] = p.first;
+    for (size_t b : planBwdPeak) planPeak = std::max(planPeak, b);
+}
+
+/* addition (prefetchWithinPeak): the nearest offloaded tensor below currLayerId that is still on the host, if
+ * holding it from now on keeps every layer down to the one that would have fetched it at or below the
+ * replay's peak */
+int Network::findPrefetchWithinPeak(int currLayerId) {
+    if (planBwdPeak.size() != (size_t)numLayers) return -1;
+    for (int id = currLayerId - 1; id >= 0; id--) {
+        if (!isOffload[id] || isPrefetched[id]) continue;
+        const int issue = planIssueLayer[id];
+        if (issue < 0 || issue >= currLayerId) return -1;
+        const size_t bytes = actBytes() * layer[id]->SrcDataSize();
+        for (int k = issue; k <= currLayerId; k++)
+            if (planBwdPeak[k] + fetchedAhead[k] + bytes > planPeak) return -1;
+        for (int k = issue; k <= currLayerId; k++) fetchedAhead[k] += bytes;
+        isPrefetched[id] = true;
+        return id;
     }
     return -1;
 }

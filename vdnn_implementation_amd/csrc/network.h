@@ -62,6 +62,14 @@ struct NetworkOptions {
     // gone before the large tensors of the shallow layers come back: the peak is elsewhere. 0: the reference's
     // policies (network.cu:898-921).
     size_t   keepTailBytes = 0;
+    // Backward fetches further tensors ahead whenever that cannot raise the step's peak: the network replays
+    // its own schedule on a context without a device, notes the bytes in use during every layer's backward,
+    // and fetches a tensor early only if, at every layer between here and the layer that would have fetched
+    // it, those bytes plus everything fetched early stay at or below the replay's highest value. The large
+    // tensors of the shallow layers then start their way back while the small deep layers run, whose working
+    // set is far below the peak. Same values, same peak, fewer waits for the link.
+    bool     prefetchWithinPeak = false;
+    bool     tracePeaks = false;          // (internal: the replay records bytes in use per backward layer)
     int      device = DEFAULT_DEVICE;
 };
 
@@ -167,6 +175,7 @@ public:
     const std::vector<float>& capturedGrad(int l) const { return capGrad[l]; }
     // the sequence (backward layer, prefetched layer) of the last backward
     const std::vector<std::pair<int, int>>& prefetchTrace() const { return prefetchLog; }
+    const std::vector<size_t>& backwardPeakTrace() const { return bwdPeakTrace; }
     const std::vector<LayerSpec>& table() const { return specs; }
     static std::vector<LayerSpec> tableFor(CNN_t cnn, int batch);
 
@@ -234,4 +243,11 @@ private:
     NetworkStats        lastStats;
     std::vector<std::vector<float>> capDst, capGrad;
     std::vector<std::pair<int, int>> prefetchLog;
+    /* prefetchWithinPeak: from the replay - bytes in use during backward of each layer, their highest value, the
+       layer whose backward fetches each offloaded tensor; and what this backward has fetched ahead of that */
+    std::vector<size_t> bwdPeakTrace, planBwdPeak, fetchedAhead;
+    std::vector<int>    planIssueLayer;
+    size_t              planPeak = 0;
+    void                buildPeakPlan(vdnn_t policy);
+    int                 findPrefetchWithinPeak(int currLayerId);
 };
