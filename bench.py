@@ -103,6 +103,50 @@ def best_offloading(results, base):
             "peak_hbm_gb": ok[k]["peak_hbm_gb"]}
 
 
+def zvc_standalone(be):
+    """The compacting kernels alone on the device: a rectified fp32 tensor of conv2_1's input size (half zeros) is packed
+    into a staging block, moved by the copy engine, and expanded again from pinned host memory. Rates in bytes of the
+    tensor per second; the packing kernel reads the tensor and writes the stream (about 0.53 of it)."""
+    import ctypes as C
+    import numpy as np
+    lib, check = be.lib, be.check
+    ctx = be.Context(pool_bytes=6 << 30)
+    out = {}
+    try:
+        for es, dtype in ((4, np.uint32), (2, np.uint16)):
+            count = 128 * 64 * 112 * 112 * (4 // es)
+            rng = np.random.default_rng(1)
+            t = rng.integers(1, 60000, size=count, dtype=np.uint32).astype(dtype)
+            t[rng.random(count) < 0.5] = 0
+            src, dst = ctx.to_device(t, dtype), ctx.alloc(count * es)
+            need = lib.vdnn_zvc_buffer_bytes(count, es)
+            stage = ctx.alloc(need)
+            host = C.c_void_p()
+            check(lib.vdnn_host_alloc_pinned(ctx.handle, C.byref(host), need))
+            be.profile_enable(ctx.handle, True)
+            for _ in range(5):
+                check(lib.vdnn_zvc_offload_staged_async(ctx.handle, host, stage.ptr, need // 2 // 16 * 16 + 65536, src.ptr, count, es, None, None, None, None))
+                ctx.synchronize()
+                check(lib.vdnn_zvc_prefetch_async(ctx.handle, dst.ptr, host, count, es, None))
+                ctx.synchronize()
+            prof = be.profile_collect(ctx.handle)
+            be.profile_enable(ctx.handle, False)
+            assert np.array_equal(dst.download((count,), dtype), t)
+            tensor_bytes, link_bytes = be.zvc_traffic(ctx.handle)
+            out["f32" if es == 4 else "bf16"] = {
+                "tensor_mb": count * es / 1e6,
+                "pack_gbs": prof["offload_zvc_pack"]["bytes"] / prof["offload_zvc_pack"]["ms"] / 1e6,
+                "pack_ms": prof["offload_zvc_pack"]["ms"] / prof["offload_zvc_pack"]["launches"],
+                "copy_gbs": prof["offload_zvc_copy"]["bytes"] / prof["offload_zvc_copy"]["ms"] / 1e6,
+                "expand_gbs": prof["prefetch_zvc"]["bytes"] / prof["prefetch_zvc"]["ms"] / 1e6}
+            check(lib.vdnn_host_free_pinned(ctx.handle, host))
+            for b in (src, dst, stage):
+                b.free()
+    finally:
+        ctx.close()
+    return out
+
+
 def cpu_baseline(batch):
     """The checker's training step on the host cores, VGG16 at a reduced batch."""
     import oracle
@@ -139,6 +183,7 @@ def main():
     ap.add_argument("--keep-tail-gb", type=float, default=0.0, help="the deepest offloaded tensors stay on the device, up to this many GB")
     ap.add_argument("--cpu-batch", type=int, default=24)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--zvc-standalone", action="store_true", help="also time the compacting kernels alone on the device")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
@@ -221,6 +266,10 @@ def main():
         "kernels": kernels,
         "step_mfma_frac": args.batch * FLOP_PER_IMAGE / (results[head]["ms_per_step"] * 1e-3) / 1e12 / peak,
     }
+    if args.zvc_standalone:
+        log("[bench] compacting kernels alone")
+        out["zvc_standalone"] = zvc_standalone(be)
+        log("[bench]   %s" % json.dumps(out["zvc_standalone"]))
     if not args.no_cpu_baseline:
         log("[bench] CPU baseline: checker, VGG16 batch %d" % args.cpu_batch)
         out["cpu_baseline"] = cpu_baseline(args.cpu_batch)

@@ -690,6 +690,13 @@ int Network::backwardPropagation(bool isDynamic) {
 
         if (options.tracePeaks) bwdPeakTrace.assign(numLayers, 0);
         fetchedAhead.assign(numLayers, 0);
+        {
+            /* what backward may hold: the highest value of the replay's backward, or what the pool has already
+               held (this step's forward, say) if that is more - either way the peak does not move */
+            size_t held = 0, extent = 0;
+            vdnn_pool_peak(ctx, &held, &extent);
+            peakBudget = std::max(planPeak, held);
+        }
         for (int l = numLayers - 1; l >= 0; l--) {
             if (options.tracePeaks) vdnn_pool_reset_peak(ctx);
             if (l != numLayers - 1) {
@@ -842,7 +849,7 @@ int Network::findPrefetchWithinPeak(int currLayerId) {
         if (issue < 0 || issue >= currLayerId) return -1;
         const size_t bytes = actBytes() * layer[id]->SrcDataSize();
         for (int k = issue; k <= currLayerId; k++)
-            if (planBwdPeak[k] + fetchedAhead[k] + bytes > planPeak) return -1;
+            if (planBwdPeak[k] + fetchedAhead[k] + bytes > peakBudget) return -1;
         for (int k = issue; k <= currLayerId; k++) fetchedAhead[k] += bytes;
         isPrefetched[id] = true;
         return id;

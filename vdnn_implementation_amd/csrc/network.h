@@ -65,7 +65,8 @@ struct NetworkOptions {
     // Backward fetches further tensors ahead whenever that cannot raise the step's peak: the network replays
     // its own schedule on a context without a device, notes the bytes in use during every layer's backward,
     // and fetches a tensor early only if, at every layer between here and the layer that would have fetched
-    // it, those bytes plus everything fetched early stay at or below the replay's highest value. The large
+    // it, those bytes plus everything fetched early stay at or below the replay's highest value (or below what
+    // the pool has already held, this step's forward for one, if that is more). The large
     // tensors of the shallow layers then start their way back while the small deep layers run, whose working
     // set is far below the peak. Same values, same peak, fewer waits for the link.
     bool     prefetchWithinPeak = false;
@@ -247,7 +248,7 @@ private:
        layer whose backward fetches each offloaded tensor; and what this backward has fetched ahead of that */
     std::vector<size_t> bwdPeakTrace, planBwdPeak, fetchedAhead;
     std::vector<int>    planIssueLayer;
-    size_t              planPeak = 0;
+    size_t              planPeak = 0, peakBudget = 0;
     void                buildPeakPlan(vdnn_t policy);
     int                 findPrefetchWithinPeak(int currLayerId);
 };
