@@ -222,7 +222,7 @@ def main():
     prof = {}
     headline_bf16 = args.bf16 or all(is_bf16(n) for n in profiles)   # (a run of bfloat16 configurations only)
     for pname, p in profiles.items():
-        if is_bf16(pname) != headline_bf16:
+        if (args.bf16 or is_bf16(pname)) != headline_bf16:
             continue  # the roofline entry is taken over the runs of the headline element type
         for k, v in p.items():
             acc = prof.setdefault(k, {"launches": 0, "ms": 0.0, "flops": 0.0, "bytes": 0.0})
