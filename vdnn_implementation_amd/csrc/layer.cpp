@@ -194,8 +194,16 @@ int Layer::forward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workS
 }
 
 /* layer.cu:514-537 */
+void Layer::waitSrcFetched() {
+    if (!srcFetchedEvent) return;
+    checkVDNN(vdnn_stream_wait_event(ctx, *stream_compute, srcFetchedEvent));
+    srcFetchedEvent = nullptr;
+}
+
 int Layer::backward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h, void* _srcDataToPrefetch,
                     unsigned long _prefetch_bytes, void* workSpace, bool isDynamic) {
+    /* CONV / FC layers wait in front of their first reader of srcData, everything else here */
+    if (layerType != CONV && layerType != FC_CONV && layerType != FC_GEMM) waitSrcFetched();
     switch (layerType) {
     case FC_GEMM: return fullyConnectedBackward(_layer_id_to_prefetch, _prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes, workSpace, isDynamic);
     case CONV:
@@ -270,6 +278,7 @@ int Layer::convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedS
         prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);
 
     if (mallocWorkSpace(workSpace, bwdDataWorkSpaceSize, &curWorkSpace, isDynamic) < 0) return -1;
+    if (gateGrad) waitSrcFetched(); /* the masked data gradient reads this layer's input */
     if (gateGrad)
         checkVDNN(vdnn_conv_bwd_data_relu(ctx, *stream_compute, &shape, vdnnAlgoMode, diffData, (const float*)filterData,
                                           srcData, gradData, curWorkSpace, bwdDataWorkSpaceSize));
@@ -283,6 +292,7 @@ int Layer::convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedS
     else checkVDNN(vdnn_conv_bwd_bias_sgd(ctx, *stream_compute, &shape, (const float*)diffData, (float*)biasData, lr));
 
     if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) return -1;
+    waitSrcFetched();
     if (filterGrad)
         checkVDNN(vdnn_conv_bwd_filter(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
                                        (float*)filterGrad, curWorkSpace, bwdFilterWorkSpaceSize));
@@ -318,10 +328,12 @@ int Layer::fullyConnectedBackward(int _layer_id_to_prefetch, DATATYPE* _prefetch
     }
     if (vdnnMode != BASELINE && _layer_id_to_prefetch >= 0)
         prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);
+    if (gateGrad) waitSrcFetched();
     if (gateGrad)
         checkVDNN(vdnn_fc_bwd_data_relu(ctx, *stream_compute, n_out, c_in, c_out, diffData, (const float*)filterData, srcData, gradData));
     else
         checkVDNN(vdnn_fc_bwd_data(ctx, *stream_compute, n_out, c_in, c_out, (const float*)diffData, (const float*)filterData, (float*)gradData));
+    waitSrcFetched();
     if (filterGrad) {
         checkVDNN(vdnn_fc_bwd_weight(ctx, *stream_compute, n_out, c_in, c_out, (const float*)srcData, (const float*)diffData, (float*)filterGrad));
         checkVDNN(vdnn_fc_bwd_bias(ctx, *stream_compute, n_out, c_out, (const float*)diffData, (float*)biasGrad));

@@ -192,6 +192,10 @@ public:
         prefetchBlockFreeEvent = blockFree; prefetchHostReadyEvent = hostReady; prefetchDoneEvent = done;
     }
     // This layer's offloaded input / the tensor this layer fetches next crosses the link without its zeros.
+    // The event behind which this layer's prefetched srcData is complete (null: it never left). Backward waits
+    // for it in front of the first kernel that reads srcData: for a CONV / FC layer that is the filter gradient
+    // (or backward data, if that masks by the input), so the data gradient runs while the copy still lands.
+    void    setSrcFetchedEvent(vdnn_event_t e)   { srcFetchedEvent = e; }
     void    setSrcPacked(bool on)                { srcPacked = on; }
     bool    SrcPacked() const                    { return srcPacked; }
     void    setPrefetchPacked(bool on)           { prefetchPacked = on; }
@@ -286,6 +290,8 @@ private:
     /* Ordering of the copies */
     vdnn_event_t srcReadyEvent, offloadDoneEvent;
     vdnn_event_t prefetchBlockFreeEvent, prefetchHostReadyEvent, prefetchDoneEvent;
+    vdnn_event_t srcFetchedEvent = nullptr;
+    void    waitSrcFetched();
     bool    srcPacked = false, prefetchPacked = false;
     void*   offloadStaging = nullptr;
     size_t  offloadStagingBytes = 0;

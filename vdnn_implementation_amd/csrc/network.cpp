@@ -719,7 +719,7 @@ int Network::backwardPropagation(bool isDynamic) {
                 }
             }
             /* this layer reads its own srcData: if that was prefetched, the copy must have landed */
-            if (!options.hostSync && isPrefetched[l]) checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evPrefetchDone[l]));
+            layer[l]->setSrcFetchedEvent(!options.hostSync && isPrefetched[l] ? evPrefetchDone[l] : nullptr);
 
             int prefId = l == 0 ? -1 : (options.prefetchDepth > 1 ? findPrefetchLayerDeep(l) : findPrefetchLayer(l));
             if (prefId >= 0) {
