@@ -171,8 +171,8 @@ def main():
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--algo", default="VDNN_MEMORY_OPT_ALGO")
     ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined,VDNN_CONV+refined+slack,"
-                    "BASELINE+fused,VDNN_CONV+refined+slack+fused,VDNN_CONV+refined+slack+zvc,VDNN_CONV+refined+ahead+zvc,"
-                    "VDNN_CONV+refined+ahead+zvc+tail,VDNN_CONV+refined+slack+zvc+tail,VDNN_ALL+refined+slack+fused+zvc,"
+                    "BASELINE+fused,VDNN_CONV+refined+slack+fused,VDNN_CONV+refined+slack+zvc,VDNN_CONV+refined+ahead+fused+zvc,"
+                    "VDNN_CONV+refined+ahead+fused+zvc+tail,VDNN_CONV+refined+slack+fused+zvc+tail,VDNN_ALL+refined+slack+fused+zvc,"
                     "BASELINE+bf16,VDNN_ALL+bf16,VDNN_CONV+refined+slack+bf16,VDNN_ALL+refined+slack+bf16,"
                     "BASELINE+bf16+fused,VDNN_CONV+refined+slack+bf16+fused,VDNN_CONV+refined+ahead+bf16+fused+zvc+tail,"
                     "VDNN_ALL+refined+slack+bf16+fused+zvc")

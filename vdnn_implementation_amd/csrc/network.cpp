@@ -453,6 +453,17 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         break;
     }
 
+    /* fused rectifiers: a layer whose input comes back by prefetch does not mask its data gradient by that input -
+       the data gradient then needs dy and W only and runs while the copy still lands (Layer::waitSrcFetched); the
+       ReLU below it does its own backward, as below a consumer that cannot mask */
+    for (int l = 1; l < numLayers; l++) {
+        if (!layer[l]->GateGrad() || !isOffload[l]) continue;
+        const Layer_t t = layer[l]->LayerType();
+        if (!is_conv(t) && t != FC_GEMM) continue; /* a pooling layer reads its input anyway */
+        layer[l]->setGateGrad(false);
+        layer[l - 1]->setElidedBackward(false);
+    }
+
     if (newVdnnType != BASELINE) {
         for (int l = 0; l < numLayers; l++)
             for (vdnn_event_t* e : {&evFwdDone[l], &evOffloadDone[l], &evBlockFree[l], &evPrefetchDone[l], &evPacked[l]})
