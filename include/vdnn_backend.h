@@ -282,8 +282,10 @@ int vdnn_cross_entropy_dense(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int cla
 
 /* ---- per-kernel timing (no counterpart in the reference, whose _PROFILE_* macros are unused:
  *      layer.h:34-38) ---------------------------------------------------------------------------
- * While enabled, every kernel launch of this library is bracketed by two events on its own stream.
- * vdnn_profile_collect synchronises the device and returns one entry per kernel class: launches,
+ * While enabled, every kernel launch of this library is bracketed by two events on its own stream - the
+ * first 2048 launches after vdnn_profile_enable, that is; the ones after them run untimed (thousands of live
+ * events slow every further one down). vdnn_profile_collect synchronises the device and returns one entry per
+ * kernel class: launches,
  * summed duration, and the algorithmic work of those launches (floating-point operations for the
  * MFMA kernels, bytes that must cross HBM for the bandwidth-bound ones). */
 typedef struct {

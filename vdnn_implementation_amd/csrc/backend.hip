@@ -340,6 +340,12 @@ int vdnn_profile_enable(vdnn_ctx* ctx, int on) {
     for (auto& r : ctx->prof_records) { ctx->prof_free_events.push_back(r.start); ctx->prof_free_events.push_back(r.stop); }
     ctx->prof_records.clear();
     ctx->profiling = on != 0;
+    // the events are made here, not in front of the first launches that need them
+    while (ctx->profiling && ctx->prof_free_events.size() < 2 * kProfMaxRecords) {
+        hipEvent_t e = nullptr;
+        if (hipEventCreate(&e) != hipSuccess) { (void)hipGetLastError(); break; }
+        ctx->prof_free_events.push_back(e);
+    }
     return VDNN_OK;
 }
 

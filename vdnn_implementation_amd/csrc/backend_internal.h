@@ -22,6 +22,9 @@ struct vdnn_ctx {
     int num_cu = 256;
     int act_dtype = VDNN_DTYPE_F32;   // element type of activation tensors handed to the kernels
     // per-kernel timing (vdnn_profile_*)
+    // At most kProfMaxRecords launches are timed between vdnn_profile_enable and vdnn_profile_collect; the
+    // launches after that run untimed. With more than about six thousand events alive, recording one became slow
+    // enough to double a step's time.
     struct ProfRecord { const char* name; hipEvent_t start, stop; double flops, bytes; };
     bool profiling = false;
     std::vector<ProfRecord> prof_records;
@@ -42,12 +45,14 @@ void set_error(const char* fmt, ...);
 inline hipStream_t stream_of(vdnn_ctx* ctx, vdnn_stream_t s) { return s ? (hipStream_t)s : ctx->compute; }
 
 hipEvent_t prof_take_event(vdnn_ctx* ctx);
+static constexpr size_t kProfMaxRecords = 2048;
 
 // Brackets the launches made during its lifetime with two timing events when profiling is on.
 // `name` must be a string literal (it is kept by pointer).
 struct ProfScope {
     vdnn_ctx* ctx; hipStream_t stream; size_t index; bool active;
-    ProfScope(vdnn_ctx* c, hipStream_t s, const char* name, double flops, double bytes) : ctx(c), stream(s), index(0), active(c->profiling) {
+    ProfScope(vdnn_ctx* c, hipStream_t s, const char* name, double flops, double bytes)
+        : ctx(c), stream(s), index(0), active(c->profiling && c->prof_records.size() < kProfMaxRecords) {
         if (!active) return;
         vdnn_ctx::ProfRecord r{name, prof_take_event(c), prof_take_event(c), flops, bytes};
         if (!r.start || !r.stop) { active = false; return; }
