@@ -58,6 +58,10 @@ def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refin
         dt = time.perf_counter() - t0
         prof = be.profile_collect(net.context)
         be.profile_enable(net.context, False)
+        # the library times the first 2048 launches after profile_enable: the share of the run they stand for
+        untimed = prof.pop("untimed", {"launches": 0})["launches"]
+        timed = sum(v["launches"] for v in prof.values())
+        timed_share = timed / max(timed + untimed, 1)
         st = net.stats()
         loss = net.loss()
         tensor_bytes, link_bytes = be.zvc_traffic(net.context)
@@ -65,7 +69,8 @@ def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refin
         net.close()
     res = {"ms_per_step": dt * 1e3 / steps, "images_per_s": batch * steps / dt, "loss": loss,
            "peak_hbm_gb": st["peak_bytes_in_use"] / 1e9, "offload_gb_per_step": st["offload_bytes"] / 1e9,
-           "prefetch_gb_per_step": st["prefetch_bytes"] / 1e9, "pinned_gb": st["pinned_bytes"] / 1e9}
+           "prefetch_gb_per_step": st["prefetch_bytes"] / 1e9, "pinned_gb": st["pinned_bytes"] / 1e9,
+           "launches_timed_share": timed_share}
     # host link: busy time and rate of the copies, and how much of the copy time ran under compute
     # (the *_zvc entries are the compacting copies: their bytes are the tensors', not what crossed the link)
     link = ("offload_d2h", "prefetch_h2d", "offload_zvc", "offload_zvc_copy", "prefetch_zvc")
@@ -79,6 +84,7 @@ def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refin
                              max(sum(prof[k]["ms"] for k in keys if k in prof), 1e-9) * 1e3 / 1e9)
         res["d2h_gbs"] = rate(("offload_d2h", "offload_zvc", "offload_zvc_copy"))
         res["h2d_gbs"] = rate(("prefetch_h2d", "prefetch_zvc"))
+        copy_ms, kernel_ms = copy_ms / timed_share, kernel_ms / timed_share   # scaled to the whole run
         res["copy_busy_ms_per_step"] = copy_ms / steps
         res["kernel_busy_ms_per_step"] = kernel_ms / steps
         # step = kernels + copies - overlap + idle  =>  overlap >= kernels + copies - step

@@ -284,8 +284,8 @@ int vdnn_cross_entropy_dense(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int cla
  *      layer.h:34-38) ---------------------------------------------------------------------------
  * While enabled, every kernel launch of this library is bracketed by two events on its own stream - the
  * first 2048 launches after vdnn_profile_enable, that is; the ones after them run untimed (thousands of live
- * events slow every further one down). vdnn_profile_collect synchronises the device and returns one entry per
- * kernel class: launches,
+ * events slow every further one down; an entry named "untimed" counts them). vdnn_profile_collect synchronises
+ * the device and returns one entry per kernel class: launches,
  * summed duration, and the algorithmic work of those launches (floating-point operations for the
  * MFMA kernels, bytes that must cross HBM for the bandwidth-bound ones). */
 typedef struct {

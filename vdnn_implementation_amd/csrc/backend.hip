@@ -339,6 +339,7 @@ int vdnn_profile_enable(vdnn_ctx* ctx, int on) {
     VDNN_HIP(hipDeviceSynchronize());
     for (auto& r : ctx->prof_records) { ctx->prof_free_events.push_back(r.start); ctx->prof_free_events.push_back(r.stop); }
     ctx->prof_records.clear();
+    ctx->prof_untimed = 0;
     ctx->profiling = on != 0;
     // the events are made here, not in front of the first launches that need them
     while (ctx->profiling && ctx->prof_free_events.size() < 2 * kProfMaxRecords) {
@@ -367,6 +368,13 @@ int vdnn_profile_collect(vdnn_ctx* ctx, vdnn_profile_entry* out, int capacity, i
             agg.push_back(e);
         }
         agg[i].launches += 1; agg[i].ms += ms; agg[i].flops += r.flops; agg[i].bytes += r.bytes;
+    }
+    if (ctx->prof_untimed) {
+        vdnn_profile_entry e;
+        memset(&e, 0, sizeof(e));
+        strncpy(e.name, "untimed", sizeof(e.name) - 1);
+        e.launches = ctx->prof_untimed;
+        agg.push_back(e);
     }
     *count = (int)agg.size();
     for (int i = 0; i < (int)agg.size() && i < capacity; i++) if (out) out[i] = agg[i];

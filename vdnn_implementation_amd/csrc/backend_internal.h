@@ -29,6 +29,7 @@ struct vdnn_ctx {
     bool profiling = false;
     std::vector<ProfRecord> prof_records;
     std::vector<hipEvent_t> prof_free_events;
+    unsigned long long prof_untimed = 0;   // launches since vdnn_profile_enable that ran beyond the limit
     // zero-value compression of offloaded tensors: device words (bytes sent over the link, then the stream
     // cursors of the offloads in flight) and bytes of the tensors that were packed
     unsigned long long* zvc_counters = nullptr;
@@ -53,6 +54,7 @@ struct ProfScope {
     vdnn_ctx* ctx; hipStream_t stream; size_t index; bool active;
     ProfScope(vdnn_ctx* c, hipStream_t s, const char* name, double flops, double bytes)
         : ctx(c), stream(s), index(0), active(c->profiling && c->prof_records.size() < kProfMaxRecords) {
+        if (!active && c->profiling) c->prof_untimed++;
         if (!active) return;
         vdnn_ctx::ProfRecord r{name, prof_take_event(c), prof_take_event(c), flops, bytes};
         if (!r.start || !r.stop) { active = false; return; }
