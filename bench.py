@@ -41,9 +41,9 @@ def log(*a):
 
 
 def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0, bf16=False, offload_lag=0, prefetch_depth=1,
-               fuse=False, compress=False, keep_tail_bytes=0, ahead=False):
+               fuse=False, compress=False, keep_tail_bytes=0, ahead=False, keep_packed=False):
     net = Network(cnn, policy, algo, batch, seed=seed, refined=refined, cap_bytes=cap_bytes, bf16=bf16,
-                  offload_lag=offload_lag, prefetch_depth=prefetch_depth, fuse=fuse, compress=compress, keep_tail_bytes=keep_tail_bytes, prefetch_within_peak=ahead)
+                  offload_lag=offload_lag, prefetch_depth=prefetch_depth, fuse=fuse, compress=compress, keep_tail_bytes=keep_tail_bytes, prefetch_within_peak=ahead, keep_packed=keep_packed)
     try:
         for _ in range(warmup):
             assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
@@ -73,7 +73,7 @@ def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refin
            "launches_timed_share": timed_share}
     # host link: busy time and rate of the copies, and how much of the copy time ran under compute
     # (the *_zvc entries are the compacting copies: their bytes are the tensors', not what crossed the link)
-    link = ("offload_d2h", "prefetch_h2d", "offload_zvc", "offload_zvc_copy", "prefetch_zvc")
+    link = ("offload_d2h", "prefetch_h2d", "offload_zvc", "offload_zvc_copy", "prefetch_zvc")   # (not prefetch_zvc_device)
     copies = [prof[k] for k in link if k in prof]
     if tensor_bytes:
         res["zvc_link_bytes_per_tensor_byte"] = link_bytes / tensor_bytes
@@ -131,7 +131,7 @@ def zvc_standalone(be):
             check(lib.vdnn_host_alloc_pinned(ctx.handle, C.byref(host), need))
             be.profile_enable(ctx.handle, True)
             for _ in range(5):
-                check(lib.vdnn_zvc_offload_staged_async(ctx.handle, host, stage.ptr, need // 2 // 16 * 16 + 65536, src.ptr, count, es, None, None, None, None))
+                check(lib.vdnn_zvc_offload_staged_async(ctx.handle, host, stage.ptr, need // 2 // 16 * 16 + 65536, src.ptr, count, es, None, None, None, None, 0))
                 ctx.synchronize()
                 check(lib.vdnn_zvc_prefetch_async(ctx.handle, dst.ptr, host, count, es, None))
                 ctx.synchronize()
@@ -179,9 +179,10 @@ def main():
     ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined,VDNN_CONV+refined+slack,"
                     "BASELINE+fused,VDNN_CONV+refined+slack+fused,VDNN_CONV+refined+slack+zvc,VDNN_CONV+refined+ahead+fused+zvc,"
                     "VDNN_CONV+refined+ahead+fused+zvc+tail,VDNN_CONV+refined+slack+fused+zvc+tail,VDNN_ALL+refined+slack+fused+zvc,"
+                    "VDNN_ALL+refined+fused+zvc+keep,VDNN_CONV+refined+fused+zvc+keep,"
                     "BASELINE+bf16,VDNN_ALL+bf16,VDNN_CONV+refined+slack+bf16,VDNN_ALL+refined+slack+bf16,"
                     "BASELINE+bf16+fused,VDNN_CONV+refined+slack+bf16+fused,VDNN_CONV+refined+ahead+bf16+fused+zvc+tail,"
-                    "VDNN_ALL+refined+slack+bf16+fused+zvc")
+                    "VDNN_ALL+refined+slack+bf16+fused+zvc,VDNN_ALL+refined+bf16+fused+zvc+keep,VDNN_CONV+refined+bf16+fused+zvc+keep")
     ap.add_argument("--cap-gb", type=float, default=0.0, help="artificial limit on pool bytes in use (0 = none)")
     ap.add_argument("--bf16", action="store_true", help="bfloat16 activation storage (products on the bfloat16 matrix cores, float accumulation and parameters)")
     ap.add_argument("--offload-lag", type=int, default=0, help="layers enqueued before an offloaded block is recycled (0 = reference schedule)")
@@ -209,14 +210,15 @@ def main():
         word, *mods = name.split("+")
         # "+tail" = the deepest offloaded tensors, 0.75 G elements of them, stay on the device
         # "+ahead" = backward fetches ahead wherever the peak cannot rise, blocks recycled six layers after their offload
-        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead"}, name
+        # "+keep" = with zvc: the packed tensors stay in device memory instead of crossing the link
+        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep"}, name
         _, policy, algo = parse("VGG16_128", word, args.algo)
         lag, depth = (6, 2) if "slack" in mods else (6, 1) if "ahead" in mods else (args.offload_lag, args.prefetch_depth)
         log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
         results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1,
                                                    refined=("refined" in mods), cap_bytes=int(args.cap_gb * 1e9),
                                                    bf16=(args.bf16 or "bf16" in mods), offload_lag=lag, prefetch_depth=depth,
-                                                   fuse=("fused" in mods), compress=("zvc" in mods), ahead=("ahead" in mods), keep_tail_bytes=(int(0.75e9) * (2 if (args.bf16 or "bf16" in mods) else 4) if "tail" in mods
+                                                   fuse=("fused" in mods), compress=("zvc" in mods), ahead=("ahead" in mods), keep_packed=("keep" in mods), keep_tail_bytes=(int(0.75e9) * (2 if (args.bf16 or "bf16" in mods) else 4) if "tail" in mods
                                                                     else int(args.keep_tail_gb * 1e9)))
         log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
             results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))

@@ -138,13 +138,19 @@ int vdnn_memcpy_h2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, si
  *     context's packing stream) behind what that stream holds, `packed` is recorded there when src_dev has been
  *     read, and the copy runs on copy_stream (NULL: the device-to-host stream) behind `packed`; with `packed`
  *     NULL everything runs on copy_stream. staging_dev must stay until the work on copy_stream is done.
- *   vdnn_zvc_prefetch_async: a kernel on `stream` reads the host buffer and expands it into dst_dev. */
+ *     With keep_on_device the copy engine is not used: bytes [0, staging_bytes) of the stream stay in staging_dev
+ *     (nothing crosses the link but what did not fit), for vdnn_zvc_prefetch_staged_async to read them there.
+ *   vdnn_zvc_prefetch_async: a kernel on `stream` reads the host buffer and expands it into dst_dev.
+ *   vdnn_zvc_prefetch_staged_async: the same, reading the stream's first staging_bytes from staging_dev (a block
+ *     that vdnn_zvc_offload_staged_async was told to keep) and the rest from the host buffer. */
 size_t vdnn_zvc_buffer_bytes(size_t count, int elem_bytes);
 int vdnn_zvc_offload_async(vdnn_ctx* ctx, void* dst_host, const void* src_dev, size_t count, int elem_bytes, vdnn_stream_t stream);
 int vdnn_zvc_offload_staged_async(vdnn_ctx* ctx, void* dst_host, void* staging_dev, size_t staging_bytes, const void* src_dev, size_t count,
                                   int elem_bytes, unsigned long long* total_host, vdnn_stream_t pack_stream, vdnn_stream_t copy_stream,
-                                  vdnn_event_t packed);
+                                  vdnn_event_t packed, int keep_on_device);
 int vdnn_zvc_prefetch_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t count, int elem_bytes, vdnn_stream_t stream);
+int vdnn_zvc_prefetch_staged_async(vdnn_ctx* ctx, void* dst_dev, const void* staging_dev, size_t staging_bytes, const void* src_host,
+                                   size_t count, int elem_bytes, vdnn_stream_t stream);
 /* Bytes of the tensors offloaded this way since the context was made, and bytes that crossed the link for
  * them (waits for the device). */
 int vdnn_zvc_traffic(vdnn_ctx* ctx, unsigned long long* tensor_bytes, unsigned long long* link_bytes);

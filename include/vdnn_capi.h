@@ -33,6 +33,8 @@ typedef struct {
     int      fuse_activations;  /* a ReLU after a CONV / FC layer runs inside the neighbouring layers' kernels (same bits, layer.cu:766-814) */
     size_t   keep_tail_bytes;   /* the deepest tensors of the policy's offload set stay on the device, up to this many bytes (0 = the reference's policies, network.cu:898-921) */
     int      prefetch_within_peak; /* backward fetches tensors ahead of the reference's schedule (network.cu:1198-1208) wherever a replay of the schedule shows that the peak cannot rise */
+    int      keep_packed_on_device; /* with compress_offload: the packed tensors stay in device memory (about 0.6 of their size) instead of crossing the link */
+    double   plan_packed_fraction;  /* what a plan-only network assumes a packed stream to be of its tensor (0 = the longest possible, 1.03) */
     int      compress_offload;  /* offloaded rectified tensors cross the link without their zero elements (lossless; layer.cu:969-987 copies them whole) */
 } vdnn_network_options;
 

@@ -89,9 +89,13 @@ STAGING = [None, 0.0, 0.37, 0.999, 1.0, 1.5]
 
 
 @pytest.mark.parametrize("dtype", [np.uint32, np.uint16])
+@pytest.mark.parametrize("keep", [False, True])
 @pytest.mark.parametrize("staging", STAGING)
 @pytest.mark.parametrize("count,zero_fraction", CASES)
-def test_round_trip_and_host_format(ctx, dtype, count, zero_fraction, staging):
+def test_round_trip_and_host_format(ctx, dtype, count, zero_fraction, staging, keep):
+    """keep: the staging block is where the stream's first bytes stay (no copy), and the expanding kernel reads them there."""
+    if keep and not staging:
+        pytest.skip("nothing to keep without a staging block")
     es = np.dtype(dtype).itemsize
     rng = np.random.default_rng(count * 7 + es)
     a = tensor(rng, count, dtype, zero_fraction)
@@ -109,49 +113,55 @@ def test_round_trip_and_host_format(ctx, dtype, count, zero_fraction, staging):
     dst.upload(np.full(count * es + 64, 0xEE, np.uint8))
     t0, l0 = C.c_ulonglong(), C.c_ulonglong()
     check(lib.vdnn_zvc_traffic(ctx.handle, C.byref(t0), C.byref(l0)))
-    announce(f"zvc round trip count={count} bytes={es} zeros={zero_fraction} staging={staging}")
-    stage_bytes, stage, word = 0, None, None
+    announce(f"zvc round trip count={count} bytes={es} zeros={zero_fraction} staging={staging} keep={keep}")
+    stage_bytes, stage, word, packed = 0, None, None, None
+    per_chunk = [int(np.count_nonzero(a[c * CHUNK:(c + 1) * CHUNK])) for c in range(chunks)]
+    length = (chunks * 4 + 15) // 16 * 16 + sum(MAP + (k * es + 15) // 16 * 16 for k in per_chunk)   # table, maps, kept elements
     if staging is None:
         check(lib.vdnn_zvc_offload_async(ctx.handle, host.ptr, src.ptr, count, es, None))
     else:
-        kept = int(np.count_nonzero(a))   # the stream's length follows from the tensor: table, maps, kept elements
-        per_chunk = [int(np.count_nonzero(a[c * CHUNK:(c + 1) * CHUNK])) for c in range(chunks)]
-        length = (chunks * 4 + 15) // 16 * 16 + sum(MAP + (k * es + 15) // 16 * 16 for k in per_chunk)
         stage_bytes = min(int(length * staging) // 16 * 16, need)
         stage = ctx.alloc(max(stage_bytes, 16))
         word = Pinned(ctx, 8)
         word.view[:] = 0xFF
-        packed = None
         if count % 2:   # with an event the kernel runs on the packing stream and the copy behind it on the copy stream
             packed = C.c_void_p()
             check(lib.vdnn_event_create(ctx.handle, C.byref(packed), 0))
-        check(lib.vdnn_zvc_offload_staged_async(ctx.handle, host.ptr, stage.ptr, stage_bytes, src.ptr, count, es, word.ptr, None, None, packed))
+        check(lib.vdnn_zvc_offload_staged_async(ctx.handle, host.ptr, stage.ptr, stage_bytes, src.ptr, count, es, word.ptr, None, None, packed, int(keep)))
     ctx.synchronize()
-    decoded, length_seen = decode(host.view, count, dtype)
-    assert np.array_equal(decoded, a), "host bytes decode to the tensor"
     t1, l1 = C.c_ulonglong(), C.c_ulonglong()
     check(lib.vdnn_zvc_traffic(ctx.handle, C.byref(t1), C.byref(l1)))
     assert t1.value - t0.value == count * es
-    assert l1.value - l0.value == max(length_seen, stage_bytes)
-    if staging is not None:
+    if keep:
+        assert l1.value - l0.value == max(0, length - stage_bytes), "only what the block could not hold crossed the link"
+        assert (host.view[:stage_bytes] == 0xA5).all(), "the kept part never reaches the host buffer"
+    else:
+        decoded, length_seen = decode(host.view, count, dtype)
+        assert np.array_equal(decoded, a), "host bytes decode to the tensor"
         assert length_seen == length
+        assert l1.value - l0.value == max(length, stage_bytes)
+    if staging is not None:
         assert int(word.view.view(np.uint64)[0]) == length, "the kernel reports the stream's length"
-        stage.free(); word.free()
-        if packed:
-            check(lib.vdnn_event_destroy(ctx.handle, packed))
-    check(lib.vdnn_zvc_prefetch_async(ctx.handle, dst.ptr, host.ptr, count, es, None))
+    if keep:
+        check(lib.vdnn_zvc_prefetch_staged_async(ctx.handle, dst.ptr, stage.ptr, stage_bytes, host.ptr, count, es, None))
+    else:
+        check(lib.vdnn_zvc_prefetch_async(ctx.handle, dst.ptr, host.ptr, count, es, None))
     ctx.synchronize()
     back = dst.download((count * es + 64,), np.uint8)
     assert np.array_equal(back[:count * es].view(dtype), a), "round trip"
     assert (back[count * es:] == 0xEE).all(), "nothing is written past the tensor"
     host.free(); src.free(); dst.free()
+    if stage is not None:
+        stage.free(); word.free()
+    if packed:
+        check(lib.vdnn_event_destroy(ctx.handle, packed))
 
 
 def test_rejects_bad_arguments(ctx):
     host = Pinned(ctx, lib.vdnn_zvc_buffer_bytes(100, 4))
     buf = ctx.alloc(400)
     stage = ctx.alloc(1 << 20)
-    staged = lambda ptr, nbytes: lib.vdnn_zvc_offload_staged_async(ctx.handle, host.ptr, ptr, nbytes, buf.ptr, 100, 4, None, None, None, None)
+    staged = lambda ptr, nbytes: lib.vdnn_zvc_offload_staged_async(ctx.handle, host.ptr, ptr, nbytes, buf.ptr, 100, 4, None, None, None, None, 0)
     assert staged(None, 64) != 0              # bytes without a buffer
     assert staged(stage.ptr, 24) != 0         # not a multiple of 16
     assert staged(stage.ptr + 4, 64) != 0     # misaligned
@@ -199,6 +209,9 @@ def test_networks_with_compressed_offload_keep_every_bit(cnn, batch, algo, bf16)
                        (VDNN_ALL, {"fuse": True}), (VDNN_CONV, {"fuse": True, "offload_lag": 3, "keep_tail_bytes": tail}),
                        (VDNN_ALL, {"refined": True, "keep_tail_bytes": tail}),
                        (VDNN_CONV, {"refined": True, "offload_lag": 6, "prefetch_within_peak": True}),
+                       (VDNN_ALL, {"refined": True, "fuse": True, "keep_packed": True}),
+                       (VDNN_CONV, {"offload_lag": 4, "keep_packed": True, "prefetch_depth": 2}),
+                       (VDNN_ALL, {"host_sync": True, "keep_packed": True}),
                        (VDNN_ALL, {"fuse": True, "offload_lag": 2, "prefetch_within_peak": True, "keep_tail_bytes": tail // 2})):
         announce("compressed offload", cnn, batch, "policy", policy, kw)
         with make(policy, compress=True, **kw) as net:
@@ -248,6 +261,8 @@ def test_losses_at_a_batch_that_keeps_the_streams_busy(bf16):
     for policy, kw in ((VDNN_CONV, {"refined": True, "offload_lag": 6, "prefetch_depth": 2}), (VDNN_ALL, {"refined": True, "offload_lag": 6, "prefetch_depth": 2}),
                        (VDNN_CONV, {}), (VDNN_ALL, {"offload_lag": 2}),
                        (VDNN_CONV, {"refined": True, "offload_lag": 6, "prefetch_within_peak": True, "keep_tail_bytes": 40 << 20}),
-                       (VDNN_ALL, {"refined": True, "offload_lag": 6, "prefetch_within_peak": True})):
+                       (VDNN_ALL, {"refined": True, "offload_lag": 6, "prefetch_within_peak": True}),
+                       (VDNN_ALL, {"refined": True, "offload_lag": 6, "keep_packed": True}),
+                       (VDNN_CONV, {"keep_packed": True, "keep_tail_bytes": 40 << 20})):
         announce("compressed offload at batch 32, policy", policy, kw, "bf16", bf16)
         assert losses(policy, fuse=True, compress=True, **kw) == want, "policy %d %s" % (policy, kw)

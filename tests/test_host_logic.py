@@ -482,3 +482,34 @@ def test_prefetch_within_peak_fetches_earlier_and_holds_the_peak():
     with plan(VGG16_128, BASELINE, batch=128, prefetch_within_peak=True) as net:
         step(net)
         assert net.prefetch_trace() == []
+
+
+def test_packed_tensors_kept_on_the_device_plan():
+    """keep_packed: the packed stream of a rectified offloaded tensor stays in its staging block; nothing of it crosses
+    the link, its own layer expands it at the start of its backward, and the peak follows the assumed stream length."""
+    kw = dict(refined=True, fuse=True, compress=True)
+    with plan(VGG16_128, VDNN_ALL, batch=128, **kw) as moved, \
+         plan(VGG16_128, VDNN_ALL, batch=128, keep_packed=True, plan_packed_fraction=0.57, **kw) as kept, \
+         plan(VGG16_128, VDNN_ALL, batch=128, keep_packed=True, **kw) as kept_worst:
+        for net in (moved, kept, kept_worst):
+            step(net); step(net)
+        sm, sk, sw = moved.stats(), kept.stats(), kept_worst.stats()
+        # only the tensors that are not rectified (the network input) still travel
+        plain = [l for l in range(kept.num_layers) if kept.is_offloaded(l)]
+        first = int(np.prod(kept.src_shape(0))) * 4
+        assert sk["offload_bytes"] == first == sk["prefetch_bytes"] and 0 in plain
+        assert sm["offload_bytes"] > 7e9
+        # every kept tensor is expanded by its own layer; the one that travelled is fetched a layer ahead
+        trace = kept.prefetch_trace()
+        assert sorted(p for _, p in trace) == plain
+        assert all(l == p for l, p in trace if p != 0) and (2, 0) in trace
+        # at 0.57 of a tensor the step holds less than a third of BASELINE's 18.65 GB; at the longest stream it does not
+        assert sk["peak_bytes_in_use"] < 18.65e9 / 3 < sw["peak_bytes_in_use"]
+        assert live_blocks(kept) == live_blocks(moved) == live_blocks(kept_worst)
+    # a forward without a backward leaves packed blocks behind; the next forward returns them
+    with plan(VGG16_128, VDNN_CONV, batch=16, keep_packed=True, plan_packed_fraction=0.6, compress=True) as net:
+        assert net.forwardPropagation() == 0
+        held = live_blocks(net)
+        assert net.forwardPropagation() == 0
+        assert live_blocks(net) == held
+        assert net.backwardPropagation() == 0

@@ -84,7 +84,8 @@ BACKEND_SYMBOLS = {
     "vdnn_memcpy_h2d_async": (_i, [_vp, _vp, _vp, _sz, _vp]),
     "vdnn_zvc_buffer_bytes": (_sz, [_sz, _i]),
     "vdnn_zvc_offload_async": (_i, [_vp, _vp, _vp, _sz, _i, _vp]),
-    "vdnn_zvc_offload_staged_async": (_i, [_vp, _vp, _vp, _sz, _vp, _sz, _i, _vp, _vp, _vp, _vp]),
+    "vdnn_zvc_offload_staged_async": (_i, [_vp, _vp, _vp, _sz, _vp, _sz, _i, _vp, _vp, _vp, _vp, _i]),
+    "vdnn_zvc_prefetch_staged_async": (_i, [_vp, _vp, _vp, _sz, _vp, _sz, _i, _vp]),
     "vdnn_zvc_prefetch_async": (_i, [_vp, _vp, _vp, _sz, _i, _vp]),
     "vdnn_zvc_traffic": (_i, [_vp, C.POINTER(C.c_ulonglong), C.POINTER(C.c_ulonglong)]),
     "vdnn_memcpy_d2h": (_i, [_vp, _vp, _vp, _sz]),

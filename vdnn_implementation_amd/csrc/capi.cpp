@@ -23,6 +23,8 @@ static NetworkOptions to_options(const vdnn_network_options* o) {
     n.fuseActivations = o->fuse_activations != 0;
     n.compressOffload = o->compress_offload != 0;
     n.keepTailBytes = o->keep_tail_bytes;
+    n.keepPackedOnDevice = o->keep_packed_on_device != 0;
+    n.planPackedFraction = o->plan_packed_fraction;
     n.prefetchWithinPeak = o->prefetch_within_peak != 0;
     return n;
 }

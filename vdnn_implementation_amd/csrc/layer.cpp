@@ -496,7 +496,7 @@ void Layer::offloadSrcData(bool*, DATATYPE** _offloadedSrcData_h) {
         vdnn_stream_t pack = srcPackedEvent ? vdnn_ctx_stream_pack(ctx) : *stream_memory;
         if (srcReadyEvent) checkVDNN(vdnn_stream_wait_event(ctx, pack, srcReadyEvent));
         checkVDNN(vdnn_zvc_offload_staged_async(ctx, _offloadedSrcData_h[layerId], offloadStaging, offloadStagingBytes, srcData, SrcDataSize(),
-                                                actBytes, offloadLengthWord, pack, *stream_memory, srcPackedEvent));
+                                                actBytes, offloadLengthWord, pack, *stream_memory, srcPackedEvent, offloadKeep ? 1 : 0));
     } else {
         if (srcReadyEvent) checkVDNN(vdnn_stream_wait_event(ctx, *stream_memory, srcReadyEvent));
         checkVDNN(vdnn_memcpy_d2h_async(ctx, _offloadedSrcData_h[layerId], srcData, SrcDataSize() * actBytes, *stream_memory));
@@ -515,7 +515,8 @@ void Layer::prefetchPreviousSrcData(DATATYPE* _prefetchedSrcData_h, void* _srcDa
     }
     if (prefetchHostReadyEvent) checkVDNN(vdnn_stream_wait_event(ctx, h2d, prefetchHostReadyEvent));
     if (prefetchPacked)
-        checkVDNN(vdnn_zvc_prefetch_async(ctx, _srcDataToPrefetch, _prefetchedSrcData_h, _prefetch_bytes / actBytes, actBytes, h2d));
+        checkVDNN(vdnn_zvc_prefetch_staged_async(ctx, _srcDataToPrefetch, prefetchStaging, prefetchStagingBytes, _prefetchedSrcData_h,
+                                                 _prefetch_bytes / actBytes, actBytes, h2d));
     else
         checkVDNN(vdnn_memcpy_h2d_async(ctx, _srcDataToPrefetch, _prefetchedSrcData_h, _prefetch_bytes, h2d));
     if (prefetchDoneEvent) checkVDNN(vdnn_event_record(ctx, prefetchDoneEvent, h2d));

@@ -202,9 +202,13 @@ public:
     // Where the packed stream of this layer's input is staged on its way out (bytes may be 0: the kernel stores
     // all of it into host memory itself), the pinned word that receives its length, and the event recorded when
     // the packing kernel has read srcData.
-    void    setOffloadStaging(void* staging, size_t bytes, unsigned long long* lengthWord, vdnn_event_t packed) {
+    // With `keep` the staging block is where the stream stays (no copy to the host but of what did not fit).
+    void    setOffloadStaging(void* staging, size_t bytes, unsigned long long* lengthWord, vdnn_event_t packed, bool keep) {
         offloadStaging = staging; offloadStagingBytes = bytes; offloadLengthWord = lengthWord; srcPackedEvent = packed;
+        offloadKeep = keep;
     }
+    // The block that holds the first bytes of the packed stream this layer fetches next (null: all of it is on the host).
+    void    setPrefetchStaging(void* staging, size_t bytes) { prefetchStaging = staging; prefetchStagingBytes = bytes; }
 
     /* Get functions */
     Layer_t LayerType()              { return layerType; }
@@ -296,6 +300,9 @@ private:
     void*   offloadStaging = nullptr;
     size_t  offloadStagingBytes = 0;
     unsigned long long* offloadLengthWord = nullptr;
+    bool    offloadKeep = false;
+    void*   prefetchStaging = nullptr;
+    size_t  prefetchStagingBytes = 0;
     vdnn_event_t srcPackedEvent = nullptr;
 
     /* Connection to other layers (GoogLeNet plumbing of the reference, unused) */

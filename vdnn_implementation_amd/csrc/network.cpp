@@ -132,6 +132,8 @@ void Network::construct(vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) {
         offloadedSrcData_h[i] = nullptr;
         evFwdDone[i] = evOffloadDone[i] = evBlockFree[i] = evPrefetchDone[i] = evPacked[i] = nullptr;
         zvcStaging[i] = nullptr;
+        zvcStagingBytes[i] = 0;
+        zvcKept[i] = false;
         srcReleasedEarly[i] = false;
     }
     zvcLength_h = nullptr;
@@ -593,6 +595,12 @@ int Network::forwardPropagation(bool isDynamic) {
     } else {
         /* everything enqueued so far (the previous step's last prefetch included) precedes this event */
         checkVDNN(vdnn_event_record(ctx, evBlockFree[0], stream_compute));
+        /* packed streams that a forward without a backward left on the device */
+        for (int l = 0; l < numLayers; l++) {
+            if (zvcKept[l] && zvcStaging[l]) ASSERT_EQ(vdnn_pool_free(ctx, zvcStaging[l]), isDynamic);
+            zvcKept[l] = false;
+            zvcStaging[l] = nullptr;
+        }
         for (int l = 0; l < numLayers; l++) {
             layer[l]->copySrcData(l == 0 ? inputData : layer[l - 1]->DstData());
             if (isOffload[l]) {
@@ -607,7 +615,9 @@ int Network::forwardPropagation(bool isDynamic) {
             srcReleasedEarly[l] = false;
             if (isOffload[l] && layer[l]->SrcPacked()) {
                 const size_t longest = vdnn_zvc_buffer_bytes(layer[l]->SrcDataSize(), (int)actBytes());
-                const size_t known = options.planOnly ? longest : (size_t)zvcLength_h[l];
+                const size_t assumed = options.planPackedFraction > 0.0
+                                           ? (size_t)(options.planPackedFraction * (double)(layer[l]->SrcDataSize() * actBytes())) : longest;
+                const size_t known = options.planOnly ? assumed : (size_t)zvcLength_h[l];
                 size_t want = known ? known + known / 32 + 65536 : 0;
                 want = std::min(longest, (want + 15) / 16 * 16);
                 if (want && ASSERT_EQ(vdnn_pool_malloc(ctx, &zvcStaging[l], want), isDynamic) < 0) return -1;
@@ -617,7 +627,9 @@ int Network::forwardPropagation(bool isDynamic) {
                     checkVDNN(vdnn_event_record(ctx, evBlockFree[l], stream_compute));
                     layer[l]->setSrcReadyEvent(evBlockFree[l]);
                 }
-                layer[l]->setOffloadStaging(zvcStaging[l], want, options.planOnly ? nullptr : &zvcLength_h[l], evPacked[l]);
+                zvcStagingBytes[l] = want;
+                zvcKept[l] = options.keepPackedOnDevice && want > 0;
+                layer[l]->setOffloadStaging(zvcStaging[l], want, options.planOnly ? nullptr : &zvcLength_h[l], evPacked[l], zvcKept[l]);
             }
 
             /* Forward propagation */
@@ -634,7 +646,7 @@ int Network::forwardPropagation(bool isDynamic) {
                a second one for its prefetch; releasing it here avoids that leak. With offloadLag the
                wait for the copy and the release move behind the next `offloadLag` layers. */
             if (isOffload[l]) {
-                lastStats.offloadBytes += layer[l]->SrcDataSize() * actBytes();
+                if (!zvcKept[l]) lastStats.offloadBytes += layer[l]->SrcDataSize() * actBytes();
                 pendingOffload.push_back(l);
                 if (zvcStaging[l]) {
                     /* the staging block has the tensor: srcData goes back behind this layer's kernels and the
@@ -653,8 +665,10 @@ int Network::forwardPropagation(bool isDynamic) {
                 const int j = pendingOffload.front();
                 pendingOffload.erase(pendingOffload.begin());
                 if (!options.hostSync) checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evOffloadDone[j]));
-                if (zvcStaging[j]) ASSERT_EQ(vdnn_pool_free(ctx, zvcStaging[j]), isDynamic);
-                zvcStaging[j] = nullptr;
+                if (zvcStaging[j] && !zvcKept[j]) {
+                    ASSERT_EQ(vdnn_pool_free(ctx, zvcStaging[j]), isDynamic);
+                    zvcStaging[j] = nullptr;
+                }
                 if (!srcReleasedEarly[j]) ASSERT_EQ(vdnn_pool_free(ctx, layer[j]->SrcData()), isDynamic);
                 if (j == 0) { inputData = nullptr; inputResident = false; }
             }
@@ -729,17 +743,38 @@ int Network::backwardPropagation(bool isDynamic) {
                     dstReleased = true;
                 }
             }
-            /* this layer reads its own srcData: if that was prefetched, the copy must have landed */
-            layer[l]->setSrcFetchedEvent(!options.hostSync && isPrefetched[l] ? evPrefetchDone[l] : nullptr);
+            /* a packed input that stayed on the device is expanded now, not a layer ahead: that takes HBM time only
+               (a millisecond for the largest), and so the tensor, its packed block and the working set of the
+               layer above are never held together; the block goes back before this layer allocates anything */
+            if (isOffload[l] && zvcKept[l] && !isPrefetched[l]) {
+                isPrefetched[l] = true;
+                if (layer[l]->cnmemMallocSrcData(isDynamic) < 0) return -1;
+                layer[l]->setPrefetchEvents(evBlockFree[l], evOffloadDone[l], evPrefetchDone[l]);
+                layer[l]->setPrefetchPacked(true);
+                layer[l]->setPrefetchStaging(zvcStaging[l], zvcStagingBytes[l]);
+                layer[l]->prefetchPreviousSrcData(offloadedSrcData_h[l], layer[l]->SrcData(), actBytes() * layer[l]->SrcDataSize());
+                prefetchLog.emplace_back(l, l);
+                if (l == 0) { inputData = layer[0]->SrcData(); inputResident = true; }
+                if (options.hostSync) afterLayerSync();
+                else checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evPrefetchDone[l]));
+                ASSERT_EQ(vdnn_pool_free(ctx, zvcStaging[l]), isDynamic);
+                zvcStaging[l] = nullptr;
+                zvcKept[l] = false;
+                layer[l]->setSrcFetchedEvent(nullptr);
+            } else {
+                /* this layer reads its own srcData: if that was prefetched, the copy must have landed */
+                layer[l]->setSrcFetchedEvent(!options.hostSync && isPrefetched[l] ? evPrefetchDone[l] : nullptr);
+            }
 
             int prefId = l == 0 ? -1 : (options.prefetchDepth > 1 ? findPrefetchLayerDeep(l) : findPrefetchLayer(l));
             if (prefId >= 0) {
                 if (layer[prefId]->cnmemMallocSrcData(isDynamic) < 0) return -1;
                 layer[l]->setPrefetchEvents(evBlockFree[prefId], evOffloadDone[prefId], evPrefetchDone[prefId]);
                 layer[l]->setPrefetchPacked(layer[prefId]->SrcPacked());
+                layer[l]->setPrefetchStaging(zvcKept[prefId] ? zvcStaging[prefId] : nullptr, zvcKept[prefId] ? zvcStagingBytes[prefId] : 0);
                 const size_t bytes = actBytes() * layer[prefId]->SrcDataSize();
                 if (layer[l]->backward(prefId, offloadedSrcData_h[prefId], layer[prefId]->SrcData(), bytes, workSpace, isDynamic) < 0) return -1;
-                lastStats.prefetchBytes += bytes;
+                if (!zvcKept[prefId]) lastStats.prefetchBytes += bytes;
                 prefetchLog.emplace_back(l, prefId);
                 if (prefId == 0) { inputData = layer[0]->SrcData(); inputResident = true; }
             } else {
@@ -753,9 +788,10 @@ int Network::backwardPropagation(bool isDynamic) {
                 if (layer[extra]->cnmemMallocSrcData(isDynamic) < 0) return -1;
                 layer[l]->setPrefetchEvents(evBlockFree[extra], evOffloadDone[extra], evPrefetchDone[extra]);
                 layer[l]->setPrefetchPacked(layer[extra]->SrcPacked());
+                layer[l]->setPrefetchStaging(zvcKept[extra] ? zvcStaging[extra] : nullptr, zvcKept[extra] ? zvcStagingBytes[extra] : 0);
                 const size_t bytes = actBytes() * layer[extra]->SrcDataSize();
                 layer[l]->prefetchPreviousSrcData(offloadedSrcData_h[extra], layer[extra]->SrcData(), bytes);
-                lastStats.prefetchBytes += bytes;
+                if (!zvcKept[extra]) lastStats.prefetchBytes += bytes;
                 prefetchLog.emplace_back(l, extra);
                 if (extra == 0) { inputData = layer[0]->SrcData(); inputResident = true; }
             }
@@ -769,6 +805,12 @@ int Network::backwardPropagation(bool isDynamic) {
             if (!dstReleased && !layer[l]->Elided()) ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DstData()), isDynamic);
             if (!(layer[l]->InPlaceOp() && layer[l]->GradData() == layer[l]->DiffData()))
                 ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DiffData()), isDynamic);
+            /* this layer's packed input has been expanded (its backward waited for that): the block goes back */
+            if (zvcKept[l] && zvcStaging[l]) {
+                ASSERT_EQ(vdnn_pool_free(ctx, zvcStaging[l]), isDynamic);
+                zvcStaging[l] = nullptr;
+                zvcKept[l] = false;
+            }
             printUsage("Bwd", l, layer[l]->BwdDataWorkSpaceSize() + layer[l]->BwdFilterWorkSpaceSize());
             if (options.tracePeaks) {
                 size_t inUse = 0, extent = 0;
@@ -824,7 +866,7 @@ int Network::findPrefetchLayerDeep(int currLayerId) {
         if (isOffload[id] && isPrefetched[id]) outstanding++;
     if (outstanding >= options.prefetchDepth) return -1;
     for (int id = currLayerId - 1; id >= 0; id--) {
-        if (isOffload[id] && !isPrefetched[id]) {
+        if (isOffload[id] && !isPrefetched[id] && !zvcKept[id]) {
             isPrefetched[id] = true;
             return id;
         }
@@ -855,7 +897,7 @@ void Network::buildPeakPlan(vdnn_t policy) {
 int Network::findPrefetchWithinPeak(int currLayerId) {
     if (planBwdPeak.size() != (size_t)numLayers) return -1;
     for (int id = currLayerId - 1; id >= 0; id--) {
-        if (!isOffload[id] || isPrefetched[id]) continue;
+        if (!isOffload[id] || isPrefetched[id] || zvcKept[id]) continue;
         const int issue = planIssueLayer[id];
         if (issue < 0 || issue >= currLayerId) return -1;
         const size_t bytes = actBytes() * layer[id]->SrcDataSize();
@@ -872,7 +914,7 @@ int Network::findPrefetchWithinPeak(int currLayerId) {
  * yet prefetched is the one to fetch; stop at the first convolution that is not eligible */
 int Network::findPrefetchLayer(int currLayerId) {
     for (int id = currLayerId - 1; id >= 0; id--) {
-        if (isOffload[id] == true && isPrefetched[id] == false) {
+        if (isOffload[id] == true && isPrefetched[id] == false && !zvcKept[id]) { /* (a kept packed input is expanded by its own layer) */
             isPrefetched[id] = true;
             return id;
         } else if (is_conv(layer[id]->LayerType())) {

@@ -62,6 +62,14 @@ struct NetworkOptions {
     // gone before the large tensors of the shallow layers come back: the peak is elsewhere. 0: the reference's
     // policies (network.cu:898-921).
     size_t   keepTailBytes = 0;
+    // With compressOffload: the packed stream of a tensor stays in its staging block on the device instead of
+    // going to the host, and backward expands it from there; the link carries only what a block sized from the
+    // step before could not hold. Trades the link for HBM: a rectified tensor then occupies about 0.6 of its size
+    // between its forward and its backward, at the price of reading and writing it once more each way.
+    bool     keepPackedOnDevice = false;
+    // What a plan-only context assumes a packed stream to be of its tensor (it has no data): 0 = the longest
+    // possible stream, 1.03 of the tensor.
+    double   planPackedFraction = 0.0;
     // Backward fetches further tensors ahead whenever that cannot raise the step's peak: the network replays
     // its own schedule on a context without a device, notes the bytes in use during every layer's backward,
     // and fetches a tensor early only if, at every layer between here and the layer that would have fetched
@@ -236,6 +244,8 @@ private:
     /* compressOffload: the packed stream of an offloaded input waits in device memory for the copy engine */
     vdnn_event_t        evPacked[DEFAULT_NUM_LAYER];      // d2h: the packing kernel has read srcData of layer l
     void*               zvcStaging[DEFAULT_NUM_LAYER];    // staging block of layer l's stream (null: none this step)
+    size_t              zvcStagingBytes[DEFAULT_NUM_LAYER];
+    bool                zvcKept[DEFAULT_NUM_LAYER];       // the block stays until backward has expanded it
     bool                srcReleasedEarly[DEFAULT_NUM_LAYER]; // srcData of layer l went back to the pool behind its forward
     unsigned long long* zvcLength_h;                       // pinned: length of each layer's stream, reported by the packing kernel
     std::vector<int>    pendingOffload;                    // offloaded layers whose block is not yet recycled (offloadLag)

@@ -57,6 +57,7 @@ int main(int argc, char** argv) {
         else if (!strcmp(argv[i], "--refined")) opt.refinedLifetimes = true;
         else if (!strcmp(argv[i], "--fuse")) opt.fuseActivations = true;
         else if (!strcmp(argv[i], "--zvc")) opt.compressOffload = true;
+        else if (!strcmp(argv[i], "--keep-packed")) opt.keepPackedOnDevice = true;
         else if (!strcmp(argv[i], "--prefetch-within-peak")) opt.prefetchWithinPeak = true;
         else if (!strcmp(argv[i], "--keep-tail-gb")) opt.keepTailBytes = (size_t)(atof(need("--keep-tail-gb needs a value")) * 1e9);
         else if (!strcmp(argv[i], "--unfused")) opt.unfusedOptimizer = true;

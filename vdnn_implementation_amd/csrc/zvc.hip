@@ -51,12 +51,14 @@ struct alignas(16) ZvcRecord {
 __global__ void zvc_begin_kernel(unsigned long long* cursor, unsigned long long table_bytes) { *cursor = table_bytes; }
 
 // total: length of the stream. link: bytes that cross the link for it (the copy engine moves `staging_bytes`
-// whatever the stream's length).
-__global__ void zvc_end_kernel(const unsigned long long* cursor, unsigned long long staging_bytes,
+// whatever the stream's length; with staging_bytes = ~0 the block stays on the device and only what did not fit
+// crossed the link - the caller passes the block's size in `kept_bytes` then).
+__global__ void zvc_end_kernel(const unsigned long long* cursor, unsigned long long staging_bytes, unsigned long long kept_bytes,
                                unsigned long long* total_host, unsigned long long* link_bytes) {
     const unsigned long long total = *cursor;
     if (total_host) *total_host = total;
-    atomicAdd(link_bytes, total > staging_bytes ? total : staging_bytes);
+    if (staging_bytes == ~0ull) atomicAdd(link_bytes, total > kept_bytes ? total - kept_bytes : 0ull);
+    else atomicAdd(link_bytes, total > staging_bytes ? total : staging_bytes);
 }
 
 // E is the element as raw bits (uint32_t for float, uint16_t for bfloat16).
@@ -138,8 +140,10 @@ __global__ __launch_bounds__(kZvcThreads) void zvc_pack_kernel(const E* __restri
     }
 }
 
+// The stream's bytes below `device_bytes` are read from `device` (a staging block that was kept), the rest from `host`.
 template <class E>
-__global__ __launch_bounds__(kZvcThreads) void zvc_unpack_kernel(const unsigned char* __restrict__ stream, E* __restrict__ dst,
+__global__ __launch_bounds__(kZvcThreads) void zvc_unpack_kernel(const unsigned char* __restrict__ device, size_t device_bytes,
+                                                                 const unsigned char* __restrict__ host, E* __restrict__ dst,
                                                                  size_t count, size_t chunks) {
     __shared__ unsigned long long words[kZvcTeams][kZvcGroups];
     __shared__ unsigned first[kZvcTeams][kZvcGroups + 1];   // kept elements ahead of each group, and their number overall
@@ -153,8 +157,10 @@ __global__ __launch_bounds__(kZvcThreads) void zvc_unpack_kernel(const unsigned 
         const size_t chunk = first_chunk + team;
         const bool live = chunk < chunks;
         if (wave == 0) {
-            const size_t at = live ? size_t(reinterpret_cast<const unsigned*>(stream)[chunk]) * 16 : 0;
-            const unsigned long long w = live ? reinterpret_cast<const unsigned long long*>(stream + at)[lane] : 0ull;
+            const size_t entry = chunk * 4;
+            const size_t at = live ? size_t(*reinterpret_cast<const unsigned*>((entry < device_bytes ? device : host) + entry)) * 16 : 0;
+            const size_t mine = at + size_t(lane) * 8;
+            const unsigned long long w = live ? *reinterpret_cast<const unsigned long long*>((mine < device_bytes ? device : host) + mine) : 0ull;
             words[team][lane] = w;
             unsigned sum = __popcll(w);
 #pragma unroll
@@ -168,9 +174,12 @@ __global__ __launch_bounds__(kZvcThreads) void zvc_unpack_kernel(const unsigned 
         __syncthreads();
         const unsigned total = first[team][kZvcGroups];
         const unsigned n16 = (total * unsigned(sizeof(E)) + 15u) / 16u;
-        const v4u* in = reinterpret_cast<const v4u*>(stream + place[team] + kZvcMapBytes);
+        const size_t values = place[team] + kZvcMapBytes;
         v4u* st = reinterpret_cast<v4u*>(kept[team]);
-        for (unsigned u = tid; u < n16; u += 256) st[u] = in[u];
+        for (unsigned u = tid; u < n16; u += 256) {
+            const size_t o = values + size_t(u) * 16;
+            st[u] = *reinterpret_cast<const v4u*>((o < device_bytes ? device : host) + o);
+        }
         __syncthreads();
         const size_t base = chunk * kZvcChunk + size_t(wave) * kZvcGroupsPerWave * 64 + lane;
 #pragma unroll
@@ -194,7 +203,8 @@ static int zvc_ensure_counters(vdnn_ctx* ctx) {
 }
 
 static int zvc_offload(vdnn_ctx* ctx, void* dst_host, void* staging_dev, size_t staging_bytes, const void* src_dev, size_t count,
-                       int elem_bytes, unsigned long long* total_host, vdnn_stream_t pack_stream, vdnn_stream_t copy_stream, vdnn_event_t packed) {
+                       int elem_bytes, unsigned long long* total_host, vdnn_stream_t pack_stream, vdnn_stream_t copy_stream, vdnn_event_t packed,
+                       bool keep_on_device) {
     VDNN_REQUIRE(ctx, "null context");
     VDNN_REQUIRE(elem_bytes == 2 || elem_bytes == 4, "elements are two or four bytes");
     if (ctx->plan_only) return VDNN_OK;
@@ -228,14 +238,15 @@ static int zvc_offload(vdnn_ctx* ctx, void* dst_host, void* staging_dev, size_t 
             zvc_pack_kernel<uint16_t><<<grid, kZvcThreads, 0, ps>>>((const uint16_t*)src_dev, count, chunks, (unsigned char*)staging_dev, staging_bytes,
                                                                      (unsigned char*)dst_host, cursor);
         VDNN_HIP(hipGetLastError());
-        zvc_end_kernel<<<1, 1, 0, ps>>>(cursor, staging_bytes, total_host, ctx->zvc_counters);
+        zvc_end_kernel<<<1, 1, 0, ps>>>(cursor, keep_on_device ? ~0ull : (unsigned long long)staging_bytes, (unsigned long long)staging_bytes, total_host,
+                                     ctx->zvc_counters);
         VDNN_HIP(hipGetLastError());
     }
     if (packed) {
         VDNN_HIP(hipEventRecord((hipEvent_t)packed, ps));
         VDNN_HIP(hipStreamWaitEvent(cs, (hipEvent_t)packed, 0));
     }
-    if (staging_bytes) {
+    if (staging_bytes && !keep_on_device) {
         ProfScope prof(ctx, cs, "offload_zvc_copy", 0.0, (double)(count * elem_bytes));
         VDNN_HIP(hipMemcpyAsync(dst_host, staging_dev, staging_bytes, hipMemcpyDeviceToHost, cs));
     }
@@ -254,33 +265,50 @@ size_t vdnn_zvc_buffer_bytes(size_t count, int elem_bytes) {
 }
 
 int vdnn_zvc_offload_async(vdnn_ctx* ctx, void* dst_host, const void* src_dev, size_t count, int elem_bytes, vdnn_stream_t stream) {
-    return zvc_offload(ctx, dst_host, nullptr, 0, src_dev, count, elem_bytes, nullptr, nullptr, stream, nullptr);
+    return zvc_offload(ctx, dst_host, nullptr, 0, src_dev, count, elem_bytes, nullptr, nullptr, stream, nullptr, false);
 }
 
 int vdnn_zvc_offload_staged_async(vdnn_ctx* ctx, void* dst_host, void* staging_dev, size_t staging_bytes, const void* src_dev, size_t count,
                                   int elem_bytes, unsigned long long* total_host, vdnn_stream_t pack_stream, vdnn_stream_t copy_stream,
-                                  vdnn_event_t packed) {
-    return zvc_offload(ctx, dst_host, staging_dev, staging_bytes, src_dev, count, elem_bytes, total_host, pack_stream, copy_stream, packed);
+                                  vdnn_event_t packed, int keep_on_device) {
+    return zvc_offload(ctx, dst_host, staging_dev, staging_bytes, src_dev, count, elem_bytes, total_host, pack_stream, copy_stream, packed,
+                       keep_on_device != 0);
 }
 
-int vdnn_zvc_prefetch_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t count, int elem_bytes, vdnn_stream_t stream) {
+static int zvc_prefetch(vdnn_ctx* ctx, void* dst_dev, const void* staging_dev, size_t staging_bytes, const void* src_host, size_t count,
+                        int elem_bytes, vdnn_stream_t stream) {
     VDNN_REQUIRE(ctx, "null context");
     VDNN_REQUIRE(elem_bytes == 2 || elem_bytes == 4, "elements are two or four bytes");
     if (ctx->plan_only || count == 0) return VDNN_OK;
     VDNN_REQUIRE(dst_dev && src_host, "null pointer");
     VDNN_REQUIRE(((uintptr_t)src_host & 15) == 0 && ((uintptr_t)dst_dev & (elem_bytes - 1)) == 0, "misaligned buffer");
+    VDNN_REQUIRE(staging_bytes == 0 || (staging_dev && ((uintptr_t)staging_dev & 15) == 0 && staging_bytes % 16 == 0),
+                 "staging buffer: 16-byte aligned, a multiple of 16 bytes");
     hipStream_t s = stream ? (hipStream_t)stream : ctx->h2d;
     const size_t chunks = (count + kZvcChunk - 1) / kZvcChunk;
-    // enough records in flight to keep the link busy across their round trips, on an eighth of the compute units
-    const size_t need = (chunks + kZvcTeams - 1) / kZvcTeams, cap = size_t(ctx->num_cu) / 8;
+    // from host memory: enough records in flight to keep the link busy across their round trips, on an eighth of
+    // the compute units; from a block on the device: the whole device, briefly
+    const size_t need = (chunks + kZvcTeams - 1) / kZvcTeams;
+    const size_t cap = staging_bytes ? size_t(ctx->num_cu) * 2 : size_t(ctx->num_cu) / 8;
     const int grid = int(need < cap ? need : cap);
-    ProfScope prof(ctx, s, "prefetch_zvc", 0.0, (double)(count * elem_bytes));
+    ProfScope prof(ctx, s, staging_bytes ? "prefetch_zvc_device" : "prefetch_zvc", 0.0, (double)(count * elem_bytes));
     if (elem_bytes == 4)
-        zvc_unpack_kernel<uint32_t><<<grid, kZvcThreads, 0, s>>>((const unsigned char*)src_host, (uint32_t*)dst_dev, count, chunks);
+        zvc_unpack_kernel<uint32_t><<<grid, kZvcThreads, 0, s>>>((const unsigned char*)staging_dev, staging_bytes, (const unsigned char*)src_host,
+                                                                  (uint32_t*)dst_dev, count, chunks);
     else
-        zvc_unpack_kernel<uint16_t><<<grid, kZvcThreads, 0, s>>>((const unsigned char*)src_host, (uint16_t*)dst_dev, count, chunks);
+        zvc_unpack_kernel<uint16_t><<<grid, kZvcThreads, 0, s>>>((const unsigned char*)staging_dev, staging_bytes, (const unsigned char*)src_host,
+                                                                  (uint16_t*)dst_dev, count, chunks);
     VDNN_HIP(hipGetLastError());
     return VDNN_OK;
+}
+
+int vdnn_zvc_prefetch_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, size_t count, int elem_bytes, vdnn_stream_t stream) {
+    return zvc_prefetch(ctx, dst_dev, nullptr, 0, src_host, count, elem_bytes, stream);
+}
+
+int vdnn_zvc_prefetch_staged_async(vdnn_ctx* ctx, void* dst_dev, const void* staging_dev, size_t staging_bytes, const void* src_host,
+                                   size_t count, int elem_bytes, vdnn_stream_t stream) {
+    return zvc_prefetch(ctx, dst_dev, staging_dev, staging_bytes, src_host, count, elem_bytes, stream);
 }
 
 int vdnn_zvc_traffic(vdnn_ctx* ctx, unsigned long long* tensor_bytes, unsigned long long* link_bytes) {

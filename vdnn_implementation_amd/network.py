@@ -16,7 +16,8 @@ class Options(C.Structure):
     _fields_ = [("seed", C.c_uint64), ("pool_bytes", _sz), ("cap_bytes", _sz), ("plan_only", _i), ("host_sync", _i),
                 ("capture", _i), ("verbose", _i), ("device", _i), ("refined_lifetimes", _i),
                 ("unfused_optimizer", _i), ("defer_optimizer", _i), ("offload_lag", _i), ("prefetch_depth", _i), ("data_type", _i),
-                ("fuse_activations", _i), ("keep_tail_bytes", _sz), ("prefetch_within_peak", _i),
+                ("fuse_activations", _i), ("keep_tail_bytes", _sz), ("prefetch_within_peak", _i), ("keep_packed_on_device", _i),
+                ("plan_packed_fraction", C.c_double),
                 ("compress_offload", _i)]
 
 
@@ -94,7 +95,8 @@ class Network:
     def __init__(self, cnn=None, policy=enums.BASELINE, algo=enums.VDNN_MEMORY_OPT_ALGO, batch=0, layers=None, seed=1,
                  pool_bytes=0, cap_bytes=0, plan_only=False, host_sync=False, capture=False, verbose=False, device=0,
                  refined=False, unfused_optimizer=False, defer_optimizer=False, bf16=False, offload_lag=0, prefetch_depth=1,
-                 fuse=False, compress=False, keep_tail_bytes=0, prefetch_within_peak=False):
+                 fuse=False, compress=False, keep_tail_bytes=0, prefetch_within_peak=False, keep_packed=False,
+                 plan_packed_fraction=0.0):
         o = Options()
         lib.vdnn_network_default_options(C.byref(o))
         o.seed, o.pool_bytes, o.cap_bytes = seed, int(pool_bytes), int(cap_bytes)
@@ -107,6 +109,8 @@ class Network:
         o.compress_offload = int(compress)
         o.keep_tail_bytes = int(keep_tail_bytes)
         o.prefetch_within_peak = int(prefetch_within_peak)
+        o.keep_packed_on_device = int(keep_packed)
+        o.plan_packed_fraction = float(plan_packed_fraction)
         if layers is not None:
             arr = (LayerSpec * len(layers))(*layers)
             self._h = lib.vdnn_network_create_custom(arr, len(layers), policy, algo, C.byref(o))
