@@ -506,10 +506,3 @@ def test_packed_tensors_kept_on_the_device_plan():
         # at 0.57 of a tensor the step holds less than a third of BASELINE's 18.65 GB; at the longest stream it does not
         assert sk["peak_bytes_in_use"] < 18.65e9 / 3 < sw["peak_bytes_in_use"]
         assert live_blocks(kept) == live_blocks(moved) == live_blocks(kept_worst)
-    # a forward without a backward leaves packed blocks behind; the next forward returns them
-    with plan(VGG16_128, VDNN_CONV, batch=16, keep_packed=True, plan_packed_fraction=0.6, compress=True) as net:
-        assert net.forwardPropagation() == 0
-        held = live_blocks(net)
-        assert net.forwardPropagation() == 0
-        assert live_blocks(net) == held
-        assert net.backwardPropagation() == 0
