@@ -126,9 +126,11 @@ int vdnn_memcpy_h2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_host, si
  * back with every bit it had. The reference copies every tensor whole; a rectified tensor is about half zeros.
  * The host buffer must come from vdnn_host_alloc_pinned and hold vdnn_zvc_buffer_bytes(count, elem_bytes).
  * It receives a packed stream: a table of one 32-bit word per chunk of 4096 elements (padded to 16 bytes), the
- * offset of the chunk's record in units of 16 bytes; a record is a 512-byte map (bit l of 64-bit word g: element
- * 64 g + l is kept) followed by the kept elements in order, zero filled to 16 bytes. Records lie without gaps in
- * no particular order, so the stream is as long as its content.
+ * offset of the chunk's record in units of 16 bytes; a record is a 512-byte map followed by the kept elements in
+ * the order of the map's bits, zero filled to 16 bytes. With V = 16 / elem_bytes, bit l of the 64-bit word
+ * b V + j of the map says whether element 64 V b + V l + j of the chunk is kept (a lane holds V consecutive
+ * elements, 64 lanes a block of 64 V). Records lie without gaps in no particular order, so the stream is as long
+ * as its content.
  *   vdnn_zvc_offload_async: a kernel on `stream` packs the tensor straight into the host buffer.
  *   vdnn_zvc_offload_staged_async: the kernel packs into `staging_dev` (device memory, 16-byte aligned,
  *     staging_bytes a multiple of 16) at HBM speed and the copy engine moves staging_bytes to the host buffer;

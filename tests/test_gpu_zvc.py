@@ -6,7 +6,7 @@ size (whole chunks, ragged tails, one element), both element widths and every bi
 denormals are kept; only all-zero bits are dropped), whether the stream goes to host memory through a staging
 buffer of any size or straight from the kernel. The host bytes are also decoded here in numpy from the documented
 format, which pins the format itself: a table of record offsets, then per chunk of 4096 elements a 512-byte map
-followed by the kept elements in order.
+followed by the kept elements in the order of the map's bits.
 """
 import ctypes as C
 
@@ -51,15 +51,19 @@ def decode(host, count, dtype):
     spans = []
     for c in range(chunks):
         at = int(table[c]) * 16
-        bits = np.unpackbits(host[at:at + MAP], bitorder="little").astype(bool)   # bit l of word g = element 64 g + l
+        bits = np.unpackbits(host[at:at + MAP], bitorder="little").astype(bool)   # bit l of word g, g = 0 .. 63
         kept = int(bits.sum())
         values = host[at + MAP:at + MAP + kept * es].view(dtype)
         padded = (kept * es + 15) // 16 * 16
         assert not host[at + MAP + kept * es:at + MAP + padded].any(), "zero fill behind the kept elements"
+        # a lane holds V consecutive elements: bit l of word b V + j is element 64 V b + V l + j of the chunk
+        v = 16 // es
+        g, l = np.divmod(np.arange(CHUNK), 64)
+        element = 64 * v * (g // v) + v * l + g % v
         piece = np.zeros(CHUNK, dtype)
-        piece[bits] = values
+        piece[element[bits]] = values
         n = min(CHUNK, count - c * CHUNK)
-        assert not bits[n:].any(), "elements past the end of the tensor are never kept"
+        assert not piece[n:].any(), "elements past the end of the tensor are never kept"
         out[c * CHUNK:c * CHUNK + n] = piece[:n]
         spans.append((at, at + MAP + padded))
     spans.sort()
@@ -266,3 +270,35 @@ def test_losses_at_a_batch_that_keeps_the_streams_busy(bf16):
                        (VDNN_CONV, {"keep_packed": True, "keep_tail_bytes": 40 << 20})):
         announce("compressed offload at batch 32, policy", policy, kw, "bf16", bf16)
         assert losses(policy, fuse=True, compress=True, **kw) == want, "policy %d %s" % (policy, kw)
+
+
+@pytest.mark.parametrize("dtype", [np.uint32, np.uint16])
+def test_tensors_off_a_sixteen_byte_boundary(ctx, dtype):
+    """The kernels read and write 128 bits per lane where the tensor allows it; one that starts an element off a
+    16-byte boundary goes element by element and gives the same stream."""
+    es = np.dtype(dtype).itemsize
+    count = 3 * CHUNK + 1234
+    rng = np.random.default_rng(99 + es)
+    a = tensor(rng, count, dtype, 0.5)
+    padded = np.concatenate([np.zeros(1, dtype), a])
+    src = ctx.to_device(padded, dtype)
+    dst = ctx.alloc((count + 1) * es + 64)
+    dst.upload(np.full((count + 1) * es + 64, 0xEE, np.uint8))
+    need = lib.vdnn_zvc_buffer_bytes(count, es)
+    host, same = Pinned(ctx, need), Pinned(ctx, need)
+    aligned = ctx.to_device(a, dtype)
+    announce(f"zvc off a 16-byte boundary, bytes={es}")
+    check(lib.vdnn_zvc_offload_async(ctx.handle, host.ptr, src.ptr + es, count, es, None))
+    check(lib.vdnn_zvc_offload_async(ctx.handle, same.ptr, aligned.ptr, count, es, None))
+    ctx.synchronize()
+    got, length = decode(host.view, count, dtype)
+    want, length2 = decode(same.view, count, dtype)
+    assert np.array_equal(got, a) and np.array_equal(want, a) and length == length2
+    check(lib.vdnn_zvc_prefetch_async(ctx.handle, dst.ptr + es, host.ptr, count, es, None))
+    ctx.synchronize()
+    back = dst.download(((count + 1) * es + 64,), np.uint8)
+    assert (back[:es] == 0xEE).all() and (back[(count + 1) * es:] == 0xEE).all()
+    assert np.array_equal(back[es:(count + 1) * es].view(dtype), a)
+    for b in (src, dst, aligned):
+        b.free()
+    host.free(); same.free()
