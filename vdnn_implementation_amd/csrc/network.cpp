@@ -462,6 +462,8 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         if (!layer[l]->GateGrad() || !isOffload[l]) continue;
         const Layer_t t = layer[l]->LayerType();
         if (!is_conv(t) && t != FC_GEMM) continue; /* a pooling layer reads its input anyway */
+        /* a packed input that stays on the device is expanded by the layer itself before its first kernel */
+        if (options.keepPackedOnDevice && layer[l]->SrcPacked()) continue;
         layer[l]->setGateGrad(false);
         layer[l - 1]->setElidedBackward(false);
     }
