@@ -264,6 +264,8 @@ def main():
         "losses_bit_identical": len({results[k]["loss"] for k in results if not is_bf16(k)}) <= 1
         and len({results[k]["loss"] for k in results if is_bf16(k)}) <= 1,
         "best_offloading_vs_fp32_baseline": best_offloading(results, base),
+        # the same among the fp32 runs only: speed and memory against BASELINE with the reference's element type
+        "best_fp32_offloading_vs_baseline": best_offloading({k: v for k, v in results.items() if not (args.bf16 or is_bf16(k))}, base),
         "conv_mfma_util": conv_all_tf / peak,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                      "frac": achieved / peak,
