@@ -59,8 +59,18 @@ inline int ASSERT_EQ(int result, bool isDynamicMode = false) {
 
 /* The two handle types of the reference's constructors (cudnnHandle_t*, cublasHandle_t*) survive as
  * two distinct thin types over the same back-end context. */
-struct vdnnConvHandle_t { vdnn_ctx* ctx; };
-struct vdnnGemmHandle_t { vdnn_ctx* ctx; };
+/* Settings every layer made through a handle takes over at construction (addition): the seed of the synthetic
+ * initialisation (the reference draws from std::random_device), the per-layer shape dump on stdout of the
+ * reference's constructors (layer.cu:96-101, 474-484), and whether parameter values are drawn and uploaded at
+ * all (a plan-only network allocates the blocks and leaves them as they are). They travel with the handle, so
+ * two networks in one process never see each other's. */
+struct vdnnLayerSettings {
+    uint64_t initSeed = 0;
+    bool     verbose = false;
+    bool     skipParameterValues = false;
+};
+struct vdnnConvHandle_t { vdnn_ctx* ctx; vdnnLayerSettings settings; };
+struct vdnnGemmHandle_t { vdnn_ctx* ctx; vdnnLayerSettings settings; };
 
 class Layer {
 public:
@@ -90,13 +100,7 @@ public:
     Layer(const Layer&) = delete;
     Layer& operator=(const Layer&) = delete;
 
-    // Seed of the synthetic initialisation (the reference draws from std::random_device).
-    static void     setInitSeed(uint64_t seed) { initSeed = seed; }
-    static uint64_t getInitSeed() { return initSeed; }
-    // Per-layer shape dump on stdout like the reference's constructors (layer.cu:96-101, 474-484)
-    static void     setVerbose(bool v) { verbose = v; }
-    // Plan-only networks allocate the parameter blocks but skip drawing and uploading their values
-    static void     setSkipParameterValues(bool v) { skipParameterValues = v; }
+    uint64_t        InitSeed() const { return settings.initSeed; }
     /* addition: keep dW / db in buffers of their own instead of fusing the SGD step into backward
      * (layer.cu:651-660, 736-761 fuse it); applyGradients then performs the step */
     void            keepGradients();
@@ -252,13 +256,11 @@ public:
     void    printFilterData();
 
 private:
-    void    construct(vdnn_ctx* _ctx);
+    void    construct(vdnn_ctx* _ctx, const vdnnLayerSettings& _settings);
     int     mallocWorkSpace(void* shared, size_t bytes, void** cur, bool isDynamic);
     void    freeWorkSpace(void* shared, size_t bytes, void* cur, bool isDynamic);
 
-    static uint64_t initSeed;
-    static bool     verbose;
-    static bool     skipParameterValues;
+    vdnnLayerSettings settings; // copied from the handle the layer was made through
 
     /* General layer info */
     vdnn_t         vdnnMode;

@@ -1,0 +1,174 @@
+"""GPU runs of the configurations that only exist at size, each through the Network C ABI:
+
+ 1. VGG16 batch 512 with bfloat16 activations, VDNN_ALL, under a 48 GB limit on pool bytes in use: two steps give
+    the losses and the post-step filters of the bfloat16 BASELINE bit for bit, move the bytes of the offload table
+    and hold what the replay of the schedule says; the float network under the same limit runs out of memory and
+    says so with -1;
+ 2. VDNN_DYNAMIC_ALGO on the device (network.cu:59-78, 946-1008; layer.cu:1091-1147): under three limits the ladder
+    of trial steps lands on the rung the replay predicts, and the network it leaves behind trains like the same
+    (policy, algorithm) built directly;
+ 3. VGG16 batch 256 (vdnn.h:59, network.cu:146-147), where the reference's int byte counts overflow
+    (network.cu:1010-1040, layer.h:240): VDNN_ALL against BASELINE;
+ 4. the command-line front end on the device.
+
+At these sizes no CPU result is affordable: what is compared is the policy against BASELINE (whose kernels the
+small-size tests check against the CPU checker), as bits.
+"""
+import hashlib
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from gpu_util import announce
+from vdnn_implementation_amd import (ALEXNET, BASELINE, VDNN_ALL, VDNN_CONV, VDNN_DYNAMIC_ALGO, VDNN_MEMORY_OPT_ALGO,
+                                     VDNN_NONE, VDNN_PERF_OPT_ALGO, VGG16_64, VGG16_256, enums)
+from vdnn_implementation_amd.network import Network
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GB = 1e9
+VGG16_TABLE_BYTES_AT_128 = 14741667840  # sum of SrcDataSize over layers 0..35, 4-byte elements, batch 128
+
+
+def params_digest(net):
+    """One SHA-1 per layer with parameters, over the filter's and the bias's bytes."""
+    out = []
+    for l in range(net.num_layers):
+        if net.has_params(l):
+            w, b = net.get_params(l)
+            out.append(hashlib.sha1(w.tobytes() + b.tobytes()).hexdigest())
+    return out
+
+
+def train(net, steps, dynamic=False):
+    losses = []
+    for _ in range(steps):
+        assert net.forwardPropagation(dynamic) == 0
+        losses.append(np.float32(net.loss()).tobytes())
+        assert net.backwardPropagation(dynamic) == 0
+    return losses
+
+
+def test_vgg16_batch_512_bfloat16_vdnn_all_under_a_48_gb_limit():
+    cap = int(48 * GB)
+    kw = dict(seed=11, bf16=True, cap_bytes=cap)
+    announce("VGG16_512 bf16 BASELINE under 48 GB")
+    with Network(enums.VGG16_512, BASELINE, VDNN_MEMORY_OPT_ALGO, 0, **kw) as net:
+        assert net.batch == 512
+        x0 = net.get_input()
+        want_losses = train(net, 2, dynamic=True)
+        want_digest = params_digest(net)
+        base_peak = net.stats()["peak_bytes_in_use"]
+    assert abs(base_peak / GB - 36.7) < 0.3  # fits under the limit with two-byte activations
+    assert np.isfinite(np.frombuffer(want_losses[0], np.float32)[0])
+    with Network(enums.VGG16_512, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 0, plan_only=True, **kw) as replay:
+        assert replay.forwardPropagation(True) == 0 and replay.backwardPropagation(True) == 0
+        plan_peak = replay.stats()["peak_bytes_in_use"]
+    assert abs(plan_peak / GB - 17.06) < 0.1
+    announce("VGG16_512 bf16 VDNN_ALL under 48 GB")
+    with Network(enums.VGG16_512, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 0, **kw) as net:
+        got_losses = train(net, 2, dynamic=True)
+        st = net.stats()
+        # the saturated loss of the second step says little: the filters after two updates say everything
+        assert got_losses == want_losses
+        assert params_digest(net) == want_digest
+        assert st["offload_bytes"] == st["prefetch_bytes"] == VGG16_TABLE_BYTES_AT_128 * 4 // 2 == st["pinned_bytes"]
+        assert st["peak_bytes_in_use"] <= plan_peak < base_peak / 2
+        assert np.array_equal(net.get_input().view(np.uint32), x0.view(np.uint32)), "input block after offload and prefetch"
+    # float activations need 72.7 GB the BASELINE way. BASELINE takes its blocks while it is built (layer.cu:94, 472,
+    # network.cu:897-904), where a failed request is fatal in the reference and here; the policy that asks layer by
+    # layer holds the same tensors and reports the failure: -1 from forwardPropagation in dynamic mode
+    announce("VGG16_512 float VDNN_NONE under 48 GB: out of memory")
+    with Network(enums.VGG16_512, VDNN_NONE, VDNN_MEMORY_OPT_ALGO, 0, seed=11, cap_bytes=cap) as net:
+        assert net.forwardPropagation(True) == -1
+        assert net.stats()["peak_bytes_in_use"] <= cap
+    # the failed step left nothing behind that the next network trips over
+    announce("VGG16_64 after the failed step")
+    with Network(VGG16_64, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 0, seed=11) as net:
+        train(net, 1)
+
+
+def _plan_peak(policy, algo):
+    with Network(VGG16_64, policy, algo, 0, plan_only=True) as net:
+        assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
+        return net.stats()["peak_bytes_in_use"]
+
+
+def test_dynamic_algo_ladder_on_the_device():
+    need_conv = _plan_peak(VDNN_CONV, VDNN_PERF_OPT_ALGO)
+    need_all = _plan_peak(VDNN_ALL, VDNN_MEMORY_OPT_ALGO)
+    cases = ((0, VDNN_NONE), (int(need_conv * 1.02), VDNN_CONV), (int(need_all * 1.02), VDNN_ALL))
+    for cap, want_policy in cases:
+        announce("VDNN_DYNAMIC_ALGO VGG16_64 cap", cap, "expects policy", want_policy)
+        with Network(VGG16_64, BASELINE, VDNN_DYNAMIC_ALGO, 0, seed=5, cap_bytes=cap) as net:
+            assert net.batch == 64 and net.policy == want_policy
+            if want_policy != VDNN_ALL:
+                assert net.algo == VDNN_PERF_OPT_ALGO
+            got_algo = net.algo
+            got = train(net, 2, dynamic=True)
+            got_digest = params_digest(net)
+            st = net.stats()
+            if cap:
+                assert st["peak_bytes_in_use"] <= cap
+        if want_policy != VDNN_ALL:
+            # the rung's configuration built directly: the trial steps left no trace (filters re-drawn by reset())
+            announce("the same configuration built directly", want_policy, got_algo)
+            with Network(VGG16_64, want_policy, got_algo, 0, seed=5) as net:
+                assert train(net, 2) == got
+                assert params_digest(net) == got_digest
+        else:
+            # the last rung chooses the variant layer by layer from what the pool can hold; the variants agree bit
+            # for bit in forward and backward data, a wider split of the filter gradient only in the last places
+            announce("VDNN_ALL built directly")
+            with Network(VGG16_64, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 0, seed=5) as net:
+                want = train(net, 2)
+            assert got[0] == want[0]
+            a, b = np.frombuffer(got[1], np.float32)[0], np.frombuffer(want[1], np.float32)[0]
+            assert abs(a - b) <= 1e-5 * abs(b)
+
+
+def test_vgg16_batch_256_vdnn_all_against_baseline():
+    announce("VGG16_256 BASELINE")
+    with Network(VGG16_256, BASELINE, VDNN_MEMORY_OPT_ALGO, 0, seed=11) as net:
+        assert net.batch == 256
+        assert net.findMaxDxDySize() == 256 * 64 * 224 * 224 * 4 > 2 ** 31
+        x0 = net.get_input()
+        want = train(net, 1)
+        assert net.forwardPropagation() == 0
+        want.append(np.float32(net.loss()).tobytes())
+        want_digest = params_digest(net)
+        base_peak = net.stats()["peak_bytes_in_use"]
+    announce("VGG16_256 VDNN_ALL")
+    with Network(VGG16_256, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 0, seed=11) as net:
+        got = train(net, 1)
+        st = net.stats()
+        assert st["offload_bytes"] == st["prefetch_bytes"] == 2 * VGG16_TABLE_BYTES_AT_128 == st["pinned_bytes"]
+        assert net.prefetch_trace() == [(l, l - 1) for l in range(36, 0, -1)]
+        assert np.array_equal(net.get_input().view(np.uint32), x0.view(np.uint32))
+        assert net.forwardPropagation() == 0
+        got.append(np.float32(net.loss()).tobytes())
+        assert got == want
+        assert params_digest(net) == want_digest
+        assert st["peak_bytes_in_use"] < base_peak / 2
+
+
+def test_command_line_front_end_on_the_device():
+    exe = os.path.join(ROOT, "vdnn_implementation_amd", "bin", "vdnn")
+    announce("bin/vdnn ALEXNET VDNN_ALL VDNN_MEMORY_OPT_ALGO --batch 8 --seed 5")
+    out = subprocess.run([exe, "ALEXNET", "VDNN_ALL", "VDNN_MEMORY_OPT_ALGO", "--batch", "8", "--seed", "5"],
+                         capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert "CNN Model Type: ALEXNET" in out.stdout and "VDNN Mode: VDNN_ALL" in out.stdout
+    line = json.loads([l for l in out.stdout.splitlines() if l.startswith("{")][-1])
+    with Network(ALEXNET, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 8, seed=5) as net:
+        assert net.forwardPropagation() == 0
+        loss = net.loss()
+        assert net.backwardPropagation() == 0
+        st = net.stats()
+    assert line["batch"] == 8 and line["steps"] == 1 and line["plan_only"] is False
+    assert abs(line["loss"] - loss) <= 1e-6 * max(1.0, abs(loss))  # printed with six decimals
+    assert line["offload_bytes"] == st["offload_bytes"] == line["prefetch_bytes"] > 0
+    assert line["peak_bytes"] == st["peak_bytes_in_use"]

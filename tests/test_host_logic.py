@@ -61,6 +61,44 @@ def test_command_line_words():
     assert bad.returncode != 0 and "VDNN type must be one of" in bad.stderr
 
 
+def test_reference_shaped_main_compiles_against_the_public_headers():
+    """The class headers a caller of the reference includes (network.h, layer.h, vdnn.h) live under include/:
+    a main of the shape of vdnn.cu:56-83 builds with the host compiler and -Iinclude alone, links against the
+    library, and its VDNN_ALL schedule (replayed without a device) moves the bytes of the offload table."""
+    import shutil
+    import tempfile
+    pkg = os.path.join(ROOT, "vdnn_implementation_amd")
+    tmp = tempfile.mkdtemp(prefix="vdnn_main_")
+    try:
+        exe = os.path.join(tmp, "ref_main")
+        cmd = ["g++", "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "include"), os.path.join(ROOT, "tests", "cpp", "reference_shaped_main.cpp"),
+               "-o", exe, "-L" + pkg, "-lvdnn_amd", "-Wl,-rpath," + pkg, "-Wl,-rpath-link,/opt/rocm/lib"]
+        built = subprocess.run(cmd, capture_output=True, text=True)
+        assert built.returncode == 0, built.stderr
+        out = subprocess.run([exe, "VGG16_64", "VDNN_ALL", "VDNN_MEMORY_OPT_ALGO", "--plan"], capture_output=True, text=True)
+        assert out.returncode == 0, out.stderr
+        want = 14741667840 // 2  # the VGG16 batch 128 table at batch 64
+        assert "status 0 0 layers 37 batch 64 input %d output 64000 offloaded %d prefetched %d dxdy %d" % (
+            64 * 3 * 224 * 224, want, want, 64 * 64 * 224 * 224 * 4) in out.stdout, out.stdout
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
+def test_default_options_set_every_field():
+    """A C caller declares the options on its stack: whatever the memory held, vdnn_network_default_options
+    leaves every field (and the padding) at its default."""
+    from vdnn_implementation_amd.network import Options
+    o = Options()
+    C.memset(C.byref(o), 0xFF, C.sizeof(o))
+    lib.vdnn_network_default_options(C.byref(o))
+    want = {"seed": 1, "prefetch_depth": 1, "plan_packed_fraction": 0.0}
+    for name, _ in Options._fields_:
+        assert getattr(o, name) == want.get(name, 0), name
+    z = Options()
+    lib.vdnn_network_default_options(C.byref(z))
+    assert bytes(o) == bytes(z), "padding bytes differ"
+
+
 # ---- pool allocator ---------------------------------------------------------------------------------
 def test_pool_best_fit_coalescing_peak_and_cap():
     ctx = be.Context(plan_only=True, pool_bytes=256 << 20)
@@ -354,6 +392,35 @@ def test_dynamic_algo_ladder():
         assert (net.policy, net.algo) == (VDNN_CONV, VDNN_PERF_OPT_ALGO)
     with plan(VGG16_64, BASELINE, VDNN_DYNAMIC_ALGO, cap_bytes=int(need_all * 1.02)) as net:
         assert net.policy == VDNN_ALL
+
+
+def test_dynamic_ladder_rebuilds_cleanly_after_trials_that_fail_half_way():
+    """A trial step of the ladder that runs out of memory in the middle of forward leaves blocks, packed streams
+    kept on the device and pending offloads behind; reset() forgets them with the pool they came from, so the
+    configuration the ladder settles on steps without touching a block of the destroyed pool, and nothing leaks.
+    A replay network built inside the constructor (prefetch_within_peak) does not change the outer one."""
+    kw = dict(refined=True, fuse=True, compress=True, keep_packed=True, prefetch_within_peak=True, plan_packed_fraction=0.6)
+    with plan(VGG16_64, VDNN_ALL, VDNN_PERF_OPT_ALGO, **kw) as net:
+        step(net)
+        need_all = net.stats()["peak_bytes_in_use"]
+    with plan(VGG16_64, VDNN_NONE, VDNN_PERF_OPT_ALGO, **kw) as net:
+        step(net)
+        need_none = net.stats()["peak_bytes_in_use"]
+    assert need_all < need_none
+    for cap, want in ((int(need_none * 1.02), VDNN_NONE), (int(need_all * 1.02), VDNN_ALL)):
+        with plan(VGG16_64, BASELINE, VDNN_DYNAMIC_ALGO, cap_bytes=cap, **kw) as net:
+            assert net.policy == want
+            n0 = live_blocks(net)
+            for _ in range(2):
+                assert net.forwardPropagation(True) == 0 and net.backwardPropagation(True) == 0
+            assert live_blocks(net) == n0
+            assert net.stats()["peak_bytes_in_use"] <= cap
+    # the same with a forward that stops half-way outside the ladder: the next network in the process is unaffected
+    with plan(VGG16_64, VDNN_NONE, cap_bytes=int(need_all), **kw) as net:
+        assert net.forwardPropagation(True) == -1
+    with plan(VGG16_64, VDNN_ALL, VDNN_PERF_OPT_ALGO, **kw) as net:
+        step(net)
+        assert net.stats()["peak_bytes_in_use"] == need_all
 
 
 def test_custom_table_shape_inference_and_sanity():

@@ -33,9 +33,21 @@ extern "C" {
 
 void vdnn_network_default_options(vdnn_network_options* o) {
     if (!o) return;
-    NetworkOptions d;
-    o->seed = d.seed; o->pool_bytes = 0; o->cap_bytes = 0; o->plan_only = 0; o->host_sync = 0;
-    o->capture = 0; o->verbose = 0; o->device = d.device; o->refined_lifetimes = 0; o->unfused_optimizer = 0; o->defer_optimizer = 0; o->data_type = VDNN_DTYPE_F32; o->offload_lag = 0; o->prefetch_depth = 1; o->fuse_activations = 0;
+    memset(o, 0, sizeof *o); /* padding and every field a later version adds start at zero */
+    const NetworkOptions d;
+    o->seed = d.seed; o->pool_bytes = d.poolBytes; o->cap_bytes = d.capBytes;
+    o->plan_only = d.planOnly; o->host_sync = d.hostSync; o->capture = d.capture; o->verbose = d.verbose;
+    o->device = d.device;
+    o->refined_lifetimes = d.refinedLifetimes;
+    o->unfused_optimizer = d.unfusedOptimizer; o->defer_optimizer = d.deferOptimizer;
+    o->offload_lag = d.offloadLag; o->prefetch_depth = d.prefetchDepth;
+    o->data_type = d.dataType;
+    o->fuse_activations = d.fuseActivations;
+    o->keep_tail_bytes = d.keepTailBytes;
+    o->prefetch_within_peak = d.prefetchWithinPeak;
+    o->keep_packed_on_device = d.keepPackedOnDevice;
+    o->plan_packed_fraction = d.planPackedFraction;
+    o->compress_offload = d.compressOffload;
 }
 
 vdnn_network* vdnn_network_create(int cnn, int policy, int algo, int batch, const vdnn_network_options* o) {

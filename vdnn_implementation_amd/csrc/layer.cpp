@@ -9,10 +9,6 @@
 
 #include "seeded_init.h"
 
-uint64_t Layer::initSeed = 0;
-bool Layer::verbose = false;
-bool Layer::skipParameterValues = false;
-
 static const char* type_name(Layer_t t) {
     switch (t) {
     case FC_GEMM: return "FC_GEMM";
@@ -39,7 +35,7 @@ Layer::Layer(vdnn_t _vdnnMode, vdnnAlgoMode_t _vdnnAlgoMode, Layer_t _layerType,
     M_ASSERT(_layerType == FC_GEMM, "Layer type is not FC_GEMM!");
     M_ASSERT(h_in == 1 && w_in == 1 && r == 1 && s == 1, "Invalid dimensions!");
     M_ASSERT(_gemmHandle && _gemmHandle->ctx, "null GEMM handle");
-    construct(_gemmHandle->ctx);
+    construct(_gemmHandle->ctx, _gemmHandle->settings);
 }
 
 /* Constructor of every other layer kind (layer.cu:104-485) */
@@ -52,11 +48,12 @@ Layer::Layer(vdnn_t _vdnnMode, vdnnAlgoMode_t _vdnnAlgoMode, Layer_t _layerType,
       convHandle(_convHandle), gemmHandle(nullptr) {
     M_ASSERT(_layerType != FC_GEMM, "FC_GEMM type layer cannot be initialized with the convolution handle!");
     M_ASSERT(_convHandle && _convHandle->ctx, "null convolution handle");
-    construct(_convHandle->ctx);
+    construct(_convHandle->ctx, _convHandle->settings);
 }
 
-void Layer::construct(vdnn_ctx* _ctx) {
+void Layer::construct(vdnn_ctx* _ctx, const vdnnLayerSettings& _settings) {
     ctx = _ctx;
+    settings = _settings;
     /* Basic settings (layer.cu:58-77, 122-142) */
     insideInceptionModule = headOfFork = tailOfFork = inPlaceOp = false;
     fuseRelu = elided = elidedBackward = gateGrad = false;
@@ -106,7 +103,7 @@ void Layer::construct(vdnn_ctx* _ctx) {
     /* Allocate GPU memory for dstData (layer.cu:94, 472) */
     if (vdnnMode == BASELINE) cnmemMallocDstData(false);
 
-    if (verbose) {
+    if (settings.verbose) {
         printf("----------------------- Layer %d -----------------------\n", layerId);
         printf("Layer Type: %s\n", type_name(layerType));
         printf("Input (n, c, h, w): (%d, %d, %d, %d)\n", n_in, c_in, h_in, w_in);
@@ -460,10 +457,10 @@ void Layer::initializeConvolutionFilterAndBias() {
     const size_t biasDataSize = (size_t)k;
     ASSERT_EQ(vdnn_pool_malloc(ctx, &filterData, sizeof(DATATYPE) * filterDataSize));
     ASSERT_EQ(vdnn_pool_malloc(ctx, &biasData, sizeof(DATATYPE) * biasDataSize));
-    if (skipParameterValues) return;
+    if (settings.skipParameterValues) return;
     std::vector<DATATYPE> filterData_h(filterDataSize), biasData_h(biasDataSize, 0.0f);
     const double fan_in = (double)c_in * r * s;
-    vdnn::seeded_fill_normal(filterData_h.data(), filterDataSize, initSeed, 100 + 2 * (uint64_t)layerId, 0.0f, (float)std::sqrt(2.0 / fan_in));
+    vdnn::seeded_fill_normal(filterData_h.data(), filterDataSize, settings.initSeed, 100 + 2 * (uint64_t)layerId, 0.0f, (float)std::sqrt(2.0 / fan_in));
     checkVDNN(vdnn_memcpy_h2d(ctx, filterData, filterData_h.data(), sizeof(DATATYPE) * filterDataSize));
     checkVDNN(vdnn_memcpy_h2d(ctx, biasData, biasData_h.data(), sizeof(DATATYPE) * biasDataSize));
 }

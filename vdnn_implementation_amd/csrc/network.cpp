@@ -144,11 +144,10 @@ void Network::construct(vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) {
     checkVDNN(vdnn_ctx_set_activation_dtype(ctx, options.dataType));
     convHandle.ctx = ctx;
     gemmHandle.ctx = ctx;
+    /* every layer of this network, also those rebuilt by reset(), takes these from its handle */
+    convHandle.settings = gemmHandle.settings = vdnnLayerSettings{options.seed, options.verbose, options.planOnly};
     stream_compute = vdnn_ctx_stream_compute(ctx);
     stream_memory = vdnn_ctx_stream_d2h(ctx);
-    Layer::setInitSeed(options.seed);
-    Layer::setVerbose(options.verbose);
-    Layer::setSkipParameterValues(options.planOnly);
 
     if (_algoMode == VDNN_DYNAMIC_ALGO) {
         /* network.cu:59-78: start from (VDNN_ALL, memory-optimal), then walk the ladder */
@@ -208,6 +207,14 @@ void Network::reset(CNN_t _cnnType, vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) 
     inputData = labelData = networkDiffData = networkGradData = workSpace = nullptr;
     lossData = nullptr;
     inputResident = false;
+    /* so is every block the last step still held: a trial step of the dynamic ladder may have stopped half-way */
+    for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
+        zvcStaging[i] = nullptr;
+        zvcStagingBytes[i] = 0;
+        zvcKept[i] = false;
+        srcReleasedEarly[i] = false;
+    }
+    pendingOffload.clear();
     cnnType = _cnnType;
     algoMode = _algoMode;
     vdnnType = _vdnnType;
