@@ -184,6 +184,20 @@ int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* 
  * bias[k] += alpha * sum_{n,p,q} dy[n,k,p,q]. Fixed summation order. */
 int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape,
                            const void* dy, float* bias, float alpha);
+/* vdnn_conv_bwd_bias_sgd for callers that cannot allocate device memory. No counterpart in the reference. It is for
+ * code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc: it takes no context (making
+ * one reserves a pool and streams), and the partial sums of its two-stage reduction live in an array of
+ * VDNN_NOALLOC_SCRATCH_BYTES that is part of the library's device image (every GPU the library runs on holds one
+ * copy until the process ends) instead of a context's staging area. Same kernels, same split of the batch, same
+ * bits as vdnn_conv_bwd_bias_sgd on the same device. `stream` is a hipStream_t of the current device (NULL: the
+ * null stream); dtype is the element type of dy (VDNN_DTYPE_F32 / VDNN_DTYPE_BF16). A shape whose partial sums
+ * (k x batch slices floats; 4 slices of the batch per compute unit divided by k, at least one) exceed the array is
+ * rejected with VDNN_EINVAL. Calls no hipMalloc, hipFree or allocating library routine. All calls on one GPU
+ * share that GPU's array: two calls that overlap there (different streams, different threads) race; calls on one
+ * stream do not. */
+#define VDNN_NOALLOC_SCRATCH_BYTES (256u << 10)
+int vdnn_conv_bwd_bias_sgd_noalloc(vdnn_stream_t stream, const vdnn_shape_t* shape, int dtype,
+                                   const void* dy, float* bias, float alpha);
 /* cudnnConvolutionBackwardFilter with alpha=-lr, beta=1 (layer.cu:651-660):
  * w[k,c,r,s] += alpha * sum_{n,p,q} dy[n,k,p,q] * x[n,c,p*sh-ph+r,q*sw-pw+s]. Fixed summation
  * order (no floating-point atomics). */

@@ -102,6 +102,7 @@ BACKEND_SYMBOLS = {
     "vdnn_fc_bwd_data_relu": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "vdnn_maxpool_bwd_relu": (_i, [_vp, _vp, _S, _vp, _vp, _vp, _vp]),
     "vdnn_conv_bwd_bias_sgd": (_i, [_vp, _vp, _S, _vp, _vp, _f]),
+    "vdnn_conv_bwd_bias_sgd_noalloc": (_i, [_vp, _S, _i, _vp, _vp, _f]),
     "vdnn_conv_bwd_filter_sgd": (_i, [_vp, _vp, _S, _i, _vp, _vp, _vp, _f, _vp, _sz]),
     "vdnn_fc_fwd": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "vdnn_fc_bwd_data": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp]),

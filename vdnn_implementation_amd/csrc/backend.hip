@@ -60,6 +60,10 @@ int vdnn_ctx_create(vdnn_ctx** out, int device, int flags) {
             delete ctx;
             return VDNN_EDEVICE;
         }
+        if (noalloc_prepare_current_device() != VDNN_OK) {
+            delete ctx;
+            return VDNN_EDEVICE;
+        }
     }
     *out = ctx;
     return VDNN_OK;

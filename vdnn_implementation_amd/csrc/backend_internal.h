@@ -46,6 +46,8 @@ void set_error(const char* fmt, ...);
 inline hipStream_t stream_of(vdnn_ctx* ctx, vdnn_stream_t s) { return s ? (hipStream_t)s : ctx->compute; }
 
 hipEvent_t prof_take_event(vdnn_ctx* ctx);
+// looks up the current device's copy of the scratch array of vdnn_conv_bwd_bias_sgd_noalloc (eltwise.hip)
+int noalloc_prepare_current_device();
 static constexpr size_t kProfMaxRecords = 2048;
 
 // Brackets the launches made during its lifetime with two timing events when profiling is on.

@@ -766,6 +766,28 @@ static int bias_add_t(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw,
     return VDNN_OK;
 }
 
+// The two launches of the convolution bias gradient, shared by the entry points below: stage 1 leaves one partial
+// sum per (channel, batch slice) in `partials`, stage 2 adds a channel's partials in slice order. The split of the
+// batch depends on the shape and the number of compute units only, so every caller computes the same bits.
+static int bias_grad_splits(int N, int K, int num_cu, int* per_out) {
+    int splits = (4 * num_cu + K - 1) / K;
+    if (splits > N) splits = N;
+    if (splits < 1) splits = 1;
+    const int per = (N + splits - 1) / splits;
+    *per_out = per;
+    return (N + per - 1) / per;
+}
+
+template <class E>
+static int bias_grad_launch(hipStream_t st, const E* dy, float* bias, float* partials, int N, int K, int PQ, int splits, int per,
+                            float alpha, int accumulate) {
+    hipLaunchKernelGGL(bias_grad_partial_kernel<E>, dim3(K * splits), dim3(EB), 0, st, dy, partials, N, K, PQ, splits, per);
+    VDNN_LAUNCH_CHECK();
+    hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB - 1) / EB), dim3(EB), 0, st, partials, bias, K, splits, alpha, accumulate);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
 template <class E>
 static int conv_bwd_bias_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* dy, float* bias, float alpha, int accumulate) {
     VDNN_KERNEL_PROLOGUE(ctx);
@@ -775,20 +797,58 @@ static int conv_bwd_bias_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
     const int Q = vdnn_out_dim(shape->w, shape->pad_w, shape->s, shape->stride_w);
     VDNN_REQUIRE(N > 0 && K > 0 && P > 0 && Q > 0, "bad geometry");
     // split the batch so that K*splits workgroups fill the chip; geometry depends on the shape only
-    int splits = (4 * ctx->num_cu + K - 1) / K;
-    if (splits > N) splits = N;
-    if (splits < 1) splits = 1;
-    const int per = (N + splits - 1) / splits;
-    splits = (N + per - 1) / per;
+    int per = 0;
+    const int splits = bias_grad_splits(N, K, ctx->num_cu, &per);
     VDNN_REQUIRE((size_t)K * splits * sizeof(float) <= ctx->reduce_scratch_bytes, "staging area too small");
     hipStream_t st = stream_of(ctx, stream);
     ProfScope prof(ctx, st, "conv_bwd_bias", 0.0, (double)sizeof(E) * (double)N * K * P * Q);
-    hipLaunchKernelGGL(bias_grad_partial_kernel<E>, dim3(K * splits), dim3(EB), 0, st, (const E*)dy, ctx->reduce_scratch, N, K, P * Q, splits, per);
-    VDNN_LAUNCH_CHECK();
-    hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB - 1) / EB), dim3(EB), 0, st, ctx->reduce_scratch, bias, K, splits, alpha, accumulate);
-    VDNN_LAUNCH_CHECK();
+    return bias_grad_launch<E>(st, (const E*)dy, bias, ctx->reduce_scratch, N, K, P * Q, splits, per, alpha, accumulate);
+}
+
+// ---- the convolution bias gradient for callers that cannot allocate ---------------------------------------------
+// Partial sums of vdnn_conv_bwd_bias_sgd_noalloc live in this array instead of a context's staging area. Every
+// device that loads the library holds its own copy at its own address until the process ends. The name below is a
+// host-side handle of the symbol, not a device address: host code only ever uses the address that
+// hipGetSymbolAddress returned for the device at hand.
+static constexpr size_t kNoAllocScratchBytes = VDNN_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) float g_noalloc_scratch[kNoAllocScratchBytes / sizeof(float)];
+
+namespace {
+struct NoAllocDevice { float* scratch = nullptr; int num_cu = 0; bool ready = false; };
+constexpr int kMaxDevices = 64;
+NoAllocDevice g_noalloc_devices[kMaxDevices];
+} // namespace
+
+// Address of the current device's copy of the array and that device's number of compute units, looked up once per
+// device with that device current. Allocates nothing.
+static int noalloc_device(NoAllocDevice** out) {
+    int dev = -1;
+    VDNN_HIP(hipGetDevice(&dev));
+    VDNN_REQUIRE(dev >= 0 && dev < kMaxDevices, "device index out of range");
+    NoAllocDevice& d = g_noalloc_devices[dev];
+    if (!d.ready) {
+        float* ptr = nullptr;
+        VDNN_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(g_noalloc_scratch)));
+        VDNN_REQUIRE(ptr != nullptr, "no address for the scratch array on this device");
+        int cus = 0;
+        VDNN_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        VDNN_REQUIRE(cus > 0, "device reports no compute units");
+        d.scratch = ptr;
+        d.num_cu = cus;
+        d.ready = true;
+    }
+    *out = &d;
     return VDNN_OK;
 }
+
+namespace vdnn {
+// Called by vdnn_ctx_create with the context's device current, so that a later vdnn_conv_bwd_bias_sgd_noalloc on
+// that device finds the address already there (a first call under stream capture then makes no query at all).
+int noalloc_prepare_current_device() {
+    NoAllocDevice* d = nullptr;
+    return noalloc_device(&d);
+}
+} // namespace vdnn
 
 template <class E>
 static int fc_bwd_bias_impl(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_out, const void* dy, float* bias, float alpha, int accumulate) {
@@ -985,6 +1045,29 @@ int vdnn_bias_add(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw, con
 
 int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* dy, float* bias, float alpha) {
     return ACT_CALL(conv_bwd_bias_impl, ctx, stream, shape, dy, bias, alpha, 1);
+}
+int vdnn_conv_bwd_bias_sgd_noalloc(vdnn_stream_t stream, const vdnn_shape_t* shape, int dtype, const void* dy, float* bias, float alpha) {
+    VDNN_REQUIRE(shape && dy && bias, "null argument");
+    VDNN_REQUIRE(dtype == VDNN_DTYPE_F32 || dtype == VDNN_DTYPE_BF16, "unknown element type");
+    const int N = shape->n, K = shape->k;
+    const int P = vdnn_out_dim(shape->h, shape->pad_h, shape->r, shape->stride_h);
+    const int Q = vdnn_out_dim(shape->w, shape->pad_w, shape->s, shape->stride_w);
+    VDNN_REQUIRE(N > 0 && K > 0 && P > 0 && Q > 0, "bad geometry");
+    NoAllocDevice* d = nullptr;
+    const int rc = noalloc_device(&d);
+    if (rc != VDNN_OK) return rc;
+    int per = 0;
+    const int splits = bias_grad_splits(N, K, d->num_cu, &per);
+    if ((size_t)K * splits * sizeof(float) > kNoAllocScratchBytes) {
+        set_error("vdnn_conv_bwd_bias_sgd_noalloc: %d channels x %d batch slices need %zu bytes of partial sums, the built-in scratch "
+                  "array holds %zu; use vdnn_conv_bwd_bias_sgd with a context", K, splits, (size_t)K * splits * sizeof(float),
+                  kNoAllocScratchBytes);
+        return VDNN_EINVAL;
+    }
+    // stage 1 writes every partial that stage 2 reads: nothing of the last call's contents has to be cleared
+    if (dtype == VDNN_DTYPE_BF16)
+        return bias_grad_launch<bf16_t>((hipStream_t)stream, (const bf16_t*)dy, bias, d->scratch, N, K, P * Q, splits, per, alpha, 1);
+    return bias_grad_launch<float>((hipStream_t)stream, (const float*)dy, bias, d->scratch, N, K, P * Q, splits, per, alpha, 1);
 }
 int vdnn_conv_bwd_bias(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* dy, float* db) {
     return ACT_CALL(conv_bwd_bias_impl, ctx, stream, shape, dy, db, 1.0f, 0);
