@@ -1,17 +1,21 @@
 """Headline benchmark: VGG16, fp32, batch 128, one MI355X.
 
-A step is one forwardPropagation + backwardPropagation (SGD fused into the backward kernels) on
-seeded synthetic data. BASELINE, VDNN_NONE, VDNN_CONV and VDNN_ALL run back to back; `value` is the
-VDNN_ALL images/s, the other policies and the ratio to BASELINE ride along in `policies`.
-The roofline entry is the convolution kernel class with the largest share of device time, timed with
-HIP events around every launch on the compute stream during the timed steps. The CPU baseline is the
-C checker under oracle/ (a port of the same layer math) on the host cores, at a reduced batch.
+A step is one forwardPropagation + backwardPropagation (SGD fused into the backward kernels) on seeded synthetic
+data, with the input resident in HBM. The reference's four policies run literally (BASELINE, VDNN_NONE, VDNN_CONV,
+VDNN_ALL), followed by the value-preserving variants; `value` is the literal VDNN_ALL's images/s, every
+configuration rides along in `policies`.
 
-One JSON line on stdout; progress goes to stderr.
+Each configuration: warm-up steps, then the timed steps with nothing else going on (this is what ms_per_step and
+images_per_s come from), then a short pass of the same steps with the library's per-launch HIP events switched on.
+From that pass come the kernel table, the roofline entry (the convolution class with the most device time) and, from
+the launches' start and end times, how much of the copies' time ran beside kernels of the compute stream.
+
+The CPU baseline is the C checker under oracle/ on the host cores. One JSON line on stdout; progress on stderr.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -21,74 +25,104 @@ sys.path.insert(0, ROOT)
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # dense; the bfloat16-storage runs multiply on the bfloat16 matrix cores
 HBM_PEAK_GBS = 8000.0
-FLOP_PER_IMAGE = 92.82e9  # 3 passes over 13 convolutions and 3 FC layers
+HOST_LINK_GBS = 56.6            # what hipMemcpyAsync from / to pinned memory reaches on this machine, each way
+FLOP_PER_IMAGE = 92.82e9        # 3 passes over 13 convolutions and 3 FC layers
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "igemm_conv_vgg16_b128_pmc_traffic.txt")
+PACKED_FRACTION = {False: 0.60, True: 0.63}   # what a plan takes a packed stream to be of its tensor (measured: 0.57 / 0.60)
 
-# Memory traffic per launch (bytes fetched into L2 plus bytes written back, averaged over a class's
-# launches in one step) of the three large convolution classes at the default workload (batch 128,
-# memory-optimal mode). Hardware counters cannot be read from inside this script: the figures come
-# from two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), whose summary is
-# kept under profiles/. FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0: what the same counters
-# read for the ReLU kernels of the same run, which move a known number of bytes.
-MEASURED_TRAFFIC_BYTES = {
-    "conv_fwd_128x128": 984.8e6,
-    "conv_bwd_data_128x128": 940.3e6,
-    "conv_bwd_filter_128x128": 1724.8e6,
-}
+DEFAULT_POLICIES = ",".join([
+    "BASELINE", "VDNN_NONE", "VDNN_CONV", "VDNN_ALL",
+    "BASELINE+fused", "VDNN_ALL+refined",
+    "VDNN_CONV+refined+ahead+fused+zvc", "VDNN_ALL+refined+ahead+fused+zvc",
+    "VDNN_ALL+refined+fused+zvc+keep",
+    "VDNN_ALL+refined+fused+zvc+budget3.0", "VDNN_ALL+refined+fused+zvc+budget3.3", "VDNN_ALL+refined+fused+zvc+budget4.0",
+    "BASELINE+bf16+fused", "VDNN_ALL+refined+ahead+bf16+fused+zvc", "VDNN_ALL+refined+bf16+fused+zvc+keep",
+    "VDNN_ALL+refined+bf16+fused+zvc+budget5.9",
+])
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def run_policy(Network, be, cnn, policy, algo, batch, steps, warmup, seed, refined=False, cap_bytes=0, bf16=False, offload_lag=0, prefetch_depth=1,
-               fuse=False, compress=False, keep_tail_bytes=0, ahead=False, keep_packed=False):
-    net = Network(cnn, policy, algo, batch, seed=seed, refined=refined, cap_bytes=cap_bytes, bf16=bf16,
-                  offload_lag=offload_lag, prefetch_depth=prefetch_depth, fuse=fuse, compress=compress, keep_tail_bytes=keep_tail_bytes, prefetch_within_peak=ahead, keep_packed=keep_packed)
+def measured_traffic():
+    """Bytes per launch (L2 fetch + write-back) of the convolution classes, read from the hardware-counter summary kept
+    under profiles/ (two `rocprofv3 --pmc` runs of this script; the file says how the counters were scaled)."""
+    out = {}
+    try:
+        for line in open(TRAFFIC_PROFILE):
+            m = re.match(r"^(conv_\S+)\s+launches.*traffic/launch.*=\s*([0-9.]+) MB", line)
+            if m:
+                out[m.group(1)] = float(m.group(2)) * 1e6
+    except OSError:
+        pass
+    return out
+
+
+def run_config(Network, be, cnn, policy, algo, batch, steps, warmup, profile_steps, **kw):
+    from vdnn_implementation_amd import trace_overlap
+    net = Network(cnn, policy, algo, batch, seed=1, **kw)
     try:
         for _ in range(warmup):
             assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
         net.synchronize()
         net.reset_peak()
-        be.profile_enable(net.context, True)
+        t_bytes0, l_bytes0 = be.zvc_traffic(net.context)
         net.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
             assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
         net.synchronize()
         dt = time.perf_counter() - t0
-        prof = be.profile_collect(net.context)
-        be.profile_enable(net.context, False)
-        # the library times the first 2048 launches after profile_enable: the share of the run they stand for
-        untimed = prof.pop("untimed", {"launches": 0})["launches"]
-        timed = sum(v["launches"] for v in prof.values())
-        timed_share = timed / max(timed + untimed, 1)
         st = net.stats()
         loss = net.loss()
-        tensor_bytes, link_bytes = be.zvc_traffic(net.context)
+        t_bytes1, l_bytes1 = be.zvc_traffic(net.context)
+        # the same steps again with every launch bracketed by events (at most 2048 launches are timed)
+        be.profile_enable(net.context, True)
+        for _ in range(profile_steps):
+            assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
+        net.synchronize()
+        prof = be.profile_collect(net.context)
+        intervals = be.profile_intervals(net.context)
+        be.profile_enable(net.context, False)
+        plan = None
+        if kw.get("hbm_budget_bytes"):
+            places = net.placement()
+            plan = {"budget_gb": kw["hbm_budget_bytes"] / 1e9, "feasible": net.plan_feasible(), "plan_peak_gb": net.plan_peak_bytes() / 1e9,
+                    "on_device": places.count(1), "packed_on_device": places.count(2), "over_the_link": places.count(3)}
     finally:
         net.close()
+    untimed = prof.pop("untimed", {"launches": 0})["launches"]
     res = {"ms_per_step": dt * 1e3 / steps, "images_per_s": batch * steps / dt, "loss": loss,
            "peak_hbm_gb": st["peak_bytes_in_use"] / 1e9, "offload_gb_per_step": st["offload_bytes"] / 1e9,
-           "prefetch_gb_per_step": st["prefetch_bytes"] / 1e9, "pinned_gb": st["pinned_bytes"] / 1e9,
-           "launches_timed_share": timed_share}
-    # host link: busy time and rate of the copies, and how much of the copy time ran under compute
-    # (the *_zvc entries are the compacting copies: their bytes are the tensors', not what crossed the link)
-    link = ("offload_d2h", "prefetch_h2d", "offload_zvc", "offload_zvc_copy", "prefetch_zvc")   # (not prefetch_zvc_device)
-    copies = [prof[k] for k in link if k in prof]
-    if tensor_bytes:
-        res["zvc_link_bytes_per_tensor_byte"] = link_bytes / tensor_bytes
-    if copies:
-        copy_ms = sum(c["ms"] for c in copies)
-        kernel_ms = sum(v["ms"] for k, v in prof.items() if k not in link)
-        rate = lambda keys: (sum(prof[k]["bytes"] for k in keys if k in prof) /
-                             max(sum(prof[k]["ms"] for k in keys if k in prof), 1e-9) * 1e3 / 1e9)
-        res["d2h_gbs"] = rate(("offload_d2h", "offload_zvc", "offload_zvc_copy"))
-        res["h2d_gbs"] = rate(("prefetch_h2d", "prefetch_zvc"))
-        copy_ms, kernel_ms = copy_ms / timed_share, kernel_ms / timed_share   # scaled to the whole run
-        res["copy_busy_ms_per_step"] = copy_ms / steps
-        res["kernel_busy_ms_per_step"] = kernel_ms / steps
-        # step = kernels + copies - overlap + idle  =>  overlap >= kernels + copies - step
-        res["overlap_fraction_lower_bound"] = max(0.0, min(1.0, (kernel_ms + copy_ms - dt * 1e3) / copy_ms))
+           "prefetch_gb_per_step": st["prefetch_bytes"] / 1e9, "pinned_gb": st["pinned_bytes"] / 1e9}
+    if plan:
+        res["plan"] = plan
+    # bytes that cross the link each way per step: tensors copied whole, plus the packed streams' bytes
+    packed_tensor = (t_bytes1 - t_bytes0) / steps
+    packed_link = (l_bytes1 - l_bytes0) / steps
+    # (packed tensors that stay on the device are counted by neither offload_bytes nor the link counter, bar what did not fit)
+    whole = max(st["offload_bytes"] - (packed_tensor if packed_link > 0.001 * packed_tensor else 0.0), 0.0)
+    link = whole + packed_link
+    res["link_gb_each_way_per_step"] = link / 1e9
+    res["link_ms_each_way"] = link / (HOST_LINK_GBS * 1e9) * 1e3
+    if packed_tensor and packed_link > 0.001 * packed_tensor:
+        res["zvc_link_bytes_per_tensor_byte"] = packed_link / packed_tensor
+    ov = trace_overlap.summarize(trace_overlap.from_profile(intervals))
+    timed = sum(v["launches"] for v in prof.values())
+    share = timed / max(timed + untimed, 1)
+    steps_seen = profile_steps * share
+    res["profile_pass"] = {"steps": profile_steps, "launches_timed_share": share,
+                           "kernel_busy_ms_per_step": ov["compute_busy"] / max(steps_seen, 1e-9)}
+    if ov["copy_busy"] > 0:
+        copies = lambda keys: [prof[k] for k in keys if k in prof]
+        rate = lambda keys: (sum(c["bytes"] for c in copies(keys)) / max(sum(c["ms"] for c in copies(keys)), 1e-9) / 1e6) if copies(keys) else None
+        res["profile_pass"].update({
+            "copy_busy_ms_per_step": ov["copy_busy"] / steps_seen, "copy_beside_kernels_ms_per_step": ov["copy_beside_compute"] / steps_seen,
+            "overlap_fraction": ov["overlap_fraction"], "both_directions_at_once_ms_per_step": ov["duplex"] / steps_seen,
+            "d2h_tensor_gbs": rate(("offload_d2h", "offload_zvc", "offload_zvc_copy")), "h2d_tensor_gbs": rate(("prefetch_h2d", "prefetch_zvc"))})
+    # what no schedule can beat: the kernels back to back, or the link busy all step long in both directions at once
+    res["step_bound_ms"] = max(res["profile_pass"]["kernel_busy_ms_per_step"], res["link_ms_each_way"])
     return res, prof
 
 
@@ -96,67 +130,24 @@ def is_bf16(policy_name):
     return "bf16" in policy_name.split("+")[1:]
 
 
-def best_offloading(results, base):
-    """The offloading run that is fastest among those holding at least 3x less device memory than the fp32 BASELINE."""
+def best_within(results, base, floor_ratio, need_link):
+    """The fastest run that holds at least floor_ratio times less device memory than the fp32 BASELINE (and, with
+    need_link, moves something over the link)."""
     if not base:
         return None
-    ok = {k: v for k, v in results.items() if v["offload_gb_per_step"] > 0 and base["peak_hbm_gb"] / v["peak_hbm_gb"] >= 3.0}
+    ok = {k: v for k, v in results.items() if base["peak_hbm_gb"] / v["peak_hbm_gb"] >= floor_ratio and k.split("+")[0] != "BASELINE"
+          and (not need_link or v["link_gb_each_way_per_step"] > 0.5)}
     if not ok:
         return None
     k = max(ok, key=lambda n: ok[n]["images_per_s"])
     return {"policy": k, "speed_vs_baseline": ok[k]["images_per_s"] / base["images_per_s"],
             "peak_hbm_reduction": base["peak_hbm_gb"] / ok[k]["peak_hbm_gb"], "images_per_s": ok[k]["images_per_s"],
-            "peak_hbm_gb": ok[k]["peak_hbm_gb"]}
+            "peak_hbm_gb": ok[k]["peak_hbm_gb"], "link_gb_each_way_per_step": ok[k]["link_gb_each_way_per_step"]}
 
 
-def zvc_standalone(be):
-    """The compacting kernels alone on the device: a rectified fp32 tensor of conv2_1's input size (half zeros) is packed
-    into a staging block, moved by the copy engine, and expanded again from pinned host memory. Rates in bytes of the
-    tensor per second; the packing kernel reads the tensor and writes the stream (about 0.53 of it)."""
-    import ctypes as C
-    import numpy as np
-    lib, check = be.lib, be.check
-    ctx = be.Context(pool_bytes=6 << 30)
-    out = {}
-    try:
-        for es, dtype in ((4, np.uint32), (2, np.uint16)):
-            count = 128 * 64 * 112 * 112 * (4 // es)
-            rng = np.random.default_rng(1)
-            t = rng.integers(1, 60000, size=count, dtype=np.uint32).astype(dtype)
-            t[rng.random(count) < 0.5] = 0
-            src, dst = ctx.to_device(t, dtype), ctx.alloc(count * es)
-            need = lib.vdnn_zvc_buffer_bytes(count, es)
-            stage = ctx.alloc(need)
-            host = C.c_void_p()
-            check(lib.vdnn_host_alloc_pinned(ctx.handle, C.byref(host), need))
-            be.profile_enable(ctx.handle, True)
-            for _ in range(5):
-                check(lib.vdnn_zvc_offload_staged_async(ctx.handle, host, stage.ptr, need // 2 // 16 * 16 + 65536, src.ptr, count, es, None, None, None, None, 0))
-                ctx.synchronize()
-                check(lib.vdnn_zvc_prefetch_async(ctx.handle, dst.ptr, host, count, es, None))
-                ctx.synchronize()
-            prof = be.profile_collect(ctx.handle)
-            be.profile_enable(ctx.handle, False)
-            assert np.array_equal(dst.download((count,), dtype), t)
-            tensor_bytes, link_bytes = be.zvc_traffic(ctx.handle)
-            out["f32" if es == 4 else "bf16"] = {
-                "tensor_mb": count * es / 1e6,
-                "pack_gbs": prof["offload_zvc_pack"]["bytes"] / prof["offload_zvc_pack"]["ms"] / 1e6,
-                "pack_ms": prof["offload_zvc_pack"]["ms"] / prof["offload_zvc_pack"]["launches"],
-                "copy_gbs": prof["offload_zvc_copy"]["bytes"] / prof["offload_zvc_copy"]["ms"] / 1e6,
-                "expand_gbs": prof["prefetch_zvc"]["bytes"] / prof["prefetch_zvc"]["ms"] / 1e6}
-            check(lib.vdnn_host_free_pinned(ctx.handle, host))
-            for b in (src, dst, stage):
-                b.free()
-    finally:
-        ctx.close()
-    return out
-
-
-def cpu_baseline(batch):
-    """The checker's training step on the host cores, VGG16 at a reduced batch."""
+def cpu_baseline(batch, threads):
+    """The checker's training step (forward, backward, SGD) on the host cores: VGG16, float."""
     import oracle
-    threads = min(16, os.cpu_count() or 1)
     oracle.set_threads(threads)
     net = oracle.Net(cnn=4, batch=batch)
     net.init_seeded(1)
@@ -165,8 +156,9 @@ def cpu_baseline(batch):
     net.backward()
     dt = time.perf_counter() - t0
     net.close()
-    return {"value": batch / dt, "unit": "images/s", "cores": threads, "kind": "port",
-            "sample": "one VGG16 fp32 step (forward+backward+SGD) at batch %d instead of 128, %.1f s" % (batch, dt)}
+    return {"value": batch / dt, "unit": "images/s", "cores": threads, "kind": "port", "host_cpus_seen": os.cpu_count(),
+            "sample": "one VGG16 fp32 step (forward+backward+SGD) at batch %d (the headline's batch is 128), %.1f s; %s" % (
+                batch, dt, oracle.build_description())}
 
 
 def main():
@@ -174,23 +166,18 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--profile-steps", type=int, default=4, help="steps of the pass that times every launch")
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--algo", default="VDNN_MEMORY_OPT_ALGO")
-    ap.add_argument("--policies", default="BASELINE,VDNN_NONE,VDNN_CONV,VDNN_ALL,VDNN_CONV+refined,VDNN_ALL+refined,VDNN_CONV+refined+slack,"
-                    "BASELINE+fused,VDNN_CONV+refined+slack+fused,VDNN_CONV+refined+slack+zvc,VDNN_CONV+refined+ahead+fused+zvc,"
-                    "VDNN_CONV+refined+ahead+fused+zvc+tail,VDNN_CONV+refined+slack+fused+zvc+tail,VDNN_ALL+refined+slack+fused+zvc,"
-                    "VDNN_ALL+refined+fused+zvc+keep,VDNN_CONV+refined+fused+zvc+keep,"
-                    "BASELINE+bf16,VDNN_ALL+bf16,VDNN_CONV+refined+slack+bf16,VDNN_ALL+refined+slack+bf16,"
-                    "BASELINE+bf16+fused,VDNN_CONV+refined+slack+bf16+fused,VDNN_CONV+refined+ahead+bf16+fused+zvc+tail,"
-                    "VDNN_ALL+refined+slack+bf16+fused+zvc,VDNN_ALL+refined+bf16+fused+zvc+keep,VDNN_CONV+refined+bf16+fused+zvc+keep")
+    ap.add_argument("--policies", default=DEFAULT_POLICIES)
     ap.add_argument("--cap-gb", type=float, default=0.0, help="artificial limit on pool bytes in use (0 = none)")
-    ap.add_argument("--bf16", action="store_true", help="bfloat16 activation storage (products on the bfloat16 matrix cores, float accumulation and parameters)")
+    ap.add_argument("--bf16", action="store_true", help="bfloat16 activation storage in every configuration")
     ap.add_argument("--offload-lag", type=int, default=0, help="layers enqueued before an offloaded block is recycled (0 = reference schedule)")
     ap.add_argument("--prefetch-depth", type=int, default=1, help="offloaded tensors fetched ahead in backward (1 = reference schedule)")
     ap.add_argument("--keep-tail-gb", type=float, default=0.0, help="the deepest offloaded tensors stay on the device, up to this many GB")
-    ap.add_argument("--cpu-batch", type=int, default=24)
+    ap.add_argument("--cpu-batch", type=int, default=0, help="batch of the CPU baseline's step (0: four images per thread, about 25 s)")
+    ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (0: the box's CPU share, at most 16)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--zvc-standalone", action="store_true", help="also time the compacting kernels alone on the device")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
@@ -201,37 +188,51 @@ def main():
     from vdnn_implementation_amd.network import Network, parse
 
     cnn = enums.VGG16_128
+    # the fp32 BASELINE's peak, from a replay of its allocation schedule: what the "+budgetX" rows divide by X
+    with Network(cnn, enums.BASELINE, 0, args.batch, plan_only=True) as replay:
+        assert replay.forwardPropagation() == 0 and replay.backwardPropagation() == 0
+        baseline_peak = replay.stats()["peak_bytes_in_use"]
+
     results, profiles = {}, {}
     for name in args.policies.split(","):
-        # suffixes: "+refined" = the value-preserving lifetime refinements; "+slack" = blocks recycled six layers
-        # after their offload and two tensors fetched ahead; "+bf16" = bfloat16 activation storage; "+fused" = ReLU
-        # layers run inside the neighbouring layers' kernels; "+zvc" = offloaded rectified tensors cross the link
-        # without their zero elements (lossless)
+        # suffixes (none changes a computed value): "+refined" lifetime refinements; "+slack" blocks recycled six layers
+        # after their offload and two tensors fetched ahead; "+ahead" the same lag, backward fetches ahead wherever the
+        # peak cannot rise; "+fused" ReLU layers run inside the neighbouring layers' kernels; "+zvc" offloaded rectified
+        # tensors are packed (no zero elements); "+keep" the packed tensors stay in device memory; "+tail" the deepest
+        # 0.75 G elements of the offload set stay on the device; "+budgetX" the policy meets a budget of the fp32
+        # BASELINE's peak / X by choosing a place for every tensor; "+bf16" bfloat16 activation storage
         word, *mods = name.split("+")
-        # "+tail" = the deepest offloaded tensors, 0.75 G elements of them, stay on the device
-        # "+ahead" = backward fetches ahead wherever the peak cannot rise, blocks recycled six layers after their offload
-        # "+keep" = with zvc: the packed tensors stay in device memory instead of crossing the link
+        budget = [float(m[6:]) for m in mods if m.startswith("budget")]
+        mods = [m for m in mods if not m.startswith("budget")]
         assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep"}, name
         _, policy, algo = parse("VGG16_128", word, args.algo)
-        lag, depth = (6, 2) if "slack" in mods else (6, 1) if "ahead" in mods else (args.offload_lag, args.prefetch_depth)
-        log("[bench] %s %s batch %d: %d warm-up + %d timed steps" % (name, args.algo, args.batch, args.warmup, args.steps))
-        results[name], profiles[name] = run_policy(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, seed=1,
-                                                   refined=("refined" in mods), cap_bytes=int(args.cap_gb * 1e9),
-                                                   bf16=(args.bf16 or "bf16" in mods), offload_lag=lag, prefetch_depth=depth,
-                                                   fuse=("fused" in mods), compress=("zvc" in mods), ahead=("ahead" in mods), keep_packed=("keep" in mods), keep_tail_bytes=(int(0.75e9) * (2 if (args.bf16 or "bf16" in mods) else 4) if "tail" in mods
-                                                                    else int(args.keep_tail_gb * 1e9)))
-        log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, loss %.6f" % (
-            results[name]["ms_per_step"], results[name]["images_per_s"], results[name]["peak_hbm_gb"], results[name]["loss"]))
+        bf16 = args.bf16 or "bf16" in mods
+        # (what a plan sends over the link gets the slack that hides it: a lag of six layers on the way out, fetched
+        # ahead on the way back wherever the peak allows)
+        ahead = "ahead" in mods or bool(budget)
+        lag, depth = (6, 2) if "slack" in mods else (6, 1) if ahead else (args.offload_lag, args.prefetch_depth)
+        kw = dict(refined="refined" in mods, cap_bytes=int(args.cap_gb * 1e9), bf16=bf16, offload_lag=lag, prefetch_depth=depth,
+                  fuse="fused" in mods, compress="zvc" in mods, prefetch_within_peak=ahead, keep_packed="keep" in mods,
+                  keep_tail_bytes=int(0.75e9) * (2 if bf16 else 4) if "tail" in mods else int(args.keep_tail_gb * 1e9))
+        if budget:
+            kw.update(hbm_budget_bytes=int(baseline_peak / budget[0]), plan_packed_fraction=PACKED_FRACTION[bf16])
+        log("[bench] %s %s batch %d: %d warm-up + %d timed + %d profiled steps" % (name, args.algo, args.batch, args.warmup, args.steps, args.profile_steps))
+        results[name], profiles[name] = run_config(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, args.profile_steps, **kw)
+        r = results[name]
+        log("[bench]   %.1f ms/step, %.1f img/s, peak %.2f GB, link %.2f GB each way (%.1f ms), overlap %s, loss %.6f%s" % (
+            r["ms_per_step"], r["images_per_s"], r["peak_hbm_gb"], r["link_gb_each_way_per_step"], r["link_ms_each_way"],
+            "%.2f" % r["profile_pass"]["overlap_fraction"] if r["profile_pass"].get("overlap_fraction") is not None else "-", r["loss"],
+            (" plan %s" % json.dumps(r["plan"])) if "plan" in r else ""))
 
     head = "VDNN_ALL" if "VDNN_ALL" in results else list(results)[0]
     base = results.get("BASELINE")
-    # dominant kernel: the convolution class with the most device time over the timed steps of all
-    # policies of this run (the same launches a kernel trace of this command sees, warm-up aside)
+    # dominant kernel: the convolution class with the most device time over the profiled passes of the runs of the
+    # headline's element type
     prof = {}
-    headline_bf16 = args.bf16 or all(is_bf16(n) for n in profiles)   # (a run of bfloat16 configurations only)
+    headline_bf16 = args.bf16 or all(is_bf16(n) for n in profiles)
     for pname, p in profiles.items():
         if (args.bf16 or is_bf16(pname)) != headline_bf16:
-            continue  # the roofline entry is taken over the runs of the headline element type
+            continue
         for k, v in p.items():
             acc = prof.setdefault(k, {"launches": 0, "ms": 0.0, "flops": 0.0, "bytes": 0.0})
             for field in acc:
@@ -247,6 +248,8 @@ def main():
                    "tflops": (v["flops"] / (v["ms"] * 1e-3) / 1e12) if v["flops"] else None,
                    "gbs": (v["bytes"] / (v["ms"] * 1e-3) / 1e9) if v["bytes"] else None}
                for k, v in sorted(prof.items(), key=lambda kv: -kv[1]["ms"])}
+    fp32 = {k: v for k, v in results.items() if not (args.bf16 or is_bf16(k))}
+    traffic = measured_traffic().get(dom) if args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" and not headline_bf16 else None
     out = {
         "metric": "VGG16-128 train img/s (VDNN_ALL vs BASELINE); peak HBM GB; conv MFMA util",
         "value": results[head]["images_per_s"], "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -257,38 +260,28 @@ def main():
         "policies": results,
         "vdnn_all_vs_baseline_speed": (results[head]["images_per_s"] / base["images_per_s"]) if base else None,
         "peak_hbm_reduction_vs_baseline": (base["peak_hbm_gb"] / results[head]["peak_hbm_gb"]) if base else None,
-        "refined_vdnn_all_vs_baseline_speed": (results["VDNN_ALL+refined"]["images_per_s"] / base["images_per_s"])
-        if base and "VDNN_ALL+refined" in results else None,
-        "refined_peak_hbm_reduction_vs_baseline": (base["peak_hbm_gb"] / results["VDNN_ALL+refined"]["peak_hbm_gb"])
-        if base and "VDNN_ALL+refined" in results else None,
-        # fp32 VDNN_ALL with every value-preserving option on (refined lifetimes, fused rectifiers, compressed offload, packed
-        # tensors kept in device memory): same losses as the literal `value` run, bit for bit
-        "tuned_vdnn_all_vs_baseline_speed": (results["VDNN_ALL+refined+fused+zvc+keep"]["images_per_s"] / base["images_per_s"])
-        if base and "VDNN_ALL+refined+fused+zvc+keep" in results else None,
-        "tuned_peak_hbm_reduction_vs_baseline": (base["peak_hbm_gb"] / results["VDNN_ALL+refined+fused+zvc+keep"]["peak_hbm_gb"])
-        if base and "VDNN_ALL+refined+fused+zvc+keep" in results else None,
         "losses_bit_identical": len({results[k]["loss"] for k in results if not is_bf16(k)}) <= 1
         and len({results[k]["loss"] for k in results if is_bf16(k)}) <= 1,
-        "best_offloading_vs_fp32_baseline": best_offloading(results, base),
-        # the same among the fp32 runs only: speed and memory against BASELINE with the reference's element type
-        "best_fp32_offloading_vs_baseline": best_offloading({k: v for k, v in results.items() if not (args.bf16 or is_bf16(k))}, base),
+        # fp32 only, same losses as the literal run bit for bit: the fastest VDNN configuration at >= 3x less memory than
+        # BASELINE, and the fastest of those that move at least 0.5 GB over the link each way
+        "best_fp32_at_3x": best_within(fp32, base, 3.0, False),
+        "best_fp32_at_3x_over_the_link": best_within(fp32, base, 3.0, True),
+        "best_any_dtype_at_3x": best_within(results, base, 3.0, False),
+        "baseline_peak_gb_replayed": baseline_peak / 1e9,
         "conv_mfma_util": conv_all_tf / peak,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-                     "frac": achieved / peak,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom) if args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" and not headline_bf16 else None,
-                     "traffic_unit": "bytes per launch (L2 fetch + write-back, counters scaled by a known-size kernel)",
+                     "frac": achieved / peak, "traffic": traffic,
+                     "traffic_unit": "bytes per launch (L2 fetch + write-back); read from profiles/%s" % os.path.basename(TRAFFIC_PROFILE),
                      "algorithmic_flop_per_launch": d["flops"] / d["launches"],
                      "avg_launch_ms": d["ms"] / d["launches"], "launches": d["launches"]},
         "kernels": kernels,
         "step_mfma_frac": args.batch * FLOP_PER_IMAGE / (results[head]["ms_per_step"] * 1e-3) / 1e12 / peak,
     }
-    if args.zvc_standalone:
-        log("[bench] compacting kernels alone")
-        out["zvc_standalone"] = zvc_standalone(be)
-        log("[bench]   %s" % json.dumps(out["zvc_standalone"]))
     if not args.no_cpu_baseline:
-        log("[bench] CPU baseline: checker, VGG16 batch %d" % args.cpu_batch)
-        out["cpu_baseline"] = cpu_baseline(args.cpu_batch)
+        threads = args.cpu_threads or min(16, os.cpu_count() or 1)
+        cpu_batch = args.cpu_batch or 4 * threads
+        log("[bench] CPU baseline: checker, VGG16 batch %d on %d threads" % (cpu_batch, threads))
+        out["cpu_baseline"] = cpu_baseline(cpu_batch, threads)
     print(json.dumps(out), flush=True)
 
 

@@ -157,6 +157,13 @@ public:
     // Offloading and prefetching functions
     void    offloadSrcData(bool* _offloaded, DATATYPE** _offloadedSrcData_h);
     void    prefetchPreviousSrcData(DATATYPE* _prefetchedSrcData_h, void* _srcDataToPrefetch, unsigned long _prefetch_bytes);
+    /* additions (compressed offload). fetchPackedSrcData: the copy engine brings the first `bytes` of a packed stream
+       from pinned host memory into a block on the device, on the host-to-device stream, ordered like
+       prefetchPreviousSrcData. expandPackedSrcData: this layer's srcData is written from its packed stream - the first
+       stagingBytes of it in a block on the device, the rest (if any) in pinned host memory - by a kernel on the compute
+       stream, behind the events given (the copy that filled the block, the offload that filled the host buffer). */
+    void    fetchPackedSrcData(DATATYPE* _packed_h, void* _staging, size_t _bytes);
+    void    expandPackedSrcData(DATATYPE* _packed_h, const void* _staging, size_t _stagingBytes, vdnn_event_t _blockFilled, vdnn_event_t _hostFilled);
 
     // Allocate device memory from the pool (the reference's names, layer.cu:989-1011)
     int     cnmemMallocSrcData(bool isDynamic);

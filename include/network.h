@@ -78,7 +78,17 @@ struct NetworkOptions {
     // tensors of the shallow layers then start their way back while the small deep layers run, whose working
     // set is far below the peak. Same values, same peak, fewer waits for the link.
     bool     prefetchWithinPeak = false;
-    bool     tracePeaks = false;          // (internal: the replay records bytes in use per backward layer)
+    // A limit on pool bytes in use that the policy has to meet, instead of an offload set fixed by the policy's name
+    // (network.cu:898-936 offloads every member whatever the device could hold). With a budget, every member of the
+    // policy's offload set gets the cheapest of three places that keeps a replay of the schedule within the budget:
+    // it stays on the device as it is, it stays on the device as a packed stream (needs compressOffload and a
+    // rectified tensor), or it crosses the link (packed where it can be). Tensors are moved one place down, the
+    // largest one that is stored at the moment of the replay's peak first, until the replay fits; if it never does,
+    // the last plan stands and Network::planFeasible() says so. The replay has no data: planPackedFraction is what it
+    // takes a packed stream to be of its tensor. 0: no budget, the policy's own offload set.
+    size_t   hbmBudgetBytes = 0;
+    std::vector<unsigned char> forcedPlacement; // (internal: the replay's placement per layer, see Placement)
+    bool     tracePeaks = false;          // (internal: the replay records bytes in use per forward and backward layer)
     int      device = DEFAULT_DEVICE;
 };
 
@@ -100,6 +110,15 @@ struct NetworkStats {
     size_t pinnedBytes = 0;        // pinned host memory held for offloaded tensors
     size_t poolBytes = 0;
     size_t weightBytes = 0;
+};
+
+/* Where a member of the policy's offload set waits between its forward and its backward (addition, see
+ * NetworkOptions::hbmBudgetBytes). */
+enum Placement : unsigned char {
+    PLACE_POLICY   = 0, // no plan: what the policy and the other options say
+    PLACE_RESIDENT = 1, // on the device, as it is
+    PLACE_PACKED   = 2, // on the device, as a packed stream
+    PLACE_LINK     = 3, // in pinned host memory
 };
 
 class Network {
@@ -185,6 +204,12 @@ public:
     // the sequence (backward layer, prefetched layer) of the last backward
     const std::vector<std::pair<int, int>>& prefetchTrace() const { return prefetchLog; }
     const std::vector<size_t>& backwardPeakTrace() const { return bwdPeakTrace; }
+    const std::vector<size_t>& forwardPeakTrace() const { return fwdPeakTrace; }
+    // hbmBudgetBytes: the place each layer's input got (PLACE_POLICY for layers outside the offload set), whether the
+    // replay met the budget, what it peaked at, and the bytes the plan sends over the link each way per step
+    Placement       placementOf(int l) const { return l >= 0 && l < (int)placement.size() ? (Placement)placement[l] : PLACE_POLICY; }
+    bool            planFeasible() const { return planFeasibleFlag; }
+    size_t          planPeakBytes() const { return planBudgetPeak; }
     const std::vector<LayerSpec>& table() const { return specs; }
     static std::vector<LayerSpec> tableFor(CNN_t cnn, int batch);
 
@@ -245,7 +270,8 @@ private:
     vdnn_event_t        evPacked[DEFAULT_NUM_LAYER];      // d2h: the packing kernel has read srcData of layer l
     void*               zvcStaging[DEFAULT_NUM_LAYER];    // staging block of layer l's stream (null: none this step)
     size_t              zvcStagingBytes[DEFAULT_NUM_LAYER];
-    bool                zvcKept[DEFAULT_NUM_LAYER];       // the block stays until backward has expanded it
+    bool                zvcKept[DEFAULT_NUM_LAYER];       // the block holds the stream until layer l's backward has expanded it
+    bool                zvcFetched[DEFAULT_NUM_LAYER];    // ... and was filled by a copy from host memory during this backward
     bool                srcReleasedEarly[DEFAULT_NUM_LAYER]; // srcData of layer l went back to the pool behind its forward
     unsigned long long* zvcLength_h;                       // pinned: length of each layer's stream, reported by the packing kernel
     std::vector<int>    pendingOffload;                    // offloaded layers whose block is not yet recycled (offloadLag)
@@ -256,9 +282,17 @@ private:
     std::vector<std::pair<int, int>> prefetchLog;
     /* prefetchWithinPeak: from the replay - bytes in use during backward of each layer, their highest value, the
        layer whose backward fetches each offloaded tensor; and what this backward has fetched ahead of that */
-    std::vector<size_t> bwdPeakTrace, planBwdPeak, fetchedAhead;
+    std::vector<size_t> bwdPeakTrace, fwdPeakTrace, planBwdPeak, fetchedAhead;
+    /* hbmBudgetBytes */
+    std::vector<unsigned char> placement;
+    bool                keepPackedLayer[DEFAULT_NUM_LAYER]; // the packed stream of layer l's input stays on the device
+    bool                planFeasibleFlag = true;
+    size_t              planBudgetPeak = 0;
+    std::vector<unsigned char> planPlacement(vdnn_t policy, const std::vector<bool>& member);
     std::vector<int>    planIssueLayer;
     size_t              planPeak = 0, peakBudget = 0;
     void                buildPeakPlan(vdnn_t policy);
     int                 findPrefetchWithinPeak(int currLayerId);
+    size_t              stagedFetchBytes(int id) const;
+    int                 fetchPackedToStaging(int issuingLayer, int id, bool isDynamic);
 };

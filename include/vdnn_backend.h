@@ -319,6 +319,16 @@ typedef struct {
 } vdnn_profile_entry;
 int vdnn_profile_enable(vdnn_ctx* ctx, int on);
 int vdnn_profile_collect(vdnn_ctx* ctx, vdnn_profile_entry* out, int capacity, int* count);
+/* The same launches one by one, in the order they were made: when each began and ended, in milliseconds since the
+ * first of them began, and the stream it ran on (0 compute, 1 device-to-host, 2 host-to-device, 3 packing, 4 any
+ * other). From these a caller works out how much of the copies' time ran beside kernels of the compute stream.
+ * *count receives the number of timed launches, of which the first `capacity` are written. */
+typedef struct {
+    char   name[48];
+    int    stream;
+    double start_ms, stop_ms;
+} vdnn_profile_interval;
+int vdnn_profile_intervals(vdnn_ctx* ctx, vdnn_profile_interval* out, int capacity, int* count);
 
 #ifdef __cplusplus
 }

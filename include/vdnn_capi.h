@@ -36,6 +36,7 @@ typedef struct {
     int      keep_packed_on_device; /* with compress_offload: the packed tensors stay in device memory (about 0.6 of their size) instead of crossing the link */
     double   plan_packed_fraction;  /* what a plan-only network assumes a packed stream to be of its tensor (0 = the longest possible, 1.03) */
     int      compress_offload;  /* offloaded rectified tensors cross the link without their zero elements (lossless; layer.cu:969-987 copies them whole) */
+    size_t   hbm_budget_bytes;  /* a limit on pool bytes in use that the policy meets by choosing, per member of its offload set (network.cu:898-936), between the device, a packed stream on the device and host memory (0 = the policy's own set) */
 } vdnn_network_options;
 
 typedef struct {
@@ -90,6 +91,11 @@ void vdnn_network_stats_get(vdnn_network* net, vdnn_network_stats* out);
 void vdnn_network_reset_peak(vdnn_network* net);
 /* Network::isOffload[] after setVdnnType (network.cu:875-940) */
 int  vdnn_network_is_offloaded(vdnn_network* net, int l);
+/* hbm_budget_bytes: the place of layer l's input (0 no plan / not a member of the offload set, 1 on the device, 2 packed on
+ * the device, 3 host memory), whether the plan's replay met the budget, and what it peaked at */
+int  vdnn_network_placement(vdnn_network* net, int l);
+int  vdnn_network_plan_feasible(vdnn_network* net);
+size_t vdnn_network_plan_peak_bytes(vdnn_network* net);
 /* (backward layer, prefetched layer) pairs of the last backward, Network::findPrefetchLayer
  * (network.cu:1198-1208); returns the number of pairs */
 int  vdnn_network_prefetch_trace(vdnn_network* net, int* bwd_layer, int* prefetched_layer, int capacity);

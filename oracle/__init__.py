@@ -18,6 +18,15 @@ def build():
     subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"], stdout=subprocess.DEVNULL)
 
 
+def build_description():
+    """How the checker was compiled, for whoever reports its speed."""
+    flags = "?"
+    for line in open(os.path.join(_HERE, "Makefile")):
+        if line.startswith("CFLAGS"):
+            flags = line.split("=", 1)[1].strip()
+    return "C port of the layer math, direct loops with OpenMP over output planes, gcc %s" % flags
+
+
 def _load():
     if not os.path.exists(_LIB_PATH):
         build()

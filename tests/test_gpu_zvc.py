@@ -186,8 +186,16 @@ def test_rejects_bad_arguments(ctx):
 from test_gpu_fused import assert_fused_matches   # noqa: E402
 from test_gpu_network import assert_bit_identical, run_steps, small_specs   # noqa: E402
 from vdnn_implementation_amd import (ALEXNET_LRN, BASELINE, OVERFEAT, VDNN_ALL, VDNN_CONV, VDNN_MEMORY_OPT_ALGO,   # noqa: E402
-                                     VDNN_PERF_OPT_ALGO, VGG16_128)
+                                     VDNN_PERF_OPT_ALGO, VGG16_128, enums)
 from vdnn_implementation_amd.network import Network   # noqa: E402
+
+
+def rectified(specs, l):
+    """The input of layer l is the output of a ReLU, directly or behind max-pool / LRN layers: what goes out packed."""
+    p = l - 1
+    while p >= 0 and specs[p].type in (enums.POOL, enums.LRN):
+        p -= 1
+    return p >= 0 and specs[p].type == enums.RELU
 
 
 @pytest.mark.parametrize("cnn,batch,algo,bf16", [(None, 4, VDNN_MEMORY_OPT_ALGO, False), (ALEXNET_LRN, 4, VDNN_MEMORY_OPT_ALGO, False),
@@ -201,9 +209,22 @@ def test_networks_with_compressed_offload_keep_every_bit(cnn, batch, algo, bf16)
             return Network(layers=small_specs(batch), policy=policy, algo=algo, capture=True, seed=3, bf16=bf16, **kw)
         return Network(cnn, policy, algo, batch, capture=True, seed=3, bf16=bf16, **kw)
 
+    def budget_for(make, policy, kw):
+        """Between what the policy holds with everything on the device and with everything moved: half-way, or (tight) a
+        byte above the lowest peak any placement reaches, found by asking for the impossible."""
+        rest = {k: v for k, v in kw.items() if k != "hbm_budget_bytes"}
+        with make(policy, compress=True, plan_only=True, hbm_budget_bytes=1, **rest) as probe:
+            floor = probe.plan_peak_bytes()
+            assert not probe.plan_feasible()
+        with make(policy, compress=True, plan_only=True, hbm_budget_bytes=1 << 50, **rest) as probe:
+            ceiling = probe.plan_peak_bytes()
+            assert probe.plan_feasible() and all(p in (0, 1) for p in probe.placement())
+        assert floor <= ceiling   # (equal for a table so small that whole 512-byte blocks decide)
+        return floor + 1 if kw["hbm_budget_bytes"] == "tight" else (floor + ceiling) // 2
+
     announce("compressed offload", cnn, batch, "BASELINE")
     with make(BASELINE) as net:
-        want = run_steps(net, 2)
+        want = run_steps(net, 3)
         # a third of the activations, counted from the last layer down, stay on the device where a case says so
         tail = sum(int(np.prod([s.n, s.c, s.h, s.w])) for s in net.specs) * (2 if bf16 else 4) // 3
         specs = list(net.specs)
@@ -217,19 +238,31 @@ def test_networks_with_compressed_offload_keep_every_bit(cnn, batch, algo, bf16)
                        (VDNN_ALL, {"refined": True, "fuse": True, "keep_packed": True}),
                        (VDNN_CONV, {"offload_lag": 4, "keep_packed": True, "prefetch_depth": 2}),
                        (VDNN_ALL, {"host_sync": True, "keep_packed": True}),
-                       (VDNN_ALL, {"fuse": True, "offload_lag": 2, "prefetch_within_peak": True, "keep_tail_bytes": tail // 2})):
+                       (VDNN_ALL, {"fuse": True, "offload_lag": 2, "prefetch_within_peak": True, "keep_tail_bytes": tail // 2}),
+                       # a budget decides, tensor by tensor, between the device, a packed stream on the device and the host
+                       (VDNN_ALL, {"refined": True, "fuse": True, "plan_packed_fraction": 0.7, "hbm_budget_bytes": "tight"}),
+                       (VDNN_ALL, {"refined": True, "plan_packed_fraction": 0.7, "hbm_budget_bytes": "middle", "offload_lag": 3}),
+                       (VDNN_CONV, {"fuse": True, "plan_packed_fraction": 0.7, "hbm_budget_bytes": "tight", "prefetch_within_peak": True})):
+        if "hbm_budget_bytes" in kw:
+            kw = dict(kw)
+            kw["hbm_budget_bytes"] = budget_for(make, policy, kw)
         announce("compressed offload", cnn, batch, "policy", policy, kw)
         with make(policy, compress=True, **kw) as net:
-            got = run_steps(net, 2)
+            got = run_steps(net, 3)   # (from the second step on a stream's length is known: it comes back through a block)
             tensor_bytes, link_bytes = be.zvc_traffic(net.context)
             packed = [l for l in range(net.num_layers) if net.is_offloaded(l)]
+            if "hbm_budget_bytes" in kw:
+                places = net.placement()
+                assert net.plan_feasible() and {1, 2, 3} & set(places), places
+                assert [l for l, p in enumerate(places) if p in (2, 3)] == packed
         if kw.get("fuse"):   # (which layers mask their gradient depends on what is offloaded: compare layer by layer)
-            # (a layer whose packed input stays on the device expands it itself and masks as in BASELINE)
-            assert_fused_matches(got, want, specs, "policy %d %s" % (policy, kw), set() if kw.get("keep_packed") else set(packed))
+            # (a layer whose input is a packed stream expands it itself at the start of its backward - from the block it
+            # was kept in or the block the copy engine brought it back into - and masks as in BASELINE)
+            assert_fused_matches(got, want, specs, "policy %d %s" % (policy, kw), {l for l in packed if not rectified(specs, l)})
         else:
             assert_bit_identical(got, want, "policy %d %s" % (policy, kw))
-        if "keep_tail_bytes" in kw:
-            continue   # (a third of the activations can be the whole offload set of the policy)
+        if "keep_tail_bytes" in kw or "hbm_budget_bytes" in kw:
+            continue   # (a third of the activations can be the whole offload set of the policy; a budget may keep all on the device)
         assert packed, "the policy offloads something"
         assert tensor_bytes > 0, "some offloaded tensor is a rectified one"
         if cnn is not None:   # (the tensors of the small table are a slot or two: the map can outweigh their few zeros)

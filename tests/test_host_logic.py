@@ -573,3 +573,75 @@ def test_packed_tensors_kept_on_the_device_plan():
         # at 0.57 of a tensor the step holds less than a third of BASELINE's 18.65 GB; at the longest stream it does not
         assert sk["peak_bytes_in_use"] < 18.65e9 / 3 < sw["peak_bytes_in_use"]
         assert live_blocks(kept) == live_blocks(moved) == live_blocks(kept_worst)
+
+
+def test_hbm_budget_places_each_tensor_and_reports_the_floor():
+    """hbm_budget_bytes: every member of the offload set stays on the device, waits there as a packed stream, or crosses
+    the link - the cheapest that keeps a replay of the step within the budget. VGG16 batch 128, float, a packed stream
+    taken as 0.57 of its tensor: a third of BASELINE's 18.65 GB needs no link at all, and below 5.63 GB no placement
+    helps - that is convolution 1_2's backward (input, output gradient, input gradient: 3 x 1.64 GB, plus the
+    parameters and the staging area), when nothing that could be moved is left on the device."""
+    kw = dict(refined=True, fuse=True, compress=True, plan_packed_fraction=0.57)
+    with plan(VGG16_128, BASELINE) as net:
+        step(net)
+        base = net.stats()["peak_bytes_in_use"]
+    seen = {}
+    for ratio in (2.0, 3.0, 3.3, 4.0):
+        budget = int(base / ratio)
+        with plan(VGG16_128, VDNN_ALL, hbm_budget_bytes=budget, **kw) as net:
+            n0 = live_blocks(net)
+            step(net); step(net)
+            assert live_blocks(net) == n0
+            st, places = net.stats(), net.placement()
+            seen[ratio] = (net.plan_feasible(), net.plan_peak_bytes(), st, places)
+            assert st["peak_bytes_in_use"] == net.plan_peak_bytes(), "the step holds what the plan's replay held"
+            members = [l for l, p in enumerate(places) if p]
+            assert members == [l for l, s in enumerate(net.specs[:-1]) if s.type != enums.RELU]   # fused, refined VDNN_ALL
+            assert [l for l in members if places[l] in (2, 3)] == [l for l in range(net.num_layers) if net.is_offloaded(l)]
+            link = sum(int(np.prod(net.src_shape(l))) * 4 for l in members if places[l] == 3)
+            assert st["offload_bytes"] == st["prefetch_bytes"] == link
+    assert seen[2.0][0] and set(seen[2.0][3]) == {0, 1}                       # fits as it is: nothing packed, nothing moved
+    assert seen[3.0][0] and seen[3.0][1] <= base / 3 and 3 not in seen[3.0][3] and 2 in seen[3.0][3]
+    assert seen[3.3][0] and abs(seen[3.3][1] / GB - 5.63) < 0.01 and 3 not in seen[3.3][3]
+    assert not seen[4.0][0] and abs(seen[4.0][1] / GB - 5.63) < 0.01       # the floor: 3.31 x below BASELINE
+    # more is packed as the budget shrinks, never less
+    packed = {r: {l for l, p in enumerate(seen[r][3]) if p >= 2} for r in seen}
+    assert packed[2.0] <= packed[3.0] <= packed[3.3] <= packed[4.0]
+    # without packing the same budget sends the largest tensors over the link instead
+    with plan(VGG16_128, VDNN_ALL, hbm_budget_bytes=int(base / 2.5), refined=True, fuse=True) as net:
+        step(net)
+        assert net.plan_feasible() and set(net.placement()) == {0, 1, 3}
+        assert net.stats()["offload_bytes"] > 1.6e9
+    # BASELINE and VDNN_NONE offload nothing: the budget is accepted and changes nothing
+    with plan(VGG16_128, VDNN_NONE, hbm_budget_bytes=int(base / 3), **kw) as net:
+        step(net)
+        assert set(net.placement()) == {0} and net.stats()["offload_bytes"] == 0
+
+
+def test_packed_streams_come_back_through_a_block_of_their_own_length():
+    """A packed stream that crossed the link returns through the copy engine into a block sized from its length, a layer
+    ahead of its backward; the layer itself expands it. What is held a layer ahead is the stream, not the tensor: the
+    refined VDNN_ALL schedule of VGG16 batch 128 peaks lower than with plain copies, and moves the same tensors."""
+    kw = dict(refined=True, fuse=True)
+    with plan(VGG16_128, VDNN_ALL, **kw) as plain, plan(VGG16_128, VDNN_ALL, compress=True, plan_packed_fraction=0.57, **kw) as packed:
+        for net in (plain, packed):
+            n0 = live_blocks(net)
+            step(net); step(net)
+            assert live_blocks(net) == n0
+        a, b = plain.stats(), packed.stats()
+        assert b["offload_bytes"] == a["offload_bytes"] == b["prefetch_bytes"] == a["prefetch_bytes"]
+        assert plain.prefetch_trace() == packed.prefetch_trace()   # the same tensors fetched by the same layers
+        assert b["peak_bytes_in_use"] < a["peak_bytes_in_use"] - 0.25 * GB
+
+
+def test_overlap_of_copies_and_kernels_from_intervals():
+    """The interval arithmetic behind the bench's and the trace summary's overlap fraction, on a case worked by hand:
+    kernels [0,10] and [12,20]; a device-to-host copy [5,15], a host-to-device copy [14,30]."""
+    from vdnn_implementation_amd import trace_overlap as t
+    s = t.summarize([("compute", 0, 10), ("compute", 12, 20), ("d2h", 5, 15), ("h2d", 14, 30), ("compute", 3, 4)])
+    assert (s["span"], s["compute_busy"], s["copy_busy"], s["d2h_busy"], s["h2d_busy"]) == (30, 18, 25, 10, 16)
+    assert s["copy_beside_compute"] == 13 and s["overlap_fraction"] == 13 / 25 and s["duplex"] == 1 and s["copy_exposed"] == 12
+    assert t.summarize([("compute", 0, 5)])["overlap_fraction"] is None
+    recs = [("conv_fwd_128x128", 0, 0.0, 2.0), ("offload_d2h", 1, 1.0, 4.0), ("offload_zvc_pack", 3, 0.5, 0.7), ("prefetch_h2d", 2, 3.0, 5.0),
+            ("prefetch_zvc_device", 0, 5.0, 5.5)]
+    assert sorted(t.from_profile(recs)) == [("compute", 0.0, 2.0), ("compute", 5.0, 5.5), ("d2h", 1.0, 4.0), ("h2d", 3.0, 5.0)]

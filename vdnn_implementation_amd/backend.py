@@ -45,6 +45,10 @@ class ProfileEntry(C.Structure):
                 ("bytes", C.c_double)]
 
 
+class ProfileInterval(C.Structure):
+    _fields_ = [("name", C.c_char * 48), ("stream", C.c_int), ("start_ms", C.c_double), ("stop_ms", C.c_double)]
+
+
 _vp, _sz, _i, _f = C.c_void_p, C.c_size_t, C.c_int, C.c_float
 _S = C.POINTER(Shape)
 _psz = C.POINTER(C.c_size_t)
@@ -132,6 +136,7 @@ BACKEND_SYMBOLS = {
     "vdnn_cross_entropy_dense": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp]),
     "vdnn_profile_enable": (_i, [_vp, _i]),
     "vdnn_profile_collect": (_i, [_vp, C.POINTER(ProfileEntry), _i, C.POINTER(_i)]),
+    "vdnn_profile_intervals": (_i, [_vp, C.POINTER(ProfileInterval), _i, C.POINTER(_i)]),
 }
 
 for _name, (_res, _args) in BACKEND_SYMBOLS.items():
@@ -160,6 +165,14 @@ def profile_collect(ctx_handle):
     check(lib.vdnn_profile_collect(ctx_handle, arr, 64, C.byref(n)))
     return {arr[i].name.decode(): {"launches": int(arr[i].launches), "ms": arr[i].ms, "flops": arr[i].flops, "bytes": arr[i].bytes}
             for i in range(min(n.value, 64))}
+
+
+def profile_intervals(ctx_handle, capacity=4096):
+    """[(kernel class, stream 0..4, start ms, stop ms)] of the launches timed since profiling was enabled (synchronises)."""
+    arr = (ProfileInterval * capacity)()
+    n = _i()
+    check(lib.vdnn_profile_intervals(ctx_handle, arr, capacity, C.byref(n)))
+    return [(arr[i].name.decode(), arr[i].stream, arr[i].start_ms, arr[i].stop_ms) for i in range(min(n.value, capacity))]
 
 
 def zvc_traffic(ctx_handle):

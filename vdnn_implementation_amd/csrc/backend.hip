@@ -385,6 +385,33 @@ int vdnn_profile_collect(vdnn_ctx* ctx, vdnn_profile_entry* out, int capacity, i
     return VDNN_OK;
 }
 
+int vdnn_profile_intervals(vdnn_ctx* ctx, vdnn_profile_interval* out, int capacity, int* count) {
+    VDNN_REQUIRE(ctx && count, "null argument");
+    *count = 0;
+    if (ctx->plan_only || ctx->prof_records.empty()) return VDNN_OK;
+    VDNN_HIP(hipDeviceSynchronize());
+    // the earliest start is the origin: the first record made need not be the first to run (streams)
+    std::vector<float> t0(ctx->prof_records.size()), t1(ctx->prof_records.size());
+    const hipEvent_t origin = ctx->prof_records[0].start;
+    float lowest = 0.0f;
+    for (size_t i = 0; i < ctx->prof_records.size(); i++) {
+        const auto& r = ctx->prof_records[i];
+        VDNN_HIP(hipEventElapsedTime(&t0[i], origin, r.start));
+        VDNN_HIP(hipEventElapsedTime(&t1[i], origin, r.stop));
+        if (t0[i] < lowest) lowest = t0[i];
+    }
+    *count = (int)ctx->prof_records.size();
+    for (int i = 0; i < *count && i < capacity && out; i++) {
+        const auto& r = ctx->prof_records[i];
+        memset(&out[i], 0, sizeof(out[i]));
+        strncpy(out[i].name, r.name, sizeof(out[i].name) - 1);
+        out[i].stream = r.stream == ctx->compute ? 0 : r.stream == ctx->d2h ? 1 : r.stream == ctx->h2d ? 2 : r.stream == ctx->pack ? 3 : 4;
+        out[i].start_ms = (double)(t0[i] - lowest);
+        out[i].stop_ms = (double)(t1[i] - lowest);
+    }
+    return VDNN_OK;
+}
+
 int vdnn_out_dim(int in, int pad, int window, int stride) {
     if (stride <= 0 || window <= 0) return 0;
     const int t = in + 2 * pad - window;

@@ -25,7 +25,7 @@ struct vdnn_ctx {
     // At most kProfMaxRecords launches are timed between vdnn_profile_enable and vdnn_profile_collect; the
     // launches after that run untimed. With more than about six thousand events alive, recording one became slow
     // enough to double a step's time.
-    struct ProfRecord { const char* name; hipEvent_t start, stop; double flops, bytes; };
+    struct ProfRecord { const char* name; hipEvent_t start, stop; double flops, bytes; hipStream_t stream; };
     bool profiling = false;
     std::vector<ProfRecord> prof_records;
     std::vector<hipEvent_t> prof_free_events;
@@ -58,7 +58,7 @@ struct ProfScope {
         : ctx(c), stream(s), index(0), active(c->profiling && c->prof_records.size() < kProfMaxRecords) {
         if (!active && c->profiling) c->prof_untimed++;
         if (!active) return;
-        vdnn_ctx::ProfRecord r{name, prof_take_event(c), prof_take_event(c), flops, bytes};
+        vdnn_ctx::ProfRecord r{name, prof_take_event(c), prof_take_event(c), flops, bytes, s};
         if (!r.start || !r.stop) { active = false; return; }
         (void)hipEventRecord(r.start, stream);
         index = c->prof_records.size();

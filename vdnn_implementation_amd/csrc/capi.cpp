@@ -26,6 +26,7 @@ static NetworkOptions to_options(const vdnn_network_options* o) {
     n.keepPackedOnDevice = o->keep_packed_on_device != 0;
     n.planPackedFraction = o->plan_packed_fraction;
     n.prefetchWithinPeak = o->prefetch_within_peak != 0;
+    n.hbmBudgetBytes = o->hbm_budget_bytes;
     return n;
 }
 
@@ -48,6 +49,7 @@ void vdnn_network_default_options(vdnn_network_options* o) {
     o->keep_packed_on_device = d.keepPackedOnDevice;
     o->plan_packed_fraction = d.planPackedFraction;
     o->compress_offload = d.compressOffload;
+    o->hbm_budget_bytes = d.hbmBudgetBytes;
 }
 
 vdnn_network* vdnn_network_create(int cnn, int policy, int algo, int batch, const vdnn_network_options* o) {
@@ -139,6 +141,10 @@ void vdnn_network_reset_peak(vdnn_network* h) { h->net->resetPeak(); }
 int vdnn_network_is_offloaded(vdnn_network* h, int l) {
     return (l >= 0 && l < h->net->numLayersCount() && h->net->isOffloaded(l)) ? 1 : 0;
 }
+
+int vdnn_network_placement(vdnn_network* h, int l) { return (int)h->net->placementOf(l); }
+int vdnn_network_plan_feasible(vdnn_network* h) { return h->net->planFeasible() ? 1 : 0; }
+size_t vdnn_network_plan_peak_bytes(vdnn_network* h) { return h->net->planPeakBytes(); }
 
 int vdnn_network_prefetch_trace(vdnn_network* h, int* bwd_layer, int* prefetched_layer, int capacity) {
     const auto& t = h->net->prefetchTrace();

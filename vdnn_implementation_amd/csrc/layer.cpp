@@ -519,6 +519,23 @@ void Layer::prefetchPreviousSrcData(DATATYPE* _prefetchedSrcData_h, void* _srcDa
     if (prefetchDoneEvent) checkVDNN(vdnn_event_record(ctx, prefetchDoneEvent, h2d));
 }
 
+void Layer::fetchPackedSrcData(DATATYPE* _packed_h, void* _staging, size_t _bytes) {
+    vdnn_stream_t h2d = vdnn_ctx_stream_h2d(ctx);
+    if (prefetchBlockFreeEvent) {
+        checkVDNN(vdnn_event_record(ctx, prefetchBlockFreeEvent, *stream_compute));
+        checkVDNN(vdnn_stream_wait_event(ctx, h2d, prefetchBlockFreeEvent));
+    }
+    if (prefetchHostReadyEvent) checkVDNN(vdnn_stream_wait_event(ctx, h2d, prefetchHostReadyEvent));
+    checkVDNN(vdnn_memcpy_h2d_async(ctx, _staging, _packed_h, _bytes, h2d));
+    if (prefetchDoneEvent) checkVDNN(vdnn_event_record(ctx, prefetchDoneEvent, h2d));
+}
+
+void Layer::expandPackedSrcData(DATATYPE* _packed_h, const void* _staging, size_t _stagingBytes, vdnn_event_t _blockFilled, vdnn_event_t _hostFilled) {
+    if (_blockFilled) checkVDNN(vdnn_stream_wait_event(ctx, *stream_compute, _blockFilled));
+    if (_hostFilled) checkVDNN(vdnn_stream_wait_event(ctx, *stream_compute, _hostFilled));
+    checkVDNN(vdnn_zvc_prefetch_staged_async(ctx, srcData, _staging, _stagingBytes, _packed_h, SrcDataSize(), actBytes, *stream_compute));
+}
+
 /* layer.cu:989-1011 */
 int Layer::cnmemMallocSrcData(bool isDynamic) {
     if (ASSERT_EQ(vdnn_pool_malloc(ctx, &srcData, actBytes * SrcDataSize()), isDynamic) < 0) return -1;

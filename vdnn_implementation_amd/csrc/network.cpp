@@ -133,8 +133,9 @@ void Network::construct(vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) {
         evFwdDone[i] = evOffloadDone[i] = evBlockFree[i] = evPrefetchDone[i] = evPacked[i] = nullptr;
         zvcStaging[i] = nullptr;
         zvcStagingBytes[i] = 0;
-        zvcKept[i] = false;
+        zvcKept[i] = zvcFetched[i] = false;
         srcReleasedEarly[i] = false;
+        keepPackedLayer[i] = false;
     }
     zvcLength_h = nullptr;
 
@@ -211,7 +212,7 @@ void Network::reset(CNN_t _cnnType, vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) 
     for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
         zvcStaging[i] = nullptr;
         zvcStagingBytes[i] = 0;
-        zvcKept[i] = false;
+        zvcKept[i] = zvcFetched[i] = false;
         srcReleasedEarly[i] = false;
     }
     pendingOffload.clear();
@@ -429,12 +430,30 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         }
     }
 
+    /* the policy's offload set (network.cu:916-922, 928-936), less what the refinements above take out of it */
+    std::vector<bool> member(numLayers, false);
+    for (int l = 0; l < numLayers - 1; l++) {
+        const bool named = newVdnnType == VDNN_ALL || (newVdnnType == VDNN_CONV && is_conv(layer[l]->LayerType()));
+        member[l] = named && !dropSrcAfterFwd[l]     /* released, not moved: nothing reads it again */
+                    && !layer[l]->Elided()           /* its input is the next layer's srcData, which has its own turn */
+                    && l < tailStart;
+    }
+    /* hbmBudgetBytes: each member's place comes from a plan (the replay is handed one, the network itself makes one) */
+    placement.assign(numLayers, PLACE_POLICY);
+    planFeasibleFlag = true;
+    if (newVdnnType == VDNN_ALL || newVdnnType == VDNN_CONV) {
+        if ((int)options.forcedPlacement.size() == numLayers) placement = options.forcedPlacement;
+        else if (options.hbmBudgetBytes > 0 && !options.tracePeaks) placement = planPlacement(newVdnnType, member);
+    }
+
     auto offload = [&](int l) {
-        if (dropSrcAfterFwd[l]) return; /* released, not moved: nothing reads it again */
-        if (layer[l]->Elided()) return;  /* its input is the next layer's srcData, which has its own turn */
-        if (l >= tailStart) return;
+        keepPackedLayer[l] = false;
+        if (!member[l]) return;
+        if (placement[l] == PLACE_RESIDENT) return;
         isOffload[l] = true;
         const bool packed = options.compressOffload && srcIsRectified(l);
+        M_ASSERT(placement[l] != PLACE_PACKED || packed, "only a rectified tensor with compressOffload can wait as a packed stream");
+        keepPackedLayer[l] = packed && (placement[l] == PLACE_PACKED || (placement[l] == PLACE_POLICY && options.keepPackedOnDevice));
         layer[l]->setSrcPacked(packed);
         const size_t bytes = packed ? vdnn_zvc_buffer_bytes(layer[l]->SrcDataSize(), (int)actBytes())
                                     : layer[l]->SrcDataSize() * actBytes();
@@ -454,11 +473,8 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
     case VDNN_NONE:
         break;
     case VDNN_ALL:
-        for (int l = 0; l < numLayers - 1; l++) offload(l);
-        break;
     case VDNN_CONV:
-        for (int l = 0; l < numLayers - 1; l++)
-            if (is_conv(layer[l]->LayerType())) offload(l);
+        for (int l = 0; l < numLayers - 1; l++) offload(l);
         break;
     }
 
@@ -470,7 +486,7 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         const Layer_t t = layer[l]->LayerType();
         if (!is_conv(t) && t != FC_GEMM) continue; /* a pooling layer reads its input anyway */
         /* a packed input that stays on the device is expanded by the layer itself before its first kernel */
-        if (options.keepPackedOnDevice && layer[l]->SrcPacked()) continue;
+        if (layer[l]->SrcPacked()) continue; /* (also one that crosses the link: it comes back into a staging block) */
         layer[l]->setGateGrad(false);
         layer[l - 1]->setElidedBackward(false);
     }
@@ -607,10 +623,12 @@ int Network::forwardPropagation(bool isDynamic) {
         /* packed streams that a forward without a backward left on the device */
         for (int l = 0; l < numLayers; l++) {
             if (zvcKept[l] && zvcStaging[l]) ASSERT_EQ(vdnn_pool_free(ctx, zvcStaging[l]), isDynamic);
-            zvcKept[l] = false;
+            zvcKept[l] = zvcFetched[l] = false;
             zvcStaging[l] = nullptr;
         }
+        if (options.tracePeaks) fwdPeakTrace.assign(numLayers, 0);
         for (int l = 0; l < numLayers; l++) {
+            if (options.tracePeaks) vdnn_pool_reset_peak(ctx);
             layer[l]->copySrcData(l == 0 ? inputData : layer[l - 1]->DstData());
             if (isOffload[l]) {
                 layer[l]->setSrcReadyEvent(l == 0 ? evBlockFree[0] : evFwdDone[l - 1]);
@@ -637,7 +655,7 @@ int Network::forwardPropagation(bool isDynamic) {
                     layer[l]->setSrcReadyEvent(evBlockFree[l]);
                 }
                 zvcStagingBytes[l] = want;
-                zvcKept[l] = options.keepPackedOnDevice && want > 0;
+                zvcKept[l] = keepPackedLayer[l] && want > 0;
                 layer[l]->setOffloadStaging(zvcStaging[l], want, options.planOnly ? nullptr : &zvcLength_h[l], evPacked[l], zvcKept[l]);
             }
 
@@ -682,6 +700,11 @@ int Network::forwardPropagation(bool isDynamic) {
                 if (j == 0) { inputData = nullptr; inputResident = false; }
             }
             printUsage("Fwd", l, layer[l]->FwdWorkSpaceSize());
+            if (options.tracePeaks) {
+                size_t inUse = 0, extent = 0;
+                vdnn_pool_peak(ctx, &inUse, &extent);
+                fwdPeakTrace[l] = inUse;
+            }
         }
     }
     /* addition: mean cross-entropy of the output against the target, for monitoring */
@@ -758,17 +781,18 @@ int Network::backwardPropagation(bool isDynamic) {
             if (isOffload[l] && zvcKept[l] && !isPrefetched[l]) {
                 isPrefetched[l] = true;
                 if (layer[l]->cnmemMallocSrcData(isDynamic) < 0) return -1;
-                layer[l]->setPrefetchEvents(evBlockFree[l], evOffloadDone[l], evPrefetchDone[l]);
-                layer[l]->setPrefetchPacked(true);
-                layer[l]->setPrefetchStaging(zvcStaging[l], zvcStagingBytes[l]);
-                layer[l]->prefetchPreviousSrcData(offloadedSrcData_h[l], layer[l]->SrcData(), actBytes() * layer[l]->SrcDataSize());
-                prefetchLog.emplace_back(l, l);
+                /* on the compute stream: behind everything that used the recycled block, behind the copy that filled
+                   the staging block (if the stream came back over the link) and behind the offload that wrote what
+                   the block is too short for into host memory */
+                layer[l]->expandPackedSrcData(offloadedSrcData_h[l], zvcStaging[l], zvcStagingBytes[l],
+                                              zvcFetched[l] && !options.hostSync ? evPrefetchDone[l] : nullptr,
+                                              options.hostSync ? nullptr : evOffloadDone[l]);
+                if (!zvcFetched[l]) prefetchLog.emplace_back(l, l);
                 if (l == 0) { inputData = layer[0]->SrcData(); inputResident = true; }
                 if (options.hostSync) afterLayerSync();
-                else checkVDNN(vdnn_stream_wait_event(ctx, stream_compute, evPrefetchDone[l]));
                 ASSERT_EQ(vdnn_pool_free(ctx, zvcStaging[l]), isDynamic);
                 zvcStaging[l] = nullptr;
-                zvcKept[l] = false;
+                zvcKept[l] = zvcFetched[l] = false;
                 layer[l]->setSrcFetchedEvent(nullptr);
             } else {
                 /* this layer reads its own srcData: if that was prefetched, the copy must have landed */
@@ -776,14 +800,19 @@ int Network::backwardPropagation(bool isDynamic) {
             }
 
             int prefId = l == 0 ? -1 : (options.prefetchDepth > 1 ? findPrefetchLayerDeep(l) : findPrefetchLayer(l));
+            /* a packed stream comes back through the copy engine into a block of its own length; its layer expands it */
+            if (prefId >= 0 && stagedFetchBytes(prefId) > 0) {
+                if (fetchPackedToStaging(l, prefId, isDynamic) < 0) return -1;
+                prefId = -1;
+            }
             if (prefId >= 0) {
                 if (layer[prefId]->cnmemMallocSrcData(isDynamic) < 0) return -1;
                 layer[l]->setPrefetchEvents(evBlockFree[prefId], evOffloadDone[prefId], evPrefetchDone[prefId]);
                 layer[l]->setPrefetchPacked(layer[prefId]->SrcPacked());
-                layer[l]->setPrefetchStaging(zvcKept[prefId] ? zvcStaging[prefId] : nullptr, zvcKept[prefId] ? zvcStagingBytes[prefId] : 0);
+                layer[l]->setPrefetchStaging(nullptr, 0);
                 const size_t bytes = actBytes() * layer[prefId]->SrcDataSize();
                 if (layer[l]->backward(prefId, offloadedSrcData_h[prefId], layer[prefId]->SrcData(), bytes, workSpace, isDynamic) < 0) return -1;
-                if (!zvcKept[prefId]) lastStats.prefetchBytes += bytes;
+                lastStats.prefetchBytes += bytes;
                 prefetchLog.emplace_back(l, prefId);
                 if (prefId == 0) { inputData = layer[0]->SrcData(); inputResident = true; }
             } else {
@@ -794,13 +823,17 @@ int Network::backwardPropagation(bool isDynamic) {
                 int extra = options.prefetchDepth > 1 ? findPrefetchLayerDeep(l) : -1;
                 if (extra < 0 && options.prefetchWithinPeak) extra = findPrefetchWithinPeak(l);
                 if (extra < 0) break;
+                if (stagedFetchBytes(extra) > 0) {
+                    if (fetchPackedToStaging(l, extra, isDynamic) < 0) return -1;
+                    continue;
+                }
                 if (layer[extra]->cnmemMallocSrcData(isDynamic) < 0) return -1;
                 layer[l]->setPrefetchEvents(evBlockFree[extra], evOffloadDone[extra], evPrefetchDone[extra]);
                 layer[l]->setPrefetchPacked(layer[extra]->SrcPacked());
-                layer[l]->setPrefetchStaging(zvcKept[extra] ? zvcStaging[extra] : nullptr, zvcKept[extra] ? zvcStagingBytes[extra] : 0);
+                layer[l]->setPrefetchStaging(nullptr, 0);
                 const size_t bytes = actBytes() * layer[extra]->SrcDataSize();
                 layer[l]->prefetchPreviousSrcData(offloadedSrcData_h[extra], layer[extra]->SrcData(), bytes);
-                if (!zvcKept[extra]) lastStats.prefetchBytes += bytes;
+                lastStats.prefetchBytes += bytes;
                 prefetchLog.emplace_back(l, extra);
                 if (extra == 0) { inputData = layer[0]->SrcData(); inputResident = true; }
             }
@@ -862,6 +895,36 @@ std::vector<float> Network::train(int steps, bool isDynamic) {
     return losses;
 }
 
+/* addition (compressOffload): the bytes of the device block that a packed stream on its way back is copied into - the
+ * stream's length one step ago plus a margin, as on the way out - or 0 if the tensor comes back the plain way: it is
+ * not packed, or its length is not known yet (first step; the expanding kernel then reads pinned memory itself). */
+size_t Network::stagedFetchBytes(int id) const {
+    if (!isOffload[id] || !layer[id]->SrcPacked() || zvcKept[id]) return 0;
+    const size_t longest = vdnn_zvc_buffer_bytes(layer[id]->SrcDataSize(), (int)actBytes());
+    const size_t assumed = options.planPackedFraction > 0.0
+                               ? (size_t)(options.planPackedFraction * (double)(layer[id]->SrcDataSize() * actBytes())) : longest;
+    const size_t known = options.planOnly ? assumed : (zvcLength_h ? (size_t)zvcLength_h[id] : 0);
+    if (!known) return 0;
+    return std::min(longest, (known + known / 32 + 65536 + 15) / 16 * 16);
+}
+
+/* addition (compressOffload): during layer `issuingLayer`'s backward the copy engine starts to bring the packed stream
+ * of layer id's input back into a block of the pool; from here on the tensor counts as kept on the device, and its own
+ * layer expands it at the start of its backward (behind evPrefetchDone[id]). Only the stream's length is held a layer
+ * ahead, not the tensor, and the link runs at the copy engine's rate whatever the kernels beside it do. */
+int Network::fetchPackedToStaging(int issuingLayer, int id, bool isDynamic) {
+    const size_t want = stagedFetchBytes(id);
+    if (ASSERT_EQ(vdnn_pool_malloc(ctx, &zvcStaging[id], want), isDynamic) < 0) return -1;
+    zvcStagingBytes[id] = want;
+    layer[issuingLayer]->setPrefetchEvents(evBlockFree[id], evOffloadDone[id], evPrefetchDone[id]);
+    layer[issuingLayer]->fetchPackedSrcData(offloadedSrcData_h[id], zvcStaging[id], want);
+    zvcKept[id] = zvcFetched[id] = true;
+    isPrefetched[id] = false; /* its own layer's turn comes at the start of its backward */
+    lastStats.prefetchBytes += actBytes() * layer[id]->SrcDataSize();
+    prefetchLog.emplace_back(issuingLayer, id);
+    return 0;
+}
+
 /* network.cu:1193-1196 */
 void Network::resetIsPrefetchedArray() {
     for (int i = 0; i < DEFAULT_NUM_LAYER; i++) isPrefetched[i] = false;
@@ -893,11 +956,66 @@ void Network::buildPeakPlan(vdnn_t policy) {
     NetworkOptions o = options;
     o.planOnly = true; o.tracePeaks = true; o.prefetchWithinPeak = false;
     o.capture = false; o.verbose = false; o.capBytes = 0;
+    o.hbmBudgetBytes = 0; o.forcedPlacement = placement; /* the replay takes this network's plan, it makes none */
     Network replay(specs, policy, algoMode == VDNN_DYNAMIC_ALGO ? VDNN_MEMORY_OPT_ALGO : algoMode, o);
     if (replay.forwardPropagation(false) < 0 || replay.backwardPropagation(false) < 0) return;
     planBwdPeak = replay.backwardPeakTrace();
     for (const auto& p : replay.prefetchTrace()) planIssueLayer[p.second] = p.first;
     for (size_t b : planBwdPeak) planPeak = std::max(planPeak, b);
+}
+
+/* addition (hbmBudgetBytes): a place for every member of the offload set such that a replay of one step stays
+ * within the budget. Everything starts on the device as it is; while the replay peaks above the budget, the largest
+ * member that is stored at the moment of the peak (its forward is over, its backward has not begun) moves one place
+ * down: to a packed stream on the device if it is rectified and streams are packed at all, else - or from there - to
+ * host memory. Ends when the replay fits or nothing that is stored at the peak can move any further: then the peak is
+ * the working set of the layer itself, which no placement changes. */
+std::vector<unsigned char> Network::planPlacement(vdnn_t policy, const std::vector<bool>& member) {
+    std::vector<unsigned char> place(numLayers, PLACE_POLICY);
+    for (int l = 0; l < numLayers; l++) if (member[l]) place[l] = PLACE_RESIDENT;
+    NetworkOptions o = options;
+    o.planOnly = true; o.tracePeaks = true; o.prefetchWithinPeak = false; o.hbmBudgetBytes = 0;
+    o.capture = false; o.verbose = false; o.capBytes = 0; o.keepPackedOnDevice = false; o.keepTailBytes = 0;
+    const vdnnAlgoMode_t mode = algoMode == VDNN_DYNAMIC_ALGO ? VDNN_MEMORY_OPT_ALGO : algoMode;
+    planFeasibleFlag = false;
+    for (int round = 0; round <= 2 * numLayers; round++) {
+        o.forcedPlacement = place;
+        size_t peak = 0; int at = 0; bool inBackward = false;
+        {
+            Network replay(specs, policy, mode, o);
+            /* two steps: the first forward of a packed stream has no length to size its block by */
+            for (int step = 0; step < 2; step++)
+                if (replay.forwardPropagation(true) < 0 || replay.backwardPropagation(true) < 0) return place;
+            for (int l = 0; l < numLayers; l++) {
+                if (replay.forwardPeakTrace()[l] > peak) { peak = replay.forwardPeakTrace()[l]; at = l; inBackward = false; }
+                if (replay.backwardPeakTrace()[l] > peak) { peak = replay.backwardPeakTrace()[l]; at = l; inBackward = true; }
+            }
+        }
+        planBudgetPeak = peak;
+        if (peak <= options.hbmBudgetBytes) { planFeasibleFlag = true; break; }
+        /* stored at the peak: every member below the layer at work (in forward it has been written and left behind, in
+           backward it still waits for its turn) */
+        const double f = options.planPackedFraction > 0.0 ? options.planPackedFraction : 1.04;
+        /* a stream on the device costs two passes at HBM speed, the link a hundred times that: everything stored at the
+           peak that can be packed is packed before anything crosses the link; within a kind, the largest gain first */
+        int pick = -1; double best = 0.0; unsigned char to = PLACE_LINK;
+        for (int pass = 0; pass < 2 && pick < 0; pass++) {
+            for (int l = 0; l < at; l++) {
+                if (!member[l] || place[l] == PLACE_LINK) continue;
+                const double size = (double)(layer[l]->SrcDataSize() * actBytes());
+                const bool canPack = options.compressOffload && srcIsRectified(l) && f < 1.0;
+                const bool pack = place[l] == PLACE_RESIDENT && canPack;
+                if (pack != (pass == 0)) continue;
+                /* what the step down gives back: packing leaves f of the tensor, the link takes what is there */
+                const double gain = pack ? (1.0 - f) * size : (place[l] == PLACE_PACKED ? f * size : size);
+                if (gain > best) { best = gain; pick = l; to = pack ? PLACE_PACKED : PLACE_LINK; }
+            }
+        }
+        (void)inBackward;
+        if (pick < 0) break;
+        place[pick] = to;
+    }
+    return place;
 }
 
 /* addition (prefetchWithinPeak): the nearest offloaded tensor below currLayerId that is still on the host, if
@@ -909,7 +1027,8 @@ int Network::findPrefetchWithinPeak(int currLayerId) {
         if (!isOffload[id] || isPrefetched[id] || zvcKept[id]) continue;
         const int issue = planIssueLayer[id];
         if (issue < 0 || issue >= currLayerId) return -1;
-        const size_t bytes = actBytes() * layer[id]->SrcDataSize();
+        const size_t staged = stagedFetchBytes(id); /* a packed stream is held ahead as its own length, not the tensor's */
+        const size_t bytes = staged ? staged : actBytes() * layer[id]->SrcDataSize();
         for (int k = issue; k <= currLayerId; k++)
             if (planBwdPeak[k] + fetchedAhead[k] + bytes > peakBudget) return -1;
         for (int k = issue; k <= currLayerId; k++) fetchedAhead[k] += bytes;
