@@ -239,17 +239,25 @@ def main():
                 acc[field] += v[field]
     conv = {k: v for k, v in prof.items() if k.startswith("conv_") and v["flops"] > 0}
     prof = {k: v for k, v in prof.items() if v["ms"] > 0}
-    dom = max(conv, key=lambda k: conv[k]["ms"])
-    d = conv[dom]
-    achieved = d["flops"] / (d["ms"] * 1e-3) / 1e12
-    peak = BF16_MFMA_PEAK_TFLOPS if "bf16mfma" in dom else FP32_MFMA_PEAK_TFLOPS
-    conv_all_tf = sum(v["flops"] for v in conv.values()) / (sum(v["ms"] for v in conv.values()) * 1e-3) / 1e12
+    peak = BF16_MFMA_PEAK_TFLOPS if headline_bf16 else FP32_MFMA_PEAK_TFLOPS
+    roofline, conv_all_tf = None, None   # (a run with --profile-steps 0, for an outside profiler, times no launch)
+    if conv:
+        dom = max(conv, key=lambda k: conv[k]["ms"])
+        d = conv[dom]
+        achieved = d["flops"] / (d["ms"] * 1e-3) / 1e12
+        peak = BF16_MFMA_PEAK_TFLOPS if "bf16mfma" in dom else FP32_MFMA_PEAK_TFLOPS
+        conv_all_tf = sum(v["flops"] for v in conv.values()) / (sum(v["ms"] for v in conv.values()) * 1e-3) / 1e12
+        traffic = measured_traffic().get(dom) if args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" and not headline_bf16 else None
+        roofline = {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+                    "frac": achieved / peak, "traffic": traffic,
+                    "traffic_unit": "bytes per launch (L2 fetch + write-back); read from profiles/%s" % os.path.basename(TRAFFIC_PROFILE),
+                    "algorithmic_flop_per_launch": d["flops"] / d["launches"],
+                    "avg_launch_ms": d["ms"] / d["launches"], "launches": d["launches"]}
     kernels = {k: {"launches": v["launches"], "avg_ms": v["ms"] / max(v["launches"], 1),
                    "tflops": (v["flops"] / (v["ms"] * 1e-3) / 1e12) if v["flops"] else None,
                    "gbs": (v["bytes"] / (v["ms"] * 1e-3) / 1e9) if v["bytes"] else None}
                for k, v in sorted(prof.items(), key=lambda kv: -kv[1]["ms"])}
     fp32 = {k: v for k, v in results.items() if not (args.bf16 or is_bf16(k))}
-    traffic = measured_traffic().get(dom) if args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" and not headline_bf16 else None
     out = {
         "metric": "VGG16-128 train img/s (VDNN_ALL vs BASELINE); peak HBM GB; conv MFMA util",
         "value": results[head]["images_per_s"], "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -268,12 +276,8 @@ def main():
         "best_fp32_at_3x_over_the_link": best_within(fp32, base, 3.0, True),
         "best_any_dtype_at_3x": best_within(results, base, 3.0, False),
         "baseline_peak_gb_replayed": baseline_peak / 1e9,
-        "conv_mfma_util": conv_all_tf / peak,
-        "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-                     "frac": achieved / peak, "traffic": traffic,
-                     "traffic_unit": "bytes per launch (L2 fetch + write-back); read from profiles/%s" % os.path.basename(TRAFFIC_PROFILE),
-                     "algorithmic_flop_per_launch": d["flops"] / d["launches"],
-                     "avg_launch_ms": d["ms"] / d["launches"], "launches": d["launches"]},
+        "conv_mfma_util": conv_all_tf / peak if conv_all_tf else None,
+        "roofline": roofline,
         "kernels": kernels,
         "step_mfma_frac": args.batch * FLOP_PER_IMAGE / (results[head]["ms_per_step"] * 1e-3) / 1e12 / peak,
     }
