@@ -245,7 +245,7 @@ def main():
         dom = max(conv, key=lambda k: conv[k]["ms"])
         d = conv[dom]
         achieved = d["flops"] / (d["ms"] * 1e-3) / 1e12
-        peak = BF16_MFMA_PEAK_TFLOPS if "bf16mfma" in dom else FP32_MFMA_PEAK_TFLOPS
+        peak = BF16_MFMA_PEAK_TFLOPS if "bf16" in dom else FP32_MFMA_PEAK_TFLOPS
         conv_all_tf = sum(v["flops"] for v in conv.values()) / (sum(v["ms"] for v in conv.values()) * 1e-3) / 1e12
         traffic = measured_traffic().get(dom) if args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" and not headline_bf16 else None
         roofline = {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",

@@ -96,6 +96,11 @@ CONV = [
     (3, 64, 16, 22, 96, 3, 3, 0, 0, 1, 1),     # no padding, plane not a multiple of the slice
     (9, 256, 14, 14, 64, 3, 3, 1, 1, 1, 1),    # 14x14: three row wraps per slice in backward filter; forward splits its reduction
     (2, 64, 40, 36, 64, 1, 1, 0, 0, 1, 1),     # 1x1 window
+    # the windowed 3x3 kernel (stride 1, padding 1, even rows): tiles of 256 pixels
+    (2, 32, 5, 260, 64, 3, 3, 1, 1, 1, 1),     # rows longer than a tile: a tile starts and ends in the middle of a row
+    (40, 64, 5, 2, 160, 3, 3, 1, 1, 1, 1),     # two-pixel rows: a tile spans 25 samples, every pixel touches both borders
+    (3, 96, 56, 56, 128, 3, 3, 1, 1, 1, 1),    # three channel blocks, 128-row tiles, 36.75 tiles of pixels
+    (44, 96, 56, 56, 64, 3, 3, 1, 1, 1, 1),    # 539 tiles on 512 places: the last 27 are split along the reduction (tail mode)
 ]
 
 

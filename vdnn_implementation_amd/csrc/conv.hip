@@ -11,6 +11,7 @@
 #include "conv_loaders.h"
 #include "conv_loaders_tap.h"
 #include "mfma_bf16.h"
+#include "conv3x3_bf16.h"
 #include "conv_smallc.h"
 
 namespace vdnn {
@@ -65,6 +66,8 @@ static const PassNames kFwdPackedNames{"conv_fwd_packed_64x256", "conv_fwd_packe
 static const PassNames kBwdDataPackedNames{"conv_bwd_data_packed_64x256", "conv_bwd_data_packed_128x128"};
 static const PassNames kFwdHalfNames{"conv_fwd_bf16mfma_64x256", "conv_fwd_bf16mfma_128x128"};
 static const PassNames kBwdDataHalfNames{"conv_bwd_data_bf16mfma_64x256", "conv_bwd_data_bf16mfma_128x128"};
+static const PassNames kFwdWin3Names{"conv_fwd_bf16win_64x256", "conv_fwd_bf16win_64x256"};
+static const PassNames kBwdDataWin3Names{"conv_bwd_data_bf16win_64x256", "conv_bwd_data_bf16win_64x256"};
 static const PassNames kBwdFilterHalfNames{"conv_bwd_filter_bf16mfma_64x256", "conv_bwd_filter_bf16mfma_128x128"};
 
 template <int TM, int TN, class AL, class BL, class EP, bool HALF = false>
@@ -139,6 +142,58 @@ static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names
     if (tail_tiles > 0)
         return launch_reduce_tail_nchw(ctx, stream, ep.out, ep.partial, tail_tiles, d.splits, TM, TN, M, N, d.mtiles, d.full_tiles, ep.bias, ep.opix, ep.relu, ep.gate);
     return launch_reduce_splits_nchw(ctx, stream, ep.out, ep.partial, (size_t)M * N, d.splits, ep.bias, ep.opix, M, ep.relu, ep.gate);
+}
+
+// The windowed 3x3 kernel (conv3x3_bf16.h): tiles of 64 rows by 256 pixels, three workgroups resident per compute
+// unit, the reduction cut at multiples of one filter row of a channel block. Splits and tail mode as in launch_by_m.
+template <int MODE>
+static int launch_win3x3(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names, const LoadPackedH& al, const Win3x3& geo, const StoreNCHW<bf16_t>& ep,
+                         int M, int N, int K, double flops, size_t partial_bytes) {
+    const int TM = W3_TM, TN = W3_TN;
+    const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
+    int splits = 1;
+    const size_t out_bytes = (size_t)M * N * sizeof(float);
+    if (tiles < 2l * ctx->num_cu && ep.partial) {
+        long cap = ((long)K + 4 * W3_DEPTH - 1) / (4 * W3_DEPTH); // at least four filter rows per split
+        const long by_mem = (long)(partial_bytes / out_bytes);
+        if (cap > by_mem) cap = by_mem;
+        splits = choose_splits(tiles, K, cap, ctx->num_cu, out_bytes, 2.0 * TM * TN * KB);
+    }
+    GemmDims d = make_dims(M, N, K, TM, TN, splits, W3_DEPTH);
+    const long slots = 3l * ctx->num_cu;
+    const long rem = tiles % slots;
+    int tail_tiles = 0;
+    if (splits == 1 && tiles > slots && rem > 0 && 2 * rem <= slots && ep.partial) {
+        long s = slots / rem;
+        const long by_depth = (long)K / (4 * W3_DEPTH);
+        const long by_mem = (long)(partial_bytes / ((size_t)rem * TM * TN * sizeof(float)));
+        if (s > by_depth) s = by_depth;
+        if (s > by_mem) s = by_mem;
+        if (s >= 2) {
+            d = make_dims(M, N, K, TM, TN, (int)s, W3_DEPTH);
+            if (d.splits >= 2) { d.full_tiles = (int)(tiles - rem); tail_tiles = (int)rem; }
+            else d = make_dims(M, N, K, TM, TN, 1, W3_DEPTH);
+        }
+    }
+    const long all_tiles = (long)d.mtiles * d.ntiles;
+    const long blocks = d.full_tiles > 0 ? d.full_tiles + (all_tiles - d.full_tiles) * d.splits : all_tiles * d.splits;
+    if (blocks <= 0 || blocks >= (1l << 31)) { set_error("conv3x3: grid of %ld workgroups out of range", blocks); return VDNN_EINVAL; }
+    {
+        ProfScope prof(ctx, stream, names.t64, flops, 0.0);
+        hipLaunchKernelGGL((conv3x3_bf16_kernel<MODE>), dim3((unsigned)blocks), dim3(NT), 0, stream, al, geo, ep, d);
+        VDNN_LAUNCH_CHECK();
+    }
+    if (d.splits == 1) return VDNN_OK;
+    if (tail_tiles > 0)
+        return launch_reduce_tail_nchw(ctx, stream, ep.out, ep.partial, tail_tiles, d.splits, TM, TN, M, N, d.mtiles, d.full_tiles, ep.bias, ep.opix, ep.relu, ep.gate);
+    return launch_reduce_splits_nchw(ctx, stream, ep.out, ep.partial, (size_t)M * N, d.splits, ep.bias, ep.opix, M, ep.relu, ep.gate);
+}
+
+// what the windowed kernel needs: a 3x3 window at stride 1 with one pixel of padding (input and output planes of
+// one extent), rows of an even number of pixels, and tiles whose samples fit one descriptor
+static bool win3x3_ok(const int R, const int S, int ph, int pw, int sh, int sw, int Hs, int Ws, int OH, int OW, long sample_elems) {
+    return R == 3 && S == 3 && ph == 1 && pw == 1 && sh == 1 && sw == 1 && Hs == OH && Ws == OW && Ws % 2 == 0 && Ws >= 2 &&
+           pixel_tile_span_ok(sample_elems, OH * OW, W3_TN, 2);
 }
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
@@ -241,6 +296,11 @@ static int conv_half_engine(vdnn_ctx* ctx, hipStream_t st, const PassNames& name
     if (rc != VDNN_OK) return rc;
     ep.partial = (float*)((char*)ctx->reduce_scratch + taken);
     LoadPackedH al{packed, (long)Cred * RS, rows, (unsigned)(filter_elems * 2)};
+    // 3x3 at stride 1 with padding 1: one staged window per filter row serves its three taps
+    if (win3x3_ok(pix.R, pix.S, pix.ph, pix.pw, pix.sh, pix.sw, pix.Hs, pix.Ws, pix.OH, pix.OW, pix.sample_elems)) {
+        const Win3x3 geo{pix.src, pix.Hs, pix.Ws, pix.sample_elems, pix.sample_elems * pix.nsamples, pix.nsamples};
+        return launch_win3x3<MODE>(ctx, st, MODE == 0 ? kFwdWin3Names : kBwdDataWin3Names, al, geo, ep, rows, N, Cred * RS, flops, ctx->reduce_scratch_bytes - taken);
+    }
     // a pixel pair per lane where the pairs of an output row are contiguous in the input
     if (pix.OW % 2 == 0 && pix.S <= 16 && pix.Ws >= pix.S && pix.Ws > pix.pw + 1 && (MODE == 1 || pix.sw == 1)) {
         LoadIm2colPixTapH2<MODE> bl2{pix};

@@ -1,0 +1,274 @@
+// 3x3, stride 1, padding 1 convolutions of bfloat16 layers - forward and backward data - on the bfloat16
+// matrix cores, with the im2col operand formed in LDS from one staged window per filter row.
+//
+// The general bfloat16 engine (mfma_bf16.h) fetches the im2col tile of every tap from memory: nine times the
+// same input elements per channel block, two elements per load instruction, and it is bound by the number of
+// those loads. Here the reduction runs in the same blocked tap-major order (32 channels of one tap per slice),
+// but the three taps of a filter row share one *window*: for the tile's 256 consecutive output pixels j (an
+// even number of them per image row, so pixel pairs never straddle a row) the element "one filter row away",
+// x[c][pix(j) + (r-1) W], for 32 channels, plus one element to the left of the first pixel and one to the right
+// of the last. Tap s of that row reads the window shifted by s - 1 pixels. A pixel whose tap falls outside the
+// image reads zero: a row outside the image is never fetched (the lane's offset is sent out of the descriptor's
+// range), a column outside is masked when the fragment is read from LDS (the window holds the neighbouring
+// row's element there). So the im2col side costs a third of the loads and LDS stores per tap; the tile is
+// 64 x 256, the fragments of each half slice are read from LDS while the half before is multiplied, and the filter
+// operand is the packed bank of the general engine (pack_filter_tap_bf16_kernel).
+//
+// Same results as the general engine up to the order of summation inside the matrix cores (none: both sum a
+// slice's 32 products in the instruction and the slices in the same order), same epilogues, same split and
+// tail modes (the reduction is cut at multiples of one filter row: 96).
+#pragma once
+#include "mfma_bf16.h"
+
+namespace vdnn {
+
+constexpr int W3_TM = 64;             // output rows (channels) per tile
+constexpr int W3_TN = 256;            // pixels per tile
+constexpr int W3_ROWS = W3_TN + 2;    // window positions: one to the left, the tile, one to the right
+constexpr int W3_DEPTH = 3 * KH;      // reduction indices of one filter row of one channel block
+
+// MODE 0: forward, src = x, the window of filter row r lies (r - 1) rows below the pixel, tap s reads one column
+// further right per s. MODE 1: backward data, src = dy, filter row r lies (1 - r) rows away and tap s reads one
+// column further left per s.
+struct Win3x3 {
+    const bf16_t* src;
+    int H, W;            // extent of a plane (input and output planes agree)
+    long sample_elems;   // reduced channels * H * W
+    long total_elems;    // samples * sample_elems
+    int nsamples;
+};
+
+template <int MODE>
+__global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH al, const Win3x3 geo, const StoreNCHW<bf16_t> ep, const GemmDims d) {
+    // 64 rows x 256 pixels per workgroup, a 64 x 64 tile per wavefront: 64 accumulator registers, three workgroups
+    // resident per compute unit. (A 128 x 256 tile with 64 x 128 per wavefront reads a quarter less from LDS per
+    // MFMA but needs 400 registers: one wavefront per SIMD, and measured 25-40 % slower than this.)
+    constexpr int TM = W3_TM;
+    constexpr int WM = 1;                // wavefronts along the rows
+    constexpr int CW = W3_TN / 4;        // columns of a wavefront
+    constexpr int NJ = CW / 32;          // 32-column blocks of a wavefront
+    __shared__ __attribute__((aligned(16))) unsigned short As[2][TM * HSTRIDE];
+    __shared__ __attribute__((aligned(16))) unsigned short Bw[2][W3_ROWS * HSTRIDE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int ntiles_all = d.mtiles * d.ntiles;
+    int tile, ks;
+    bool whole;
+    if ((int)blockIdx.x < d.full_tiles) {
+        tile = xcd_remap(blockIdx.x, d.full_tiles); ks = 0; whole = true;
+    } else if (d.full_tiles > 0) {
+        const int r = blockIdx.x - d.full_tiles, tl = ntiles_all - d.full_tiles;
+        tile = d.full_tiles + r % tl; ks = r / tl; whole = false;
+    } else {
+        const int bid = xcd_remap(blockIdx.x, gridDim.x);
+        tile = bid % ntiles_all; ks = bid / ntiles_all; whole = d.splits == 1;
+    }
+    const int mt = tile % d.mtiles, nt = tile / d.mtiles;
+    const int m0 = mt * TM, j0 = nt * W3_TN;
+    const int k_begin = whole ? 0 : ks * d.kchunk;
+    const int k_end = whole ? d.K : min(d.K, k_begin + d.kchunk);
+    const int row_begin = k_begin / W3_DEPTH, row_end = (k_end + W3_DEPTH - 1) / W3_DEPTH; // (channel block, filter row) steps
+
+    const int W = geo.W, plane = geo.H * geo.W;
+    const int n_first = j0 / plane;
+    int n_last = (j0 + W3_TN - 1) / plane;
+    if (n_last > geo.nsamples - 1) n_last = geo.nsamples - 1;
+    // the descriptor starts W + 2 elements ahead of the first sample (a four-byte boundary: W is even) so that
+    // every offset below is non-negative, and ends with the last sample the tile touches
+    const long first = (long)n_first * geo.sample_elems;
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(geo.src + first - (W + 2), clamp_range(((long)(n_last - n_first + 1) * geo.sample_elems + (W + 2)) * 2));
+
+    // ---- filter operand: rows tid/4 + 64 i, eight reduction values at 8 (tid%4) ------------------------
+    typename LoadPackedH::template State<TM> sa;
+    typename LoadPackedH::template Regs<TM> ra;
+    al.template init<TM>(sa, m0, tid, d.M, k_begin);
+
+    // ---- window: thread = (pixel pair tid % 128, channel groups tid / 128 and tid / 128 + 2 of eight channels) ----
+    int voff;                 // byte offset of the pair's first pixel in its sample's first plane, or out of range
+    unsigned rowinv;          // bit r: filter row r of this pair's image row lies outside the image
+    {
+        const int j = j0 + 2 * (tid & 127);
+        const bool valid = j < d.N;
+        const int jj = valid ? j : j0;
+        const int n = jj / plane, pix = jj - n * plane;
+        const int p = pix / W;
+        voff = valid ? (int)(((long)(n - n_first) * geo.sample_elems + pix) * 2) : OOB;
+        rowinv = 0;
+#pragma unroll
+        for (int r = 0; r < 3; r++) {
+            const int ih = MODE == 0 ? p + r - 1 : p + 1 - r;
+            if (!((unsigned)ih < (unsigned)geo.H)) rowinv |= 1u << r;
+        }
+    }
+    // the two elements beside the tile, for 32 channels: lanes of wavefront 0, side = lane / 32, channel = lane % 32.
+    // The left one is needed (and inside the image row) when the tile's first pixel is not the first of its row,
+    // the right one when the tile's last pixel is not the last of its row.
+    int hoff = OOB;
+    unsigned hrowinv = 0;
+    if (wave == 0) {
+        const int side = lane >> 5, ch = lane & 31;
+        const int j = side ? j0 + W3_TN - 1 : j0;
+        if (j < d.N) {
+            const int n = j / plane, pix = j - n * plane;
+            const int p = pix / W, q = pix - p * W;
+            const bool needed = side ? q < W - 1 : q > 0;
+            if (needed) hoff = (int)(((long)(n - n_first) * geo.sample_elems + (long)ch * plane + pix + (side ? 1 : -1)) * 2);
+#pragma unroll
+            for (int r = 0; r < 3; r++) {
+                const int ih = MODE == 0 ? p + r - 1 : p + 1 - r;
+                if (!((unsigned)ih < (unsigned)geo.H)) hrowinv |= 1u << r;
+            }
+        }
+    }
+    // column masks of this lane's fragment columns: bit 2 jt: the tap that reads the column to the left falls
+    // outside; bit 2 jt + 1: the one that reads the column to the right does
+    const int wm0 = (wave % WM) * 64, wn0 = (wave / WM) * CW;
+    const int l32 = lane & 31, lk = lane >> 5;
+    unsigned colmask = 0;
+#pragma unroll
+    for (int jt = 0; jt < NJ; jt++) {
+        const int j = j0 + wn0 + jt * 32 + l32;
+        const int pix = j % plane, q = pix % W;
+        if (q == 0) colmask |= 1u << (2 * jt);
+        if (q == W - 1) colmask |= 2u << (2 * jt);
+    }
+
+    uintx4 wr[2][2];   // [item][pixel of the pair]: eight channels each, ready for LDS
+    unsigned hr = 0;   // the halo element of this lane (wavefront 0)
+    const int g0 = __builtin_amdgcn_readfirstlane(tid >> 7); // channel group of the thread's first item: uniform per wavefront
+
+    auto load_window = [&](int row_step) {
+        const int cb = row_step / 3, r = row_step - cb * 3;
+        const int rowoff = MODE == 0 ? (r - 1) * W : (1 - r) * W;
+        const int vo = voff | bit_to_all_ones(rowinv, r);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int ch = cb * KH + 8 * (g0 + 2 * i);
+            const int soff = (ch * plane + rowoff + W + 2) * 2, step = plane * 2;
+            unsigned c[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) c[e] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rsrc, vo, soff + e * step, 0);
+            // 2 x 8 transpose of 16-bit values: the low halves are the first pixel's channels, the high halves the second's
+            wr[i][0].x = __builtin_amdgcn_perm(c[1], c[0], 0x05040100u); wr[i][0].y = __builtin_amdgcn_perm(c[3], c[2], 0x05040100u);
+            wr[i][0].z = __builtin_amdgcn_perm(c[5], c[4], 0x05040100u); wr[i][0].w = __builtin_amdgcn_perm(c[7], c[6], 0x05040100u);
+            wr[i][1].x = __builtin_amdgcn_perm(c[1], c[0], 0x07060302u); wr[i][1].y = __builtin_amdgcn_perm(c[3], c[2], 0x07060302u);
+            wr[i][1].z = __builtin_amdgcn_perm(c[5], c[4], 0x07060302u); wr[i][1].w = __builtin_amdgcn_perm(c[7], c[6], 0x07060302u);
+        }
+        if (wave == 0) {
+            const int soff = (cb * KH * plane + rowoff + W + 2) * 2;
+            hr = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc, hoff | bit_to_all_ones(hrowinv, r), soff, 0);
+        }
+    };
+    auto store_window = [&](unsigned short* lds) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int e = 0; e < 2; e++)
+                *(uintx4*)(lds + (1 + 2 * (tid & 127) + e) * HSTRIDE + 8 * ((tid >> 7) + 2 * i)) = wr[i][e];
+        if (wave == 0) lds[((lane >> 5) ? W3_ROWS - 1 : 0) * HSTRIDE + (lane & 31)] = (unsigned short)hr;
+    };
+
+    floatx16 acc[NJ / 2][2][2]; // [64-column half][row block][column block]
+#pragma unroll
+    for (int q = 0; q < NJ / 2; q++)
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[q][i][j][v] = 0.0f;
+
+    // Pipeline. Step g = (row step, tap s) multiplies from As[g % 2] and the window buffer row_step % 2, as two halves
+    // of the slice's 32 reduction values (h = 0, 1), with one barrier between them:
+    //   first half:   read the fragments of (g, h = 1), multiply (g, h = 0) (fragments already in registers), write the
+    //                 registers holding the filter tile of step g + 1 to the other As buffer and, at s = 2, the window
+    //                 of the next row step to the other window buffer;
+    //   barrier;
+    //   second half:  issue the fetches of step g + 2 (at s = 2 also of the row step after the next), read the
+    //                 fragments of (g + 1, h = 0) from the buffers just completed, multiply (g, h = 1).
+    // Every fragment is thus read while the half before it is multiplied; all reads of a buffer precede the barrier
+    // after which it is overwritten. Fetches past the end of the range are never used.
+    auto read_a = [&](const unsigned short* buf, int h, bf16x8 (&a)[2]) {
+        const unsigned short* ap = buf + (wm0 + l32) * HSTRIDE + 8 * lk + 16 * h;
+#pragma unroll
+        for (int i = 0; i < 2; i++) a[i] = *(const bf16x8*)(ap + i * 32 * HSTRIDE);
+    };
+    // tap s reads the window position column + (s - 1) (forward) or column + (1 - s) (backward data): LDS row + 1;
+    // the tap that reads the left neighbour is s = 0 in forward, s = 2 in backward data
+    auto read_b = [&](const unsigned short* win, int s, int h, uintx4 (&b)[NJ]) {
+        const int shift = MODE == 0 ? s : 2 - s;
+        const unsigned short* bp = win + (wn0 + l32 + shift) * HSTRIDE + 8 * lk + 16 * h;
+#pragma unroll
+        for (int jt = 0; jt < NJ; jt++) b[jt] = *(const uintx4*)(bp + jt * 32 * HSTRIDE);
+    };
+    auto mask_b = [&](int s, uintx4 (&b)[NJ]) {
+        if (s == 1) return;
+        const bool left = MODE == 0 ? s == 0 : s == 2;
+#pragma unroll
+        for (int jt = 0; jt < NJ; jt++) {
+            const unsigned keep = ~(unsigned)bit_to_all_ones(colmask, 2 * jt + (left ? 0 : 1));
+            b[jt].x &= keep; b[jt].y &= keep; b[jt].z &= keep; b[jt].w &= keep;
+        }
+    };
+    auto multiply = [&](const bf16x8 (&a)[2], const uintx4 (&b)[NJ]) {
+#pragma unroll
+        for (int jt = 0; jt < NJ; jt++)
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                acc[jt / 2][i][jt % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], __builtin_bit_cast(bf16x8, b[jt]), acc[jt / 2][i][jt % 2], 0, 0, 0);
+    };
+
+    al.template load<TM>(sa, row_begin * W3_DEPTH, k_end, tid, ra);
+    load_window(row_begin);
+    LoadPackedH::template store<TM>(As[0], tid, ra);
+    store_window(Bw[0]);
+    al.template load<TM>(sa, row_begin * W3_DEPTH + KH, k_end, tid, ra);
+    load_window(row_begin + 1);
+    __syncthreads();
+    bf16x8 a0[2], a1[2];
+    uintx4 b0[NJ], b1[NJ];
+    read_a(As[0], 0, a0);
+    read_b(Bw[0], 0, 0, b0);
+    for (int row_step = row_begin; row_step < row_end; row_step++) {
+        const int wb = (row_step - row_begin) & 1;
+#pragma unroll
+        for (int s = 0; s < 3; s++) {
+            const int g = (row_step - row_begin) * 3 + s;
+            const int cur = g & 1, nxt = cur ^ 1;
+            read_a(As[cur], 1, a1);
+            read_b(Bw[wb], s, 1, b1);
+            mask_b(s, b0);
+            multiply(a0, b0);
+            LoadPackedH::template store<TM>(As[nxt], tid, ra);
+            if (s == 2) store_window(Bw[wb ^ 1]);
+            // issue order of the first half: an LDS access behind every MFMA
+#pragma unroll
+            for (int i = 0; i < 2 * NJ; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x300, 2, 0); }
+            __syncthreads();
+            al.template load<TM>(sa, row_begin * W3_DEPTH + (g + 2) * KH, k_end, tid, ra);
+            if (s == 2) load_window(row_step + 2);
+            read_a(As[nxt], 0, a0);
+            read_b(s == 2 ? Bw[wb ^ 1] : Bw[wb], s == 2 ? 0 : s + 1, 0, b0);
+            mask_b(s, b1);
+            multiply(a1, b1);
+            // second half: a memory instruction and an LDS read behind every MFMA
+#pragma unroll
+            for (int i = 0; i < 2 * NJ; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int q = 0; q < NJ / 2; q++) {
+        if (StoreNCHW<bf16_t>::TAIL && d.full_tiles > 0 && !whole)
+            ep.store_tail(acc[q], wm0, wn0 + 64 * q, lane, (long)(tile - d.full_tiles) * d.splits + ks, TM, W3_TN);
+        else
+            ep.store(acc[q], m0 + wm0, j0 + wn0 + 64 * q, lane, ks, d, !whole);
+    }
+}
+
+} // namespace vdnn
