@@ -12,10 +12,13 @@
 #endif
 
 static int g_acc_double = 0;
+static int g_blocked = 0; /* stride-1 convolutions through the blocked SGEMM of vdnn_oracle_gemm.c (float accumulation only) */
 static int g_threads = 0;
 
 void orc_set_accumulate_double(int on) { g_acc_double = on ? 1 : 0; }
 int  orc_get_accumulate_double(void) { return g_acc_double; }
+void orc_set_blocked_gemm(int on) { g_blocked = on ? 1 : 0; }
+int  orc_get_blocked_gemm(void) { return g_blocked; }
 void orc_set_threads(int n) {
     g_threads = n;
 #ifdef _OPENMP
@@ -106,6 +109,7 @@ DEFINE_CONV_FWD(conv_fwd_f32, float)
 DEFINE_CONV_FWD(conv_fwd_f64, double)
 
 void orc_conv_fwd(const orc_shape* g, const float* x, const float* w, const float* bias, float* y) {
+    if (g_blocked && !g_acc_double && orc_blocked_conv_ok(g)) { orc_blocked_conv_fwd(g, x, w, bias, y); return; }
     if (g_acc_double) conv_fwd_f64(g, x, w, bias, y);
     else conv_fwd_f32(g, x, w, bias, y);
 }
@@ -158,6 +162,7 @@ DEFINE_CONV_BWD_DATA(conv_bwd_data_f32, float)
 DEFINE_CONV_BWD_DATA(conv_bwd_data_f64, double)
 
 void orc_conv_bwd_data(const orc_shape* g, const float* dy, const float* w, float* dx) {
+    if (g_blocked && !g_acc_double && orc_blocked_conv_ok(g)) { orc_blocked_conv_bwd_data(g, dy, w, dx); return; }
     if (g_acc_double) conv_bwd_data_f64(g, dy, w, dx);
     else conv_bwd_data_f32(g, dy, w, dx);
 }
@@ -224,6 +229,7 @@ DEFINE_CONV_BWD_FILTER(conv_bwd_filter_f32, float)
 DEFINE_CONV_BWD_FILTER(conv_bwd_filter_f64, double)
 
 void orc_conv_bwd_filter_sgd(const orc_shape* g, const float* x, const float* dy, float* w, float alpha) {
+    if (g_blocked && !g_acc_double && orc_blocked_conv_ok(g)) { orc_blocked_conv_bwd_filter_sgd(g, x, dy, w, alpha); return; }
     if (g_acc_double) conv_bwd_filter_f64(g, x, dy, w, alpha);
     else conv_bwd_filter_f32(g, x, dy, w, alpha);
 }

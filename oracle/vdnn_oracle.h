@@ -48,6 +48,16 @@ typedef struct {
 /* accumulate convolution / GEMM sums in double (1) or float (0, default) */
 void orc_set_accumulate_double(int on);
 int  orc_get_accumulate_double(void);
+/* Route stride-1 convolutions (forward, backward data, backward filter) through im2col + cache-blocked SGEMM
+ * (vdnn_oracle_gemm.c) instead of the direct loops: the same sums in another order, several times faster. For the
+ * timed CPU baseline; off by default, ignored while sums are accumulated in double. Pinned by comparison with the
+ * direct loops on every convolution geometry of the fixtures (tests/test_oracle_layers.py). */
+void orc_set_blocked_gemm(int on);
+int  orc_get_blocked_gemm(void);
+int  orc_blocked_conv_ok(const orc_shape* g);
+void orc_blocked_conv_fwd(const orc_shape* g, const float* x, const float* w, const float* bias, float* y);
+void orc_blocked_conv_bwd_data(const orc_shape* g, const float* dy, const float* w, float* dx);
+void orc_blocked_conv_bwd_filter_sgd(const orc_shape* g, const float* x, const float* dy, float* w, float alpha);
 void orc_set_threads(int n);
 int  orc_get_threads(void);
 

@@ -40,6 +40,49 @@ def test_conv_brute_force_agrees(name):
     assert_close(oracle.conv_bwd_filter_brute(g, f["x"], f["dy"]), f["dw"], 1e-6, "brute bwd filter")
 
 
+@pytest.fixture
+def blocked():
+    oracle.set_blocked_gemm(True)
+    yield
+    oracle.set_blocked_gemm(False)
+
+
+@pytest.mark.parametrize("name", [n for n in CONV if "_s4" not in n and "_s2" not in n])
+def test_blocked_gemm_convolutions_against_torch(name, blocked):
+    """The im2col + blocked-SGEMM route (what the CPU baseline times) on the stride-1 fixtures: the same torch
+    expectations, the tolerance of float accumulation in another order."""
+    f = golden("conv_" + name)
+    g = shape_from_geom(oracle, f["geom"])
+    assert_close(oracle.conv_fwd(g, f["x"], f["w"], f["b"]), f["y"], 5e-6, "fwd")
+    assert_close(oracle.conv_bwd_data(g, f["dy"], f["w"]), f["dx"], 5e-6, "bwd data")
+    alpha = np.float32(-0.37)
+    assert_close(oracle.conv_bwd_filter_sgd(g, f["x"], f["dy"], f["w"], alpha), f["w"] + alpha * f["dw"], 5e-6, "bwd filter")
+
+
+@pytest.mark.parametrize("geom", [(3, 5, 9, 20, 7, 3, 3, 1, 1, 1, 1),     # nothing divides the 6 x 16 tiles
+                                  (2, 70, 14, 14, 130, 3, 3, 1, 1, 1, 1),  # several reduction blocks, rows shorter than a strip
+                                  (5, 16, 40, 36, 33, 3, 3, 1, 1, 1, 1),   # more than one pixel block per sample
+                                  (2, 6, 11, 13, 9, 5, 4, 2, 0, 1, 1),     # asymmetric window and padding
+                                  (4, 8, 10, 12, 12, 3, 3, 1, 1, 2, 1)])   # strided: falls back to the direct loops
+def test_blocked_gemm_convolutions_against_the_direct_loops(geom, blocked):
+    rng = np.random.default_rng(sum(geom))
+    g = oracle.shape(*geom)
+    x = rng.standard_normal((g.n, g.c, g.h, g.w)).astype(np.float32)
+    w = rng.standard_normal((g.k, g.c, g.r, g.s)).astype(np.float32)
+    b = rng.standard_normal(g.k).astype(np.float32)
+    got_y = oracle.conv_fwd(g, x, w, b)
+    dy = rng.standard_normal(got_y.shape).astype(np.float32)
+    got = (got_y, oracle.conv_bwd_data(g, dy, w), oracle.conv_bwd_filter_sgd(g, x, dy, w, np.float32(0.5)))
+    oracle.set_blocked_gemm(False)
+    oracle.set_accumulate_double(True)
+    try:
+        want = (oracle.conv_fwd(g, x, w, b), oracle.conv_bwd_data(g, dy, w), oracle.conv_bwd_filter_sgd(g, x, dy, w, np.float32(0.5)))
+    finally:
+        oracle.set_accumulate_double(False)
+    for a, e, what in zip(got, want, ("fwd", "bwd data", "bwd filter")):
+        assert_close(a, e, 1e-5, what)
+
+
 def test_conv_without_bias_and_zero_alpha():
     f = golden("conv_vgg_3x3_p1")
     g = shape_from_geom(oracle, f["geom"])
