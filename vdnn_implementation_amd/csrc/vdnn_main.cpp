@@ -1,5 +1,6 @@
 // Command-line front end: vdnn MODEL POLICY ALGO [--steps N] [--warmup N] [--batch N] [--seed N]
-//                                               [--cap-gb X] [--host-sync] [--plan] [--verbose]
+//                                               [--cap-gb X] [--host-sync] [--plan] [--verbose] [--refined] [--fuse]
+//                                               [--zvc] [--keep-packed] [--hbm-budget-gb X] [--packed-fraction F] ...
 // The three positional words are the reference's grammar (vdnn.cu:8-54, README.md:18-60). The
 // reference times one unsynchronised iteration and prints microseconds labelled "ms"
 // (vdnn.cu:72-79); here the device is synchronised on both sides of the timed region and the
@@ -60,6 +61,8 @@ int main(int argc, char** argv) {
         else if (!strcmp(argv[i], "--keep-packed")) opt.keepPackedOnDevice = true;
         else if (!strcmp(argv[i], "--prefetch-within-peak")) opt.prefetchWithinPeak = true;
         else if (!strcmp(argv[i], "--keep-tail-gb")) opt.keepTailBytes = (size_t)(atof(need("--keep-tail-gb needs a value")) * 1e9);
+        else if (!strcmp(argv[i], "--hbm-budget-gb")) opt.hbmBudgetBytes = (size_t)(atof(need("--hbm-budget-gb needs a value")) * 1e9);
+        else if (!strcmp(argv[i], "--packed-fraction")) opt.planPackedFraction = atof(need("--packed-fraction needs a value"));
         else if (!strcmp(argv[i], "--unfused")) opt.unfusedOptimizer = true;
         else if (!strcmp(argv[i], "--bf16")) opt.dataType = VDNN_DTYPE_BF16;
         else if (!strcmp(argv[i], "--offload-lag")) opt.offloadLag = atoi(need("--offload-lag needs a value"));
@@ -92,9 +95,10 @@ int main(int argc, char** argv) {
     cout << "Elapsed Time: " << us / 1000.0 << " ms for " << steps << " step(s)" << endl;
     printf("{\"model\": \"%s\", \"policy\": \"%s\", \"algo\": \"%s\", \"batch\": %d, \"steps\": %d, \"ms_per_step\": %.3f, "
            "\"images_per_s\": %.2f, \"loss\": %.6f, \"peak_bytes\": %zu, \"peak_extent\": %zu, \"offload_bytes\": %zu, "
-           "\"prefetch_bytes\": %zu, \"pinned_bytes\": %zu, \"plan_only\": %s}\n",
+           "\"prefetch_bytes\": %zu, \"pinned_bytes\": %zu, \"plan_only\": %s, \"plan_feasible\": %s, \"plan_peak_bytes\": %zu}\n",
            argv[1], argv[2], argv[3], network.batch(), steps, us / 1000.0 / steps,
            opt.planOnly ? 0.0 : network.batch() * steps / (us * 1e-6), network.loss(), st.peakBytesInUse, st.peakExtent,
-           st.offloadBytes, st.prefetchBytes, st.pinnedBytes, opt.planOnly ? "true" : "false");
+           st.offloadBytes, st.prefetchBytes, st.pinnedBytes, opt.planOnly ? "true" : "false",
+           network.planFeasible() ? "true" : "false", network.planPeakBytes());
     return 0;
 }
