@@ -137,7 +137,7 @@ def best_within(results, base, floor_ratio, need_link):
     if not base:
         return None
     ok = {k: v for k, v in results.items() if base["peak_hbm_gb"] / v["peak_hbm_gb"] >= floor_ratio and k.split("+")[0] != "BASELINE"
-          and (not need_link or v["link_gb_each_way_per_step"] > 0.5)}
+          and (not need_link or v["link_gb_each_way_per_step"] > 0.5) and v.get("plan", {}).get("feasible", True)}
     if not ok:
         return None
     k = max(ok, key=lambda n: ok[n]["images_per_s"])
