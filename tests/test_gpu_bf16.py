@@ -101,6 +101,14 @@ CONV = [
     (40, 64, 5, 2, 160, 3, 3, 1, 1, 1, 1),     # two-pixel rows: a tile spans 25 samples, every pixel touches both borders
     (3, 96, 56, 56, 128, 3, 3, 1, 1, 1, 1),    # three channel blocks, 128-row tiles, 36.75 tiles of pixels
     (44, 96, 56, 56, 64, 3, 3, 1, 1, 1, 1),    # 539 tiles on 512 places: the last 27 are split along the reduction (tail mode)
+    # backward filter with one filter row and 64 input channels per workgroup (rows of whole 8-pixel groups, C % 64 == 0)
+    (2, 64, 4, 32, 64, 3, 3, 1, 1, 1, 1),      # 64-row tile, one reduction split (results stored directly), rows one slice long
+    (7, 128, 6, 32, 192, 3, 3, 1, 1, 1, 1),    # two channel blocks, a ragged second row tile, five splits that straddle samples, the last shorter
+    (3, 64, 56, 56, 130, 3, 3, 1, 1, 1, 1),    # VGG-sized rows: a slice wraps an image row in the middle; two rows in the last tile
+    (2, 192, 8, 40, 128, 3, 3, 1, 1, 1, 1),    # rows of five groups: slices start at every group of a row
+    (2, 128, 12, 20, 192, 3, 3, 1, 1, 1, 1),   # rows of two and a half groups: every other row begins in the middle of a group
+    (5, 64, 2, 16, 64, 3, 3, 1, 1, 1, 1),      # a slice covers a whole two-row sample: every row touches the upper or the lower border
+    (3, 64, 6, 28, 96, 3, 3, 1, 1, 1, 1),      # 28-pixel rows, plane not a multiple of the slice: slices straddle samples
 ]
 
 

@@ -12,6 +12,7 @@
 #include "conv_loaders_tap.h"
 #include "mfma_bf16.h"
 #include "conv3x3_bf16.h"
+#include "wgrad3x3_bf16.h"
 #include "conv_smallc.h"
 
 namespace vdnn {
@@ -69,6 +70,7 @@ static const PassNames kBwdDataHalfNames{"conv_bwd_data_bf16mfma_64x256", "conv_
 static const PassNames kFwdWin3Names{"conv_fwd_bf16win_64x256", "conv_fwd_bf16win_64x256"};
 static const PassNames kBwdDataWin3Names{"conv_bwd_data_bf16win_64x256", "conv_bwd_data_bf16win_64x256"};
 static const PassNames kBwdFilterHalfNames{"conv_bwd_filter_bf16mfma_64x256", "conv_bwd_filter_bf16mfma_128x128"};
+static const PassNames kBwdFilterWin3Names{"conv_bwd_filter_bf16win_64x192", "conv_bwd_filter_bf16win_128x192"};
 
 template <int TM, int TN, class AL, class BL, class EP, bool HALF = false>
 static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, const AL& al, const BL& bl, const EP& ep, const GemmDims& d, double flops = 0.0) {
@@ -320,6 +322,80 @@ static int launch_pack_filter(vdnn_ctx* ctx, hipStream_t st, const float* w, flo
     return VDNN_OK;
 }
 
+// Workgroups of wgrad3x3_bf16_kernel that are resident on a compute unit (its launch bounds).
+constexpr int kWgrad3PerCU = 2;
+
+static bool wgrad3x3_ok(const ConvGeo& g) {
+    return g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W &&
+           g.W % 4 == 0 && g.W >= 16 && (g.H * g.W) % 8 == 0 && g.C % WG3_CH == 0; // a slice wraps at most two image rows
+}
+
+// One filter row, 64 input channels and 128 (64) output channels per workgroup; the pixel reduction is split so
+// that one round of workgroups fills the chip, as far as the staging area holds the partial sums.
+static int launch_wgrad3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const bf16_t* x, const bf16_t* dy, float* w, float alpha, int accumulate,
+                           float* staging, size_t staging_bytes, bool* taken) {
+    *taken = false;
+    const int M = g.K, N = g.C * 9, PQ = g.H * g.W;
+    const long Kred = (long)g.N * PQ;
+    const bool narrow = M <= 64;
+    const int TM = narrow ? 64 : 128;
+    const int mtiles = (M + TM - 1) / TM, ntiles = 3 * (g.C / WG3_CH);
+    const long tiles = (long)mtiles * ntiles;
+    const size_t out_bytes = (size_t)M * N * sizeof(float);
+    long splits = (long)kWgrad3PerCU * ctx->num_cu / tiles;
+    const long by_len = Kred / (8 * KH); // at least eight slices per split
+    const long by_mem = staging ? (long)(staging_bytes / out_bytes) : 1;
+    if (splits > by_len) splits = by_len;
+    if (splits > by_mem) splits = by_mem;
+    if (splits < 1) splits = 1;
+    GemmDims d = make_dims(M, N, (int)Kred, TM, 3 * WG3_CH, (int)splits, KH);
+    d.mtiles = mtiles; d.ntiles = ntiles;
+    const long nspan = d.kchunk / PQ + 2;
+    if (nspan * g.K * PQ * 2 >= (long)MAX_SUM_RANGE || nspan * g.C * PQ * 2 >= (long)MAX_SUM_RANGE) return VDNN_OK; // not taken
+    if (d.splits > 1 && !staging) return VDNN_OK;
+    const long blocks = tiles * d.splits;
+    if (blocks <= 0 || blocks >= (1l << 31)) return VDNN_OK;
+    *taken = true;
+    const Wgrad3x3 geo{dy, x, g.N, g.K, g.C, g.H, g.W, w, staging, (long)M * N, alpha, accumulate};
+    {
+        ProfScope prof(ctx, st, narrow ? kBwdFilterWin3Names.t64 : kBwdFilterWin3Names.t128, 2.0 * M * (double)N * (double)Kred, 0.0);
+        const bool halfrow = g.W % 8 != 0 || g.W < KH; // the general variant: groups across two image rows, two row wraps per slice
+        if (narrow && halfrow) hipLaunchKernelGGL((wgrad3x3_bf16_kernel<32, true>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        else if (narrow) hipLaunchKernelGGL((wgrad3x3_bf16_kernel<32, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        else if (halfrow) hipLaunchKernelGGL((wgrad3x3_bf16_kernel<64, true>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        else hipLaunchKernelGGL((wgrad3x3_bf16_kernel<64, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        VDNN_LAUNCH_CHECK();
+    }
+    if (d.splits > 1) return launch_reduce_splits_tap(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, accumulate, g.C, 9);
+    return VDNN_OK;
+}
+
+// Backward filter of a bfloat16 3x3 / stride 1 / padding 1 layer with the vector loaders: picks the instantiation
+// for the number of taps per tile and the pixel group (combinations whose loads would mix taps do not exist).
+template <int TM, int TN, int NTAP, int G>
+static int launch_wgrad_vec_one(vdnn_ctx* ctx, hipStream_t st, const char* name, const LoadDyRedVecH<8>& al, const LoadIm2colRedTapVecH<1, 8>& geo,
+                                const StoreFilterTap& ep, const GemmDims& d) {
+    if constexpr ((TN / NTAP) % (NT / (KH / G)) != 0) {
+        set_error("backward filter: %d taps per %d-column tile with groups of %d pixels", NTAP, TN, G);
+        return VDNN_EINVAL;
+    } else {
+        LoadIm2colRedTapVecH<NTAP, G> bl{geo.x, geo.N, geo.C, geo.H, geo.W, geo.ncols, geo.kchunk, geo.Ktot, geo.divC};
+        return launch_igemm<TM, TN, LoadDyRedVecH<8>, LoadIm2colRedTapVecH<NTAP, G>, StoreFilterTap, true>(ctx, st, name, al, bl, ep, d);
+    }
+}
+template <int TM, int TN>
+static int launch_wgrad_vec(vdnn_ctx* ctx, hipStream_t st, const char* name, const LoadDyRedVecH<8>& al, const LoadIm2colRedTapVecH<1, 8>& geo,
+                            const StoreFilterTap& ep, const GemmDims& d, int ntap, int group) {
+    if (group == 8) {
+        if (ntap == 1) return launch_wgrad_vec_one<TM, TN, 1, 8>(ctx, st, name, al, geo, ep, d);
+        if (ntap == 2) return launch_wgrad_vec_one<TM, TN, 2, 8>(ctx, st, name, al, geo, ep, d);
+        return launch_wgrad_vec_one<TM, TN, 4, 8>(ctx, st, name, al, geo, ep, d);
+    }
+    if (ntap == 1) return launch_wgrad_vec_one<TM, TN, 1, 4>(ctx, st, name, al, geo, ep, d);
+    if (ntap == 2) return launch_wgrad_vec_one<TM, TN, 2, 4>(ctx, st, name, al, geo, ep, d);
+    return launch_wgrad_vec_one<TM, TN, 4, 4>(ctx, st, name, al, geo, ep, d);
+}
+
 } // namespace vdnn
 
 using namespace vdnn;
@@ -562,6 +638,11 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     const int ntap = g.C % tile_n == 0 ? 1 : (g.C % (tile_n / 2) == 0 ? 2 : (g.C % (tile_n / 4) == 0 ? 4 : 0));
     if constexpr (sizeof(E) == 2) {
         // bfloat16 activations: both factors of every product are bfloat16 already
+        if (wgrad3x3_ok(g) && aligned16(dy) && aligned16(x)) {
+            bool taken = false;
+            const int rcw = launch_wgrad3x3(ctx, st, g, x, dy, w, alpha, accumulate, staging, staging_bytes, &taken);
+            if (taken || rcw != VDNN_OK) return rcw;
+        }
         if (vec && ntap != 0 && PQ >= KH && 3 * g.Q >= KH && g.Q % 2 == 0 && ((uintptr_t)x & 3) == 0 && staging) {
             long caph = (Kred + 4 * KH - 1) / (4 * KH);
             if (caph > by_mem) caph = by_mem;
@@ -573,6 +654,20 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
                 StoreFilterTap ept{w, staging, g.C, RS, (long)M * N, alpha, accumulate, dC};
                 LoadDyRedIncH al{dy, g.N, g.K, PQ, dh.kchunk, dh.K};
                 int rch;
+                // 3x3, stride 1, padding 1: a tap's im2col operand is the plane shifted by a constant, fetched in
+                // groups of eight (four) pixels when the image rows are whole groups
+                const int vg = g.W % 8 == 0 ? 8 : (g.W % 4 == 0 ? 4 : 0);
+                const int tap_cols = tile_n / ntap; // columns of the tile that share a tap
+                if (g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W && PQ % 8 == 0 &&
+                    vg != 0 && tap_cols % (8 * vg) == 0 && (long)g.C * g.H * g.W * 2 < (long)MAX_SUM_RANGE) {
+                    LoadDyRedVecH<8> alv{dy, g.N, g.K, PQ, dh.kchunk, dh.K};
+                    LoadIm2colRedTapVecH<1, 8> geo{x, g.N, g.C, g.H, g.W, N, dh.kchunk, dh.K, dC};
+                    rch = narrow ? launch_wgrad_vec<64, 256>(ctx, st, kBwdFilterHalfNames.t64, alv, geo, ept, dh, ntap, vg)
+                                 : launch_wgrad_vec<128, 128>(ctx, st, kBwdFilterHalfNames.t128, alv, geo, ept, dh, ntap, vg);
+                    if (rch != VDNN_OK) return rch;
+                    if (dh.splits > 1) return launch_reduce_splits_tap(ctx, st, w, staging, (size_t)M * N, dh.splits, alpha, accumulate, g.C, RS);
+                    return VDNN_OK;
+                }
 #define VDNN_WGRAD_TAP_H(NTAP)                                                                                              \
                 do {                                                                                                        \
                     if (g.sw == 1) {                                                                                        \

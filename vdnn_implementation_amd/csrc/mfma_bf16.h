@@ -348,6 +348,178 @@ struct LoadIm2colRedTapH {
     }
 };
 
+// ---- backward filter of 3x3 / stride 1 / padding 1 layers: vector loads along the reduction -------------
+// Through tap (r, s) output pixel j of a sample reads element j + (r-1)*W + (s-1) of an input plane: one tap's
+// im2col operand is the plane shifted by a constant, and so are G consecutive pixels as long as they share an
+// image row (G divides W) - one G-element load per (column, pixel group), at two-byte alignment for the outer
+// filter columns (buffer loads take it; a double word that would cross the end of the descriptor's range
+// reads as zero, so no load here may do that). A group in an image row outside the input is not fetched. The
+// one element per row that reads the padding left or right of the image belongs to the row's first / last
+// group: that group is fetched through the centre tap's position, moved one element up / down in registers,
+// and zero enters at the free end - so no load reaches below the first or past the last element of a plane.
+// G = 8 (128-bit loads) or 4 (64-bit); dy, the other operand, comes in groups of GA pixels (GA divides P*Q:
+// a group never leaves its sample).
+template <int G> struct PixVec;
+template <> struct PixVec<8> {
+    typedef uintx4 type;
+    static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, int voff) {
+        return __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
+    }
+    // element e of the result = element e+1 of v where `edge`, the last one zero
+    static __device__ __forceinline__ type down(type v, bool edge) {
+        const unsigned sh = edge ? 16u : 0u;
+        type o;
+        o.x = __builtin_amdgcn_alignbit(v.y, v.x, sh); o.y = __builtin_amdgcn_alignbit(v.z, v.y, sh);
+        o.z = __builtin_amdgcn_alignbit(v.w, v.z, sh); o.w = __builtin_amdgcn_alignbit(0u, v.w, sh);
+        return o;
+    }
+    // element e of the result = element e-1 of v where `edge`, the first one zero
+    static __device__ __forceinline__ type up(type v, bool edge) {
+        type o;
+        o.w = edge ? __builtin_amdgcn_alignbit(v.w, v.z, 16u) : v.w; o.z = edge ? __builtin_amdgcn_alignbit(v.z, v.y, 16u) : v.z;
+        o.y = edge ? __builtin_amdgcn_alignbit(v.y, v.x, 16u) : v.y; o.x = edge ? v.x << 16 : v.x;
+        return o;
+    }
+};
+template <> struct PixVec<4> {
+    typedef uintx2 type;
+    static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, int voff) {
+        return __builtin_bit_cast(uintx2, __builtin_amdgcn_raw_buffer_load_b64(r, voff, 0, 0));
+    }
+    static __device__ __forceinline__ type down(type v, bool edge) {
+        const unsigned sh = edge ? 16u : 0u;
+        type o;
+        o.x = __builtin_amdgcn_alignbit(v.y, v.x, sh); o.y = __builtin_amdgcn_alignbit(0u, v.y, sh);
+        return o;
+    }
+    static __device__ __forceinline__ type up(type v, bool edge) {
+        type o;
+        o.y = edge ? __builtin_amdgcn_alignbit(v.y, v.x, 16u) : v.y; o.x = edge ? v.x << 16 : v.x;
+        return o;
+    }
+};
+
+// dy as A[k][(n,p,q)]: thread t fetches pixel group t % (32/GA) of rows t / (32/GA) + (8*GA)*i.
+template <int GA>
+struct LoadDyRedVecH {
+    const bf16_t* dy;
+    int N, K, PQ;
+    int kchunk, Ktot;
+    static constexpr int PG = KH / GA; // pixel groups of a slice
+    static constexpr int RL = NT / PG; // rows one load instruction of the workgroup covers
+    typedef typename PixVec<GA>::type V;
+    template <int T> struct Regs { V v[T / RL]; };
+    template <int T> struct State { int mrow[T / RL]; int pq, off; __amdgpu_buffer_rsrc_t rsrc; };
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int row0, int tid, int, int k_begin) const {
+        const int n_first = k_begin / PQ;
+        int k_last = k_begin + kchunk; if (k_last > Ktot) k_last = Ktot;
+        const int n_last = k_last > k_begin ? (k_last - 1) / PQ : n_first;
+        st.rsrc = make_rsrc(dy + (long)n_first * K * PQ, clamp_range((long)(n_last - n_first + 1) * K * PQ * 2));
+        const int kk = k_begin + GA * (tid % PG);
+        const int n = kk / PQ;
+        st.pq = kk - n * PQ;
+        st.off = (int)(((long)(n - n_first) * K * PQ + st.pq) * 2);
+#pragma unroll
+        for (int i = 0; i < T / RL; i++) { const int m = row0 + tid / PG + RL * i; st.mrow[i] = m < K ? m * PQ * 2 : SENT; }
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int, int, int, Regs<T>& r) const {
+#pragma unroll
+        for (int i = 0; i < T / RL; i++) r.v[i] = PixVec<GA>::load(st.rsrc, st.mrow[i] + st.off);
+        st.pq += KH;
+        const bool wrap = st.pq >= PQ;
+        st.pq -= wrap ? PQ : 0;
+        st.off += wrap ? (KH + (K - 1) * PQ) * 2 : KH * 2;
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(unsigned short* lds, int tid, const Regs<T>& r) {
+#pragma unroll
+        for (int i = 0; i < T / RL; i++) *(V*)(lds + (tid / PG + RL * i) * HSTRIDE + GA * (tid % PG)) = r.v[i];
+    }
+};
+
+// im2col operand in tap-major column order, B[(tap, c)][(n,p,q)]: thread t fetches pixel group t % (32/G) of the
+// columns t / (32/G) + (8*G)*i. The columns of one load instruction share a tap (T/NTAP is a multiple of 8*G), so
+// the tap's row and column are wave-uniform and select the code path.
+template <int NTAP, int G>
+struct LoadIm2colRedTapVecH {
+    const bf16_t* x;
+    int N, C, H, W;
+    int ncols; // 9*C
+    int kchunk, Ktot;
+    FastDiv divC;
+    static constexpr int PG = KH / G;
+    static constexpr int CL = NT / PG; // columns one load instruction of the workgroup covers
+    typedef typename PixVec<G>::type V;
+    // as fetched; the move of a row's first / last group waits until the values are stored, so that a slice's
+    // loads are all issued before any of them is waited for
+    template <int T> struct Regs { V v[T / CL]; bool edge[T / CL]; int ts[T / CL]; };
+    template <int T> struct State {
+        int p0, q0; // output row / column of the group's first pixel
+        int pos;    // byte offset of input element (p0, q0) of channel 0 in the group's sample, from the descriptor's base
+        int coloff[T / CL]; // + the column's channel plane and its tap's shift; SENT past the last column
+        int tr[T / CL], ts[T / CL]; // the load's filter row / column (wave-uniform)
+        __amdgpu_buffer_rsrc_t rsrc;
+    };
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int j0, int tid, int, int k_begin) const {
+        static_assert((T / NTAP) % CL == 0, "the columns of one load share a tap");
+        const int PQ = H * W;
+        const long chw = (long)C * PQ;
+        const int n_first = k_begin / PQ;
+        int k_last = k_begin + kchunk; if (k_last > Ktot) k_last = Ktot;
+        const int n_last = k_last > k_begin ? (k_last - 1) / PQ : n_first;
+        st.rsrc = make_rsrc(x + (long)n_first * chw, clamp_range((long)(n_last - n_first + 1) * chw * 2));
+        const int kk = k_begin + G * (tid % PG);
+        const int n = kk / PQ, pq = kk - n * PQ;
+        st.p0 = pq / W; st.q0 = pq - st.p0 * W;
+        st.pos = (int)(((long)(n - n_first) * chw + pq) * 2);
+#pragma unroll
+        for (int i = 0; i < T / CL; i++) {
+            const int jl = j0 + CL * i;             // first column of this load: uniform
+            const int tap = divC.div(jl);
+            const int r = tap / 3, s_ = tap - 3 * r;
+            const int c = jl - tap * C + tid / PG;
+            const bool valid = jl < ncols;
+            st.tr[i] = valid ? r : 1; st.ts[i] = valid ? s_ : 1;
+            st.coloff[i] = valid ? (c * PQ + (r - 1) * W + (s_ - 1)) * 2 : SENT;
+        }
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int, int, int, Regs<T>& r) const {
+#pragma unroll
+        for (int i = 0; i < T / CL; i++) {
+            const int tr = __builtin_amdgcn_readfirstlane(st.tr[i]), ts = __builtin_amdgcn_readfirstlane(st.ts[i]);
+            const bool row_ok = (unsigned)(st.p0 + tr - 1) < (unsigned)H;
+            const int at = st.pos + st.coloff[i];
+            // the group that holds the row's padded element is fetched through the centre tap's position
+            const bool edge = st.q0 == (ts == 0 ? 0 : W - G) && ts != 1;
+            r.v[i] = PixVec<G>::load(st.rsrc, row_ok ? at + (edge ? 2 - 2 * ts : 0) : OOB);
+            r.edge[i] = edge; r.ts[i] = ts;
+        }
+        // next slice: KH pixels further (W >= G; rows of fewer than KH pixels wrap more than once)
+        st.q0 += KH; st.pos += KH * 2;
+#pragma unroll
+        for (int w = 0; w < 3; w++) {
+            const bool wrap = st.q0 >= W;
+            st.q0 -= wrap ? W : 0; st.p0 += wrap ? 1 : 0;
+        }
+        const bool next = st.p0 >= H;
+        st.p0 -= next ? H : 0;
+        st.pos += next ? (C - 1) * H * W * 2 : 0;
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(unsigned short* lds, int tid, const Regs<T>& r) {
+#pragma unroll
+        for (int i = 0; i < T / CL; i++) {
+            const int ts = __builtin_amdgcn_readfirstlane(r.ts[i]);
+            const V v = ts == 0 ? PixVec<G>::up(r.v[i], r.edge[i]) : (ts == 2 ? PixVec<G>::down(r.v[i], r.edge[i]) : r.v[i]);
+            *(V*)(lds + (tid / PG + CL * i) * HSTRIDE + G * (tid % PG)) = v;
+        }
+    }
+};
+
 } // namespace vdnn
 
 namespace vdnn {

@@ -1,0 +1,234 @@
+// Backward filter of 3x3 / stride 1 / padding 1 layers with bfloat16 activations whose image rows are whole
+// groups of four pixels and whose planes are whole groups of eight (W % 4 == 0, W >= 16, H*W % 8 == 0, C % 64 == 0).
+//
+//   dW[k][c][r][s] = sum over (n,p,q) of dy[n,k,p,q] * x[n,c,p+r-1,q+s-1]
+//
+// The reduction runs over output pixels; dy and x both have it contiguous in memory, and through tap (r, s)
+// pixel j of a sample meets element j + (r-1)*W + (s-1) of the input plane: the three taps of a filter row read
+// the same run of the plane one element apart. The general engine gives every (tap, 128 channels) a tile of
+// its own, which fetches dy and its shifted copy of x again - it is bound by the number of global loads. Here a
+// workgroup owns one filter row r, 64 input channels and TM output channels:
+//   * per 32-pixel slice it fetches dy (TM rows) and x (64 rows, the run shifted by (r-1)*W) with aligned
+//     128-bit loads, eight pixels per lane, straight into reduction-major LDS rows - and two more elements per
+//     channel, the one before and the one after the run (rows of the image outside the input are not fetched
+//     and stay zero);
+//   * a wavefront multiplies its WR x 32 block of dy with 32 channels: the fragment of the centre tap is read
+//     from LDS once, the fragments of the left and right tap are that fragment moved by one element in
+//     registers (three funnel shifts shared by both, the element that enters comes from the neighbouring group
+//     or the two extra elements; it is zero where the tap reads the padding left or right of the image).
+// A group of eight pixels never leaves its sample; when W is not a multiple of eight it can hold the last four
+// pixels of one image row and the first four of the next: the two halves are then in or outside the input
+// separately (masked when the group is stored), and the padding is met in the middle of the fragment as well.
+// One LDS fragment and a third of the global loads serve three taps. Accumulators: WR/32 x 3 blocks of 32x32.
+// Partial sums of a reduction split go to the staging area in the tap-major order that reduce_splits_tap sums.
+#pragma once
+#include "mfma_bf16.h"
+
+namespace vdnn {
+
+constexpr int WG3_CH = 64; // input channels of a workgroup's tile
+
+struct Wgrad3x3 {
+    const bf16_t* dy;
+    const bf16_t* x;
+    int N, K, C, H, W;
+    float* out;          // filter gradient target [K][C][3][3]
+    float* partial;      // staging area: [split][K][9*C], column = tap*C + c
+    long partial_stride; // K*9*C
+    float alpha;
+    int accumulate;
+};
+
+// d.M = K, d.N = 9*C, d.K = N*H*W; d.mtiles tiles of 2*WR output channels, d.ntiles = 3 * C/64 (filter row
+// fastest), d.splits reduction splits of d.kchunk pixels (a multiple of 32).
+// HALFROW: the general variant - W not a multiple of eight (groups that hold the end of one image row and the start of
+// the next) or shorter than a slice (two row wraps per slice); without it W % 8 == 0 and W >= 32.
+template <int WR, bool HALFROW>
+__global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, const GemmDims d) {
+    constexpr int TM = 2 * WR, RB = WR / 32, AL = TM / 64;
+    __shared__ __attribute__((aligned(16))) unsigned short As[2][TM * HSTRIDE];
+    __shared__ __attribute__((aligned(16))) unsigned short Bs[2][WG3_CH * HSTRIDE];
+    __shared__ unsigned short Hs[2][2][WG3_CH]; // [buffer][before / after the run][channel]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lk = lane >> 5;
+    const int ntiles_all = d.mtiles * d.ntiles;
+    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int tile = bid % ntiles_all, ks = bid / ntiles_all;
+    const int mt = tile % d.mtiles, nt = tile / d.mtiles;
+    const int r = nt % 3, c0 = (nt / 3) * WG3_CH;
+    const int m0 = mt * TM;
+    const int k_begin = ks * d.kchunk;
+    const int k_end = min(d.K, k_begin + d.kchunk);
+    const int H = g.H, W = g.W, PQ = H * W;
+
+    const int n_first = k_begin / PQ;
+    const int n_last = k_end > k_begin ? (k_end - 1) / PQ : n_first;
+    const __amdgpu_buffer_rsrc_t rsA = make_rsrc(g.dy + (long)n_first * g.K * PQ, clamp_range((long)(n_last - n_first + 1) * g.K * PQ * 2));
+    const __amdgpu_buffer_rsrc_t rsB = make_rsrc(g.x + (long)n_first * g.C * PQ, clamp_range((long)(n_last - n_first + 1) * g.C * PQ * 2));
+
+    // loader state: this thread's pixel group of the slice (eight pixels) and its row of the operands
+    const int pg = tid & 3, rl = tid >> 2;
+    int mrow[AL];
+#pragma unroll
+    for (int i = 0; i < AL; i++) { const int m = m0 + rl + 64 * i; mrow[i] = m < g.K ? m * PQ * 2 : SENT; }
+    int pqA, offA, pB, qB, posB;
+    {
+        const int kk = k_begin + 8 * pg;
+        const int n = kk / PQ, pq = kk - n * PQ;
+        pqA = pq;
+        offA = (int)(((long)(n - n_first) * g.K * PQ + pq) * 2);
+        pB = pq / W; qB = pq - pB * W;
+        posB = (int)(((long)(n - n_first) * g.C * PQ + pq) * 2);
+    }
+    const int colB = ((c0 + rl) * PQ + (r - 1) * W) * 2; // the channel's plane and the filter row's shift
+    // wavefronts 0 and 1 also fetch the element before (after) the slice's run, one channel per lane
+    const int side = wave & 1;
+    int pH, qH, posH;
+    {
+        const int kk = k_begin + (side ? 24 : 0); // the group the element is the neighbour of
+        const int n = kk / PQ, pq = kk - n * PQ;
+        pH = pq / W; qH = pq - pH * W;
+        posH = (int)(((long)(n - n_first) * g.C * PQ + pq) * 2);
+    }
+    const int colH = ((c0 + lane) * PQ + (r - 1) * W) * 2 + (side ? 16 : -2);
+
+    uintx4 ra[AL], rb;
+    unsigned rh = 0, keep_lo = 0, keep_hi = 0;
+    // a group's image row / column / byte offset one slice further: up to two image rows, at most one sample
+    auto advance = [&](int& p, int& q, int& pos) {
+        q += KH; pos += KH * 2;
+#pragma unroll
+        for (int t = 0; t < (HALFROW ? 2 : 1); t++) { // W >= 32 when it is a multiple of eight: one wrap
+            const bool wrap = q >= W;
+            q -= wrap ? W : 0; p += wrap ? 1 : 0;
+        }
+        const bool next = p >= H;
+        p -= next ? H : 0; pos += next ? (g.C - 1) * PQ * 2 : 0;
+    };
+    auto fetch = [&]() {
+#pragma unroll
+        for (int i = 0; i < AL; i++) ra[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(rsA, mrow[i] + offA, 0, 0));
+        pqA += KH;
+        const bool wrapA = pqA >= PQ;
+        pqA -= wrapA ? PQ : 0;
+        offA += wrapA ? (KH + (g.K - 1) * PQ) * 2 : KH * 2;
+
+        {
+            const bool lo_ok = (unsigned)(pB + r - 1) < (unsigned)H;                 // the row of the group's first pixel
+            const bool hi_ok = (HALFROW && qB == W - 4) ? (unsigned)(pB + r) < (unsigned)H : lo_ok; // its last four may be in the next row
+            // only the last four inside (the image's first row through the upper filter row): fetched from there on, so that
+            // the load does not begin below the first element of the plane - and of the descriptor, where all of it reads zero
+            const bool late = hi_ok & !lo_ok;
+            rb = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(rsB, (lo_ok | hi_ok) ? posB + colB + (late ? 8 : 0) : OOB, 0, 0));
+            keep_lo = lo_ok ? ~0u : 0u; keep_hi = hi_ok ? ~0u : 0u;
+        }
+        advance(pB, qB, posB);
+
+        if (wave < 2) {
+            // the neighbour of the slice's first (last) group, in the image row of that group's first (last) pixel; not
+            // fetched where the tap reads the padding there
+            const int prow = pH + r - 1 + ((HALFROW && side && qH == W - 4) ? 1 : 0);
+            const bool used = (unsigned)prow < (unsigned)H && qH != (side ? W - 8 : 0);
+            rh = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsB, used ? posH + colH : OOB, 0, 0);
+            advance(pH, qH, posH);
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < AL; i++) *(uintx4*)(As[buf] + (rl + 64 * i) * HSTRIDE + 8 * pg) = ra[i];
+        uintx4 v = rb; // a group outside the input was not fetched: zero
+        if (HALFROW) {
+            const bool late = (keep_hi & ~keep_lo) != 0u;
+            v.x = rb.x & keep_lo; v.y = rb.y & keep_lo;
+            v.z = (late ? rb.x : rb.z) & keep_hi; v.w = (late ? rb.y : rb.w) & keep_hi;
+        }
+        *(uintx4*)(Bs[buf] + rl * HSTRIDE + 8 * pg) = v;
+        if (wave < 2) Hs[buf][side][lane] = (unsigned short)rh;
+    };
+
+    floatx16 acc[RB][3];
+#pragma unroll
+    for (int i = 0; i < RB; i++)
+#pragma unroll
+        for (int s = 0; s < 3; s++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][s][v] = 0.0f;
+
+    const int wm0 = (wave & 1) * WR, wc0 = (wave >> 1) * 32; // this wavefront's rows of dy and channels
+    int qs = k_begin % W;                                      // image column of the slice's first pixel
+
+    const int nslices = (k_end - k_begin + KH - 1) / KH;
+    fetch();
+    stash(0);
+    fetch();
+    __syncthreads();
+    for (int s = 0; s < nslices; s++) {
+        const int cur = s & 1;
+        const unsigned short* arow = As[cur] + (wm0 + l32) * HSTRIDE + 8 * lk;
+        const unsigned short* brow = Bs[cur] + (wc0 + l32) * HSTRIDE + 8 * lk;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            bf16x8 a[RB];
+#pragma unroll
+            for (int i = 0; i < RB; i++) a[i] = *(const bf16x8*)(arow + i * 32 * HSTRIDE + 16 * h);
+            const uintx4 v = *(const uintx4*)(brow + 16 * h);
+            // the element before / after this lane's eight: in the row unless the lane holds the slice's first / last group
+            const unsigned short* pp = (h == 0 && lk == 0) ? &Hs[cur][0][wc0 + l32] : brow + 16 * h - 1;
+            const unsigned short* np = (h == 1 && lk == 1) ? &Hs[cur][1][wc0 + l32] : brow + 16 * h + 8;
+            unsigned prev = *pp, next = *np;
+            int qg = qs + 16 * h + 8 * lk;
+            qg -= qg >= W ? W : 0;
+            if (HALFROW) qg -= qg >= W ? W : 0;
+            prev = qg == 0 ? 0u : prev;     // left of the image
+            next = qg == W - 8 ? 0u : next; // right of the image
+            const bool mid = HALFROW && qg == W - 4; // pixels 4.. of the eight begin an image row
+            const unsigned t1 = __builtin_amdgcn_alignbit(v.y, v.x, 16u), t2 = __builtin_amdgcn_alignbit(v.z, v.y, 16u),
+                           t3 = __builtin_amdgcn_alignbit(v.w, v.z, 16u);
+            uintx4 up, dn;
+            up.x = (v.x << 16) | prev; up.y = t1; up.z = t2; up.w = t3;
+            dn.x = t1; dn.y = t2; dn.z = t3; dn.w = (next << 16) | (v.w >> 16);
+            if (HALFROW) {
+                up.z &= mid ? 0xFFFF0000u : ~0u; // pixel 4 reads left of the image through the left tap
+                dn.y &= mid ? 0x0000FFFFu : ~0u; // pixel 3 reads right of the image through the right tap
+            }
+            const bf16x8 b0 = __builtin_bit_cast(bf16x8, up), b1 = __builtin_bit_cast(bf16x8, v), b2 = __builtin_bit_cast(bf16x8, dn);
+#pragma unroll
+            for (int i = 0; i < RB; i++) {
+                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b0, acc[i][0], 0, 0, 0);
+                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b1, acc[i][1], 0, 0, 0);
+                acc[i][2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b2, acc[i][2], 0, 0, 0);
+            }
+        }
+        qs += KH;
+        qs -= qs >= W ? W : 0;
+        if (HALFROW) qs -= qs >= W ? W : 0;
+        stash(cur ^ 1);
+        __syncthreads();
+        fetch();
+    }
+
+    // acc[i][s][v]: output channel m0 + wm0 + 32*i + 8*(v/4) + 4*lk + v%4, input channel c0 + wc0 + l32, tap (r, s)
+    const int c = c0 + wc0 + l32;
+    const int ncols = 9 * g.C;
+    const bool to_partial = d.splits > 1;
+#pragma unroll
+    for (int i = 0; i < RB; i++)
+#pragma unroll
+        for (int s = 0; s < 3; s++) {
+            const int tap = 3 * r + s;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = m0 + wm0 + 32 * i + 8 * (v / 4) + 4 * lk + (v % 4);
+                if (m >= g.K || c >= g.C) continue;
+                const float a = acc[i][s][v];
+                if (to_partial) g.partial[(long)ks * g.partial_stride + (long)m * ncols + (long)tap * g.C + c] = a;
+                else {
+                    const long idx = (long)m * ncols + (long)c * 9 + tap;
+                    g.out[idx] = g.accumulate ? __fmaf_rn(g.alpha, a, g.out[idx]) : g.alpha * a;
+                }
+            }
+        }
+}
+
+} // namespace vdnn
