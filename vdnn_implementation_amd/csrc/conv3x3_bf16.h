@@ -262,6 +262,57 @@ __global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH a
         }
     }
 
+    // A whole tile's result leaves through LDS: each wavefront lays its 64 x 64 block out row by row (bias and rectifier
+    // applied, rounded to bfloat16) and writes it eight pixels - 16 bytes - per lane, gated by eight elements of the gate
+    // tensor fetched the same way; lane by lane the block would leave in two-byte stores of 64-byte runs. Same values.
+    // Needs planes of whole groups of eight pixels (a group stays in its sample) and 16-byte aligned tensors.
+    if (whole && ep.opix % 8 == 0 && (((uintptr_t)ep.out | (uintptr_t)ep.gate) & 15) == 0) {
+        static_assert(NJ == 2 && WM == 1, "one 64 x 64 block per wavefront");
+        constexpr int STG = 72; // row stride of the block in LDS, 16-bit units
+        static_assert(4 * 64 * STG <= 2 * W3_ROWS * HSTRIDE, "the four blocks fit the window buffers");
+        __syncthreads(); // every wavefront has read its last fragments
+        unsigned short* stg = &Bw[0][0] + wave * (64 * STG);
+#pragma unroll
+        for (int it = 0; it < 2; it++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+                const int m = m0 + row;
+                const float b = (ep.bias && m < d.M) ? ep.bias[m] : 0.0f;
+#pragma unroll
+                for (int jt = 0; jt < 2; jt++) {
+                    float r = acc[0][it][jt][v];
+                    if (ep.bias) r += b;
+                    if (ep.relu) r = relu_value(r);
+                    stg[row * STG + jt * 32 + l32] = float_to_bf16_bits(r);
+                }
+            }
+        __builtin_amdgcn_wave_barrier(); // the block is read by other lanes of the same wavefront: LDS keeps a wavefront's order
+        const int grp = lane & 7;
+        const int j = j0 + wn0 + 8 * grp;
+        const int n = j / ep.opix, pix = j - n * ep.opix;
+        const size_t base = (size_t)n * d.M * ep.opix + pix;
+        if (j < d.N) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int row = (lane >> 3) + 8 * i;
+                const int m = m0 + row;
+                if (m >= d.M) continue;
+                uintx4 val = *(const uintx4*)(stg + row * STG + 8 * grp);
+                const size_t idx = base + (size_t)m * ep.opix;
+                if (ep.gate) {
+                    // kept where gate > 0: a positive bfloat16 that is not a NaN has bits 0x0001 .. 0x7F80
+                    const uintx4 gv = *(const uintx4*)(ep.gate + idx);
+                    auto keep = [](unsigned w) {
+                        return ((((w & 0xFFFFu) - 1u) < 0x7F80u) ? 0x0000FFFFu : 0u) | ((((w >> 16) - 1u) < 0x7F80u) ? 0xFFFF0000u : 0u);
+                    };
+                    val.x &= keep(gv.x); val.y &= keep(gv.y); val.z &= keep(gv.z); val.w &= keep(gv.w);
+                }
+                *(uintx4*)(ep.out + idx) = val;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int q = 0; q < NJ / 2; q++) {
         if (StoreNCHW<bf16_t>::TAIL && d.full_tiles > 0 && !whole)
