@@ -67,6 +67,11 @@ CONV_RANDOM = [
     (2, 4, 17, 19, 8, 3, 3, 1, 1, 2, 2),       # four input channels, strided: the vector-ALU filter gradient
     (3, 1, 9, 9, 12, 3, 3, 0, 0, 1, 1),        # one input channel, no padding
     (7, 3, 40, 36, 16, 3, 3, 1, 1, 1, 1),      # three input channels, several pixel chunks per sample
+    # backward filter with one filter row and 64 input channels per workgroup (3x3, stride 1, padding 1, W % 4 == 0, C % 64 == 0)
+    (2, 64, 4, 16, 64, 3, 3, 1, 1, 1, 1),      # 64-row tile, one reduction split (results stored directly), rows one slice long
+    (7, 128, 6, 20, 192, 3, 3, 1, 1, 1, 1),    # two channel blocks, a ragged second row tile, splits that straddle samples, slices that straddle rows
+    (3, 64, 56, 56, 130, 3, 3, 1, 1, 1, 1),    # VGG-sized rows; two rows in the last tile
+    (3, 64, 6, 28, 96, 3, 3, 1, 1, 1, 1),      # plane not a multiple of the slice: slices straddle samples
 ]
 
 

@@ -13,6 +13,7 @@
 #include "mfma_bf16.h"
 #include "conv3x3_bf16.h"
 #include "wgrad3x3_bf16.h"
+#include "wgrad3x3_f32.h"
 #include "conv_smallc.h"
 
 namespace vdnn {
@@ -71,6 +72,7 @@ static const PassNames kFwdWin3Names{"conv_fwd_bf16win_64x256", "conv_fwd_bf16wi
 static const PassNames kBwdDataWin3Names{"conv_bwd_data_bf16win_64x256", "conv_bwd_data_bf16win_64x256"};
 static const PassNames kBwdFilterHalfNames{"conv_bwd_filter_bf16mfma_64x256", "conv_bwd_filter_bf16mfma_128x128"};
 static const PassNames kBwdFilterWin3Names{"conv_bwd_filter_bf16win_64x192", "conv_bwd_filter_bf16win_128x192"};
+static const PassNames kBwdFilterRow3Names{"conv_bwd_filter_row_64x192", "conv_bwd_filter_row_128x192"};
 
 template <int TM, int TN, class AL, class BL, class EP, bool HALF = false>
 static int launch_igemm(vdnn_ctx* ctx, hipStream_t stream, const char* name, const AL& al, const BL& bl, const EP& ep, const GemmDims& d, double flops = 0.0) {
@@ -364,6 +366,53 @@ static int launch_wgrad3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, cons
         else if (narrow) hipLaunchKernelGGL((wgrad3x3_bf16_kernel<32, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
         else if (halfrow) hipLaunchKernelGGL((wgrad3x3_bf16_kernel<64, true>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
         else hipLaunchKernelGGL((wgrad3x3_bf16_kernel<64, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        VDNN_LAUNCH_CHECK();
+    }
+    if (d.splits > 1) return launch_reduce_splits_tap(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, accumulate, g.C, 9);
+    return VDNN_OK;
+}
+
+// Workgroups of wgrad3x3_f32_kernel that are resident on a compute unit (by its registers).
+constexpr int kWgrad3FPerCU = 2;
+
+static bool wgrad3x3_f32_ok(const ConvGeo& g) {
+    return g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W &&
+           g.W % 4 == 0 && g.W >= KB && g.C % WG3F_CH == 0; // a slice wraps at most one image row
+}
+
+// The float counterpart of launch_wgrad3x3.
+static int launch_wgrad3x3_f32(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const float* x, const float* dy, float* w, float alpha, int accumulate,
+                               float* staging, size_t staging_bytes, bool* taken) {
+    *taken = false;
+    const int M = g.K, N = g.C * 9, PQ = g.H * g.W;
+    const long Kred = (long)g.N * PQ;
+    const bool narrow = M <= 64;
+    const int TM = narrow ? 64 : 128;
+    const int mtiles = (M + TM - 1) / TM, ntiles = 3 * (g.C / WG3F_CH);
+    const long tiles = (long)mtiles * ntiles;
+    const size_t out_bytes = (size_t)M * N * sizeof(float);
+    const long slots = (long)kWgrad3FPerCU * ctx->num_cu;
+    // as many rounds of workgroups as the tiles alone need, each filled by the splits
+    const long rounds = (tiles + slots - 1) / slots;
+    long splits = rounds * slots / tiles;
+    const long by_len = Kred / (8 * KB); // at least eight slices per split
+    const long by_mem = staging ? (long)(staging_bytes / out_bytes) : 1;
+    if (splits > by_len) splits = by_len;
+    if (splits > by_mem) splits = by_mem;
+    if (splits < 1) splits = 1;
+    GemmDims d = make_dims(M, N, (int)Kred, TM, 3 * WG3F_CH, (int)splits, KB);
+    d.mtiles = mtiles; d.ntiles = ntiles;
+    const long nspan = d.kchunk / PQ + 2;
+    if (nspan * g.K * PQ * 4 >= (long)MAX_SUM_RANGE || nspan * g.C * PQ * 4 >= (long)MAX_SUM_RANGE) return VDNN_OK; // not taken
+    if (d.splits > 1 && !staging) return VDNN_OK;
+    const long blocks = tiles * d.splits;
+    if (blocks <= 0 || blocks >= (1l << 31)) return VDNN_OK;
+    *taken = true;
+    const Wgrad3x3F geo{dy, x, g.N, g.K, g.C, g.H, g.W, w, staging, (long)M * N, alpha, accumulate};
+    {
+        ProfScope prof(ctx, st, narrow ? kBwdFilterRow3Names.t64 : kBwdFilterRow3Names.t128, 2.0 * M * (double)N * (double)Kred, 0.0);
+        if (narrow) hipLaunchKernelGGL((wgrad3x3_f32_kernel<32>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        else hipLaunchKernelGGL((wgrad3x3_f32_kernel<64>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
         VDNN_LAUNCH_CHECK();
     }
     if (d.splits > 1) return launch_reduce_splits_tap(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, accumulate, g.C, 9);
@@ -688,6 +737,14 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
                 if (dh.splits > 1) return launch_reduce_splits_tap(ctx, st, w, staging, (size_t)M * N, dh.splits, alpha, accumulate, g.C, RS);
                 return VDNN_OK;
             }
+        }
+    }
+    if constexpr (sizeof(E) == 4) {
+        // 3x3, stride 1, padding 1: one filter row and 64 input channels per workgroup, one fetch for three taps
+        if (wgrad3x3_f32_ok(g) && aligned16(dy) && aligned16(x)) {
+            bool taken = false;
+            const int rcw = launch_wgrad3x3_f32(ctx, st, g, x, dy, w, alpha, accumulate, staging, staging_bytes, &taken);
+            if (taken || rcw != VDNN_OK) return rcw;
         }
     }
     if (vec && ntap != 0 && PQ >= KB && 2 * g.Q >= KB) {

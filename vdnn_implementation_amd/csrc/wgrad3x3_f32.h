@@ -1,0 +1,217 @@
+// Backward filter of 3x3 / stride 1 / padding 1 layers with float activations whose image rows are whole groups of
+// four pixels (W % 4 == 0, W >= 16, C % 64 == 0). The float counterpart of wgrad3x3_bf16_kernel:
+//
+//   dW[k][c][r][s] = sum over (n,p,q) of dy[n,k,p,q] * x[n,c,p+r-1,q+s-1]
+//
+// Through tap (r, s) pixel j of a sample meets element j + (r-1)*W + (s-1) of the input plane. A workgroup owns one
+// filter row r, 64 input channels and TM output channels; per 16-pixel slice it fetches dy (TM rows) and one run of x
+// (64 rows, shifted by (r-1)*W) with 128-bit loads, four pixels per lane, into reduction-major LDS rows, plus the
+// element before and the one after the run. A lane's four values of the centre tap are one 128-bit LDS read; the left
+// and right tap take the same registers one place apart, the value that enters at the end comes from the neighbouring
+// group (or the two extra elements) and is zero where the tap reads the padding beside the image. Rows of the image
+// outside the input are not fetched and stay zero. One fetch of dy and of x serves three taps (the tile-per-tap
+// engine fetches both again for every tap), which halves the requests to L2 per multiply.
+// Accumulators: WR/32 x 3 blocks of 32x32. Partial sums of a reduction split go to the staging area in the
+// tap-major order that reduce_splits_tap sums.
+#pragma once
+#include "mfma_gemm.h"
+
+namespace vdnn {
+
+constexpr int WG3F_CH = 64; // input channels of a workgroup's tile
+
+struct Wgrad3x3F {
+    const float* dy;
+    const float* x;
+    int N, K, C, H, W;
+    float* out;          // filter gradient target [K][C][3][3]
+    float* partial;      // staging area: [split][K][9*C], column = tap*C + c
+    long partial_stride; // K*9*C
+    float alpha;
+    int accumulate;
+};
+
+// d.M = K, d.N = 9*C, d.K = N*H*W; d.mtiles tiles of 2*WR output channels, d.ntiles = 3 * C/64 (filter row
+// fastest), d.splits reduction splits of d.kchunk pixels (a multiple of 16).
+template <int WR>
+__global__ void __launch_bounds__(NT) wgrad3x3_f32_kernel(const Wgrad3x3F g, const GemmDims d) {
+    constexpr int TM = 2 * WR, RB = WR / 32, AL = TM / 64;
+    __shared__ __attribute__((aligned(16))) float As[2][TM * RED_STRIDE];
+    __shared__ __attribute__((aligned(16))) float Bs[2][WG3F_CH * RED_STRIDE];
+    __shared__ float Hs[2][2][WG3F_CH]; // [buffer][before / after the run][channel]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lk = lane >> 5;
+    const int ntiles_all = d.mtiles * d.ntiles;
+    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int tile = bid % ntiles_all, ks = bid / ntiles_all;
+    const int mt = tile % d.mtiles, nt = tile / d.mtiles;
+    const int r = nt % 3, c0 = (nt / 3) * WG3F_CH;
+    const int m0 = mt * TM;
+    const int k_begin = ks * d.kchunk;
+    const int k_end = min(d.K, k_begin + d.kchunk);
+    const int H = g.H, W = g.W, PQ = H * W;
+
+    const int n_first = k_begin / PQ;
+    const int n_last = k_end > k_begin ? (k_end - 1) / PQ : n_first;
+    const __amdgpu_buffer_rsrc_t rsA = make_rsrc(g.dy + (long)n_first * g.K * PQ, clamp_range((long)(n_last - n_first + 1) * g.K * PQ * 4));
+    const __amdgpu_buffer_rsrc_t rsB = make_rsrc(g.x + (long)n_first * g.C * PQ, clamp_range((long)(n_last - n_first + 1) * g.C * PQ * 4));
+
+    // loader state: this thread's pixel group of the slice (four pixels) and its row of the operands
+    const int pg = tid & 3, rl = tid >> 2;
+    int mrow[AL];
+#pragma unroll
+    for (int i = 0; i < AL; i++) { const int m = m0 + rl + 64 * i; mrow[i] = m < g.K ? m * PQ * 4 : SENT; }
+    int pqA, offA, pB, qB, posB;
+    {
+        const int kk = k_begin + 4 * pg;
+        const int n = kk / PQ, pq = kk - n * PQ;
+        pqA = pq;
+        offA = (int)(((long)(n - n_first) * g.K * PQ + pq) * 4);
+        pB = pq / W; qB = pq - pB * W;
+        posB = (int)(((long)(n - n_first) * g.C * PQ + pq) * 4);
+    }
+    const int colB = ((c0 + rl) * PQ + (r - 1) * W) * 4; // the channel's plane and the filter row's shift
+    // wavefronts 0 and 1 also fetch the element before (after) the slice's run, one channel per lane
+    const int side = wave & 1;
+    int pH, qH, posH;
+    {
+        const int kk = k_begin + (side ? 12 : 0); // the group the element is the neighbour of
+        const int n = kk / PQ, pq = kk - n * PQ;
+        pH = pq / W; qH = pq - pH * W;
+        posH = (int)(((long)(n - n_first) * g.C * PQ + pq) * 4);
+    }
+    const int colH = ((c0 + lane) * PQ + (r - 1) * W) * 4 + (side ? 16 : -4);
+
+    floatx4 ra[AL], rb;
+    float rh = 0.0f;
+    // a group's image row / column / byte offset one slice further: W >= 16, one row wrap; at most one sample
+    auto advance = [&](int& p, int& q, int& pos) {
+        q += KB; pos += KB * 4;
+        const bool wrap = q >= W;
+        q -= wrap ? W : 0; p += wrap ? 1 : 0;
+        const bool next = p >= H;
+        p -= next ? H : 0; pos += next ? (g.C - 1) * PQ * 4 : 0;
+    };
+    auto fetch = [&]() {
+#pragma unroll
+        for (int i = 0; i < AL; i++) ra[i] = buf_load4(rsA, mrow[i] + offA, 0);
+        pqA += KB;
+        const bool wrapA = pqA >= PQ;
+        pqA -= wrapA ? PQ : 0;
+        offA += wrapA ? (KB + (g.K - 1) * PQ) * 4 : KB * 4;
+
+        const bool row_ok = (unsigned)(pB + r - 1) < (unsigned)H;
+        rb = buf_load4(rsB, row_ok ? posB + colB : OOB, 0);
+        advance(pB, qB, posB);
+
+        if (wave < 2) {
+            // not fetched where the tap reads the padding (the element would belong to another image row)
+            const bool used = (unsigned)(pH + r - 1) < (unsigned)H && qH != (side ? W - 4 : 0);
+            rh = buf_load(rsB, used ? posH + colH : OOB, 0);
+            advance(pH, qH, posH);
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < AL; i++) *(floatx4*)(As[buf] + (rl + 64 * i) * RED_STRIDE + 4 * pg) = ra[i];
+        *(floatx4*)(Bs[buf] + rl * RED_STRIDE + 4 * pg) = rb;
+        if (wave < 2) Hs[buf][side][lane] = rh;
+    };
+
+    floatx16 acc[RB][3];
+#pragma unroll
+    for (int i = 0; i < RB; i++)
+#pragma unroll
+        for (int s = 0; s < 3; s++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][s][v] = 0.0f;
+
+    const int wm0 = (wave & 1) * WR, wc0 = (wave >> 1) * 32; // this wavefront's rows of dy and channels
+    int qs = k_begin % W;                                      // image column of the slice's first pixel
+
+    // fragments of half hf (pixels 8 hf .. 8 hf + 7) of the slice in buffer `buf` whose first pixel has image column q0:
+    // a lane holds pixels 8 hf + 4 lk .. + 3 of its row / channel, and the elements before and after them
+    struct Frag { floatx4 a[RB]; floatx4 v; float prev, next; };
+    auto read = [&](int buf, int hf, int q0, Frag& f) {
+        const float* arow = As[buf] + (wm0 + l32) * RED_STRIDE + 8 * hf + 4 * lk;
+        const float* brow = Bs[buf] + (wc0 + l32) * RED_STRIDE + 8 * hf + 4 * lk;
+#pragma unroll
+        for (int i = 0; i < RB; i++) f.a[i] = *(const floatx4*)(arow + i * 32 * RED_STRIDE);
+        f.v = *(const floatx4*)brow;
+        const float* pp = (hf == 0 && lk == 0) ? &Hs[buf][0][wc0 + l32] : brow - 1;
+        const float* np = (hf == 1 && lk == 1) ? &Hs[buf][1][wc0 + l32] : brow + 4;
+        const float prev = *pp, next = *np;
+        int qg = q0 + 8 * hf + 4 * lk;
+        qg -= qg >= W ? W : 0;
+        f.prev = qg == 0 ? 0.0f : prev;     // left of the image
+        f.next = qg == W - 4 ? 0.0f : next; // right of the image
+    };
+    auto multiply = [&](const Frag& f) {
+        const float up[4] = {f.prev, f.v.x, f.v.y, f.v.z};
+        const float ce[4] = {f.v.x, f.v.y, f.v.z, f.v.w};
+        const float dn[4] = {f.v.y, f.v.z, f.v.w, f.next};
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int i = 0; i < RB; i++) {
+                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[i][e], up[e], acc[i][0], 0, 0, 0);
+                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[i][e], ce[e], acc[i][1], 0, 0, 0);
+                acc[i][2] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[i][e], dn[e], acc[i][2], 0, 0, 0);
+            }
+    };
+
+    // Software pipeline of the tile engine: one barrier per slice, in the middle of it; each half's fragments are read
+    // while the half before is multiplied; a slice's fetch has a full slice of multiplies to return.
+    const int nslices = (k_end - k_begin + KB - 1) / KB;
+    fetch();
+    stash(0);
+    fetch();
+    __syncthreads();
+    Frag f0, f1;
+    read(0, 0, qs, f0);
+    for (int s = 0; s < nslices; s++) {
+        const int cur = s & 1, nxt = cur ^ 1;
+        read(cur, 1, qs, f1);
+        multiply(f0);
+        stash(nxt);
+#pragma unroll
+        for (int i = 0; i < 12 * RB; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x300, 1, 0); }
+        __syncthreads();
+        fetch();
+        qs += KB;
+        qs -= qs >= W ? W : 0;
+        read(nxt, 0, qs, f0);
+        multiply(f1);
+#pragma unroll
+        for (int i = 0; i < 12 * RB; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    }
+
+    // acc[i][s][v]: output channel m0 + wm0 + 32*i + 8*(v/4) + 4*lk + v%4, input channel c0 + wc0 + l32, tap (r, s)
+    const int c = c0 + wc0 + l32;
+    const int ncols = 9 * g.C;
+    const bool to_partial = d.splits > 1;
+#pragma unroll
+    for (int i = 0; i < RB; i++)
+#pragma unroll
+        for (int s = 0; s < 3; s++) {
+            const int tap = 3 * r + s;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = m0 + wm0 + 32 * i + 8 * (v / 4) + 4 * lk + (v % 4);
+                if (m >= g.K || c >= g.C) continue;
+                const float a = acc[i][s][v];
+                if (to_partial) g.partial[(long)ks * g.partial_stride + (long)m * ncols + (long)tap * g.C + c] = a;
+                else {
+                    const long idx = (long)m * ncols + (long)c * 9 + tap;
+                    g.out[idx] = g.accumulate ? __fmaf_rn(g.alpha, a, g.out[idx]) : g.alpha * a;
+                }
+            }
+        }
+}
+
+} // namespace vdnn
