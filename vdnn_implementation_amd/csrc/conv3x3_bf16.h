@@ -134,11 +134,14 @@ __global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH a
         if (q == W - 1) colmask |= 2u << (2 * jt);
     }
 
-    uintx4 wr[2][2];   // [item][pixel of the pair]: eight channels each, ready for LDS
-    unsigned hr = 0;   // the halo element of this lane (wavefront 0)
+    // Two windows are in flight: the one fetched for the row step after the next, and the one for the step after
+    // that. [item][pixel of the pair]: eight channels each, ready for LDS; the halo element of this lane (wavefront 0).
+    struct Fetched { uintx4 wr[2][2]; unsigned hr; };
+    Fetched fa, fb;
+    fa.hr = 0; fb.hr = 0;
     const int g0 = __builtin_amdgcn_readfirstlane(tid >> 7); // channel group of the thread's first item: uniform per wavefront
 
-    auto load_window = [&](int row_step) {
+    auto load_window = [&](int row_step, Fetched& f) {
         const int cb = row_step / 3, r = row_step - cb * 3;
         const int rowoff = MODE == 0 ? (r - 1) * W : (1 - r) * W;
         const int vo = voff | bit_to_all_ones(rowinv, r);
@@ -150,23 +153,23 @@ __global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH a
 #pragma unroll
             for (int e = 0; e < 8; e++) c[e] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rsrc, vo, soff + e * step, 0);
             // 2 x 8 transpose of 16-bit values: the low halves are the first pixel's channels, the high halves the second's
-            wr[i][0].x = __builtin_amdgcn_perm(c[1], c[0], 0x05040100u); wr[i][0].y = __builtin_amdgcn_perm(c[3], c[2], 0x05040100u);
-            wr[i][0].z = __builtin_amdgcn_perm(c[5], c[4], 0x05040100u); wr[i][0].w = __builtin_amdgcn_perm(c[7], c[6], 0x05040100u);
-            wr[i][1].x = __builtin_amdgcn_perm(c[1], c[0], 0x07060302u); wr[i][1].y = __builtin_amdgcn_perm(c[3], c[2], 0x07060302u);
-            wr[i][1].z = __builtin_amdgcn_perm(c[5], c[4], 0x07060302u); wr[i][1].w = __builtin_amdgcn_perm(c[7], c[6], 0x07060302u);
+            f.wr[i][0].x = __builtin_amdgcn_perm(c[1], c[0], 0x05040100u); f.wr[i][0].y = __builtin_amdgcn_perm(c[3], c[2], 0x05040100u);
+            f.wr[i][0].z = __builtin_amdgcn_perm(c[5], c[4], 0x05040100u); f.wr[i][0].w = __builtin_amdgcn_perm(c[7], c[6], 0x05040100u);
+            f.wr[i][1].x = __builtin_amdgcn_perm(c[1], c[0], 0x07060302u); f.wr[i][1].y = __builtin_amdgcn_perm(c[3], c[2], 0x07060302u);
+            f.wr[i][1].z = __builtin_amdgcn_perm(c[5], c[4], 0x07060302u); f.wr[i][1].w = __builtin_amdgcn_perm(c[7], c[6], 0x07060302u);
         }
         if (wave == 0) {
             const int soff = (cb * KH * plane + rowoff + W + 2) * 2;
-            hr = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc, hoff | bit_to_all_ones(hrowinv, r), soff, 0);
+            f.hr = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc, hoff | bit_to_all_ones(hrowinv, r), soff, 0);
         }
     };
-    auto store_window = [&](unsigned short* lds) {
+    auto store_window = [&](unsigned short* lds, const Fetched& f) {
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int e = 0; e < 2; e++)
-                *(uintx4*)(lds + (1 + 2 * (tid & 127) + e) * HSTRIDE + 8 * ((tid >> 7) + 2 * i)) = wr[i][e];
-        if (wave == 0) lds[((lane >> 5) ? W3_ROWS - 1 : 0) * HSTRIDE + (lane & 31)] = (unsigned short)hr;
+                *(uintx4*)(lds + (1 + 2 * (tid & 127) + e) * HSTRIDE + 8 * ((tid >> 7) + 2 * i)) = f.wr[i][e];
+        if (wave == 0) lds[((lane >> 5) ? W3_ROWS - 1 : 0) * HSTRIDE + (lane & 31)] = (unsigned short)f.hr;
     };
 
     floatx16 acc[NJ / 2][2][2]; // [64-column half][row block][column block]
@@ -220,17 +223,20 @@ __global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH a
     };
 
     al.template load<TM>(sa, row_begin * W3_DEPTH, k_end, tid, ra);
-    load_window(row_begin);
+    load_window(row_begin, fa);
     LoadPackedH::template store<TM>(As[0], tid, ra);
-    store_window(Bw[0]);
+    store_window(Bw[0], fa);
     al.template load<TM>(sa, row_begin * W3_DEPTH + KH, k_end, tid, ra);
-    load_window(row_begin + 1);
+    load_window(row_begin + 1, fb);
+    load_window(row_begin + 2, fa);
     __syncthreads();
     bf16x8 a0[2], a1[2];
     uintx4 b0[NJ], b1[NJ];
     read_a(As[0], 0, a0);
     read_b(Bw[0], 0, 0, b0);
-    for (int row_step = row_begin; row_step < row_end; row_step++) {
+    // one row step; `f` holds the window of the next row step (fetched two row steps ago): it is written to LDS in the
+    // first half of the last tap, and the registers then take the fetch of the window three row steps ahead
+    auto row_step_body = [&](int row_step, Fetched& f) {
         const int wb = (row_step - row_begin) & 1;
 #pragma unroll
         for (int s = 0; s < 3; s++) {
@@ -241,13 +247,13 @@ __global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH a
             mask_b(s, b0);
             multiply(a0, b0);
             LoadPackedH::template store<TM>(As[nxt], tid, ra);
-            if (s == 2) store_window(Bw[wb ^ 1]);
+            if (s == 2) store_window(Bw[wb ^ 1], f);
             // issue order of the first half: an LDS access behind every MFMA
 #pragma unroll
             for (int i = 0; i < 2 * NJ; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x300, 2, 0); }
             __syncthreads();
             al.template load<TM>(sa, row_begin * W3_DEPTH + (g + 2) * KH, k_end, tid, ra);
-            if (s == 2) load_window(row_step + 2);
+            if (s == 2) load_window(row_step + 3, f);
             read_a(As[nxt], 0, a0);
             read_b(s == 2 ? Bw[wb ^ 1] : Bw[wb], s == 2 ? 0 : s + 1, 0, b0);
             mask_b(s, b1);
@@ -260,6 +266,10 @@ __global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH a
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             }
         }
+    };
+    for (int row_step = row_begin; row_step < row_end; row_step += 2) {
+        row_step_body(row_step, fb);
+        if (row_step + 1 < row_end) row_step_body(row_step + 1, fa);
     }
 
     // A whole tile's result leaves through LDS: each wavefront lays its 64 x 64 block out row by row (bias and rectifier
