@@ -93,8 +93,10 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
     }
     const int colH = ((c0 + lane) * PQ + (r - 1) * W) * 2 + (side ? 16 : -2);
 
-    uintx4 ra[AL], rb;
-    unsigned rh = 0, keep_lo = 0, keep_hi = 0;
+    // what a slice's fetch leaves in registers; two slices are in flight
+    struct Fetched { uintx4 ra[AL], rb; unsigned rh, keep_lo, keep_hi; };
+    Fetched fa, fb;
+    fa.rh = 0; fb.rh = 0;
     // a group's image row / column / byte offset one slice further: up to two image rows, at most one sample
     auto advance = [&](int& p, int& q, int& pos) {
         q += KH; pos += KH * 2;
@@ -106,9 +108,9 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
         const bool next = p >= H;
         p -= next ? H : 0; pos += next ? (g.C - 1) * PQ * 2 : 0;
     };
-    auto fetch = [&]() {
+    auto fetch = [&](Fetched& f) {
 #pragma unroll
-        for (int i = 0; i < AL; i++) ra[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(rsA, mrow[i] + offA, 0, 0));
+        for (int i = 0; i < AL; i++) f.ra[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(rsA, mrow[i] + offA, 0, 0));
         pqA += KH;
         const bool wrapA = pqA >= PQ;
         pqA -= wrapA ? PQ : 0;
@@ -120,8 +122,8 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
             // only the last four inside (the image's first row through the upper filter row): fetched from there on, so that
             // the load does not begin below the first element of the plane - and of the descriptor, where all of it reads zero
             const bool late = hi_ok & !lo_ok;
-            rb = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(rsB, (lo_ok | hi_ok) ? posB + colB + (late ? 8 : 0) : OOB, 0, 0));
-            keep_lo = lo_ok ? ~0u : 0u; keep_hi = hi_ok ? ~0u : 0u;
+            f.rb = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(rsB, (lo_ok | hi_ok) ? posB + colB + (late ? 8 : 0) : OOB, 0, 0));
+            f.keep_lo = lo_ok ? ~0u : 0u; f.keep_hi = hi_ok ? ~0u : 0u;
         }
         advance(pB, qB, posB);
 
@@ -130,21 +132,21 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
             // fetched where the tap reads the padding there
             const int prow = pH + r - 1 + ((HALFROW && side && qH == W - 4) ? 1 : 0);
             const bool used = (unsigned)prow < (unsigned)H && qH != (side ? W - 8 : 0);
-            rh = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsB, used ? posH + colH : OOB, 0, 0);
+            f.rh = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsB, used ? posH + colH : OOB, 0, 0);
             advance(pH, qH, posH);
         }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](int buf, const Fetched& f) {
 #pragma unroll
-        for (int i = 0; i < AL; i++) *(uintx4*)(As[buf] + (rl + 64 * i) * HSTRIDE + 8 * pg) = ra[i];
-        uintx4 v = rb; // a group outside the input was not fetched: zero
+        for (int i = 0; i < AL; i++) *(uintx4*)(As[buf] + (rl + 64 * i) * HSTRIDE + 8 * pg) = f.ra[i];
+        uintx4 v = f.rb; // a group outside the input was not fetched: zero
         if (HALFROW) {
-            const bool late = (keep_hi & ~keep_lo) != 0u;
-            v.x = rb.x & keep_lo; v.y = rb.y & keep_lo;
-            v.z = (late ? rb.x : rb.z) & keep_hi; v.w = (late ? rb.y : rb.w) & keep_hi;
+            const bool late = (f.keep_hi & ~f.keep_lo) != 0u;
+            v.x = f.rb.x & f.keep_lo; v.y = f.rb.y & f.keep_lo;
+            v.z = (late ? f.rb.x : f.rb.z) & f.keep_hi; v.w = (late ? f.rb.y : f.rb.w) & f.keep_hi;
         }
         *(uintx4*)(Bs[buf] + rl * HSTRIDE + 8 * pg) = v;
-        if (wave < 2) Hs[buf][side][lane] = (unsigned short)rh;
+        if (wave < 2) Hs[buf][side][lane] = (unsigned short)f.rh;
     };
 
     floatx16 acc[RB][3];
@@ -159,11 +161,14 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
     int qs = k_begin % W;                                      // image column of the slice's first pixel
 
     const int nslices = (k_end - k_begin + KH - 1) / KH;
-    fetch();
-    stash(0);
-    fetch();
+    // slice s is multiplied from LDS buffer s % 2; `f` holds slice s + 1 (fetched two slices ago): it is written to the
+    // other buffer behind the multiplies, and the registers then take the fetch of slice s + 3
+    fetch(fa);
+    stash(0, fa);
+    fetch(fb);
+    fetch(fa);
     __syncthreads();
-    for (int s = 0; s < nslices; s++) {
+    auto slice_body = [&](int s, Fetched& f) {
         const int cur = s & 1;
         const unsigned short* arow = As[cur] + (wm0 + l32) * HSTRIDE + 8 * lk;
         const unsigned short* brow = Bs[cur] + (wc0 + l32) * HSTRIDE + 8 * lk;
@@ -203,9 +208,13 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
         qs += KH;
         qs -= qs >= W ? W : 0;
         if (HALFROW) qs -= qs >= W ? W : 0;
-        stash(cur ^ 1);
+        stash(cur ^ 1, f);
         __syncthreads();
-        fetch();
+        fetch(f);
+    };
+    for (int s = 0; s < nslices; s += 2) {
+        slice_body(s, fb);
+        if (s + 1 < nslices) slice_body(s + 1, fa);
     }
 
     // acc[i][s][v]: output channel m0 + wm0 + 32*i + 8*(v/4) + 4*lk + v%4, input channel c0 + wc0 + l32, tap (r, s)
