@@ -72,6 +72,8 @@ CONV_RANDOM = [
     (7, 128, 6, 20, 192, 3, 3, 1, 1, 1, 1),    # two channel blocks, a ragged second row tile, splits that straddle samples, slices that straddle rows
     (3, 64, 56, 56, 130, 3, 3, 1, 1, 1, 1),    # VGG-sized rows; two rows in the last tile
     (3, 64, 6, 28, 96, 3, 3, 1, 1, 1, 1),      # plane not a multiple of the slice: slices straddle samples
+    (3, 64, 6, 18, 96, 3, 3, 1, 1, 1, 1),      # rows of four and a half groups: every other row begins in the middle of a group
+    (4, 64, 14, 14, 64, 3, 3, 1, 1, 1, 1),     # 14 x 14: rows shorter than a slice, two row wraps per slice
 ]
 
 

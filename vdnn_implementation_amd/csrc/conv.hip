@@ -372,12 +372,12 @@ static int launch_wgrad3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, cons
     return VDNN_OK;
 }
 
-// Workgroups of wgrad3x3_f32_kernel that are resident on a compute unit (by its registers).
+// Workgroups of wgrad3x3_f32_kernel that are resident on a compute unit (its launch bounds; three, at 167 registers, measured 10 % slower).
 constexpr int kWgrad3FPerCU = 2;
 
 static bool wgrad3x3_f32_ok(const ConvGeo& g) {
     return g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W &&
-           g.W % 4 == 0 && g.W >= KB && g.C % WG3F_CH == 0; // a slice wraps at most one image row
+           g.W % 2 == 0 && g.W >= 14 && (g.H * g.W) % 4 == 0 && g.C % WG3F_CH == 0; // a slice wraps at most two image rows
 }
 
 // The float counterpart of launch_wgrad3x3.
@@ -411,8 +411,11 @@ static int launch_wgrad3x3_f32(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, 
     const Wgrad3x3F geo{dy, x, g.N, g.K, g.C, g.H, g.W, w, staging, (long)M * N, alpha, accumulate};
     {
         ProfScope prof(ctx, st, narrow ? kBwdFilterRow3Names.t64 : kBwdFilterRow3Names.t128, 2.0 * M * (double)N * (double)Kred, 0.0);
-        if (narrow) hipLaunchKernelGGL((wgrad3x3_f32_kernel<32>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
-        else hipLaunchKernelGGL((wgrad3x3_f32_kernel<64>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        const bool halfrow = g.W % 4 != 0 || g.W < KB; // the general variant: groups across two image rows, two row wraps per slice
+        if (narrow && halfrow) hipLaunchKernelGGL((wgrad3x3_f32_kernel<32, true>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        else if (narrow) hipLaunchKernelGGL((wgrad3x3_f32_kernel<32, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        else if (halfrow) hipLaunchKernelGGL((wgrad3x3_f32_kernel<64, true>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        else hipLaunchKernelGGL((wgrad3x3_f32_kernel<64, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
         VDNN_LAUNCH_CHECK();
     }
     if (d.splits > 1) return launch_reduce_splits_tap(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, accumulate, g.C, 9);

@@ -1,5 +1,6 @@
 // Backward filter of 3x3 / stride 1 / padding 1 layers with float activations whose image rows are whole groups of
-// four pixels (W % 4 == 0, W >= 16, C % 64 == 0). The float counterpart of wgrad3x3_bf16_kernel:
+// two pixels and whose planes are whole groups of four (W % 2 == 0, W >= 14, H*W % 4 == 0, C % 64 == 0). The float
+// counterpart of wgrad3x3_bf16_kernel:
 //
 //   dW[k][c][r][s] = sum over (n,p,q) of dy[n,k,p,q] * x[n,c,p+r-1,q+s-1]
 //
@@ -11,6 +12,9 @@
 // group (or the two extra elements) and is zero where the tap reads the padding beside the image. Rows of the image
 // outside the input are not fetched and stay zero. One fetch of dy and of x serves three taps (the tile-per-tap
 // engine fetches both again for every tap), which halves the requests to L2 per multiply.
+// When W is not a multiple of four (HALFROW) a group of four pixels can hold the last two of one image row and the
+// first two of the next: the halves are in or outside the input separately (masked when the group is stored), and
+// the padding is met in the middle of a lane's four values as well.
 // Accumulators: WR/32 x 3 blocks of 32x32. Partial sums of a reduction split go to the staging area in the
 // tap-major order that reduce_splits_tap sums.
 #pragma once
@@ -33,8 +37,8 @@ struct Wgrad3x3F {
 
 // d.M = K, d.N = 9*C, d.K = N*H*W; d.mtiles tiles of 2*WR output channels, d.ntiles = 3 * C/64 (filter row
 // fastest), d.splits reduction splits of d.kchunk pixels (a multiple of 16).
-template <int WR>
-__global__ void __launch_bounds__(NT) wgrad3x3_f32_kernel(const Wgrad3x3F g, const GemmDims d) {
+template <int WR, bool HALFROW>
+__global__ void __launch_bounds__(NT, 2) wgrad3x3_f32_kernel(const Wgrad3x3F g, const GemmDims d) {
     constexpr int TM = 2 * WR, RB = WR / 32, AL = TM / 64;
     __shared__ __attribute__((aligned(16))) float As[2][TM * RED_STRIDE];
     __shared__ __attribute__((aligned(16))) float Bs[2][WG3F_CH * RED_STRIDE];
@@ -85,11 +89,15 @@ __global__ void __launch_bounds__(NT) wgrad3x3_f32_kernel(const Wgrad3x3F g, con
 
     floatx4 ra[AL], rb;
     float rh = 0.0f;
-    // a group's image row / column / byte offset one slice further: W >= 16, one row wrap; at most one sample
+    bool keep_lo = true, keep_hi = true;
+    // a group's image row / column / byte offset one slice further: one row wrap when W >= 16, else two; at most one sample
     auto advance = [&](int& p, int& q, int& pos) {
         q += KB; pos += KB * 4;
-        const bool wrap = q >= W;
-        q -= wrap ? W : 0; p += wrap ? 1 : 0;
+#pragma unroll
+        for (int t = 0; t < (HALFROW ? 2 : 1); t++) {
+            const bool wrap = q >= W;
+            q -= wrap ? W : 0; p += wrap ? 1 : 0;
+        }
         const bool next = p >= H;
         p -= next ? H : 0; pos += next ? (g.C - 1) * PQ * 4 : 0;
     };
@@ -101,13 +109,21 @@ __global__ void __launch_bounds__(NT) wgrad3x3_f32_kernel(const Wgrad3x3F g, con
         pqA -= wrapA ? PQ : 0;
         offA += wrapA ? (KB + (g.K - 1) * PQ) * 4 : KB * 4;
 
-        const bool row_ok = (unsigned)(pB + r - 1) < (unsigned)H;
-        rb = buf_load4(rsB, row_ok ? posB + colB : OOB, 0);
+        {
+            const bool lo_ok = (unsigned)(pB + r - 1) < (unsigned)H;                               // the row of the group's first pixel
+            const bool hi_ok = (HALFROW && qB == W - 2) ? (unsigned)(pB + r) < (unsigned)H : lo_ok; // its last two may be in the next row
+            // only the last two inside (the image's first row through the upper filter row): fetched from there on, so that the
+            // load does not begin below the first element of the plane - and of the descriptor, where all of it reads zero
+            const bool late = hi_ok & !lo_ok;
+            rb = buf_load4(rsB, (lo_ok | hi_ok) ? posB + colB + (late ? 8 : 0) : OOB, 0);
+            keep_lo = lo_ok; keep_hi = hi_ok;
+        }
         advance(pB, qB, posB);
 
         if (wave < 2) {
             // not fetched where the tap reads the padding (the element would belong to another image row)
-            const bool used = (unsigned)(pH + r - 1) < (unsigned)H && qH != (side ? W - 4 : 0);
+            const int prow = pH + r - 1 + ((HALFROW && side && qH == W - 2) ? 1 : 0);
+            const bool used = (unsigned)prow < (unsigned)H && qH != (side ? W - 4 : 0);
             rh = buf_load(rsB, used ? posH + colH : OOB, 0);
             advance(pH, qH, posH);
         }
@@ -115,7 +131,13 @@ __global__ void __launch_bounds__(NT) wgrad3x3_f32_kernel(const Wgrad3x3F g, con
     auto stash = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < AL; i++) *(floatx4*)(As[buf] + (rl + 64 * i) * RED_STRIDE + 4 * pg) = ra[i];
-        *(floatx4*)(Bs[buf] + rl * RED_STRIDE + 4 * pg) = rb;
+        floatx4 v = rb; // a group outside the input was not fetched: zero
+        if (HALFROW) {
+            const bool late = keep_hi & !keep_lo;
+            v.x = keep_lo ? rb.x : 0.0f; v.y = keep_lo ? rb.y : 0.0f;
+            v.z = keep_hi ? (late ? rb.x : rb.z) : 0.0f; v.w = keep_hi ? (late ? rb.y : rb.w) : 0.0f;
+        }
+        *(floatx4*)(Bs[buf] + rl * RED_STRIDE + 4 * pg) = v;
         if (wave < 2) Hs[buf][side][lane] = rh;
     };
 
@@ -132,7 +154,7 @@ __global__ void __launch_bounds__(NT) wgrad3x3_f32_kernel(const Wgrad3x3F g, con
 
     // fragments of half hf (pixels 8 hf .. 8 hf + 7) of the slice in buffer `buf` whose first pixel has image column q0:
     // a lane holds pixels 8 hf + 4 lk .. + 3 of its row / channel, and the elements before and after them
-    struct Frag { floatx4 a[RB]; floatx4 v; float prev, next; };
+    struct Frag { floatx4 a[RB]; floatx4 v; float prev, next; bool mid; };
     auto read = [&](int buf, int hf, int q0, Frag& f) {
         const float* arow = As[buf] + (wm0 + l32) * RED_STRIDE + 8 * hf + 4 * lk;
         const float* brow = Bs[buf] + (wc0 + l32) * RED_STRIDE + 8 * hf + 4 * lk;
@@ -146,11 +168,13 @@ __global__ void __launch_bounds__(NT) wgrad3x3_f32_kernel(const Wgrad3x3F g, con
         qg -= qg >= W ? W : 0;
         f.prev = qg == 0 ? 0.0f : prev;     // left of the image
         f.next = qg == W - 4 ? 0.0f : next; // right of the image
+        f.mid = HALFROW && qg == W - 2;     // pixels 2.. of the four begin an image row
     };
     auto multiply = [&](const Frag& f) {
-        const float up[4] = {f.prev, f.v.x, f.v.y, f.v.z};
+        // pixel 2 reads left of the image through the left tap, pixel 1 right of it through the right tap, where a row begins inside
+        const float up[4] = {f.prev, f.v.x, (HALFROW && f.mid) ? 0.0f : f.v.y, f.v.z};
         const float ce[4] = {f.v.x, f.v.y, f.v.z, f.v.w};
-        const float dn[4] = {f.v.y, f.v.z, f.v.w, f.next};
+        const float dn[4] = {f.v.y, (HALFROW && f.mid) ? 0.0f : f.v.z, f.v.w, f.next};
 #pragma unroll
         for (int e = 0; e < 4; e++)
 #pragma unroll
@@ -181,6 +205,7 @@ __global__ void __launch_bounds__(NT) wgrad3x3_f32_kernel(const Wgrad3x3F g, con
         fetch();
         qs += KB;
         qs -= qs >= W ? W : 0;
+        if (HALFROW) qs -= qs >= W ? W : 0;
         read(nxt, 0, qs, f0);
         multiply(f1);
 #pragma unroll
