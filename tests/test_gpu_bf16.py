@@ -109,6 +109,7 @@ CONV = [
     (2, 128, 12, 20, 192, 3, 3, 1, 1, 1, 1),   # rows of two and a half groups: every other row begins in the middle of a group
     (5, 64, 2, 16, 64, 3, 3, 1, 1, 1, 1),      # a slice covers a whole two-row sample: every row touches the upper or the lower border
     (3, 64, 6, 28, 96, 3, 3, 1, 1, 1, 1),      # 28-pixel rows, plane not a multiple of the slice: slices straddle samples
+    (2, 96, 12, 20, 128, 3, 3, 1, 1, 1, 1),    # 96 channels: backward filter on the tile engine, four taps per tile, four pixels per load
 ]
 
 
@@ -286,8 +287,8 @@ def test_bf16_engine_in_a_split_last_round_agrees_with_two_half_batches(ctx):
 
 
 def test_conv_bf16_tensors_at_odd_element_offsets(ctx):
-    """Activation tensors that start two bytes off a four-byte boundary (a view into a larger buffer): the pixel-pair
-    loads of the bfloat16 engine do not depend on the alignment of the tensor, and backward filter leaves the engine."""
+    """Activation tensors that start two bytes off a four-byte boundary (a view into a larger buffer): neither the pixel-pair
+    loads of forward / backward data nor the eight-pixel loads of backward filter depend on the alignment of the tensor."""
     geom = (3, 64, 12, 16, 96, 3, 3, 1, 1, 1, 1)
     g, og = be.shape(*geom), oracle.shape(*geom)
     rng = np.random.default_rng(77)

@@ -425,7 +425,7 @@ static int launch_wgrad3x3_f32(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, 
 // Backward filter of a bfloat16 3x3 / stride 1 / padding 1 layer with the vector loaders: picks the instantiation
 // for the number of taps per tile and the pixel group (combinations whose loads would mix taps do not exist).
 template <int TM, int TN, int NTAP, int G>
-static int launch_wgrad_vec_one(vdnn_ctx* ctx, hipStream_t st, const char* name, const LoadDyRedVecH<8>& al, const LoadIm2colRedTapVecH<1, 8>& geo,
+static int launch_wgrad_vec_one(vdnn_ctx* ctx, hipStream_t st, const char* name, const LoadDyRedVecH<8>& al, const LoadIm2colRedTapVecH<1, 4>& geo,
                                 const StoreFilterTap& ep, const GemmDims& d) {
     if constexpr ((TN / NTAP) % (NT / (KH / G)) != 0) {
         set_error("backward filter: %d taps per %d-column tile with groups of %d pixels", NTAP, TN, G);
@@ -436,13 +436,9 @@ static int launch_wgrad_vec_one(vdnn_ctx* ctx, hipStream_t st, const char* name,
     }
 }
 template <int TM, int TN>
-static int launch_wgrad_vec(vdnn_ctx* ctx, hipStream_t st, const char* name, const LoadDyRedVecH<8>& al, const LoadIm2colRedTapVecH<1, 8>& geo,
+static int launch_wgrad_vec(vdnn_ctx* ctx, hipStream_t st, const char* name, const LoadDyRedVecH<8>& al, const LoadIm2colRedTapVecH<1, 4>& geo,
                             const StoreFilterTap& ep, const GemmDims& d, int ntap, int group) {
-    if (group == 8) {
-        if (ntap == 1) return launch_wgrad_vec_one<TM, TN, 1, 8>(ctx, st, name, al, geo, ep, d);
-        if (ntap == 2) return launch_wgrad_vec_one<TM, TN, 2, 8>(ctx, st, name, al, geo, ep, d);
-        return launch_wgrad_vec_one<TM, TN, 4, 8>(ctx, st, name, al, geo, ep, d);
-    }
+    if (group != 4) { set_error("backward filter: groups of %d pixels", group); return VDNN_EINVAL; }
     if (ntap == 1) return launch_wgrad_vec_one<TM, TN, 1, 4>(ctx, st, name, al, geo, ep, d);
     if (ntap == 2) return launch_wgrad_vec_one<TM, TN, 2, 4>(ctx, st, name, al, geo, ep, d);
     return launch_wgrad_vec_one<TM, TN, 4, 4>(ctx, st, name, al, geo, ep, d);
@@ -690,7 +686,7 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     const int ntap = g.C % tile_n == 0 ? 1 : (g.C % (tile_n / 2) == 0 ? 2 : (g.C % (tile_n / 4) == 0 ? 4 : 0));
     if constexpr (sizeof(E) == 2) {
         // bfloat16 activations: both factors of every product are bfloat16 already
-        if (wgrad3x3_ok(g) && aligned16(dy) && aligned16(x)) {
+        if (wgrad3x3_ok(g)) { // loads of eight pixels take any alignment of the tensors
             bool taken = false;
             const int rcw = launch_wgrad3x3(ctx, st, g, x, dy, w, alpha, accumulate, staging, staging_bytes, &taken);
             if (taken || rcw != VDNN_OK) return rcw;
@@ -706,14 +702,14 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
                 StoreFilterTap ept{w, staging, g.C, RS, (long)M * N, alpha, accumulate, dC};
                 LoadDyRedIncH al{dy, g.N, g.K, PQ, dh.kchunk, dh.K};
                 int rch;
-                // 3x3, stride 1, padding 1: a tap's im2col operand is the plane shifted by a constant, fetched in
-                // groups of eight (four) pixels when the image rows are whole groups
-                const int vg = g.W % 8 == 0 ? 8 : (g.W % 4 == 0 ? 4 : 0);
+                // 3x3, stride 1, padding 1, channel counts the kernel above does not take: a tap's im2col operand is the plane
+                // shifted by a constant, fetched in groups of four pixels when the image rows are whole groups
+                const int vg = g.W % 4 == 0 ? 4 : 0;
                 const int tap_cols = tile_n / ntap; // columns of the tile that share a tap
                 if (g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W && PQ % 8 == 0 &&
                     vg != 0 && tap_cols % (8 * vg) == 0 && (long)g.C * g.H * g.W * 2 < (long)MAX_SUM_RANGE) {
                     LoadDyRedVecH<8> alv{dy, g.N, g.K, PQ, dh.kchunk, dh.K};
-                    LoadIm2colRedTapVecH<1, 8> geo{x, g.N, g.C, g.H, g.W, N, dh.kchunk, dh.K, dC};
+                    LoadIm2colRedTapVecH<1, 4> geo{x, g.N, g.C, g.H, g.W, N, dh.kchunk, dh.K, dC};
                     rch = narrow ? launch_wgrad_vec<64, 256>(ctx, st, kBwdFilterHalfNames.t64, alv, geo, ept, dh, ntap, vg)
                                  : launch_wgrad_vec<128, 128>(ctx, st, kBwdFilterHalfNames.t128, alv, geo, ept, dh, ntap, vg);
                     if (rch != VDNN_OK) return rch;
@@ -744,7 +740,7 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     }
     if constexpr (sizeof(E) == 4) {
         // 3x3, stride 1, padding 1: one filter row and 64 input channels per workgroup, one fetch for three taps
-        if (wgrad3x3_f32_ok(g) && aligned16(dy) && aligned16(x)) {
+        if (wgrad3x3_f32_ok(g)) { // loads of four pixels take any alignment of the tensors
             bool taken = false;
             const int rcw = launch_wgrad3x3_f32(ctx, st, g, x, dy, w, alpha, accumulate, staging, staging_bytes, &taken);
             if (taken || rcw != VDNN_OK) return rcw;
