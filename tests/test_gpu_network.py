@@ -9,6 +9,8 @@
     decision that flips on a last-bit difference changes single elements by O(1));
  4. an offloaded and prefetched tensor is byte-identical (the network input after a step).
 """
+import hashlib
+
 import numpy as np
 import pytest
 
@@ -320,6 +322,11 @@ def _losses_and_stats(cnn, policy, algo, batch, steps=2, **kw):
             assert net.forwardPropagation() == 0
             losses.append(np.float32(net.loss()).tobytes())
             assert net.backwardPropagation() == 0
+        # one digest per layer with parameters, over the bytes of the filter and the bias after the last step
+        for l in range(net.num_layers):
+            if net.has_params(l):
+                w, b = net.get_params(l)
+                losses.append(hashlib.sha1(w.tobytes() + b.tobytes()).digest())
         return losses, net.stats()
 
 
@@ -330,11 +337,11 @@ def _losses_and_stats(cnn, policy, algo, batch, steps=2, **kw):
 ], ids=["overfeat128_conv", "vgg16_64_all_perfopt", "vgg16_128_all_policies"])
 def test_full_size_configurations_keep_the_baseline_losses(cnn, batch, algo, policies):
     """At full size no CPU result is affordable; what must hold at any size: every policy computes the
-    bits BASELINE computes (two steps, so the weight updates are covered), moves the bytes its
-    offload table says, and holds less device memory."""
+    bits BASELINE computes (the losses of two steps and a digest of every layer's parameters after them),
+    moves the bytes its offload table says, and holds less device memory."""
     announce("full size", cnn, batch, algo, "BASELINE")
     base_losses, base_stats = _losses_and_stats(cnn, BASELINE, algo, batch)
-    assert all(np.isfinite(np.frombuffer(b, np.float32)[0]) for b in base_losses)
+    assert all(np.isfinite(np.frombuffer(b, np.float32)[0]) for b in base_losses[:2])
     for policy in policies:
         for refined in (False, True):
             announce("full size", cnn, batch, algo, "policy", policy, "refined", refined)

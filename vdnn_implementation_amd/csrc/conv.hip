@@ -15,6 +15,7 @@
 #include "wgrad3x3_bf16.h"
 #include "wgrad3x3_f32.h"
 #include "conv_smallc.h"
+#include "conv_smallc_mfma.h"
 
 namespace vdnn {
 
@@ -422,6 +423,34 @@ static int launch_wgrad3x3_f32(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, 
     return VDNN_OK;
 }
 
+// Forward of a 3x3 / stride 1 / padding 1 layer with at most four input and 64 output channels: wavefronts stream over
+// the pixels, three workgroups per compute unit.
+static bool fwd_smallc3x3_ok(const ConvGeo& g, size_t elem_bytes) {
+    return g.C <= 4 && g.K <= 64 && g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W &&
+           (long)g.N * g.C * g.H * g.W * (long)elem_bytes < (1l << 31) && (long)g.N * g.K * g.H * g.W * (long)elem_bytes < (1l << 31);
+}
+template <class E>
+static int launch_fwd_smallc3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const E* x, const float* w, const float* bias, E* y, int relu) {
+    const long units = ((long)g.N * g.H * g.W + 31) / 32;
+    long blocks = (units + 3) / 4;
+    if (blocks > 3l * ctx->num_cu) blocks = 3l * ctx->num_cu; // bound by its stores from two workgroups per unit on (four measured 20 % slower)
+    ProfScope prof(ctx, st, "conv_fwd_smallc", 2.0 * g.K * 9.0 * g.C * (double)g.N * g.H * g.W, 0.0);
+#define VDNN_FWD_SMALLC(CC)                                                                                                              \
+    do {                                                                                                                                 \
+        if (g.K <= 32) hipLaunchKernelGGL((conv_fwd_smallc3x3_kernel<CC, 1, E>), dim3((unsigned)blocks), dim3(256), 0, st, x, w, bias, y, g.N, g.K, g.H, g.W, relu); \
+        else hipLaunchKernelGGL((conv_fwd_smallc3x3_kernel<CC, 2, E>), dim3((unsigned)blocks), dim3(256), 0, st, x, w, bias, y, g.N, g.K, g.H, g.W, relu);          \
+    } while (0)
+    switch (g.C) {
+    case 1: VDNN_FWD_SMALLC(1); break;
+    case 2: VDNN_FWD_SMALLC(2); break;
+    case 3: VDNN_FWD_SMALLC(3); break;
+    default: VDNN_FWD_SMALLC(4); break;
+    }
+#undef VDNN_FWD_SMALLC
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
+}
+
 // Backward filter of a bfloat16 3x3 / stride 1 / padding 1 layer with the vector loaders: picks the instantiation
 // for the number of taps per tile and the pixel group (combinations whose loads would mix taps do not exist).
 template <int TM, int TN, int NTAP, int G>
@@ -479,6 +508,7 @@ static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
         VDNN_REQUIRE(w != nullptr, "filter too large for the staging area (bfloat16 layer outside the bfloat16 engine)");
         VDNN_LAUNCH_CHECK();
     }
+    if (fwd_smallc3x3_ok(g, sizeof(E))) return launch_fwd_smallc3x3<E>(ctx, st, g, x, w, bias, y, relu);
     if (g.R * g.S <= 32 && g.C % KB == 0) {
         // blocked tap-major reduction: one slice = one tap x 16 input channels
         const int RS = g.R * g.S;
