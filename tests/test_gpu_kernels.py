@@ -74,6 +74,7 @@ CONV_RANDOM = [
     (3, 64, 6, 28, 96, 3, 3, 1, 1, 1, 1),      # plane not a multiple of the slice: slices straddle samples
     (3, 64, 6, 18, 96, 3, 3, 1, 1, 1, 1),      # rows of four and a half groups: every other row begins in the middle of a group
     (4, 64, 14, 14, 64, 3, 3, 1, 1, 1, 1),     # 14 x 14: rows shorter than a slice, two row wraps per slice
+    (3, 2, 6, 20, 96, 3, 3, 1, 1, 1, 1),       # two input channels, 96 output channels (a ragged second row tile), slices that straddle samples
 ]
 
 

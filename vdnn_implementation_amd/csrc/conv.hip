@@ -663,6 +663,35 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     const long Kred = (long)g.N * PQ;
     VDNN_REQUIRE(Kred < (1l << 31), "reduction too long");
     VDNN_REQUIRE((long)(PQ + KB) * PQ < (1l << 32), "output plane too large for the pixel cursor's exact division");
+    if (g.C <= 3 && g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W && g.W % 4 == 0 && g.W >= KB &&
+        ctx->reduce_scratch) {
+        // few input channels, rows of whole groups of four pixels: dy streamed once through the matrix cores, then the ordered split sum
+        const int mtiles = (g.K + 63) / 64;
+        const size_t out_bytes = (size_t)M * N * sizeof(float);
+        long splits = 3l * ctx->num_cu / mtiles;
+        const long by_len = Kred / (4 * WSC_SLICE), by_mem = (long)(ctx->reduce_scratch_bytes / out_bytes);
+        if (splits > by_len) splits = by_len;
+        if (splits > by_mem) splits = by_mem;
+        if (splits < 1) splits = 1;
+        long kchunk = (Kred + splits - 1) / splits;
+        kchunk = (kchunk + WSC_SLICE - 1) / WSC_SLICE * WSC_SLICE;
+        splits = (Kred + kchunk - 1) / kchunk;
+        const long nspan = kchunk / PQ + 2;
+        if (PQ >= WSC_SLICE && nspan * g.K * PQ * (long)sizeof(E) < (long)MAX_SUM_RANGE && nspan * g.C * PQ * (long)sizeof(E) < (long)MAX_SUM_RANGE) {
+            const WgradSmallC geo{dy, x, g.N, g.K, g.H, g.W, ctx->reduce_scratch, (int)kchunk};
+            {
+                ProfScope prof(ctx, st, "conv_bwd_filter_smallc", 2.0 * (double)M * N * (double)Kred, 0.0);
+                const dim3 grid((unsigned)(mtiles * splits));
+                switch (g.C) {
+                case 1: hipLaunchKernelGGL((wgrad_smallc3x3_mfma_kernel<1, E>), grid, dim3(NT), 0, st, geo); break;
+                case 2: hipLaunchKernelGGL((wgrad_smallc3x3_mfma_kernel<2, E>), grid, dim3(NT), 0, st, geo); break;
+                default: hipLaunchKernelGGL((wgrad_smallc3x3_mfma_kernel<3, E>), grid, dim3(NT), 0, st, geo); break;
+                }
+                VDNN_LAUNCH_CHECK();
+            }
+            return launch_reduce_splits(ctx, st, w, ctx->reduce_scratch, (size_t)M * N, (int)splits, alpha, accumulate, nullptr, 0);
+        }
+    }
     if (g.C <= 4 && g.R == 3 && g.S == 3 && g.K % 4 == 0 && ctx->reduce_scratch) {
         // few input channels: vector-ALU kernel over chunks of output pixels, then the ordered chunk sum
         const long total = Kred;

@@ -141,3 +141,189 @@ __global__ void __launch_bounds__(256) conv_fwd_smallc3x3_kernel(const E* __rest
 }
 
 } // namespace vdnn
+
+namespace vdnn {
+
+// Backward filter of 3x3 / stride 1 / padding 1 layers with at most three input channels (9*C <= 32 columns), rows of
+// whole groups of four pixels (W % 4 == 0, W >= 16). The pass reads dy once and is bound by that; the reduction runs
+// over pixels, contiguous in dy and x, so - as in wgrad3x3_f32_kernel - a slice of pixels is fetched with 128-bit loads
+// along the pixels into reduction-major LDS rows: 64 rows of dy, and one row of x per (channel, filter row) shifted by
+// (r-1)*W, plus the element before and after each run. Slices are 64 pixels long: with 16 the barrier and the latency
+// of a fetch (one slice ahead) cost more than the slice's four multiplies per wavefront. Column n = (c, r, s) of the
+// product takes row (c, r) of x one place left / in place / one place right by s: every lane forms the three variants
+// from one 128-bit read and picks its own. Four wavefronts share a slice's multiplies: 32 output channels x half of the
+// slice's pixels each; the halves are added through LDS at the end. Partial sums of a reduction split go to the
+// staging area as [split][K][C][3][3], which reduce_splits adds in split order.
+struct WgradSmallC {
+    const void* dy;
+    const void* x;
+    int N, K, H, W;
+    float* partial; // [split][K][9*C]
+    int kchunk;     // pixels per split, a multiple of WSC_SLICE
+};
+constexpr int WSC_SLICE = 64;            // pixels per slice
+constexpr int WSC_STRIDE = WSC_SLICE + 4; // LDS row stride in floats: 128-bit reads of 16 consecutive rows hit 16 different bank groups
+
+template <int CC, class E>
+__global__ void __launch_bounds__(NT) wgrad_smallc3x3_mfma_kernel(const WgradSmallC g) {
+    constexpr int ROWS = 3 * CC, NCOL = 9 * CC, ES = ElemBytes<E>::V;
+    constexpr int SL = WSC_SLICE, GPS = SL / 4; // groups of four pixels per slice
+    static_assert(NCOL <= 32, "one block of 32 columns");
+    static_assert(ROWS * GPS <= NT && 2 * ROWS <= 64, "one x group per thread");
+    __shared__ __attribute__((aligned(16))) float As[2][64 * WSC_STRIDE];
+    __shared__ __attribute__((aligned(16))) float Bs[2][ROWS * WSC_STRIDE];
+    __shared__ float Hs[2][2][ROWS];
+    __shared__ float Red[2][64][17]; // the second half's sums, [row block][lane][value]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lk = lane >> 5;
+    const int H = g.H, W = g.W, PQ = H * W;
+    const int Kred = g.N * PQ;
+    const int mtiles = (g.K + 63) / 64;
+    const int mt = blockIdx.x % mtiles, ks = blockIdx.x / mtiles;
+    const int m0 = mt * 64;
+    const int k_begin = ks * g.kchunk;
+    const int k_end = min(Kred, k_begin + g.kchunk);
+    const E* dy = (const E*)g.dy;
+    const E* x = (const E*)g.x;
+
+    const int n_first = k_begin / PQ;
+    const int n_last = k_end > k_begin ? (k_end - 1) / PQ : n_first;
+    const __amdgpu_buffer_rsrc_t rsA = make_rsrc(dy + (long)n_first * g.K * PQ, clamp_range((long)(n_last - n_first + 1) * g.K * PQ * ES));
+    const __amdgpu_buffer_rsrc_t rsB = make_rsrc(x + (long)n_first * CC * PQ, clamp_range((long)(n_last - n_first + 1) * CC * PQ * ES));
+
+    // loaders: thread t fetches pixel group t % 16 of the dy rows t / 16 + 16 i; threads below 16*ROWS also that group
+    // of x row t / 16 = (channel, filter row); lanes of wavefront 3 below 2*ROWS the element before / after the run of
+    // row lane / 2
+    const int pg = tid & (GPS - 1), rl = tid / GPS;
+    int mrow[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { const int m = m0 + rl + 16 * i; mrow[i] = m < g.K ? m * PQ * ES : SENT; }
+    int pqA, offA;
+    {
+        const int kk = k_begin + 4 * pg;
+        const int n = kk / PQ, pq = kk - n * PQ;
+        pqA = pq;
+        offA = (n - n_first) * g.K * PQ * ES + pq * ES;
+    }
+    struct Cursor { int p, q, pos; };
+    auto cursor_at = [&](int kk) {
+        const int n = kk / PQ, pq = kk - n * PQ;
+        Cursor c;
+        c.p = pq / W; c.q = pq - c.p * W;
+        c.pos = ((n - n_first) * CC * PQ + pq) * ES;
+        return c;
+    };
+    auto advance = [&](Cursor& c) { // one slice further: several image rows when they are short, at most one sample
+        c.q += SL; c.pos += SL * ES;
+        while (c.q >= W) { c.q -= W; c.p += 1; }
+        const bool next = c.p >= H;
+        c.p -= next ? H : 0; c.pos += next ? (CC - 1) * PQ * ES : 0;
+    };
+    const bool loads_b = rl < ROWS;
+    const int rB = rl % 3;
+    const int colB = loads_b ? ((rl / 3) * PQ + (rB - 1) * W) * ES : SENT;
+    Cursor cb = cursor_at(k_begin + 4 * pg);
+    const bool loads_h = wave == 3 && lane < 2 * ROWS;
+    const int side = lane & 1, rowH = (lane >> 1) % ROWS, rH = rowH % 3;
+    const int colH = loads_h ? ((rowH / 3) * PQ + (rH - 1) * W) * ES + (side ? 4 * ES : -ES) : SENT;
+    Cursor ch = cursor_at(k_begin + (side ? SL - 4 : 0));
+
+    // what a slice's fetch leaves in registers; two slices are in flight (the pass is bound by the latency of dy)
+    struct Fetched { floatx4 ra[4], rb; float rh; };
+    Fetched fa, fb;
+    fa.rh = 0.0f; fb.rh = 0.0f;
+    auto fetch = [&](Fetched& f) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) f.ra[i] = buf_load4_e<E>(rsA, mrow[i] + offA, 0);
+        pqA += SL;
+        const bool wrapA = pqA >= PQ; // H*W >= 64: one sample at most
+        pqA -= wrapA ? PQ : 0;
+        offA += wrapA ? (SL + (g.K - 1) * PQ) * ES : SL * ES;
+        if (tid < ROWS * GPS) {
+            const bool row_ok = (unsigned)(cb.p + rB - 1) < (unsigned)H;
+            f.rb = buf_load4_e<E>(rsB, row_ok ? cb.pos + colB : OOB, 0);
+        }
+        advance(cb);
+        if (wave == 3) {
+            const bool used = (unsigned)(ch.p + rH - 1) < (unsigned)H && ch.q != (side ? W - 4 : 0);
+            f.rh = buf_load_e<E>(rsB, used ? ch.pos + colH : OOB, 0);
+            advance(ch);
+        }
+    };
+    auto stash = [&](int buf, const Fetched& f) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) *(floatx4*)(As[buf] + (rl + 16 * i) * WSC_STRIDE + 4 * pg) = f.ra[i];
+        if (loads_b) *(floatx4*)(Bs[buf] + rl * WSC_STRIDE + 4 * pg) = f.rb;
+        if (loads_h) Hs[buf][side][rowH] = f.rh;
+    };
+
+    floatx16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+    const int rowblk = wave & 1, hf = wave >> 1; // this wavefront: 32 output channels, pixels 32*hf .. 32*hf + 31 of every slice
+    // this lane's column (c, r, s): its row of x in LDS and which neighbour it takes
+    const bool col_live = l32 < NCOL;
+    const int bro = col_live ? l32 / 3 : 0, sB = col_live ? l32 % 3 : 1;
+    int qs = k_begin % W;
+
+    const int nslices = (k_end - k_begin + SL - 1) / SL;
+    // slice s is multiplied from LDS buffer s % 2; `f` holds slice s + 1 (fetched two slices ago): it is written to the
+    // other buffer behind the multiplies, and the registers then take the fetch of slice s + 3
+    fetch(fa);
+    stash(0, fa);
+    fetch(fb);
+    fetch(fa);
+    __syncthreads();
+    auto slice_body = [&](int s, Fetched& f) {
+        const int cur = s & 1;
+        const float* arow = As[cur] + (32 * rowblk + l32) * WSC_STRIDE + 32 * hf + 4 * lk;
+        const float* brow = Bs[cur] + bro * WSC_STRIDE + 32 * hf + 4 * lk;
+#pragma unroll
+        for (int gq = 0; gq < 4; gq++) { // eight pixels: four per half of the lanes
+            const floatx4 a = *(const floatx4*)(arow + 8 * gq);
+            const floatx4 v = *(const floatx4*)(brow + 8 * gq);
+            const float* pp = (hf == 0 && gq == 0 && lk == 0) ? &Hs[cur][0][bro] : brow + 8 * gq - 1;
+            const float* np = (hf == 1 && gq == 3 && lk == 1) ? &Hs[cur][1][bro] : brow + 8 * gq + 4;
+            float prev = *pp, next = *np;
+            int qg = qs + 32 * hf + 8 * gq + 4 * lk;
+            while (qg >= W) qg -= W;
+            prev = qg == 0 ? 0.0f : prev;     // left of the image
+            next = qg == W - 4 ? 0.0f : next; // right of the image
+            const float b0 = !col_live ? 0.0f : sB == 0 ? prev : sB == 1 ? v.x : v.y;
+            const float b1 = !col_live ? 0.0f : sB == 0 ? v.x : sB == 1 ? v.y : v.z;
+            const float b2 = !col_live ? 0.0f : sB == 0 ? v.y : sB == 1 ? v.z : v.w;
+            const float b3 = !col_live ? 0.0f : sB == 0 ? v.z : sB == 1 ? v.w : next;
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b0, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b1, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b2, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b3, acc, 0, 0, 0);
+        }
+        qs += SL;
+        while (qs >= W) qs -= W;
+        stash(cur ^ 1, f);
+        __syncthreads();
+        fetch(f);
+    };
+    for (int s = 0; s < nslices; s += 2) {
+        slice_body(s, fb);
+        if (s + 1 < nslices) slice_body(s + 1, fa);
+    }
+
+    // the two halves of the slices: wavefronts 2 and 3 hand their sums to 0 and 1 (fixed order: first half + second half)
+    if (hf == 1) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) Red[rowblk][lane][v] = acc[v];
+    }
+    __syncthreads();
+    if (hf == 0 && col_live) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int m = m0 + 32 * rowblk + 8 * (v / 4) + 4 * lk + (v % 4);
+            if (m >= g.K) continue;
+            g.partial[((long)ks * g.K + m) * NCOL + l32] = acc[v] + Red[rowblk][lane][v];
+        }
+    }
+}
+
+} // namespace vdnn

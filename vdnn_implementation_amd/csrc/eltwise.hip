@@ -173,10 +173,55 @@ __global__ void __launch_bounds__(EB) reduce_splits_kernel(E* __restrict__ out, 
     }
 }
 
+// The same sums when the splits are many (a reduction split over the whole chip for a small filter bank): a thread per
+// output would walk hundreds of partial sums one after the other on a handful of workgroups. Here a workgroup owns 32
+// outputs and eight groups of consecutive splits; a thread adds its group's splits in order, the eight group sums are
+// added in group order through LDS. TAP: the partial sums are in tap-major column order (see reduce_splits_tap_kernel).
+template <bool TAP>
+__global__ void __launch_bounds__(256) reduce_splits_wide_kernel(float* __restrict__ out, const float* __restrict__ partial, size_t count,
+                                                                 int splits, float alpha, int accumulate, int C, int RS) {
+    __shared__ float sums[8][33];
+    const int o = threadIdx.x & 31, grp = threadIdx.x >> 5;
+    const size_t i = (size_t)blockIdx.x * 32 + o;
+    const int per = (splits + 7) / 8;
+    const int k0 = grp * per, k1 = k0 + per < splits ? k0 + per : splits;
+    float s = 0.0f;
+    if (i < count && k0 < k1) {
+        size_t src = i;
+        if (TAP) {
+            const int ncols = C * RS;
+            const size_t m = i / ncols;
+            const int rem = (int)(i - m * ncols);
+            const int c = rem / RS, tap = rem - c * RS;
+            src = m * ncols + (size_t)tap * C + c;
+        }
+        s = partial[(size_t)k0 * count + src];
+        for (int k = k0 + 1; k < k1; k++) s += partial[(size_t)k * count + src];
+    }
+    sums[grp][o] = s;
+    __syncthreads();
+    if (grp == 0 && i < count) {
+        float t = sums[0][o];
+#pragma unroll
+        for (int g = 1; g < 8; g++) t += (g * per < splits) ? sums[g][o] : 0.0f;
+        out[i] = accumulate ? __fmaf_rn(alpha, t, out[i]) : alpha * t;
+    }
+}
+constexpr int kWideReduceSplits = 32;        // from this many splits on,
+constexpr size_t kWideReduceCount = 131072; // up to this many outputs (beyond, a thread per output fills the chip)
+
 template <class E>
 static int launch_reduce_splits_t(vdnn_ctx* ctx, hipStream_t stream, E* out, const float* partial, size_t count,
                                   int splits, float alpha, int accumulate, const float* bias_j, int ncols, int relu, const E* gate) {
     ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)count * (splits + 2));
+    if constexpr (sizeof(E) == 4) {
+        if (splits >= kWideReduceSplits && count <= kWideReduceCount && !bias_j && !relu && !gate) {
+            hipLaunchKernelGGL(reduce_splits_wide_kernel<false>, dim3((unsigned)((count + 31) / 32)), dim3(256), 0, stream,
+                               (float*)out, partial, count, splits, alpha, accumulate, 0, 0);
+            VDNN_LAUNCH_CHECK();
+            return VDNN_OK;
+        }
+    }
     hipLaunchKernelGGL(reduce_splits_kernel<E>, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
                        out, partial, count, splits, alpha, accumulate, bias_j, ncols, relu, gate);
     VDNN_LAUNCH_CHECK();
@@ -253,6 +298,10 @@ __global__ void __launch_bounds__(EB) reduce_splits_tap_kernel(float* __restrict
 int launch_reduce_splits_tap(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
                              float alpha, int accumulate, int C, int RS) {
     ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)count * (splits + 2));
+    if (splits >= kWideReduceSplits && count <= kWideReduceCount)
+        hipLaunchKernelGGL(reduce_splits_wide_kernel<true>, dim3((unsigned)((count + 31) / 32)), dim3(256), 0, stream,
+                           out, partial, count, splits, alpha, accumulate, C, RS);
+    else
     hipLaunchKernelGGL(reduce_splits_tap_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
                        out, partial, count, splits, alpha, accumulate, C, RS);
     VDNN_LAUNCH_CHECK();
