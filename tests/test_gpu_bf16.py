@@ -110,6 +110,7 @@ CONV = [
     (5, 64, 2, 16, 64, 3, 3, 1, 1, 1, 1),      # a slice covers a whole two-row sample: every row touches the upper or the lower border
     (3, 64, 6, 28, 96, 3, 3, 1, 1, 1, 1),      # 28-pixel rows, plane not a multiple of the slice: slices straddle samples
     (2, 96, 12, 20, 128, 3, 3, 1, 1, 1, 1),    # 96 channels: backward filter on the tile engine, four taps per tile, four pixels per load
+    (2, 3, 11, 140, 32, 3, 3, 1, 1, 1, 1),     # three input channels: the streaming first-layer kernels, two backward-data column blocks
 ]
 
 

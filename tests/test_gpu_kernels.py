@@ -75,6 +75,7 @@ CONV_RANDOM = [
     (3, 64, 6, 18, 96, 3, 3, 1, 1, 1, 1),      # rows of four and a half groups: every other row begins in the middle of a group
     (4, 64, 14, 14, 64, 3, 3, 1, 1, 1, 1),     # 14 x 14: rows shorter than a slice, two row wraps per slice
     (3, 2, 6, 20, 96, 3, 3, 1, 1, 1, 1),       # two input channels, 96 output channels (a ragged second row tile), slices that straddle samples
+    (2, 3, 11, 140, 32, 3, 3, 1, 1, 1, 1),     # three input channels, rows wider than a backward-data column block, strips of eight and three rows
 ]
 
 

@@ -591,6 +591,23 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
         VDNN_REQUIRE(blocks < (1l << 31), "grid too large");
         ProfScope prof(ctx, st, "conv_bwd_data_smallc", 2.0 * g.C * (double)g.N * g.P * g.Q * g.K * g.R * g.S, 0.0);
         const bool s1_3x3 = g.sh == 1 && g.sw == 1 && g.R == 3 && g.S == 3;
+        // 3x3, padding 1, at most three input and 64 output channels: the products once, on the matrix cores, row by row
+        if (s1_3x3 && g.C <= 3 && g.K <= 64 && g.ph == 1 && g.pw == 1 && g.P == g.H && g.Q == g.W &&
+            (long)g.K * g.P * g.Q * (long)sizeof(E) < (long)MAX_SUM_RANGE) {
+            // about three workgroups per compute unit, strips of at least eight image rows
+            const int cblocks = (g.W + BDS_EMIT - 1) / BDS_EMIT;
+            int strips = (int)((3l * ctx->num_cu + (long)g.N * cblocks - 1) / ((long)g.N * cblocks));
+            int rows = (g.H + strips - 1) / strips;
+            if (rows < 8) rows = 8;
+            if (rows > g.H) rows = g.H;
+            strips = (g.H + rows - 1) / rows;
+            const dim3 grid((unsigned)(g.N * strips * cblocks));
+            if (g.C == 1) hipLaunchKernelGGL((conv_bwd_data_smallc3x3_mfma_kernel<1, E>), grid, dim3(256), 0, st, dy, w, dx, g.N, g.K, g.H, g.W, rows);
+            else if (g.C == 2) hipLaunchKernelGGL((conv_bwd_data_smallc3x3_mfma_kernel<2, E>), grid, dim3(256), 0, st, dy, w, dx, g.N, g.K, g.H, g.W, rows);
+            else hipLaunchKernelGGL((conv_bwd_data_smallc3x3_mfma_kernel<3, E>), grid, dim3(256), 0, st, dy, w, dx, g.N, g.K, g.H, g.W, rows);
+            VDNN_LAUNCH_CHECK();
+            return VDNN_OK;
+        }
         if (s1_3x3 && g.C == 3) hipLaunchKernelGGL((conv_bwd_data_smallc_s1_kernel<3, 3, 3, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
         else if (s1_3x3 && g.C == 4) hipLaunchKernelGGL((conv_bwd_data_smallc_s1_kernel<3, 3, 4, E>), dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);
         else if (g.sh == 1 && g.sw == 1) hipLaunchKernelGGL(conv_bwd_data_smallc_kernel<E>, dim3((unsigned)blocks), dim3(256), 0, st, dy, w, dx, g);

@@ -327,3 +327,93 @@ __global__ void __launch_bounds__(NT) wgrad_smallc3x3_mfma_kernel(const WgradSma
 }
 
 } // namespace vdnn
+
+namespace vdnn {
+
+// Backward data of 3x3 / stride 1 / padding 1 layers with at most three input channels and at most 64 output channels
+// (the first layer). dx has three rows per pixel, far too few for a matrix tile, and the vector-ALU kernel read dy
+// nine times per pixel. Here the products are formed once, on the matrix cores, as a 1x1 convolution with 9*C <= 32
+// output rows over dy, one image row at a time:
+//     T_j[(c,r,s)][q] = sum over k of w[k][c][r][s] * dy[k][j][q]
+// (A = the transposed filter bank in registers, 32 steps of two output channels; B = dy fetched straight from memory,
+// lanes along q), and a workgroup that walks down a strip of image rows, 126 columns wide, keeps the last three T rows
+// (128 columns: one more on either side) in LDS and emits
+//     dx[c][ih][iw] = sum over (r,s) of T_(ih-r+1)[(c,r,s)][iw-s+1]
+// for the row above the one just computed (nine LDS reads per value; rows outside the image are skipped, columns
+// outside it hold zero because nothing was fetched for them). Each of the four wavefronts owns 32 of the 128 columns;
+// the next row's values are fetched before the barrier and the emission of the current one. dy is read once, plus two
+// rows per strip and two columns per 126.
+constexpr int BDS_COLS = 128;          // T columns of a workgroup
+constexpr int BDS_EMIT = BDS_COLS - 2; // dx columns of a workgroup
+template <int CC, class E>
+__global__ void __launch_bounds__(256) conv_bwd_data_smallc3x3_mfma_kernel(const E* __restrict__ dy, const float* __restrict__ w, E* __restrict__ dx,
+                                                                            int N, int K, int H, int W, int strip_rows) {
+    constexpr int NROW = 9 * CC, ES = ElemBytes<E>::V, KS = 32; // up to 64 output channels
+    constexpr int WP = BDS_COLS + 1, TROW = NROW * WP;          // odd row stride: the nine reads of a value fall on different banks
+    static_assert(NROW <= 32, "one block of 32 rows");
+    __shared__ float T[3 * TROW];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lk = lane >> 5;
+    const int PQ = H * W;
+    const int strips = (H + strip_rows - 1) / strip_rows, cblocks = (W + BDS_EMIT - 1) / BDS_EMIT;
+    const int cbk = blockIdx.x % cblocks, sid = (blockIdx.x / cblocks) % strips, n = blockIdx.x / (cblocks * strips);
+    const int p0 = sid * strip_rows, p1 = p0 + strip_rows < H ? p0 + strip_rows : H;
+    const int e0 = cbk * BDS_EMIT, e1 = e0 + BDS_EMIT < W ? e0 + BDS_EMIT : W; // dx columns of this workgroup
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(dy + (long)n * K * PQ, clamp_range((long)K * PQ * ES));
+
+    float a[KS];
+    int koff[KS];
+#pragma unroll
+    for (int t = 0; t < KS; t++) {
+        const int k = 2 * t + lk;
+        a[t] = (l32 < NROW && k < K) ? w[(long)k * NROW + l32] : 0.0f;
+        koff[t] = k < K ? k * PQ * ES : SENT;
+    }
+    // this lane's T column: image column e0 - 1 + 32*wave + l32, LDS column 32*wave + l32
+    const int tc = 32 * wave + l32, q = e0 - 1 + tc;
+    const bool q_in = q >= 0 && q < W;
+    float b[KS];
+    auto fetch = [&](int j) {
+        const int base = (q_in && j >= 0 && j < H) ? (j * W + q) * ES : SENT;
+#pragma unroll
+        for (int t = 0; t < KS; t++) b[t] = buf_load_e<E>(rs, base + koff[t], 0);
+    };
+
+    fetch(p0 - 1);
+    for (int j = p0 - 1; j <= p1; j++) {
+        if (j >= 0 && j < H) { // (a row outside the image is never read below)
+            floatx16 acc;
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+#pragma unroll
+            for (int t = 0; t < KS; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b[t], acc, 0, 0, 0);
+            float* Tj = T + (j % 3) * TROW;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = 8 * (v / 4) + 4 * lk + (v % 4);
+                if (m < NROW) Tj[m * WP + tc] = acc[v];
+            }
+        }
+        if (j < p1) fetch(j + 1);
+        __syncthreads();
+        const int ih = j - 1;
+        if (ih >= p0 && ih < p1) {
+            for (int o = tid; o < CC * (e1 - e0); o += 256) {
+                const int c = o / (e1 - e0), ew = o - c * (e1 - e0); // dx column e0 + ew: T columns ew, ew + 1, ew + 2 by s = 2, 1, 0
+                float sum = 0.0f;
+#pragma unroll
+                for (int r = 0; r < 3; r++) {
+                    const int jj = ih - r + 1;
+                    if (jj < 0 || jj >= H) continue;
+                    const float* row = T + (jj % 3) * TROW + (c * 9 + r * 3) * WP + ew + 2;
+#pragma unroll
+                    for (int s = 0; s < 3; s++) sum += row[s * WP - s];
+                }
+                store_elem(dx + ((long)n * CC + c) * PQ + (long)ih * W + e0 + ew, sum);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+} // namespace vdnn
