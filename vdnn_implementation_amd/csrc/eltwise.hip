@@ -358,7 +358,23 @@ __global__ void __launch_bounds__(EB) bias_grad_partial_kernel(const E* __restri
     const int k = blockIdx.x / splits, sp = blockIdx.x % splits;
     const int n0 = sp * n_per_split, n1 = min(N, n0 + n_per_split);
     float acc = 0.0f;
-    if ((PQ & 3) == 0 && (((uintptr_t)dy & 15) == 0)) {
+    if (sizeof(E) == 2 && (PQ & 7) == 0 && (((uintptr_t)dy & 15) == 0)) {
+        // bfloat16: eight elements (16 bytes) per access, eight independent partial sums per thread
+        typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+        float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        const int pq8 = PQ >> 3;
+        for (int n = n0; n < n1; n++) {
+            const u32x4* p = (const u32x4*)(dy + ((size_t)n * K + k) * PQ);
+            for (int i = threadIdx.x; i < pq8; i += EB) {
+                const u32x4 v = p[i];
+                s[0] += __builtin_bit_cast(float, v.x << 16); s[1] += __builtin_bit_cast(float, v.x & 0xFFFF0000u);
+                s[2] += __builtin_bit_cast(float, v.y << 16); s[3] += __builtin_bit_cast(float, v.y & 0xFFFF0000u);
+                s[4] += __builtin_bit_cast(float, v.z << 16); s[5] += __builtin_bit_cast(float, v.z & 0xFFFF0000u);
+                s[6] += __builtin_bit_cast(float, v.w << 16); s[7] += __builtin_bit_cast(float, v.w & 0xFFFF0000u);
+            }
+        }
+        acc = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
+    } else if ((PQ & 3) == 0 && (((uintptr_t)dy & 15) == 0)) {
         // four elements per access, four independent partial sums per thread (a fixed order, combined below)
         float4 a4 = make_float4(0.f, 0.f, 0.f, 0.f);
         const int pq4 = PQ >> 2;
