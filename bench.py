@@ -209,10 +209,11 @@ def main():
         assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep"}, name
         _, policy, algo = parse("VGG16_128", word, args.algo)
         bf16 = args.bf16 or "bf16" in mods
-        # (what a plan sends over the link gets the slack that hides it: a lag of six layers on the way out, fetched
+        # (what a plan sends over the link gets the slack that hides it: a lag of fourteen layers on the way out, fetched
         # ahead on the way back wherever the peak allows)
         ahead = "ahead" in mods or bool(budget)
-        lag, depth = (6, 2) if "slack" in mods else (6, 1) if ahead else (args.offload_lag, args.prefetch_depth)
+        # (a plan holds what waits for its copy as a packed stream, and its replay counts it: a long lag costs it no memory)
+        lag, depth = (6, 2) if "slack" in mods else (14, 1) if budget else (6, 1) if ahead else (args.offload_lag, args.prefetch_depth)
         kw = dict(refined="refined" in mods, cap_bytes=int(args.cap_gb * 1e9), bf16=bf16, offload_lag=lag, prefetch_depth=depth,
                   fuse="fused" in mods, compress="zvc" in mods, prefetch_within_peak=ahead, keep_packed="keep" in mods,
                   keep_tail_bytes=int(0.75e9) * (2 if bf16 else 4) if "tail" in mods else int(args.keep_tail_gb * 1e9))
