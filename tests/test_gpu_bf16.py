@@ -148,7 +148,7 @@ def test_conv_bf16(ctx, geom, algo):
         assert_close(gb.download(b.shape), oracle.conv_bwd_bias_sgd(og, dy, np.zeros_like(b), 1.0), 1e-4, "bwd bias")
 
 
-@pytest.mark.parametrize("n,cin,cout", [(128, 1000, 520), (64, 2304, 512), (5, 41, 33)])
+@pytest.mark.parametrize("n,cin,cout", [(128, 1000, 520), (64, 2304, 512), (5, 41, 33), (72, 264, 136), (128, 12544, 200), (40, 72, 1000)])
 def test_fc_bf16(ctx, n, cin, cout):
     rng = np.random.default_rng(n + cin)
     x, dy = rnd(rng, (n, cin)), rnd(rng, (n, cout))

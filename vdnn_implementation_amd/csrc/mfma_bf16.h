@@ -94,7 +94,7 @@ struct LoadIm2colPixTapH {
 // packed[row][(cb*RS + tap)*32 + l] = bf16(w[row*row_stride + (cb*32 + l)*red_stride + tap])
 //   forward:       rows = output channels, reduced channels = input channels:  row_stride = C*RS, red_stride = RS
 //   backward data: rows = input channels,  reduced channels = output channels: row_stride = RS,   red_stride = C*RS
-__global__ void __launch_bounds__(256) pack_filter_tap_bf16_kernel(const float* __restrict__ w, unsigned short* __restrict__ packed,
+static __global__ void __launch_bounds__(256) pack_filter_tap_bf16_kernel(const float* __restrict__ w, unsigned short* __restrict__ packed,
                                                                    int rows, int Cred, int RS, int row_stride, int red_stride, long total) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
@@ -104,6 +104,9 @@ __global__ void __launch_bounds__(256) pack_filter_tap_bf16_kernel(const float* 
     const int cb = slice / RS, tap = slice - cb * RS;
     packed[i] = float_to_bf16_bits(w[(long)row * row_stride + (long)(cb * 32 + l) * red_stride + tap]);
 }
+
+// Order of the tiles over the workgroup index: rows fastest unless the epilogue type says otherwise.
+template <class EP> struct TileOrder { static constexpr bool COLUMNS_FASTEST = false; };
 
 // Out tile = A tile x B tile over this workgroup's share of the reduction; tile decoding and epilogues are
 // those of the float engine (igemm_kernel), slices are KH deep.
@@ -127,7 +130,9 @@ __global__ void __launch_bounds__(NT) igemm_bf16_kernel(const AL al, const BL bl
         const int bid = xcd_remap(blockIdx.x, gridDim.x);
         tile = bid % ntiles_all; ks = bid / ntiles_all; whole = d.splits == 1;
     }
-    const int mt = tile % d.mtiles, nt = tile / d.mtiles;
+    // the column tile runs fastest for epilogues that ask for it (workgroups at work together then write one run of rows)
+    const int mt = TileOrder<EP>::COLUMNS_FASTEST ? tile / d.ntiles : tile % d.mtiles;
+    const int nt = TileOrder<EP>::COLUMNS_FASTEST ? tile % d.ntiles : tile / d.mtiles;
     const int m0 = mt * TM, j0 = nt * TN;
     const int k_begin = whole ? 0 : ks * d.kchunk;
     const int k_end = whole ? d.K : min(d.K, k_begin + d.kchunk);
