@@ -280,6 +280,20 @@ __global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH a
         static_assert(NJ == 2 && WM == 1, "one 64 x 64 block per wavefront");
         constexpr int STG = 72; // row stride of the block in LDS, 16-bit units
         static_assert(4 * 64 * STG <= 2 * W3_ROWS * HSTRIDE, "the four blocks fit the window buffers");
+        // the gate's elements first (what the lane will overwrite, if the gradient goes over the layer's own input):
+        // fetched one after the other behind each store they would cost a round trip to memory each
+        const int grp = lane & 7;
+        const int j = j0 + wn0 + 8 * grp;
+        const int n = j / ep.opix, pix = j - n * ep.opix;
+        const size_t base = (size_t)n * d.M * ep.opix + pix;
+        uintx4 gv[8];
+        if (ep.gate && j < d.N) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int m = m0 + (lane >> 3) + 8 * i;
+                gv[i] = m < d.M ? *(const uintx4*)(ep.gate + base + (size_t)m * ep.opix) : uintx4{0, 0, 0, 0};
+            }
+        }
         __syncthreads(); // every wavefront has read its last fragments
         unsigned short* stg = &Bw[0][0] + wave * (64 * STG);
 #pragma unroll
@@ -298,10 +312,6 @@ __global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH a
                 }
             }
         __builtin_amdgcn_wave_barrier(); // the block is read by other lanes of the same wavefront: LDS keeps a wavefront's order
-        const int grp = lane & 7;
-        const int j = j0 + wn0 + 8 * grp;
-        const int n = j / ep.opix, pix = j - n * ep.opix;
-        const size_t base = (size_t)n * d.M * ep.opix + pix;
         if (j < d.N) {
 #pragma unroll
             for (int i = 0; i < 8; i++) {
@@ -312,11 +322,10 @@ __global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH a
                 const size_t idx = base + (size_t)m * ep.opix;
                 if (ep.gate) {
                     // kept where gate > 0: a positive bfloat16 that is not a NaN has bits 0x0001 .. 0x7F80
-                    const uintx4 gv = *(const uintx4*)(ep.gate + idx);
                     auto keep = [](unsigned w) {
                         return ((((w & 0xFFFFu) - 1u) < 0x7F80u) ? 0x0000FFFFu : 0u) | ((((w >> 16) - 1u) < 0x7F80u) ? 0xFFFF0000u : 0u);
                     };
-                    val.x &= keep(gv.x); val.y &= keep(gv.y); val.z &= keep(gv.z); val.w &= keep(gv.w);
+                    val.x &= keep(gv[i].x); val.y &= keep(gv[i].y); val.z &= keep(gv[i].z); val.w &= keep(gv[i].w);
                 }
                 *(uintx4*)(ep.out + idx) = val;
             }
