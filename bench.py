@@ -37,8 +37,9 @@ DEFAULT_POLICIES = ",".join([
     "VDNN_CONV+refined+ahead+fused+zvc", "VDNN_ALL+refined+ahead+fused+zvc",
     "VDNN_ALL+refined+fused+zvc+keep",
     "VDNN_ALL+refined+fused+zvc+budget3.0", "VDNN_ALL+refined+fused+zvc+budget3.3", "VDNN_ALL+refined+fused+zvc+budget4.0",
+    "VDNN_ALL+refined+fused+zvc+inplace+budget3.4", "VDNN_ALL+refined+fused+zvc+inplace+budget3.6+lag10",
     "BASELINE+bf16+fused", "VDNN_ALL+refined+ahead+bf16+fused+zvc", "VDNN_ALL+refined+bf16+fused+zvc+keep",
-    "VDNN_ALL+refined+bf16+fused+zvc+budget5.9",
+    "VDNN_ALL+refined+bf16+fused+zvc+budget5.9", "VDNN_ALL+refined+bf16+fused+zvc+keep+inplace",
 ])
 
 
@@ -146,6 +147,19 @@ def best_within(results, base, floor_ratio, need_link):
             "peak_hbm_gb": ok[k]["peak_hbm_gb"], "link_gb_each_way_per_step": ok[k]["link_gb_each_way_per_step"]}
 
 
+def smallest_within(results, base, speed_floor):
+    """The run that holds the least device memory among those at least speed_floor times as fast as the fp32 BASELINE."""
+    if not base:
+        return None
+    ok = {k: v for k, v in results.items() if v["images_per_s"] >= speed_floor * base["images_per_s"] and k.split("+")[0] != "BASELINE"}
+    if not ok:
+        return None
+    k = min(ok, key=lambda n: ok[n]["peak_hbm_gb"])
+    return {"policy": k, "speed_vs_baseline": ok[k]["images_per_s"] / base["images_per_s"],
+            "peak_hbm_reduction": base["peak_hbm_gb"] / ok[k]["peak_hbm_gb"], "images_per_s": ok[k]["images_per_s"],
+            "peak_hbm_gb": ok[k]["peak_hbm_gb"], "link_gb_each_way_per_step": ok[k]["link_gb_each_way_per_step"]}
+
+
 def cpu_baseline(batch, threads):
     """The checker's training step (forward, backward, SGD) on the host cores: VGG16, float."""
     import oracle
@@ -202,11 +216,13 @@ def main():
         # peak cannot rise; "+fused" ReLU layers run inside the neighbouring layers' kernels; "+zvc" offloaded rectified
         # tensors are packed (no zero elements); "+keep" the packed tensors stay in device memory; "+tail" the deepest
         # 0.75 G elements of the offload set stay on the device; "+budgetX" the policy meets a budget of the fp32
-        # BASELINE's peak / X by choosing a place for every tensor; "+bf16" bfloat16 activation storage
+        # BASELINE's peak / X by choosing a place for every tensor; "+bf16" bfloat16 activation storage; "+inplace" input
+        # gradients written over the inputs nothing reads again; "+lagN" blocks recycled N layers after their offload
         word, *mods = name.split("+")
         budget = [float(m[6:]) for m in mods if m.startswith("budget")]
-        mods = [m for m in mods if not m.startswith("budget")]
-        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep"}, name
+        lag_given = [int(m[3:]) for m in mods if m.startswith("lag")]
+        mods = [m for m in mods if not m.startswith("budget") and not m.startswith("lag")]
+        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep", "inplace"}, name
         _, policy, algo = parse("VGG16_128", word, args.algo)
         bf16 = args.bf16 or "bf16" in mods
         # (what a plan sends over the link gets the slack that hides it: a lag of fourteen layers on the way out, fetched
@@ -214,7 +230,9 @@ def main():
         ahead = "ahead" in mods or bool(budget)
         # (a plan holds what waits for its copy as a packed stream, and its replay counts it: a long lag costs it no memory)
         lag, depth = (6, 2) if "slack" in mods else (14, 1) if budget else (6, 1) if ahead else (args.offload_lag, args.prefetch_depth)
-        kw = dict(refined="refined" in mods, cap_bytes=int(args.cap_gb * 1e9), bf16=bf16, offload_lag=lag, prefetch_depth=depth,
+        if lag_given:
+            lag = lag_given[0]
+        kw = dict(refined="refined" in mods, in_place="inplace" in mods, cap_bytes=int(args.cap_gb * 1e9), bf16=bf16, offload_lag=lag, prefetch_depth=depth,
                   fuse="fused" in mods, compress="zvc" in mods, prefetch_within_peak=ahead, keep_packed="keep" in mods,
                   keep_tail_bytes=int(0.75e9) * (2 if bf16 else 4) if "tail" in mods else int(args.keep_tail_gb * 1e9))
         if budget:
@@ -277,6 +295,7 @@ def main():
         # BASELINE, and the fastest of those that move at least 0.5 GB over the link each way
         "best_fp32_at_3x": best_within(fp32, base, 3.0, False),
         "best_fp32_at_3x_over_the_link": best_within(fp32, base, 3.0, True),
+        "least_memory_fp32_at_85pct": smallest_within(fp32, base, 0.85),
         "best_any_dtype_at_3x": best_within(results, base, 3.0, False),
         "baseline_peak_gb_replayed": baseline_peak / 1e9,
         "conv_mfma_util": conv_all_tf / peak if conv_all_tf else None,

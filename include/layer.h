@@ -130,6 +130,8 @@ public:
     int     convolutionForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workSpace, bool isDynamic);
     int     convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
                                 void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
+    int     convolutionBackwardOverSrc(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
+                                       void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
     // FC_GEMM layer
     int     fullyConnectedForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workSpace, bool isDynamic);
     int     fullyConnectedBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
@@ -194,6 +196,12 @@ public:
     void    setGateGrad(bool v) { gateGrad = v; }
     bool    GateGrad() const { return gateGrad; }
     bool    InPlaceOp() const { return inPlaceOp; }
+    /* Addition: backward writes gradData over srcData (CONV with stride 1 and more than four input channels, 2x2 /
+       stride 2 POOL): gradData then *is* srcData and no block is taken for it. The Network sets it where the layer
+       below does not read that tensor in its own backward. */
+    void    setGradOverSrc(bool v) { gradOverSrc = v; }
+    bool    GradOverSrc() const { return gradOverSrc; }
+    bool    canGradOverSrc() const;
     void    setAlgoMode(vdnnAlgoMode_t m);
     // Event the offload copy waits for (srcData fully written) and the events this layer's copies
     // signal; owned by the Network. Null events mean "no ordering needed" (plan-only contexts).
@@ -319,6 +327,7 @@ private:
     int  refCntFwd, refCntBwd;
     bool inPlaceOp, insideInceptionModule, headOfFork, tailOfFork;
     bool fuseRelu, elided, elidedBackward, gateGrad;
+    bool gradOverSrc = false;
     int  forkId, concatenateChannelOffset;
 
     vdnnConvHandle_t* convHandle;

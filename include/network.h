@@ -87,6 +87,16 @@ struct NetworkOptions {
     // the last plan stands and Network::planFeasible() says so. The replay has no data: planPackedFraction is what it
     // takes a packed stream to be of its tensor. 0: no budget, the policy's own offload set.
     size_t   hbmBudgetBytes = 0;
+    // Backward writes a layer's input gradient over the layer's own input where nothing reads that input again: a
+    // convolution (stride 1, more than four input channels) computes its filter gradient first, into a block of the
+    // filter's size, then the data gradient - still with the old filter, as layer.cu:616-660 has it - over its
+    // srcData, then applies the update (param += alpha * grad, the fused call's arithmetic: same bits); a 2x2 / stride 2
+    // max-pool reads its two windows and writes them back. The layer below must be one whose backward does not read
+    // its own output (with refinedLifetimes: convolution, FC, pooling, or a ReLU that is fused away), and the filter
+    // must be smaller than the input (or the block for its gradient would outweigh the one saved). The reference
+    // holds x, dy and dx of a layer together (layer.cu:599, 999-1011); here the largest layer holds two of them.
+    // Needs refinedLifetimes; not BASELINE (whose dx/dy pair is shared by all layers).
+    bool     inPlaceBackward = false;
     std::vector<unsigned char> forcedPlacement; // (internal: the replay's placement per layer, see Placement)
     bool     tracePeaks = false;          // (internal: the replay records bytes in use per forward and backward layer)
     int      device = DEFAULT_DEVICE;
@@ -181,6 +191,8 @@ public:
     vdnnAlgoMode_t  algo() const            { return algoMode; }
     vdnn_ctx*       context()               { return ctx; }
     bool            isOffloaded(int l) const { return isOffload[l]; }
+    // inPlaceBackward: layer l's backward writes its input gradient over its input
+    bool            gradOverSrc(int l) const { return l >= 0 && l < numLayers && layer[l] && layer[l]->GradOverSrc(); }
     // synthetic data: N(0,1) input, integer labels in [0, classes) as a one-hot target, seeded filters
     void            setInput(const float* host);
     void            setLabels(const int32_t* labels);

@@ -235,6 +235,14 @@ int vdnn_fc_bwd_data_relu(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c_in, 
                           const void* dy, const float* w, const void* x, void* dx);
 int vdnn_maxpool_bwd_relu(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape,
                           const void* x, const void* y, const void* dy, void* dx);
+/* Whether dx may be the very tensor x in vdnn_conv_bwd_data[_relu] / vdnn_maxpool_bwd[_relu] (no counterpart in the
+ * reference, which allocates gradData beside srcData, layer.cu:599, 897): 1 for stride-1 convolutions with more than
+ * four input channels that are not one dense product, and for 2x2 / stride 2 / unpadded pooling over planes of even
+ * height and a width that is a multiple of four. There every lane reads the elements it overwrites before it does, and
+ * nothing else reads x. (The filter gradient reads x: the caller computes it first.) Other shapes return an error
+ * when handed dx == x as the gate. */
+int vdnn_conv_bwd_data_in_place_ok(const vdnn_shape_t* shape);
+int vdnn_maxpool_bwd_in_place_ok(const vdnn_shape_t* shape);
 
 /* ---- fully connected (replaces cuBLAS: layer.cu:667-764) ------------------------------------- */
 /* Sgemm(T,N) + rank-1 bias broadcast (layer.cu:677-706): y[n,o] = sum_i w[o,i] x[n,i] + bias[o].

@@ -105,6 +105,8 @@ BACKEND_SYMBOLS = {
     "vdnn_fc_fwd_relu": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "vdnn_fc_bwd_data_relu": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "vdnn_maxpool_bwd_relu": (_i, [_vp, _vp, _S, _vp, _vp, _vp, _vp]),
+    "vdnn_conv_bwd_data_in_place_ok": (_i, [_S]),
+    "vdnn_maxpool_bwd_in_place_ok": (_i, [_S]),
     "vdnn_conv_bwd_bias_sgd": (_i, [_vp, _vp, _S, _vp, _vp, _f]),
     "vdnn_conv_bwd_bias_sgd_noalloc": (_i, [_vp, _S, _i, _vp, _vp, _f]),
     "vdnn_conv_bwd_filter_sgd": (_i, [_vp, _vp, _S, _i, _vp, _vp, _vp, _f, _vp, _sz]),

@@ -27,6 +27,7 @@ static NetworkOptions to_options(const vdnn_network_options* o) {
     n.planPackedFraction = o->plan_packed_fraction;
     n.prefetchWithinPeak = o->prefetch_within_peak != 0;
     n.hbmBudgetBytes = o->hbm_budget_bytes;
+    n.inPlaceBackward = o->in_place_backward != 0;
     return n;
 }
 
@@ -50,6 +51,7 @@ void vdnn_network_default_options(vdnn_network_options* o) {
     o->plan_packed_fraction = d.planPackedFraction;
     o->compress_offload = d.compressOffload;
     o->hbm_budget_bytes = d.hbmBudgetBytes;
+    o->in_place_backward = d.inPlaceBackward;
 }
 
 vdnn_network* vdnn_network_create(int cnn, int policy, int algo, int batch, const vdnn_network_options* o) {
@@ -141,6 +143,8 @@ void vdnn_network_reset_peak(vdnn_network* h) { h->net->resetPeak(); }
 int vdnn_network_is_offloaded(vdnn_network* h, int l) {
     return (l >= 0 && l < h->net->numLayersCount() && h->net->isOffloaded(l)) ? 1 : 0;
 }
+
+int vdnn_network_grad_over_src(vdnn_network* h, int l) { return h->net->gradOverSrc(l) ? 1 : 0; }
 
 int vdnn_network_placement(vdnn_network* h, int l) { return (int)h->net->placementOf(l); }
 int vdnn_network_plan_feasible(vdnn_network* h) { return h->net->planFeasible() ? 1 : 0; }

@@ -534,6 +534,13 @@ static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
     return conv_fwd_with(ctx, st, g, al, x, bias, y, relu);
 }
 
+// The kernels that a stride-1 layer with more than four input channels takes store through StoreNCHW or one of the
+// split reductions: a lane reads the gate's element before it writes the gradient's, and no kernel reads the layer's
+// input otherwise. (Layers that are one dense product are left out: their filter gradient is as large as the filter.)
+static bool conv_bwd_data_in_place_ok(const ConvGeo& g) {
+    return g.sh == 1 && g.sw == 1 && g.C > 4 && !is_dense(g);
+}
+
 template <class E>
 static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
                               const E* dy, const float* w, E* dx,
@@ -542,6 +549,9 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
     ConvGeo g;
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(dy && w && dx, "null tensor");
+    VDNN_REQUIRE((const void*)dx != (const void*)dy, "the input gradient cannot be written over the output gradient");
+    VDNN_REQUIRE((const void*)dx != (const void*)gate || conv_bwd_data_in_place_ok(g),
+                 "the input gradient may be written over the gating input only where vdnn_conv_bwd_data_in_place_ok says so");
     if (is_dense(g))
         return gate ? vdnn_fc_bwd_data_relu(ctx, stream, g.N, g.C * g.H * g.W, g.K, dy, w, gate, dx)
                     : vdnn_fc_bwd_data(ctx, stream, g.N, g.C * g.H * g.W, g.K, dy, w, dx);
@@ -904,6 +914,11 @@ int vdnn_conv_bwd_data(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* 
                        void* workspace, size_t workspace_bytes) {
     return VDNN_BY_ACT(ctx, conv_bwd_data_impl<float>(ctx, stream, shape, algo_mode, (const float*)dy, w, (float*)dx, workspace, workspace_bytes, nullptr),
                        conv_bwd_data_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)dy, w, (bf16_t*)dx, workspace, workspace_bytes, nullptr));
+}
+
+int vdnn_conv_bwd_data_in_place_ok(const vdnn_shape_t* shape) {
+    ConvGeo g;
+    return shape && geo_from_shape(shape, g) && conv_bwd_data_in_place_ok(g);
 }
 
 int vdnn_conv_bwd_data_relu(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,

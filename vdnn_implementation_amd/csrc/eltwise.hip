@@ -156,11 +156,12 @@ __global__ void __launch_bounds__(EB) bias_add_kernel(E* __restrict__ y, const f
     }
 }
 
-// out[i] = (accumulate ? out[i] : 0) + alpha * (p[0][i] + p[1][i] + ...) (+ bias[i % ncols]); split order fixed
+// out[i] = (accumulate ? out[i] : 0) + alpha * (p[0][i] + p[1][i] + ...) (+ bias[i % ncols]); split order fixed.
+// out and gate may be one tensor (a gradient written over the input that gates it): an element is read before it is written.
 template <class E>
-__global__ void __launch_bounds__(EB) reduce_splits_kernel(E* __restrict__ out, const float* __restrict__ partial, size_t count,
+__global__ void __launch_bounds__(EB) reduce_splits_kernel(E* out, const float* __restrict__ partial, size_t count,
                                                            int splits, float alpha, int accumulate, const float* __restrict__ bias_j, int ncols,
-                                                           int relu, const E* __restrict__ gate) {
+                                                           int relu, const E* gate) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < count; i += stride) {
         float s = partial[i];
@@ -239,9 +240,9 @@ int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, bf16_t* out, const f
 // tiles of a convolution result that were split (tail mode): out[n][m][pix] = sum over the tile's splits (+ bias[m]);
 // partial[(t*splits + ks)*TM*TN + row*TN + col] for the t-th split tile, tiles numbered m-tile fastest
 template <class E>
-__global__ void __launch_bounds__(EB) reduce_tail_nchw_kernel(E* __restrict__ out, const float* __restrict__ partial, int splits, int TM, int TN,
+__global__ void __launch_bounds__(EB) reduce_tail_nchw_kernel(E* out, const float* __restrict__ partial, int splits, int TM, int TN,
                                                               int M, int N, int mtiles, int full_tiles, const float* __restrict__ bias, int opix, size_t total,
-                                                              int relu, const E* __restrict__ gate) {
+                                                              int relu, const E* gate) { // (out and gate may be one tensor)
     const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
     if (i >= total) return;
     const int per = TM * TN;
@@ -310,9 +311,9 @@ int launch_reduce_splits_tap(vdnn_ctx* ctx, hipStream_t stream, float* out, cons
 
 // NCHW result of a split convolution: out[i] = p[0][i] + p[1][i] + ... (+ bias[channel of i]); split order fixed
 template <class E>
-__global__ void __launch_bounds__(EB) reduce_splits_nchw_kernel(E* __restrict__ out, const float* __restrict__ partial, size_t count,
+__global__ void __launch_bounds__(EB) reduce_splits_nchw_kernel(E* out, const float* __restrict__ partial, size_t count,
                                                                 int splits, const float* __restrict__ bias, int opix, int channels,
-                                                                int relu, const E* __restrict__ gate) {
+                                                                int relu, const E* gate) { // (out and gate may be one tensor)
     const size_t i = (size_t)blockIdx.x * EB + threadIdx.x;
     if (i >= count) return;
     float s = partial[i];
@@ -564,9 +565,10 @@ __global__ void __launch_bounds__(EB) maxpool_bwd_planes_kernel(const E* __restr
     }
 }
 
-// 2x2 stride 2 exact cover: one thread per pair of windows, writes all eight inputs
+// 2x2 stride 2 exact cover: one thread per pair of windows, writes all eight inputs. dx may be x itself: a thread has
+// read its eight inputs before it writes the eight gradients, and no other thread touches them.
 template <class E>
-__global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const E* __restrict__ x, const E* __restrict__ dy, E* __restrict__ dx,
+__global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const E* x, const E* __restrict__ dy, E* dx,
                                                             int H, int W, size_t total_pairs, int gate) {
     const int Q2 = W / 4, P = H / 2;
     const size_t stride = (size_t)gridDim.x * EB;
@@ -969,6 +971,8 @@ static int maxpool_bwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
     VDNN_REQUIRE(x && dy && dx, "null tensor");
     hipStream_t st = stream_of(ctx, stream);
     ProfScope prof(ctx, st, "maxpool_bwd", 0.0, (double)sizeof(E) * (2.0 * g.N * g.C * g.H * g.W + (double)g.N * g.C * g.P * g.Q));
+    VDNN_REQUIRE((const void*)x != (const void*)dx || (pool_is_2x2_exact(g, x, dx, dy) && (g.W / 2) % 2 == 0),
+                 "the gradient may be written over the input only by the 2x2 / stride 2 kernel (vdnn_maxpool_bwd_in_place_ok)");
     if (pool_is_2x2_exact(g, x, dx, dy) && (g.W / 2) % 2 == 0) {
         const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
         hipLaunchKernelGGL(maxpool2x2_bwd_kernel<E>, dim3(grid_for(pairs, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g.H, g.W, pairs, gate);
@@ -1162,6 +1166,11 @@ int vdnn_maxpool_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* sh
 }
 int vdnn_maxpool_bwd_relu(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* x, const void* y, const void* dy, void* dx) {
     return ACT_CALL(maxpool_bwd_t, ctx, stream, shape, x, y, dy, dx, 1);
+}
+int vdnn_maxpool_bwd_in_place_ok(const vdnn_shape_t* shape) {
+    PoolGeo g;
+    if (!shape || !pool_geo(shape, g)) return 0;
+    return g.R == 2 && g.S == 2 && g.sh == 2 && g.sw == 2 && g.ph == 0 && g.pw == 0 && g.H % 2 == 0 && g.W % 4 == 0;
 }
 int vdnn_lrn_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const void* x, void* y) { return ACT_CALL(lrn_fwd_t, ctx, stream, n, c, hw, x, y); }
 int vdnn_lrn_bwd(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int c, int hw, const void* x, const void* y, const void* dy, void* dx) {

@@ -260,9 +260,57 @@ int Layer::convolutionForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, 
     return 0;
 }
 
+/* The kernels that may write a layer's input gradient over its input: every lane reads what it overwrites before it
+ * does, and nothing else reads the input (vdnn_conv_bwd_data_in_place_ok / vdnn_maxpool_bwd_in_place_ok). */
+bool Layer::canGradOverSrc() const {
+    if (layerType == CONV || layerType == FC_CONV) return vdnn_conv_bwd_data_in_place_ok(&shape) != 0;
+    if (layerType == POOL) return vdnn_maxpool_bwd_in_place_ok(&shape) != 0;
+    return false;
+}
+
+/* Addition (gradOverSrc): the filter gradient first, into a block of its own, because it is the last reader of the
+ * input; then the data gradient over the input - with the filter as it was, the order of layer.cu:616-660 - and only
+ * then the update, param += alpha * grad with the fused call's arithmetic. */
+int Layer::convolutionBackwardOverSrc(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h, void* _srcDataToPrefetch,
+                                      unsigned long _prefetch_bytes, void* workSpace, bool isDynamic) {
+    void* curWorkSpace = nullptr;
+    const DATATYPE lr = LEARNING_RATE * -1.0f;
+    gradData = srcData;
+    if (_layer_id_to_prefetch >= 0) prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);
+
+    if (filterGrad) checkVDNN(vdnn_conv_bwd_bias(ctx, *stream_compute, &shape, (const float*)diffData, (float*)biasGrad));
+    else checkVDNN(vdnn_conv_bwd_bias_sgd(ctx, *stream_compute, &shape, (const float*)diffData, (float*)biasData, lr));
+
+    void* dw = filterGrad;
+    if (!dw && ASSERT_EQ(vdnn_pool_malloc(ctx, &dw, sizeof(DATATYPE) * (size_t)k * c_in * r * s), isDynamic) < 0) return -1;
+    auto releaseDw = [&]() { if (!filterGrad) ASSERT_EQ(vdnn_pool_free(ctx, dw), isDynamic); };
+    if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { releaseDw(); return -1; }
+    waitSrcFetched();
+    checkVDNN(vdnn_conv_bwd_filter(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
+                                   (float*)dw, curWorkSpace, bwdFilterWorkSpaceSize));
+    freeWorkSpace(workSpace, bwdFilterWorkSpaceSize, curWorkSpace, isDynamic);
+
+    if (mallocWorkSpace(workSpace, bwdDataWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { releaseDw(); return -1; }
+    if (gateGrad)
+        checkVDNN(vdnn_conv_bwd_data_relu(ctx, *stream_compute, &shape, vdnnAlgoMode, diffData, (const float*)filterData,
+                                          srcData, gradData, curWorkSpace, bwdDataWorkSpaceSize));
+    else
+        checkVDNN(vdnn_conv_bwd_data(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)diffData, (const float*)filterData,
+                                     (float*)gradData, curWorkSpace, bwdDataWorkSpaceSize));
+    freeWorkSpace(workSpace, bwdDataWorkSpaceSize, curWorkSpace, isDynamic);
+
+    if (!filterGrad) {
+        checkVDNN(vdnn_sgd_apply(ctx, *stream_compute, (size_t)k * c_in * r * s, lr, (const float*)dw, (float*)filterData));
+        releaseDw();
+    }
+    return 0;
+}
+
 /* layer.cu:591-665: gradData, prefetch, backward data (old filter), bias update, filter update */
 int Layer::convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h, void* _srcDataToPrefetch,
                                unsigned long _prefetch_bytes, void* workSpace, bool isDynamic) {
+    if (gradOverSrc && vdnnMode != BASELINE)
+        return convolutionBackwardOverSrc(_layer_id_to_prefetch, _prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes, workSpace, isDynamic);
     void* curWorkSpace = nullptr;
     const DATATYPE lr = LEARNING_RATE * -1.0f;
 
@@ -414,7 +462,8 @@ int Layer::poolingForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void
 int Layer::poolingBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h, void* _srcDataToPrefetch,
                            unsigned long _prefetch_bytes, void*, bool isDynamic) {
     if (vdnnMode != BASELINE) {
-        if (cnmemMallocGradData(isDynamic) < 0) return -1;
+        if (gradOverSrc) gradData = srcData; /* every thread reads its windows whole before it writes them back */
+        else if (cnmemMallocGradData(isDynamic) < 0) return -1;
     }
     if (vdnnMode != BASELINE && _layer_id_to_prefetch >= 0)
         prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);

@@ -491,6 +491,23 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         layer[l - 1]->setElidedBackward(false);
     }
 
+    /* inPlaceBackward: the input gradient of a convolution or a 2x2 pooling layer goes over the layer's input where the
+       layer below does not read that tensor - its own output - in its backward: convolution, FC and pooling layers
+       (refined lifetimes release it before their backward as it is), and a ReLU whose backward is fused away. Never
+       layer 0: the network input outlives the step. */
+    for (int l = 0; l < numLayers; l++) layer[l]->setGradOverSrc(false);
+    if (options.inPlaceBackward && refined) {
+        for (int l = 1; l < numLayers; l++) {
+            if (!layer[l]->canGradOverSrc()) continue;
+            /* a convolution then takes a block of its filter's size for the filter gradient: no gain where that is the larger one */
+            if (layer[l]->FilterDataSize() * sizeof(DATATYPE) >= layer[l]->SrcDataSize() * actBytes()) continue;
+            const Layer_t below = layer[l - 1]->LayerType();
+            const bool belowLeavesIt = is_conv(below) || below == FC_GEMM || below == POOL ||
+                                       (layer[l - 1]->Elided() && layer[l - 1]->ElidedBackward());
+            if (belowLeavesIt) layer[l]->setGradOverSrc(true);
+        }
+    }
+
     if (newVdnnType != BASELINE) {
         for (int l = 0; l < numLayers; l++)
             for (vdnn_event_t* e : {&evFwdDone[l], &evOffloadDone[l], &evBlockFree[l], &evPrefetchDone[l], &evPacked[l]})
@@ -766,8 +783,11 @@ int Network::backwardPropagation(bool isDynamic) {
             /* refined lifetimes: convolution, FC and pooling backward never read their output, so
                its block (the next layer's srcData) goes back to the pool before anything is
                allocated for this layer */
+            /* the layer above wrote its input gradient over its input: this layer's output and the gradient that
+               arrives for it are one block, released once, as the gradient */
+            const bool dstIsDiff = l != numLayers - 1 && layer[l]->DstData() == layer[l]->DiffData();
             bool dstReleased = false;
-            if (options.refinedLifetimes && l != numLayers - 1) {
+            if (options.refinedLifetimes && l != numLayers - 1 && !dstIsDiff) {
                 const Layer_t t = layer[l]->LayerType();
                 if (is_conv(t) || t == FC_GEMM || t == POOL) {
                     ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DstData()), isDynamic);
@@ -844,7 +864,7 @@ int Network::backwardPropagation(bool isDynamic) {
             /* Release dstData and diffData: every reader is already enqueued on the compute stream.
                An in-place ReLU's diffData is its gradData and lives on as the next layer's diffData. */
             /* an elided ReLU's block is released by the layer below, as its dstData */
-            if (!dstReleased && !layer[l]->Elided()) ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DstData()), isDynamic);
+            if (!dstReleased && !dstIsDiff && !layer[l]->Elided()) ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DstData()), isDynamic);
             if (!(layer[l]->InPlaceOp() && layer[l]->GradData() == layer[l]->DiffData()))
                 ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->DiffData()), isDynamic);
             /* this layer's packed input has been expanded (its backward waited for that): the block goes back */
