@@ -37,7 +37,7 @@ DEFAULT_POLICIES = ",".join([
     "VDNN_CONV+refined+ahead+fused+zvc", "VDNN_ALL+refined+ahead+fused+zvc",
     "VDNN_ALL+refined+fused+zvc+keep",
     "VDNN_ALL+refined+fused+zvc+budget3.0", "VDNN_ALL+refined+fused+zvc+budget3.3", "VDNN_ALL+refined+fused+zvc+budget4.0",
-    "VDNN_ALL+refined+fused+zvc+inplace+budget3.4", "VDNN_ALL+refined+fused+zvc+inplace+budget3.6+lag10",
+    "VDNN_ALL+refined+fused+zvc+inplace+budget3.4", "VDNN_ALL+refined+fused+zvc+inplace+budget3.5+lag10",
     "BASELINE+bf16+fused", "VDNN_ALL+refined+ahead+bf16+fused+zvc", "VDNN_ALL+refined+bf16+fused+zvc+keep",
     "VDNN_ALL+refined+bf16+fused+zvc+budget5.9", "VDNN_ALL+refined+bf16+fused+zvc+keep+inplace",
 ])
