@@ -59,6 +59,16 @@ def test_command_line_words():
     assert out.returncode == 0 and "CNN Model Type: VGG16_64" in out.stdout and '"batch": 64' in out.stdout
     bad = subprocess.run([exe, "VGG16_64", "VDNN_SOME", "VDNN_MEMORY_OPT_ALGO", "--plan"], capture_output=True, text=True)
     assert bad.returncode != 0 and "VDNN type must be one of" in bad.stderr
+    # the options of the recommended run: a budget, compressed offload, gradients written over inputs
+    import json
+    peaks = {}
+    for extra in ([], ["--in-place"]):
+        out = subprocess.run([exe, "VGG16_128", "VDNN_ALL", "VDNN_MEMORY_OPT_ALGO", "--plan", "--refined", "--fuse", "--zvc", "--offload-lag", "14",
+                              "--prefetch-within-peak", "--packed-fraction", "0.6", "--hbm-budget-gb", "5.48"] + extra, capture_output=True, text=True)
+        assert out.returncode == 0, out.stderr
+        peaks[bool(extra)] = json.loads(out.stdout.strip().splitlines()[-1])
+    assert not peaks[False]["plan_feasible"] and peaks[True]["plan_feasible"]
+    assert peaks[True]["peak_bytes"] <= 5.48e9 < peaks[False]["peak_bytes"]
 
 
 def test_reference_shaped_main_compiles_against_the_public_headers():
