@@ -37,9 +37,10 @@ DEFAULT_POLICIES = ",".join([
     "VDNN_CONV+refined+ahead+fused+zvc", "VDNN_ALL+refined+ahead+fused+zvc",
     "VDNN_ALL+refined+fused+zvc+keep",
     "VDNN_ALL+refined+fused+zvc+budget3.0", "VDNN_ALL+refined+fused+zvc+budget3.3", "VDNN_ALL+refined+fused+zvc+budget4.0",
-    "VDNN_ALL+refined+fused+zvc+inplace+budget3.4", "VDNN_ALL+refined+fused+zvc+inplace+budget3.5+lag10",
+    "VDNN_ALL+refined+fused+zvc+inplace+budget3.4", "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.0",
+    "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.1", "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.2+lag8",
     "BASELINE+bf16+fused", "VDNN_ALL+refined+ahead+bf16+fused+zvc", "VDNN_ALL+refined+bf16+fused+zvc+keep",
-    "VDNN_ALL+refined+bf16+fused+zvc+budget5.9", "VDNN_ALL+refined+bf16+fused+zvc+keep+inplace",
+    "VDNN_ALL+refined+bf16+fused+zvc+budget5.9", "VDNN_ALL+refined+bf16+fused+zvc+keep+inplace+recompute",
 ])
 
 
@@ -217,12 +218,13 @@ def main():
         # tensors are packed (no zero elements); "+keep" the packed tensors stay in device memory; "+tail" the deepest
         # 0.75 G elements of the offload set stay on the device; "+budgetX" the policy meets a budget of the fp32
         # BASELINE's peak / X by choosing a place for every tensor; "+bf16" bfloat16 activation storage; "+inplace" input
-        # gradients written over the inputs nothing reads again; "+lagN" blocks recycled N layers after their offload
+        # gradients written over the inputs nothing reads again; "+recompute" the first layer's output computed again in
+        # backward instead of kept; "+lagN" blocks recycled N layers after their offload
         word, *mods = name.split("+")
         budget = [float(m[6:]) for m in mods if m.startswith("budget")]
         lag_given = [int(m[3:]) for m in mods if m.startswith("lag")]
         mods = [m for m in mods if not m.startswith("budget") and not m.startswith("lag")]
-        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep", "inplace"}, name
+        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep", "inplace", "recompute"}, name
         _, policy, algo = parse("VGG16_128", word, args.algo)
         bf16 = args.bf16 or "bf16" in mods
         # (what a plan sends over the link gets the slack that hides it: a lag of fourteen layers on the way out, fetched
@@ -232,7 +234,7 @@ def main():
         lag, depth = (6, 2) if "slack" in mods else (14, 1) if budget else (6, 1) if ahead else (args.offload_lag, args.prefetch_depth)
         if lag_given:
             lag = lag_given[0]
-        kw = dict(refined="refined" in mods, in_place="inplace" in mods, cap_bytes=int(args.cap_gb * 1e9), bf16=bf16, offload_lag=lag, prefetch_depth=depth,
+        kw = dict(refined="refined" in mods, in_place="inplace" in mods, recompute_first="recompute" in mods, cap_bytes=int(args.cap_gb * 1e9), bf16=bf16, offload_lag=lag, prefetch_depth=depth,
                   fuse="fused" in mods, compress="zvc" in mods, prefetch_within_peak=ahead, keep_packed="keep" in mods,
                   keep_tail_bytes=int(0.75e9) * (2 if bf16 else 4) if "tail" in mods else int(args.keep_tail_gb * 1e9))
         if budget:

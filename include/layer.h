@@ -130,6 +130,8 @@ public:
     int     convolutionForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, void* workSpace, bool isDynamic);
     int     convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
                                 void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
+    /* Addition (recomputeFirstLayer): the forward kernel once more, from this layer's srcData into the given block */
+    int     forwardAgainInto(void* into, bool isDynamic);
     int     convolutionBackwardOverSrc(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
                                        void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
     // FC_GEMM layer

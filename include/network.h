@@ -97,6 +97,14 @@ struct NetworkOptions {
     // holds x, dy and dx of a layer together (layer.cu:599, 999-1011); here the largest layer holds two of them.
     // Needs refinedLifetimes; not BASELINE (whose dx/dy pair is shared by all layers).
     bool     inPlaceBackward = false;
+    // The output of a first layer that is a convolution over at most four input channels (half a millisecond for
+    // VGG16's, against 16 ms on the link or 1.6 GB of device memory for the tensor) is released once its consumer's
+    // forward has read it and computed again, by the same kernel from the same filter (layer 0's update comes last), into
+    // a fresh block just before the consumer's backward: the same bits. The network input then stays on the device
+    // whatever the policy says. Applies where the consumer is layer 1, or layer 2 behind a ReLU that layer 0 applies
+    // itself (fuseActivations); needs refinedLifetimes; not BASELINE. The reference keeps or offloads every such
+    // tensor (network.cu:916-936).
+    bool     recomputeFirstLayer = false;
     std::vector<unsigned char> forcedPlacement; // (internal: the replay's placement per layer, see Placement)
     bool     tracePeaks = false;          // (internal: the replay records bytes in use per forward and backward layer)
     int      device = DEFAULT_DEVICE;
@@ -191,6 +199,8 @@ public:
     vdnnAlgoMode_t  algo() const            { return algoMode; }
     vdnn_ctx*       context()               { return ctx; }
     bool            isOffloaded(int l) const { return isOffload[l]; }
+    // recomputeFirstLayer: the layer whose input is computed again before its backward (-1: none)
+    int             recomputedSrcLayer() const { return recomputedLayer; }
     // inPlaceBackward: layer l's backward writes its input gradient over its input
     bool            gradOverSrc(int l) const { return l >= 0 && l < numLayers && layer[l] && layer[l]->GradOverSrc(); }
     // synthetic data: N(0,1) input, integer labels in [0, classes) as a one-hot target, seeded filters
@@ -271,6 +281,7 @@ private:
     bool                isOffload[DEFAULT_NUM_LAYER];
     bool                isPrefetched[DEFAULT_NUM_LAYER];
     bool                dropSrcAfterFwd[DEFAULT_NUM_LAYER]; // refined lifetimes: srcData is dead after forward
+    int                 recomputedLayer = -1;               // recomputeFirstLayer: the layer whose srcData layer 0 computes again in backward
     DATATYPE*           offloadedSrcData_h[DEFAULT_NUM_LAYER];
 
     /* Events that order the copy streams against the compute stream (addition) */

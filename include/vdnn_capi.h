@@ -38,6 +38,7 @@ typedef struct {
     int      compress_offload;  /* offloaded rectified tensors cross the link without their zero elements (lossless; layer.cu:969-987 copies them whole) */
     size_t   hbm_budget_bytes;  /* a limit on pool bytes in use that the policy meets by choosing, per member of its offload set (network.cu:898-936), between the device, a packed stream on the device and host memory (0 = the policy's own set) */
     int      in_place_backward; /* a layer's input gradient is written over its input where nothing reads that again (layer.cu:599 allocates it beside x and dy); needs refined_lifetimes */
+    int      recompute_first_layer; /* the output of a first convolution over at most four channels is computed again before its consumer's backward instead of kept or offloaded (network.cu:916-936 keeps or moves it); needs refined_lifetimes */
 } vdnn_network_options;
 
 typedef struct {
@@ -94,6 +95,8 @@ void vdnn_network_reset_peak(vdnn_network* net);
 int  vdnn_network_is_offloaded(vdnn_network* net, int l);
 /* in_place_backward: 1 where layer l's backward writes its input gradient over its input */
 int  vdnn_network_grad_over_src(vdnn_network* net, int l);
+/* recompute_first_layer: the layer whose input layer 0 computes again before that layer's backward, or -1 */
+int  vdnn_network_recomputed_layer(vdnn_network* net);
 /* hbm_budget_bytes: the place of layer l's input (0 no plan / not a member of the offload set, 1 on the device, 2 packed on
  * the device, 3 host memory), whether the plan's replay met the budget, and what it peaked at */
 int  vdnn_network_placement(vdnn_network* net, int l);

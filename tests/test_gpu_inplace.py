@@ -166,14 +166,21 @@ def test_networks_that_write_gradients_over_inputs_keep_every_bit(cnn, batch, al
     for policy, kw in ((VDNN_NONE, {}), (VDNN_CONV, {}), (VDNN_ALL, {}), (VDNN_ALL, {"host_sync": True}),
                        (VDNN_ALL, {"offload_lag": 6, "prefetch_depth": 3}), (VDNN_ALL, {"unfused_optimizer": True}),
                        (VDNN_ALL, {"compress": True}), (VDNN_ALL, {"compress": True, "keep_packed": True}),
-                       (VDNN_CONV, {"compress": True, "prefetch_within_peak": True, "offload_lag": 4})):
+                       (VDNN_CONV, {"compress": True, "prefetch_within_peak": True, "offload_lag": 4}),
+                       # the first layer's output computed again before its consumer's backward instead of kept or moved
+                       (VDNN_NONE, {"recompute_first": True}), (VDNN_ALL, {"recompute_first": True, "offload_lag": 2}),
+                       (VDNN_ALL, {"recompute_first": True, "compress": True, "keep_packed": True}),
+                       (VDNN_CONV, {"recompute_first": True, "compress": True, "host_sync": True}),
+                       (VDNN_ALL, {"recompute_first": True, "unfused_optimizer": True, "prefetch_depth": 2})):
         announce("in-place networks", cnn, batch, "policy", policy, kw, "fused rectifiers")
-        with make(policy, refined=True, fuse=True, **kw) as net:
+        with make(policy, refined=True, fuse=True, **{k: v for k, v in kw.items() if k != "recompute_first"}) as net:
             peak_apart = net_peak(net)
         with make(policy, refined=True, fuse=True, in_place=True, **kw) as net:
             got = run_steps(net, 2)
             peak = net.stats()["peak_bytes_in_use"]
             offloaded = {l for l in range(net.num_layers) if net.is_offloaded(l)}
+            if kw.get("recompute_first"):   # (every table here starts convolution, ReLU, consumer)
+                assert net.recomputed_layer() == 2 and not net.is_offloaded(0) and not net.is_offloaded(2)
         if kw.get("compress"):   # a layer whose input is a packed stream expands it itself and masks as in BASELINE
             offloaded = {l for l in offloaded if not rectified(specs, l)}
         assert_fused_matches(got, plain, specs, "policy %d %s" % (policy, kw), offloaded)

@@ -28,6 +28,7 @@ static NetworkOptions to_options(const vdnn_network_options* o) {
     n.prefetchWithinPeak = o->prefetch_within_peak != 0;
     n.hbmBudgetBytes = o->hbm_budget_bytes;
     n.inPlaceBackward = o->in_place_backward != 0;
+    n.recomputeFirstLayer = o->recompute_first_layer != 0;
     return n;
 }
 
@@ -52,6 +53,7 @@ void vdnn_network_default_options(vdnn_network_options* o) {
     o->compress_offload = d.compressOffload;
     o->hbm_budget_bytes = d.hbmBudgetBytes;
     o->in_place_backward = d.inPlaceBackward;
+    o->recompute_first_layer = d.recomputeFirstLayer;
 }
 
 vdnn_network* vdnn_network_create(int cnn, int policy, int algo, int batch, const vdnn_network_options* o) {
@@ -145,6 +147,7 @@ int vdnn_network_is_offloaded(vdnn_network* h, int l) {
 }
 
 int vdnn_network_grad_over_src(vdnn_network* h, int l) { return h->net->gradOverSrc(l) ? 1 : 0; }
+int vdnn_network_recomputed_layer(vdnn_network* h) { return h->net->recomputedSrcLayer(); }
 
 int vdnn_network_placement(vdnn_network* h, int l) { return (int)h->net->placementOf(l); }
 int vdnn_network_plan_feasible(vdnn_network* h) { return h->net->planFeasible() ? 1 : 0; }

@@ -260,6 +260,22 @@ int Layer::convolutionForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, 
     return 0;
 }
 
+/* Addition (recomputeFirstLayer): what convolutionForward computed, again, from the same input and filter into `into`
+ * (the workspace of the pass comes from the pool as in the forward of the offloading policies). */
+int Layer::forwardAgainInto(void* into, bool isDynamic) {
+    M_ASSERT((layerType == CONV || layerType == FC_CONV) && srcData && into, "only a convolution with its input on the device computes its output again");
+    void* curWorkSpace = nullptr;
+    if (mallocWorkSpace(nullptr, fwdWorkSpaceSize, &curWorkSpace, isDynamic) < 0) return -1;
+    if (fuseRelu)
+        checkVDNN(vdnn_conv_fwd_relu(ctx, *stream_compute, &shape, vdnnAlgoMode, srcData, (const float*)filterData,
+                                     (const float*)biasData, into, curWorkSpace, fwdWorkSpaceSize));
+    else
+        checkVDNN(vdnn_conv_fwd(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)filterData,
+                                (const float*)biasData, (float*)into, curWorkSpace, fwdWorkSpaceSize));
+    freeWorkSpace(nullptr, fwdWorkSpaceSize, curWorkSpace, isDynamic);
+    return 0;
+}
+
 /* The kernels that may write a layer's input gradient over its input: every lane reads what it overwrites before it
  * does, and nothing else reads the input (vdnn_conv_bwd_data_in_place_ok / vdnn_maxpool_bwd_in_place_ok). */
 bool Layer::canGradOverSrc() const {

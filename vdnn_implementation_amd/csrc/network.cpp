@@ -415,6 +415,17 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
         }
     }
 
+    /* recomputeFirstLayer: the first layer's output is dead after its consumer's forward and comes back by running layer 0
+       again; the network input stays on the device for that */
+    recomputedLayer = -1;
+    if (options.recomputeFirstLayer && refined && numLayers > 2 && is_conv(layer[0]->LayerType()) && layer[0]->InputC() <= 4) {
+        const int consumer = layer[1]->Elided() ? 2 : (specs[1].type == RELU || specs[1].type == TANH || specs[1].type == SIGMOID ? -1 : 1);
+        if (consumer > 0 && consumer < numLayers - 1) {
+            recomputedLayer = consumer;
+            dropSrcAfterFwd[consumer] = true;
+        }
+    }
+
     /* keepTailBytes: the deepest members of the offload set stay on the device */
     int tailStart = numLayers;
     {
@@ -434,7 +445,8 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
     std::vector<bool> member(numLayers, false);
     for (int l = 0; l < numLayers - 1; l++) {
         const bool named = newVdnnType == VDNN_ALL || (newVdnnType == VDNN_CONV && is_conv(layer[l]->LayerType()));
-        member[l] = named && !dropSrcAfterFwd[l]     /* released, not moved: nothing reads it again */
+        member[l] = named && !dropSrcAfterFwd[l]     /* released, not moved: nothing reads it again (or layer 0 computes it again) */
+                    && !(l == 0 && recomputedLayer > 0)  /* the input that layer 0 will read again */
                     && !layer[l]->Elided()           /* its input is the next layer's srcData, which has its own turn */
                     && l < tailStart;
     }
@@ -794,6 +806,12 @@ int Network::backwardPropagation(bool isDynamic) {
                     layer[l]->copyDstData(nullptr);
                     dstReleased = true;
                 }
+            }
+            /* recomputeFirstLayer: this layer's input was released behind its forward; layer 0 computes it again */
+            if (l == recomputedLayer) {
+                M_ASSERT(inputResident && layer[0]->SrcData() != nullptr, "the first layer's input has to be on the device to compute its output again");
+                if (layer[l]->cnmemMallocSrcData(isDynamic) < 0) return -1;
+                if (layer[0]->forwardAgainInto(layer[l]->SrcData(), isDynamic) < 0) return -1;
             }
             /* a packed input that stayed on the device is expanded now, not a layer ahead: that takes HBM time only
                (a millisecond for the largest), and so the tensor, its packed block and the working set of the

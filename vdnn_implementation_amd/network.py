@@ -18,7 +18,7 @@ class Options(C.Structure):
                 ("unfused_optimizer", _i), ("defer_optimizer", _i), ("offload_lag", _i), ("prefetch_depth", _i), ("data_type", _i),
                 ("fuse_activations", _i), ("keep_tail_bytes", _sz), ("prefetch_within_peak", _i), ("keep_packed_on_device", _i),
                 ("plan_packed_fraction", C.c_double),
-                ("compress_offload", _i), ("hbm_budget_bytes", _sz), ("in_place_backward", _i)]
+                ("compress_offload", _i), ("hbm_budget_bytes", _sz), ("in_place_backward", _i), ("recompute_first_layer", _i)]
 
 
 class LayerSpec(C.Structure):
@@ -65,6 +65,7 @@ CAPI_SYMBOLS = {
     "vdnn_network_reset_peak": (None, [_vp]),
     "vdnn_network_is_offloaded": (_i, [_vp, _i]),
     "vdnn_network_grad_over_src": (_i, [_vp, _i]),
+    "vdnn_network_recomputed_layer": (_i, [_vp]),
     "vdnn_network_placement": (_i, [_vp, _i]),
     "vdnn_network_plan_feasible": (_i, [_vp]),
     "vdnn_network_plan_peak_bytes": (_sz, [_vp]),
@@ -100,7 +101,7 @@ class Network:
                  pool_bytes=0, cap_bytes=0, plan_only=False, host_sync=False, capture=False, verbose=False, device=0,
                  refined=False, unfused_optimizer=False, defer_optimizer=False, bf16=False, offload_lag=0, prefetch_depth=1,
                  fuse=False, compress=False, keep_tail_bytes=0, prefetch_within_peak=False, keep_packed=False,
-                 plan_packed_fraction=0.0, hbm_budget_bytes=0, in_place=False):
+                 plan_packed_fraction=0.0, hbm_budget_bytes=0, in_place=False, recompute_first=False):
         o = Options()
         lib.vdnn_network_default_options(C.byref(o))
         o.seed, o.pool_bytes, o.cap_bytes = seed, int(pool_bytes), int(cap_bytes)
@@ -117,6 +118,7 @@ class Network:
         o.plan_packed_fraction = float(plan_packed_fraction)
         o.hbm_budget_bytes = int(hbm_budget_bytes)
         o.in_place_backward = int(in_place)
+        o.recompute_first_layer = int(recompute_first)
         if layers is not None:
             arr = (LayerSpec * len(layers))(*layers)
             self._h = lib.vdnn_network_create_custom(arr, len(layers), policy, algo, C.byref(o))
@@ -281,6 +283,10 @@ class Network:
     def grad_over_src(self, l):
         """in_place: layer l's backward writes its input gradient over its input"""
         return bool(lib.vdnn_network_grad_over_src(self._h, l))
+
+    def recomputed_layer(self):
+        """recompute_first: the layer whose input layer 0 computes again before that layer's backward, or -1"""
+        return lib.vdnn_network_recomputed_layer(self._h)
 
     def placement(self):
         """hbm_budget_bytes: per layer, 0 = outside the plan, 1 = on the device, 2 = packed on the device, 3 = host memory."""
