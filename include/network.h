@@ -293,6 +293,7 @@ private:
     vdnn_event_t        evPacked[DEFAULT_NUM_LAYER];      // d2h: the packing kernel has read srcData of layer l
     void*               zvcStaging[DEFAULT_NUM_LAYER];    // staging block of layer l's stream (null: none this step)
     size_t              zvcStagingBytes[DEFAULT_NUM_LAYER];
+    size_t              zvcLengthSeen[DEFAULT_NUM_LAYER] = {};   // the stream length a step's forward sized its block from (0: none known)
     bool                zvcKept[DEFAULT_NUM_LAYER];       // the block holds the stream until layer l's backward has expanded it
     bool                zvcFetched[DEFAULT_NUM_LAYER];    // ... and was filled by a copy from host memory during this backward
     bool                srcReleasedEarly[DEFAULT_NUM_LAYER]; // srcData of layer l went back to the pool behind its forward

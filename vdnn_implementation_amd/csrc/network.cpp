@@ -132,7 +132,7 @@ void Network::construct(vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) {
         offloadedSrcData_h[i] = nullptr;
         evFwdDone[i] = evOffloadDone[i] = evBlockFree[i] = evPrefetchDone[i] = evPacked[i] = nullptr;
         zvcStaging[i] = nullptr;
-        zvcStagingBytes[i] = 0;
+        zvcStagingBytes[i] = 0; zvcLengthSeen[i] = 0;
         zvcKept[i] = zvcFetched[i] = false;
         srcReleasedEarly[i] = false;
         keepPackedLayer[i] = false;
@@ -211,7 +211,7 @@ void Network::reset(CNN_t _cnnType, vdnn_t _vdnnType, vdnnAlgoMode_t _algoMode) 
     /* so is every block the last step still held: a trial step of the dynamic ladder may have stopped half-way */
     for (int i = 0; i < DEFAULT_NUM_LAYER; i++) {
         zvcStaging[i] = nullptr;
-        zvcStagingBytes[i] = 0;
+        zvcStagingBytes[i] = 0; zvcLengthSeen[i] = 0;
         zvcKept[i] = zvcFetched[i] = false;
         srcReleasedEarly[i] = false;
     }
@@ -674,6 +674,7 @@ int Network::forwardPropagation(bool isDynamic) {
                 const size_t assumed = options.planPackedFraction > 0.0
                                            ? (size_t)(options.planPackedFraction * (double)(layer[l]->SrcDataSize() * actBytes())) : longest;
                 const size_t known = options.planOnly ? assumed : (size_t)zvcLength_h[l];
+                zvcLengthSeen[l] = known; /* backward sizes the way back from the same figure, whatever the word holds by then */
                 size_t want = known ? known + known / 32 + 65536 : 0;
                 want = std::min(longest, (want + 15) / 16 * 16);
                 if (want && ASSERT_EQ(vdnn_pool_malloc(ctx, &zvcStaging[l], want), isDynamic) < 0) return -1;
@@ -941,7 +942,9 @@ size_t Network::stagedFetchBytes(int id) const {
     const size_t longest = vdnn_zvc_buffer_bytes(layer[id]->SrcDataSize(), (int)actBytes());
     const size_t assumed = options.planPackedFraction > 0.0
                                ? (size_t)(options.planPackedFraction * (double)(layer[id]->SrcDataSize() * actBytes())) : longest;
-    const size_t known = options.planOnly ? assumed : (zvcLength_h ? (size_t)zvcLength_h[id] : 0);
+    /* the length this step's forward went by (the step before's; none in a first step, whose streams then come back
+       through the expanding kernel): the pinned word itself changes while the step runs */
+    const size_t known = options.planOnly ? assumed : zvcLengthSeen[id];
     if (!known) return 0;
     return std::min(longest, (known + known / 32 + 65536 + 15) / 16 * 16);
 }
