@@ -373,20 +373,11 @@ struct StoreNCHW {
     }
     __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int ks, const GemmDims& d, bool to_partial) const {
         const int l32 = lane & 31, lk = lane >> 5;
-        // Bias and gate values are read before the stores they feed, a column block at a time: a load that follows
-        // a store through a pointer it might share has to be issued behind it, and with the load's result needed
-        // for the next store that is one round trip to memory per element. (A gate that *is* the output tensor -
-        // the gradient written over the layer's own input - is read by the lane that overwrites it, before it does.)
-        float bv[2][16];
-        if (!to_partial && bias) {
-#pragma unroll
-            for (int it = 0; it < 2; it++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const int m = m0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
-                    bv[it][v] = m < d.M ? bias[m] : 0.0f;
-                }
-        }
+        // Bias and gate values are read before the stores they feed, eight at a time: a load that follows a store
+        // through a pointer it might share has to be issued behind it, and with the load's result needed for the next
+        // store that is one round trip to memory per element. Eight, not the whole tile: the registers they wait in
+        // count against the three workgroups a compute unit holds. (A gate that *is* the output tensor - the gradient
+        // written over the layer's own input - is read by the lane that overwrites it, before it does.)
 #pragma unroll
         for (int jt = 0; jt < 2; jt++) {
             const int j = j0 + jt * 32 + l32;
@@ -395,30 +386,38 @@ struct StoreNCHW {
             const size_t base = (size_t)n * d.M * opix + pix;
             E* o = out + base;
             float* po = partial + (size_t)ks * d.M * d.N + base;
-            float gt[2][16];
-            if (!to_partial && gate) {
-#pragma unroll
-                for (int it = 0; it < 2; it++)
-#pragma unroll
-                    for (int v = 0; v < 16; v++) {
-                        const int m = m0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
-                        gt[it][v] = m < d.M ? load_elem(gate + base + (size_t)m * opix) : 1.0f;
-                    }
-            }
 #pragma unroll
             for (int it = 0; it < 2; it++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const int m = m0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
-                    if (m >= d.M) continue;
-                    float r = acc[it][jt][v];
-                    if (to_partial) {
-                        po[(size_t)m * opix] = r;
-                    } else {
-                        if (bias) r += bv[it][v];
-                        if (relu) r = relu_value(r);
-                        if (gate) r = gt[it][v] > 0.0f ? r : 0.0f;
-                        store_elem(o + (size_t)m * opix, r);
+                for (int h = 0; h < 2; h++) {
+                    float bv[8], gt[8];
+                    if (!to_partial && bias) {
+#pragma unroll
+                        for (int u = 0; u < 8; u++) {
+                            const int v = 8 * h + u, m = m0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+                            bv[u] = m < d.M ? bias[m] : 0.0f;
+                        }
+                    }
+                    if (!to_partial && gate) {
+#pragma unroll
+                        for (int u = 0; u < 8; u++) {
+                            const int v = 8 * h + u, m = m0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+                            gt[u] = m < d.M ? load_elem(gate + base + (size_t)m * opix) : 1.0f;
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        const int v = 8 * h + u, m = m0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+                        if (m >= d.M) continue;
+                        float r = acc[it][jt][v];
+                        if (to_partial) {
+                            po[(size_t)m * opix] = r;
+                        } else {
+                            if (bias) r += bv[u];
+                            if (relu) r = relu_value(r);
+                            if (gate) r = gt[u] > 0.0f ? r : 0.0f;
+                            store_elem(o + (size_t)m * opix, r);
+                        }
                     }
                 }
         }
