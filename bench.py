@@ -38,7 +38,7 @@ DEFAULT_POLICIES = ",".join([
     "VDNN_ALL+refined+fused+zvc+keep",
     "VDNN_ALL+refined+fused+zvc+budget3.0", "VDNN_ALL+refined+fused+zvc+budget3.3", "VDNN_ALL+refined+fused+zvc+budget4.0",
     "VDNN_ALL+refined+fused+zvc+inplace+budget3.4", "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.0",
-    "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.1", "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.2+lag8",
+    "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.1", "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.2",
     "BASELINE+bf16+fused", "VDNN_ALL+refined+ahead+bf16+fused+zvc", "VDNN_ALL+refined+bf16+fused+zvc+keep",
     "VDNN_ALL+refined+bf16+fused+zvc+budget5.9", "VDNN_ALL+refined+bf16+fused+zvc+keep+inplace+recompute",
 ])
@@ -91,7 +91,7 @@ def run_config(Network, be, cnn, policy, algo, batch, steps, warmup, profile_ste
         plan = None
         if kw.get("hbm_budget_bytes"):
             places = net.placement()
-            plan = {"budget_gb": kw["hbm_budget_bytes"] / 1e9, "feasible": net.plan_feasible(), "plan_peak_gb": net.plan_peak_bytes() / 1e9,
+            plan = {"budget_gb": kw["hbm_budget_bytes"] / 1e9, "feasible": net.plan_feasible(), "plan_peak_gb": net.plan_peak_bytes() / 1e9, "offload_lag": net.offload_lag(),
                     "on_device": places.count(1), "packed_on_device": places.count(2), "over_the_link": places.count(3)}
     finally:
         net.close()
@@ -227,11 +227,10 @@ def main():
         assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep", "inplace", "recompute"}, name
         _, policy, algo = parse("VGG16_128", word, args.algo)
         bf16 = args.bf16 or "bf16" in mods
-        # (what a plan sends over the link gets the slack that hides it: a lag of fourteen layers on the way out, fetched
-        # ahead on the way back wherever the peak allows)
+        # (what a plan sends over the link gets the slack that hides it: the plan chooses the offload lag itself - the
+        # longest of those that fit with the fewest bytes on the link - and backward fetches ahead wherever the peak allows)
         ahead = "ahead" in mods or bool(budget)
-        # (a plan holds what waits for its copy as a packed stream, and its replay counts it: a long lag costs it no memory)
-        lag, depth = (6, 2) if "slack" in mods else (14, 1) if budget else (6, 1) if ahead else (args.offload_lag, args.prefetch_depth)
+        lag, depth = (6, 2) if "slack" in mods else (-1, 1) if budget else (6, 1) if ahead else (args.offload_lag, args.prefetch_depth)
         if lag_given:
             lag = lag_given[0]
         kw = dict(refined="refined" in mods, in_place="inplace" in mods, recompute_first="recompute" in mods, cap_bytes=int(args.cap_gb * 1e9), bf16=bf16, offload_lag=lag, prefetch_depth=depth,

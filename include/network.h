@@ -41,7 +41,7 @@ struct NetworkOptions {
     // copy that is longer than its own layer's kernels overlaps the following layers instead of stalling
     // them. prefetchDepth: up to that many offloaded tensors below the current layer are in flight or
     // resident ahead of their backward (the reference fetches one, network.cu:1193-1208).
-    int      offloadLag = 0;
+    int      offloadLag = 0;        // negative with hbmBudgetBytes: the placement plan chooses the lag as well (0 otherwise)
     int      prefetchDepth = 1;
     bool     unfusedOptimizer = false;
     bool     deferOptimizer = false;
@@ -232,6 +232,8 @@ public:
     Placement       placementOf(int l) const { return l >= 0 && l < (int)placement.size() ? (Placement)placement[l] : PLACE_POLICY; }
     bool            planFeasible() const { return planFeasibleFlag; }
     size_t          planPeakBytes() const { return planBudgetPeak; }
+    // the offload lag the step runs with: offloadLag, or - where that is negative - the one the placement plan chose
+    int             offloadLagInUse() const { return options.offloadLag >= 0 ? options.offloadLag : plannedLag; }
     const std::vector<LayerSpec>& table() const { return specs; }
     static std::vector<LayerSpec> tableFor(CNN_t cnn, int batch);
 
@@ -312,6 +314,7 @@ private:
     bool                keepPackedLayer[DEFAULT_NUM_LAYER]; // the packed stream of layer l's input stays on the device
     bool                planFeasibleFlag = true;
     size_t              planBudgetPeak = 0;
+    int                 plannedLag = 0;
     std::vector<unsigned char> planPlacement(vdnn_t policy, const std::vector<bool>& member);
     std::vector<int>    planIssueLayer;
     size_t              planPeak = 0, peakBudget = 0;

@@ -101,6 +101,8 @@ int  vdnn_network_recomputed_layer(vdnn_network* net);
  * the device, 3 host memory), whether the plan's replay met the budget, and what it peaked at */
 int  vdnn_network_placement(vdnn_network* net, int l);
 int  vdnn_network_plan_feasible(vdnn_network* net);
+/* the offload lag in use: offload_lag, or the one the placement plan chose where that is negative */
+int  vdnn_network_offload_lag(vdnn_network* net);
 size_t vdnn_network_plan_peak_bytes(vdnn_network* net);
 /* (backward layer, prefetched layer) pairs of the last backward, Network::findPrefetchLayer
  * (network.cu:1198-1208); returns the number of pairs */

@@ -171,9 +171,19 @@ def test_networks_that_write_gradients_over_inputs_keep_every_bit(cnn, batch, al
                        (VDNN_NONE, {"recompute_first": True}), (VDNN_ALL, {"recompute_first": True, "offload_lag": 2}),
                        (VDNN_ALL, {"recompute_first": True, "compress": True, "keep_packed": True}),
                        (VDNN_CONV, {"recompute_first": True, "compress": True, "host_sync": True}),
-                       (VDNN_ALL, {"recompute_first": True, "unfused_optimizer": True, "prefetch_depth": 2})):
+                       (VDNN_ALL, {"recompute_first": True, "unfused_optimizer": True, "prefetch_depth": 2}),
+                       # a budget halfway between the floor and what the schedule holds unplaced; the plan chooses the lag
+                       (VDNN_ALL, {"recompute_first": True, "compress": True, "plan_packed_fraction": 0.7, "hbm_budget_bytes": "middle",
+                                   "offload_lag": -1, "prefetch_within_peak": True})):
+        if kw.get("hbm_budget_bytes") == "middle":
+            rest = {k: v for k, v in kw.items() if k != "hbm_budget_bytes"}
+            with make(policy, refined=True, fuse=True, in_place=True, plan_only=True, hbm_budget_bytes=1, **rest) as probe:
+                floor = probe.plan_peak_bytes()
+            with make(policy, refined=True, fuse=True, in_place=True, plan_only=True, hbm_budget_bytes=1 << 50, **rest) as probe:
+                ceiling = probe.plan_peak_bytes()
+            kw = dict(kw, hbm_budget_bytes=(floor + ceiling) // 2)
         announce("in-place networks", cnn, batch, "policy", policy, kw, "fused rectifiers")
-        with make(policy, refined=True, fuse=True, **{k: v for k, v in kw.items() if k != "recompute_first"}) as net:
+        with make(policy, refined=True, fuse=True, **{k: v for k, v in kw.items() if k not in ("recompute_first", "hbm_budget_bytes")}) as net:
             peak_apart = net_peak(net)
         with make(policy, refined=True, fuse=True, in_place=True, **kw) as net:
             got = run_steps(net, 2)
@@ -184,6 +194,8 @@ def test_networks_that_write_gradients_over_inputs_keep_every_bit(cnn, batch, al
         if kw.get("compress"):   # a layer whose input is a packed stream expands it itself and masks as in BASELINE
             offloaded = {l for l in offloaded if not rectified(specs, l)}
         assert_fused_matches(got, plain, specs, "policy %d %s" % (policy, kw), offloaded)
+        if "hbm_budget_bytes" in kw:
+            continue   # (a budget keeps on the device what fits: more than the policy's own offload set would)
         assert peak <= peak_apart
         shrinks += peak < peak_apart
     if cnn == VGG16_128:   # (the small tables' peaks are the parameters and the staging area)

@@ -716,6 +716,37 @@ def test_first_layer_computed_again_instead_of_kept():
             assert live_blocks(net) == n0
 
 
+def test_the_plan_chooses_the_offload_lag():
+    """offload_lag < 0 with a budget: the lag is part of the plan. What waits for its copy counts against the budget for
+    as long as the lag, so the longest lag is not always the one that fits with the fewest bytes on the link. VGG16 batch
+    128 with gradients over inputs and the first layer computed again: down to BASELINE / 4.1 fourteen layers fit, at
+    BASELINE / 4.2 eight, and below the floor the plan with the lowest peak stands."""
+    kw = dict(refined=True, fuse=True, compress=True, plan_packed_fraction=0.6, in_place=True, recompute_first=True, prefetch_within_peak=True)
+    with plan(VGG16_128, BASELINE) as net:
+        step(net)
+        base = net.stats()["peak_bytes_in_use"]
+    seen = {}
+    for ratio in (4.0, 4.1, 4.2, 4.5, 5.0):
+        with plan(VGG16_128, VDNN_ALL, hbm_budget_bytes=int(base / ratio), offload_lag=-1, **kw) as net:
+            n0 = live_blocks(net)
+            step(net); step(net)
+            assert live_blocks(net) == n0
+            seen[ratio] = (net.offload_lag(), net.plan_feasible(), net.placement().count(3), net.stats()["peak_bytes_in_use"])
+            assert net.stats()["peak_bytes_in_use"] == net.plan_peak_bytes()
+            # the same plan with that lag spelt out
+            with plan(VGG16_128, VDNN_ALL, hbm_budget_bytes=int(base / ratio), offload_lag=net.offload_lag(), **kw) as fixed:
+                assert fixed.placement() == net.placement() and fixed.plan_peak_bytes() == net.plan_peak_bytes()
+    assert seen[4.0][:3] == (14, True, 0) and seen[4.1][:3] == (14, True, 1) and seen[4.2][:3] == (8, True, 1)
+    assert seen[4.5][1] and seen[4.5][0] < 8 and seen[4.5][2] == 1
+    assert not seen[5.0][1] and abs(seen[5.0][3] / GB - 3.99) < 0.01
+    for ratio in (4.0, 4.1, 4.2, 4.5):
+        assert seen[ratio][3] <= base / ratio
+    # without a budget a negative lag is no lag
+    with plan(VGG16_128, VDNN_ALL, offload_lag=-1, refined=True) as a, plan(VGG16_128, VDNN_ALL, offload_lag=0, refined=True) as b:
+        step(a); step(b)
+        assert a.offload_lag() == 0 and a.stats() == b.stats()
+
+
 def test_packed_streams_come_back_through_a_block_of_their_own_length():
     """A packed stream that crossed the link returns through the copy engine into a block sized from its length, a layer
     ahead of its backward; the layer itself expands it. What is held a layer ahead is the stream, not the tensor: the

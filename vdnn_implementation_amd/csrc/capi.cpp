@@ -147,6 +147,7 @@ int vdnn_network_is_offloaded(vdnn_network* h, int l) {
 }
 
 int vdnn_network_grad_over_src(vdnn_network* h, int l) { return h->net->gradOverSrc(l) ? 1 : 0; }
+int vdnn_network_offload_lag(vdnn_network* h) { return h->net->offloadLagInUse(); }
 int vdnn_network_recomputed_layer(vdnn_network* h) { return h->net->recomputedSrcLayer(); }
 
 int vdnn_network_placement(vdnn_network* h, int l) { return (int)h->net->placementOf(l); }

@@ -453,6 +453,7 @@ void Network::setVdnnType(vdnn_t newVdnnType) {
     /* hbmBudgetBytes: each member's place comes from a plan (the replay is handed one, the network itself makes one) */
     placement.assign(numLayers, PLACE_POLICY);
     planFeasibleFlag = true;
+    plannedLag = 0;
     if (newVdnnType == VDNN_ALL || newVdnnType == VDNN_CONV) {
         if ((int)options.forcedPlacement.size() == numLayers) placement = options.forcedPlacement;
         else if (options.hbmBudgetBytes > 0 && !options.tracePeaks) placement = planPlacement(newVdnnType, member);
@@ -717,7 +718,7 @@ int Network::forwardPropagation(bool isDynamic) {
                 ASSERT_EQ(vdnn_pool_free(ctx, layer[l]->SrcData()), isDynamic);
                 layer[l]->copySrcData(nullptr);
             }
-            const int lag = options.hostSync ? 0 : options.offloadLag;
+            const int lag = options.hostSync ? 0 : offloadLagInUse();
             while (!pendingOffload.empty() && (pendingOffload.front() + lag <= l || l == numLayers - 1)) {
                 const int j = pendingOffload.front();
                 pendingOffload.erase(pendingOffload.begin());
@@ -998,6 +999,7 @@ void Network::buildPeakPlan(vdnn_t policy) {
     o.planOnly = true; o.tracePeaks = true; o.prefetchWithinPeak = false;
     o.capture = false; o.verbose = false; o.capBytes = 0;
     o.hbmBudgetBytes = 0; o.forcedPlacement = placement; /* the replay takes this network's plan, it makes none */
+    o.offloadLag = offloadLagInUse();
     Network replay(specs, policy, algoMode == VDNN_DYNAMIC_ALGO ? VDNN_MEMORY_OPT_ALGO : algoMode, o);
     if (replay.forwardPropagation(false) < 0 || replay.backwardPropagation(false) < 0) return;
     planBwdPeak = replay.backwardPeakTrace();
@@ -1012,51 +1014,78 @@ void Network::buildPeakPlan(vdnn_t policy) {
  * host memory. Ends when the replay fits or nothing that is stored at the peak can move any further: then the peak is
  * the working set of the layer itself, which no placement changes. */
 std::vector<unsigned char> Network::planPlacement(vdnn_t policy, const std::vector<bool>& member) {
-    std::vector<unsigned char> place(numLayers, PLACE_POLICY);
-    for (int l = 0; l < numLayers; l++) if (member[l]) place[l] = PLACE_RESIDENT;
     NetworkOptions o = options;
     o.planOnly = true; o.tracePeaks = true; o.prefetchWithinPeak = false; o.hbmBudgetBytes = 0;
     o.capture = false; o.verbose = false; o.capBytes = 0; o.keepPackedOnDevice = false; o.keepTailBytes = 0;
     const vdnnAlgoMode_t mode = algoMode == VDNN_DYNAMIC_ALGO ? VDNN_MEMORY_OPT_ALGO : algoMode;
-    planFeasibleFlag = false;
-    for (int round = 0; round <= 2 * numLayers; round++) {
-        o.forcedPlacement = place;
-        size_t peak = 0; int at = 0; bool inBackward = false;
-        {
-            Network replay(specs, policy, mode, o);
-            /* two steps: the first forward of a packed stream has no length to size its block by */
-            for (int step = 0; step < 2; step++)
-                if (replay.forwardPropagation(true) < 0 || replay.backwardPropagation(true) < 0) return place;
-            for (int l = 0; l < numLayers; l++) {
-                if (replay.forwardPeakTrace()[l] > peak) { peak = replay.forwardPeakTrace()[l]; at = l; inBackward = false; }
-                if (replay.backwardPeakTrace()[l] > peak) { peak = replay.backwardPeakTrace()[l]; at = l; inBackward = true; }
+    struct Plan { std::vector<unsigned char> place; bool feasible = false; size_t peak = 0; double link = 0.0; int lag = 0; };
+    auto plan_with = [&](int lag) {
+        Plan p;
+        p.lag = lag;
+        p.place.assign(numLayers, PLACE_POLICY);
+        std::vector<unsigned char>& place = p.place;
+        for (int l = 0; l < numLayers; l++) if (member[l]) place[l] = PLACE_RESIDENT;
+        o.offloadLag = lag;
+        for (int round = 0; round <= 2 * numLayers; round++) {
+            o.forcedPlacement = place;
+            size_t peak = 0; int at = 0;
+            {
+                Network replay(specs, policy, mode, o);
+                /* two steps: the first forward of a packed stream has no length to size its block by */
+                for (int step = 0; step < 2; step++)
+                    if (replay.forwardPropagation(true) < 0 || replay.backwardPropagation(true) < 0) return p;
+                for (int l = 0; l < numLayers; l++) {
+                    if (replay.forwardPeakTrace()[l] > peak) { peak = replay.forwardPeakTrace()[l]; at = l; }
+                    if (replay.backwardPeakTrace()[l] > peak) { peak = replay.backwardPeakTrace()[l]; at = l; }
+                }
             }
-        }
-        planBudgetPeak = peak;
-        if (peak <= options.hbmBudgetBytes) { planFeasibleFlag = true; break; }
-        /* stored at the peak: every member below the layer at work (in forward it has been written and left behind, in
-           backward it still waits for its turn) */
-        const double f = options.planPackedFraction > 0.0 ? options.planPackedFraction : 1.04;
-        /* a stream on the device costs two passes at HBM speed, the link a hundred times that: everything stored at the
-           peak that can be packed is packed before anything crosses the link; within a kind, the largest gain first */
-        int pick = -1; double best = 0.0; unsigned char to = PLACE_LINK;
-        for (int pass = 0; pass < 2 && pick < 0; pass++) {
-            for (int l = 0; l < at; l++) {
-                if (!member[l] || place[l] == PLACE_LINK) continue;
-                const double size = (double)(layer[l]->SrcDataSize() * actBytes());
-                const bool canPack = options.compressOffload && srcIsRectified(l) && f < 1.0;
-                const bool pack = place[l] == PLACE_RESIDENT && canPack;
-                if (pack != (pass == 0)) continue;
-                /* what the step down gives back: packing leaves f of the tensor, the link takes what is there */
-                const double gain = pack ? (1.0 - f) * size : (place[l] == PLACE_PACKED ? f * size : size);
-                if (gain > best) { best = gain; pick = l; to = pack ? PLACE_PACKED : PLACE_LINK; }
+            p.peak = peak;
+            if (peak <= options.hbmBudgetBytes) { p.feasible = true; break; }
+            /* stored at the peak: every member below the layer at work (in forward it has been written and left behind,
+               in backward it still waits for its turn) */
+            const double f = options.planPackedFraction > 0.0 ? options.planPackedFraction : 1.04;
+            /* a stream on the device costs two passes at HBM speed, the link a hundred times that: everything stored at
+               the peak that can be packed is packed before anything crosses the link; within a kind, the largest gain first */
+            int pick = -1; double best = 0.0; unsigned char to = PLACE_LINK;
+            for (int pass = 0; pass < 2 && pick < 0; pass++) {
+                for (int l = 0; l < at; l++) {
+                    if (!member[l] || place[l] == PLACE_LINK) continue;
+                    const double size = (double)(layer[l]->SrcDataSize() * actBytes());
+                    const bool canPack = options.compressOffload && srcIsRectified(l) && f < 1.0;
+                    const bool pack = place[l] == PLACE_RESIDENT && canPack;
+                    if (pack != (pass == 0)) continue;
+                    /* what the step down gives back: packing leaves f of the tensor, the link takes what is there */
+                    const double gain = pack ? (1.0 - f) * size : (place[l] == PLACE_PACKED ? f * size : size);
+                    if (gain > best) { best = gain; pick = l; to = pack ? PLACE_PACKED : PLACE_LINK; }
+                }
             }
+            if (pick < 0) break;
+            place[pick] = to;
         }
-        (void)inBackward;
-        if (pick < 0) break;
-        place[pick] = to;
+        for (int l = 0; l < numLayers; l++)
+            if (place[l] == PLACE_LINK) p.link += (double)(layer[l]->SrcDataSize() * actBytes());
+        return p;
+    };
+    /* offloadLag < 0: the lag is part of the plan. What waits for its copy counts against the budget for as many layers
+       as the lag is long, so a long lag may force more tensors out than a short one; what crosses the link costs time
+       whatever the lag, a short lag only makes the compute stream wait for it sooner. So: of the lags tried, the one
+       whose plan fits with the fewest bytes on the link, the longest of those; if none fits, the lowest peak. */
+    Plan chosen;
+    if (options.offloadLag >= 0) {
+        chosen = plan_with(options.offloadLag);
+    } else {
+        bool have = false;
+        for (int lag : {14, 10, 8, 6, 4, 2, 0}) {
+            Plan p = plan_with(lag);
+            const bool better = !have || (p.feasible != chosen.feasible ? p.feasible
+                                          : p.feasible ? p.link < chosen.link : p.peak < chosen.peak);
+            if (better) { chosen = p; have = true; }
+        }
     }
-    return place;
+    plannedLag = chosen.lag;
+    planFeasibleFlag = chosen.feasible;
+    planBudgetPeak = chosen.peak;
+    return chosen.place;
 }
 
 /* addition (prefetchWithinPeak): the nearest offloaded tensor below currLayerId that is still on the host, if

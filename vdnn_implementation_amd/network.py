@@ -65,6 +65,7 @@ CAPI_SYMBOLS = {
     "vdnn_network_reset_peak": (None, [_vp]),
     "vdnn_network_is_offloaded": (_i, [_vp, _i]),
     "vdnn_network_grad_over_src": (_i, [_vp, _i]),
+    "vdnn_network_offload_lag": (_i, [_vp]),
     "vdnn_network_recomputed_layer": (_i, [_vp]),
     "vdnn_network_placement": (_i, [_vp, _i]),
     "vdnn_network_plan_feasible": (_i, [_vp]),
@@ -283,6 +284,10 @@ class Network:
     def grad_over_src(self, l):
         """in_place: layer l's backward writes its input gradient over its input"""
         return bool(lib.vdnn_network_grad_over_src(self._h, l))
+
+    def offload_lag(self):
+        """the offload lag in use (offload_lag, or what the placement plan chose where that is negative)"""
+        return lib.vdnn_network_offload_lag(self._h)
 
     def recomputed_layer(self):
         """recompute_first: the layer whose input layer 0 computes again before that layer's backward, or -1"""
