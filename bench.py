@@ -41,6 +41,7 @@ DEFAULT_POLICIES = ",".join([
     "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.1", "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.2",
     "BASELINE+bf16+fused", "VDNN_ALL+refined+ahead+bf16+fused+zvc", "VDNN_ALL+refined+bf16+fused+zvc+keep",
     "VDNN_ALL+refined+bf16+fused+zvc+budget5.9", "VDNN_ALL+refined+bf16+fused+zvc+keep+inplace+recompute",
+    "VDNN_ALL+refined+bf16+fused+zvc+inplace+recompute+budget5.0", "VDNN_ALL+refined+bf16+fused+zvc+inplace+recompute+budget6.0",
 ])
 
 
