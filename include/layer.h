@@ -132,6 +132,8 @@ public:
                                 void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
     /* Addition (recomputeFirstLayer): the forward kernel once more, from this layer's srcData into the given block */
     int     forwardAgainInto(void* into, bool isDynamic);
+    void    biasGradientBeside(DATATYPE lr);
+    void    joinBiasGradient();
     int     convolutionBackwardOverSrc(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
                                        void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);
     // FC_GEMM layer
@@ -330,6 +332,7 @@ private:
     bool inPlaceOp, insideInceptionModule, headOfFork, tailOfFork;
     bool fuseRelu, elided, elidedBackward, gateGrad;
     bool gradOverSrc = false;
+    vdnn_event_t evBiasFork = nullptr, evBiasJoin = nullptr; // order the bias gradient's stream against the compute stream
     int  forkId, concatenateChannelOffset;
 
     vdnnConvHandle_t* convHandle;

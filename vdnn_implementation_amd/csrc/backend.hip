@@ -137,7 +137,9 @@ int vdnn_pool_init(vdnn_ctx* ctx, size_t bytes) {
     }
     uintptr_t s = ctx->pool.allocate(kReduceScratchBytes);
     ctx->reduce_scratch = (float*)s;
-    ctx->reduce_scratch_bytes = kReduceScratchBytes;
+    ctx->reduce_scratch_bytes = kReduceScratchBytes - kBiasScratchBytes;
+    ctx->bias_scratch = (float*)(s + ctx->reduce_scratch_bytes);
+    ctx->bias_scratch_bytes = kBiasScratchBytes;
     return VDNN_OK;
 }
 
@@ -151,6 +153,8 @@ int vdnn_pool_finalize(vdnn_ctx* ctx) {
     ctx->pool_base = nullptr;
     ctx->reduce_scratch = nullptr;
     ctx->reduce_scratch_bytes = 0;
+    ctx->bias_scratch = nullptr;
+    ctx->bias_scratch_bytes = 0;
     ctx->pool.clear();
     return VDNN_OK;
 }

@@ -19,6 +19,10 @@ struct vdnn_ctx {
     // Taken from the pool at vdnn_pool_init so the usage meter sees it; bounded, shape-independent.
     float* reduce_scratch = nullptr;
     size_t reduce_scratch_bytes = 0;
+    // The last megabyte of the staging area belongs to the convolution bias gradient alone, so that it can run
+    // on another stream beside the kernels that keep their partial sums in the rest.
+    float* bias_scratch = nullptr;
+    size_t bias_scratch_bytes = 0;
     int num_cu = 256;
     int act_dtype = VDNN_DTYPE_F32;   // element type of activation tensors handed to the kernels
     // per-kernel timing (vdnn_profile_*)
@@ -40,6 +44,7 @@ struct vdnn_ctx {
 namespace vdnn {
 
 static constexpr size_t kReduceScratchBytes = size_t(64) << 20;
+static constexpr size_t kBiasScratchBytes = size_t(1) << 20;     // its last part: the convolution bias gradient's partial sums
 
 void set_error(const char* fmt, ...);
 

@@ -866,10 +866,11 @@ static int conv_bwd_bias_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
     // split the batch so that K*splits workgroups fill the chip; geometry depends on the shape only
     int per = 0;
     const int splits = bias_grad_splits(N, K, ctx->num_cu, &per);
-    VDNN_REQUIRE((size_t)K * splits * sizeof(float) <= ctx->reduce_scratch_bytes, "staging area too small");
+    // (partial sums in a part of the staging area that no other kernel uses: the call may run on a stream of its own)
+    VDNN_REQUIRE(ctx->bias_scratch && (size_t)K * splits * sizeof(float) <= ctx->bias_scratch_bytes, "staging area too small");
     hipStream_t st = stream_of(ctx, stream);
     ProfScope prof(ctx, st, "conv_bwd_bias", 0.0, (double)sizeof(E) * (double)N * K * P * Q);
-    return bias_grad_launch<E>(st, (const E*)dy, bias, ctx->reduce_scratch, N, K, P * Q, splits, per, alpha, accumulate);
+    return bias_grad_launch<E>(st, (const E*)dy, bias, ctx->bias_scratch, N, K, P * Q, splits, per, alpha, accumulate);
 }
 
 // ---- the convolution bias gradient for callers that cannot allocate ---------------------------------------------

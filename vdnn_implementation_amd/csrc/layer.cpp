@@ -126,6 +126,8 @@ Layer::~Layer() {
     if (filterGrad) vdnn_pool_free(ctx, filterGrad);
     if (biasGrad) vdnn_pool_free(ctx, biasGrad);
     if (vdnnMode == BASELINE && dstData && !elided) vdnn_pool_free(ctx, dstData);
+    if (evBiasFork) vdnn_event_destroy(ctx, evBiasFork);
+    if (evBiasJoin) vdnn_event_destroy(ctx, evBiasJoin);
 }
 
 /* an elided ReLU has no output block of its own: under BASELINE the one taken at construction goes back */
@@ -260,6 +262,28 @@ int Layer::convolutionForward(bool* _offloaded, DATATYPE** _offloadedSrcData_h, 
     return 0;
 }
 
+/* The bias gradient (layer.cu:631-637) reads the output gradient once at memory speed and shares nothing with the two
+ * matrix-core kernels of the layer's backward but that input: it is enqueued on the context's fourth stream, behind
+ * whatever produced the output gradient, and runs beside them (its partial sums have a part of the staging area to
+ * themselves). joinBiasGradient makes the compute stream wait for it before the layer's backward returns: the caller
+ * may recycle the output gradient's block after that, and the next forward reads the bias. Same kernels, same bits. */
+void Layer::biasGradientBeside(DATATYPE lr) {
+    if (!evBiasFork) {
+        checkVDNN(vdnn_event_create(ctx, &evBiasFork, 0));
+        checkVDNN(vdnn_event_create(ctx, &evBiasJoin, 0));
+    }
+    vdnn_stream_t beside = vdnn_ctx_stream_pack(ctx);
+    checkVDNN(vdnn_event_record(ctx, evBiasFork, *stream_compute));
+    checkVDNN(vdnn_stream_wait_event(ctx, beside, evBiasFork));
+    if (filterGrad) checkVDNN(vdnn_conv_bwd_bias(ctx, beside, &shape, (const float*)diffData, (float*)biasGrad));
+    else checkVDNN(vdnn_conv_bwd_bias_sgd(ctx, beside, &shape, (const float*)diffData, (float*)biasData, lr));
+    checkVDNN(vdnn_event_record(ctx, evBiasJoin, beside));
+}
+
+void Layer::joinBiasGradient() {
+    checkVDNN(vdnn_stream_wait_event(ctx, *stream_compute, evBiasJoin));
+}
+
 /* Addition (recomputeFirstLayer): what convolutionForward computed, again, from the same input and filter into `into`
  * (the workspace of the pass comes from the pool as in the forward of the offloading policies). */
 int Layer::forwardAgainInto(void* into, bool isDynamic) {
@@ -294,8 +318,7 @@ int Layer::convolutionBackwardOverSrc(int _layer_id_to_prefetch, DATATYPE* _pref
     gradData = srcData;
     if (_layer_id_to_prefetch >= 0) prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);
 
-    if (filterGrad) checkVDNN(vdnn_conv_bwd_bias(ctx, *stream_compute, &shape, (const float*)diffData, (float*)biasGrad));
-    else checkVDNN(vdnn_conv_bwd_bias_sgd(ctx, *stream_compute, &shape, (const float*)diffData, (float*)biasData, lr));
+    biasGradientBeside(lr);
 
     void* dw = filterGrad;
     if (!dw && ASSERT_EQ(vdnn_pool_malloc(ctx, &dw, sizeof(DATATYPE) * (size_t)k * c_in * r * s), isDynamic) < 0) return -1;
@@ -319,6 +342,7 @@ int Layer::convolutionBackwardOverSrc(int _layer_id_to_prefetch, DATATYPE* _pref
         checkVDNN(vdnn_sgd_apply(ctx, *stream_compute, (size_t)k * c_in * r * s, lr, (const float*)dw, (float*)filterData));
         releaseDw();
     }
+    joinBiasGradient();
     return 0;
 }
 
@@ -349,8 +373,7 @@ int Layer::convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedS
     freeWorkSpace(workSpace, bwdDataWorkSpaceSize, curWorkSpace, isDynamic);
 
     /* Backward Bias Propagation: the learning rate is folded into the update */
-    if (filterGrad) checkVDNN(vdnn_conv_bwd_bias(ctx, *stream_compute, &shape, (const float*)diffData, (float*)biasGrad));
-    else checkVDNN(vdnn_conv_bwd_bias_sgd(ctx, *stream_compute, &shape, (const float*)diffData, (float*)biasData, lr));
+    biasGradientBeside(lr);
 
     if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) return -1;
     waitSrcFetched();
@@ -361,6 +384,7 @@ int Layer::convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedS
         checkVDNN(vdnn_conv_bwd_filter_sgd(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
                                            (float*)filterData, lr, curWorkSpace, bwdFilterWorkSpaceSize));
     freeWorkSpace(workSpace, bwdFilterWorkSpaceSize, curWorkSpace, isDynamic);
+    joinBiasGradient();
     return 0;
 }
 
