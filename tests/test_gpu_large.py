@@ -130,6 +130,37 @@ def test_dynamic_algo_ladder_on_the_device():
             assert abs(a - b) <= 1e-5 * abs(b)
 
 
+def test_dynamic_algo_with_the_lifetime_options():
+    """The ladder's trial steps fail in the middle of a forward or a backward; with gradients written over inputs and the
+    first layer computed again the blocks of a failed step still go back once each, and the step that follows the last
+    trial gives the bits of BASELINE."""
+    kw = dict(refined=True, fuse=True, in_place=True, recompute_first=True)
+    announce("VGG16_64 BASELINE + fused")
+    with Network(VGG16_64, BASELINE, VDNN_MEMORY_OPT_ALGO, 0, seed=5, fuse=True) as net:
+        want = train(net, 2)
+        want_digest = params_digest(net)
+    with Network(VGG16_64, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 0, plan_only=True, **kw) as replay:
+        assert replay.forwardPropagation() == 0 and replay.backwardPropagation() == 0
+        need_all = replay.stats()["peak_bytes_in_use"]
+    with Network(VGG16_64, VDNN_CONV, VDNN_PERF_OPT_ALGO, 0, plan_only=True, **kw) as replay:
+        assert replay.forwardPropagation() == 0 and replay.backwardPropagation() == 0
+        need_conv = replay.stats()["peak_bytes_in_use"]
+    assert need_all < need_conv
+    cap = (need_all + need_conv) // 2   # the VDNN_NONE and VDNN_CONV rungs fail, VDNN_ALL fits
+    announce("VDNN_DYNAMIC_ALGO VGG16_64 with gradients over inputs, cap", cap)
+    with Network(VGG16_64, BASELINE, VDNN_DYNAMIC_ALGO, 0, seed=5, cap_bytes=cap, **kw) as net:
+        assert net.policy == VDNN_ALL and net.recomputed_layer() == 2 and any(net.grad_over_src(l) for l in range(net.num_layers))
+        got = train(net, 2, dynamic=True)
+        assert net.stats()["peak_bytes_in_use"] <= cap
+        # (the last rung chooses the convolution variant layer by layer: a wider split of a filter gradient differs in the last places)
+        assert got[0] == want[0]
+        a, b = np.frombuffer(got[1], np.float32)[0], np.frombuffer(want[1], np.float32)[0]
+        assert abs(a - b) <= 1e-5 * abs(b)
+    announce("the same options built directly")
+    with Network(VGG16_64, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 0, seed=5, **kw) as net:
+        assert train(net, 2) == want and params_digest(net) == want_digest
+
+
 def test_vgg16_batch_256_vdnn_all_against_baseline():
     announce("VGG16_256 BASELINE")
     with Network(VGG16_256, BASELINE, VDNN_MEMORY_OPT_ALGO, 0, seed=11) as net:
