@@ -424,29 +424,28 @@ struct StoreDense {
     __device__ __forceinline__ void store_tail(const floatx16 (&)[2][2], int, int, int, long, int, int) const {}
     __device__ __forceinline__ void store(const floatx16 (&acc)[2][2], int m0, int j0, int lane, int ks, const GemmDims& d, bool to_partial) const {
         const int l32 = lane & 31, lk = lane >> 5;
-        // What the result is combined with is read for a whole column block before anything is stored: a load
-        // issued after a store through the same pointer would have to wait for it (the compiler cannot know that
-        // the rows differ), and sixty-four round trips to memory in a row are the kernel's whole time when the
-        // output is large (the filter of a fully connected layer, updated in place).
+        // What the result is combined with is read sixteen elements ahead of the stores: a load issued after a store
+        // through the same pointer would have to wait for it (the compiler cannot know that the rows differ), and
+        // sixty-four round trips to memory in a row are the kernel's whole time when the output is large (the filter of
+        // a fully connected layer, updated in place). Sixteen, not more: the registers they wait in count against the
+        // workgroups a compute unit holds.
         const bool combine = !to_partial && (accumulate || gate != nullptr);
 #pragma unroll
         for (int jt = 0; jt < 2; jt++) {
             const int j = j0 + jt * 32 + l32;
             if (j >= d.N) continue;
-            float old[2][16], gt[2][16];
-            if (combine) {
+            const float bj = (!to_partial && bias_j) ? bias_j[j] : 0.0f;
 #pragma unroll
-                for (int it = 0; it < 2; it++)
+            for (int it = 0; it < 2; it++) {
+                float aux[16]; // the old value (accumulate) or the gate: a call asks for one of the two at most
+                if (combine) {
 #pragma unroll
                     for (int v = 0; v < 16; v++) {
                         const int m = m0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
                         const long idx = (long)m * ld_m + j;
-                        old[it][v] = accumulate && m < d.M ? load_elem(out + idx) : 0.0f;
-                        gt[it][v] = gate && m < d.M ? load_elem(gate + idx) : 1.0f;
+                        aux[v] = m < d.M ? (accumulate ? load_elem(out + idx) : load_elem(gate + idx)) : 0.0f;
                     }
-            }
-#pragma unroll
-            for (int it = 0; it < 2; it++)
+                }
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
                     const int m = m0 + it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
@@ -457,13 +456,14 @@ struct StoreDense {
                         partial[(long)ks * partial_stride + idx] = a;
                     } else {
                         // one fused multiply-add: every route to "out += alpha * sum" rounds the same way
-                        float r = accumulate ? __fmaf_rn(alpha, a, old[it][v]) : alpha * a;
-                        if (bias_j) r += bias_j[j];
+                        float r = accumulate ? __fmaf_rn(alpha, a, aux[v]) : alpha * a;
+                        if (bias_j) r += bj;
                         if (relu) r = relu_value(r);
-                        if (gate) r = gt[it][v] > 0.0f ? r : 0.0f;
+                        if (gate) r = (accumulate ? load_elem(gate + idx) : aux[v]) > 0.0f ? r : 0.0f;
                         store_elem(out + idx, r);
                     }
                 }
+            }
         }
     }
 };
