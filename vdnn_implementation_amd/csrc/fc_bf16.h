@@ -110,4 +110,7 @@ struct LoadRowAsH {
     }
 };
 
+// the transposing loader holds sixteen loads' worth of registers per operand: two workgroups per compute unit
+template <class A, class SRC> struct MinResident<A, LoadRowAsH<SRC>> { static constexpr int V = 2; };
+
 } // namespace vdnn

@@ -110,8 +110,12 @@ template <class EP> struct TileOrder { static constexpr bool COLUMNS_FASTEST = f
 
 // Out tile = A tile x B tile over this workgroup's share of the reduction; tile decoding and epilogues are
 // those of the float engine (igemm_kernel), slices are KH deep.
+// How many workgroups a compute unit is to hold at least (the register budget follows): three with the
+// convolution operands, which the compiler meets without spills; an operand type that needs more registers says so.
+template <class AL, class BL> struct MinResident { static constexpr int V = 3; };
+
 template <int TM, int TN, class AL, class BL, class EP>
-__global__ void __launch_bounds__(NT) igemm_bf16_kernel(const AL al, const BL bl, const EP ep, const GemmDims d) {
+__global__ void __launch_bounds__(NT, (MinResident<AL, BL>::V)) igemm_bf16_kernel(const AL al, const BL bl, const EP ep, const GemmDims d) {
     static_assert(TM % 64 == 0 && TN % 64 == 0 && (TM / 64) * (TN / 64) == 4, "four 64x64 wave tiles");
     __shared__ __attribute__((aligned(16))) unsigned short As[2][TM * HSTRIDE];
     __shared__ __attribute__((aligned(16))) unsigned short Bs[2][TN * HSTRIDE];
