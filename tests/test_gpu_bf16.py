@@ -81,6 +81,34 @@ def ws(d, g, algo, which):
     return (d.raw(n).ptr, n) if n else (None, 0)
 
 
+def test_rounding_on_the_device_is_the_checkers(ctx):
+    """Every store of a bfloat16 activation rounds a float on the device with the hardware's conversion; the checker
+    rounds in integer arithmetic (nearest, ties to even, NaN stays NaN). bias_add on a tensor of zeros stores
+    round(0 + b): ties, neighbours of ties, denormals, the largest finite value, infinities and random bit patterns
+    must come back with the checker's bits."""
+    rng = np.random.default_rng(5)
+    edge = np.array([0x3F808000, 0x3F818000, 0x3F807FFF, 0x3F808001, 0x3F817FFF, 0x3F818001, 0x7F7FFFFF, 0x7F7F8000, 0x7F7F7FFF,
+                     0x00000001, 0x00008000, 0x00008001, 0x00018000, 0x00017FFF, 0x007FFFFF, 0x00800000, 0x7F800000, 0x00000000,
+                     0x7FC00000, 0x7FC12345, 0x7FFFFFFF], np.uint32)
+    bits = np.concatenate([edge, edge | np.uint32(0x80000000), rng.integers(0, 2 ** 32, 60000, dtype=np.uint64).astype(np.uint32)])
+    b = bits.view(np.float32)
+    c = b.size
+    announce("rounding to bf16 on the device, %d values" % c)
+    with Dev(ctx) as d:
+        y = d.act(np.zeros((1, c, 1, 1), np.float32))
+        db = d.f32(b)
+        check(lib.vdnn_bias_add(ctx.handle, None, 1, c, 1, db.ptr, y.ptr))
+        got = y.download((c,), np.uint16)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = (oracle.round_bf16(np.float32(0) + b).view(np.uint32) >> 16).astype(np.uint16)
+    nan = np.isnan(b)
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.all(np.isnan(from_bf16_bits(got[nan])))
+    # quiet NaNs keep their sign and the upper bits of their payload
+    quiet = nan & ((bits & 0x00400000) != 0)
+    assert np.array_equal(got[quiet], (bits[quiet] >> 16).astype(np.uint16))
+
+
 CONV = [
     (3, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1),     # blocked tap-major loaders, 64-row tile
     (2, 128, 14, 14, 256, 3, 3, 1, 1, 1, 1),   # two row tiles
@@ -111,6 +139,8 @@ CONV = [
     (3, 64, 6, 28, 96, 3, 3, 1, 1, 1, 1),      # 28-pixel rows, plane not a multiple of the slice: slices straddle samples
     (2, 96, 12, 20, 128, 3, 3, 1, 1, 1, 1),    # 96 channels: backward filter on the tile engine, four taps per tile, four pixels per load
     (2, 3, 11, 140, 32, 3, 3, 1, 1, 1, 1),     # three input channels: the streaming first-layer kernels, two backward-data column blocks
+    (7, 3, 40, 36, 16, 3, 3, 1, 1, 1, 1),      # first layer: pixels that do not fill the last unit of 64, half a block of output channels
+    (5, 2, 7, 9, 40, 3, 3, 1, 1, 1, 1),        # two input channels, rows shorter than a block of pixels, a ragged second block of output channels
 ]
 
 

@@ -431,14 +431,21 @@ static bool fwd_smallc3x3_ok(const ConvGeo& g, size_t elem_bytes) {
 }
 template <class E>
 static int launch_fwd_smallc3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const E* x, const float* w, const float* bias, E* y, int relu) {
-    const long units = ((long)g.N * g.H * g.W + 31) / 32;
+    // two blocks of 32 pixels per unit where that makes a store a whole 128-byte line (two-byte elements: 0.47 -> 0.38 ms
+    // for VGG16's first layer at batch 128); with floats a block's 32 pixels are a line already and two measured the same
+    const int up = sizeof(E) == 2 ? 2 : 1;
+    const long units = ((long)g.N * g.H * g.W + 32 * up - 1) / (32 * up);
     long blocks = (units + 3) / 4;
-    if (blocks > 3l * ctx->num_cu) blocks = 3l * ctx->num_cu; // bound by its stores from two workgroups per unit on (four measured 20 % slower)
+    // bound by its stores from two workgroups per unit on (four measured 20 % slower); with two blocks per unit the
+    // registers allow two
+    const long resident = (up == 2 ? 2l : 3l) * ctx->num_cu;
+    if (blocks > resident) blocks = resident;
     ProfScope prof(ctx, st, "conv_fwd_smallc", 2.0 * g.K * 9.0 * g.C * (double)g.N * g.H * g.W, 0.0);
-#define VDNN_FWD_SMALLC(CC)                                                                                                              \
-    do {                                                                                                                                 \
-        if (g.K <= 32) hipLaunchKernelGGL((conv_fwd_smallc3x3_kernel<CC, 1, E>), dim3((unsigned)blocks), dim3(256), 0, st, x, w, bias, y, g.N, g.K, g.H, g.W, relu); \
-        else hipLaunchKernelGGL((conv_fwd_smallc3x3_kernel<CC, 2, E>), dim3((unsigned)blocks), dim3(256), 0, st, x, w, bias, y, g.N, g.K, g.H, g.W, relu);          \
+#define VDNN_FWD_SMALLC_UP(CC, RB, UP) hipLaunchKernelGGL((conv_fwd_smallc3x3_kernel<CC, RB, UP, E>), dim3((unsigned)blocks), dim3(256), 0, st, x, w, bias, y, g.N, g.K, g.H, g.W, relu)
+#define VDNN_FWD_SMALLC(CC)                                                                         \
+    do {                                                                                            \
+        if (g.K <= 32) { if (up == 2) VDNN_FWD_SMALLC_UP(CC, 1, 2); else VDNN_FWD_SMALLC_UP(CC, 1, 1); } \
+        else { if (up == 2) VDNN_FWD_SMALLC_UP(CC, 2, 2); else VDNN_FWD_SMALLC_UP(CC, 2, 1); }           \
     } while (0)
     switch (g.C) {
     case 1: VDNN_FWD_SMALLC(1); break;
@@ -446,6 +453,7 @@ static int launch_fwd_smallc3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g,
     case 3: VDNN_FWD_SMALLC(3); break;
     default: VDNN_FWD_SMALLC(4); break;
     }
+#undef VDNN_FWD_SMALLC_UP
 #undef VDNN_FWD_SMALLC
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;

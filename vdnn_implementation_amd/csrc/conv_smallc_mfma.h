@@ -22,10 +22,14 @@ template <> __device__ __forceinline__ void buf_store_e<bf16_t>(__amdgpu_buffer_
     __builtin_amdgcn_raw_buffer_store_b16((unsigned short)float_to_bf16_bits(v), r, voff, soff, 0);
 }
 
-// x and y below 2 GiB each (offsets are 32-bit), N*H*W below 2^31.
-template <int CC, int RBLK, class E>
+// x and y below 2 GiB each (offsets are 32-bit), N*H*W below 2^31. UP = blocks of 32 pixels per unit: with two, the
+// halves of the wavefront exchange what they hold of the two blocks (v_permlane32_swap), so that one store covers 64
+// consecutive pixels of one output row instead of 32 pixels of two rows - whole 128-byte lines also with two-byte
+// elements.
+template <int CC, int RBLK, int UP, class E>
 __global__ void __launch_bounds__(256) conv_fwd_smallc3x3_kernel(const E* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias,
                                                                   E* __restrict__ y, int N, int K, int H, int W, int relu) {
+    static_assert(UP == 1 || UP == 2, "one block of 32 pixels per unit, or two");
     constexpr int KRED = 9 * CC, ES = ElemBytes<E>::V;
     // with an odd reduction length the bias rides in the unused last index (input value 1); otherwise it is added afterwards
     constexpr bool BIAS_SLOT = KRED % 2 == 1;
@@ -33,7 +37,7 @@ __global__ void __launch_bounds__(256) conv_fwd_smallc3x3_kernel(const E* __rest
     const int lane = threadIdx.x & 63, l32 = lane & 31, lk = lane >> 5;
     const int PQ = H * W;
     const int total = N * PQ;
-    const int nunits = (total + 31) / 32;
+    const int nunits = (total + 32 * UP - 1) / (32 * UP);
     const int nwaves = (int)gridDim.x * 4;
     const int wave0 = (int)blockIdx.x * 4 + (int)(threadIdx.x >> 6);
     const __amdgpu_buffer_rsrc_t rs = make_rsrc(x, clamp_range((long)N * CC * PQ * ES));
@@ -74,26 +78,27 @@ __global__ void __launch_bounds__(256) conv_fwd_smallc3x3_kernel(const E* __rest
     }
 
     // a wavefront walks a run of consecutive units (its 64 output rows are 64 sequential streams); the lane's pixel
-    // (sample, row, column) is carried from unit to unit
+    // of each block (sample, row, column) is carried from unit to unit
     const int per = (nunits + nwaves - 1) / nwaves;
     const int first = wave0 * per, last = first + per < nunits ? first + per : nunits;
-    int px = first * 32 + l32;
-    int n, p, q;
-    {
-        const int pc = px < total ? px : 0;
-        n = pc / PQ;
-        const int pq = pc - n * PQ;
-        p = pq / W; q = pq - p * W;
+    struct Pix { int px, n, p, q; };
+    Pix pix[UP];
+#pragma unroll
+    for (int u = 0; u < UP; u++) {
+        pix[u].px = (first * UP + u) * 32 + l32;
+        const int pc = pix[u].px < total ? pix[u].px : 0;
+        pix[u].n = pc / PQ;
+        const int pq = pc - pix[u].n * PQ;
+        pix[u].p = pq / W; pix[u].q = pq - pix[u].p * W;
     }
-    float b[KS];
-    int obase = OOB; // byte offset of (n, output channel 4*lk, p, q) in y, or out of range
-    auto fetch = [&](bool in_run, float (&dst)[KS], int& out_base) {
-        const bool inside = in_run && px < total;
-        const int pq = p * W + q;
-        const int base = (n * CC * PQ + pq) * ES;
+    // byte offset in y of the pixel's value in output channel 0 (UP == 2) or 4*lk (UP == 1), or out of range
+    auto fetch = [&](bool in_run, Pix& px, float (&dst)[KS], int& out_base) {
+        const bool inside = in_run && px.px < total;
+        const int pq = px.p * W + px.q;
+        const int base = (px.n * CC * PQ + pq) * ES;
         // the nine places of the window that lie inside the image, as bits r*3 + s
-        const unsigned colok = (q > 0 ? 1u : 0u) | 2u | (q < W - 1 ? 4u : 0u);
-        const unsigned win = inside ? ((p > 0 ? colok : 0u) | (colok << 3) | (p < H - 1 ? colok << 6 : 0u)) : 0u;
+        const unsigned colok = (px.q > 0 ? 1u : 0u) | 2u | (px.q < W - 1 ? 4u : 0u);
+        const unsigned win = inside ? ((px.p > 0 ? colok : 0u) | (colok << 3) | (px.p < H - 1 ? colok << 6 : 0u)) : 0u;
 #pragma unroll
         for (int t = 0; t < KS; t++) {
             const unsigned tap = (unsigned)(ktap[t / 16] >> (4 * (t % 16))) & 15u;
@@ -101,42 +106,71 @@ __global__ void __launch_bounds__(256) conv_fwd_smallc3x3_kernel(const E* __rest
             if (BIAS_SLOT && t == KS - 1) v = lk ? 1.0f : v; // reduction index KRED: the bias' factor
             dst[t] = v;
         }
-        out_base = inside ? ((n * K + 4 * lk) * PQ + pq) * ES : OOB;
-        // one unit further: 32 pixels
-        px += 32; q += 32;
-        while (q >= W) { q -= W; p += 1; }
-        while (p >= H) { p -= H; n += 1; }
+        out_base = inside ? ((px.n * K + (UP == 1 ? 4 * lk : 0)) * PQ + pq) * ES : OOB;
+        // one unit further
+        px.px += 32 * UP; px.q += 32 * UP;
+        while (px.q >= W) { px.q -= W; px.p += 1; }
+        while (px.p >= H) { px.p -= H; px.n += 1; }
     };
 
-    fetch(first < last, b, obase);
+    float b[UP][KS];
+    int obase[UP];
+#pragma unroll
+    for (int u = 0; u < UP; u++) fetch(first < last, pix[u], b[u], obase[u]);
     for (int unit = first; unit < last; unit++) {
-        float bn[KS];
-        int obase_next;
-        fetch(unit + 1 < last, bn, obase_next);
-        floatx16 acc[RBLK];
+        float bn[UP][KS];
+        int obase_next[UP];
 #pragma unroll
-        for (int i = 0; i < RBLK; i++)
+        for (int u = 0; u < UP; u++) fetch(unit + 1 < last, pix[u], bn[u], obase_next[u]);
+        floatx16 acc[UP][RBLK];
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][v] = 0.0f;
+        for (int u = 0; u < UP; u++)
+#pragma unroll
+            for (int i = 0; i < RBLK; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[u][i][v] = 0.0f;
 #pragma unroll
         for (int t = 0; t < KS; t++)
 #pragma unroll
-            for (int i = 0; i < RBLK; i++) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][t], b[t], acc[i], 0, 0, 0);
+            for (int u = 0; u < UP; u++)
+#pragma unroll
+                for (int i = 0; i < RBLK; i++) acc[u][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][t], b[u][t], acc[u][i], 0, 0, 0);
+        // the lane's store address with two blocks: lanes 0-31 write the first block's pixels, lanes 32-63 the second's
+        const int obase2 = UP == 2 ? (lk ? obase[UP - 1] : obase[0]) : 0;
 #pragma unroll
         for (int i = 0; i < RBLK; i++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int mrow = 32 * i + 8 * (v / 4) + (v % 4); // + 4*lk, which the lane's offset carries
-                float r = acc[i][v];
-                if (!BIAS_SLOT && bias) r += bv[i][v];
-                if (relu) r = relu_value(r);
+                const int mrow = 32 * i + 8 * (v / 4) + (v % 4); // the lane holds row mrow + 4*lk
+                float r[UP];
+#pragma unroll
+                for (int u = 0; u < UP; u++) {
+                    r[u] = acc[u][i][v];
+                    if (!BIAS_SLOT && bias) r[u] += bv[i][v];
+                    if (relu) r[u] = relu_value(r[u]);
+                }
                 // rows past K (the last block of a layer with fewer channels) are sent out of range
-                const int soff = __builtin_amdgcn_readfirstlane(mrow * PQ * ES);
-                buf_store_e<E>(ro, r, (mrow + 4 * lk < K) ? obase : OOB, soff);
+                if constexpr (UP == 1) {
+                    // the lane's offset carries the 4*lk rows
+                    const int soff = __builtin_amdgcn_readfirstlane(mrow * PQ * ES);
+                    buf_store_e<E>(ro, r[0], (mrow + 4 * lk < K) ? obase[0] : OOB, soff);
+                } else {
+                    // [first block: rows mrow | mrow + 4] x [second block: rows mrow | mrow + 4]  ->
+                    // row mrow of both blocks, row mrow + 4 of both blocks (the builtin's result is read through a
+                    // 64-bit integer: subscripts of the two-element vector both gave its first element)
+                    const unsigned long long sw = __builtin_bit_cast(unsigned long long,
+                        __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, r[0]), __builtin_bit_cast(unsigned, r[UP - 1]), false, false));
+                    const int soff0 = __builtin_amdgcn_readfirstlane(mrow * PQ * ES), soff1 = __builtin_amdgcn_readfirstlane((mrow + 4) * PQ * ES);
+                    buf_store_e<E>(ro, __builtin_bit_cast(float, (unsigned)sw), (mrow < K) ? obase2 : OOB, soff0);
+                    buf_store_e<E>(ro, __builtin_bit_cast(float, (unsigned)(sw >> 32)), (mrow + 4 < K) ? obase2 : OOB, soff1);
+                }
             }
 #pragma unroll
-        for (int t = 0; t < KS; t++) b[t] = bn[t];
-        obase = obase_next;
+        for (int u = 0; u < UP; u++) {
+#pragma unroll
+            for (int t = 0; t < KS; t++) b[u][t] = bn[u][t];
+            obase[u] = obase_next[u];
+        }
     }
 }
 

@@ -58,8 +58,8 @@ __device__ __forceinline__ float4 ld4(const bf16_t* p) {
 __device__ __forceinline__ void st4(float* p, float4 v) { *(float4*)p = v; }
 __device__ __forceinline__ void st4(bf16_t* p, float4 v) {
     uint2 w;
-    w.x = (unsigned)float_to_bf16_bits(v.x) | ((unsigned)float_to_bf16_bits(v.y) << 16);
-    w.y = (unsigned)float_to_bf16_bits(v.z) | ((unsigned)float_to_bf16_bits(v.w) << 16);
+    w.x = pack2_bf16(v.x, v.y);
+    w.y = pack2_bf16(v.z, v.w);
     *(uint2*)p = w;
 }
 __device__ __forceinline__ float2 ld2(const float* p) { return *(const float2*)p; }
@@ -69,7 +69,7 @@ __device__ __forceinline__ float2 ld2(const bf16_t* p) {
 }
 __device__ __forceinline__ void st2(float* p, float2 v) { *(float2*)p = v; }
 __device__ __forceinline__ void st2(bf16_t* p, float2 v) {
-    *(unsigned*)p = (unsigned)float_to_bf16_bits(v.x) | ((unsigned)float_to_bf16_bits(v.y) << 16);
+    *(unsigned*)p = pack2_bf16(v.x, v.y);
 }
 
 // ---- ReLU ---------------------------------------------------------------------------------------

@@ -15,10 +15,10 @@ namespace vdnn {
 
 __device__ __forceinline__ uintx4 pack8_bf16(const float (&f)[8]) {
     uintx4 q;
-    q.x = float_to_bf16_bits(f[0]) | ((unsigned)float_to_bf16_bits(f[1]) << 16);
-    q.y = float_to_bf16_bits(f[2]) | ((unsigned)float_to_bf16_bits(f[3]) << 16);
-    q.z = float_to_bf16_bits(f[4]) | ((unsigned)float_to_bf16_bits(f[5]) << 16);
-    q.w = float_to_bf16_bits(f[6]) | ((unsigned)float_to_bf16_bits(f[7]) << 16);
+    q.x = pack2_bf16(f[0], f[1]);
+    q.y = pack2_bf16(f[2], f[3]);
+    q.z = pack2_bf16(f[4], f[5]);
+    q.w = pack2_bf16(f[6], f[7]);
     return q;
 }
 

@@ -321,15 +321,17 @@ int Layer::convolutionBackwardOverSrc(int _layer_id_to_prefetch, DATATYPE* _pref
     biasGradientBeside(lr);
 
     void* dw = filterGrad;
-    if (!dw && ASSERT_EQ(vdnn_pool_malloc(ctx, &dw, sizeof(DATATYPE) * (size_t)k * c_in * r * s), isDynamic) < 0) return -1;
+    if (!dw && ASSERT_EQ(vdnn_pool_malloc(ctx, &dw, sizeof(DATATYPE) * (size_t)k * c_in * r * s), isDynamic) < 0) { joinBiasGradient(); return -1; }
+    /* a trial of the dynamic mode that runs out of memory gives up here: the caller recycles the output gradient's
+     * block next, so the bias gradient's stream is joined on these paths too */
     auto releaseDw = [&]() { if (!filterGrad) ASSERT_EQ(vdnn_pool_free(ctx, dw), isDynamic); };
-    if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { releaseDw(); return -1; }
+    if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { releaseDw(); joinBiasGradient(); return -1; }
     waitSrcFetched();
     checkVDNN(vdnn_conv_bwd_filter(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
                                    (float*)dw, curWorkSpace, bwdFilterWorkSpaceSize));
     freeWorkSpace(workSpace, bwdFilterWorkSpaceSize, curWorkSpace, isDynamic);
 
-    if (mallocWorkSpace(workSpace, bwdDataWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { releaseDw(); return -1; }
+    if (mallocWorkSpace(workSpace, bwdDataWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { releaseDw(); joinBiasGradient(); return -1; }
     if (gateGrad)
         checkVDNN(vdnn_conv_bwd_data_relu(ctx, *stream_compute, &shape, vdnnAlgoMode, diffData, (const float*)filterData,
                                           srcData, gradData, curWorkSpace, bwdDataWorkSpaceSize));
@@ -375,7 +377,9 @@ int Layer::convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedS
     /* Backward Bias Propagation: the learning rate is folded into the update */
     biasGradientBeside(lr);
 
-    if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) return -1;
+    /* a trial of the dynamic mode that runs out of memory gives up here: the caller recycles the output gradient's
+     * block next, so the bias gradient's stream is joined first */
+    if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { joinBiasGradient(); return -1; }
     waitSrcFetched();
     if (filterGrad)
         checkVDNN(vdnn_conv_bwd_filter(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,

@@ -90,11 +90,24 @@ template <class E> struct ElemBytes { static constexpr int V = (int)sizeof(E); }
 __host__ __device__ __forceinline__ float bf16_bits_to_float(unsigned bits) {
     return __builtin_bit_cast(float, bits << 16);
 }
+// On the device the conversion is one instruction (v_cvt_pk_bf16_f32, two values at a time); it gives the bits of
+// the arithmetic below for every one of the 2^32 inputs, NaN payloads and denormals included.
 __host__ __device__ __forceinline__ unsigned short float_to_bf16_bits(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_bit_cast(unsigned short, (__bf16)f);
+#else
     unsigned u = __builtin_bit_cast(unsigned, f);
     if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (unsigned short)((u >> 16) | 0x40u);
     u += 0x7FFFu + ((u >> 16) & 1u);
     return (unsigned short)(u >> 16);
+#endif
+}
+// two values in one word, the first in the lower half
+__device__ __forceinline__ unsigned pack2_bf16(float lo, float hi) {
+    typedef float float_x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16_x2 __attribute__((ext_vector_type(2)));
+    float_x2 f; f.x = lo; f.y = hi;
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16_x2));
 }
 __device__ __forceinline__ float load_elem(const float* p) { return *p; }
 __device__ __forceinline__ float load_elem(const bf16_t* p) { return bf16_bits_to_float(p->bits); }
