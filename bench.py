@@ -162,6 +162,51 @@ def smallest_within(results, base, speed_floor):
             "peak_hbm_gb": ok[k]["peak_hbm_gb"], "link_gb_each_way_per_step": ok[k]["link_gb_each_way_per_step"]}
 
 
+def zvc_standalone(be):
+    """The kernels of the compressed offload alone on the device: a rectified tensor of 411 MB (VGG16 conv2_1's input at
+    batch 128 in float; twice the elements in bfloat16), half of its elements zero, five times: packed into a staging
+    block, moved to pinned host memory by the copy engine, expanded from there. Rates in bytes of the tensor per second;
+    the packing kernel reads the tensor and writes the stream (about 0.53 of it)."""
+    import ctypes as C
+    import numpy as np
+    lib, check = be.lib, be.check
+    ctx = be.Context(pool_bytes=6 << 30)
+    out = {}
+    try:
+        for es, dtype in ((4, np.uint32), (2, np.uint16)):
+            count = 128 * 64 * 112 * 112 * (4 // es)
+            rng = np.random.default_rng(1)
+            t = rng.integers(1, 60000, size=count, dtype=np.uint32).astype(dtype)
+            t[rng.random(count) < 0.5] = 0
+            src, dst = ctx.to_device(t, dtype), ctx.alloc(count * es)
+            need = lib.vdnn_zvc_buffer_bytes(count, es)
+            stage = ctx.alloc(need)
+            host = C.c_void_p()
+            check(lib.vdnn_host_alloc_pinned(ctx.handle, C.byref(host), need))
+            be.profile_enable(ctx.handle, True)
+            for _ in range(5):
+                check(lib.vdnn_zvc_offload_staged_async(ctx.handle, host, stage.ptr, need // 2 // 16 * 16 + 65536, src.ptr, count, es,
+                                                        None, None, None, None, 0))
+                ctx.synchronize()
+                check(lib.vdnn_zvc_prefetch_async(ctx.handle, dst.ptr, host, count, es, None))
+                ctx.synchronize()
+            prof = be.profile_collect(ctx.handle)
+            be.profile_enable(ctx.handle, False)
+            assert np.array_equal(dst.download((count,), dtype), t)
+            out["f32" if es == 4 else "bf16"] = {
+                "tensor_mb": count * es / 1e6,
+                "pack_ms": prof["offload_zvc_pack"]["ms"] / prof["offload_zvc_pack"]["launches"],
+                "pack_gbs": prof["offload_zvc_pack"]["bytes"] / prof["offload_zvc_pack"]["ms"] / 1e6,
+                "copy_gbs": prof["offload_zvc_copy"]["bytes"] / prof["offload_zvc_copy"]["ms"] / 1e6,
+                "expand_gbs": prof["prefetch_zvc"]["bytes"] / prof["prefetch_zvc"]["ms"] / 1e6}
+            check(lib.vdnn_host_free_pinned(ctx.handle, host))
+            for b in (src, dst, stage):
+                b.free()
+    finally:
+        ctx.close()
+    return out
+
+
 def cpu_baseline(batch, threads):
     """The checker's training step (forward, backward, SGD) on the host cores: VGG16, float."""
     import oracle
@@ -196,6 +241,7 @@ def main():
     ap.add_argument("--cpu-batch", type=int, default=0, help="batch of the CPU baseline's step (0: 128, the headline's batch; about 15-30 s on 16 threads)")
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (0: the box's CPU share, at most 16)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--zvc-standalone", action="store_true", help="also time the kernels of the compressed offload alone on the device")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
@@ -305,6 +351,10 @@ def main():
         "kernels": kernels,
         "step_mfma_frac": args.batch * FLOP_PER_IMAGE / (results[head]["ms_per_step"] * 1e-3) / 1e12 / peak,
     }
+    if args.zvc_standalone:
+        log("[bench] compressed offload alone on the device")
+        out["zvc_standalone"] = zvc_standalone(be)
+        log("[bench]   %s" % json.dumps(out["zvc_standalone"]))
     if not args.no_cpu_baseline:
         threads = args.cpu_threads or min(16, os.cpu_count() or 1)
         cpu_batch = args.cpu_batch or 128

@@ -207,3 +207,43 @@ def net_peak(net):
         assert net.forwardPropagation() == 0 and net.backwardPropagation() == 0
     net.synchronize()
     return net.stats()["peak_bytes_in_use"]
+
+
+@pytest.mark.parametrize("cnn,batch,algo,bf16", [(VGG16_128, 2, VDNN_MEMORY_OPT_ALGO, False), (VGG16_128, 2, VDNN_MEMORY_OPT_ALGO, True),
+                                                 (ALEXNET_LRN, 4, VDNN_PERF_OPT_ALGO, False), (OVERFEAT, 3, VDNN_MEMORY_OPT_ALGO, True)])
+def test_schedule_options_drawn_at_random_keep_every_bit(cnn, batch, algo, bf16):
+    """The options that change when and where a tensor lives (policy, lifetimes, lag, depth of prefetch, packing, keeping
+    packed blocks, placement by a budget between the plan's floor and what fits unplaced, gradients over inputs, the
+    first layer computed again, the update apart, host synchronisation) combined at random from a fixed seed: every
+    combination must leave the losses, outputs and gradients of two steps as BASELINE leaves them."""
+    import random
+    rnd = random.Random(hash((cnn, batch, bf16)) & 0xFFFF)
+
+    def make(policy, **kw):
+        return Network(cnn, policy, algo, batch, capture=True, seed=3, bf16=bf16, **kw)
+
+    announce("random schedules", cnn, batch, "bf16" if bf16 else "f32", "BASELINE")
+    with make(BASELINE) as net:
+        plain = run_steps(net, 2)
+        specs = list(net.specs)
+    for _ in range(10):
+        policy = rnd.choice([VDNN_NONE, VDNN_CONV, VDNN_ALL])
+        kw = dict(refined=True, fuse=True, in_place=rnd.random() < 0.6, recompute_first=rnd.random() < 0.5, host_sync=rnd.random() < 0.15,
+                  offload_lag=rnd.choice([0, 0, 2, 6, 14, -1]), prefetch_depth=rnd.choice([1, 1, 2, 3]),
+                  prefetch_within_peak=rnd.random() < 0.3, unfused_optimizer=rnd.random() < 0.2, compress=rnd.random() < 0.6)
+        if kw["compress"]:
+            kw["keep_packed"] = rnd.random() < 0.5
+            if rnd.random() < 0.5:
+                kw["plan_packed_fraction"] = 0.7
+                with make(policy, plan_only=True, hbm_budget_bytes=1, **kw) as probe:
+                    floor = probe.plan_peak_bytes()
+                with make(policy, plan_only=True, hbm_budget_bytes=1 << 50, **kw) as probe:
+                    ceiling = probe.plan_peak_bytes()
+                kw["hbm_budget_bytes"] = int(floor + (ceiling - floor) * rnd.choice([0.0, 0.3, 0.6, 1.0]))
+        announce("random schedules", cnn, batch, "bf16" if bf16 else "f32", "policy", policy, kw)
+        with make(policy, **kw) as net:
+            got = run_steps(net, 2)
+            offloaded = {l for l in range(net.num_layers) if net.is_offloaded(l)}
+        if kw["compress"]:
+            offloaded = {l for l in offloaded if not rectified(specs, l)}
+        assert_fused_matches(got, plain, specs, "policy %d %s" % (policy, kw), offloaded)
