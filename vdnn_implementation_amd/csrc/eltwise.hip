@@ -351,6 +351,41 @@ __global__ void __launch_bounds__(EB) sgd_apply_kernel(const float* __restrict__
 }
 
 // ---- bias gradient of a convolution: bias[k] += alpha * sum_{n,pq} dy[n,k,pq] -------------------
+// Sum of V consecutive elements (one access), in a fixed order.
+template <int V, class E> __device__ __forceinline__ float sum_of_run(const E* p);
+template <> __device__ __forceinline__ float sum_of_run<1, float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float sum_of_run<1, bf16_t>(const bf16_t* p) { return load_elem(p); }
+template <> __device__ __forceinline__ float sum_of_run<4, float>(const float* p) { const float4 v = ld4(p); return (v.x + v.y) + (v.z + v.w); }
+template <> __device__ __forceinline__ float sum_of_run<4, bf16_t>(const bf16_t* p) { const float4 v = ld4(p); return (v.x + v.y) + (v.z + v.w); }
+template <> __device__ __forceinline__ float sum_of_run<8, bf16_t>(const bf16_t* p) {
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4 v = *(const u32x4*)p;
+    return ((__builtin_bit_cast(float, v.x << 16) + __builtin_bit_cast(float, v.x & 0xFFFF0000u)) +
+            (__builtin_bit_cast(float, v.y << 16) + __builtin_bit_cast(float, v.y & 0xFFFF0000u))) +
+           ((__builtin_bit_cast(float, v.z << 16) + __builtin_bit_cast(float, v.z & 0xFFFF0000u)) +
+            (__builtin_bit_cast(float, v.w << 16) + __builtin_bit_cast(float, v.w & 0xFFFF0000u)));
+}
+// Planes with fewer accesses than the workgroup has threads (13 x 13, 14 x 14 ...): walking them sample by sample
+// leaves most threads idle and a thread's loads one behind the other (83 GB/s on AlexNet's layers). Here the
+// workgroup's samples are one index space (sample, access), a thread takes every EB-th of it, four in flight.
+template <int V, class E>
+__device__ __forceinline__ float bias_grad_small_planes(const E* __restrict__ dy, int n0, int n1, int K, int k, int PQ) {
+    const int pqv = PQ / V, total = (n1 - n0) * pqv;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int j = threadIdx.x; j < total; j += 4 * EB) {
+        float t[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int jj = j + u * EB;
+            const int n = jj / pqv, i = jj - n * pqv;
+            t[u] = jj < total ? sum_of_run<V>(dy + ((size_t)(n0 + n) * K + k) * PQ + (size_t)i * V) : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) s[u] += t[u];
+    }
+    return (s[0] + s[1]) + (s[2] + s[3]);
+}
+
 // stage 1: workgroup (k, split) sums samples [n0, n1) of channel k into partial[k*splits + split]
 template <class E>
 __global__ void __launch_bounds__(EB) bias_grad_partial_kernel(const E* __restrict__ dy, float* __restrict__ partial,
@@ -359,7 +394,14 @@ __global__ void __launch_bounds__(EB) bias_grad_partial_kernel(const E* __restri
     const int k = blockIdx.x / splits, sp = blockIdx.x % splits;
     const int n0 = sp * n_per_split, n1 = min(N, n0 + n_per_split);
     float acc = 0.0f;
-    if (sizeof(E) == 2 && (PQ & 7) == 0 && (((uintptr_t)dy & 15) == 0)) {
+    const bool aligned = (((uintptr_t)dy & 15) == 0);
+    if (sizeof(E) == 2 && (PQ & 7) == 0 && aligned && (PQ >> 3) < EB) {
+        if constexpr (sizeof(E) == 2) acc = bias_grad_small_planes<8>(dy, n0, n1, K, k, PQ);
+    } else if ((PQ & 3) == 0 && aligned && (PQ >> 2) < EB && !(sizeof(E) == 2 && (PQ & 7) == 0)) {
+        acc = bias_grad_small_planes<4>(dy, n0, n1, K, k, PQ);
+    } else if (!((PQ & 3) == 0 && aligned) && PQ < EB) {
+        acc = bias_grad_small_planes<1>(dy, n0, n1, K, k, PQ);
+    } else if (sizeof(E) == 2 && (PQ & 7) == 0 && (((uintptr_t)dy & 15) == 0)) {
         // bfloat16: eight elements (16 bytes) per access, eight independent partial sums per thread
         typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
         float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
