@@ -12,6 +12,7 @@ import pytest
 import oracle
 import vdnn_implementation_amd.backend as be
 from gpu_util import announce
+from test_gpu_kernels import drawn_geometries
 from util import assert_close, assert_close_bf16, from_bf16_bits, to_bf16_bits
 from vdnn_implementation_amd.backend import check, lib
 
@@ -176,6 +177,12 @@ def test_conv_bf16(ctx, geom, algo):
         gb = d.f32(np.zeros_like(b))
         check(lib.vdnn_conv_bwd_bias(ctx.handle, None, g, ddy.ptr, gb.ptr))
         assert_close(gb.download(b.shape), oracle.conv_bwd_bias_sgd(og, dy, np.zeros_like(b), 1.0), 1e-4, "bwd bias")
+
+
+@pytest.mark.parametrize("geom", drawn_geometries(6, 16), ids=lambda g: "x".join(map(str, g)))
+@pytest.mark.parametrize("algo", [0, 1])
+def test_conv_bf16_drawn_geometries(ctx, geom, algo):
+    test_conv_bf16(ctx, geom, algo)
 
 
 @pytest.mark.parametrize("n,cin,cout", [(128, 1000, 520), (64, 2304, 512), (5, 41, 33), (72, 264, 136), (128, 12544, 200), (40, 72, 1000)])

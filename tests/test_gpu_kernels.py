@@ -103,6 +103,40 @@ def test_conv_random_against_oracle(ctx, geom):
     assert_close(gpu_conv_bwd_bias(ctx, g, dy, b, np.float32(-0.5)), oracle.conv_bwd_bias_sgd(og, dy, b, -0.5), TOL, "bwd bias")
 
 
+def drawn_geometries(seed, count, budget=2.5e8):
+    """Convolution geometries drawn from a seeded generator: channel counts around the kernels' tile and block sizes,
+    windows of 1 to 5, strides, paddings, planes around the sizes the vector loaders distinguish; small enough
+    (budget multiply-adds) for the checker."""
+    import random
+    rnd = random.Random(seed)
+    channels = [1, 2, 3, 4, 8, 16, 24, 32, 48, 64, 64, 64, 96, 128, 128, 130, 192, 256]
+    out = []
+    while len(out) < count:
+        n, c, k = rnd.randint(1, 6), rnd.choice(channels), rnd.choice(channels)
+        if rnd.random() < 0.6:
+            r = s = 3
+        else:
+            r, s = rnd.choice([1, 3, 5, 2]), rnd.choice([1, 3, 5, 2])
+        h = rnd.choice([rnd.randint(r, 40), rnd.choice([4, 6, 7, 8, 12, 14, 16, 28, 56])])
+        w = rnd.choice([rnd.randint(s, 40), rnd.choice([4, 8, 12, 14, 16, 20, 28, 32, 56, 64])])
+        ph, pw = rnd.choice([0, r // 2, r // 2, r // 2]), rnd.choice([0, s // 2, s // 2, s // 2])
+        sh = sw = 1
+        if rnd.random() < 0.2:
+            sh, sw = rnd.choice([1, 2]), rnd.choice([1, 2, 3])
+        if h < r or w < s:
+            continue
+        p, q = (h + 2 * ph - r) // sh + 1, (w + 2 * pw - s) // sw + 1
+        if p < 1 or q < 1 or n * c * k * r * s * p * q > budget:
+            continue
+        out.append((n, c, h, w, k, r, s, ph, pw, sh, sw))
+    return out
+
+
+@pytest.mark.parametrize("geom", drawn_geometries(5, 24), ids=lambda g: "x".join(map(str, g)))
+def test_conv_drawn_geometries_against_oracle(ctx, geom):
+    test_conv_random_against_oracle(ctx, geom)
+
+
 PERF_OPT_GEOMS = [
     (3, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1),
     (2, 128, 14, 14, 256, 3, 3, 1, 1, 1, 1),
