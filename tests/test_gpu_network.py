@@ -391,3 +391,54 @@ def test_unfused_optimizer_gives_the_bits_of_the_fused_step():
                     wf, bf = fused.get_params(l)
                     w1, b1 = net.get_params(l)
                     assert np.array_equal(wf.view(np.uint32), w1.view(np.uint32)) and np.array_equal(bf.view(np.uint32), b1.view(np.uint32))
+
+
+def drawn_stack(rnd):
+    """A layer table drawn from a seeded generator: one to four convolutions (windows 1 to 5, strides, paddings) with
+    ReLU / tanh / sigmoid, LRN and 2x2 or 3x3 pooling between them, one to three fully connected layers, softmax."""
+    n = rnd.randint(1, 5)
+    c, h, w = rnd.choice([1, 3, 3, 4]), rnd.randint(12, 34), rnd.randint(12, 34)
+    specs = []
+    for _ in range(rnd.randint(1, 4)):
+        k, r = rnd.choice([4, 8, 12, 16, 32, 64, 70]), rnd.choice([1, 3, 3, 3, 5])
+        pad, stride = rnd.choice([0, r // 2, r // 2]), rnd.choice([1, 1, 1, 2])
+        if h + 2 * pad < r or w + 2 * pad < r:
+            break
+        specs.append(layer_spec(rnd.choice([enums.CONV, enums.FC_CONV]), n, c, h, w, pad, stride, k, r))
+        h, w, c = (h + 2 * pad - r) // stride + 1, (w + 2 * pad - r) // stride + 1, k
+        act = rnd.choice([enums.RELU, enums.RELU, enums.RELU, enums.TANH, enums.SIGMOID, None])
+        if act is not None:
+            specs.append(layer_spec(act, n, c, h, w))
+        if rnd.random() < 0.25 and c >= 5:
+            specs.append(layer_spec(enums.LRN, n, c, h, w))
+        if rnd.random() < 0.6 and h >= 4 and w >= 4:
+            win, st = rnd.choice([(2, 2), (2, 2), (3, 2)])
+            specs.append(layer_spec(enums.POOL, n, c, h, w, 0, st, 0, win))
+            h, w = (h - win) // st + 1, (w - win) // st + 1
+        if h < 3 or w < 3:
+            break
+    feat = c * h * w
+    for depth in range(rnd.randint(1, 3)):
+        out = rnd.choice([10, 16, 33, 64, 100])
+        specs.append(layer_spec(enums.FC_GEMM, n, feat, 1, 1, 0, 0, out, 1))
+        feat = out
+        if depth < 2 and rnd.random() < 0.7:
+            specs.append(layer_spec(enums.RELU, n, feat, 1, 1))
+    if specs[-1].type == enums.RELU:
+        specs.pop()
+    specs.append(layer_spec(enums.SOFTMAX, n, feat, 1, 1))
+    return specs
+
+
+@pytest.mark.parametrize("index", range(12))
+def test_drawn_layer_tables_against_the_checker(index):
+    """Tables the built-in networks do not have (strided and unpadded convolutions in the middle, tanh and sigmoid,
+    LRN behind any layer, odd planes), each under a policy, an algorithm mode, lifetimes and an element type drawn
+    with it: layer by layer against the checker."""
+    import random
+    rnd = random.Random(1000 + index)
+    specs = drawn_stack(rnd)
+    policy = rnd.choice([enums.BASELINE, enums.VDNN_NONE, enums.VDNN_CONV, enums.VDNN_ALL])
+    algo = rnd.choice([enums.VDNN_MEMORY_OPT_ALGO, enums.VDNN_PERF_OPT_ALGO])
+    refined, bf16 = rnd.random() < 0.5, rnd.random() < 0.4
+    check_network_against_the_checker(None, specs[0].n, policy, algo, layers=specs, refined=refined, bf16=bf16)
