@@ -314,3 +314,62 @@ def test_bf16_rounding_against_torch():
     n = oracle.round_bf16(np.array([np.nan], np.float32))
     assert np.isnan(n[0]) and not (n.view(np.uint32)[0] & 0xFFFF)
     assert np.array_equal(oracle.round_bf16(got).view(np.uint32), got.view(np.uint32))  # idempotent
+
+
+def _drawn_small_geometries(seed, count):
+    """Convolution geometries from a seeded generator, small enough for torch in float64 on the CPU: windows 1 to 5,
+    strides 1 to 3, with and without padding, channel counts on both sides of the blocked GEMM's panel widths."""
+    import random
+    rnd = random.Random(seed)
+    out = []
+    while len(out) < count:
+        n, c, k = rnd.randint(1, 4), rnd.choice([1, 2, 3, 5, 8, 16, 17, 33]), rnd.choice([1, 2, 4, 7, 16, 24, 40])
+        r, s = rnd.choice([1, 2, 3, 3, 5]), rnd.choice([1, 2, 3, 3, 5])
+        h, w = rnd.randint(r, 19), rnd.randint(s, 19)
+        ph, pw = rnd.choice([0, r // 2, r - 1]), rnd.choice([0, s // 2, s - 1])
+        sh, sw = rnd.choice([1, 1, 2, 3]), rnd.choice([1, 1, 2, 3])
+        out.append((n, c, h, w, k, r, s, ph, pw, sh, sw))
+    return out
+
+
+@pytest.mark.parametrize("geom", _drawn_small_geometries(3, 24), ids=lambda g: "x".join(map(str, g)))
+def test_conv_drawn_geometries_against_torch_autograd(geom, acc):
+    """The checker's four convolution passes against torch's float64 convolution and its autograd on geometries drawn
+    from a seeded generator (the fixtures hold seven hand-picked ones): asymmetric windows, strides that leave columns
+    unread, paddings up to window - 1."""
+    import torch
+    n, c, h, w_, k, r, s, ph, pw, sh, sw = geom
+    g = oracle.shape(*geom)
+    rng = np.random.default_rng(sum(geom))
+    x = rng.standard_normal((n, c, h, w_)).astype(np.float32)
+    w = (rng.standard_normal((k, c, r, s)) / np.sqrt(c * r * s)).astype(np.float32)
+    b = rng.standard_normal(k).astype(np.float32)
+    xt = torch.tensor(x.astype(np.float64), requires_grad=True)
+    wt = torch.tensor(w.astype(np.float64), requires_grad=True)
+    bt = torch.tensor(b.astype(np.float64), requires_grad=True)
+    yt = torch.nn.functional.conv2d(xt, wt, bt, stride=(sh, sw), padding=(ph, pw))
+    dy = rng.standard_normal(tuple(yt.shape)).astype(np.float32)
+    yt.backward(torch.tensor(dy.astype(np.float64)))
+    assert oracle.conv_out_shape(g) == tuple(yt.shape)
+    assert_close(oracle.conv_fwd(g, x, w, b), yt.detach().numpy(), TOL, "fwd")
+    assert_close(oracle.conv_bwd_data(g, dy, w), xt.grad.numpy(), TOL, "bwd data")
+    alpha = np.float32(0.5)
+    assert_close(oracle.conv_bwd_filter_sgd(g, x, dy, w, alpha), w + alpha * wt.grad.numpy(), TOL, "bwd filter")
+    assert_close(oracle.conv_bwd_bias_sgd(g, dy, b, alpha), b + alpha * bt.grad.numpy(), TOL, "bwd bias")
+
+
+@pytest.mark.parametrize("case", [(2, 3, 9, 11, 2, 2), (1, 5, 13, 13, 3, 2), (3, 2, 8, 12, 2, 1), (2, 4, 7, 7, 3, 3), (1, 1, 6, 10, 3, 1)])
+def test_maxpool_drawn_shapes_against_torch_autograd(case):
+    """Unpadded max pooling with distinct values (no ties): forward and the gradient's route against torch."""
+    import torch
+    n, c, h, w_, win, stride = case
+    g = oracle.shape(n, c, h, w_, 0, win, win, 0, 0, stride, stride)
+    rng = np.random.default_rng(sum(case))
+    x = rng.permutation(n * c * h * w_).astype(np.float32).reshape(n, c, h, w_) / 7.0
+    xt = torch.tensor(x.astype(np.float64), requires_grad=True)
+    yt = torch.nn.functional.max_pool2d(xt, win, stride)
+    dy = rng.standard_normal(tuple(yt.shape)).astype(np.float32)
+    yt.backward(torch.tensor(dy.astype(np.float64)))
+    y = oracle.maxpool_fwd(g, x)
+    assert np.array_equal(y, yt.detach().numpy().astype(np.float32))
+    assert_close(oracle.maxpool_bwd(g, x, y, dy), xt.grad.numpy(), 1e-6, "bwd")
