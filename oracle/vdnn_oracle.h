@@ -10,7 +10,9 @@
  *
  * What pins each function (tests/test_oracle_*.py):
  *   conv fwd / bwd-data / bwd-filter : torch-CPU conv2d + autograd fixtures (tests/golden), adjoint
- *                                      identities in fp64, brute-force 7-deep loops
+ *                                      identities in fp64, brute-force 7-deep loops; torch's float64
+ *                                      conv2d + autograd at test time on geometries drawn from a seeded
+ *                                      generator (asymmetric windows, strides to 3, paddings to window - 1)
  *   bias add / bias grad / sub / fill: closed form
  *   fc fwd / bwd-data / bwd-weight   : numpy matmul
  *   relu                             : closed form incl. -0, NaN, inf
@@ -19,7 +21,8 @@
  *   tanh / sigmoid fwd / bwd         : torch.tanh / torch.sigmoid + autograd in float64, special values,
  *                                      the identities tanh(-x) = -tanh(x), sigmoid(x) + sigmoid(-x) = 1
  *   maxpool fwd / bwd                : torch max_pool2d + autograd fixtures on tie-free data
- *                                      (3x3 s2 overlapping and 2x2 s2); brute force.
+ *                                      (3x3 s2 overlapping and 2x2 s2), and at test time on five more
+ *                                      window / stride / plane shapes; brute force.
  *                                      TIE RULE OF maxpool bwd: PARITY UNPINNED (cuDNN closed, no
  *                                      test in the reference). First maximum in row-major window
  *                                      order is chosen here.
