@@ -29,7 +29,8 @@
  *   lrn fwd / bwd                    : torch local_response_norm fixtures, finite differences
  *   softmax fwd / bwd, softmax-CE    : torch fixtures; rows sum to 1; sum dx = 0; shift invariance
  *   network step                     : torch-CPU autograd fixture of a small net built from the same
- *                                      layer kinds; finite differences of the loss
+ *                                      layer kinds; finite differences of the loss; torch's float64
+ *                                      autograd at test time on ten layer tables drawn from a seeded generator
  *   seeded generator                 : fixture of first values + moments
  */
 #ifndef VDNN_ORACLE_H_

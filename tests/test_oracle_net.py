@@ -120,3 +120,100 @@ def test_alexnet_lrn_batch2_step_runs_and_is_finite():
     assert all(np.isfinite(net.grad(l)).all() for l in range(net.num_layers))
     assert np.abs(net.grad(0)).max() > 0
     net.close()
+
+
+CONV, TANH, SIGMOID = 1, 4, 5
+
+
+def drawn_table(rnd):
+    """A layer table from a seeded generator: one to three convolutions (windows 1 to 5, strides, paddings) with ReLU /
+    tanh / sigmoid, LRN and 2x2 or 3x3 pooling between them, one or two fully connected layers, softmax."""
+    n = rnd.randint(1, 4)
+    c, h, w = rnd.choice([1, 3, 4]), rnd.randint(10, 22), rnd.randint(10, 22)
+    t = []
+    for _ in range(rnd.randint(1, 3)):
+        k, r = rnd.choice([4, 8, 12, 17]), rnd.choice([1, 3, 3, 5])
+        pad, stride = rnd.choice([0, r // 2, r // 2]), rnd.choice([1, 1, 2])
+        t.append(L(rnd.choice([CONV, FC_CONV]), n, c, h, w, pad, stride, k, r))
+        h, w, c = (h + 2 * pad - r) // stride + 1, (w + 2 * pad - r) // stride + 1, k
+        act = rnd.choice([RELU, RELU, TANH, SIGMOID, None])
+        if act is not None:
+            t.append(L(act, n, c, h, w))
+        if rnd.random() < 0.3 and c >= 5:
+            t.append(L(LRN, n, c, h, w))
+        if rnd.random() < 0.6 and h >= 4 and w >= 4:
+            win = rnd.choice([2, 2, 3])
+            t.append(L(POOL, n, c, h, w, 0, 2, 0, win))
+            h, w = (h - win) // 2 + 1, (w - win) // 2 + 1
+        if h < 5 or w < 5:
+            break
+    feat = c * h * w
+    for depth in range(rnd.randint(1, 2)):
+        out = rnd.choice([7, 10, 16])
+        t.append(L(FC_GEMM, n, feat, 1, 1, 0, 0, out, 1))
+        feat = out
+        if depth == 0 and rnd.random() < 0.5:
+            t.append(L(rnd.choice([RELU, TANH]), n, feat, 1, 1))
+    if t[-1].type != FC_GEMM:
+        t.pop()
+    t.append(L(SOFTMAX, n, feat, 1, 1))
+    return t
+
+
+@pytest.mark.parametrize("index", range(10))
+def test_drawn_layer_tables_against_torch_autograd(index):
+    """The checker's step on tables the fixture does not have, against torch built at test time in float64: every
+    layer's output, the reported loss, every layer's input gradient (the reference's: no 1/N)."""
+    import random
+    import torch
+    F = torch.nn.functional
+    rnd = random.Random(500 + index)
+    table = drawn_table(rnd)
+    oracle.set_accumulate_double(True)
+    try:
+        net = oracle.Net(layers=table)
+        net.init_seeded(index + 1)
+        x = torch.tensor(net.input().astype(np.float64), requires_grad=True)
+        labels = net.label().reshape(table[-1].g.n, -1)
+        cur, outs, params = x, [], {}
+        for l, d in enumerate(table):
+            g = d.g
+            if d.type in (CONV, FC_CONV):
+                wt = torch.tensor(net.filter(l).astype(np.float64).reshape(g.k, g.c, g.r, g.s))
+                bt = torch.tensor(net.bias(l).astype(np.float64))
+                cur = F.conv2d(cur, wt, bt, stride=(g.stride_h, g.stride_w), padding=(g.pad_h, g.pad_w))
+            elif d.type == FC_GEMM:
+                wt = torch.tensor(net.filter(l).astype(np.float64).reshape(g.k, g.c))
+                bt = torch.tensor(net.bias(l).astype(np.float64))
+                cur = F.linear(cur.reshape(g.n, -1), wt, bt)
+            elif d.type == RELU:
+                cur = F.relu(cur)
+            elif d.type == TANH:
+                cur = torch.tanh(cur)
+            elif d.type == SIGMOID:
+                cur = torch.sigmoid(cur)
+            elif d.type == LRN:
+                cur = F.local_response_norm(cur, 5, alpha=1e-4, beta=0.75, k=2.0)
+            elif d.type == POOL:
+                cur = F.max_pool2d(cur, g.r, g.stride_h)
+            elif d.type == SOFTMAX:
+                cur = F.softmax(cur.reshape(g.n, -1), dim=1)
+            cur.retain_grad()
+            outs.append(cur)
+        target = torch.tensor(labels.astype(np.float64))
+        ce_sum = -(target * torch.log(outs[-1])).sum()
+        ce = net.forward()
+        for l in range(len(table)):
+            assert_close(net.dst(l).reshape(tuple(outs[l].shape)), outs[l].detach().numpy(), 2e-5, "dst %d" % l)
+        net.backward()
+        # the reference starts backward from dy = y - label at the softmax OUTPUT and passes it through the softmax
+        # layer's own backward (network.cu:1042-1054): the gradient of 0.5 * ||softmax(z) - label||^2, no 1/N
+        (0.5 * ((outs[-1] - target) ** 2).sum()).backward()
+        want_ce = float(ce_sum.detach()) / table[-1].g.n   # the reported loss: cross-entropy, mean over the batch
+        assert abs(ce - want_ce) <= 1e-5 * abs(want_ce)
+        assert_close(net.grad(0), x.grad.numpy(), 5e-5, "dx")
+        for l in range(1, len(table) - 1):
+            want = outs[l - 1].grad.numpy()
+            assert_close(net.grad(l).reshape(want.shape), want, 5e-5, "grad %d" % l)
+    finally:
+        oracle.set_accumulate_double(False)
