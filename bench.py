@@ -231,6 +231,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--profile-steps", type=int, default=4, help="steps of the pass that times every launch")
     ap.add_argument("--batch", type=int, default=128)
+    ap.add_argument("--cnn", default="VGG16", choices=["VGG16", "ALEXNET", "ALEXNET_LRN", "OVERFEAT"], help="the network (the metric is VGG16's)")
     ap.add_argument("--algo", default="VDNN_MEMORY_OPT_ALGO")
     ap.add_argument("--policies", default=DEFAULT_POLICIES)
     ap.add_argument("--cap-gb", type=float, default=0.0, help="artificial limit on pool bytes in use (0 = none)")
@@ -251,7 +252,9 @@ def main():
     from vdnn_implementation_amd import enums
     from vdnn_implementation_amd.network import Network, parse
 
-    cnn = enums.VGG16_128
+    # the headline is VGG16; the other built-in tables are there for profiles of the kernels VGG16 does not have (LRN,
+    # overlapping pooling, strided and large-window convolutions)
+    cnn = {"VGG16": enums.VGG16_128, "ALEXNET": enums.ALEXNET, "ALEXNET_LRN": enums.ALEXNET_LRN, "OVERFEAT": enums.OVERFEAT}[args.cnn]
     # the fp32 BASELINE's peak, from a replay of its allocation schedule: what the "+budgetX" rows divide by X
     with Network(cnn, enums.BASELINE, 0, args.batch, plan_only=True) as replay:
         assert replay.forwardPropagation() == 0 and replay.backwardPropagation() == 0
@@ -316,7 +319,7 @@ def main():
         achieved = d["flops"] / (d["ms"] * 1e-3) / 1e12
         peak = BF16_MFMA_PEAK_TFLOPS if "bf16" in dom else FP32_MFMA_PEAK_TFLOPS
         conv_all_tf = sum(v["flops"] for v in conv.values()) / (sum(v["ms"] for v in conv.values()) * 1e-3) / 1e12
-        traffic = measured_traffic().get(dom) if args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" and not headline_bf16 else None
+        traffic = measured_traffic().get(dom) if args.cnn == "VGG16" and args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" and not headline_bf16 else None
         roofline = {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                     "frac": achieved / peak, "traffic": traffic,
                     "traffic_unit": "bytes per launch (L2 fetch + write-back); read from profiles/%s" % os.path.basename(TRAFFIC_PROFILE),
@@ -328,11 +331,11 @@ def main():
                for k, v in sorted(prof.items(), key=lambda kv: -kv[1]["ms"])}
     fp32 = {k: v for k, v in results.items() if not (args.bf16 or is_bf16(k))}
     out = {
-        "metric": "VGG16-128 train img/s (VDNN_ALL vs BASELINE); peak HBM GB; conv MFMA util",
+        "metric": "VGG16-128 train img/s (VDNN_ALL vs BASELINE); peak HBM GB; conv MFMA util" if args.cnn == "VGG16" else "%s train img/s (not the metric's network)" % args.cnn,
         "value": results[head]["images_per_s"], "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": results[head]["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 (bf16 MFMA products, f32 accumulation, f32 master weights)" if headline_bf16 else "f32", "data": "synthetic (seeded N(0,1) inputs, integer labels, He-normal filters)",
-        "config": {"workload": "VGG16 %s batch %d, one SGD step (fwd+bwd), policy %s, %s" % ("bf16-storage" if headline_bf16 else "fp32", args.batch, head, args.algo),
+        "config": {"workload": "%s %s batch %d, one SGD step (fwd+bwd), policy %s, %s" % (args.cnn, "bf16-storage" if headline_bf16 else "fp32", args.batch, head, args.algo),
                    "batch": args.batch, "policy": head, "algo": args.algo},
         "policies": results,
         "vdnn_all_vs_baseline_speed": (results[head]["images_per_s"] / base["images_per_s"]) if base else None,
@@ -349,7 +352,7 @@ def main():
         "conv_mfma_util": conv_all_tf / peak if conv_all_tf else None,
         "roofline": roofline,
         "kernels": kernels,
-        "step_mfma_frac": args.batch * FLOP_PER_IMAGE / (results[head]["ms_per_step"] * 1e-3) / 1e12 / peak,
+        "step_mfma_frac": args.batch * FLOP_PER_IMAGE / (results[head]["ms_per_step"] * 1e-3) / 1e12 / peak if args.cnn == "VGG16" else None,
     }
     if args.zvc_standalone:
         log("[bench] compressed offload alone on the device")
