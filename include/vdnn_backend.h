@@ -194,8 +194,13 @@ int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape
  * (k x batch slices floats; 4 slices of the batch per compute unit divided by k, at least one) exceed the array is
  * rejected with VDNN_EINVAL. Calls no hipMalloc, hipFree or allocating library routine. All calls on one GPU
  * share that GPU's array: two calls that overlap there (different streams, different threads) race; calls on one
- * stream do not. */
+ * stream do not.
+ * The first call on a device looks up that device's address of the array and its number of compute units (two
+ * runtime queries, made once per device, thread-safe). Those queries must not run while a stream is being captured:
+ * before capturing on a device, call vdnn_conv_bwd_bias_sgd_noalloc_prepare() with that device current (vdnn_ctx_create
+ * on the device does the same). It allocates nothing either and may be called any number of times. */
 #define VDNN_NOALLOC_SCRATCH_BYTES (256u << 10)
+int vdnn_conv_bwd_bias_sgd_noalloc_prepare(void);
 int vdnn_conv_bwd_bias_sgd_noalloc(vdnn_stream_t stream, const vdnn_shape_t* shape, int dtype,
                                    const void* dy, float* bias, float alpha);
 /* cudnnConvolutionBackwardFilter with alpha=-lr, beta=1 (layer.cu:651-660):

@@ -71,6 +71,23 @@ def test_command_line_words():
     assert peaks[True]["peak_bytes"] <= 5.48e9 < peaks[False]["peak_bytes"]
 
 
+def test_command_line_reports_a_step_that_ran_out_of_memory():
+    """Under an artificial cap a step that does not fit returns -1 (layer.h:110-128 of the reference); the program then
+    prints no throughput and exits non-zero. A cap that the policy fits under runs as before."""
+    import json
+    exe = os.path.join(ROOT, "vdnn_implementation_amd", "bin", "vdnn")
+    out = subprocess.run([exe, "VGG16_64", "VDNN_NONE", "VDNN_MEMORY_OPT_ALGO", "--plan", "--cap-gb", "4", "--warmup", "1"], capture_output=True, text=True)
+    assert out.returncode == 3, (out.returncode, out.stderr)
+    assert "forwardPropagation returned -1" in out.stderr and "warm-up step 0" in out.stderr
+    last = json.loads(out.stdout.strip().splitlines()[-1])
+    assert last["error"] == "out of memory" and "images_per_s" not in last and "Elapsed Time" not in out.stdout
+    ok = subprocess.run([exe, "VGG16_64", "VDNN_ALL", "VDNN_MEMORY_OPT_ALGO", "--plan", "--cap-gb", "8"], capture_output=True, text=True)
+    assert ok.returncode == 0 and json.loads(ok.stdout.strip().splitlines()[-1])["peak_bytes"] < 8e9
+    # backward is where VDNN_ALL peaks (4.73 GB): a cap between the forward's need and that fails there
+    mid = subprocess.run([exe, "VGG16_64", "VDNN_ALL", "VDNN_MEMORY_OPT_ALGO", "--plan", "--cap-gb", "4.5"], capture_output=True, text=True)
+    assert mid.returncode == 3 and json.loads(mid.stdout.strip().splitlines()[-1])["failed_in"] in ("forward", "backward")
+
+
 def test_reference_shaped_main_compiles_against_the_public_headers():
     """The class headers a caller of the reference includes (network.h, layer.h, vdnn.h) live under include/:
     a main of the shape of vdnn.cu:56-83 builds with the host compiler and -Iinclude alone, links against the
@@ -322,6 +339,36 @@ def test_scheduling_slack_moves_the_same_bytes_and_leaks_nothing():
     with plan(VGG16_128, VDNN_ALL, offload_lag=2, prefetch_depth=4) as net:
         step(net)
         assert [p for _, p in net.prefetch_trace()] == list(range(35, -1, -1))
+
+
+def test_prefetch_depth_counts_packed_streams_on_their_way_back():
+    """prefetchDepth bounds the tensors held ahead of their backward, whether they come back whole or as packed streams
+    through the copy engine: at every fetch, the fetched tensors of layers still below the issuing layer (the new one
+    included) number at most prefetchDepth, and the sequence is the same top-down order with and without compression."""
+    traces = {}
+    for compress in (False, True):
+        for depth in (1, 2, 3):
+            with plan(VGG16_128, VDNN_ALL, refined=True, fuse=True, compress=compress, offload_lag=6, prefetch_depth=depth) as net:
+                step(net)
+                trace = net.prefetch_trace()
+                st = net.stats()
+            fetched = [p for _, p in trace]
+            assert sorted(fetched, reverse=True) == fetched and len(set(fetched)) == len(fetched)
+            assert st["offload_bytes"] == st["prefetch_bytes"] > 0
+            held_most = 0
+            for i, (issuer, ident) in enumerate(trace):
+                if issuer == ident:
+                    continue   # a layer that expands or fetches its own input at the start of its backward holds nothing ahead
+                held = [p for j, p in trace[:i + 1] if p < issuer and j != p]
+                held_most = max(held_most, len(held))
+                # (depth 1 is the reference's scan, network.cu:1198-1208: every layer's backward fetches the next tensor
+                # down, also a layer whose own input was fetched by the layer above; the bound holds from depth 2 on)
+                assert depth == 1 or len(held) <= depth, (compress, depth, issuer, held)
+            assert depth == 1 or held_most == depth, (compress, depth, held_most)
+            traces[compress, depth] = trace
+    for depth in (1, 2, 3):
+        assert [p for _, p in traces[True, depth]] == [p for _, p in traces[False, depth]]
+        assert traces[True, depth] == traces[False, depth]
 
 
 def test_unfused_optimizer_costs_one_more_copy_of_the_parameters():

@@ -109,6 +109,7 @@ BACKEND_SYMBOLS = {
     "vdnn_maxpool_bwd_in_place_ok": (_i, [_S]),
     "vdnn_conv_bwd_bias_sgd": (_i, [_vp, _vp, _S, _vp, _vp, _f]),
     "vdnn_conv_bwd_bias_sgd_noalloc": (_i, [_vp, _S, _i, _vp, _vp, _f]),
+    "vdnn_conv_bwd_bias_sgd_noalloc_prepare": (_i, []),
     "vdnn_conv_bwd_filter_sgd": (_i, [_vp, _vp, _S, _i, _vp, _vp, _vp, _f, _vp, _sz]),
     "vdnn_fc_fwd": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "vdnn_fc_bwd_data": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp]),

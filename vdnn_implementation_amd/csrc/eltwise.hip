@@ -6,7 +6,9 @@
 #include "backend_internal.h"
 #include "mfma_gemm.h"
 
+#include <atomic>
 #include <cfloat>
+#include <mutex>
 
 namespace vdnn {
 
@@ -924,28 +926,37 @@ static constexpr size_t kNoAllocScratchBytes = VDNN_NOALLOC_SCRATCH_BYTES;
 static __device__ __align__(256) float g_noalloc_scratch[kNoAllocScratchBytes / sizeof(float)];
 
 namespace {
-struct NoAllocDevice { float* scratch = nullptr; int num_cu = 0; bool ready = false; };
+// `ready` is published with release order after `scratch` and `num_cu` are written, and read with acquire order:
+// a thread that sees it set sees the two fields. The look-up itself is serialised by a mutex, so two threads that make
+// their first call on a device together query once.
+struct NoAllocDevice { float* scratch = nullptr; int num_cu = 0; std::atomic<bool> ready{false}; };
 constexpr int kMaxDevices = 64;
 NoAllocDevice g_noalloc_devices[kMaxDevices];
+std::mutex g_noalloc_lookup;
 } // namespace
 
 // Address of the current device's copy of the array and that device's number of compute units, looked up once per
-// device with that device current. Allocates nothing.
+// device with that device current. Allocates nothing. The look-up makes two runtime queries (hipGetSymbolAddress,
+// hipDeviceGetAttribute): it must not happen while a stream of the calling thread is being captured, so a caller that
+// captures runs vdnn_conv_bwd_bias_sgd_noalloc_prepare (or creates a context) on the device beforehand.
 static int noalloc_device(NoAllocDevice** out) {
     int dev = -1;
     VDNN_HIP(hipGetDevice(&dev));
     VDNN_REQUIRE(dev >= 0 && dev < kMaxDevices, "device index out of range");
     NoAllocDevice& d = g_noalloc_devices[dev];
-    if (!d.ready) {
-        float* ptr = nullptr;
-        VDNN_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(g_noalloc_scratch)));
-        VDNN_REQUIRE(ptr != nullptr, "no address for the scratch array on this device");
-        int cus = 0;
-        VDNN_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        VDNN_REQUIRE(cus > 0, "device reports no compute units");
-        d.scratch = ptr;
-        d.num_cu = cus;
-        d.ready = true;
+    if (!d.ready.load(std::memory_order_acquire)) {
+        std::lock_guard<std::mutex> lock(g_noalloc_lookup);
+        if (!d.ready.load(std::memory_order_relaxed)) {
+            float* ptr = nullptr;
+            VDNN_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(g_noalloc_scratch)));
+            VDNN_REQUIRE(ptr != nullptr, "no address for the scratch array on this device");
+            int cus = 0;
+            VDNN_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+            VDNN_REQUIRE(cus > 0, "device reports no compute units");
+            d.scratch = ptr;
+            d.num_cu = cus;
+            d.ready.store(true, std::memory_order_release);
+        }
     }
     *out = &d;
     return VDNN_OK;
@@ -1158,6 +1169,7 @@ int vdnn_bias_add(vdnn_ctx* ctx, vdnn_stream_t stream, int n, int k, int hw, con
 int vdnn_conv_bwd_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, const void* dy, float* bias, float alpha) {
     return ACT_CALL(conv_bwd_bias_impl, ctx, stream, shape, dy, bias, alpha, 1);
 }
+int vdnn_conv_bwd_bias_sgd_noalloc_prepare(void) { return vdnn::noalloc_prepare_current_device(); }
 int vdnn_conv_bwd_bias_sgd_noalloc(vdnn_stream_t stream, const vdnn_shape_t* shape, int dtype, const void* dy, float* bias, float alpha) {
     VDNN_REQUIRE(shape && dy && bias, "null argument");
     VDNN_REQUIRE(dtype == VDNN_DTYPE_F32 || dtype == VDNN_DTYPE_BF16, "unknown element type");

@@ -973,11 +973,13 @@ void Network::resetIsPrefetchedArray() {
 }
 
 /* addition (prefetchDepth > 1): the nearest offloaded, not yet fetched layer below currLayerId, as long
- * as fewer than prefetchDepth fetched tensors below currLayerId are still waiting for their backward */
+ * as fewer than prefetchDepth fetched tensors below currLayerId are still waiting for their backward. A packed
+ * stream that the copy engine has brought back into a staging block (fetchPackedToStaging: zvcFetched) waits for
+ * its backward like a tensor fetched whole, and counts. */
 int Network::findPrefetchLayerDeep(int currLayerId) {
     int outstanding = 0;
     for (int id = currLayerId - 1; id >= 0; id--)
-        if (isOffload[id] && isPrefetched[id]) outstanding++;
+        if (isOffload[id] && (isPrefetched[id] || zvcFetched[id])) outstanding++;
     if (outstanding >= options.prefetchDepth) return -1;
     for (int id = currLayerId - 1; id >= 0; id--) {
         if (isOffload[id] && !isPrefetched[id] && !zvcKept[id]) {

@@ -76,19 +76,37 @@ int main(int argc, char** argv) {
     /* Initialize network */
     Network network(cnnType, vdnnType, algoMode, batch, opt);
 
-    for (int i = 0; i < warmup; i++) {
-        network.forwardPropagation();
-        network.backwardPropagation();
-    }
+    /* A step that runs out of pool memory returns -1 when asked to (layer.h:110-128 of the reference: dynamic mode);
+     * under an artificial cap or a budget that is the expected failure, so the steps are run that way and the
+     * program says so and exits non-zero instead of printing a throughput. Without either, a failed request
+     * aborts as in the reference. */
+    const bool soft = opt.capBytes != 0 || opt.hbmBudgetBytes != 0;
+    auto step = [&](const char* phase, int i) {
+        int rc = network.forwardPropagation(soft);
+        const char* pass = "forward";
+        if (rc >= 0) { rc = network.backwardPropagation(soft); pass = "backward"; }
+        if (rc < 0) {
+            const NetworkStats st = network.stats();
+            fprintf(stderr, "vdnn: %s step %d: %sPropagation returned %d (out of pool memory: %zu bytes in use at the peak, cap %zu, "
+                            "budget %zu, plan_feasible %s, plan_peak_bytes %zu); no throughput to report\n",
+                    phase, i, pass, rc, st.peakBytesInUse, opt.capBytes, opt.hbmBudgetBytes, network.planFeasible() ? "true" : "false",
+                    network.planPeakBytes());
+            printf("{\"model\": \"%s\", \"policy\": \"%s\", \"algo\": \"%s\", \"batch\": %d, \"error\": \"out of memory\", \"failed_in\": \"%s\", "
+                   "\"plan_only\": %s, \"plan_feasible\": %s, \"plan_peak_bytes\": %zu}\n",
+                   argv[1], argv[2], argv[3], network.batch(), pass, opt.planOnly ? "true" : "false",
+                   network.planFeasible() ? "true" : "false", network.planPeakBytes());
+            fflush(stdout);
+            exit(3);
+        }
+    };
+
+    for (int i = 0; i < warmup; i++) step("warm-up", i);
     network.synchronize();
     network.resetPeak();
 
     /* Perform `steps` iterations of fwd/bwd propagation */
     auto t1 = high_resolution_clock::now();
-    for (int i = 0; i < steps; i++) {
-        network.forwardPropagation();
-        network.backwardPropagation();
-    }
+    for (int i = 0; i < steps; i++) step("timed", i);
     network.synchronize();
     auto t2 = high_resolution_clock::now();
 
