@@ -35,10 +35,11 @@ FLOP_PER_IMAGE = 92.82e9        # 3 passes over 13 convolutions and 3 FC layers
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "igemm_conv_vgg16_b128_pmc_traffic.txt")
 PACKED_FRACTION = {False: 0.60, True: 0.63}   # what a plan takes a packed stream to be of its tensor (measured: 0.57 / 0.60)
 
-# the default run: the reference's four policies as they are, BASELINE with fused rectifiers, the two fastest float
+# the default run: the reference's four policies as they are, BASELINE with fused rectifiers, BASELINE in the
+# perf-optimal algorithm mode (the policies above run the memory-optimal one), the two fastest float
 # configurations that hold a third of BASELINE's memory (one with the link unused, one that uses it) and one bfloat16 run
 DEFAULT_POLICIES = ",".join([
-    "BASELINE", "VDNN_NONE", "VDNN_CONV", "VDNN_ALL", "BASELINE+fused",
+    "BASELINE", "VDNN_NONE", "VDNN_CONV", "VDNN_ALL", "BASELINE+fused", "BASELINE+perf",
     "VDNN_ALL+refined+fused+zvc+budget3.0", "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.1",
     "VDNN_ALL+refined+bf16+fused+zvc+keep+inplace+recompute",
 ])
@@ -144,6 +145,10 @@ def run_config(Network, be, cnn, policy, algo, batch, steps, warmup, profile_ste
 
 def is_bf16(policy_name):
     return "bf16" in policy_name.split("+")[1:]
+
+
+def is_perf(policy_name):
+    return "perf" in policy_name.split("+")[1:]
 
 
 def best_within(results, base, floor_ratio, need_link):
@@ -289,8 +294,10 @@ def main():
         budget = [float(m[6:]) for m in mods if m.startswith("budget")]
         lag_given = [int(m[3:]) for m in mods if m.startswith("lag")]
         mods = [m for m in mods if not m.startswith("budget") and not m.startswith("lag")]
-        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep", "inplace", "recompute"}, name
-        _, policy, algo = parse("VGG16_128", word, args.algo)
+        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep", "inplace", "recompute", "perf"}, name
+        # "+perf": VDNN_PERF_OPT_ALGO, the workspace-using kernel variants (wide 3x3 layers as Winograd F(4x4, 3x3)): other
+        # sums than the memory-optimal kernels', so its loss is compared within the mode only
+        _, policy, algo = parse("VGG16_128", word, "VDNN_PERF_OPT_ALGO" if "perf" in mods else args.algo)
         bf16 = args.bf16 or "bf16" in mods
         # (what a plan sends over the link gets the slack that hides it: the plan chooses the offload lag itself - the
         # longest of those that fit with the fewest bytes on the link - and backward fetches ahead wherever the peak allows)
@@ -318,8 +325,8 @@ def main():
     prof = {}
     headline_bf16 = args.bf16 or all(is_bf16(n) for n in profiles)
     for pname, p in profiles.items():
-        if (args.bf16 or is_bf16(pname)) != headline_bf16:
-            continue
+        if (args.bf16 or is_bf16(pname)) != headline_bf16 or is_perf(pname) != is_perf(head):
+            continue   # (the kernel table and the roofline entry are those of the headline's element type and algorithm mode)
         for k, v in p.items():
             acc = prof.setdefault(k, {"launches": 0, "ms": 0.0, "flops": 0.0, "bytes": 0.0})
             for field in acc:
@@ -361,14 +368,15 @@ def main():
         # images/s over BASELINE's, both measured in this run
         "vs_baseline": ratio,
         "dtype": "bf16" if headline_bf16 else "f32", "data": "synthetic",
-        "config": {"workload": "%s %s batch %d, one SGD step (fwd+bwd), policy %s, %s" % (args.cnn, "bf16-storage" if headline_bf16 else "fp32", args.batch, head, args.algo),
+        "config": {"workload": "%s %s batch %d, one SGD step (fwd+bwd), policy %s, %s" % (args.cnn, "bf16-storage" if headline_bf16 else "fp32", args.batch, head, "VDNN_PERF_OPT_ALGO" if is_perf(head) else args.algo),
                    "batch": args.batch, "policy": head, "algo": args.algo, "configurations_run": len(results)},
         "roofline": roofline,
         "baseline_images_per_s": base["images_per_s"] if base else None,
         "peak_hbm_gb": results[head]["peak_hbm_gb"],
         "peak_hbm_reduction_vs_baseline": (base["peak_hbm_gb"] / results[head]["peak_hbm_gb"]) if base else None,
-        "losses_bit_identical": len({results[k]["loss"] for k in results if not is_bf16(k)}) <= 1
-        and len({results[k]["loss"] for k in results if is_bf16(k)}) <= 1,
+        # within an element type and an algorithm mode every configuration runs the same kernels on the same values
+        "losses_bit_identical": all(len({results[k]["loss"] for k in results if is_bf16(k) == b and is_perf(k) == p}) <= 1 for b in (False, True) for p in (False, True)),
+        "perf_opt_speed_vs_memory_opt": (results["BASELINE+perf"]["images_per_s"] / base["images_per_s"]) if base and "BASELINE+perf" in results else None,
         "conv_mfma_util": conv_all_tf / peak if conv_all_tf else None,
         # float only, same losses as the literal run bit for bit: the fastest VDNN configuration at >= 3x less memory than
         # BASELINE, and the fastest of those that move at least 0.5 GB over the link each way

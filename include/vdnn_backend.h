@@ -167,8 +167,21 @@ int vdnn_memcpy_d2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_dev, siz
  * layer.cu:432-439). */
 int vdnn_out_dim(int in, int pad, int window, int stride);
 /* cudnnGetConvolution*WorkspaceSize (layer.cu:268-294). algo_mode is a vdnnAlgoMode_t value.
- * VDNN_MEMORY_OPT_ALGO always returns 0. */
+ * VDNN_MEMORY_OPT_ALGO always returns 0. VDNN_PERF_OPT_ALGO (the reference asks cuDNN for its fastest algorithm,
+ * layer.cu:1013-1089): forward / backward data of 3x3, stride 1, padding 1 layers with at least 128 reduced and more
+ * than 64 produced channels and float activations run as Winograd F(4x4, 3x3) and take the transformed filter plus the
+ * transformed input and output of a chunk of samples (up to 512 MiB); other layers take a re-laid-out copy of the
+ * filter; backward filter takes room for the partial sums of its split reduction. A pass handed less than this runs
+ * the memory-optimal kernels. The _dtype form takes the element type of the activations (VDNN_DTYPE_*); the plain
+ * form assumes float. */
 size_t vdnn_conv_workspace_bytes(const vdnn_shape_t* shape, int algo_mode, int pass);
+size_t vdnn_conv_workspace_bytes_dtype(const vdnn_shape_t* shape, int algo_mode, int pass, int dtype);
+/* Tuning (no counterpart in the reference): the bytes that the transformed input and output of one chunk of samples
+ * may take in the Winograd variant's workspace; 0 restores the default (512 MiB). Returns the previous value. A
+ * process-wide setting: it changes what vdnn_conv_workspace_bytes reports and how the passes split the batch, so set
+ * it before networks are built, not between a query and the pass that uses its answer. Results do not depend on it
+ * (samples are independent in forward and backward data). */
+size_t vdnn_conv_winograd_chunk_bytes(size_t bytes);
 /* cudnnConvolutionForward + cudnnAddTensor (layer.cu:560-582): y = x (*) w + bias[k], the bias is
  * added once after the full reduction. bias may be NULL (no add). */
 int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,

@@ -147,20 +147,44 @@ PERF_OPT_GEOMS = [
 ]
 
 
+def winograd_workspace(geom, bwd, chunk_bytes=512 << 20):
+    """Bytes the Winograd variant of the perf-optimal mode takes for forward (bwd False) or backward data, 0 where the
+    variant does not apply: 3x3 / stride 1 / padding 1, at least 128 reduced channels (a multiple of 16), more than 64
+    produced ones. The transformed filter (36 x rows x reduced), then the transformed input (reduced x 36 x Tpad) and
+    output (rows x 36 x Tpad) of one chunk of samples, each rounded up to 256 bytes; Tpad = the chunk's 4x4 tiles rounded
+    up to 128; chunks of equal size whose input + output stay within chunk_bytes."""
+    n, c, h, w, k, r, s, ph, pw, sh, sw = geom
+    rows, red = (c, k) if bwd else (k, c)
+    if (r, s, ph, pw, sh, sw) != (3, 3, 1, 1, 1, 1) or red < 128 or red % 16 or rows <= 64 or h < 4 or w < 4:
+        return 0
+    per = ((h + 3) // 4) * ((w + 3) // 4)
+    most = max(1, min(n, chunk_bytes // ((rows + red) * 36 * per * 4)))
+    chunks = -(-n // most)
+    nc = -(-n // chunks)
+    tpad = -(-nc * per // 128) * 128
+    up = lambda b: -(-b // 256) * 256
+    return up(36 * rows * red * 4) + up(red * 36 * tpad * 4) + up(rows * 36 * tpad * 4)
+
+
 @pytest.mark.parametrize("geom", PERF_OPT_GEOMS, ids=lambda g: "x".join(map(str, g)))
 def test_conv_perf_opt_variants(ctx, geom):
-    """The workspace-using variants: forward and backward data read a re-laid-out filter bank in the
-    same reduction order, so they return the bits of the workspace-free kernels; backward filter may
-    split the reduction differently and is held to the tolerance against the checker."""
+    """The workspace-using variants. Wide 3x3 layers run forward and backward data as Winograd F(4x4, 3x3): other sums,
+    held to the tolerance against the checker (or, at sizes the checker cannot afford, against the workspace-free
+    kernels). Elsewhere forward and backward data read a re-laid-out filter bank in the same reduction order and return
+    the bits of the workspace-free kernels. Backward filter may split the reduction differently and is held to the
+    tolerance."""
     rng = np.random.default_rng(hash(geom) % (2 ** 31) + 1)
     g, og = be.shape(*geom), oracle.shape(*geom)
     n, c, h, w_, k, r, s_ = geom[:7]
     filter_bytes = k * c * r * s_ * 4
     fwd_ok = r * s_ <= 32 and c % 16 == 0
     bwd_ok = c > 4 and geom[9] == 1 and geom[10] == 1 and r * s_ <= 32 and k % 16 == 0
+    wino = winograd_workspace(geom, False), winograd_workspace(geom, True)
     assert lib.vdnn_conv_workspace_bytes(g, 0, 0) == lib.vdnn_conv_workspace_bytes(g, 0, 1) == lib.vdnn_conv_workspace_bytes(g, 0, 2) == 0
-    assert lib.vdnn_conv_workspace_bytes(g, 1, 0) == (filter_bytes if fwd_ok else 0)
-    assert lib.vdnn_conv_workspace_bytes(g, 1, 1) == (filter_bytes if bwd_ok else 0)
+    assert lib.vdnn_conv_workspace_bytes(g, 1, 0) == (wino[0] or (filter_bytes if fwd_ok else 0))
+    assert lib.vdnn_conv_workspace_bytes(g, 1, 1) == (wino[1] or (filter_bytes if bwd_ok else 0))
+    # with bfloat16 activations the variant does not apply: the packed filter's size, as before
+    assert lib.vdnn_conv_workspace_bytes_dtype(g, 1, 0, 1) == (filter_bytes if fwd_ok else 0)
     assert lib.vdnn_conv_workspace_bytes(g, 1, 2) % filter_bytes == 0
     if geom[0] == 128:
         assert lib.vdnn_conv_workspace_bytes(g, 1, 2) > (64 << 20)
@@ -169,18 +193,94 @@ def test_conv_perf_opt_variants(ctx, geom):
     b = rng.standard_normal(g.k).astype(np.float32)
     announce("conv perf-opt", geom, "fwd")
     y0, y1 = gpu_conv_fwd(ctx, g, x, w, b, algo=0), gpu_conv_fwd(ctx, g, x, w, b, algo=1)
-    assert np.array_equal(y0, y1)
+    if wino[0]:
+        assert_close(y1, y0, TOL, "fwd, Winograd against direct")
+        assert not np.array_equal(y0, y1)
+    else:
+        assert np.array_equal(y0, y1)
     dy = rng.standard_normal(y0.shape).astype(np.float32)
     announce("conv perf-opt", geom, "bwd_data")
-    assert np.array_equal(gpu_conv_bwd_data(ctx, g, dy, w, algo=0), gpu_conv_bwd_data(ctx, g, dy, w, algo=1))
+    d0, d1 = gpu_conv_bwd_data(ctx, g, dy, w, algo=0), gpu_conv_bwd_data(ctx, g, dy, w, algo=1)
+    if wino[1]:
+        assert_close(d1, d0, TOL, "bwd data, Winograd against direct")
+        assert not np.array_equal(d0, d1)
+    else:
+        assert np.array_equal(d0, d1)
     announce("conv perf-opt", geom, "bwd_filter")
     zero = np.zeros_like(w)
     got = gpu_conv_bwd_filter(ctx, g, x, dy, zero, np.float32(1.0), algo=1)
     if n * c * h * w_ * k <= 2 ** 28:  # sizes the checker finishes in seconds
         assert_close(got, oracle.conv_bwd_filter_sgd(og, x, dy, zero, 1.0), TOL, "bwd filter")
         assert_close(y1, oracle.conv_fwd(og, x, w, b), TOL, "fwd")
+        assert_close(d1, oracle.conv_bwd_data(og, dy, w), TOL, "bwd data")
     else:
         assert_close(got, gpu_conv_bwd_filter(ctx, g, x, dy, zero, np.float32(1.0), algo=0), TOL, "bwd filter, two split counts")
+
+
+# Winograd F(4x4, 3x3): planes that are whole 4x4 tiles and planes that are not (tiles stored in part, rows that are not
+# whole groups of four pixels take the scalar loads), channel counts at and beside the limits
+WINOGRAD_GEOMS = [
+    (3, 128, 8, 8, 128, 3, 3, 1, 1, 1, 1),
+    (2, 128, 14, 14, 256, 3, 3, 1, 1, 1, 1),   # 14 x 14: 4 x 4 tiles, the last ones half outside
+    (3, 144, 7, 9, 80, 3, 3, 1, 1, 1, 1),      # odd plane; 80 produced rows: one ragged row tile; backward data does not apply (80 < 128)
+    (2, 256, 13, 20, 96, 3, 3, 1, 1, 1, 1),    # rows of whole groups, a ragged last tile row
+    (5, 160, 4, 4, 65, 3, 3, 1, 1, 1, 1),      # one tile per sample, 65 rows
+    (1, 512, 28, 28, 192, 3, 3, 1, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("geom", WINOGRAD_GEOMS, ids=lambda g: "x".join(map(str, g)))
+@pytest.mark.parametrize("small_chunks", [False, True], ids=["one-chunk", "small-chunks"])
+def test_conv_winograd_against_oracle(ctx, geom, small_chunks):
+    """Forward (with and without the fused rectifier) and backward data (plain, gated, and written over the gating
+    input) of the perf-optimal mode's Winograd variant against the checker; with small chunks the batch is processed in
+    several pieces (two samples at a time), the last one shorter."""
+    per_sample = (geom[1] + geom[4]) * 36 * ((geom[2] + 3) // 4) * ((geom[3] + 3) // 4) * 4
+    chunk_bytes = int(2.5 * per_sample) if small_chunks else 0
+    rng = np.random.default_rng(hash(geom) % (2 ** 31) + 3)
+    g, og = be.shape(*geom), oracle.shape(*geom)
+    x = rng.standard_normal((g.n, g.c, g.h, g.w)).astype(np.float32)
+    w = (rng.standard_normal((g.k, g.c, 3, 3)) * np.sqrt(2.0 / (g.c * 9))).astype(np.float32)
+    b = rng.standard_normal(g.k).astype(np.float32)
+    want_y = oracle.conv_fwd(og, x, w, b)
+    dy = rng.standard_normal(want_y.shape).astype(np.float32)
+    want_dx = oracle.conv_bwd_data(og, dy, w)
+    lib.vdnn_conv_winograd_chunk_bytes(chunk_bytes)
+    try:
+        fwd_bytes, bwd_bytes = int(lib.vdnn_conv_workspace_bytes(g, 1, 0)), int(lib.vdnn_conv_workspace_bytes(g, 1, 1))
+        assert fwd_bytes == winograd_workspace(geom, False, chunk_bytes or 512 << 20) > 0
+        bwd_applies = winograd_workspace(geom, True, chunk_bytes or 512 << 20) > 0
+        if bwd_applies:
+            assert bwd_bytes == winograd_workspace(geom, True, chunk_bytes or 512 << 20)
+        with Dev(ctx) as d:
+            dx_, dw, db, ddy = d.up(x), d.up(w), d.up(b), d.up(dy)
+            y, gx = d.empty(want_y.shape), d.empty(x.shape)
+            ws = d.empty((max(fwd_bytes, bwd_bytes) // 4,))
+            announce("winograd", geom, chunk_bytes, "fwd")
+            check(lib.vdnn_conv_fwd(ctx.handle, None, g, 1, dx_.ptr, dw.ptr, db.ptr, y.ptr, ws.ptr, fwd_bytes))
+            assert_close(y.download(want_y.shape), want_y, TOL, "fwd")
+            announce("winograd", geom, chunk_bytes, "fwd + relu")
+            check(lib.vdnn_conv_fwd_relu(ctx.handle, None, g, 1, dx_.ptr, dw.ptr, db.ptr, y.ptr, ws.ptr, fwd_bytes))
+            got = y.download(want_y.shape)
+            assert_close(got, np.maximum(want_y, 0), TOL, "fwd + relu")
+            assert np.all(got >= 0)
+            # a workspace that is too small: the memory-optimal kernels run instead
+            check(lib.vdnn_conv_fwd(ctx.handle, None, g, 1, dx_.ptr, dw.ptr, db.ptr, y.ptr, ws.ptr, fwd_bytes - 256))
+            assert_close(y.download(want_y.shape), want_y, TOL, "fwd, short workspace")
+            announce("winograd", geom, chunk_bytes, "bwd_data")
+            check(lib.vdnn_conv_bwd_data(ctx.handle, None, g, 1, ddy.ptr, dw.ptr, gx.ptr, ws.ptr, bwd_bytes))
+            assert_close(gx.download(x.shape), want_dx, TOL, "bwd data")
+            announce("winograd", geom, chunk_bytes, "bwd_data gated")
+            check(lib.vdnn_conv_bwd_data_relu(ctx.handle, None, g, 1, ddy.ptr, dw.ptr, dx_.ptr, gx.ptr, ws.ptr, bwd_bytes))
+            gated = gx.download(x.shape)
+            assert_close(gated, np.where(x > 0, want_dx, 0), TOL, "bwd data gated")
+            assert np.all(gated[x <= 0] == 0)
+            announce("winograd", geom, chunk_bytes, "bwd_data over the gating input")
+            assert lib.vdnn_conv_bwd_data_in_place_ok(g)
+            check(lib.vdnn_conv_bwd_data_relu(ctx.handle, None, g, 1, ddy.ptr, dw.ptr, dx_.ptr, dx_.ptr, ws.ptr, bwd_bytes))
+            assert np.array_equal(dx_.download(x.shape), gated)
+    finally:
+        lib.vdnn_conv_winograd_chunk_bytes(0)
 
 
 def test_conv_tail_round_is_split_and_agrees_with_two_half_batches(ctx):

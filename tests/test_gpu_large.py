@@ -120,14 +120,15 @@ def test_dynamic_algo_ladder_on_the_device():
                 assert train(net, 2) == got
                 assert params_digest(net) == got_digest
         else:
-            # the last rung chooses the variant layer by layer from what the pool can hold; the variants agree bit
-            # for bit in forward and backward data, a wider split of the filter gradient only in the last places
+            # the last rung chooses the variant layer by layer from what the pool can hold; where it takes the
+            # workspace-using variant, wide 3x3 layers run as Winograd (other sums, same values to float rounding) and
+            # the filter gradient may split its reduction wider: the losses agree in all but the last places
             announce("VDNN_ALL built directly")
             with Network(VGG16_64, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 0, seed=5) as net:
                 want = train(net, 2)
-            assert got[0] == want[0]
-            a, b = np.frombuffer(got[1], np.float32)[0], np.frombuffer(want[1], np.float32)[0]
-            assert abs(a - b) <= 1e-5 * abs(b)
+            for step_got, step_want in zip(got, want):
+                a, b = np.frombuffer(step_got, np.float32)[0], np.frombuffer(step_want, np.float32)[0]
+                assert abs(a - b) <= 1e-5 * abs(b)
 
 
 def test_dynamic_algo_with_the_lifetime_options():
@@ -152,10 +153,11 @@ def test_dynamic_algo_with_the_lifetime_options():
         assert net.policy == VDNN_ALL and net.recomputed_layer() == 2 and any(net.grad_over_src(l) for l in range(net.num_layers))
         got = train(net, 2, dynamic=True)
         assert net.stats()["peak_bytes_in_use"] <= cap
-        # (the last rung chooses the convolution variant layer by layer: a wider split of a filter gradient differs in the last places)
-        assert got[0] == want[0]
-        a, b = np.frombuffer(got[1], np.float32)[0], np.frombuffer(want[1], np.float32)[0]
-        assert abs(a - b) <= 1e-5 * abs(b)
+        # (the last rung chooses the convolution variant layer by layer: Winograd forward / backward data and a wider split
+        # of a filter gradient differ from the memory-optimal kernels in the last places)
+        for step_got, step_want in zip(got, want):
+            a, b = np.frombuffer(step_got, np.float32)[0], np.frombuffer(step_want, np.float32)[0]
+            assert abs(a - b) <= 1e-5 * abs(b)
     announce("the same options built directly")
     with Network(VGG16_64, VDNN_ALL, VDNN_MEMORY_OPT_ALGO, 0, seed=5, **kw) as net:
         assert train(net, 2) == want and params_digest(net) == want_digest

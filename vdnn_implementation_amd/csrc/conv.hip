@@ -16,6 +16,7 @@
 #include "wgrad3x3_f32.h"
 #include "conv_smallc.h"
 #include "conv_smallc_mfma.h"
+#include "winograd_f32.h"
 
 namespace vdnn {
 
@@ -239,6 +240,105 @@ static bool is_dense(const ConvGeo& g) { return g.P == 1 && g.Q == 1 && g.ph == 
 static bool packed_fwd_ok(const ConvGeo& g) { return g.R * g.S <= 32 && g.C % KB == 0; }
 static bool packed_bwd_data_ok(const ConvGeo& g) {
     return g.C > 4 && g.sh == 1 && g.sw == 1 && g.R * g.S <= 32 && g.K % KB == 0;
+}
+
+// ---- Winograd F(4x4, 3x3): the perf-optimal mode's forward / backward data of wide 3x3 layers (winograd_f32.h) -----
+// Samples are processed in chunks so that the transformed input V and the transformed output M of a chunk stay
+// within g_wino_chunk_bytes (512 MiB unless vdnn_conv_winograd_chunk_bytes says otherwise; and each below 2 GiB, the range of the product's descriptors). The plan depends on the shape
+// alone: vdnn_conv_workspace_bytes reports it, the pass follows it.
+constexpr size_t kWinoChunkBytesDefault = (size_t)512 << 20;
+static size_t g_wino_chunk_bytes = kWinoChunkBytesDefault; // vdnn_conv_winograd_chunk_bytes
+constexpr int kWinoMinReduced = 128;  // reduced channels from which the product's short reduction pays
+struct WinoPlan {
+    int rows, cred;        // output rows of the product (forward: K, backward data: C) and its reduction (C / K)
+    int th, tw, per;       // tiles per column, per row, per sample
+    int nc, chunks;        // samples per chunk, chunks
+    long Tpad;             // columns per xi of a full chunk
+    size_t u_bytes, v_bytes, m_bytes, total;
+};
+static bool wino_ok(const ConvGeo& g, bool bwd) {
+    const int rows = bwd ? g.C : g.K, cred = bwd ? g.K : g.C;
+    return g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W &&
+           cred >= kWinoMinReduced && cred % KB == 0 && rows > 64 && g.H >= 4 && g.W >= 4;
+}
+static WinoPlan wino_plan(const ConvGeo& g, bool bwd) {
+    WinoPlan p;
+    p.rows = bwd ? g.C : g.K; p.cred = bwd ? g.K : g.C;
+    p.th = (g.H + 3) / 4; p.tw = (g.W + 3) / 4; p.per = p.th * p.tw;
+    const size_t per_sample = (size_t)(p.rows + p.cred) * WINO_XI * p.per * sizeof(float);
+    long most = (long)(g_wino_chunk_bytes / per_sample);
+    if (most < 1) most = 1;
+    if (most > g.N) most = g.N;
+    p.chunks = (int)((g.N + most - 1) / most);
+    p.nc = (g.N + p.chunks - 1) / p.chunks;
+    p.Tpad = ((long)p.nc * p.per + WINO_TN - 1) / WINO_TN * WINO_TN;
+    auto up = [](size_t b) { return (b + 255) / 256 * 256; };
+    p.u_bytes = up((size_t)WINO_XI * p.rows * p.cred * sizeof(float));
+    p.v_bytes = up((size_t)p.cred * WINO_XI * p.Tpad * sizeof(float));
+    p.m_bytes = up((size_t)p.rows * WINO_XI * p.Tpad * sizeof(float));
+    p.total = p.u_bytes + p.v_bytes + p.m_bytes;
+    return p;
+}
+static bool wino_plan_ok(const WinoPlan& p) {
+    return p.v_bytes < 0x7FFF0000ul && p.m_bytes < 0x7FFF0000ul && (long)WINO_XI * p.Tpad < (1l << 31) && p.rows <= 65535 && p.cred <= 65535;
+}
+
+// in: x (forward) or dy (backward data); out: y or dx. Returns VDNN_OK with *taken false when the shape or the
+// workspace does not allow the variant.
+static int launch_winograd(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, bool bwd, const float* in, const float* w, const float* bias, float* out,
+                           int relu, const float* gate, void* workspace, size_t workspace_bytes, bool* taken) {
+    *taken = false;
+    if (!wino_ok(g, bwd) || !workspace || !aligned16(workspace)) return VDNN_OK;
+    const WinoPlan p = wino_plan(g, bwd);
+    if (!wino_plan_ok(p) || workspace_bytes < p.total) return VDNN_OK;
+    *taken = true;
+    float* U = (float*)workspace;
+    float* V = (float*)((char*)workspace + p.u_bytes);
+    float* Mo = (float*)((char*)workspace + p.u_bytes + p.v_bytes);
+    {
+        const long total = (long)p.rows * p.cred;
+        ProfScope prof(ctx, st, "conv_wino_filter", 0.0, (9.0 + WINO_XI) * 4.0 * (double)total);
+        if (bwd) hipLaunchKernelGGL(wino_filter_kernel<true>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, U, p.rows, p.cred);
+        else hipLaunchKernelGGL(wino_filter_kernel<false>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, U, p.rows, p.cred);
+        VDNN_LAUNCH_CHECK();
+    }
+    const long plane = (long)g.H * g.W;
+    const bool vec = g.W % 4 == 0 && aligned16(in) && aligned16(out) && (!gate || aligned16(gate));
+    for (int n0 = 0; n0 < g.N; n0 += p.nc) {
+        const int nc = g.N - n0 < p.nc ? g.N - n0 : p.nc;
+        const int T = nc * p.per;
+        const long Tpad = ((long)T + WINO_TN - 1) / WINO_TN * WINO_TN;
+        const unsigned tblocks = (unsigned)((T + 255) / 256);
+        {
+            const WinoTiles ti{g.H, g.W, p.th, p.tw, p.cred, T, Tpad};
+            ProfScope prof(ctx, st, bwd ? "conv_bwd_data_wino_in" : "conv_fwd_wino_in", 0.0, 4.0 * ((double)nc * p.cred * plane + (double)p.cred * WINO_XI * T));
+            const float* src = in + (long)n0 * p.cred * plane;
+            if (vec) hipLaunchKernelGGL(wino_input_kernel<true>, dim3(tblocks, (unsigned)p.cred), dim3(256), 0, st, src, V, ti);
+            else hipLaunchKernelGGL(wino_input_kernel<false>, dim3(tblocks, (unsigned)p.cred), dim3(256), 0, st, src, V, ti);
+            VDNN_LAUNCH_CHECK();
+        }
+        {
+            GemmDims d = make_dims(p.rows, (int)(WINO_XI * Tpad), p.cred, 128, WINO_TN, 1);
+            LoadWinoU al{{U, (long)p.cred, p.rows, (unsigned)((size_t)p.rows * p.cred * sizeof(float))}, (long)p.rows * p.cred, d.mtiles, d.mtiles * d.ntiles,
+                         (int)(Tpad / WINO_TN)};
+            LoadDenseRowVec4 bl{V, WINO_XI * Tpad, (int)(WINO_XI * Tpad), (unsigned)((size_t)p.cred * WINO_XI * Tpad * sizeof(float))};
+            StoreDense<float> ep{Mo, nullptr, nullptr, WINO_XI * Tpad, 0, 1.0f, 0, 0, nullptr};
+            // work counted in the transformed domain: 36 products per 4x4 outputs and channel pair
+            const int rc = launch_igemm<128, WINO_TN>(ctx, st, bwd ? "conv_bwd_data_wino_gemm" : "conv_fwd_wino_gemm", al, bl, ep, d,
+                                                      2.0 * p.rows * (double)p.cred * WINO_XI * T);
+            if (rc != VDNN_OK) return rc;
+        }
+        {
+            const WinoTiles to{g.H, g.W, p.th, p.tw, p.rows, T, Tpad};
+            ProfScope prof(ctx, st, bwd ? "conv_bwd_data_wino_out" : "conv_fwd_wino_out", 0.0,
+                           4.0 * ((double)p.rows * WINO_XI * T + (double)nc * p.rows * plane * (gate ? 2.0 : 1.0)));
+            const long off = (long)n0 * p.rows * plane;
+            if (vec) hipLaunchKernelGGL(wino_output_kernel<true>, dim3(tblocks, (unsigned)p.rows), dim3(256), 0, st, Mo, out + off, bias, gate ? gate + off : nullptr, relu, to);
+            else hipLaunchKernelGGL(wino_output_kernel<false>, dim3(tblocks, (unsigned)p.rows), dim3(256), 0, st, Mo, out + off, bias, gate ? gate + off : nullptr, relu, to);
+            VDNN_LAUNCH_CHECK();
+        }
+    }
+    return VDNN_OK;
 }
 
 // The bfloat16 engine's filter operand lives at the front of the staging area (rounded and re-laid-out by a
@@ -517,6 +617,14 @@ static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
         VDNN_LAUNCH_CHECK();
     }
     if (fwd_smallc3x3_ok(g, sizeof(E))) return launch_fwd_smallc3x3<E>(ctx, st, g, x, w, bias, y, relu);
+    if constexpr (sizeof(E) == 4) {
+        if (algo_mode == 1) {
+            // perf-optimal: wide 3x3 layers as Winograd F(4x4, 3x3) through the workspace
+            bool taken = false;
+            const int rc = launch_winograd(ctx, st, g, false, x, w, bias, y, relu, nullptr, workspace, workspace_bytes, &taken);
+            if (taken || rc != VDNN_OK) return rc;
+        }
+    }
     if (g.R * g.S <= 32 && g.C % KB == 0) {
         // blocked tap-major reduction: one slice = one tap x 16 input channels
         const int RS = g.R * g.S;
@@ -641,6 +749,13 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
         return VDNN_OK;
     }
     VDNN_REQUIRE(pixel_tile_span_ok((long)g.K * g.P * g.Q, g.H * g.W, 256, (int)sizeof(E)), "output-gradient samples too large for one tile's descriptor");
+    if constexpr (sizeof(E) == 4) {
+        if (algo_mode == 1) {
+            bool taken = false;
+            const int rc = launch_winograd(ctx, st, g, true, dy, w, nullptr, dx, 0, gate, workspace, workspace_bytes, &taken);
+            if (taken || rc != VDNN_OK) return rc;
+        }
+    }
     const int RS = g.R * g.S;
     LoadFilterT al{w, g.C, RS, (unsigned)((long)g.K * g.C * RS * 4), FastDiv::make(RS)};
     StoreNCHW<E> ep{dx, nullptr, g.H * g.W, ctx->reduce_scratch, 0, gate};
@@ -879,14 +994,29 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
 
 extern "C" {
 
+size_t vdnn_conv_winograd_chunk_bytes(size_t bytes) {
+    const size_t before = g_wino_chunk_bytes;
+    g_wino_chunk_bytes = bytes ? bytes : kWinoChunkBytesDefault;
+    return before;
+}
+
 size_t vdnn_conv_workspace_bytes(const vdnn_shape_t* shape, int algo_mode, int pass) {
+    return vdnn_conv_workspace_bytes_dtype(shape, algo_mode, pass, VDNN_DTYPE_F32);
+}
+
+size_t vdnn_conv_workspace_bytes_dtype(const vdnn_shape_t* shape, int algo_mode, int pass, int dtype) {
     ConvGeo g;
     if (!shape || !geo_from_shape(shape, g)) return 0;
     if (algo_mode == 0 /* VDNN_MEMORY_OPT_ALGO */ || is_dense(g)) return 0;
-    // Perf-optimal mode: forward and backward data re-lay the filter bank out for 128-bit operand
-    // loads; backward filter takes a staging area large enough for the split count that fills the chip.
+    // Perf-optimal mode: wide 3x3 layers with float activations run forward and backward data as Winograd F(4x4, 3x3)
+    // and take the transformed filter, input and output of a chunk of samples; other layers re-lay the filter bank out
+    // for 128-bit operand loads; backward filter takes a staging area large enough for the split count that fills the chip.
     const int RS = g.R * g.S;
     const size_t filter_bytes = (size_t)g.K * g.C * RS * sizeof(float);
+    if (dtype == VDNN_DTYPE_F32 && pass != 2 && wino_ok(g, pass == 1)) {
+        const WinoPlan p = wino_plan(g, pass == 1);
+        if (wino_plan_ok(p)) return p.total;
+    }
     if (pass == 0) return packed_fwd_ok(g) ? filter_bytes : 0;
     if (pass == 1) return packed_bwd_data_ok(g) ? filter_bytes : 0;
     const int M = g.K, N = g.C * RS;

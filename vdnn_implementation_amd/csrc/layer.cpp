@@ -151,21 +151,21 @@ void Layer::setAlgoMode(vdnnAlgoMode_t m) {
 
 /* layer.cu:1013-1089: the two-way switch between workspace-free and workspace-using kernels; the
  * workspace sizes come from the back end (cudnnGet*WorkspaceSize, layer.cu:268-294) */
-void Layer::findMemOptFwdAlgo()       { fwdWorkSpaceSize = vdnn_conv_workspace_bytes(&shape, VDNN_MEMORY_OPT_ALGO, VDNN_PASS_FWD); }
-void Layer::findMemOptBwdFilterAlgo() { bwdFilterWorkSpaceSize = vdnn_conv_workspace_bytes(&shape, VDNN_MEMORY_OPT_ALGO, VDNN_PASS_BWD_FILTER); }
-void Layer::findMemOptBwdDataAlgo()   { bwdDataWorkSpaceSize = vdnn_conv_workspace_bytes(&shape, VDNN_MEMORY_OPT_ALGO, VDNN_PASS_BWD_DATA); }
-void Layer::findPerfOptFwdAlgo()      { fwdWorkSpaceSize = vdnn_conv_workspace_bytes(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_FWD); }
-void Layer::findPerfOptBwdFilterAlgo(){ bwdFilterWorkSpaceSize = vdnn_conv_workspace_bytes(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_BWD_FILTER); }
-void Layer::findPerfOptBwdDataAlgo()  { bwdDataWorkSpaceSize = vdnn_conv_workspace_bytes(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_BWD_DATA); }
+void Layer::findMemOptFwdAlgo()       { fwdWorkSpaceSize = vdnn_conv_workspace_bytes_dtype(&shape, VDNN_MEMORY_OPT_ALGO, VDNN_PASS_FWD, vdnn_ctx_activation_dtype(ctx)); }
+void Layer::findMemOptBwdFilterAlgo() { bwdFilterWorkSpaceSize = vdnn_conv_workspace_bytes_dtype(&shape, VDNN_MEMORY_OPT_ALGO, VDNN_PASS_BWD_FILTER, vdnn_ctx_activation_dtype(ctx)); }
+void Layer::findMemOptBwdDataAlgo()   { bwdDataWorkSpaceSize = vdnn_conv_workspace_bytes_dtype(&shape, VDNN_MEMORY_OPT_ALGO, VDNN_PASS_BWD_DATA, vdnn_ctx_activation_dtype(ctx)); }
+void Layer::findPerfOptFwdAlgo()      { fwdWorkSpaceSize = vdnn_conv_workspace_bytes_dtype(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_FWD, vdnn_ctx_activation_dtype(ctx)); }
+void Layer::findPerfOptBwdFilterAlgo(){ bwdFilterWorkSpaceSize = vdnn_conv_workspace_bytes_dtype(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_BWD_FILTER, vdnn_ctx_activation_dtype(ctx)); }
+void Layer::findPerfOptBwdDataAlgo()  { bwdDataWorkSpaceSize = vdnn_conv_workspace_bytes_dtype(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_BWD_DATA, vdnn_ctx_activation_dtype(ctx)); }
 
 /* layer.cu:1091-1147: per-layer greedy choice by trial allocation. With two variants per pass this
  * reduces to: use the workspace variant when its workspace can be allocated right now. */
 void Layer::findDynamicAlgo() {
     if (layerType != CONV && layerType != FC_CONV) return;
-    size_t need = vdnn_conv_workspace_bytes(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_FWD);
-    size_t t = vdnn_conv_workspace_bytes(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_BWD_DATA);
+    size_t need = vdnn_conv_workspace_bytes_dtype(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_FWD, vdnn_ctx_activation_dtype(ctx));
+    size_t t = vdnn_conv_workspace_bytes_dtype(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_BWD_DATA, vdnn_ctx_activation_dtype(ctx));
     if (t > need) need = t;
-    t = vdnn_conv_workspace_bytes(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_BWD_FILTER);
+    t = vdnn_conv_workspace_bytes_dtype(&shape, VDNN_PERF_OPT_ALGO, VDNN_PASS_BWD_FILTER, vdnn_ctx_activation_dtype(ctx));
     if (t > need) need = t;
     void* probe = nullptr;
     if (need == 0 || vdnn_pool_malloc(ctx, &probe, need) == VDNN_OK) {

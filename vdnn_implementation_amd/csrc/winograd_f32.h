@@ -1,0 +1,257 @@
+// Winograd F(4x4, 3x3) for the forward and backward-data passes of 3x3 / stride 1 / padding 1 layers with float
+// activations: the perf-optimal mode's workspace-using variant (the reference asks cuDNN for its fastest algorithm and
+// hands it the workspace that algorithm wants, layer.cu:1013-1089, 268-294).
+//
+// An output tile of 4x4 pixels is computed from the 6x6 input patch around it as
+//     Y = At [ sum_c (G g_c Gt) .* (Bt d_c B) ] A
+// (g_c: the 3x3 filter of one input channel, d_c: the patch of that channel): 36 multiplies per channel for 16
+// outputs instead of 144 - a quarter of the direct convolution's. The sum over channels, for each of the 36 positions
+// xi of the transformed patch, is a matrix product  M_xi[m][t] = sum_c U_xi[m][c] * V_xi[c][t]  over all tiles t of a
+// chunk of samples; the 36 products run as ONE launch of the fp32 MFMA tile engine (columns j = xi * Tpad + t; the A
+// loader below picks U_xi from the column tile's index). Four kernels per call:
+//   1. wino_filter_kernel    U[xi][m][c]   = (G g Gt)[xi]            (backward data: the filter flipped and transposed)
+//   2. wino_input_kernel     V[c][xi][t]   = (Bt d B)[xi]            per chunk of samples
+//   3. igemm_kernel          M[m][xi][t]   = sum_c U[xi][m][c] V[c][xi][t]
+//   4. wino_output_kernel    y[n][m][tile] = At M A + bias, rectifier / gate applied
+// U, V and M live in the caller's workspace. Backward data is the same computation on dy with the filter
+// w'[c][k][r][s] = w[k][c][2-r][2-s]. Tiles at the right / lower edge of a plane whose extent is not a multiple of
+// four are computed whole and stored in part. The sums differ from the direct kernels' in order and by the
+// transforms' rounding (about 1.5e-5 of the largest output for 512 channels, against 3e-7 direct): results are
+// not bit-equal to the memory-optimal mode's, and equal from run to run and policy to policy within this mode.
+#pragma once
+#include "mfma_gemm.h"
+
+namespace vdnn {
+
+constexpr int WINO_XI = 36;   // positions of the transformed 6x6 patch
+constexpr int WINO_TN = 128;  // column tile of the product: a tile's columns share one xi
+
+// Bt v for the six values of a patch row / column
+__device__ __forceinline__ void wino_bt6(const float (&d)[6], float (&t)[6]) {
+    t[0] = 4.0f * d[0] - 5.0f * d[2] + d[4];
+    t[1] = -4.0f * (d[1] + d[2]) + d[3] + d[4];
+    t[2] = 4.0f * (d[1] - d[2]) - d[3] + d[4];
+    t[3] = 2.0f * (d[3] - d[1]) - d[2] + d[4];
+    t[4] = 2.0f * (d[1] - d[3]) - d[2] + d[4];
+    t[5] = 4.0f * d[1] - 5.0f * d[3] + d[5];
+}
+// At v: four outputs from six transformed values
+__device__ __forceinline__ void wino_at4(const float (&m)[6], float (&o)[4]) {
+    const float s12 = m[1] + m[2], d12 = m[1] - m[2], s34 = m[3] + m[4], d34 = m[3] - m[4];
+    o[0] = m[0] + s12 + s34;
+    o[1] = d12 + 2.0f * d34;
+    o[2] = s12 + 4.0f * s34;
+    o[3] = d12 + 8.0f * d34 + m[5];
+}
+// G v: six transformed values from three filter taps
+__device__ __forceinline__ void wino_g6(const float (&g)[3], float (&u)[6]) {
+    u[0] = g[0] * 0.25f;
+    u[1] = -(g[0] + g[1] + g[2]) * (1.0f / 6.0f);
+    u[2] = (g[1] - g[0] - g[2]) * (1.0f / 6.0f);
+    u[3] = g[0] * (1.0f / 24.0f) + g[1] * (1.0f / 12.0f) + g[2] * (1.0f / 6.0f);
+    u[4] = g[0] * (1.0f / 24.0f) - g[1] * (1.0f / 12.0f) + g[2] * (1.0f / 6.0f);
+    u[5] = g[2];
+}
+
+// U[(xi * rows + m) * cred + c]. Forward: m = k, c = c, taps as stored. Backward data: m = c, reduced index = k, taps
+// flipped. One thread per (m, c), lanes along c.
+template <bool BWD>
+__global__ void __launch_bounds__(256) wino_filter_kernel(const float* __restrict__ w, float* __restrict__ U, int rows, int cred) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (long)rows * cred) return;
+    const int m = (int)(i / cred), c = (int)(i - (long)m * cred);
+    // filter element (k, cc, r, s) at ((k * C + cc) * 3 + r) * 3 + s, with C = cred (forward) or rows (backward data)
+    const float* g = BWD ? w + ((long)c * rows + m) * 9 : w + ((long)m * cred + c) * 9;
+    float a[3][3];
+#pragma unroll
+    for (int r = 0; r < 3; r++)
+#pragma unroll
+        for (int s = 0; s < 3; s++) a[r][s] = BWD ? g[(2 - r) * 3 + (2 - s)] : g[r * 3 + s];
+    float t[6][3]; // G a
+#pragma unroll
+    for (int s = 0; s < 3; s++) {
+        const float col[3] = {a[0][s], a[1][s], a[2][s]};
+        float u[6];
+        wino_g6(col, u);
+#pragma unroll
+        for (int x = 0; x < 6; x++) t[x][s] = u[x];
+    }
+#pragma unroll
+    for (int x = 0; x < 6; x++) {
+        float u[6];
+        wino_g6(t[x], u);
+#pragma unroll
+        for (int y = 0; y < 6; y++) U[((long)(x * 6 + y) * rows + m) * cred + c] = u[y];
+    }
+}
+
+struct WinoTiles {
+    int H, W;          // plane (input and output planes have one extent)
+    int th, tw;        // tiles per column / row: ceil(H/4), ceil(W/4)
+    int chan;          // channels of the tensor (input transform: reduced channels; output transform: rows)
+    int T;             // tiles of the chunk: samples * th * tw
+    long Tpad;         // T rounded up to the product's column tile
+};
+
+// V[(c * 36 + xi) * Tpad + t] for the chunk's samples (src points at the chunk's first sample). One thread per
+// (c, t), lanes along t: the 36 stores of a wavefront are 256 contiguous bytes each. VEC: rows are whole groups of four
+// pixels, so a tile's four inner columns are one aligned 128-bit load.
+template <bool VEC>
+__global__ void __launch_bounds__(256) wino_input_kernel(const float* __restrict__ src, float* __restrict__ V, const WinoTiles g) {
+    const int t = blockIdx.x * 256 + threadIdx.x, c = blockIdx.y;
+    if (t >= g.T) return;
+    const int per = g.th * g.tw;
+    const int n = t / per, rem = t - n * per;
+    const int ty = rem / g.tw, tx = rem - ty * g.tw;
+    const float* plane = src + ((long)n * g.chan + c) * g.H * g.W;
+    float d[6][6];
+#pragma unroll
+    for (int i = 0; i < 6; i++) {
+        const int row = 4 * ty - 1 + i;
+        const bool rok = (unsigned)row < (unsigned)g.H;
+        const float* p = plane + (long)row * g.W + 4 * tx;
+        if (VEC) {
+            floatx4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (rok) v = *(const floatx4*)p;
+            d[i][0] = (rok && tx > 0) ? p[-1] : 0.0f;
+            d[i][1] = v.x; d[i][2] = v.y; d[i][3] = v.z; d[i][4] = v.w;
+            d[i][5] = (rok && 4 * tx + 4 < g.W) ? p[4] : 0.0f;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 6; j++) {
+                const int col = 4 * tx - 1 + j;
+                d[i][j] = (rok && (unsigned)col < (unsigned)g.W) ? p[j - 1] : 0.0f;
+            }
+        }
+    }
+    // Bt d: down the columns; then (Bt d) B: along the rows
+#pragma unroll
+    for (int j = 0; j < 6; j++) {
+        const float col[6] = {d[0][j], d[1][j], d[2][j], d[3][j], d[4][j], d[5][j]};
+        float r[6];
+        wino_bt6(col, r);
+#pragma unroll
+        for (int i = 0; i < 6; i++) d[i][j] = r[i];
+    }
+    float* out = V + (long)c * WINO_XI * g.Tpad + t;
+#pragma unroll
+    for (int i = 0; i < 6; i++) {
+        float r[6];
+        wino_bt6(d[i], r);
+#pragma unroll
+        for (int j = 0; j < 6; j++) out[(long)(i * 6 + j) * g.Tpad] = r[j];
+    }
+}
+
+// dst[n][m][4 ty + i][4 tx + j] = (At M A)[i][j] + bias[m], rectified / gated like the direct kernels' epilogue
+// (bias, then the rectifier, then the gate: kept where gate > 0). M[(m * 36 + xi) * Tpad + t]. One thread per (m, t),
+// lanes along t. A gate that is the output tensor itself is read by the thread that overwrites it, before it does.
+template <bool VEC>
+__global__ void __launch_bounds__(256) wino_output_kernel(const float* __restrict__ M, float* dst, const float* __restrict__ bias, const float* gate,
+                                                          int relu, const WinoTiles g) {
+    const int t = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
+    if (t >= g.T) return;
+    const int per = g.th * g.tw;
+    const int n = t / per, rem = t - n * per;
+    const int ty = rem / g.tw, tx = rem - ty * g.tw;
+    const float* in = M + (long)m * WINO_XI * g.Tpad + t;
+    float a[4][6]; // At M
+#pragma unroll
+    for (int j = 0; j < 6; j++) {
+        float col[6];
+#pragma unroll
+        for (int i = 0; i < 6; i++) col[i] = in[(long)(i * 6 + j) * g.Tpad];
+        float o[4];
+        wino_at4(col, o);
+#pragma unroll
+        for (int i = 0; i < 4; i++) a[i][j] = o[i];
+    }
+    const float b = bias ? bias[m] : 0.0f;
+    const long plane = ((long)n * g.chan + m) * g.H * g.W;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int row = 4 * ty + i;
+        if (row >= g.H) break;
+        float o[4];
+        wino_at4(a[i], o);
+        const long at = plane + (long)row * g.W + 4 * tx;
+        if (VEC) {
+            floatx4 gt = {1.0f, 1.0f, 1.0f, 1.0f};
+            if (gate) gt = *(const floatx4*)(gate + at);
+            floatx4 r;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float v = o[j] + b;
+                if (relu) v = relu_value(v);
+                r[j] = gt[j] > 0.0f ? v : 0.0f;
+            }
+            *(floatx4*)(dst + at) = r;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (4 * tx + j >= g.W) break;
+                float v = o[j] + b;
+                if (relu) v = relu_value(v);
+                if (gate) v = gate[at + j] > 0.0f ? v : 0.0f;
+                dst[at + j] = v;
+            }
+        }
+    }
+}
+
+// The product's A operand: U_xi, a dense reduction-major matrix of `rows` x `ld`, where xi belongs to the column tile
+// of the workgroup. The loader decodes the workgroup's tile the way igemm_kernel does for an unsplit launch.
+struct LoadWinoU : LoadDenseRed<true, float> {
+    long xi_stride;   // elements of one U_xi
+    int mtiles, ntiles_all, tiles_per_xi;
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int row0, int tid, int, int) const {
+        const int bid = xcd_remap(blockIdx.x, gridDim.x);
+        const int nt = (bid % ntiles_all) / mtiles;
+        const int xi = nt / tiles_per_xi;
+        st.rsrc = make_rsrc(base + (long)xi * xi_stride, bytes);
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) {
+            const int row = row0 + (tid >> 2) + 64 * i;
+            st.vrow[i] = row < rows ? (int)(((long)row * ld + 4 * (tid & 3)) * 4) : OOB;
+        }
+    }
+};
+
+// The product's B operand: V as a dense row-major matrix (element (column j, kk) at base[kk * ld_k + j]) whose rows
+// are whole groups of four columns, 16-byte aligned, and whose reduction is a whole number of slices: a thread moves two
+// 128-bit chunks per slice (chunk tid % (T/4) of reduction rows tid / (T/4) + (NT / (T/4)) * i) instead of eight single
+// elements. The thread's own reduction row rides in its vector offset, the slice's in the scalar offset.
+struct LoadDenseRowVec4 {
+    static constexpr bool RED_MAJOR = false;
+    const float* base;
+    long ld_k;        // elements between consecutive kk (a multiple of four)
+    int rows;         // columns of the matrix (a multiple of four)
+    unsigned bytes;   // extent in bytes (below 2 GiB)
+    template <int T> struct Regs { floatx4 v[T * KB / (4 * NT)]; };
+    template <int T> struct State { int vrow; __amdgpu_buffer_rsrc_t rsrc; };
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int row0, int tid, int, int) const {
+        st.rsrc = make_rsrc(base, bytes);
+        const int row = row0 + 4 * (tid % (T / 4));
+        st.vrow = row < rows ? (int)(((long)(tid / (T / 4)) * ld_k + row) * 4) : OOB;
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int kk0, int kend, int, Regs<T>& r) const {
+        constexpr int PER = NT / (T / 4); // reduction rows covered by one round of the workgroup's loads
+#pragma unroll
+        for (int i = 0; i < T * KB / (4 * NT); i++) {
+            const int kk = kk0 + PER * i; // wave-uniform; a slice lies wholly inside the reduction or wholly beyond it
+            const int soff = kk < kend ? (int)((long)kk * ld_k * 4) : 0x7FFFFFF0;
+            r.v[i] = buf_load4(st.rsrc, st.vrow, soff);
+        }
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(float* lds, int tid, const Regs<T>& r) {
+        constexpr int PER = NT / (T / 4);
+#pragma unroll
+        for (int i = 0; i < T * KB / (4 * NT); i++) *(floatx4*)(lds + (tid / (T / 4) + PER * i) * T + 4 * (tid % (T / 4))) = r.v[i];
+    }
+};
+
+} // namespace vdnn
