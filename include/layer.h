@@ -133,6 +133,7 @@ public:
     /* Addition (recomputeFirstLayer): the forward kernel once more, from this layer's srcData into the given block */
     int     forwardAgainInto(void* into, bool isDynamic);
     void    biasGradientBeside(DATATYPE lr);
+    bool    biasGradientInFilterKernel() const;
     void    joinBiasGradient();
     int     convolutionBackwardOverSrc(int _layer_id_to_prefetch, DATATYPE* _prefetchedSrcData_h,
                                        void* _srcDataToPrefetch, unsigned long _prefetch_bytes, void* workSpace, bool isDynamic);

@@ -223,6 +223,26 @@ int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sha
                              const void* x, const void* dy, float* w, float alpha,
                              void* workspace, size_t workspace_bytes);
 
+/* cudnnConvolutionBackwardBias and cudnnConvolutionBackwardFilter (layer.cu:631-637, 651-660) in one call: both read
+ * dy, and for most shapes the filter-gradient kernel adds up the bias gradient from the values it streams (the
+ * filter-row kernel of 3x3 / stride 1 / padding 1 layers, the first-layer kernel, the Winograd variant; float
+ * activations) instead of a second pass over dy. vdnn_conv_bwd_filter_sums_bias says whether a shape's kernel does;
+ * where it does not, the call runs the kernels of vdnn_conv_bwd_bias[_sgd] behind the filter gradient on the same
+ * stream (a caller that wants them side by side on another stream issues the two calls itself). The bias gradient's
+ * sums take another order than vdnn_conv_bwd_bias_sgd's (same value to float rounding, fixed from run to run).
+ *   _bias_sgd:       w += alpha dW,  bias += alpha db
+ *   _bias:           dw = dW,        db = sum dy                 (optimizer step left out, see below)
+ *   _then_bias_sgd:  dw = dW,        bias += alpha db            (for a caller that applies dW later) */
+int vdnn_conv_bwd_filter_sums_bias(const vdnn_shape_t* shape, int algo_mode, int dtype);
+int vdnn_conv_bwd_filter_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                                  const void* x, const void* dy, float* w, float* bias, float alpha,
+                                  void* workspace, size_t workspace_bytes);
+int vdnn_conv_bwd_filter_bias(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                              const void* x, const void* dy, float* dw, float* db, void* workspace, size_t workspace_bytes);
+int vdnn_conv_bwd_filter_then_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                                       const void* x, const void* dy, float* dw, float* bias, float alpha,
+                                       void* workspace, size_t workspace_bytes);
+
 /* The same two reductions with the optimizer step left out: db[k] = sum dy, dw = sum dy*x (beta = 0).
  * The reference always fuses SGD into these calls (alpha=-lr, beta=1); a training loop that keeps
  * gradients (to average them over devices, or to apply another optimizer) needs them separately.

@@ -160,7 +160,7 @@ def test_networks_that_write_gradients_over_inputs_keep_every_bit(cnn, batch, al
             got = run_steps(net, 2)
             peak = net.stats()["peak_bytes_in_use"]
         assert_bit_identical(got, plain, "policy %d %s" % (policy, kw))
-        assert peak <= peak_apart
+        assert peak <= peak_apart + (512 * 512 * 9 * 4 if algo == VDNN_PERF_OPT_ALGO else 0)   # (see below)
     # fused rectifiers: every convolution above the first and every 2x2 pooling layer
     shrinks = 0
     for policy, kw in ((VDNN_NONE, {}), (VDNN_CONV, {}), (VDNN_ALL, {}), (VDNN_ALL, {"host_sync": True}),
@@ -196,7 +196,11 @@ def test_networks_that_write_gradients_over_inputs_keep_every_bit(cnn, batch, al
         assert_fused_matches(got, plain, specs, "policy %d %s" % (policy, kw), offloaded)
         if "hbm_budget_bytes" in kw:
             continue   # (a budget keeps on the device what fits: more than the policy's own offload set would)
-        assert peak <= peak_apart
+        # The in-place order keeps a filter-sized gradient block while backward filter runs. In the perf-optimal mode that
+        # pass holds its Winograd workspace at the same time, and at a batch of two the block (9.4 MB for 512 x 512 x 3 x 3)
+        # outweighs the activation gradient it saves (3.2 MB): the peak may exceed the separate-blocks one by that block.
+        slack = 512 * 512 * 9 * 4 if algo == VDNN_PERF_OPT_ALGO else 0
+        assert peak <= peak_apart + slack
         shrinks += peak < peak_apart
     if cnn == VGG16_128:   # (the small tables' peaks are the parameters and the staging area)
         assert shrinks > 0, "writing gradients over inputs never lowered a peak"

@@ -166,6 +166,13 @@ def winograd_workspace(geom, bwd, chunk_bytes=512 << 20):
     return up(36 * rows * red * 4) + up(red * 36 * tpad * 4) + up(rows * 36 * tpad * 4)
 
 
+def winograd_wgrad_applies(geom):
+    """Backward filter as Winograd F(3x3, 4x4): 3x3 / stride 1 / padding 1, input channels a multiple of 128, more than
+    64 output channels."""
+    n, c, h, w, k, r, s, ph, pw, sh, sw = geom
+    return (r, s, ph, pw, sh, sw) == (3, 3, 1, 1, 1, 1) and c % 128 == 0 and k > 64 and h >= 4 and w >= 4
+
+
 @pytest.mark.parametrize("geom", PERF_OPT_GEOMS, ids=lambda g: "x".join(map(str, g)))
 def test_conv_perf_opt_variants(ctx, geom):
     """The workspace-using variants. Wide 3x3 layers run forward and backward data as Winograd F(4x4, 3x3): other sums,
@@ -185,7 +192,14 @@ def test_conv_perf_opt_variants(ctx, geom):
     assert lib.vdnn_conv_workspace_bytes(g, 1, 1) == (wino[1] or (filter_bytes if bwd_ok else 0))
     # with bfloat16 activations the variant does not apply: the packed filter's size, as before
     assert lib.vdnn_conv_workspace_bytes_dtype(g, 1, 0, 1) == (filter_bytes if fwd_ok else 0)
-    assert lib.vdnn_conv_workspace_bytes(g, 1, 2) % filter_bytes == 0
+    wino_filter = winograd_wgrad_applies(geom)
+    if wino_filter:
+        # the transformed input and output gradient of a chunk of samples and at least one partial result
+        tpad = -(-((h + 3) // 4) * ((w_ + 3) // 4) // 128) * 128
+        assert lib.vdnn_conv_workspace_bytes(g, 1, 2) >= (c + k) * 36 * tpad * 4 + 36 * k * c * 4
+    else:
+        assert lib.vdnn_conv_workspace_bytes(g, 1, 2) % filter_bytes == 0
+    assert lib.vdnn_conv_workspace_bytes_dtype(g, 1, 2, 1) % filter_bytes == 0
     if geom[0] == 128:
         assert lib.vdnn_conv_workspace_bytes(g, 1, 2) > (64 << 20)
     x = rng.standard_normal((g.n, g.c, g.h, g.w)).astype(np.float32)
@@ -275,12 +289,95 @@ def test_conv_winograd_against_oracle(ctx, geom, small_chunks):
             gated = gx.download(x.shape)
             assert_close(gated, np.where(x > 0, want_dx, 0), TOL, "bwd data gated")
             assert np.all(gated[x <= 0] == 0)
+            if winograd_wgrad_applies(geom):
+                # before the input is overwritten below: the filter gradient alone, then applied to the filter
+                announce("winograd", geom, chunk_bytes, "bwd_filter")
+                flt_bytes = int(lib.vdnn_conv_workspace_bytes(g, 1, 2))
+                assert flt_bytes > 0
+                ws2, gw, wu = d.empty((flt_bytes // 4,)), d.empty(w.shape), d.up(w)
+                check(lib.vdnn_conv_bwd_filter(ctx.handle, None, g, 1, dx_.ptr, ddy.ptr, gw.ptr, ws2.ptr, flt_bytes))
+                want_dw = oracle.conv_bwd_filter_sgd(og, x, dy, np.zeros_like(w), 1.0)
+                assert_close(gw.download(w.shape), want_dw, TOL, "bwd filter")
+                check(lib.vdnn_conv_bwd_filter_sgd(ctx.handle, None, g, 1, dx_.ptr, ddy.ptr, wu.ptr, np.float32(-0.37), ws2.ptr, flt_bytes))
+                assert_close(wu.download(w.shape), oracle.conv_bwd_filter_sgd(og, x, dy, w, -0.37), TOL, "bwd filter + sgd")
+                # twice the same bits: the sums have a fixed order
+                first = gw.download(w.shape)
+                check(lib.vdnn_conv_bwd_filter(ctx.handle, None, g, 1, dx_.ptr, ddy.ptr, gw.ptr, ws2.ptr, flt_bytes))
+                assert np.array_equal(gw.download(w.shape), first)
             announce("winograd", geom, chunk_bytes, "bwd_data over the gating input")
             assert lib.vdnn_conv_bwd_data_in_place_ok(g)
             check(lib.vdnn_conv_bwd_data_relu(ctx.handle, None, g, 1, ddy.ptr, dw.ptr, dx_.ptr, dx_.ptr, ws.ptr, bwd_bytes))
             assert np.array_equal(dx_.download(x.shape), gated)
     finally:
         lib.vdnn_conv_winograd_chunk_bytes(0)
+
+
+# (geometry, algorithm mode, whether the filter-gradient kernel of the shape adds up the bias gradient itself)
+FILTER_BIAS_GEOMS = [
+    ((7, 3, 40, 36, 16, 3, 3, 1, 1, 1, 1), 0, True),       # first-layer kernel: the product's spare column multiplies dy by one
+    ((2, 2, 16, 64, 70, 3, 3, 1, 1, 1, 1), 0, True),       # two input channels, a ragged second block of output channels
+    ((3, 64, 56, 56, 130, 3, 3, 1, 1, 1, 1), 0, True),     # filter-row kernel, three row tiles, the last ragged, many splits
+    ((4, 64, 14, 14, 64, 3, 3, 1, 1, 1, 1), 0, True),      # filter-row kernel, 64-row tile, groups across image rows
+    ((7, 128, 6, 20, 192, 3, 3, 1, 1, 1, 1), 0, True),     # two channel blocks: only the first block's workgroups sum
+    ((2, 128, 14, 14, 256, 3, 3, 1, 1, 1, 1), 1, True),    # Winograd: the dy transform sums what it reads
+    ((3, 128, 9, 7, 80, 3, 3, 1, 1, 1, 1), 1, True),       # Winograd, ragged tiles, odd rows (scalar loads)
+    ((2, 48, 27, 27, 96, 5, 5, 2, 2, 1, 1), 0, False),     # tile engine: the bias kernels run behind the filter gradient
+    ((2, 70, 9, 13, 130, 3, 3, 1, 1, 1, 1), 1, False),
+    ((5, 64, 6, 6, 200, 6, 6, 0, 0, 1, 1), 0, False),      # one dense product
+]
+
+
+@pytest.mark.parametrize("geom,algo,inside", FILTER_BIAS_GEOMS, ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v))
+def test_conv_bwd_filter_with_the_bias_gradient(ctx, geom, algo, inside):
+    """vdnn_conv_bwd_filter_bias_sgd / _bias / _then_bias_sgd (layer.cu:631-660 in one call) against the checker's two
+    reductions: the filter as with the separate call (same bits), the bias gradient within the tolerance (its sums take
+    another order inside the filter-gradient kernel), twice the same bits."""
+    rng = np.random.default_rng(hash(geom) % (2 ** 31) + 11)
+    g, og = be.shape(*geom), oracle.shape(*geom)
+    assert bool(lib.vdnn_conv_bwd_filter_sums_bias(g, algo, 0)) == inside
+    assert not lib.vdnn_conv_bwd_filter_sums_bias(g, algo, 1)      # bfloat16 activations: the separate kernels
+    x = rng.standard_normal((g.n, g.c, g.h, g.w)).astype(np.float32)
+    w = (rng.standard_normal((g.k, g.c, g.r, g.s)) * np.sqrt(2.0 / (g.c * g.r * g.s))).astype(np.float32)
+    b = rng.standard_normal(g.k).astype(np.float32)
+    P, Q = lib.vdnn_out_dim(g.h, g.pad_h, g.r, g.stride_h), lib.vdnn_out_dim(g.w, g.pad_w, g.s, g.stride_w)
+    dy = (rng.standard_normal((g.n, g.k, P, Q)) + 0.25).astype(np.float32)   # a mean: the bias gradient is not a sum that cancels
+    alpha = np.float32(-0.37)
+    want_w, want_b = oracle.conv_bwd_filter_sgd(og, x, dy, w, alpha), oracle.conv_bwd_bias_sgd(og, dy, b, alpha)
+    want_dw = oracle.conv_bwd_filter_sgd(og, x, dy, np.zeros_like(w), 1.0)
+    want_db = oracle.conv_bwd_bias_sgd(og, dy, np.zeros_like(b), 1.0)
+    nws = int(lib.vdnn_conv_workspace_bytes(g, algo, 2))
+    with Dev(ctx) as d:
+        dx_, ddy = d.up(x), d.up(dy)
+        ws = d.empty((max(nws, 4) // 4,)).ptr if nws else None
+        announce("bwd filter + bias", geom, algo, "sgd")
+        dw, db = d.up(w), d.up(b)
+        check(lib.vdnn_conv_bwd_filter_bias_sgd(ctx.handle, None, g, algo, dx_.ptr, ddy.ptr, dw.ptr, db.ptr, alpha, ws, nws))
+        got_w, got_b = dw.download(w.shape), db.download(b.shape)
+        assert_close(got_w, want_w, TOL, "filter")
+        assert_close(got_b, want_b, TOL, "bias")
+        assert not np.array_equal(got_b, b)
+        # the filter's bits are those of the call without the bias
+        dw2 = d.up(w)
+        check(lib.vdnn_conv_bwd_filter_sgd(ctx.handle, None, g, algo, dx_.ptr, ddy.ptr, dw2.ptr, alpha, ws, nws))
+        assert np.array_equal(dw2.download(w.shape), got_w)
+        announce("bwd filter + bias", geom, algo, "gradients")
+        gw, gb = d.up(np.full_like(w, 7.0)), d.up(np.full_like(b, 7.0))
+        check(lib.vdnn_conv_bwd_filter_bias(ctx.handle, None, g, algo, dx_.ptr, ddy.ptr, gw.ptr, gb.ptr, ws, nws))
+        got_dw, got_db = gw.download(w.shape), gb.download(b.shape)
+        assert_close(got_dw, want_dw, TOL, "dW")
+        assert_close(got_db, want_db, TOL, "db")
+        # db applied afterwards = the fused update (one fused multiply-add either way)
+        b2 = d.up(b)
+        check(lib.vdnn_sgd_apply(ctx.handle, None, g.k, alpha, gb.ptr, b2.ptr))
+        assert np.array_equal(b2.download(b.shape), got_b)
+        announce("bwd filter + bias", geom, algo, "gradient, then the bias step")
+        gw3, b3 = d.up(np.zeros_like(w)), d.up(b)
+        check(lib.vdnn_conv_bwd_filter_then_bias_sgd(ctx.handle, None, g, algo, dx_.ptr, ddy.ptr, gw3.ptr, b3.ptr, alpha, ws, nws))
+        assert np.array_equal(gw3.download(w.shape), got_dw)
+        assert np.array_equal(b3.download(b.shape), got_b)
+        # repeatable
+        check(lib.vdnn_conv_bwd_filter_bias(ctx.handle, None, g, algo, dx_.ptr, ddy.ptr, gw.ptr, gb.ptr, ws, nws))
+        assert np.array_equal(gb.download(b.shape), got_db) and np.array_equal(gw.download(w.shape), got_dw)
 
 
 def test_conv_tail_round_is_split_and_agrees_with_two_half_batches(ctx):

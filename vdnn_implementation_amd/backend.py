@@ -119,6 +119,10 @@ BACKEND_SYMBOLS = {
     "vdnn_fc_bwd_bias_sgd": (_i, [_vp, _vp, _i, _i, _vp, _vp, _f]),
     "vdnn_conv_bwd_bias": (_i, [_vp, _vp, _S, _vp, _vp]),
     "vdnn_conv_bwd_filter": (_i, [_vp, _vp, _S, _i, _vp, _vp, _vp, _vp, _sz]),
+    "vdnn_conv_bwd_filter_sums_bias": (_i, [_S, _i, _i]),
+    "vdnn_conv_bwd_filter_bias_sgd": (_i, [_vp, _vp, _S, _i, _vp, _vp, _vp, _vp, _f, _vp, _sz]),
+    "vdnn_conv_bwd_filter_bias": (_i, [_vp, _vp, _S, _i, _vp, _vp, _vp, _vp, _vp, _sz]),
+    "vdnn_conv_bwd_filter_then_bias_sgd": (_i, [_vp, _vp, _S, _i, _vp, _vp, _vp, _vp, _f, _vp, _sz]),
     "vdnn_fc_bwd_weight": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
     "vdnn_fc_bwd_bias": (_i, [_vp, _vp, _i, _i, _vp, _vp]),
     "vdnn_sgd_apply": (_i, [_vp, _vp, _sz, _f, _vp, _vp]),

@@ -206,6 +206,23 @@ static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
                          int splits, float alpha, int accumulate, const float* bias_j, int ncols, int relu = 0, const float* gate = nullptr);
+int launch_bias_grad_final(vdnn_ctx* ctx, hipStream_t st, const float* partial, float* bias, int K, int splits, float alpha, int accumulate);
+
+// The bias gradient as a by-product of backward filter (cudnnConvolutionBackwardBias, layer.cu:631-637, reads the same dy
+// as cudnnConvolutionBackwardFilter, :651-660): where the filter-gradient kernel of a shape can add up the dy values it
+// streams, it leaves per-channel partial sums in the context's bias staging area and `done` is set; the caller runs the
+// ordered final sum. out = (accumulate ? out : 0) + alpha * sum over n, p, q of dy.
+struct BiasOut {
+    float* out = nullptr;
+    float alpha = 1.0f;
+    int accumulate = 0;
+    bool done = false;
+    bool wanted() const { return out != nullptr; }
+};
+// room for K x parts partial sums in the bias staging area?
+static bool bias_parts_fit(const vdnn_ctx* ctx, int K, long parts) {
+    return ctx->bias_scratch && parts > 0 && (size_t)K * (size_t)parts * sizeof(float) <= ctx->bias_scratch_bytes;
+}
 
 // forward with the given A loader (128-bit or 32-bit filter loads)
 template <class AL, class E>
@@ -308,13 +325,13 @@ static int launch_winograd(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, bool
         const int nc = g.N - n0 < p.nc ? g.N - n0 : p.nc;
         const int T = nc * p.per;
         const long Tpad = ((long)T + WINO_TN - 1) / WINO_TN * WINO_TN;
-        const unsigned tblocks = (unsigned)((T + 255) / 256);
+        const unsigned tblocks = (unsigned)((T + 255) / 256), pblocks = (unsigned)((Tpad + 255) / 256);
         {
             const WinoTiles ti{g.H, g.W, p.th, p.tw, p.cred, T, Tpad};
             ProfScope prof(ctx, st, bwd ? "conv_bwd_data_wino_in" : "conv_fwd_wino_in", 0.0, 4.0 * ((double)nc * p.cred * plane + (double)p.cred * WINO_XI * T));
             const float* src = in + (long)n0 * p.cred * plane;
-            if (vec) hipLaunchKernelGGL(wino_input_kernel<true>, dim3(tblocks, (unsigned)p.cred), dim3(256), 0, st, src, V, ti);
-            else hipLaunchKernelGGL(wino_input_kernel<false>, dim3(tblocks, (unsigned)p.cred), dim3(256), 0, st, src, V, ti);
+            if (vec) hipLaunchKernelGGL(wino_input_kernel<true>, dim3(pblocks, (unsigned)p.cred), dim3(256), 0, st, src, V, ti);
+            else hipLaunchKernelGGL(wino_input_kernel<false>, dim3(pblocks, (unsigned)p.cred), dim3(256), 0, st, src, V, ti);
             VDNN_LAUNCH_CHECK();
         }
         {
@@ -337,6 +354,130 @@ static int launch_winograd(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, bool
             else hipLaunchKernelGGL(wino_output_kernel<false>, dim3(tblocks, (unsigned)p.rows), dim3(256), 0, st, Mo, out + off, bias, gate ? gate + off : nullptr, relu, to);
             VDNN_LAUNCH_CHECK();
         }
+    }
+    return VDNN_OK;
+}
+
+// Backward filter as Winograd F(3x3, 4x4) (winograd_f32.h): per chunk of samples the transformed input V and the
+// transformed output gradient D, then one launch of the tile engine for the 36 products S_xi = D_xi V_xi^t with the
+// reduction over the chunk's tiles split so that the grid fills the chip; every (chunk, split) leaves one partial
+// result, and a last kernel adds them in order, transforms back and applies alpha. The plan depends on the shape alone.
+constexpr size_t kWinoWgradPartialBytes = (size_t)256 << 20;
+struct WinoWgradPlan {
+    int th, tw, per, nc, chunks, splits;
+    long Tpad;
+    size_t v_bytes, d_bytes, part_bytes, total;   // part_bytes: one partial result
+};
+static bool wino_wgrad_ok(const ConvGeo& g) {
+    return g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W &&
+           g.C >= 128 && g.C % 128 == 0 && g.K > 64 && g.H >= 4 && g.W >= 4;
+}
+static WinoWgradPlan wino_wgrad_plan(const ConvGeo& g) {
+    WinoWgradPlan p;
+    p.th = (g.H + 3) / 4; p.tw = (g.W + 3) / 4; p.per = p.th * p.tw;
+    const size_t per_sample = (size_t)(g.K + g.C) * WINO_XI * p.per * sizeof(float);
+    long most = (long)(g_wino_chunk_bytes / per_sample);
+    if (most < 1) most = 1;
+    if (most > g.N) most = g.N;
+    p.chunks = (int)((g.N + most - 1) / most);
+    p.nc = (g.N + p.chunks - 1) / p.chunks;
+    p.chunks = (g.N + p.nc - 1) / p.nc;
+    p.Tpad = ((long)p.nc * p.per + WINO_TN - 1) / WINO_TN * WINO_TN;
+    auto up = [](size_t b) { return (b + 255) / 256 * 256; };
+    p.v_bytes = up((size_t)g.C * WINO_XI * p.Tpad * sizeof(float));
+    p.d_bytes = up((size_t)g.K * WINO_XI * p.Tpad * sizeof(float));
+    p.part_bytes = up((size_t)g.K * WINO_XI * g.C * sizeof(float));
+    // splits of a chunk's reduction: one round of resident workgroups, at least eight slices each, partial results within their budget
+    const long tiles = (long)WINO_XI * ((g.K + 127) / 128) * (g.C / 128);
+    long splits = 3l * kPlanningCUs / tiles;
+    const long by_len = p.Tpad / (8 * KB), by_mem = (long)(kWinoWgradPartialBytes / p.part_bytes) / p.chunks;
+    if (splits > by_len) splits = by_len;
+    if (splits > by_mem) splits = by_mem;
+    if (splits < 1) splits = 1;
+    // (the launch re-derives the split count from the chunk size through make_dims; this is its upper bound)
+    p.splits = (int)splits;
+    p.total = p.v_bytes + p.d_bytes + (size_t)p.chunks * p.splits * p.part_bytes;
+    return p;
+}
+static bool wino_wgrad_plan_ok(const WinoWgradPlan& p, const ConvGeo& g) {
+    return p.v_bytes < 0x7FFF0000ul && p.d_bytes < 0x7FFF0000ul && (long)WINO_XI * g.C < (1l << 24) && g.K <= 65535 && g.C <= 65535 &&
+           (long)p.chunks * p.splits < 4096;
+}
+
+static int launch_winograd_wgrad(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const float* x, const float* dy, float* w, float alpha, int accumulate,
+                                 void* workspace, size_t workspace_bytes, bool* taken, BiasOut* bias) {
+    *taken = false;
+    if (!wino_wgrad_ok(g) || !workspace || !aligned16(workspace)) return VDNN_OK;
+    const WinoWgradPlan p = wino_wgrad_plan(g);
+    if (!wino_wgrad_plan_ok(p, g) || workspace_bytes < p.total) return VDNN_OK;
+    *taken = true;
+    float* V = (float*)workspace;
+    float* D = (float*)((char*)workspace + p.v_bytes);
+    float* P = (float*)((char*)workspace + p.v_bytes + p.d_bytes);
+    const long part_stride = (long)(p.part_bytes / sizeof(float));
+    const long plane = (long)g.H * g.W;
+    const bool vec = g.W % 4 == 0 && aligned16(x) && aligned16(dy);
+    int nparts = 0;
+    // the bias gradient: every workgroup of the dy transform leaves the sum of the values it read
+    long bias_parts = 0;
+    for (int n0 = 0; n0 < g.N; n0 += p.nc) {
+        const int nc = g.N - n0 < p.nc ? g.N - n0 : p.nc;
+        bias_parts += (((long)nc * p.per + WINO_TN - 1) / WINO_TN * WINO_TN + 255) / 256;
+    }
+    const bool with_bias = bias && bias->wanted() && bias_parts < (1 << 20) && bias_parts_fit(ctx, g.K, bias_parts);
+    int bias_first = 0;
+    for (int n0 = 0; n0 < g.N; n0 += p.nc) {
+        const int nc = g.N - n0 < p.nc ? g.N - n0 : p.nc;
+        const int T = nc * p.per;
+        const long Tpad = ((long)T + WINO_TN - 1) / WINO_TN * WINO_TN;
+        const unsigned pblocks = (unsigned)((Tpad + 255) / 256);
+        {
+            const WinoTiles ti{g.H, g.W, p.th, p.tw, g.C, T, Tpad};
+            ProfScope prof(ctx, st, "conv_bwd_filter_wino_in", 0.0, 4.0 * ((double)nc * g.C * plane + (double)g.C * WINO_XI * Tpad));
+            const float* src = x + (long)n0 * g.C * plane;
+            if (vec) hipLaunchKernelGGL(wino_input_kernel<true>, dim3(pblocks, (unsigned)g.C), dim3(256), 0, st, src, V, ti);
+            else hipLaunchKernelGGL(wino_input_kernel<false>, dim3(pblocks, (unsigned)g.C), dim3(256), 0, st, src, V, ti);
+            VDNN_LAUNCH_CHECK();
+        }
+        {
+            const WinoTiles td{g.H, g.W, p.th, p.tw, g.K, T, Tpad};
+            ProfScope prof(ctx, st, "conv_bwd_filter_wino_dy", 0.0, 4.0 * ((double)nc * g.K * plane + (double)g.K * WINO_XI * Tpad));
+            const float* src = dy + (long)n0 * g.K * plane;
+            float* bp = with_bias ? ctx->bias_scratch : nullptr;
+            if (vec && with_bias) hipLaunchKernelGGL((wino_dy_kernel<true, true>), dim3(pblocks, (unsigned)g.K), dim3(256), 0, st, src, D, td, bp, (int)bias_parts, bias_first);
+            else if (vec) hipLaunchKernelGGL((wino_dy_kernel<true, false>), dim3(pblocks, (unsigned)g.K), dim3(256), 0, st, src, D, td, bp, 0, 0);
+            else if (with_bias) hipLaunchKernelGGL((wino_dy_kernel<false, true>), dim3(pblocks, (unsigned)g.K), dim3(256), 0, st, src, D, td, bp, (int)bias_parts, bias_first);
+            else hipLaunchKernelGGL((wino_dy_kernel<false, false>), dim3(pblocks, (unsigned)g.K), dim3(256), 0, st, src, D, td, bp, 0, 0);
+            VDNN_LAUNCH_CHECK();
+            bias_first += (int)pblocks;
+        }
+        {
+            GemmDims d = make_dims(g.K, WINO_XI * g.C, (int)Tpad, 128, WINO_TN, p.splits);
+            LoadWinoRed<true> al{D, Tpad, g.K, (unsigned)((size_t)g.K * WINO_XI * Tpad * sizeof(float)), g.C, d.mtiles, d.mtiles * d.ntiles, WINO_TN};
+            LoadWinoRed<false> bl{V, Tpad, g.C, (unsigned)((size_t)g.C * WINO_XI * Tpad * sizeof(float)), g.C, d.mtiles, d.mtiles * d.ntiles, WINO_TN};
+            float* slot = P + (long)nparts * part_stride;
+            StoreDense<float> ep{slot, slot, nullptr, (long)WINO_XI * g.C, part_stride, 1.0f, 0, 0, nullptr};
+            const int rc = launch_igemm<128, WINO_TN>(ctx, st, "conv_bwd_filter_wino_gemm", al, bl, ep, d, 2.0 * g.K * (double)g.C * WINO_XI * T);
+            if (rc != VDNN_OK) return rc;
+            nparts += d.splits;
+        }
+    }
+    {
+        const long total = (long)g.K * g.C, count = total * WINO_XI;
+        ProfScope prof(ctx, st, "conv_bwd_filter_wino_out", 0.0, 4.0 * ((double)nparts * WINO_XI + 18.0) * (double)total);
+        if (nparts > 2) {
+            // many partial results: summed with one thread per element first
+            hipLaunchKernelGGL(wino_wgrad_sum_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st, P, part_stride, nparts, count);
+            VDNN_LAUNCH_CHECK();
+            nparts = 1;
+        }
+        hipLaunchKernelGGL(wino_wgrad_out_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, P, part_stride, nparts, w, g.K, g.C, g.C, alpha, accumulate);
+        VDNN_LAUNCH_CHECK();
+    }
+    if (with_bias) {
+        const int rc = launch_bias_grad_final(ctx, st, ctx->bias_scratch, bias->out, g.K, (int)bias_parts, bias->alpha, bias->accumulate);
+        if (rc != VDNN_OK) return rc;
+        bias->done = true;
     }
     return VDNN_OK;
 }
@@ -483,7 +624,7 @@ static bool wgrad3x3_f32_ok(const ConvGeo& g) {
 
 // The float counterpart of launch_wgrad3x3.
 static int launch_wgrad3x3_f32(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const float* x, const float* dy, float* w, float alpha, int accumulate,
-                               float* staging, size_t staging_bytes, bool* taken) {
+                               float* staging, size_t staging_bytes, bool* taken, BiasOut* bias) {
     *taken = false;
     const int M = g.K, N = g.C * 9, PQ = g.H * g.W;
     const long Kred = (long)g.N * PQ;
@@ -509,7 +650,8 @@ static int launch_wgrad3x3_f32(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, 
     const long blocks = tiles * d.splits;
     if (blocks <= 0 || blocks >= (1l << 31)) return VDNN_OK;
     *taken = true;
-    const Wgrad3x3F geo{dy, x, g.N, g.K, g.C, g.H, g.W, w, staging, (long)M * N, alpha, accumulate};
+    const bool with_bias = bias && bias->wanted() && bias_parts_fit(ctx, g.K, d.splits);
+    const Wgrad3x3F geo{dy, x, g.N, g.K, g.C, g.H, g.W, w, staging, (long)M * N, alpha, accumulate, with_bias ? ctx->bias_scratch : nullptr, d.splits};
     {
         ProfScope prof(ctx, st, narrow ? kBwdFilterRow3Names.t64 : kBwdFilterRow3Names.t128, 2.0 * M * (double)N * (double)Kred, 0.0);
         const bool halfrow = g.W % 4 != 0 || g.W < KB; // the general variant: groups across two image rows, two row wraps per slice
@@ -518,6 +660,11 @@ static int launch_wgrad3x3_f32(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, 
         else if (halfrow) hipLaunchKernelGGL((wgrad3x3_f32_kernel<64, true>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
         else hipLaunchKernelGGL((wgrad3x3_f32_kernel<64, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
         VDNN_LAUNCH_CHECK();
+    }
+    if (with_bias) {
+        const int rc = launch_bias_grad_final(ctx, st, ctx->bias_scratch, bias->out, g.K, d.splits, bias->alpha, bias->accumulate);
+        if (rc != VDNN_OK) return rc;
+        bias->done = true;
     }
     if (d.splits > 1) return launch_reduce_splits_tap(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, accumulate, g.C, 9);
     return VDNN_OK;
@@ -795,13 +942,12 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
     return launch_by_m(ctx, st, kBwdDataNames, al, bl, ep, M, N, K, flops);
 }
 
-// out = (accumulate ? out : 0) + alpha * dW
+// out = (accumulate ? out : 0) + alpha * dW; the bias gradient too where the chosen kernel can (bias->done)
 template <class E>
-static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+static int conv_bwd_filter_core(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
                                 const E* x, const E* dy, float* w, float alpha, int accumulate,
-                                void* workspace, size_t workspace_bytes) {
+                                void* workspace, size_t workspace_bytes, BiasOut* bias) {
     VDNN_KERNEL_PROLOGUE(ctx);
-    (void)algo_mode;
     ConvGeo g;
     VDNN_REQUIRE(shape && geo_from_shape(shape, g), "unsupported convolution geometry");
     VDNN_REQUIRE(x && dy && w, "null tensor");
@@ -813,6 +959,14 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     const long Kred = (long)g.N * PQ;
     VDNN_REQUIRE(Kred < (1l << 31), "reduction too long");
     VDNN_REQUIRE((long)(PQ + KB) * PQ < (1l << 32), "output plane too large for the pixel cursor's exact division");
+    if constexpr (sizeof(E) == 4) {
+        if (algo_mode == 1) {
+            // perf-optimal: wide 3x3 layers as Winograd F(3x3, 4x4) through the workspace
+            bool taken = false;
+            const int rc = launch_winograd_wgrad(ctx, st, g, x, dy, w, alpha, accumulate, workspace, workspace_bytes, &taken, bias);
+            if (taken || rc != VDNN_OK) return rc;
+        }
+    }
     if (g.C <= 3 && g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W && g.W % 4 == 0 && g.W >= KB &&
         ctx->reduce_scratch) {
         // few input channels, rows of whole groups of four pixels: dy streamed once through the matrix cores, then the ordered split sum
@@ -828,7 +982,8 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
         splits = (Kred + kchunk - 1) / kchunk;
         const long nspan = kchunk / PQ + 2;
         if (PQ >= WSC_SLICE && nspan * g.K * PQ * (long)sizeof(E) < (long)MAX_SUM_RANGE && nspan * g.C * PQ * (long)sizeof(E) < (long)MAX_SUM_RANGE) {
-            const WgradSmallC geo{dy, x, g.N, g.K, g.H, g.W, ctx->reduce_scratch, (int)kchunk};
+            const bool with_bias = bias && bias->wanted() && bias_parts_fit(ctx, g.K, splits);
+            const WgradSmallC geo{dy, x, g.N, g.K, g.H, g.W, ctx->reduce_scratch, (int)kchunk, with_bias ? ctx->bias_scratch : nullptr, (int)splits};
             {
                 ProfScope prof(ctx, st, "conv_bwd_filter_smallc", 2.0 * (double)M * N * (double)Kred, 0.0);
                 const dim3 grid((unsigned)(mtiles * splits));
@@ -838,6 +993,11 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
                 default: hipLaunchKernelGGL((wgrad_smallc3x3_mfma_kernel<3, E>), grid, dim3(NT), 0, st, geo); break;
                 }
                 VDNN_LAUNCH_CHECK();
+            }
+            if (with_bias) {
+                const int rcb = launch_bias_grad_final(ctx, st, ctx->bias_scratch, bias->out, g.K, (int)splits, bias->alpha, bias->accumulate);
+                if (rcb != VDNN_OK) return rcb;
+                bias->done = true;
             }
             return launch_reduce_splits(ctx, st, w, ctx->reduce_scratch, (size_t)M * N, (int)splits, alpha, accumulate, nullptr, 0);
         }
@@ -951,7 +1111,7 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
         // 3x3, stride 1, padding 1: one filter row and 64 input channels per workgroup, one fetch for three taps
         if (wgrad3x3_f32_ok(g)) { // loads of four pixels take any alignment of the tensors
             bool taken = false;
-            const int rcw = launch_wgrad3x3_f32(ctx, st, g, x, dy, w, alpha, accumulate, staging, staging_bytes, &taken);
+            const int rcw = launch_wgrad3x3_f32(ctx, st, g, x, dy, w, alpha, accumulate, staging, staging_bytes, &taken, bias);
             if (taken || rcw != VDNN_OK) return rcw;
         }
     }
@@ -992,7 +1152,61 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     return VDNN_OK;
 }
 
+// Backward filter, and with `bias` the bias gradient as well: inside the filter-gradient kernel where the shape's kernel
+// can, otherwise by the kernels of vdnn_conv_bwd_bias[_sgd] behind it on the same stream.
+template <class E>
+static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                                const E* x, const E* dy, float* w, float alpha, int accumulate,
+                                void* workspace, size_t workspace_bytes, BiasOut* bias = nullptr) {
+    const int rc = conv_bwd_filter_core<E>(ctx, stream, shape, algo_mode, x, dy, w, alpha, accumulate, workspace, workspace_bytes, bias);
+    if (rc != VDNN_OK || !bias || !bias->wanted() || bias->done || ctx->plan_only) return rc;
+    return bias->accumulate ? vdnn_conv_bwd_bias_sgd(ctx, stream, shape, dy, bias->out, bias->alpha)
+                            : vdnn_conv_bwd_bias(ctx, stream, shape, dy, bias->out);
+}
+
+// Does backward filter of this shape add up the bias gradient inside its own kernel? (The shapes' dispatch above: the
+// Winograd variant, the first-layer kernel, the filter-row kernel; float activations.)
+static bool bwd_filter_sums_bias(const ConvGeo& g, int algo_mode, int dtype) {
+    if (dtype != VDNN_DTYPE_F32 || is_dense(g)) return false;
+    if (algo_mode == 1 && wino_wgrad_ok(g) && wino_wgrad_plan_ok(wino_wgrad_plan(g), g)) return true;
+    if (g.C <= 3 && g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W && g.W % 4 == 0 && g.W >= KB &&
+        g.P * g.Q >= WSC_SLICE)
+        return true;
+    return g.C > 4 && wgrad3x3_f32_ok(g);
+}
+
 extern "C" {
+
+int vdnn_conv_bwd_filter_sums_bias(const vdnn_shape_t* shape, int algo_mode, int dtype) {
+    ConvGeo g;
+    return shape && geo_from_shape(shape, g) && bwd_filter_sums_bias(g, algo_mode, dtype);
+}
+
+int vdnn_conv_bwd_filter_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                                  const void* x, const void* dy, float* w, float* bias, float alpha,
+                                  void* workspace, size_t workspace_bytes) {
+    VDNN_REQUIRE(bias != nullptr, "null bias");
+    BiasOut b; b.out = bias; b.alpha = alpha; b.accumulate = 1;
+    return VDNN_BY_ACT(ctx, conv_bwd_filter_impl<float>(ctx, stream, shape, algo_mode, (const float*)x, (const float*)dy, w, alpha, 1, workspace, workspace_bytes, &b),
+                       conv_bwd_filter_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)x, (const bf16_t*)dy, w, alpha, 1, workspace, workspace_bytes, &b));
+}
+
+int vdnn_conv_bwd_filter_bias(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                              const void* x, const void* dy, float* dw, float* db, void* workspace, size_t workspace_bytes) {
+    VDNN_REQUIRE(db != nullptr, "null bias gradient");
+    BiasOut b; b.out = db; b.alpha = 1.0f; b.accumulate = 0;
+    return VDNN_BY_ACT(ctx, conv_bwd_filter_impl<float>(ctx, stream, shape, algo_mode, (const float*)x, (const float*)dy, dw, 1.0f, 0, workspace, workspace_bytes, &b),
+                       conv_bwd_filter_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)x, (const bf16_t*)dy, dw, 1.0f, 0, workspace, workspace_bytes, &b));
+}
+
+int vdnn_conv_bwd_filter_then_bias_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,
+                                       const void* x, const void* dy, float* dw, float* bias, float alpha,
+                                       void* workspace, size_t workspace_bytes) {
+    VDNN_REQUIRE(bias != nullptr, "null bias");
+    BiasOut b; b.out = bias; b.alpha = alpha; b.accumulate = 1;
+    return VDNN_BY_ACT(ctx, conv_bwd_filter_impl<float>(ctx, stream, shape, algo_mode, (const float*)x, (const float*)dy, dw, 1.0f, 0, workspace, workspace_bytes, &b),
+                       conv_bwd_filter_impl<bf16_t>(ctx, stream, shape, algo_mode, (const bf16_t*)x, (const bf16_t*)dy, dw, 1.0f, 0, workspace, workspace_bytes, &b));
+}
 
 size_t vdnn_conv_winograd_chunk_bytes(size_t bytes) {
     const size_t before = g_wino_chunk_bytes;
@@ -1016,6 +1230,10 @@ size_t vdnn_conv_workspace_bytes_dtype(const vdnn_shape_t* shape, int algo_mode,
     if (dtype == VDNN_DTYPE_F32 && pass != 2 && wino_ok(g, pass == 1)) {
         const WinoPlan p = wino_plan(g, pass == 1);
         if (wino_plan_ok(p)) return p.total;
+    }
+    if (dtype == VDNN_DTYPE_F32 && pass == 2 && wino_wgrad_ok(g)) {
+        const WinoWgradPlan p = wino_wgrad_plan(g);
+        if (wino_wgrad_plan_ok(p, g)) return p.total;
     }
     if (pass == 0) return packed_fwd_ok(g) ? filter_bytes : 0;
     if (pass == 1) return packed_bwd_data_ok(g) ? filter_bytes : 0;

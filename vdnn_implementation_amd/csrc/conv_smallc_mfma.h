@@ -194,6 +194,10 @@ struct WgradSmallC {
     int N, K, H, W;
     float* partial; // [split][K][9*C]
     int kchunk;     // pixels per split, a multiple of WSC_SLICE
+    // optional: the bias gradient's partial sums, [K][bias_splits] (split ks of channel m at m * bias_splits + ks). The
+    // product has 32 columns of which 9*C are taken: column 9*C multiplies dy by one, so its sums are those of dy.
+    float* bias_partial;
+    int bias_splits;
 };
 constexpr int WSC_SLICE = 64;            // pixels per slice
 constexpr int WSC_STRIDE = WSC_SLICE + 4; // LDS row stride in floats: 128-bit reads of 16 consecutive rows hit 16 different bank groups
@@ -298,6 +302,7 @@ __global__ void __launch_bounds__(NT) wgrad_smallc3x3_mfma_kernel(const WgradSma
     const int rowblk = wave & 1, hf = wave >> 1; // this wavefront: 32 output channels, pixels 32*hf .. 32*hf + 31 of every slice
     // this lane's column (c, r, s): its row of x in LDS and which neighbour it takes
     const bool col_live = l32 < NCOL;
+    const float idle = (g.bias_partial != nullptr && l32 == NCOL) ? 1.0f : 0.0f; // what a lane beyond the filter's columns multiplies by
     const int bro = col_live ? l32 / 3 : 0, sB = col_live ? l32 % 3 : 1;
     int qs = k_begin % W;
 
@@ -324,10 +329,10 @@ __global__ void __launch_bounds__(NT) wgrad_smallc3x3_mfma_kernel(const WgradSma
             while (qg >= W) qg -= W;
             prev = qg == 0 ? 0.0f : prev;     // left of the image
             next = qg == W - 4 ? 0.0f : next; // right of the image
-            const float b0 = !col_live ? 0.0f : sB == 0 ? prev : sB == 1 ? v.x : v.y;
-            const float b1 = !col_live ? 0.0f : sB == 0 ? v.x : sB == 1 ? v.y : v.z;
-            const float b2 = !col_live ? 0.0f : sB == 0 ? v.y : sB == 1 ? v.z : v.w;
-            const float b3 = !col_live ? 0.0f : sB == 0 ? v.z : sB == 1 ? v.w : next;
+            const float b0 = !col_live ? idle : sB == 0 ? prev : sB == 1 ? v.x : v.y;
+            const float b1 = !col_live ? idle : sB == 0 ? v.x : sB == 1 ? v.y : v.z;
+            const float b2 = !col_live ? idle : sB == 0 ? v.y : sB == 1 ? v.z : v.w;
+            const float b3 = !col_live ? idle : sB == 0 ? v.z : sB == 1 ? v.w : next;
             acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b0, acc, 0, 0, 0);
             acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b1, acc, 0, 0, 0);
             acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b2, acc, 0, 0, 0);
@@ -356,6 +361,14 @@ __global__ void __launch_bounds__(NT) wgrad_smallc3x3_mfma_kernel(const WgradSma
             const int m = m0 + 32 * rowblk + 8 * (v / 4) + 4 * lk + (v % 4);
             if (m >= g.K) continue;
             g.partial[((long)ks * g.K + m) * NCOL + l32] = acc[v] + Red[rowblk][lane][v];
+        }
+    }
+    if (hf == 0 && g.bias_partial != nullptr && l32 == NCOL) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int m = m0 + 32 * rowblk + 8 * (v / 4) + 4 * lk + (v % 4);
+            if (m >= g.K) continue;
+            g.bias_partial[(long)m * g.bias_splits + ks] = acc[v] + Red[rowblk][lane][v];
         }
     }
 }

@@ -11,6 +11,7 @@
 #include <mutex>
 
 namespace vdnn {
+int launch_bias_grad_final(vdnn_ctx* ctx, hipStream_t st, const float* partial, float* bias, int K, int splits, float alpha, int accumulate);
 
 constexpr int EB = 256; // threads per workgroup
 
@@ -887,6 +888,14 @@ static int bias_grad_splits(int N, int K, int num_cu, int* per_out) {
     const int per = (N + splits - 1) / splits;
     *per_out = per;
     return (N + per - 1) / per;
+}
+
+// stage 2 alone, for kernels that leave the bias gradient's partial sums themselves (partial[k * splits + i])
+int vdnn::launch_bias_grad_final(vdnn_ctx* ctx, hipStream_t st, const float* partial, float* bias, int K, int splits, float alpha, int accumulate) {
+    ProfScope prof(ctx, st, "conv_bwd_bias_final", 0.0, 4.0 * (double)K * (splits + 2));
+    hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB - 1) / EB), dim3(EB), 0, st, partial, bias, K, splits, alpha, accumulate);
+    VDNN_LAUNCH_CHECK();
+    return VDNN_OK;
 }
 
 template <class E>

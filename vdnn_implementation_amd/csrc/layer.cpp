@@ -280,6 +280,12 @@ void Layer::biasGradientBeside(DATATYPE lr) {
     checkVDNN(vdnn_event_record(ctx, evBiasJoin, beside));
 }
 
+/* Whether this layer's backward filter adds up the bias gradient itself (a property of the shape, the algorithm mode and
+ * the element type: the same answer under every policy, so the same sums). */
+bool Layer::biasGradientInFilterKernel() const {
+    return biasData != nullptr && vdnn_conv_bwd_filter_sums_bias(&shape, vdnnAlgoMode, vdnn_ctx_activation_dtype(ctx)) != 0;
+}
+
 void Layer::joinBiasGradient() {
     checkVDNN(vdnn_stream_wait_event(ctx, *stream_compute, evBiasJoin));
 }
@@ -318,20 +324,30 @@ int Layer::convolutionBackwardOverSrc(int _layer_id_to_prefetch, DATATYPE* _pref
     gradData = srcData;
     if (_layer_id_to_prefetch >= 0) prefetchPreviousSrcData(_prefetchedSrcData_h, _srcDataToPrefetch, _prefetch_bytes);
 
-    biasGradientBeside(lr);
+    /* the bias gradient: inside the filter-gradient kernel where that kernel sums the dy it streams, else beside it */
+    const bool biasInFilter = biasGradientInFilterKernel();
+    auto joinBias = [&]() { if (!biasInFilter) joinBiasGradient(); };
+    if (!biasInFilter) biasGradientBeside(lr);
 
     void* dw = filterGrad;
-    if (!dw && ASSERT_EQ(vdnn_pool_malloc(ctx, &dw, sizeof(DATATYPE) * (size_t)k * c_in * r * s), isDynamic) < 0) { joinBiasGradient(); return -1; }
+    if (!dw && ASSERT_EQ(vdnn_pool_malloc(ctx, &dw, sizeof(DATATYPE) * (size_t)k * c_in * r * s), isDynamic) < 0) { joinBias(); return -1; }
     /* a trial of the dynamic mode that runs out of memory gives up here: the caller recycles the output gradient's
      * block next, so the bias gradient's stream is joined on these paths too */
     auto releaseDw = [&]() { if (!filterGrad) ASSERT_EQ(vdnn_pool_free(ctx, dw), isDynamic); };
-    if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { releaseDw(); joinBiasGradient(); return -1; }
+    if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { releaseDw(); joinBias(); return -1; }
     waitSrcFetched();
-    checkVDNN(vdnn_conv_bwd_filter(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
-                                   (float*)dw, curWorkSpace, bwdFilterWorkSpaceSize));
+    if (biasInFilter && filterGrad)
+        checkVDNN(vdnn_conv_bwd_filter_bias(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
+                                            (float*)dw, (float*)biasGrad, curWorkSpace, bwdFilterWorkSpaceSize));
+    else if (biasInFilter)
+        checkVDNN(vdnn_conv_bwd_filter_then_bias_sgd(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
+                                                     (float*)dw, (float*)biasData, lr, curWorkSpace, bwdFilterWorkSpaceSize));
+    else
+        checkVDNN(vdnn_conv_bwd_filter(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
+                                       (float*)dw, curWorkSpace, bwdFilterWorkSpaceSize));
     freeWorkSpace(workSpace, bwdFilterWorkSpaceSize, curWorkSpace, isDynamic);
 
-    if (mallocWorkSpace(workSpace, bwdDataWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { releaseDw(); joinBiasGradient(); return -1; }
+    if (mallocWorkSpace(workSpace, bwdDataWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { releaseDw(); joinBias(); return -1; }
     if (gateGrad)
         checkVDNN(vdnn_conv_bwd_data_relu(ctx, *stream_compute, &shape, vdnnAlgoMode, diffData, (const float*)filterData,
                                           srcData, gradData, curWorkSpace, bwdDataWorkSpaceSize));
@@ -344,7 +360,7 @@ int Layer::convolutionBackwardOverSrc(int _layer_id_to_prefetch, DATATYPE* _pref
         checkVDNN(vdnn_sgd_apply(ctx, *stream_compute, (size_t)k * c_in * r * s, lr, (const float*)dw, (float*)filterData));
         releaseDw();
     }
-    joinBiasGradient();
+    joinBias();
     return 0;
 }
 
@@ -374,21 +390,29 @@ int Layer::convolutionBackward(int _layer_id_to_prefetch, DATATYPE* _prefetchedS
                                      (float*)gradData, curWorkSpace, bwdDataWorkSpaceSize));
     freeWorkSpace(workSpace, bwdDataWorkSpaceSize, curWorkSpace, isDynamic);
 
-    /* Backward Bias Propagation: the learning rate is folded into the update */
-    biasGradientBeside(lr);
+    /* Backward Bias Propagation (layer.cu:631-637), the learning rate folded into the update: summed inside the
+     * filter-gradient kernel below where that kernel can (it streams the same dy), else by a kernel of its own beside it */
+    const bool biasInFilter = biasGradientInFilterKernel();
+    if (!biasInFilter) biasGradientBeside(lr);
 
     /* a trial of the dynamic mode that runs out of memory gives up here: the caller recycles the output gradient's
      * block next, so the bias gradient's stream is joined first */
-    if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { joinBiasGradient(); return -1; }
+    if (mallocWorkSpace(workSpace, bwdFilterWorkSpaceSize, &curWorkSpace, isDynamic) < 0) { if (!biasInFilter) joinBiasGradient(); return -1; }
     waitSrcFetched();
-    if (filterGrad)
+    if (filterGrad && biasInFilter)
+        checkVDNN(vdnn_conv_bwd_filter_bias(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
+                                            (float*)filterGrad, (float*)biasGrad, curWorkSpace, bwdFilterWorkSpaceSize));
+    else if (filterGrad)
         checkVDNN(vdnn_conv_bwd_filter(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
                                        (float*)filterGrad, curWorkSpace, bwdFilterWorkSpaceSize));
+    else if (biasInFilter)
+        checkVDNN(vdnn_conv_bwd_filter_bias_sgd(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
+                                                (float*)filterData, (float*)biasData, lr, curWorkSpace, bwdFilterWorkSpaceSize));
     else
         checkVDNN(vdnn_conv_bwd_filter_sgd(ctx, *stream_compute, &shape, vdnnAlgoMode, (const float*)srcData, (const float*)diffData,
                                            (float*)filterData, lr, curWorkSpace, bwdFilterWorkSpaceSize));
     freeWorkSpace(workSpace, bwdFilterWorkSpaceSize, curWorkSpace, isDynamic);
-    joinBiasGradient();
+    if (!biasInFilter) joinBiasGradient();
     return 0;
 }
 

@@ -20,6 +20,8 @@
 #pragma once
 #include "mfma_gemm.h"
 
+#include <type_traits>
+
 namespace vdnn {
 
 constexpr int WG3F_CH = 64; // input channels of a workgroup's tile
@@ -33,6 +35,10 @@ struct Wgrad3x3F {
     long partial_stride; // K*9*C
     float alpha;
     int accumulate;
+    // optional: the bias gradient's partial sums, [K][bias_splits] (split ks of channel m at m * bias_splits + ks). The
+    // workgroups of the centre filter row and the first block of input channels add up the dy values they multiply.
+    float* bias_partial;
+    int bias_splits;
 };
 
 // d.M = K, d.N = 9*C, d.K = N*H*W; d.mtiles tiles of 2*WR output channels, d.ntiles = 3 * C/64 (filter row
@@ -170,7 +176,17 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_f32_kernel(const Wgrad3x3F g, 
         f.next = qg == W - 4 ? 0.0f : next; // right of the image
         f.mid = HALFROW && qg == W - 2;     // pixels 2.. of the four begin an image row
     };
-    auto multiply = [&](const Frag& f) {
+    // The workgroups that also sum dy run a copy of the loop of their own (chosen once, before the loop), so that the
+    // loop of all others stays one basic block. Wavefronts 0 and 1 (input channels 0-31) cover the tile's rows of dy.
+    const bool sums_bias = g.bias_partial != nullptr && nt == 1 && wave < 2;
+    float bsum[RB];
+#pragma unroll
+    for (int i = 0; i < RB; i++) bsum[i] = 0.0f;
+    auto multiply = [&](const Frag& f, auto with_bias) {
+        if constexpr (decltype(with_bias)::value) {
+#pragma unroll
+            for (int i = 0; i < RB; i++) bsum[i] += (f.a[i][0] + f.a[i][1]) + (f.a[i][2] + f.a[i][3]);
+        }
         // pixel 2 reads left of the image through the left tap, pixel 1 right of it through the right tap, where a row begins inside
         const float up[4] = {f.prev, f.v.x, (HALFROW && f.mid) ? 0.0f : f.v.y, f.v.z};
         const float ce[4] = {f.v.x, f.v.y, f.v.z, f.v.w};
@@ -194,25 +210,39 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_f32_kernel(const Wgrad3x3F g, 
     __syncthreads();
     Frag f0, f1;
     read(0, 0, qs, f0);
-    for (int s = 0; s < nslices; s++) {
-        const int cur = s & 1, nxt = cur ^ 1;
-        read(cur, 1, qs, f1);
-        multiply(f0);
-        stash(nxt);
+    auto run = [&](auto with_bias) {
+        for (int s = 0; s < nslices; s++) {
+            const int cur = s & 1, nxt = cur ^ 1;
+            read(cur, 1, qs, f1);
+            multiply(f0, with_bias);
+            stash(nxt);
 #pragma unroll
-        for (int i = 0; i < 12 * RB; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x300, 1, 0); }
-        __syncthreads();
-        fetch();
-        qs += KB;
-        qs -= qs >= W ? W : 0;
-        if (HALFROW) qs -= qs >= W ? W : 0;
-        read(nxt, 0, qs, f0);
-        multiply(f1);
+            for (int i = 0; i < 12 * RB; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x300, 1, 0); }
+            __syncthreads();
+            fetch();
+            qs += KB;
+            qs -= qs >= W ? W : 0;
+            if (HALFROW) qs -= qs >= W ? W : 0;
+            read(nxt, 0, qs, f0);
+            multiply(f1, with_bias);
 #pragma unroll
-        for (int i = 0; i < 12 * RB; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            for (int i = 0; i < 12 * RB; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+        }
+    };
+    if (sums_bias) run(std::true_type{});
+    else run(std::false_type{});
+
+    if (sums_bias) {
+        // a lane summed pixels 4 lk .. 4 lk + 3 of every group of eight of its row: the two halves of the wavefront together
+#pragma unroll
+        for (int i = 0; i < RB; i++) {
+            const float whole = bsum[i] + __shfl_xor(bsum[i], 32);
+            const int m = m0 + wm0 + 32 * i + l32;
+            if (lk == 0 && m < g.K) g.bias_partial[(long)m * g.bias_splits + ks] = whole;
         }
     }
 

@@ -99,7 +99,13 @@ struct WinoTiles {
 template <bool VEC>
 __global__ void __launch_bounds__(256) wino_input_kernel(const float* __restrict__ src, float* __restrict__ V, const WinoTiles g) {
     const int t = blockIdx.x * 256 + threadIdx.x, c = blockIdx.y;
-    if (t >= g.T) return;
+    if (t >= g.Tpad) return;
+    if (t >= g.T) { // the columns that round the chunk up to whole tiles of the product: zero, so that sums over them add nothing
+        float* pad = V + (long)c * WINO_XI * g.Tpad + t;
+#pragma unroll
+        for (int xi = 0; xi < WINO_XI; xi++) pad[(long)xi * g.Tpad] = 0.0f;
+        return;
+    }
     const int per = g.th * g.tw;
     const int n = t / per, rem = t - n * per;
     const int ty = rem / g.tw, tx = rem - ty * g.tw;
@@ -253,5 +259,181 @@ struct LoadDenseRowVec4 {
         for (int i = 0; i < T * KB / (4 * NT); i++) *(floatx4*)(lds + (tid / (T / 4) + PER * i) * T + 4 * (tid % (T / 4))) = r.v[i];
     }
 };
+
+// ---- backward filter: F(3x3, 4x4) --------------------------------------------------------------------------------
+// The filter gradient of one 4x4 tile of output pixels is the 3x3 "output" of correlating the 6x6 input patch with the
+// 4x4 tile of dy as a "filter": dW = A't [ sum over tiles and samples of (G' dy G't) .* (Bt x B) ] A' with the same
+// six interpolation points (0, 1, -1, 2, -2, infinity), hence the same Bt (and the same transformed input V as the
+// forward pass), G' = the 6x4 and A't the 3x6 matrices of those points. The sum over tiles, for each of the 36
+// positions, is a matrix product S_xi[k][c] = sum_t D_xi[k][t] V_xi[c][t] with a long reduction (all tiles of the
+// batch): split along t, partial sums added in split order, then transformed back and applied to the filter.
+__device__ __forceinline__ void wino_g6x4(const float (&g)[4], float (&u)[6]) {
+    const float e = g[0] + g[2], o = g[1] + g[3];
+    u[0] = g[0] * 0.25f;
+    u[1] = -(e + o) * (1.0f / 6.0f);
+    u[2] = (o - e) * (1.0f / 6.0f);
+    const float a = g[0] * (1.0f / 24.0f) + g[2] * (1.0f / 6.0f), b = g[1] * (1.0f / 12.0f) + g[3] * (1.0f / 3.0f);
+    u[3] = a + b;
+    u[4] = a - b;
+    u[5] = g[3];
+}
+__device__ __forceinline__ void wino_at3(const float (&m)[6], float (&o)[3]) {
+    const float s12 = m[1] + m[2], d12 = m[1] - m[2], s34 = m[3] + m[4], d34 = m[3] - m[4];
+    o[0] = m[0] + s12 + s34;
+    o[1] = d12 + 2.0f * d34;
+    o[2] = s12 + 4.0f * s34 + m[5];
+}
+
+// D[(k * 36 + xi) * Tpad + t] = (G' dy_tile G't)[xi]; pixels of the tile outside the plane count as zero; columns
+// t >= T are zero. One thread per (k, t), lanes along t. BIAS: the workgroup also adds up the dy values it read - the
+// bias gradient's share of its 256 tiles - in a fixed order (lanes by halving, then the four wavefronts in turn) and
+// leaves the sum at bias_partial[k * bias_parts + bias_first + blockIdx.x].
+template <bool VEC, bool BIAS>
+__global__ void __launch_bounds__(256) wino_dy_kernel(const float* __restrict__ src, float* __restrict__ D, const WinoTiles g,
+                                                      float* __restrict__ bias_partial, int bias_parts, int bias_first) {
+    __shared__ float wave_sums[4];
+    const int t = blockIdx.x * 256 + threadIdx.x, k = blockIdx.y;
+    float mine = 0.0f;
+    if (t < g.Tpad) {
+        float* out = D + (long)k * WINO_XI * g.Tpad + t;
+        if (t >= g.T) {
+#pragma unroll
+            for (int xi = 0; xi < WINO_XI; xi++) out[(long)xi * g.Tpad] = 0.0f;
+        } else {
+            const int per = g.th * g.tw;
+            const int n = t / per, rem = t - n * per;
+            const int ty = rem / g.tw, tx = rem - ty * g.tw;
+            const float* plane = src + ((long)n * g.chan + k) * g.H * g.W;
+            float d[4][4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = 4 * ty + i;
+                const bool rok = row < g.H;
+                const float* p = plane + (long)row * g.W + 4 * tx;
+                if (VEC) {
+                    floatx4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+                    if (rok) v = *(const floatx4*)p;
+                    d[i][0] = v.x; d[i][1] = v.y; d[i][2] = v.z; d[i][3] = v.w;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) d[i][j] = (rok && 4 * tx + j < g.W) ? p[j] : 0.0f;
+                }
+                if (BIAS) mine += (d[i][0] + d[i][1]) + (d[i][2] + d[i][3]);
+            }
+            float h[6][4]; // G' d
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float col[4] = {d[0][j], d[1][j], d[2][j], d[3][j]};
+                float u[6];
+                wino_g6x4(col, u);
+#pragma unroll
+                for (int i = 0; i < 6; i++) h[i][j] = u[i];
+            }
+#pragma unroll
+            for (int i = 0; i < 6; i++) {
+                float u[6];
+                wino_g6x4(h[i], u);
+#pragma unroll
+                for (int j = 0; j < 6; j++) out[(long)(i * 6 + j) * g.Tpad] = u[j];
+            }
+        }
+    }
+    if (BIAS) {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) mine += __shfl_xor(mine, off);
+        if ((threadIdx.x & 63) == 0) wave_sums[threadIdx.x >> 6] = mine;
+        __syncthreads();
+        if (threadIdx.x == 0)
+            bias_partial[(long)k * bias_parts + bias_first + blockIdx.x] = ((wave_sums[0] + wave_sums[1]) + wave_sums[2]) + wave_sums[3];
+    }
+}
+
+// An operand of the backward-filter product: rows (output channels of D, input channels of V) by tiles, reduction-major,
+// element (row, kk) of position xi at base[(row * 36 + xi) * Tpad + kk]. The product's columns are j = xi * cpad + c.
+// BY_COLUMN_TILE (the A operand, D): xi comes from the workgroup's column tile, decoded the way igemm_kernel does;
+// otherwise (the B operand, V) from the tile's first column, which init is handed.
+template <bool BY_COLUMN_TILE>
+struct LoadWinoRed {
+    static constexpr bool RED_MAJOR = true;
+    const float* base;
+    long tpad;        // reduction extent per (row, xi); rows are 36 * tpad apart
+    int rows;         // valid rows of the tensor
+    unsigned bytes;   // extent of the tensor in bytes (below 2 GiB)
+    int cpad;         // columns per xi
+    int mtiles, ntiles_all, tn;
+    template <int T> struct Regs { floatx4 v[T / 64]; };
+    template <int T> struct State { int vrow[T / 64]; __amdgpu_buffer_rsrc_t rsrc; };
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int row0, int tid, int, int) const {
+        int xi, first;
+        if (BY_COLUMN_TILE) {
+            const int bid = xcd_remap(blockIdx.x, gridDim.x);
+            const int nt = (bid % ntiles_all) / mtiles;
+            xi = nt * tn / cpad; first = row0;
+        } else {
+            xi = row0 / cpad; first = row0 - xi * cpad;
+        }
+        st.rsrc = make_rsrc(base + (long)xi * tpad, bytes - (unsigned)(xi * tpad * 4));
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) {
+            const int row = first + (tid >> 2) + 64 * i;
+            st.vrow[i] = row < rows ? (int)(((long)row * WINO_XI * tpad + 4 * (tid & 3)) * 4) : OOB;
+        }
+    }
+    // the reduction is a whole number of slices; a fetch past a split's end reads the next split's values or zeros and is never used
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int kk0, int, int, Regs<T>& r) const {
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) r.v[i] = buf_load4(st.rsrc, st.vrow[i], kk0 * 4);
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(float* lds, int tid, const Regs<T>& r) {
+#pragma unroll
+        for (int i = 0; i < T / 64; i++) *(floatx4*)(lds + ((tid >> 2) + 64 * i) * RED_STRIDE + 4 * (tid & 3)) = r.v[i];
+    }
+};
+
+// partial[0][i] = sum over p, in order, of partial[p][i]: the partial results of all chunks and splits, one thread per
+// element (each thread reads its own element of the first result before it overwrites it).
+__global__ void __launch_bounds__(256) wino_wgrad_sum_kernel(float* partial, long part_stride, int nparts, long count) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    float sum = 0.0f;
+    for (int p = 0; p < nparts; p++) sum += partial[(long)p * part_stride + i];
+    partial[i] = sum;
+}
+
+// w[k][c][r][s] = (accumulate ? w : 0) + alpha * (A't S A')[r][s], S[xi] = sum over the partial results, in their order,
+// of partial[p][k][xi * cpad + c]. One thread per (k, c), lanes along c.
+__global__ void __launch_bounds__(256) wino_wgrad_out_kernel(const float* __restrict__ partial, long part_stride, int nparts, float* w, int K, int C, int cpad,
+                                                             float alpha, int accumulate) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (long)K * C) return;
+    const int k = (int)(i / C), c = (int)(i - (long)k * C);
+    const float* in = partial + (long)k * WINO_XI * cpad + c;
+    float a[3][6]; // A't S
+#pragma unroll
+    for (int y = 0; y < 6; y++) {
+        float col[6];
+#pragma unroll
+        for (int x = 0; x < 6; x++) {
+            float sum = 0.0f;
+            for (int p = 0; p < nparts; p++) sum += in[(long)p * part_stride + (long)(x * 6 + y) * cpad];
+            col[x] = sum;
+        }
+        float o[3];
+        wino_at3(col, o);
+#pragma unroll
+        for (int r = 0; r < 3; r++) a[r][y] = o[r];
+    }
+    float* out = w + i * 9;
+#pragma unroll
+    for (int r = 0; r < 3; r++) {
+        float o[3];
+        wino_at3(a[r], o);
+#pragma unroll
+        for (int s2 = 0; s2 < 3; s2++) out[r * 3 + s2] = accumulate ? __fmaf_rn(alpha, o[s2], out[r * 3 + s2]) : alpha * o[s2];
+    }
+}
 
 } // namespace vdnn
