@@ -293,7 +293,8 @@ def main():
         word, *mods = name.split("+")
         budget = [float(m[6:]) for m in mods if m.startswith("budget")]
         lag_given = [int(m[3:]) for m in mods if m.startswith("lag")]
-        mods = [m for m in mods if not m.startswith("budget") and not m.startswith("lag")]
+        link_first = [float(m[4:]) for m in mods if m.startswith("link")]   # "+linkX": X GB each way go over the link before anything is packed on the device
+        mods = [m for m in mods if not m.startswith("budget") and not m.startswith("lag") and not m.startswith("link")]
         assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep", "inplace", "recompute", "perf"}, name
         # "+perf": VDNN_PERF_OPT_ALGO, the workspace-using kernel variants (wide 3x3 layers as Winograd F(4x4, 3x3)): other
         # sums than the memory-optimal kernels', so its loss is compared within the mode only
@@ -310,6 +311,8 @@ def main():
                   keep_tail_bytes=int(0.75e9) * (2 if bf16 else 4) if "tail" in mods else int(args.keep_tail_gb * 1e9))
         if budget:
             kw.update(hbm_budget_bytes=int(baseline_peak / budget[0]), plan_packed_fraction=PACKED_FRACTION[bf16])
+            if link_first:
+                kw.update(plan_link_bytes=int(link_first[0] * 1e9))
         log("[bench] %s %s batch %d: %d warm-up + %d timed + %d profiled steps" % (name, args.algo, args.batch, args.warmup, args.steps, args.profile_steps))
         results[name], profiles[name] = run_config(Network, be, cnn, policy, algo, args.batch, args.steps, args.warmup, args.profile_steps, **kw)
         r = results[name]

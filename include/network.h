@@ -87,6 +87,14 @@ struct NetworkOptions {
     // the last plan stands and Network::planFeasible() says so. The replay has no data: planPackedFraction is what it
     // takes a packed stream to be of its tensor. 0: no budget, the policy's own offload set.
     size_t   hbmBudgetBytes = 0;
+    // With hbmBudgetBytes: how many bytes per step and direction the plan may send over the host link BEFORE it packs
+    // anything on the device. The planner's own order is the other way round (a stream on the device costs two passes
+    // at HBM speed, the link a hundred times that), which leaves the link idle until the budget forces a tensor out. A
+    // step whose kernels take T seconds can hide about T x 56 GB/s each way if the copies are spread well: with this
+    // many bytes allowed, the members that must leave the device go over the link first (the largest gain first, a
+    // rectified tensor as its packed stream, counted at planPackedFraction of its size), and are packed on the device
+    // only once the allowance is used up. 0: pack first (the planner's own order).
+    size_t   planLinkBytes = 0;
     // Backward writes a layer's input gradient over the layer's own input where nothing reads that input again: a
     // convolution (stride 1, more than four input channels) computes its filter gradient first, into a block of the
     // filter's size, then the data gradient - still with the old filter, as layer.cu:616-660 has it - over its

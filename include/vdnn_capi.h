@@ -39,6 +39,7 @@ typedef struct {
     size_t   hbm_budget_bytes;  /* a limit on pool bytes in use that the policy meets by choosing, per member of its offload set (network.cu:898-936), between the device, a packed stream on the device and host memory (0 = the policy's own set) */
     int      in_place_backward; /* a layer's input gradient is written over its input where nothing reads that again (layer.cu:599 allocates it beside x and dy); needs refined_lifetimes */
     int      recompute_first_layer; /* the output of a first convolution over at most four channels is computed again before its consumer's backward instead of kept or offloaded (network.cu:916-936 keeps or moves it); needs refined_lifetimes */
+    size_t   plan_link_bytes;   /* with hbm_budget_bytes: bytes per step and direction that the plan sends over the link before it packs anything on the device (0 = pack first) */
 } vdnn_network_options;
 
 typedef struct {

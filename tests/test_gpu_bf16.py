@@ -179,6 +179,42 @@ def test_conv_bf16(ctx, geom, algo):
         assert_close(gb.download(b.shape), oracle.conv_bwd_bias_sgd(og, dy, np.zeros_like(b), 1.0), 1e-4, "bwd bias")
 
 
+@pytest.mark.parametrize("geom,inside", [
+    ((7, 3, 40, 36, 16, 3, 3, 1, 1, 1, 1), True),      # first-layer kernel: the product's spare column multiplies dy by one
+    ((2, 64, 4, 32, 64, 3, 3, 1, 1, 1, 1), True),      # filter-row kernel, one split
+    ((7, 128, 6, 32, 192, 3, 3, 1, 1, 1, 1), True),    # two channel blocks, a ragged second row tile, several splits
+    ((3, 64, 6, 28, 96, 3, 3, 1, 1, 1, 1), True),      # the variant with groups across image rows
+    ((9, 256, 14, 14, 64, 3, 3, 1, 1, 1, 1), False),   # 14 x 14: the tile engine; the bias kernels run behind it
+], ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v))
+def test_conv_bwd_filter_with_the_bias_gradient_bf16(ctx, geom, inside):
+    """vdnn_conv_bwd_filter_bias_sgd / _bias with bfloat16 activations (layer.cu:631-660 in one call): the filter with
+    the bits of the separate call, the bias gradient within the float tolerance, twice the same bits."""
+    rng = np.random.default_rng(hash(geom) % (2 ** 31) + 13)
+    g, og = be.shape(*geom), oracle.shape(*geom)
+    assert bool(lib.vdnn_conv_bwd_filter_sums_bias(g, 0, BF16)) == inside
+    x = rnd(rng, (g.n, g.c, g.h, g.w))
+    w = (rng.standard_normal((g.k, g.c, g.r, g.s)) * np.sqrt(2.0 / (g.c * g.r * g.s))).astype(np.float32)
+    b = rng.standard_normal(g.k).astype(np.float32)
+    dy = oracle.round_bf16((rng.standard_normal((g.n, g.k, g.h, g.w)) + 0.25).astype(np.float32))
+    alpha = np.float32(-0.37)
+    announce("bwd filter + bias bf16", geom)
+    with Dev(ctx) as d:
+        dx_, ddy, dw, db = d.act(x), d.act(dy), d.f32(w), d.f32(b)
+        check(lib.vdnn_conv_bwd_filter_bias_sgd(ctx.handle, None, g, 0, dx_.ptr, ddy.ptr, dw.ptr, db.ptr, alpha, None, 0))
+        got_w, got_b = dw.download(w.shape), db.download(b.shape)
+        assert_close(got_w, oracle.conv_bwd_filter_sgd(og, x, dy, w, alpha), 1e-4, "filter")
+        assert_close(got_b, oracle.conv_bwd_bias_sgd(og, dy, b, alpha), 1e-4, "bias")
+        dw2 = d.f32(w)
+        check(lib.vdnn_conv_bwd_filter_sgd(ctx.handle, None, g, 0, dx_.ptr, ddy.ptr, dw2.ptr, alpha, None, 0))
+        assert np.array_equal(dw2.download(w.shape), got_w)
+        gw, gb = d.f32(np.full_like(w, 7.0)), d.f32(np.full_like(b, 7.0))
+        check(lib.vdnn_conv_bwd_filter_bias(ctx.handle, None, g, 0, dx_.ptr, ddy.ptr, gw.ptr, gb.ptr, None, 0))
+        got_db = gb.download(b.shape)
+        assert_close(got_db, oracle.conv_bwd_bias_sgd(og, dy, np.zeros_like(b), 1.0), 1e-4, "db")
+        check(lib.vdnn_conv_bwd_filter_bias(ctx.handle, None, g, 0, dx_.ptr, ddy.ptr, gw.ptr, gb.ptr, None, 0))
+        assert np.array_equal(gb.download(b.shape), got_db)
+
+
 @pytest.mark.parametrize("geom", drawn_geometries(6, 16), ids=lambda g: "x".join(map(str, g)))
 @pytest.mark.parametrize("algo", [0, 1])
 def test_conv_bf16_drawn_geometries(ctx, geom, algo):

@@ -371,6 +371,31 @@ def test_prefetch_depth_counts_packed_streams_on_their_way_back():
         assert traces[True, depth] == traces[False, depth]
 
 
+def test_plan_link_bytes_sends_tensors_over_the_link_before_packing_any():
+    """planLinkBytes is an allowance of bytes per step and direction that a budget's plan spends on the link first: the
+    members that must leave go over the link while their (packed) bytes fit it, and only then wait packed on the
+    device. Same budget, same feasibility; fewer tensors packed; the bytes planned for the link within the allowance."""
+    with plan(VGG16_128, BASELINE, batch=256) as r:
+        step(r)
+        base = r.stats()["peak_bytes_in_use"]
+    kw = dict(refined=True, fuse=True, compress=True, in_place=True, recompute_first=True, offload_lag=-1, prefetch_within_peak=True,
+              plan_packed_fraction=0.6, hbm_budget_bytes=int(base / 4.4))
+    seen = {}
+    for allowance in (0, int(2.5e9), int(3.5e9)):
+        with plan(VGG16_128, VDNN_ALL, batch=256, plan_link_bytes=allowance, **kw) as net:
+            step(net)
+            step(net)
+            places = net.placement()
+            over = [l for l, p in enumerate(places) if p == 3]
+            planned = sum(0.6 * 4 * net.specs[l].n * net.specs[l].c * net.specs[l].h * net.specs[l].w for l in over)
+            assert net.plan_feasible() and net.stats()["peak_bytes_in_use"] <= kw["hbm_budget_bytes"]
+            seen[allowance] = (over, places.count(2))
+            if allowance:
+                assert planned <= allowance
+    assert seen[0][0] == [4] and seen[int(2.5e9)][0] == [4, 5] and seen[int(3.5e9)][0] == [4, 7]
+    assert seen[0][1] > seen[int(2.5e9)][1] > seen[int(3.5e9)][1] == 0
+
+
 def test_unfused_optimizer_costs_one_more_copy_of_the_parameters():
     for policy in (BASELINE, VDNN_ALL):
         with plan(VGG16_128, policy) as net:

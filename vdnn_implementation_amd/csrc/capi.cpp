@@ -29,6 +29,7 @@ static NetworkOptions to_options(const vdnn_network_options* o) {
     n.hbmBudgetBytes = o->hbm_budget_bytes;
     n.inPlaceBackward = o->in_place_backward != 0;
     n.recomputeFirstLayer = o->recompute_first_layer != 0;
+    n.planLinkBytes = o->plan_link_bytes;
     return n;
 }
 
@@ -54,6 +55,7 @@ void vdnn_network_default_options(vdnn_network_options* o) {
     o->hbm_budget_bytes = d.hbmBudgetBytes;
     o->in_place_backward = d.inPlaceBackward;
     o->recompute_first_layer = d.recomputeFirstLayer;
+    o->plan_link_bytes = d.planLinkBytes;
 }
 
 vdnn_network* vdnn_network_create(int cnn, int policy, int algo, int batch, const vdnn_network_options* o) {

@@ -206,23 +206,6 @@ static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 int launch_reduce_splits(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count,
                          int splits, float alpha, int accumulate, const float* bias_j, int ncols, int relu = 0, const float* gate = nullptr);
-int launch_bias_grad_final(vdnn_ctx* ctx, hipStream_t st, const float* partial, float* bias, int K, int splits, float alpha, int accumulate);
-
-// The bias gradient as a by-product of backward filter (cudnnConvolutionBackwardBias, layer.cu:631-637, reads the same dy
-// as cudnnConvolutionBackwardFilter, :651-660): where the filter-gradient kernel of a shape can add up the dy values it
-// streams, it leaves per-channel partial sums in the context's bias staging area and `done` is set; the caller runs the
-// ordered final sum. out = (accumulate ? out : 0) + alpha * sum over n, p, q of dy.
-struct BiasOut {
-    float* out = nullptr;
-    float alpha = 1.0f;
-    int accumulate = 0;
-    bool done = false;
-    bool wanted() const { return out != nullptr; }
-};
-// room for K x parts partial sums in the bias staging area?
-static bool bias_parts_fit(const vdnn_ctx* ctx, int K, long parts) {
-    return ctx->bias_scratch && parts > 0 && (size_t)K * (size_t)parts * sizeof(float) <= ctx->bias_scratch_bytes;
-}
 
 // forward with the given A loader (128-bit or 32-bit filter loads)
 template <class AL, class E>
@@ -257,6 +240,24 @@ static bool is_dense(const ConvGeo& g) { return g.P == 1 && g.Q == 1 && g.ph == 
 static bool packed_fwd_ok(const ConvGeo& g) { return g.R * g.S <= 32 && g.C % KB == 0; }
 static bool packed_bwd_data_ok(const ConvGeo& g) {
     return g.C > 4 && g.sh == 1 && g.sw == 1 && g.R * g.S <= 32 && g.K % KB == 0;
+}
+
+int launch_bias_grad_final(vdnn_ctx* ctx, hipStream_t st, const float* partial, float* bias, int K, int splits, float alpha, int accumulate);
+
+// The bias gradient as a by-product of backward filter (cudnnConvolutionBackwardBias, layer.cu:631-637, reads the same dy
+// as cudnnConvolutionBackwardFilter, :651-660): where the filter-gradient kernel of a shape can add up the dy values it
+// streams, it leaves per-channel partial sums in the context's bias staging area and `done` is set; the caller runs the
+// ordered final sum. out = (accumulate ? out : 0) + alpha * sum over n, p, q of dy.
+struct BiasOut {
+    float* out = nullptr;
+    float alpha = 1.0f;
+    int accumulate = 0;
+    bool done = false;
+    bool wanted() const { return out != nullptr; }
+};
+// room for K x parts partial sums in the bias staging area?
+static bool bias_parts_fit(const vdnn_ctx* ctx, int K, long parts) {
+    return ctx->bias_scratch && parts > 0 && (size_t)K * (size_t)parts * sizeof(float) <= ctx->bias_scratch_bytes;
 }
 
 // ---- Winograd F(4x4, 3x3): the perf-optimal mode's forward / backward data of wide 3x3 layers (winograd_f32.h) -----
@@ -569,6 +570,7 @@ static int launch_pack_filter(vdnn_ctx* ctx, hipStream_t st, const float* w, flo
 // Workgroups of wgrad3x3_bf16_kernel that are resident on a compute unit (its launch bounds).
 constexpr int kWgrad3PerCU = 2;
 
+
 static bool wgrad3x3_ok(const ConvGeo& g) {
     return g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W &&
            g.W % 4 == 0 && g.W >= 16 && (g.H * g.W) % 8 == 0 && g.C % WG3_CH == 0; // a slice wraps at most two image rows
@@ -577,7 +579,7 @@ static bool wgrad3x3_ok(const ConvGeo& g) {
 // One filter row, 64 input channels and 128 (64) output channels per workgroup; the pixel reduction is split so
 // that one round of workgroups fills the chip, as far as the staging area holds the partial sums.
 static int launch_wgrad3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const bf16_t* x, const bf16_t* dy, float* w, float alpha, int accumulate,
-                           float* staging, size_t staging_bytes, bool* taken) {
+                           float* staging, size_t staging_bytes, bool* taken, BiasOut* bias) {
     *taken = false;
     const int M = g.K, N = g.C * 9, PQ = g.H * g.W;
     const long Kred = (long)g.N * PQ;
@@ -600,7 +602,8 @@ static int launch_wgrad3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, cons
     const long blocks = tiles * d.splits;
     if (blocks <= 0 || blocks >= (1l << 31)) return VDNN_OK;
     *taken = true;
-    const Wgrad3x3 geo{dy, x, g.N, g.K, g.C, g.H, g.W, w, staging, (long)M * N, alpha, accumulate};
+    const bool with_bias = bias && bias->wanted() && bias_parts_fit(ctx, g.K, d.splits);
+    const Wgrad3x3 geo{dy, x, g.N, g.K, g.C, g.H, g.W, w, staging, (long)M * N, alpha, accumulate, with_bias ? ctx->bias_scratch : nullptr, d.splits};
     {
         ProfScope prof(ctx, st, narrow ? kBwdFilterWin3Names.t64 : kBwdFilterWin3Names.t128, 2.0 * M * (double)N * (double)Kred, 0.0);
         const bool halfrow = g.W % 8 != 0 || g.W < KH; // the general variant: groups across two image rows, two row wraps per slice
@@ -609,6 +612,11 @@ static int launch_wgrad3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, cons
         else if (halfrow) hipLaunchKernelGGL((wgrad3x3_bf16_kernel<64, true>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
         else hipLaunchKernelGGL((wgrad3x3_bf16_kernel<64, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
         VDNN_LAUNCH_CHECK();
+    }
+    if (with_bias) {
+        const int rc = launch_bias_grad_final(ctx, st, ctx->bias_scratch, bias->out, g.K, d.splits, bias->alpha, bias->accumulate);
+        if (rc != VDNN_OK) return rc;
+        bias->done = true;
     }
     if (d.splits > 1) return launch_reduce_splits_tap(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, accumulate, g.C, 9);
     return VDNN_OK;
@@ -1057,7 +1065,7 @@ static int conv_bwd_filter_core(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
         // bfloat16 activations: both factors of every product are bfloat16 already
         if (wgrad3x3_ok(g)) { // loads of eight pixels take any alignment of the tensors
             bool taken = false;
-            const int rcw = launch_wgrad3x3(ctx, st, g, x, dy, w, alpha, accumulate, staging, staging_bytes, &taken);
+            const int rcw = launch_wgrad3x3(ctx, st, g, x, dy, w, alpha, accumulate, staging, staging_bytes, &taken, bias);
             if (taken || rcw != VDNN_OK) return rcw;
         }
         if (vec && ntap != 0 && PQ >= KH && 3 * g.Q >= KH && g.Q % 2 == 0 && ((uintptr_t)x & 3) == 0 && staging) {
@@ -1165,14 +1173,15 @@ static int conv_bwd_filter_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
 }
 
 // Does backward filter of this shape add up the bias gradient inside its own kernel? (The shapes' dispatch above: the
-// Winograd variant, the first-layer kernel, the filter-row kernel; float activations.)
+// Winograd variant - float activations only -, the first-layer kernel, the filter-row kernels.)
 static bool bwd_filter_sums_bias(const ConvGeo& g, int algo_mode, int dtype) {
-    if (dtype != VDNN_DTYPE_F32 || is_dense(g)) return false;
-    if (algo_mode == 1 && wino_wgrad_ok(g) && wino_wgrad_plan_ok(wino_wgrad_plan(g), g)) return true;
+    if (is_dense(g)) return false;
+    const bool f32 = dtype == VDNN_DTYPE_F32;
+    if (f32 && algo_mode == 1 && wino_wgrad_ok(g) && wino_wgrad_plan_ok(wino_wgrad_plan(g), g)) return true;
     if (g.C <= 3 && g.R == 3 && g.S == 3 && g.ph == 1 && g.pw == 1 && g.sh == 1 && g.sw == 1 && g.P == g.H && g.Q == g.W && g.W % 4 == 0 && g.W >= KB &&
         g.P * g.Q >= WSC_SLICE)
         return true;
-    return g.C > 4 && wgrad3x3_f32_ok(g);
+    return g.C > 4 && (f32 ? wgrad3x3_f32_ok(g) : wgrad3x3_ok(g));
 }
 
 extern "C" {

@@ -1049,6 +1049,23 @@ std::vector<unsigned char> Network::planPlacement(vdnn_t policy, const std::vect
             /* a stream on the device costs two passes at HBM speed, the link a hundred times that: everything stored at
                the peak that can be packed is packed before anything crosses the link; within a kind, the largest gain first */
             int pick = -1; double best = 0.0; unsigned char to = PLACE_LINK;
+            /* planLinkBytes: an allowance of bytes on the link that is spent first - whatever is stored at the peak and
+               whose bytes on the link (its packed stream where it can be packed) still fit goes there, the largest gain
+               first; packing on the device begins when nothing fits the rest of the allowance */
+            if (options.planLinkBytes > 0) {
+                double on_link = 0.0;
+                auto link_bytes = [&](int l) {
+                    const double size = (double)(layer[l]->SrcDataSize() * actBytes());
+                    return (options.compressOffload && srcIsRectified(l) && f < 1.0) ? f * size : size;
+                };
+                for (int l = 0; l < numLayers; l++) if (member[l] && place[l] == PLACE_LINK) on_link += link_bytes(l);
+                for (int l = 0; l < at; l++) {
+                    if (!member[l] || place[l] == PLACE_LINK || on_link + link_bytes(l) > (double)options.planLinkBytes) continue;
+                    const double size = (double)(layer[l]->SrcDataSize() * actBytes());
+                    const double gain = place[l] == PLACE_PACKED ? f * size : size;
+                    if (gain > best) { best = gain; pick = l; to = PLACE_LINK; }
+                }
+            }
             for (int pass = 0; pass < 2 && pick < 0; pass++) {
                 for (int l = 0; l < at; l++) {
                     if (!member[l] || place[l] == PLACE_LINK) continue;

@@ -1,6 +1,6 @@
 // Command-line front end: vdnn MODEL POLICY ALGO [--steps N] [--warmup N] [--batch N] [--seed N]
 //                                               [--cap-gb X] [--host-sync] [--plan] [--verbose] [--refined] [--fuse]
-//                                               [--zvc] [--keep-packed] [--hbm-budget-gb X] [--packed-fraction F] [--in-place] [--recompute-first] ...
+//                                               [--zvc] [--keep-packed] [--hbm-budget-gb X] [--plan-link-gb X] [--packed-fraction F] [--in-place] [--recompute-first] ...
 // The three positional words are the reference's grammar (vdnn.cu:8-54, README.md:18-60). The
 // reference times one unsynchronised iteration and prints microseconds labelled "ms"
 // (vdnn.cu:72-79); here the device is synchronised on both sides of the timed region and the
@@ -62,6 +62,7 @@ int main(int argc, char** argv) {
         else if (!strcmp(argv[i], "--prefetch-within-peak")) opt.prefetchWithinPeak = true;
         else if (!strcmp(argv[i], "--keep-tail-gb")) opt.keepTailBytes = (size_t)(atof(need("--keep-tail-gb needs a value")) * 1e9);
         else if (!strcmp(argv[i], "--hbm-budget-gb")) opt.hbmBudgetBytes = (size_t)(atof(need("--hbm-budget-gb needs a value")) * 1e9);
+        else if (!strcmp(argv[i], "--plan-link-gb")) opt.planLinkBytes = (size_t)(atof(need("--plan-link-gb needs a value")) * 1e9);
         else if (!strcmp(argv[i], "--packed-fraction")) opt.planPackedFraction = atof(need("--packed-fraction needs a value"));
         else if (!strcmp(argv[i], "--in-place")) opt.inPlaceBackward = true;
         else if (!strcmp(argv[i], "--recompute-first")) opt.recomputeFirstLayer = true;

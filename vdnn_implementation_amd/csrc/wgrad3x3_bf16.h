@@ -24,6 +24,8 @@
 #pragma once
 #include "mfma_bf16.h"
 
+#include <type_traits>
+
 namespace vdnn {
 
 constexpr int WG3_CH = 64; // input channels of a workgroup's tile
@@ -37,6 +39,10 @@ struct Wgrad3x3 {
     long partial_stride; // K*9*C
     float alpha;
     int accumulate;
+    // optional: the bias gradient's partial sums, [K][bias_splits] (split ks of channel m at m * bias_splits + ks). The
+    // workgroups of the centre filter row and the first block of input channels multiply dy by a block of ones as well.
+    float* bias_partial;
+    int bias_splits;
 };
 
 // d.M = K, d.N = 9*C, d.K = N*H*W; d.mtiles tiles of 2*WR output channels, d.ntiles = 3 * C/64 (filter row
@@ -168,7 +174,18 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
     fetch(fb);
     fetch(fa);
     __syncthreads();
-    auto slice_body = [&](int s, Fetched& f) {
+    // The workgroups that also sum dy (wavefronts 0 and 1 of them: input channels 0-31, all of the tile's rows of dy) run
+    // a copy of the loop of their own, chosen once, so that the loop of all others is unchanged. The sums of dy are one
+    // more product per fragment of dy, with ones: every column of the block holds them.
+    const bool sums_bias = g.bias_partial != nullptr && nt == 1 && wave < 2;
+    floatx16 bacc[RB];
+#pragma unroll
+    for (int i = 0; i < RB; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) bacc[i][v] = 0.0f;
+    const uintx4 ones_bits = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+    const bf16x8 ones = __builtin_bit_cast(bf16x8, ones_bits);
+    auto slice_body = [&](int s, Fetched& f, auto with_bias) {
         const int cur = s & 1;
         const unsigned short* arow = As[cur] + (wm0 + l32) * HSTRIDE + 8 * lk;
         const unsigned short* brow = Bs[cur] + (wc0 + l32) * HSTRIDE + 8 * lk;
@@ -203,6 +220,7 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
                 acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b0, acc[i][0], 0, 0, 0);
                 acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b1, acc[i][1], 0, 0, 0);
                 acc[i][2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b2, acc[i][2], 0, 0, 0);
+                if constexpr (decltype(with_bias)::value) bacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], ones, bacc[i], 0, 0, 0);
             }
         }
         qs += KH;
@@ -212,9 +230,22 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
         __syncthreads();
         fetch(f);
     };
-    for (int s = 0; s < nslices; s += 2) {
-        slice_body(s, fb);
-        if (s + 1 < nslices) slice_body(s + 1, fa);
+    auto run = [&](auto with_bias) {
+        for (int s = 0; s < nslices; s += 2) {
+            slice_body(s, fb, with_bias);
+            if (s + 1 < nslices) slice_body(s + 1, fa, with_bias);
+        }
+    };
+    if (sums_bias) run(std::true_type{});
+    else run(std::false_type{});
+    if (sums_bias && l32 == 0) {
+#pragma unroll
+        for (int i = 0; i < RB; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = m0 + wm0 + 32 * i + 8 * (v / 4) + 4 * lk + (v % 4);
+                if (m < g.K) g.bias_partial[(long)m * g.bias_splits + ks] = bacc[i][v];
+            }
     }
 
     // acc[i][s][v]: output channel m0 + wm0 + 32*i + 8*(v/4) + 4*lk + v%4, input channel c0 + wc0 + l32, tap (r, s)

@@ -18,7 +18,8 @@ class Options(C.Structure):
                 ("unfused_optimizer", _i), ("defer_optimizer", _i), ("offload_lag", _i), ("prefetch_depth", _i), ("data_type", _i),
                 ("fuse_activations", _i), ("keep_tail_bytes", _sz), ("prefetch_within_peak", _i), ("keep_packed_on_device", _i),
                 ("plan_packed_fraction", C.c_double),
-                ("compress_offload", _i), ("hbm_budget_bytes", _sz), ("in_place_backward", _i), ("recompute_first_layer", _i)]
+                ("compress_offload", _i), ("hbm_budget_bytes", _sz), ("in_place_backward", _i), ("recompute_first_layer", _i),
+                ("plan_link_bytes", _sz)]
 
 
 class LayerSpec(C.Structure):
@@ -102,7 +103,7 @@ class Network:
                  pool_bytes=0, cap_bytes=0, plan_only=False, host_sync=False, capture=False, verbose=False, device=0,
                  refined=False, unfused_optimizer=False, defer_optimizer=False, bf16=False, offload_lag=0, prefetch_depth=1,
                  fuse=False, compress=False, keep_tail_bytes=0, prefetch_within_peak=False, keep_packed=False,
-                 plan_packed_fraction=0.0, hbm_budget_bytes=0, in_place=False, recompute_first=False):
+                 plan_packed_fraction=0.0, hbm_budget_bytes=0, in_place=False, recompute_first=False, plan_link_bytes=0):
         o = Options()
         lib.vdnn_network_default_options(C.byref(o))
         o.seed, o.pool_bytes, o.cap_bytes = seed, int(pool_bytes), int(cap_bytes)
@@ -120,6 +121,7 @@ class Network:
         o.hbm_budget_bytes = int(hbm_budget_bytes)
         o.in_place_backward = int(in_place)
         o.recompute_first_layer = int(recompute_first)
+        o.plan_link_bytes = int(plan_link_bytes)
         if layers is not None:
             arr = (LayerSpec * len(layers))(*layers)
             self._h = lib.vdnn_network_create_custom(arr, len(layers), policy, algo, C.byref(o))
