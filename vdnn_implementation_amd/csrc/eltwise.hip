@@ -554,6 +554,94 @@ __global__ void __launch_bounds__(EB) maxpool_bwd_kernel(const E* __restrict__ x
     }
 }
 
+// Unpadded pooling with a compile-time window and stride (AlexNet's 3x3 / stride 2) on planes that fit LDS: a
+// workgroup stages `group` consecutive (n,c) planes - one contiguous run of memory - and writes their outputs, another
+// contiguous run. The general kernels address every element with 64-bit divisions by run-time extents and run-time
+// loop bounds, which cost more than the memory accesses; here every division is by a constant or a 32-bit multiply-high.
+// Same comparison, same order: the same bits.
+template <class E, int R, int S, int SH, int SW>
+__global__ void __launch_bounds__(EB) maxpool_fwd_planes_kernel(const E* __restrict__ x, E* __restrict__ y, int H, int W, int P, int Q,
+                                                                long planes, int group, FastDiv dPQ, FastDiv dQ) {
+    extern __shared__ float pool_lds[];
+    const int HW = H * W, PQ = P * Q;
+    const long plane0 = (long)blockIdx.x * group;
+    const int here = (int)(planes - plane0 < group ? planes - plane0 : group);
+    const E* xp = x + plane0 * HW;
+    for (int i = threadIdx.x; i < here * HW; i += EB) pool_lds[i] = load_elem(xp + i);
+    __syncthreads();
+    E* yp = y + plane0 * PQ;
+    for (int o = threadIdx.x; o < here * PQ; o += EB) {
+        const int pl = dPQ.div(o), pq = o - pl * PQ;
+        const int p = dQ.div(pq), q = pq - p * Q;
+        const float* b = pool_lds + pl * HW + p * SH * W + q * SW;
+        float m = -FLT_MAX;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int s_ = 0; s_ < S; s_++) {
+                const float v = b[r * W + s_];
+                if (v > m) m = v;
+            }
+        store_elem(yp + o, m);
+    }
+}
+
+// The backward counterpart: x and dy of `group` planes in LDS, every window's winner found once (first strict maximum
+// in row-major order, the window's first element if nothing exceeds -FLT_MAX), then every input element adds up the dy
+// of the windows that contain it and chose it, windows in row-major order - the general kernels' rule and order.
+template <class E, int R, int S, int SH, int SW>
+__global__ void __launch_bounds__(EB) maxpool_bwd_planes_fixed_kernel(const E* __restrict__ x, const E* __restrict__ dy, E* __restrict__ dx,
+                                                                      int H, int W, int P, int Q, long planes, int group, int gate,
+                                                                      FastDiv dPQ, FastDiv dQ, FastDiv dHW, FastDiv dW) {
+    extern __shared__ float pool_lds[];
+    const int HW = H * W, PQ = P * Q;
+    float* xs = pool_lds;                      // [group][HW]
+    float* dys = xs + group * HW;              // [group][PQ]
+    int* arg = (int*)(dys + group * PQ);       // [group][PQ] winner's index in its plane
+    const long plane0 = (long)blockIdx.x * group;
+    const int here = (int)(planes - plane0 < group ? planes - plane0 : group);
+    const E* xp = x + plane0 * HW;
+    const E* dyp = dy + plane0 * PQ;
+    for (int i = threadIdx.x; i < here * HW; i += EB) xs[i] = load_elem(xp + i);
+    for (int i = threadIdx.x; i < here * PQ; i += EB) dys[i] = load_elem(dyp + i);
+    __syncthreads();
+    for (int o = threadIdx.x; o < here * PQ; o += EB) {
+        const int pl = dPQ.div(o), pq = o - pl * PQ;
+        const int p = dQ.div(pq), q = pq - p * Q;
+        const int first = p * SH * W + q * SW;
+        const float* b = xs + pl * HW + first;
+        float m = -FLT_MAX;
+        int a = first;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int s_ = 0; s_ < S; s_++) {
+                const float v = b[r * W + s_];
+                if (v > m) { m = v; a = first + r * W + s_; }
+            }
+        arg[o] = a;
+    }
+    __syncthreads();
+    E* dxp = dx + plane0 * HW;
+    for (int i = threadIdx.x; i < here * HW; i += EB) {
+        const int pl = dHW.div(i), self = i - pl * HW;
+        const int h = dW.div(self), w = self - h * W;
+        // windows containing (h, w): p * SH <= h <= p * SH + R - 1
+        int p_lo = h - R + 1; p_lo = p_lo <= 0 ? 0 : (p_lo + SH - 1) / SH;
+        int p_hi = h / SH; if (p_hi > P - 1) p_hi = P - 1;
+        int q_lo = w - S + 1; q_lo = q_lo <= 0 ? 0 : (q_lo + SW - 1) / SW;
+        int q_hi = w / SW; if (q_hi > Q - 1) q_hi = Q - 1;
+        const int* ap = arg + pl * PQ;
+        const float* dp = dys + pl * PQ;
+        float acc = 0.0f;
+        for (int p = p_lo; p <= p_hi; p++)
+            for (int q = q_lo; q <= q_hi; q++)
+                if (ap[p * Q + q] == self) acc += dp[p * Q + q];
+        if (gate && !(xs[i] > 0.0f)) acc = 0.0f;
+        store_elem(dxp + i, acc);
+    }
+}
+
 // Overlapping windows on planes that fit LDS (AlexNet's 3x3 stride 2): a workgroup stages `group` whole
 // (n,c) planes and their dy, finds every window's winner once, and each input element then asks the few
 // windows that contain it. Same winner rule and the same summation order as the gather kernel above, so the
@@ -652,6 +740,14 @@ __global__ void __launch_bounds__(EB) maxpool2x2_bwd_kernel(const E* x, const E*
 // order, and a value crosses HBM once apart from the halo.
 constexpr int LRN_CH = 16;
 
+// scale^-3/4 = r * sqrt(r) with r = scale^-1/2: two hardware approximations of one unit in the last place each and a
+// multiply, instead of the general powf (dozens of instructions, which made the kernels wait for the vector ALU, not
+// for memory). scale >= 2 always (k = 2, the rest a sum of squares).
+__device__ __forceinline__ float lrn_pow_m075(float scale) {
+    const float r = __builtin_amdgcn_rsqf(scale);
+    return r * __builtin_amdgcn_sqrtf(r);
+}
+
 template <class E>
 __global__ void __launch_bounds__(EB) lrn_fwd_kernel(const E* __restrict__ x, E* __restrict__ y, int C, int hw, int chunks, size_t total) {
     const size_t i = (size_t)blockIdx.x * EB + threadIdx.x; // (sample, chunk, pixel), pixel fastest
@@ -676,7 +772,7 @@ __global__ void __launch_bounds__(EB) lrn_fwd_kernel(const E* __restrict__ x, E*
 #pragma unroll
         for (int d = 0; d < 5; d++) ss += v[k + d] * v[k + d];
         const float scale = LRN_KC + LRN_A5 * ss;
-        store_elem(yp + (size_t)(c0 + k) * hw, v[k + 2] * powf(scale, -LRN_BETA));
+        store_elem(yp + (size_t)(c0 + k) * hw, v[k + 2] * lrn_pow_m075(scale));
     }
 }
 
@@ -693,6 +789,8 @@ __global__ void __launch_bounds__(EB) lrn_bwd_kernel(const E* __restrict__ x, co
     const size_t base = (n * C) * hw + pix;
     float xv[LRN_CH + 8];  // channels c0-4 .. c0+LRN_CH+3
     float term[LRN_CH + 4]; // dy*y/scale of channels c0-2 .. c0+LRN_CH+1
+    float dyv[LRN_CH + 4];  // dy of the same channels: the thread's own sixteen are among them
+    float yv[LRN_CH + 4];
     float scale_own[LRN_CH];
 #pragma unroll
     for (int k = 0; k < LRN_CH + 8; k++) {
@@ -700,14 +798,20 @@ __global__ void __launch_bounds__(EB) lrn_bwd_kernel(const E* __restrict__ x, co
         xv[k] = (c >= 0 && c < C) ? load_elem(x + base + (size_t)c * hw) : 0.0f;
     }
 #pragma unroll
-    for (int k = 0; k < LRN_CH + 4; k++) {
+    for (int k = 0; k < LRN_CH + 4; k++) { // every fetch is issued before the first value is used
         const int c = c0 - 2 + k;
-        float ss = 0.0f; // the window of channel c, ascending
+        const bool in = c >= 0 && c < C;
+        dyv[k] = in ? load_elem(dy + base + (size_t)c * hw) : 0.0f;
+        yv[k] = in ? load_elem(y + base + (size_t)c * hw) : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < LRN_CH + 4; k++) {
+        float ss = 0.0f; // the window of channel c0 - 2 + k, ascending
 #pragma unroll
         for (int e = 0; e < 5; e++) ss += xv[k + e] * xv[k + e];
         const float scale = LRN_KC + LRN_A5 * ss;
         if (k >= 2 && k < LRN_CH + 2) scale_own[k - 2] = scale;
-        term[k] = (c >= 0 && c < C) ? load_elem(dy + base + (size_t)c * hw) * load_elem(y + base + (size_t)c * hw) / scale : 0.0f;
+        term[k] = dyv[k] * yv[k] * __builtin_amdgcn_rcpf(scale); // (zero outside the tensor: dy and y read as zero there)
     }
 #pragma unroll
     for (int k = 0; k < LRN_CH; k++) {
@@ -716,8 +820,8 @@ __global__ void __launch_bounds__(EB) lrn_bwd_kernel(const E* __restrict__ x, co
         float tsum = 0.0f;
 #pragma unroll
         for (int d = 0; d < 5; d++) tsum += term[k + d];
-        const float dyc = load_elem(dy + base + (size_t)c * hw);
-        store_elem(dx + base + (size_t)c * hw, dyc * powf(scale_own[k], -LRN_BETA) - (2.0f * 1e-4f * LRN_BETA / 5.0f) * xv[k + 4] * tsum);
+        const float dyc = dyv[k + 2];
+        store_elem(dx + base + (size_t)c * hw, dyc * lrn_pow_m075(scale_own[k]) - (2.0f * 1e-4f * LRN_BETA / 5.0f) * xv[k + 4] * tsum);
     }
 }
 
@@ -998,6 +1102,12 @@ static bool pool_geo(const vdnn_shape_t* s, PoolGeo& g) {
     return g.P > 0 && g.Q > 0 && (long)g.H * g.W < (1l << 31);
 }
 
+// 3x3 / stride 2 without padding, every window inside the plane (what (H - 3) / 2 + 1 outputs per axis give)
+static bool pool_is_3x3_s2(const PoolGeo& g) {
+    return g.R == 3 && g.S == 3 && g.sh == 2 && g.sw == 2 && g.ph == 0 && g.pw == 0 && g.H >= 3 && g.W >= 3 &&
+           2 * (g.P - 1) + 3 <= g.H && 2 * (g.Q - 1) + 3 <= g.W;
+}
+
 static bool pool_is_2x2_exact(const PoolGeo& g, const void* a, const void* b, const void* c) {
     return g.R == 2 && g.S == 2 && g.sh == 2 && g.sw == 2 && g.ph == 0 && g.pw == 0 && g.H % 2 == 0 && g.W % 4 == 0 &&
            aligned16(a) && aligned16(b) && (!c || aligned16(c));
@@ -1015,6 +1125,17 @@ static int maxpool_fwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
     if (pool_is_2x2_exact(g, x, y, nullptr)) {
         const size_t pairs = (size_t)g.N * g.C * (g.H / 2) * (g.W / 4);
         hipLaunchKernelGGL(maxpool2x2_fwd_kernel<E>, dim3(grid_for(pairs, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, y, g.H, g.W, pairs);
+    } else if (pool_is_3x3_s2(g) && (size_t)g.H * g.W * 4 <= 48 * 1024) {
+        // whole planes in LDS: as many per workgroup as give every thread a few elements
+        const size_t per_plane = (size_t)g.H * g.W * 4;
+        int group = (int)((8 * EB + g.H * g.W - 1) / (g.H * g.W));
+        if ((size_t)group * per_plane > 48 * 1024) group = (int)(48 * 1024 / per_plane);
+        if (group < 1) group = 1;
+        const long planes = (long)g.N * g.C;
+        const long blocks = (planes + group - 1) / group;
+        VDNN_REQUIRE(blocks < (1l << 31), "grid too large");
+        hipLaunchKernelGGL((maxpool_fwd_planes_kernel<E, 3, 3, 2, 2>), dim3((unsigned)blocks), dim3(EB), group * per_plane, st, x, y, g.H, g.W, g.P, g.Q,
+                           planes, group, FastDiv::make(g.P * g.Q), FastDiv::make(g.Q));
     } else {
         const size_t total = (size_t)g.N * g.C * g.P * g.Q;
         hipLaunchKernelGGL(maxpool_fwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, y, g, total);
@@ -1048,7 +1169,11 @@ static int maxpool_bwd_t(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
         const long planes = (long)g.N * g.C;
         const long blocks = (planes + group - 1) / group;
         VDNN_REQUIRE(blocks < (1l << 31), "grid too large");
-        hipLaunchKernelGGL(maxpool_bwd_planes_kernel<E>, dim3((unsigned)blocks), dim3(EB), group * per_plane, st, x, dy, dx, g, planes, group, gate);
+        if (pool_is_3x3_s2(g))
+            hipLaunchKernelGGL((maxpool_bwd_planes_fixed_kernel<E, 3, 3, 2, 2>), dim3((unsigned)blocks), dim3(EB), group * per_plane, st, x, dy, dx,
+                               g.H, g.W, g.P, g.Q, planes, group, gate, FastDiv::make(g.P * g.Q), FastDiv::make(g.Q), FastDiv::make(g.H * g.W), FastDiv::make(g.W));
+        else
+            hipLaunchKernelGGL(maxpool_bwd_planes_kernel<E>, dim3((unsigned)blocks), dim3(EB), group * per_plane, st, x, dy, dx, g, planes, group, gate);
     } else {
         const size_t total = (size_t)g.N * g.C * g.H * g.W;
         hipLaunchKernelGGL(maxpool_bwd_kernel<E>, dim3(grid_for(total, EB, 0x7FFFFFFF)), dim3(EB), 0, st, x, dy, dx, g, total, gate);
