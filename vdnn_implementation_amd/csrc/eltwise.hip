@@ -441,13 +441,17 @@ __global__ void __launch_bounds__(EB) bias_grad_partial_kernel(const E* __restri
     acc = block_sum(acc, sh);
     if (threadIdx.x == 0) partial[blockIdx.x] = acc;
 }
-// stage 2: one thread per channel adds its partials in split order
+// stage 2: one wavefront per channel; lane l adds partials l, l + 64, ... in that order, the 64 lane sums are added by
+// halving (a fixed order: the same bits every time). A channel's partials can be a few hundred (one per reduction split
+// of the filter-gradient kernel that left them): one thread walking them took longer than the kernel before it.
 __global__ void __launch_bounds__(EB) bias_grad_final_kernel(const float* __restrict__ partial, float* __restrict__ bias, int K, int splits, float alpha, int accumulate) {
-    const int k = blockIdx.x * EB + threadIdx.x;
+    const int k = blockIdx.x * (EB / 64) + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (k >= K) return;
     float s = 0.0f;
-    for (int i = 0; i < splits; i++) s += partial[(size_t)k * splits + i];
-    bias[k] = accumulate ? __fmaf_rn(alpha, s, bias[k]) : alpha * s;
+    for (int i = lane; i < splits; i += 64) s += partial[(size_t)k * splits + i];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off);
+    if (lane == 0) bias[k] = accumulate ? __fmaf_rn(alpha, s, bias[k]) : alpha * s;
 }
 
 // bias[o] += alpha * sum_n dy[n,o]
@@ -997,7 +1001,7 @@ static int bias_grad_splits(int N, int K, int num_cu, int* per_out) {
 // stage 2 alone, for kernels that leave the bias gradient's partial sums themselves (partial[k * splits + i])
 int vdnn::launch_bias_grad_final(vdnn_ctx* ctx, hipStream_t st, const float* partial, float* bias, int K, int splits, float alpha, int accumulate) {
     ProfScope prof(ctx, st, "conv_bwd_bias_final", 0.0, 4.0 * (double)K * (splits + 2));
-    hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB - 1) / EB), dim3(EB), 0, st, partial, bias, K, splits, alpha, accumulate);
+    hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB / 64 - 1) / (EB / 64)), dim3(EB), 0, st, partial, bias, K, splits, alpha, accumulate);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
@@ -1007,7 +1011,7 @@ static int bias_grad_launch(hipStream_t st, const E* dy, float* bias, float* par
                             float alpha, int accumulate) {
     hipLaunchKernelGGL(bias_grad_partial_kernel<E>, dim3(K * splits), dim3(EB), 0, st, dy, partials, N, K, PQ, splits, per);
     VDNN_LAUNCH_CHECK();
-    hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB - 1) / EB), dim3(EB), 0, st, partials, bias, K, splits, alpha, accumulate);
+    hipLaunchKernelGGL(bias_grad_final_kernel, dim3((K + EB / 64 - 1) / (EB / 64)), dim3(EB), 0, st, partials, bias, K, splits, alpha, accumulate);
     VDNN_LAUNCH_CHECK();
     return VDNN_OK;
 }
