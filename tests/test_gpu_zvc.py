@@ -242,7 +242,10 @@ def test_networks_with_compressed_offload_keep_every_bit(cnn, batch, algo, bf16)
                        # a budget decides, tensor by tensor, between the device, a packed stream on the device and the host
                        (VDNN_ALL, {"refined": True, "fuse": True, "plan_packed_fraction": 0.7, "hbm_budget_bytes": "tight"}),
                        (VDNN_ALL, {"refined": True, "plan_packed_fraction": 0.7, "hbm_budget_bytes": "middle", "offload_lag": 3}),
-                       (VDNN_CONV, {"fuse": True, "plan_packed_fraction": 0.7, "hbm_budget_bytes": "tight", "prefetch_within_peak": True})):
+                       (VDNN_CONV, {"fuse": True, "plan_packed_fraction": 0.7, "hbm_budget_bytes": "tight", "prefetch_within_peak": True}),
+                       # ... with an allowance of bytes that go over the link before anything is packed on the device
+                       (VDNN_ALL, {"refined": True, "fuse": True, "plan_packed_fraction": 0.7, "hbm_budget_bytes": "tight", "plan_link_bytes": 1 << 40,
+                                   "offload_lag": -1, "prefetch_within_peak": True})):
         if "hbm_budget_bytes" in kw:
             kw = dict(kw)
             kw["hbm_budget_bytes"] = budget_for(make, policy, kw)
@@ -255,6 +258,8 @@ def test_networks_with_compressed_offload_keep_every_bit(cnn, batch, algo, bf16)
                 places = net.placement()
                 assert net.plan_feasible() and {1, 2, 3} & set(places), places
                 assert [l for l, p in enumerate(places) if p in (2, 3)] == packed
+                if kw.get("plan_link_bytes"):   # an allowance without end: whatever leaves the device crosses the link
+                    assert 2 not in places, places
         if kw.get("fuse"):   # (which layers mask their gradient depends on what is offloaded: compare layer by layer)
             # (a layer whose input is a packed stream expands it itself at the start of its backward - from the block it
             # was kept in or the block the copy engine brought it back into - and masks as in BASELINE)

@@ -336,15 +336,18 @@ static int launch_winograd(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, bool
             VDNN_LAUNCH_CHECK();
         }
         {
-            GemmDims d = make_dims(p.rows, (int)(WINO_XI * Tpad), p.cred, 128, WINO_TN, 1);
-            LoadWinoU al{{U, (long)p.cred, p.rows, (unsigned)((size_t)p.rows * p.cred * sizeof(float))}, (long)p.rows * p.cred, d.mtiles, d.mtiles * d.ntiles,
-                         (int)(Tpad / WINO_TN)};
-            LoadDenseRowVec4 bl{V, WINO_XI * Tpad, (int)(WINO_XI * Tpad), (unsigned)((size_t)p.cred * WINO_XI * Tpad * sizeof(float))};
-            StoreDense<float> ep{Mo, nullptr, nullptr, WINO_XI * Tpad, 0, 1.0f, 0, 0, nullptr};
+            // several column tiles per workgroup, so that all workgroups make about one round of resident ones
+            const int mtiles = (p.rows + 127) / 128, tiles_per_xi = (int)(Tpad / WINO_TN);
+            const long all_tiles = (long)WINO_XI * mtiles * tiles_per_xi, slots = 3l * ctx->num_cu;
+            int group = (int)((all_tiles + slots - 1) / slots);
+            if (group < 1) group = 1;
+            if (group > tiles_per_xi) group = tiles_per_xi;
+            const int groups_per_xi = (tiles_per_xi + group - 1) / group;
+            const WinoGemm gm{U, V, Mo, p.rows, p.cred, Tpad, mtiles, tiles_per_xi, group, groups_per_xi};
             // work counted in the transformed domain: 36 products per 4x4 outputs and channel pair
-            const int rc = launch_igemm<128, WINO_TN>(ctx, st, bwd ? "conv_bwd_data_wino_gemm" : "conv_fwd_wino_gemm", al, bl, ep, d,
-                                                      2.0 * p.rows * (double)p.cred * WINO_XI * T);
-            if (rc != VDNN_OK) return rc;
+            ProfScope prof(ctx, st, bwd ? "conv_bwd_data_wino_gemm" : "conv_fwd_wino_gemm", 2.0 * p.rows * (double)p.cred * WINO_XI * T, 0.0);
+            hipLaunchKernelGGL(wino_gemm_kernel, dim3((unsigned)(WINO_XI * mtiles * groups_per_xi)), dim3(NT), 0, st, gm);
+            VDNN_LAUNCH_CHECK();
         }
         {
             const WinoTiles to{g.H, g.W, p.th, p.tw, p.rows, T, Tpad};

@@ -260,6 +260,148 @@ struct LoadDenseRowVec4 {
     }
 };
 
+// ---- the 36 products of forward / backward data, several column tiles per workgroup ------------------------------
+// M[m][xi * Tpad + t] = sum_c U[xi][m][c] * V[c][xi * Tpad + t]. The reduction is only cred / 16 slices long (8 for 128
+// channels): with one 128 x 128 tile per workgroup (igemm_kernel) the wait for the first operands and the 64 stores per
+// lane at the end weigh as much as the multiplies. Here a workgroup computes `group` consecutive column tiles of one
+// (xi, 128 rows): the software pipeline of igemm_kernel - global loads two slices ahead, LDS double-buffered, one barrier
+// per slice, fragments of the next half slice read while the current one is multiplied - runs on across the tile
+// boundaries (the slice after a tile's last is the next tile's first), so only the first tile pays the wait, and a tile's
+// result is stored while the wavefronts of the other resident workgroups multiply. Same products, same order of summation.
+struct WinoGemm {
+    const float* U;   // [36][rows][cred]
+    const float* V;   // [cred][36 * Tpad]
+    float* M;         // [rows][36 * Tpad]
+    int rows, cred;
+    long Tpad;        // a multiple of 128
+    int mtiles, tiles_per_xi, group, groups_per_xi;
+};
+
+__global__ void __launch_bounds__(NT) wino_gemm_kernel(const WinoGemm g) {
+    constexpr int TM = 128, TN = 128;
+    __shared__ __attribute__((aligned(16))) float As[2][TM * RED_STRIDE];
+    __shared__ __attribute__((aligned(16))) float Bs[2][KB * TN];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bid = xcd_remap(blockIdx.x, gridDim.x);
+    const int mt = bid % g.mtiles, rest = bid / g.mtiles;
+    const int grp = rest % g.groups_per_xi, xi = rest / g.groups_per_xi;
+    const int tile0 = grp * g.group;
+    const int ntile = min(g.group, g.tiles_per_xi - tile0);
+    const int m0 = mt * TM;
+    const int nsl = g.cred / KB;
+    const long ld = (long)WINO_XI * g.Tpad;          // row length of V and of M
+    const long col0 = (long)xi * g.Tpad + (long)tile0 * TN; // first column of the workgroup
+
+    // A: rows tid/4 + 64 i of U_xi, four reduction values at 4 (tid % 4); B: reduction rows tid/32 + 8 i, columns 4 (tid % 32)
+    const __amdgpu_buffer_rsrc_t rsA = make_rsrc(g.U + (long)xi * g.rows * g.cred, (unsigned)((size_t)g.rows * g.cred * sizeof(float)));
+    const __amdgpu_buffer_rsrc_t rsB = make_rsrc(g.V + col0, clamp_range(((long)(g.cred - 1) * ld + (long)ntile * TN) * 4));
+    int arow[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int row = m0 + (tid >> 2) + 64 * i;
+        arow[i] = row < g.rows ? (row * g.cred + 4 * (tid & 3)) * 4 : OOB;
+    }
+    const int brow = (int)(((long)(tid >> 5) * ld + 4 * (tid & 31)) * 4);
+    floatx4 ra[2], rb[2];
+    // the slice the next fetch is for: its reduction offset and its tile's column offset (bytes)
+    int ps = 0, pcol = 0, ptile = 0;
+    auto fetch = [&]() {
+        const bool live = ptile < ntile;   // past the last tile nothing is fetched (the values would never be used)
+#pragma unroll
+        for (int i = 0; i < 2; i++) ra[i] = buf_load4(rsA, live ? arow[i] : OOB, ps * KB * 4);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const long soff = ((long)(ps * KB + 8 * i) * ld) * 4 + pcol;
+            rb[i] = buf_load4(rsB, live ? brow : OOB, (int)soff);
+        }
+        ps += 1;
+        const bool wrap = ps == nsl;
+        ps = wrap ? 0 : ps; pcol += wrap ? TN * 4 : 0; ptile += wrap ? 1 : 0;
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) *(floatx4*)(As[buf] + ((tid >> 2) + 64 * i) * RED_STRIDE + 4 * (tid & 3)) = ra[i];
+#pragma unroll
+        for (int i = 0; i < 2; i++) *(floatx4*)(Bs[buf] + ((tid >> 5) + 8 * i) * TN + 4 * (tid & 31)) = rb[i];
+    };
+
+    floatx16 acc[2][2];
+    auto clear = [&]() {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+    };
+    clear();
+    const int wm0 = (wave & 1) * 64, wn0 = (wave >> 1) * 64;
+    const int l32 = lane & 31, lk = lane >> 5;
+    constexpr int A_TILE = 32 * RED_STRIDE, B_TILE = 32;
+    const int a_off = wm0 * RED_STRIDE, b_off = wn0;
+
+    fetch();
+    stash(0);
+    fetch();
+    __syncthreads();
+    floatx4 a0[2], b0[2], a1[2], b1[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) a0[i] = read_frag<TM, true>(As[0] + a_off + i * A_TILE, l32, lk, 0);
+#pragma unroll
+    for (int j = 0; j < 2; j++) b0[j] = read_frag<TN, false>(Bs[0] + b_off + j * B_TILE, l32, lk, 0);
+    int v = 0; // slices done so far (over all tiles): LDS buffer v & 1 holds the current one
+    for (int t = 0; t < ntile; t++) {
+        for (int s2 = 0; s2 < nsl; s2++, v++) {
+            const int cur = v & 1, nxt = cur ^ 1;
+#pragma unroll
+            for (int i = 0; i < 2; i++) a1[i] = read_frag<TM, true>(As[cur] + a_off + i * A_TILE, l32, lk, 1);
+#pragma unroll
+            for (int j = 0; j < 2; j++) b1[j] = read_frag<TN, false>(Bs[cur] + b_off + j * B_TILE, l32, lk, 1);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i][e], b0[j][e], acc[i][j], 0, 0, 0);
+            stash(nxt);
+#pragma unroll
+            for (int i = 0; i < 16; i++) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x300, 2, 0); }
+            __syncthreads();
+            fetch();
+#pragma unroll
+            for (int i = 0; i < 2; i++) a0[i] = read_frag<TM, true>(As[nxt] + a_off + i * A_TILE, l32, lk, 0);
+#pragma unroll
+            for (int j = 0; j < 2; j++) b0[j] = read_frag<TN, false>(Bs[nxt] + b_off + j * B_TILE, l32, lk, 0);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i][e], b1[j][e], acc[i][j], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+        }
+        // the tile's result: acc[it][jt][v2] is row m0 + wm0 + 32 it + 8 (v2 / 4) + 4 lk + v2 % 4, column wn0 + 32 jt + l32
+        float* out = g.M + col0 + (long)t * TN + wn0 + l32;
+#pragma unroll
+        for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+            for (int it = 0; it < 2; it++)
+#pragma unroll
+                for (int v2 = 0; v2 < 16; v2++) {
+                    const int m = m0 + wm0 + it * 32 + 8 * (v2 / 4) + 4 * lk + (v2 % 4);
+                    if (m < g.rows) out[(long)m * ld + jt * 32] = acc[it][jt][v2];
+                }
+        clear();
+    }
+}
+
 // ---- backward filter: F(3x3, 4x4) --------------------------------------------------------------------------------
 // The filter gradient of one 4x4 tile of output pixels is the 3x3 "output" of correlating the 6x6 input patch with the
 // 4x4 tile of dy as a "filter": dW = A't [ sum over tiles and samples of (G' dy G't) .* (Bt x B) ] A' with the same
