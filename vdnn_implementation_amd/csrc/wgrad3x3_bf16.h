@@ -185,55 +185,70 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
         for (int v = 0; v < 16; v++) bacc[i][v] = 0.0f;
     const uintx4 ones_bits = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
     const bf16x8 ones = __builtin_bit_cast(bf16x8, ones_bits);
-    auto slice_body = [&](int s, Fetched& f, auto with_bias) {
-        const int cur = s & 1;
-        const unsigned short* arow = As[cur] + (wm0 + l32) * HSTRIDE + 8 * lk;
-        const unsigned short* brow = Bs[cur] + (wc0 + l32) * HSTRIDE + 8 * lk;
+    // What a wavefront reads from LDS for half a slice (16 pixels): its rows of dy, the centre tap's fragment of x and
+    // the element before / after this lane's eight (in the row, unless the lane holds the slice's first / last group).
+    struct Frag { bf16x8 a[RB]; uintx4 v; unsigned prev, next; };
+    auto read_frag = [&](int buf, int h, Frag& fr) {
+        const unsigned short* arow = As[buf] + (wm0 + l32) * HSTRIDE + 8 * lk + 16 * h;
+        const unsigned short* brow = Bs[buf] + (wc0 + l32) * HSTRIDE + 8 * lk + 16 * h;
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            bf16x8 a[RB];
-#pragma unroll
-            for (int i = 0; i < RB; i++) a[i] = *(const bf16x8*)(arow + i * 32 * HSTRIDE + 16 * h);
-            const uintx4 v = *(const uintx4*)(brow + 16 * h);
-            // the element before / after this lane's eight: in the row unless the lane holds the slice's first / last group
-            const unsigned short* pp = (h == 0 && lk == 0) ? &Hs[cur][0][wc0 + l32] : brow + 16 * h - 1;
-            const unsigned short* np = (h == 1 && lk == 1) ? &Hs[cur][1][wc0 + l32] : brow + 16 * h + 8;
-            unsigned prev = *pp, next = *np;
-            int qg = qs + 16 * h + 8 * lk;
-            qg -= qg >= W ? W : 0;
-            if (HALFROW) qg -= qg >= W ? W : 0;
-            prev = qg == 0 ? 0u : prev;     // left of the image
-            next = qg == W - 8 ? 0u : next; // right of the image
-            const bool mid = HALFROW && qg == W - 4; // pixels 4.. of the eight begin an image row
-            const unsigned t1 = __builtin_amdgcn_alignbit(v.y, v.x, 16u), t2 = __builtin_amdgcn_alignbit(v.z, v.y, 16u),
-                           t3 = __builtin_amdgcn_alignbit(v.w, v.z, 16u);
-            uintx4 up, dn;
-            up.x = (v.x << 16) | prev; up.y = t1; up.z = t2; up.w = t3;
-            dn.x = t1; dn.y = t2; dn.z = t3; dn.w = (next << 16) | (v.w >> 16);
-            if (HALFROW) {
-                up.z &= mid ? 0xFFFF0000u : ~0u; // pixel 4 reads left of the image through the left tap
-                dn.y &= mid ? 0x0000FFFFu : ~0u; // pixel 3 reads right of the image through the right tap
-            }
-            const bf16x8 b0 = __builtin_bit_cast(bf16x8, up), b1 = __builtin_bit_cast(bf16x8, v), b2 = __builtin_bit_cast(bf16x8, dn);
-#pragma unroll
-            for (int i = 0; i < RB; i++) {
-                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b0, acc[i][0], 0, 0, 0);
-                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b1, acc[i][1], 0, 0, 0);
-                acc[i][2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b2, acc[i][2], 0, 0, 0);
-                if constexpr (decltype(with_bias)::value) bacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], ones, bacc[i], 0, 0, 0);
-            }
+        for (int i = 0; i < RB; i++) fr.a[i] = *(const bf16x8*)(arow + i * 32 * HSTRIDE);
+        fr.v = *(const uintx4*)brow;
+        const unsigned short* pp = (h == 0 && lk == 0) ? &Hs[buf][0][wc0 + l32] : brow - 1;
+        const unsigned short* np = (h == 1 && lk == 1) ? &Hs[buf][1][wc0 + l32] : brow + 8;
+        fr.prev = *pp; fr.next = *np;
+    };
+    auto multiply = [&](const Frag& fr, int h, auto with_bias) {
+        const uintx4 v = fr.v;
+        unsigned prev = fr.prev, next = fr.next;
+        int qg = qs + 16 * h + 8 * lk;
+        qg -= qg >= W ? W : 0;
+        if (HALFROW) qg -= qg >= W ? W : 0;
+        prev = qg == 0 ? 0u : prev;     // left of the image
+        next = qg == W - 8 ? 0u : next; // right of the image
+        const bool mid = HALFROW && qg == W - 4; // pixels 4.. of the eight begin an image row
+        const unsigned t1 = __builtin_amdgcn_alignbit(v.y, v.x, 16u), t2 = __builtin_amdgcn_alignbit(v.z, v.y, 16u),
+                       t3 = __builtin_amdgcn_alignbit(v.w, v.z, 16u);
+        uintx4 up, dn;
+        up.x = (v.x << 16) | prev; up.y = t1; up.z = t2; up.w = t3;
+        dn.x = t1; dn.y = t2; dn.z = t3; dn.w = (next << 16) | (v.w >> 16);
+        if (HALFROW) {
+            up.z &= mid ? 0xFFFF0000u : ~0u; // pixel 4 reads left of the image through the left tap
+            dn.y &= mid ? 0x0000FFFFu : ~0u; // pixel 3 reads right of the image through the right tap
         }
-        qs += KH;
-        qs -= qs >= W ? W : 0;
-        if (HALFROW) qs -= qs >= W ? W : 0;
+        const bf16x8 b0 = __builtin_bit_cast(bf16x8, up), b1 = __builtin_bit_cast(bf16x8, v), b2 = __builtin_bit_cast(bf16x8, dn);
+#pragma unroll
+        for (int i = 0; i < RB; i++) {
+            acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.a[i], b0, acc[i][0], 0, 0, 0);
+            acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.a[i], b1, acc[i][1], 0, 0, 0);
+            acc[i][2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.a[i], b2, acc[i][2], 0, 0, 0);
+            if constexpr (decltype(with_bias)::value) bacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.a[i], ones, bacc[i], 0, 0, 0);
+        }
+    };
+    // Slice s (LDS buffer `cur`), as two halves of 16 pixels with the barrier between them; every half's fragments are
+    // read while the half before it is multiplied:
+    //   read (s, 1); multiply (s, 0); write slice s + 1 to the other buffer; barrier;
+    //   fetch slice s + 3; read (s + 1, 0) from the buffer just completed; multiply (s, 1).
+    // All reads of a buffer precede the barrier after which it is written again.
+    Frag f0, f1;
+    read_frag(0, 0, f0);
+    auto slice_body = [&](auto parity, Fetched& f, auto with_bias) {
+        constexpr int cur = decltype(parity)::value;
+        read_frag(cur, 1, f1);
+        multiply(f0, 0, with_bias);
         stash(cur ^ 1, f);
         __syncthreads();
         fetch(f);
+        read_frag(cur ^ 1, 0, f0);
+        multiply(f1, 1, with_bias);
+        qs += KH;
+        qs -= qs >= W ? W : 0;
+        if (HALFROW) qs -= qs >= W ? W : 0;
     };
     auto run = [&](auto with_bias) {
         for (int s = 0; s < nslices; s += 2) {
-            slice_body(s, fb, with_bias);
-            if (s + 1 < nslices) slice_body(s + 1, fa, with_bias);
+            slice_body(std::integral_constant<int, 0>{}, fb, with_bias);
+            if (s + 1 < nslices) slice_body(std::integral_constant<int, 1>{}, fa, with_bias);
         }
     };
     if (sums_bias) run(std::true_type{});
