@@ -41,10 +41,11 @@ struct Win3x3 {
 };
 
 template <int MODE>
-__global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH al, const Win3x3 geo, const StoreNCHW<bf16_t> ep, const GemmDims d) {
+__global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH al, const Win3x3 geo, const StoreNCHW<bf16_t> ep, const GemmDims d) {
     // 64 rows x 256 pixels per workgroup, a 64 x 64 tile per wavefront: 64 accumulator registers, three workgroups
-    // resident per compute unit. (A 128 x 256 tile with 64 x 128 per wavefront reads a quarter less from LDS per
-    // MFMA but needs 400 registers: one wavefront per SIMD, and measured 25-40 % slower than this.)
+    // resident per compute unit. (A 128 x 256 tile with 64 x 128 per wavefront - three LDS fragment reads per four
+    // MFMAs instead of four, half the window traffic and barriers per MFMA, two workgroups per compute unit - measured
+    // the same on the large layers and 20 % slower on 14 x 14 planes.)
     constexpr int TM = W3_TM;
     constexpr int WM = 1;                // wavefronts along the rows
     constexpr int CW = W3_TN / 4;        // columns of a wavefront
@@ -150,6 +151,8 @@ __global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH a
     Fetched fa, fb;
     fa.hr = 0; fb.hr = 0;
     const int g0 = __builtin_amdgcn_readfirstlane(tid >> 7); // channel group of the thread's first item: uniform per wavefront
+    const int swapped = (tid >> 3) & 1;                      // this lane stores its second pixel first
+    const unsigned sel_first = swapped ? 0x07060302u : 0x05040100u, sel_second = swapped ? 0x05040100u : 0x07060302u;
 
     auto load_window = [&](int row_step, Fetched& f) {
         const int cb = row_step / 3, r = row_step - cb * 3;
@@ -162,23 +165,29 @@ __global__ void __launch_bounds__(NT, 2) conv3x3_bf16_kernel(const LoadPackedH a
             unsigned c[8];
 #pragma unroll
             for (int e = 0; e < 8; e++) c[e] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rsrc, vo, soff + e * step, 0);
-            // 2 x 8 transpose of 16-bit values: the low halves are the first pixel's channels, the high halves the second's
-            f.wr[i][0].x = __builtin_amdgcn_perm(c[1], c[0], 0x05040100u); f.wr[i][0].y = __builtin_amdgcn_perm(c[3], c[2], 0x05040100u);
-            f.wr[i][0].z = __builtin_amdgcn_perm(c[5], c[4], 0x05040100u); f.wr[i][0].w = __builtin_amdgcn_perm(c[7], c[6], 0x05040100u);
-            f.wr[i][1].x = __builtin_amdgcn_perm(c[1], c[0], 0x07060302u); f.wr[i][1].y = __builtin_amdgcn_perm(c[3], c[2], 0x07060302u);
-            f.wr[i][1].z = __builtin_amdgcn_perm(c[5], c[4], 0x07060302u); f.wr[i][1].w = __builtin_amdgcn_perm(c[7], c[6], 0x07060302u);
+            // 2 x 8 transpose of 16-bit values: the low halves are the first pixel's channels, the high halves the second's.
+            // wr[i][0] is the pixel this lane stores first: its first pixel in lanes 0-7 of every sixteen, its second in
+            // lanes 8-15 (store_window)
+            f.wr[i][0].x = __builtin_amdgcn_perm(c[1], c[0], sel_first); f.wr[i][0].y = __builtin_amdgcn_perm(c[3], c[2], sel_first);
+            f.wr[i][0].z = __builtin_amdgcn_perm(c[5], c[4], sel_first); f.wr[i][0].w = __builtin_amdgcn_perm(c[7], c[6], sel_first);
+            f.wr[i][1].x = __builtin_amdgcn_perm(c[1], c[0], sel_second); f.wr[i][1].y = __builtin_amdgcn_perm(c[3], c[2], sel_second);
+            f.wr[i][1].z = __builtin_amdgcn_perm(c[5], c[4], sel_second); f.wr[i][1].w = __builtin_amdgcn_perm(c[7], c[6], sel_second);
         }
         if (wave == 0) {
             const int soff = (cb * KH * plane + rowoff + W + 2) * 2;
             f.hr = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc, hoff | bit_to_all_ones(hrowinv, r), soff, 0);
         }
     };
+    // A lane's two pixels are neighbouring LDS rows, lane after lane two rows on: sixteen lanes storing their first
+    // pixels would meet only eight of the sixteen groups of four banks (160 bytes from lane to lane). Lanes 8-15 of
+    // every sixteen therefore store their second pixel first: odd rows, the other eight groups (a third fewer
+    // bank-conflict cycles in the kernel as a whole).
     auto store_window = [&](unsigned short* lds, const Fetched& f) {
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int e = 0; e < 2; e++)
-                *(uintx4*)(lds + (1 + 2 * (tid & 127) + e) * HSTRIDE + 8 * ((tid >> 7) + 2 * i)) = f.wr[i][e];
+                *(uintx4*)(lds + (1 + 2 * (tid & 127) + (e ^ swapped)) * HSTRIDE + 8 * ((tid >> 7) + 2 * i)) = f.wr[i][e];
         if (wave == 0) lds[((lane >> 5) ? W3_ROWS - 1 : 0) * HSTRIDE + (lane & 31)] = (unsigned short)f.hr;
     };
 
