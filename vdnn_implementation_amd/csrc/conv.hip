@@ -340,6 +340,9 @@ static int launch_winograd(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, bool
             const int mtiles = (p.rows + 127) / 128, tiles_per_xi = (int)(Tpad / WINO_TN);
             const long all_tiles = (long)WINO_XI * mtiles * tiles_per_xi, slots = 3l * ctx->num_cu;
             int group = (int)((all_tiles + slots - 1) / slots);
+            // ... unless that round would leave more than a seventh of the places idle (few tiles: 14 x 14 planes,
+            // 256 produced rows at 28 x 28): single tiles then, which the hardware hands out as places come free
+            if (20 * all_tiles < 17 * (long)group * slots) group = 1;
             if (group < 1) group = 1;
             if (group > tiles_per_xi) group = tiles_per_xi;
             const int groups_per_xi = (tiles_per_xi + group - 1) / group;
