@@ -14,8 +14,8 @@ The CPU baseline is the C checker under oracle/ on the host cores (convolutions 
 step at the same batch.
 
 Output: ONE line of strict JSON on stdout, a few KB: the metric, the roofline entry, the CPU baseline and a handful of
-scalars. Everything else (every configuration's figures, the kernel table) goes to stderr and into
-gpurun_out/bench_details.json. The default run has eight configurations; --sweep runs the whole table.
+scalars. Everything else (every configuration's figures, the kernel table) goes to stderr and into the file that
+--details names. The default run has nine configurations; --sweep runs the whole table.
 """
 import argparse
 import json
