@@ -40,7 +40,8 @@ struct Wgrad3x3 {
     float alpha;
     int accumulate;
     // optional: the bias gradient's partial sums, [K][bias_splits] (split ks of channel m at m * bias_splits + ks). The
-    // workgroups of the centre filter row and the first block of input channels multiply dy by a block of ones as well.
+    // workgroups add up the dy values they multiply; those of the centre filter row and the first block of input channels
+    // write the sums.
     float* bias_partial;
     int bias_splits;
 };
@@ -174,17 +175,22 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
     fetch(fb);
     fetch(fa);
     __syncthreads();
-    // The workgroups that also sum dy (wavefronts 0 and 1 of them: input channels 0-31, all of the tile's rows of dy) run
-    // a copy of the loop of their own, chosen once, so that the loop of all others is unchanged. The sums of dy are one
-    // more product per fragment of dy, with ones: every column of the block holds them.
-    const bool sums_bias = g.bias_partial != nullptr && nt == 1 && wave < 2;
-    floatx16 bacc[RB];
+    // A launch that also sums dy runs a copy of the loop of its own, chosen once, so that the loop of a launch without
+    // is unchanged: wavefronts 0 and 1 (input channels 0-31, all of the tile's rows of dy) add the eight values of every
+    // dy fragment to a running sum of the lane's row, two per v_dot2c_f32_bf16 with a pair of ones. With up to 128 input
+    // channels every workgroup of such a launch does, though only those of the centre filter row and the first block of
+    // input channels write their sums: the few workgroups of a reduction split read the same dy and x through L2 at the
+    // same time, and one with a longer loop falls behind until its lines are gone (the sums as one more MFMA per fragment
+    // in those workgroups alone: conv1_2 at batch 128 0.96 ms and 2.7 GB fetched against 0.85 ms and 1.8 GB without the
+    // sums; now 0.80 ms and 1.8 GB). With more channels a split has 24 workgroups and more, the straggler's share of the
+    // fetches is small, and the sixteen extra instructions per slice in all of them cost more (256 channels: + 5 %).
+    const bool bias_loop = g.bias_partial != nullptr && wave < 2 && (g.C <= 128 || nt == 1);
+    const bool sums_bias = bias_loop && nt == 1;
+    float bsum[RB];
 #pragma unroll
-    for (int i = 0; i < RB; i++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) bacc[i][v] = 0.0f;
-    const uintx4 ones_bits = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-    const bf16x8 ones = __builtin_bit_cast(bf16x8, ones_bits);
+    for (int i = 0; i < RB; i++) bsum[i] = 0.0f;
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const bf16x2 ones = __builtin_bit_cast(bf16x2, 0x3F803F80u);
     // What a wavefront reads from LDS for half a slice (16 pixels): its rows of dy, the centre tap's fragment of x and
     // the element before / after this lane's eight (in the row, unless the lane holds the slice's first / last group).
     struct Frag { bf16x8 a[RB]; uintx4 v; unsigned prev, next; };
@@ -222,7 +228,13 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
             acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.a[i], b0, acc[i][0], 0, 0, 0);
             acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.a[i], b1, acc[i][1], 0, 0, 0);
             acc[i][2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.a[i], b2, acc[i][2], 0, 0, 0);
-            if constexpr (decltype(with_bias)::value) bacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr.a[i], ones, bacc[i], 0, 0, 0);
+            if constexpr (decltype(with_bias)::value) {
+                // (pairs taken with shufflevector: bit casts of the elements of a 4 x 32-bit view all read the first one)
+                bsum[i] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(fr.a[i], fr.a[i], 0, 1), ones, bsum[i], false);
+                bsum[i] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(fr.a[i], fr.a[i], 2, 3), ones, bsum[i], false);
+                bsum[i] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(fr.a[i], fr.a[i], 4, 5), ones, bsum[i], false);
+                bsum[i] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(fr.a[i], fr.a[i], 6, 7), ones, bsum[i], false);
+            }
         }
     };
     // Slice s (LDS buffer `cur`), as two halves of 16 pixels with the barrier between them; every half's fragments are
@@ -251,16 +263,16 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
             if (s + 1 < nslices) slice_body(std::integral_constant<int, 1>{}, fa, with_bias);
         }
     };
-    if (sums_bias) run(std::true_type{});
+    if (bias_loop) run(std::true_type{});
     else run(std::false_type{});
-    if (sums_bias && l32 == 0) {
+    if (sums_bias) {
+        // a lane summed pixels 8 lk .. 8 lk + 7 of every 16 of its row: the two halves of the wavefront together
 #pragma unroll
-        for (int i = 0; i < RB; i++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int m = m0 + wm0 + 32 * i + 8 * (v / 4) + 4 * lk + (v % 4);
-                if (m < g.K) g.bias_partial[(long)m * g.bias_splits + ks] = bacc[i][v];
-            }
+        for (int i = 0; i < RB; i++) {
+            const float whole = bsum[i] + __shfl_xor(bsum[i], 32);
+            const int m = m0 + wm0 + 32 * i + l32;
+            if (lk == 0 && m < g.K) g.bias_partial[(long)m * g.bias_splits + ks] = whole;
+        }
     }
 
     // acc[i][s][v]: output channel m0 + wm0 + 32*i + 8*(v/4) + 4*lk + v%4, input channel c0 + wc0 + l32, tap (r, s)
