@@ -159,6 +159,30 @@ __global__ void __launch_bounds__(EB) bias_add_kernel(E* __restrict__ y, const f
     }
 }
 
+// p[0] + p[stride] + p[2 stride] + ... (`splits` terms), added in that order. The adds wait for one another; the loads
+// need not: eight splits are fetched at a time (a thread that fetches, adds, fetches pays a trip to memory per split).
+__device__ __forceinline__ float ordered_sum(const float* __restrict__ p, size_t stride, int splits) {
+    float s = p[0];
+    int k = 1;
+    for (; k + 8 <= splits; k += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = p[(size_t)(k + j) * stride];
+#pragma unroll
+        for (int j = 0; j < 8; j++) s += v[j];
+    }
+    if (k + 4 <= splits) {
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = p[(size_t)(k + j) * stride];
+#pragma unroll
+        for (int j = 0; j < 4; j++) s += v[j];
+        k += 4;
+    }
+    for (; k < splits; k++) s += p[(size_t)k * stride];
+    return s;
+}
+
 // out[i] = (accumulate ? out[i] : 0) + alpha * (p[0][i] + p[1][i] + ...) (+ bias[i % ncols]); split order fixed.
 // out and gate may be one tensor (a gradient written over the input that gates it): an element is read before it is written.
 template <class E>
@@ -167,8 +191,7 @@ __global__ void __launch_bounds__(EB) reduce_splits_kernel(E* out, const float* 
                                                            int relu, const E* gate) {
     const size_t stride = (size_t)gridDim.x * EB;
     for (size_t i = (size_t)blockIdx.x * EB + threadIdx.x; i < count; i += stride) {
-        float s = partial[i];
-        for (int k = 1; k < splits; k++) s += partial[(size_t)k * count + i];
+        const float s = ordered_sum(partial + i, count, splits);
         float r = accumulate ? __fmaf_rn(alpha, s, load_elem(out + i)) : alpha * s; // one fused multiply-add on every route
         if (bias_j) r += bias_j[i % ncols];
         if (relu) r = relu_value(r);
@@ -180,7 +203,9 @@ __global__ void __launch_bounds__(EB) reduce_splits_kernel(E* out, const float* 
 // The same sums when the splits are many (a reduction split over the whole chip for a small filter bank): a thread per
 // output would walk hundreds of partial sums one after the other on a handful of workgroups. Here a workgroup owns 32
 // outputs and eight groups of consecutive splits; a thread adds its group's splits in order, the eight group sums are
-// added in group order through LDS. TAP: the partial sums are in tap-major column order (see reduce_splits_tap_kernel).
+// added in group order through LDS. TAP: the partial sums are in tap-major column order (see reduce_splits_tap_kernel);
+// the workgroup's 32 outputs are then 32 neighbours in that order (one 128-byte run per split), written to their places
+// in the filter's order - the reads are `splits` times the writes.
 template <bool TAP>
 __global__ void __launch_bounds__(256) reduce_splits_wide_kernel(float* __restrict__ out, const float* __restrict__ partial, size_t count,
                                                                  int splits, float alpha, int accumulate, int C, int RS) {
@@ -190,25 +215,22 @@ __global__ void __launch_bounds__(256) reduce_splits_wide_kernel(float* __restri
     const int per = (splits + 7) / 8;
     const int k0 = grp * per, k1 = k0 + per < splits ? k0 + per : splits;
     float s = 0.0f;
-    if (i < count && k0 < k1) {
-        size_t src = i;
-        if (TAP) {
-            const int ncols = C * RS;
-            const size_t m = i / ncols;
-            const int rem = (int)(i - m * ncols);
-            const int c = rem / RS, tap = rem - c * RS;
-            src = m * ncols + (size_t)tap * C + c;
-        }
-        s = partial[(size_t)k0 * count + src];
-        for (int k = k0 + 1; k < k1; k++) s += partial[(size_t)k * count + src];
-    }
+    if (i < count && k0 < k1) s = ordered_sum(partial + (size_t)k0 * count + i, count, k1 - k0);
     sums[grp][o] = s;
     __syncthreads();
     if (grp == 0 && i < count) {
         float t = sums[0][o];
 #pragma unroll
         for (int g = 1; g < 8; g++) t += (g * per < splits) ? sums[g][o] : 0.0f;
-        out[i] = accumulate ? __fmaf_rn(alpha, t, out[i]) : alpha * t;
+        size_t dst = i;
+        if (TAP) {
+            const int ncols = C * RS;
+            const size_t m = i / ncols;
+            const int rem = (int)(i - m * ncols);
+            const int tap = rem / C, c = rem - tap * C;
+            dst = m * ncols + (size_t)c * RS + tap;
+        }
+        out[dst] = accumulate ? __fmaf_rn(alpha, t, out[dst]) : alpha * t;
     }
 }
 constexpr int kWideReduceSplits = 32;        // from this many splits on,
@@ -254,9 +276,7 @@ __global__ void __launch_bounds__(EB) reduce_tail_nchw_kernel(E* out, const floa
     const int tile = full_tiles + t;
     const int m = (tile % mtiles) * TM + row, j = (tile / mtiles) * TN + col;
     if (m >= M || j >= N) return;
-    const float* p = partial + (size_t)t * splits * per + local;
-    float s = p[0];
-    for (int k = 1; k < splits; k++) s += p[(size_t)k * per];
+    float s = ordered_sum(partial + (size_t)t * splits * per + local, (size_t)per, splits);
     if (bias) s += bias[m];
     if (relu) s = relu_value(s);
     const int n = j / opix, pix = j - n * opix;
@@ -294,17 +314,48 @@ __global__ void __launch_bounds__(EB) reduce_splits_tap_kernel(float* __restrict
     const int rem = (int)(i - m * ncols);
     const int c = rem / RS, tap = rem - c * RS;
     const size_t src = m * ncols + (size_t)tap * C + c;
-    float s = partial[src];
-    for (int k = 1; k < splits; k++) s += partial[(size_t)k * count + src];
+    const float s = ordered_sum(partial + src, count, splits);
     out[i] = accumulate ? __fmaf_rn(alpha, s, out[i]) : alpha * s;
+}
+
+// The same for filters of up to 16 taps, a workgroup per output channel and 64 input channels: the partial sums are read
+// in their own order (for a tap, 64 consecutive channels: whole lines), the sums pass through LDS and leave in the
+// filter's order (64 channels x taps: one run). A thread per output reads its partial sums C elements apart from its
+// neighbour's of the next tap - a line fetched for 28 bytes of it. Same sums in the same order: the same bits.
+constexpr int kTapTileC = 64, kTapTileMaxRS = 16;
+__global__ void __launch_bounds__(256) reduce_splits_tap_tile_kernel(float* __restrict__ out, const float* __restrict__ partial, size_t count,
+                                                                     int splits, float alpha, int accumulate, int C, int RS, int cblocks) {
+    __shared__ float tile[kTapTileMaxRS][kTapTileC + 1];
+    const int m = blockIdx.x / cblocks, c0 = (blockIdx.x - m * cblocks) * kTapTileC;
+    const size_t row = (size_t)m * C * RS;
+    for (int idx = threadIdx.x; idx < RS * kTapTileC; idx += 256) {
+        const int tap = idx / kTapTileC, cc = idx - tap * kTapTileC;
+        if (c0 + cc < C) {
+            const size_t src = row + (size_t)tap * C + c0 + cc;
+            tile[tap][cc] = ordered_sum(partial + src, count, splits);
+        }
+    }
+    __syncthreads();
+    const int here = C - c0 < kTapTileC ? C - c0 : kTapTileC;
+    float* o = out + row + (size_t)c0 * RS;
+    for (int idx = threadIdx.x; idx < here * RS; idx += 256) {
+        const int cc = idx / RS, tap = idx - cc * RS;
+        const float s = tile[tap][cc];
+        o[idx] = accumulate ? __fmaf_rn(alpha, s, o[idx]) : alpha * s;
+    }
 }
 
 int launch_reduce_splits_tap(vdnn_ctx* ctx, hipStream_t stream, float* out, const float* partial, size_t count, int splits,
                              float alpha, int accumulate, int C, int RS) {
     ProfScope prof(ctx, stream, "reduce_splits", 0.0, 4.0 * (double)count * (splits + 2));
+    const size_t rows = count / ((size_t)C * RS);
+    const int cblocks = (C + kTapTileC - 1) / kTapTileC;
     if (splits >= kWideReduceSplits && count <= kWideReduceCount)
         hipLaunchKernelGGL(reduce_splits_wide_kernel<true>, dim3((unsigned)((count + 31) / 32)), dim3(256), 0, stream,
                            out, partial, count, splits, alpha, accumulate, C, RS);
+    else if (RS <= kTapTileMaxRS && rows * (size_t)C * RS == count && rows * cblocks < (1ul << 31))
+        hipLaunchKernelGGL(reduce_splits_tap_tile_kernel, dim3((unsigned)(rows * cblocks)), dim3(256), 0, stream,
+                           out, partial, count, splits, alpha, accumulate, C, RS, cblocks);
     else
     hipLaunchKernelGGL(reduce_splits_tap_kernel, dim3(grid_for(count, EB, 0x7FFFFFFF)), dim3(EB), 0, stream,
                        out, partial, count, splits, alpha, accumulate, C, RS);
