@@ -505,6 +505,28 @@ def test_dynamic_ladder_rebuilds_cleanly_after_trials_that_fail_half_way():
         assert net.stats()["peak_bytes_in_use"] == need_all
 
 
+def test_dynamic_ladder_tries_its_last_rung():
+    """network.cu:89-98 ends with a per-layer choice of algorithm, each workspace tried against an empty pool
+    (layer.cu:1091-1147). Between the peaks of (VDNN_ALL, memory-optimal) and (VDNN_ALL, perf-optimal) that choice
+    takes workspaces that no longer fit once the activations are there; the ladder tries the step and sends layers
+    back to the memory-optimal kernels until it fits, so whatever it settles on steps within the cap."""
+    for kw in ({}, dict(refined=True, fuse=True, in_place=True, recompute_first=True, offload_lag=4)):
+        with plan(VGG16_64, VDNN_ALL, **kw) as net:
+            step(net)
+            lo = net.stats()["peak_bytes_in_use"]
+        with plan(VGG16_64, VDNN_ALL, VDNN_PERF_OPT_ALGO, **kw) as net:
+            step(net)
+            hi = net.stats()["peak_bytes_in_use"]
+        assert lo < hi
+        for f in (0.02, 0.3, 0.6, 0.9, 0.995):
+            cap = int(lo + (hi - lo) * f)
+            with plan(VGG16_64, BASELINE, VDNN_DYNAMIC_ALGO, cap_bytes=cap, **kw) as net:
+                assert net.policy == VDNN_ALL
+                for _ in range(2):
+                    assert net.forwardPropagation(True) == 0 and net.backwardPropagation(True) == 0
+                assert net.stats()["peak_bytes_in_use"] <= cap
+
+
 def test_custom_table_shape_inference_and_sanity():
     layers = [layer_spec(enums.FC_CONV, 2, 3, 20, 20, 1, 1, 8, 3), layer_spec(enums.RELU, 2, 8, 20, 20),
               layer_spec(enums.POOL, 2, 8, 20, 20, 0, 2, 0, 2), layer_spec(enums.FC_GEMM, 2, 800, 1, 1, 0, 0, 10, 1),

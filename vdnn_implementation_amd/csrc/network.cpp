@@ -579,10 +579,33 @@ void Network::vdnnDynamicAlgo() {
         }
     }
     if (options.verbose) printf("\n5. Dynamic Algorithm with VDNN_ALL\n");
-    reset(cnnType, VDNN_ALL, VDNN_PERF_OPT_ALGO);
-    for (int id = 0; id < DEFAULT_NUM_LAYER; id++) {
-        if (layer[id] == NULL) continue;
-        if (is_conv(layer[id]->LayerType())) layer[id]->findDynamicAlgo();
+    /* network.cu:89-98 stops at the per-layer choice, which tries every workspace against an empty pool: a workspace of
+     * hundreds of megabytes chosen that way need not fit once the activations are there, and the first training step
+     * would return -1. Here the choice is tried like the rungs above; while the trial step fails, the layer with the
+     * largest workspace still in use goes back to the memory-optimal kernels (with all of them there it is rung 1,
+     * which passed). */
+    std::vector<bool> demoted(DEFAULT_NUM_LAYER, false);
+    bool verified = false;
+    for (;;) {
+        reset(cnnType, VDNN_ALL, VDNN_PERF_OPT_ALGO);
+        for (int id = 0; id < DEFAULT_NUM_LAYER; id++) {
+            if (layer[id] == NULL || !is_conv(layer[id]->LayerType())) continue;
+            if (demoted[id]) layer[id]->setAlgoMode(VDNN_MEMORY_OPT_ALGO);
+            else layer[id]->findDynamicAlgo();
+        }
+        int largest = -1;
+        size_t most = 0;
+        for (int id = 0; id < DEFAULT_NUM_LAYER; id++) {
+            if (layer[id] == NULL || !is_conv(layer[id]->LayerType()) || layer[id]->AlgoMode() != VDNN_PERF_OPT_ALGO) continue;
+            const size_t w = std::max(layer[id]->FwdWorkSpaceSize(), std::max(layer[id]->BwdDataWorkSpaceSize(), layer[id]->BwdFilterWorkSpaceSize()));
+            if (w > most) { most = w; largest = id; }
+        }
+        if (verified || largest < 0) return; /* the tried choice, rebuilt; or nothing left to give up */
+        ret = forwardPropagation(true);
+        if (ret >= 0) ret = backwardPropagation(true);
+        if (ret >= 0) { verified = true; continue; } /* rebuild once more: the trial step changed the parameters */
+        if (options.verbose) printf("layer %d goes back to the memory-optimal kernels\n", largest);
+        demoted[largest] = true;
     }
 }
 
