@@ -523,6 +523,14 @@ struct StagingCarve {
     ~StagingCarve() { if (taken) { ctx->reduce_scratch = base; ctx->reduce_scratch_bytes = total; } }
 };
 
+// Room for a re-laid-out filter bank at the front of the staging area: only if nothing was taken from it yet and at
+// least half of it stays for the partial sums of split reductions (the largest need of a layer is a round of partial
+// tiles: 768 x 64 KB). Null otherwise.
+static float* packed_filter_place(vdnn_ctx* ctx, StagingCarve& carve, size_t bytes) {
+    if (carve.taken || !ctx->reduce_scratch || 2 * ((bytes + 255) / 256 * 256) > ctx->reduce_scratch_bytes) return nullptr;
+    return (float*)carve.take(bytes);
+}
+
 __global__ void __launch_bounds__(256) round_filter_bf16_kernel(const float* __restrict__ w, float* __restrict__ out, long count) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i < count) out[i] = round_to_bf16_value(w[i]);
@@ -791,14 +799,17 @@ static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
         const int RS = g.R * g.S;
         LoadIm2colPixTap<0, E> bl{{x, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, (long)g.C * g.H * g.W, g.N,
                                 FastDiv::make(RS), FastDiv::make(g.S)}};
+        // The filter bank re-laid-out in the blocked tap-major order is a dense operand read with 128-bit loads (in the
+        // master copy's order a slice's sixteen channels of one tap lie R*S floats apart). Perf-optimal: in the
+        // workspace. Memory-optimal: at the front of the context's staging area, where it leaves room for the partial sums.
+        const bool in_workspace = algo_mode == 1 && workspace && workspace_bytes >= wbytes && aligned16(workspace);
+        float* packed = in_workspace ? (float*)workspace : packed_filter_place(ctx, carve, wbytes);
         StoreNCHW<E> ep{y, bias, g.P * g.Q, ctx->reduce_scratch, relu, nullptr};
-        if (algo_mode == 1 && workspace && workspace_bytes >= wbytes && aligned16(workspace)) {
-            // perf-optimal: the filter bank, re-laid-out in the workspace, is a dense 128-bit operand
-            float* packed = (float*)workspace;
+        if (packed) {
             const int rc = launch_pack_filter(ctx, st, w, packed, g.K, g.C, RS, g.C * RS, RS);
             if (rc != VDNN_OK) return rc;
             LoadDenseRed<true> alp{packed, (long)K, g.K, wbytes};
-            return launch_by_m(ctx, st, kFwdPackedNames, alp, bl, ep, g.K, g.N * g.P * g.Q, K);
+            return launch_by_m(ctx, st, in_workspace ? kFwdPackedNames : kFwdNames, alp, bl, ep, g.K, g.N * g.P * g.Q, K);
         }
         LoadFilterTap<false> al{w, g.C * RS, RS, g.K, RS, wbytes, FastDiv::make(RS)};
         return launch_by_m(ctx, st, kFwdNames, al, bl, ep, g.K, g.N * g.P * g.Q, K);
@@ -935,12 +946,14 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
             // blocked tap-major reduction: one slice = one tap x 16 output channels
             const unsigned wbytes = (unsigned)((long)g.K * g.C * RS * 4);
             LoadIm2colPixTap<1, E> bl{{dy, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS}};
-            if (algo_mode == 1 && workspace && workspace_bytes >= wbytes && aligned16(workspace)) {
-                float* packed = (float*)workspace; // [c][(kb*RS + tap)*16 + l]
+            const bool in_workspace = algo_mode == 1 && workspace && workspace_bytes >= wbytes && aligned16(workspace);
+            float* packed = in_workspace ? (float*)workspace : packed_filter_place(ctx, carve, wbytes); // [c][(kb*RS + tap)*16 + l]
+            if (packed) {
+                ep.partial = ctx->reduce_scratch; // (behind the filter bank, if that lies in the staging area)
                 const int rc = launch_pack_filter(ctx, st, w, packed, g.C, g.K, RS, RS, g.C * RS);
                 if (rc != VDNN_OK) return rc;
                 LoadDenseRed<true> alp{packed, (long)K, g.C, wbytes};
-                return launch_by_m(ctx, st, kBwdDataPackedNames, alp, bl, ep, M, N, K, flops);
+                return launch_by_m(ctx, st, in_workspace ? kBwdDataPackedNames : kBwdDataNames, alp, bl, ep, M, N, K, flops);
             }
             LoadFilterTap<true> alt{w, RS, g.C * RS, g.C, RS, wbytes, dRS};
             return launch_by_m(ctx, st, kBwdDataNames, alt, bl, ep, M, N, K, flops);
