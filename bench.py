@@ -148,7 +148,14 @@ def is_bf16(policy_name):
 
 
 def is_perf(policy_name):
-    return "perf" in policy_name.split("+")[1:]
+    mods = policy_name.split("+")[1:]
+    return "perf" in mods or "wino" in mods
+
+
+def perf_kind(policy_name):
+    """0: memory-optimal, 1: perf-optimal, 2: perf-optimal with the Winograd variant (each sums in its own order)."""
+    mods = policy_name.split("+")[1:]
+    return 2 if "wino" in mods else 1 if "perf" in mods else 0
 
 
 def best_within(results, base, floor_ratio, need_link):
@@ -295,10 +302,12 @@ def main():
         lag_given = [int(m[3:]) for m in mods if m.startswith("lag")]
         link_first = [float(m[4:]) for m in mods if m.startswith("link")]   # "+linkX": X GB each way go over the link before anything is packed on the device
         mods = [m for m in mods if not m.startswith("budget") and not m.startswith("lag") and not m.startswith("link")]
-        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep", "inplace", "recompute", "perf"}, name
-        # "+perf": VDNN_PERF_OPT_ALGO, the workspace-using kernel variants (wide 3x3 layers as Winograd F(4x4, 3x3)): other
-        # sums than the memory-optimal kernels', so its loss is compared within the mode only
-        _, policy, algo = parse("VGG16_128", word, "VDNN_PERF_OPT_ALGO" if "perf" in mods else args.algo)
+        assert set(mods) <= {"refined", "slack", "bf16", "fused", "zvc", "tail", "ahead", "keep", "inplace", "recompute", "perf", "wino"}, name
+        # "+perf": VDNN_PERF_OPT_ALGO, the workspace-using kernel variants (3x3 layers on the bfloat16 matrix cores with every
+        # float operand as two bfloat16 parts): other sums than the memory-optimal kernels', so its loss is compared within
+        # the mode only. "+wino": the same mode with its Winograd variant where that applies (vdnn_conv_perf_variant).
+        _, policy, algo = parse("VGG16_128", word, "VDNN_PERF_OPT_ALGO" if ("perf" in mods or "wino" in mods) else args.algo)
+        be.lib.vdnn_conv_perf_variant(1 if "wino" in mods else 0)
         bf16 = args.bf16 or "bf16" in mods
         # (what a plan sends over the link gets the slack that hides it: the plan chooses the offload lag itself - the
         # longest of those that fit with the fewest bytes on the link - and backward fetches ahead wherever the peak allows)
@@ -343,12 +352,15 @@ def main():
         d = conv[dom]
         achieved = d["flops"] / (d["ms"] * 1e-3) / 1e12
         peak = BF16_MFMA_PEAK_TFLOPS if "bf16" in dom else FP32_MFMA_PEAK_TFLOPS
-        conv_all_tf = sum(v["flops"] for v in conv.values()) / (sum(v["ms"] for v in conv.values()) * 1e-3) / 1e12
+        if "split" in dom:
+            # float operands as two bfloat16 parts: three bfloat16 matrix instructions per product, priced as issued
+            achieved, peak = 3.0 * achieved, BF16_MFMA_PEAK_TFLOPS
+        conv_all_tf = sum((3.0 if "split" in k and "split" in dom else 1.0) * v["flops"] for k, v in conv.items()) / (sum(v["ms"] for v in conv.values()) * 1e-3) / 1e12
         traffic = measured_traffic().get(dom) if args.cnn == "VGG16" and args.batch == 128 and args.algo == "VDNN_MEMORY_OPT_ALGO" and not headline_bf16 else None
         roofline = {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                     "frac": achieved / peak, "traffic": traffic,
                     "traffic_unit": "bytes/launch, L2 fetch + write-back, profiles/%s" % os.path.basename(TRAFFIC_PROFILE),
-                    "algorithmic_flop_per_launch": d["flops"] / d["launches"],
+                    "algorithmic_flop_per_launch": (3.0 if "split" in dom else 1.0) * d["flops"] / d["launches"],
                     "avg_launch_ms": d["ms"] / d["launches"], "launches": d["launches"]}
     kernels = {k: {"launches": v["launches"], "avg_ms": v["ms"] / max(v["launches"], 1),
                    "tflops": (v["flops"] / (v["ms"] * 1e-3) / 1e12) if v["flops"] else None,
@@ -378,7 +390,7 @@ def main():
         "peak_hbm_gb": results[head]["peak_hbm_gb"],
         "peak_hbm_reduction_vs_baseline": (base["peak_hbm_gb"] / results[head]["peak_hbm_gb"]) if base else None,
         # within an element type and an algorithm mode every configuration runs the same kernels on the same values
-        "losses_bit_identical": all(len({results[k]["loss"] for k in results if is_bf16(k) == b and is_perf(k) == p}) <= 1 for b in (False, True) for p in (False, True)),
+        "losses_bit_identical": all(len({results[k]["loss"] for k in results if is_bf16(k) == b and perf_kind(k) == p}) <= 1 for b in (False, True) for p in (0, 1, 2)),
         "perf_opt_speed_vs_memory_opt": (results["BASELINE+perf"]["images_per_s"] / base["images_per_s"]) if base and "BASELINE+perf" in results else None,
         "conv_mfma_util": conv_all_tf / peak if conv_all_tf else None,
         # float only, same losses as the literal run bit for bit: the fastest VDNN configuration at >= 3x less memory than

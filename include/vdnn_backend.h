@@ -182,6 +182,14 @@ size_t vdnn_conv_workspace_bytes_dtype(const vdnn_shape_t* shape, int algo_mode,
  * it before networks are built, not between a query and the pass that uses its answer. Results do not depend on it
  * (samples are independent in forward and backward data). */
 size_t vdnn_conv_winograd_chunk_bytes(size_t bytes);
+/* Tuning (no counterpart in the reference; cuDNN's perf-optimal choice is made by cudnnGet*Algorithm, layer.cu:1012-1090):
+ * which kernels VDNN_PERF_OPT_ALGO takes for 3x3 / stride 1 / padding 1 layers with float activations where both
+ * apply. 0 (default): the bfloat16 matrix cores with every float operand as two bfloat16 parts and three matrix
+ * instructions per product (about 5e-6 of the largest output from the exact result; workspace = the filter's bytes);
+ * 1: Winograd F(4x4, 3x3) / F(3x3, 4x4) (about 2e-5; workspace of a third to three quarters of a gigabyte). Returns
+ * the previous value; other arguments only query. Process-wide, and it changes what vdnn_conv_workspace_bytes reports:
+ * set it before networks are built. */
+int vdnn_conv_perf_variant(int variant);
 /* cudnnConvolutionForward + cudnnAddTensor (layer.cu:560-582): y = x (*) w + bias[k], the bias is
  * added once after the full reduction. bias may be NULL (no add). */
 int vdnn_conv_fwd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t* shape, int algo_mode,

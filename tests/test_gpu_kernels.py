@@ -33,6 +33,14 @@ def accurate_oracle():
     oracle.set_accumulate_double(False)
 
 
+@pytest.fixture
+def winograd_variant():
+    """The perf-optimal mode takes Winograd where it applies (its default is the split-bfloat16 kernels)."""
+    before = lib.vdnn_conv_perf_variant(1)
+    yield
+    lib.vdnn_conv_perf_variant(before)
+
+
 CONV_GOLDEN = ["vgg_3x3_p1", "alex_11x11_s4", "alex_5x5_p2", "overfeat_5x5_p0", "overfeat_6x6_to_1x1",
                "overfeat_1x1", "odd_3x3_s2_p1"]
 
@@ -174,7 +182,7 @@ def winograd_wgrad_applies(geom):
 
 
 @pytest.mark.parametrize("geom", PERF_OPT_GEOMS, ids=lambda g: "x".join(map(str, g)))
-def test_conv_perf_opt_variants(ctx, geom):
+def test_conv_perf_opt_variants(ctx, geom, winograd_variant):
     """The workspace-using variants. Wide 3x3 layers run forward and backward data as Winograd F(4x4, 3x3): other sums,
     held to the tolerance against the checker (or, at sizes the checker cannot afford, against the workspace-free
     kernels). Elsewhere forward and backward data read a re-laid-out filter bank in the same reduction order and return
@@ -245,7 +253,7 @@ WINOGRAD_GEOMS = [
 
 @pytest.mark.parametrize("geom", WINOGRAD_GEOMS, ids=lambda g: "x".join(map(str, g)))
 @pytest.mark.parametrize("small_chunks", [False, True], ids=["one-chunk", "small-chunks"])
-def test_conv_winograd_against_oracle(ctx, geom, small_chunks):
+def test_conv_winograd_against_oracle(ctx, geom, small_chunks, winograd_variant):
     """Forward (with and without the fused rectifier) and backward data (plain, gated, and written over the gating
     input) of the perf-optimal mode's Winograd variant against the checker; with small chunks the batch is processed in
     several pieces (two samples at a time), the last one shorter."""
@@ -310,6 +318,107 @@ def test_conv_winograd_against_oracle(ctx, geom, small_chunks):
             assert np.array_equal(dx_.download(x.shape), gated)
     finally:
         lib.vdnn_conv_winograd_chunk_bytes(0)
+
+
+# The perf-optimal mode's default for 3x3 / stride 1 / padding 1 float layers: operands as two bfloat16 parts, three
+# matrix instructions per product. Forward needs C % 16 == 0, backward data K % 16 == 0, both an even W; backward filter
+# W % 4 == 0, W >= 16, H*W % 8 == 0 and C % 64 == 0. Tile edges, ragged row tiles, split and tail reductions, rows that
+# are not whole groups of eight pixels.
+SPLIT_GEOMS = [
+    (3, 64, 16, 16, 64, 3, 3, 1, 1, 1, 1),
+    (2, 128, 28, 28, 96, 3, 3, 1, 1, 1, 1),     # 96 rows: a ragged second row tile
+    (2, 64, 12, 20, 130, 3, 3, 1, 1, 1, 1),     # rows of two and a half groups; 130 output channels: backward data takes another kernel
+    (5, 16, 6, 10, 32, 3, 3, 1, 1, 1, 1),       # one slice of channels; backward filter takes another kernel
+    (1, 512, 28, 28, 192, 3, 3, 1, 1, 1, 1),    # deep reduction, few tiles: split
+    (3, 64, 56, 56, 130, 3, 3, 1, 1, 1, 1),     # several pixel tiles per sample, tiles that straddle samples
+    (7, 128, 6, 20, 192, 3, 3, 1, 1, 1, 1),     # planes smaller than a pixel tile
+    (2, 64, 16, 36, 64, 3, 3, 1, 1, 1, 1),      # rows of four and a half groups
+    (130, 32, 14, 14, 48, 3, 3, 1, 1, 1, 1),    # more tiles than one round: the tail round is split
+]
+
+
+def split_applies(geom):
+    """(forward, backward data, backward filter) of the split-bfloat16 variant."""
+    n, c, h, w, k, r, s, ph, pw, sh, sw = geom
+    base = (r, s, ph, pw, sh, sw) == (3, 3, 1, 1, 1, 1) and w % 2 == 0 and c > 4
+    return (base and c % 16 == 0, base and k % 16 == 0,
+            (r, s, ph, pw, sh, sw) == (3, 3, 1, 1, 1, 1) and w % 4 == 0 and w >= 16 and (h * w) % 8 == 0 and c % 64 == 0)
+
+
+@pytest.mark.parametrize("geom", SPLIT_GEOMS, ids=lambda g: "x".join(map(str, g)))
+def test_conv_split_bf16_against_oracle(ctx, geom):
+    """Forward (with and without the fused rectifier), backward data (plain, gated, written over the gating input) and
+    backward filter (alone, applied, with the bias gradient) of the perf-optimal mode's default variant against the
+    checker. Its error is that of two dropped low-order terms per product, about 5e-6 of the largest output: held to
+    3e-5 here where the mode's bound is 1e-4. The same bits twice."""
+    tight = 3e-5
+    fwd_ok, bwd_ok, flt_ok = split_applies(geom)
+    rng = np.random.default_rng(hash(geom) % (2 ** 31) + 5)
+    g, og = be.shape(*geom), oracle.shape(*geom)
+    filter_bytes = g.k * g.c * 9 * 4
+    x = rng.standard_normal((g.n, g.c, g.h, g.w)).astype(np.float32)
+    w = (rng.standard_normal((g.k, g.c, 3, 3)) * np.sqrt(2.0 / (g.c * 9))).astype(np.float32)
+    b = rng.standard_normal(g.k).astype(np.float32)
+    want_y = oracle.conv_fwd(og, x, w, b)
+    dy = (rng.standard_normal(want_y.shape) + 0.25).astype(np.float32)
+    want_dx = oracle.conv_bwd_data(og, dy, w)
+    assert lib.vdnn_conv_perf_variant(-1) == 0
+    fwd_bytes, bwd_bytes, flt_bytes = (int(lib.vdnn_conv_workspace_bytes(g, 1, p)) for p in range(3))
+    if fwd_ok:
+        assert fwd_bytes == filter_bytes
+    if bwd_ok:
+        assert bwd_bytes == filter_bytes
+    with Dev(ctx) as d:
+        dx_, dw, db, ddy = d.up(x), d.up(w), d.up(b), d.up(dy)
+        y, gx = d.empty(want_y.shape), d.empty(x.shape)
+        ws = d.empty((max(fwd_bytes, bwd_bytes, flt_bytes, 4) // 4,))
+        announce("split bf16", geom, "fwd")
+        check(lib.vdnn_conv_fwd(ctx.handle, None, g, 1, dx_.ptr, dw.ptr, db.ptr, y.ptr, ws.ptr, fwd_bytes))
+        first = y.download(want_y.shape)
+        assert_close(first, want_y, tight, "fwd")
+        if fwd_ok:
+            y0 = d.empty(want_y.shape)
+            check(lib.vdnn_conv_fwd(ctx.handle, None, g, 0, dx_.ptr, dw.ptr, db.ptr, y0.ptr, None, 0))
+            assert not np.array_equal(y0.download(want_y.shape), first)   # (the variant ran)
+        check(lib.vdnn_conv_fwd(ctx.handle, None, g, 1, dx_.ptr, dw.ptr, db.ptr, y.ptr, ws.ptr, fwd_bytes))
+        assert np.array_equal(y.download(want_y.shape), first)
+        announce("split bf16", geom, "fwd + relu")
+        check(lib.vdnn_conv_fwd_relu(ctx.handle, None, g, 1, dx_.ptr, dw.ptr, db.ptr, y.ptr, ws.ptr, fwd_bytes))
+        assert np.array_equal(y.download(want_y.shape), np.maximum(first, 0))
+        if fwd_bytes:
+            # a workspace that is too small: the memory-optimal kernels run instead
+            check(lib.vdnn_conv_fwd(ctx.handle, None, g, 1, dx_.ptr, dw.ptr, db.ptr, y.ptr, ws.ptr, fwd_bytes - 256))
+            assert_close(y.download(want_y.shape), want_y, tight, "fwd, short workspace")
+        announce("split bf16", geom, "bwd_data")
+        check(lib.vdnn_conv_bwd_data(ctx.handle, None, g, 1, ddy.ptr, dw.ptr, gx.ptr, ws.ptr, bwd_bytes))
+        plain = gx.download(x.shape)
+        assert_close(plain, want_dx, tight, "bwd data")
+        announce("split bf16", geom, "bwd_data gated")
+        check(lib.vdnn_conv_bwd_data_relu(ctx.handle, None, g, 1, ddy.ptr, dw.ptr, dx_.ptr, gx.ptr, ws.ptr, bwd_bytes))
+        gated = gx.download(x.shape)
+        assert np.array_equal(gated, np.where(x > 0, plain, 0))
+        announce("split bf16", geom, "bwd_filter")
+        assert bool(lib.vdnn_conv_bwd_filter_sums_bias(g, 1, 0)) or not flt_ok
+        gw, gb, wu, bu = d.empty(w.shape), d.empty(b.shape), d.up(w), d.up(b)
+        fws = ws.ptr if flt_bytes else None
+        check(lib.vdnn_conv_bwd_filter_bias(ctx.handle, None, g, 1, dx_.ptr, ddy.ptr, gw.ptr, gb.ptr, fws, flt_bytes))
+        got_dw, got_db = gw.download(w.shape), gb.download(b.shape)
+        assert_close(got_dw, oracle.conv_bwd_filter_sgd(og, x, dy, np.zeros_like(w), 1.0), tight, "bwd filter")
+        assert_close(got_db, oracle.conv_bwd_bias_sgd(og, dy, np.zeros_like(b), 1.0), tight, "bias gradient")
+        alpha = np.float32(-0.37)
+        check(lib.vdnn_conv_bwd_filter_bias_sgd(ctx.handle, None, g, 1, dx_.ptr, ddy.ptr, wu.ptr, bu.ptr, alpha, fws, flt_bytes))
+        assert_close(wu.download(w.shape), oracle.conv_bwd_filter_sgd(og, x, dy, w, alpha), tight, "bwd filter + sgd")
+        assert_close(bu.download(b.shape), oracle.conv_bwd_bias_sgd(og, dy, b, alpha), tight, "bias + sgd")
+        check(lib.vdnn_conv_bwd_filter(ctx.handle, None, g, 1, dx_.ptr, ddy.ptr, gw.ptr, fws, flt_bytes))
+        assert np.array_equal(gw.download(w.shape), got_dw)
+        if flt_ok:
+            g0 = d.empty(w.shape)
+            check(lib.vdnn_conv_bwd_filter(ctx.handle, None, g, 0, dx_.ptr, ddy.ptr, g0.ptr, None, 0))
+            assert not np.array_equal(g0.download(w.shape), got_dw)   # (the variant ran)
+        announce("split bf16", geom, "bwd_data over the gating input")
+        assert lib.vdnn_conv_bwd_data_in_place_ok(g)
+        check(lib.vdnn_conv_bwd_data_relu(ctx.handle, None, g, 1, ddy.ptr, dw.ptr, dx_.ptr, dx_.ptr, ws.ptr, bwd_bytes))
+        assert np.array_equal(dx_.download(x.shape), gated)
 
 
 # (geometry, algorithm mode, whether the filter-gradient kernel of the shape adds up the bias gradient itself)

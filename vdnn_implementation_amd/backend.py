@@ -99,6 +99,7 @@ BACKEND_SYMBOLS = {
     "vdnn_conv_workspace_bytes": (_sz, [_S, _i, _i]),
     "vdnn_conv_workspace_bytes_dtype": (_sz, [_S, _i, _i, _i]),
     "vdnn_conv_winograd_chunk_bytes": (_sz, [_sz]),
+    "vdnn_conv_perf_variant": (_i, [_i]),
     "vdnn_conv_fwd": (_i, [_vp, _vp, _S, _i, _vp, _vp, _vp, _vp, _vp, _sz]),
     "vdnn_bias_add": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     "vdnn_conv_bwd_data": (_i, [_vp, _vp, _S, _i, _vp, _vp, _vp, _vp, _sz]),

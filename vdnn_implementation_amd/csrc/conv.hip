@@ -14,6 +14,7 @@
 #include "conv3x3_bf16.h"
 #include "wgrad3x3_bf16.h"
 #include "wgrad3x3_f32.h"
+#include "wgrad3x3_split.h"
 #include "conv_smallc.h"
 #include "conv_smallc_mfma.h"
 #include "winograd_f32.h"
@@ -72,6 +73,8 @@ static const PassNames kFwdHalfNames{"conv_fwd_bf16mfma_64x256", "conv_fwd_bf16m
 static const PassNames kBwdDataHalfNames{"conv_bwd_data_bf16mfma_64x256", "conv_bwd_data_bf16mfma_128x128"};
 static const PassNames kFwdWin3Names{"conv_fwd_bf16win_64x256", "conv_fwd_bf16win_64x256"};
 static const PassNames kBwdDataWin3Names{"conv_bwd_data_bf16win_64x256", "conv_bwd_data_bf16win_64x256"};
+static const PassNames kFwdSplitNames{"conv_fwd_split_64x256", "conv_fwd_split_64x256"};
+static const PassNames kBwdDataSplitNames{"conv_bwd_data_split_64x256", "conv_bwd_data_split_64x256"};
 static const PassNames kBwdFilterHalfNames{"conv_bwd_filter_bf16mfma_64x256", "conv_bwd_filter_bf16mfma_128x128"};
 static const PassNames kBwdFilterWin3Names{"conv_bwd_filter_bf16win_64x192", "conv_bwd_filter_bf16win_128x192"};
 static const PassNames kBwdFilterRow3Names{"conv_bwd_filter_row_64x192", "conv_bwd_filter_row_128x192"};
@@ -151,10 +154,14 @@ static int launch_by_m(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names
 }
 
 // The windowed 3x3 kernel (conv3x3_bf16.h): tiles of 64 rows by 256 pixels, three workgroups resident per compute
-// unit, the reduction cut at multiples of one filter row of a channel block. Splits and tail mode as in launch_by_m.
-template <int MODE>
-static int launch_win3x3(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names, const LoadPackedH& al, const Win3x3& geo, const StoreNCHW<bf16_t>& ep,
+// unit (two on float layers, where the kernel holds more registers), the reduction cut at multiples of one filter
+// row of a channel block. Splits and tail mode as in launch_by_m. K counts 16-bit values of a row of the filter
+// operand (float layers: two per filter element).
+constexpr int kWin3SplitPerCU = 2;
+template <int MODE, class E>
+static int launch_win3x3(vdnn_ctx* ctx, hipStream_t stream, const PassNames& names, const LoadPackedH& al, const Win3x3T<E>& geo, const StoreNCHW<E>& ep,
                          int M, int N, int K, double flops, size_t partial_bytes) {
+    constexpr bool SPLIT = sizeof(E) == 4;
     const int TM = W3_TM, TN = W3_TN;
     const long tiles = (long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
     int splits = 1;
@@ -166,7 +173,7 @@ static int launch_win3x3(vdnn_ctx* ctx, hipStream_t stream, const PassNames& nam
         splits = choose_splits(tiles, K, cap, ctx->num_cu, out_bytes, 2.0 * TM * TN * KB);
     }
     GemmDims d = make_dims(M, N, K, TM, TN, splits, W3_DEPTH);
-    const long slots = 3l * ctx->num_cu;
+    const long slots = (SPLIT ? kWin3SplitPerCU : 3l) * ctx->num_cu;
     const long rem = tiles % slots;
     int tail_tiles = 0;
     if (splits == 1 && tiles > slots && rem > 0 && 2 * rem <= slots && ep.partial) {
@@ -186,7 +193,7 @@ static int launch_win3x3(vdnn_ctx* ctx, hipStream_t stream, const PassNames& nam
     if (blocks <= 0 || blocks >= (1l << 31)) { set_error("conv3x3: grid of %ld workgroups out of range", blocks); return VDNN_EINVAL; }
     {
         ProfScope prof(ctx, stream, names.t64, flops, 0.0);
-        hipLaunchKernelGGL((conv3x3_bf16_kernel<MODE>), dim3((unsigned)blocks), dim3(NT), 0, stream, al, geo, ep, d);
+        hipLaunchKernelGGL((conv3x3_bf16_kernel<MODE, E, SPLIT ? kWin3SplitPerCU : 3>), dim3((unsigned)blocks), dim3(NT), 0, stream, al, geo, ep, d);
         VDNN_LAUNCH_CHECK();
     }
     if (d.splits == 1) return VDNN_OK;
@@ -197,9 +204,9 @@ static int launch_win3x3(vdnn_ctx* ctx, hipStream_t stream, const PassNames& nam
 
 // what the windowed kernel needs: a 3x3 window at stride 1 with one pixel of padding (input and output planes of
 // one extent), rows of an even number of pixels, and tiles whose samples fit one descriptor
-static bool win3x3_ok(const int R, const int S, int ph, int pw, int sh, int sw, int Hs, int Ws, int OH, int OW, long sample_elems) {
+static bool win3x3_ok(const int R, const int S, int ph, int pw, int sh, int sw, int Hs, int Ws, int OH, int OW, long sample_elems, int elem_bytes = 2) {
     return R == 3 && S == 3 && ph == 1 && pw == 1 && sh == 1 && sw == 1 && Hs == OH && Ws == OW && Ws % 2 == 0 && Ws >= 2 &&
-           pixel_tile_span_ok(sample_elems, OH * OW, W3_TN, 2);
+           pixel_tile_span_ok(sample_elems, OH * OW, W3_TN, elem_bytes);
 }
 
 static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
@@ -560,7 +567,7 @@ static int conv_half_engine(vdnn_ctx* ctx, hipStream_t st, const PassNames& name
     // 3x3 at stride 1 with padding 1: one staged window per filter row serves its three taps
     if (win3x3_ok(pix.R, pix.S, pix.ph, pix.pw, pix.sh, pix.sw, pix.Hs, pix.Ws, pix.OH, pix.OW, pix.sample_elems)) {
         const Win3x3 geo{pix.src, pix.Hs, pix.Ws, pix.sample_elems, pix.sample_elems * pix.nsamples, pix.nsamples};
-        return launch_win3x3<MODE>(ctx, st, MODE == 0 ? kFwdWin3Names : kBwdDataWin3Names, al, geo, ep, rows, N, Cred * RS, flops, ctx->reduce_scratch_bytes - taken);
+        return launch_win3x3<MODE, bf16_t>(ctx, st, MODE == 0 ? kFwdWin3Names : kBwdDataWin3Names, al, geo, ep, rows, N, Cred * RS, flops, ctx->reduce_scratch_bytes - taken);
     }
     // a pixel pair per lane where the pairs of an output row are contiguous in the input
     if (pix.OW % 2 == 0 && pix.S <= 16 && pix.Ws >= pix.S && pix.Ws > pix.pw + 1 && (MODE == 1 || pix.sw == 1)) {
@@ -569,6 +576,44 @@ static int conv_half_engine(vdnn_ctx* ctx, hipStream_t st, const PassNames& name
     }
     LoadIm2colPixTapH<MODE> bl{pix};
     return launch_by_m<LoadPackedH, LoadIm2colPixTapH<MODE>, bf16_t, true>(ctx, st, names, al, bl, ep, rows, N, Cred * RS, flops, ctx->reduce_scratch_bytes - taken);
+}
+
+// ---- perf-optimal mode, float layers: 3x3 / stride 1 / padding 1 on the bfloat16 matrix cores ------------------
+// Every float operand as two bfloat16 parts, three matrix instructions per product (conv3x3_bf16.h): forward and
+// backward data through the windowed kernel, the split filter bank (as many bytes as the filter) in the workspace.
+// Which variant the perf-optimal mode takes where both apply: 0 = this one (faster on every VGG16 layer, closer to
+// the exact result, no transformed tensors), 1 = Winograd. vdnn_conv_perf_variant.
+static int g_perf_variant = 0;
+
+// MODE 0: rows = output channels, reduced = input channels; MODE 1: rows = input channels, reduced = output channels
+static bool split3x3_ok(const ConvGeo& g, int mode) {
+    const int reduced = mode == 0 ? g.C : g.K, rows = mode == 0 ? g.K : g.C;
+    const long sample = mode == 0 ? (long)g.C * g.H * g.W : (long)g.K * g.P * g.Q;
+    return reduced % 16 == 0 && g.C > 4 && (long)rows * reduced * 9 * 4 < (1l << 31) &&
+           win3x3_ok(g.R, g.S, g.ph, g.pw, g.sh, g.sw, g.H, g.W, g.P, g.Q, sample, 4);
+}
+
+template <int MODE>
+static int launch_split3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const float* src, const float* w, const StoreNCHW<float>& ep,
+                           void* workspace, size_t workspace_bytes, bool* taken) {
+    *taken = false;
+    const int rows = MODE == 0 ? g.K : g.C, reduced = MODE == 0 ? g.C : g.K;
+    const size_t bank = (size_t)rows * reduced * 9 * 4;
+    if (!split3x3_ok(g, MODE) || !workspace || workspace_bytes < bank || !aligned16(workspace)) return VDNN_OK;
+    *taken = true;
+    unsigned short* packed = (unsigned short*)workspace;
+    {
+        const long total = (long)rows * reduced * 9;
+        ProfScope prof(ctx, st, "conv_pack_filter", 0.0, 8.0 * (double)total);
+        hipLaunchKernelGGL(pack_filter_split_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, packed, rows, reduced, 9,
+                           MODE == 0 ? g.C * 9 : 9, MODE == 0 ? 9 : g.C * 9, total);
+        VDNN_LAUNCH_CHECK();
+    }
+    const long sample = MODE == 0 ? (long)g.C * g.H * g.W : (long)g.K * g.P * g.Q;
+    const LoadPackedH al{packed, (long)reduced * 18, rows, (unsigned)bank};
+    const Win3x3T<float> geo{src, g.H, g.W, sample, sample * g.N, g.N};
+    return launch_win3x3<MODE, float>(ctx, st, MODE == 0 ? kFwdSplitNames : kBwdDataSplitNames, al, geo, ep, rows, g.N * g.H * g.W, reduced * 18,
+                                      2.0 * g.N * (double)g.K * g.C * 9 * g.P * g.Q, ctx->reduce_scratch_bytes);
 }
 
 static int launch_pack_filter(vdnn_ctx* ctx, hipStream_t st, const float* w, float* packed, int rows, int Cred, int RS,
@@ -625,6 +670,54 @@ static int launch_wgrad3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, cons
         else if (narrow) hipLaunchKernelGGL((wgrad3x3_bf16_kernel<32, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
         else if (halfrow) hipLaunchKernelGGL((wgrad3x3_bf16_kernel<64, true>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
         else hipLaunchKernelGGL((wgrad3x3_bf16_kernel<64, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        VDNN_LAUNCH_CHECK();
+    }
+    if (with_bias) {
+        const int rc = launch_bias_grad_final(ctx, st, ctx->bias_scratch, bias->out, g.K, d.splits, bias->alpha, bias->accumulate);
+        if (rc != VDNN_OK) return rc;
+        bias->done = true;
+    }
+    if (d.splits > 1) return launch_reduce_splits_tap(ctx, st, w, staging, (size_t)M * N, d.splits, alpha, accumulate, g.C, 9);
+    return VDNN_OK;
+}
+
+// The perf-optimal float counterpart of launch_wgrad3x3 (wgrad3x3_split.h): the same tiles and splits, slices of 16 pixels.
+static int launch_wgrad3x3_split(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const float* x, const float* dy, float* w, float alpha, int accumulate,
+                                 float* staging, size_t staging_bytes, bool* taken, BiasOut* bias) {
+    *taken = false;
+    const int M = g.K, N = g.C * 9, PQ = g.H * g.W;
+    const long Kred = (long)g.N * PQ;
+    const bool narrow = M <= 64;
+    const int TM = narrow ? 64 : 128;
+    const int mtiles = (M + TM - 1) / TM, ntiles = 3 * (g.C / WG3_CH);
+    const long tiles = (long)mtiles * ntiles;
+    const size_t out_bytes = (size_t)M * N * sizeof(float);
+    const long slots = (long)kWgrad3PerCU * ctx->num_cu;
+    // as many rounds of workgroups as the tiles alone need, each filled by the splits
+    const long rounds = (tiles + slots - 1) / slots;
+    long splits = rounds * slots / tiles;
+    const long by_len = Kred / (16 * WG3S_SLICE); // at least sixteen slices per split
+    const long by_mem = staging ? (long)(staging_bytes / out_bytes) : 1;
+    if (splits > by_len) splits = by_len;
+    if (splits > by_mem) splits = by_mem;
+    if (splits < 1) splits = 1;
+    GemmDims d = make_dims(M, N, (int)Kred, TM, 3 * WG3_CH, (int)splits, WG3S_SLICE);
+    d.mtiles = mtiles; d.ntiles = ntiles;
+    const long nspan = d.kchunk / PQ + 2;
+    if (nspan * g.K * PQ * 4 >= (long)MAX_SUM_RANGE || nspan * g.C * PQ * 4 >= (long)MAX_SUM_RANGE) return VDNN_OK; // not taken
+    if (d.splits > 1 && !staging) return VDNN_OK;
+    const long blocks = tiles * d.splits;
+    if (blocks <= 0 || blocks >= (1l << 31)) return VDNN_OK;
+    *taken = true;
+    const bool with_bias = bias && bias->wanted() && bias_parts_fit(ctx, g.K, d.splits);
+    const Wgrad3x3S geo{dy, x, g.N, g.K, g.C, g.H, g.W, w, staging, (long)M * N, alpha, accumulate, with_bias ? ctx->bias_scratch : nullptr, d.splits};
+    {
+        ProfScope prof(ctx, st, narrow ? "conv_bwd_filter_split_64x192" : "conv_bwd_filter_split_128x192", 2.0 * M * (double)N * (double)Kred, 0.0);
+        const bool halfrow = g.W % 8 != 0; // groups of eight pixels across two image rows
+        if (narrow && halfrow) hipLaunchKernelGGL((wgrad3x3_split_kernel<32, true>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        else if (narrow) hipLaunchKernelGGL((wgrad3x3_split_kernel<32, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        else if (halfrow) hipLaunchKernelGGL((wgrad3x3_split_kernel<64, true>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
+        else hipLaunchKernelGGL((wgrad3x3_split_kernel<64, false>), dim3((unsigned)blocks), dim3(NT), 0, st, geo, d);
         VDNN_LAUNCH_CHECK();
     }
     if (with_bias) {
@@ -788,8 +881,13 @@ static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
     if (fwd_smallc3x3_ok(g, sizeof(E))) return launch_fwd_smallc3x3<E>(ctx, st, g, x, w, bias, y, relu);
     if constexpr (sizeof(E) == 4) {
         if (algo_mode == 1) {
-            // perf-optimal: wide 3x3 layers as Winograd F(4x4, 3x3) through the workspace
+            // perf-optimal: 3x3 layers on the bfloat16 matrix cores, or as Winograd F(4x4, 3x3), through the workspace
             bool taken = false;
+            if (g_perf_variant == 0) {
+                const StoreNCHW<float> eps{y, bias, g.P * g.Q, ctx->reduce_scratch, relu, nullptr};
+                const int rc = launch_split3x3<0>(ctx, st, g, x, w, eps, workspace, workspace_bytes, &taken);
+                if (taken || rc != VDNN_OK) return rc;
+            }
             const int rc = launch_winograd(ctx, st, g, false, x, w, bias, y, relu, nullptr, workspace, workspace_bytes, &taken);
             if (taken || rc != VDNN_OK) return rc;
         }
@@ -924,6 +1022,11 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
     if constexpr (sizeof(E) == 4) {
         if (algo_mode == 1) {
             bool taken = false;
+            if (g_perf_variant == 0) {
+                const StoreNCHW<float> eps{dx, nullptr, g.H * g.W, ctx->reduce_scratch, 0, gate};
+                const int rc = launch_split3x3<1>(ctx, st, g, dy, w, eps, workspace, workspace_bytes, &taken);
+                if (taken || rc != VDNN_OK) return rc;
+            }
             const int rc = launch_winograd(ctx, st, g, true, dy, w, nullptr, dx, 0, gate, workspace, workspace_bytes, &taken);
             if (taken || rc != VDNN_OK) return rc;
         }
@@ -988,8 +1091,16 @@ static int conv_bwd_filter_core(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_
     VDNN_REQUIRE((long)(PQ + KB) * PQ < (1l << 32), "output plane too large for the pixel cursor's exact division");
     if constexpr (sizeof(E) == 4) {
         if (algo_mode == 1) {
-            // perf-optimal: wide 3x3 layers as Winograd F(3x3, 4x4) through the workspace
+            // perf-optimal: 3x3 layers on the bfloat16 matrix cores (partial sums in the staging area, or in the workspace
+            // if that is larger), or as Winograd F(3x3, 4x4) through the workspace
             bool taken = false;
+            if (g_perf_variant == 0 && wgrad3x3_ok(g)) {
+                float* staging = ctx->reduce_scratch;
+                size_t staging_bytes = ctx->reduce_scratch_bytes;
+                if (workspace && workspace_bytes > staging_bytes && aligned16(workspace)) { staging = (float*)workspace; staging_bytes = workspace_bytes; }
+                const int rcs = launch_wgrad3x3_split(ctx, st, g, x, dy, w, alpha, accumulate, staging, staging_bytes, &taken, bias);
+                if (taken || rcs != VDNN_OK) return rcs;
+            }
             const int rc = launch_winograd_wgrad(ctx, st, g, x, dy, w, alpha, accumulate, workspace, workspace_bytes, &taken, bias);
             if (taken || rc != VDNN_OK) return rc;
         }
@@ -1242,6 +1353,12 @@ size_t vdnn_conv_winograd_chunk_bytes(size_t bytes) {
     return before;
 }
 
+int vdnn_conv_perf_variant(int variant) {
+    const int before = g_perf_variant;
+    if (variant == 0 || variant == 1) g_perf_variant = variant;
+    return before;
+}
+
 size_t vdnn_conv_workspace_bytes(const vdnn_shape_t* shape, int algo_mode, int pass) {
     return vdnn_conv_workspace_bytes_dtype(shape, algo_mode, pass, VDNN_DTYPE_F32);
 }
@@ -1255,11 +1372,13 @@ size_t vdnn_conv_workspace_bytes_dtype(const vdnn_shape_t* shape, int algo_mode,
     // for 128-bit operand loads; backward filter takes a staging area large enough for the split count that fills the chip.
     const int RS = g.R * g.S;
     const size_t filter_bytes = (size_t)g.K * g.C * RS * sizeof(float);
+    if (dtype == VDNN_DTYPE_F32 && pass != 2 && g_perf_variant == 0 && split3x3_ok(g, pass)) return filter_bytes;
     if (dtype == VDNN_DTYPE_F32 && pass != 2 && wino_ok(g, pass == 1)) {
         const WinoPlan p = wino_plan(g, pass == 1);
         if (wino_plan_ok(p)) return p.total;
     }
-    if (dtype == VDNN_DTYPE_F32 && pass == 2 && wino_wgrad_ok(g)) {
+    const bool split_wgrad = dtype == VDNN_DTYPE_F32 && pass == 2 && g_perf_variant == 0 && wgrad3x3_ok(g);
+    if (dtype == VDNN_DTYPE_F32 && pass == 2 && !split_wgrad && wino_wgrad_ok(g)) {
         const WinoWgradPlan p = wino_wgrad_plan(g);
         if (wino_wgrad_plan_ok(p, g)) return p.total;
     }

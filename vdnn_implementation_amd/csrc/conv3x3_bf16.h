@@ -18,6 +18,17 @@
 // Same results as the general engine up to the order of summation inside the matrix cores (none: both sum a
 // slice's 32 products in the instruction and the slices in the same order), same epilogues, same split and
 // tail modes (the reduction is cut at multiples of one filter row: 96).
+//
+// Float layers (E = float), the perf-optimal mode's kernel: every float operand is the sum of two bfloat16 values up to
+// 2^-17 of itself - hi = bf16(v), lo = bf16(v - hi), both rounded to nearest - and a product is taken as
+// hi*hi + hi*lo + lo*hi on the bfloat16 matrix cores, accumulated in float: three instructions of the 16x faster kind
+// for one of the float kind, with a relative error of about 2^-16 per product (the dropped lo*lo term and the two
+// remainders), which random signs average down like the rounding of the float instruction's own sums. A slice is then
+// 16 channels of one tap, an LDS row holds [hi of 16 channels | lo of 16 channels] where the bfloat16 layers hold 32
+// channels, the filter bank comes split the same way (pack_filter_split_kernel) and the "halves" of a slice are its
+// hi and lo parts: same pipeline, same LDS traffic and barriers per step, twelve matrix instructions per step
+// instead of eight. The window is fetched as 64-bit pixel pairs and split when it is written to LDS, two row
+// steps after its fetch. An infinite input gives NaN (inf - inf in lo) where the float kernels give an infinity.
 #pragma once
 #include <type_traits>
 #include "mfma_bf16.h"
@@ -32,16 +43,48 @@ constexpr int W3_DEPTH = 3 * KH;      // reduction indices of one filter row of 
 // MODE 0: forward, src = x, the window of filter row r lies (r - 1) rows below the pixel, tap s reads one column
 // further right per s. MODE 1: backward data, src = dy, filter row r lies (1 - r) rows away and tap s reads one
 // column further left per s.
-struct Win3x3 {
-    const bf16_t* src;
+template <class E>
+struct Win3x3T {
+    const E* src;
     int H, W;            // extent of a plane (input and output planes agree)
     long sample_elems;   // reduced channels * H * W
     long total_elems;    // samples * sample_elems
     int nsamples;
 };
+typedef Win3x3T<bf16_t> Win3x3;
 
-template <int MODE>
-__global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH al, const Win3x3 geo, const StoreNCHW<bf16_t> ep, const GemmDims d) {
+// Filter bank of a float layer split into bfloat16 parts for the kernel below: 16-channel blocks, tap-major,
+// packed[row][((cb*RS + tap)*2 + part)*16 + l] = part of w[row*row_stride + (cb*16 + l)*red_stride + tap], part 0 = hi, 1 = lo
+// (row_stride / red_stride as in pack_filter_tap_bf16_kernel). One thread per filter element.
+static __global__ void __launch_bounds__(256) pack_filter_split_kernel(const float* __restrict__ w, unsigned short* __restrict__ packed,
+                                                                int rows, int Cred, int RS, int row_stride, int red_stride, long total) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int per_row = Cred * RS;
+    const int row = (int)(i / per_row), kk = (int)(i - (long)row * per_row);
+    const int l = kk & 15, slice = kk >> 4;
+    const int cb = slice / RS, tap = slice - cb * RS;
+    const float v = w[(long)row * row_stride + (long)(cb * 16 + l) * red_stride + tap];
+    const unsigned short hi = float_to_bf16_bits(v);
+    const unsigned short lo = float_to_bf16_bits(v - __builtin_bit_cast(float, (unsigned)hi << 16));
+    unsigned short* at = packed + (long)row * per_row * 2 + (long)slice * 32 + l;
+    at[0] = hi; at[16] = lo;
+}
+
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+// (hi, lo) parts of two floats, each pair packed into one word (first value in the low half)
+__device__ __forceinline__ void split_pair(float a, float b, unsigned& hi, unsigned& lo) {
+    hi = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{a, b}, bf16x2));
+    const float ha = __builtin_bit_cast(float, hi << 16), hb = __builtin_bit_cast(float, hi & 0xFFFF0000u);
+    lo = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{a - ha, b - hb}, bf16x2));
+}
+
+template <int MODE, class E = bf16_t, int RESIDENT = 3>
+__global__ void __launch_bounds__(NT, RESIDENT) conv3x3_bf16_kernel(const LoadPackedH al, const Win3x3T<E> geo, const StoreNCHW<E> ep, const GemmDims d) {
+    constexpr bool SPLIT = std::is_same<E, float>::value;
+    constexpr int EB = (int)sizeof(E);
+    constexpr int CH = SPLIT ? 16 : KH;  // channels of a slice
     // 64 rows x 256 pixels per workgroup, a 64 x 64 tile per wavefront: 64 accumulator registers, three workgroups
     // resident per compute unit. (A 128 x 256 tile with 64 x 128 per wavefront - three LDS fragment reads per four
     // MFMAs instead of four, half the window traffic and barriers per MFMA, two workgroups per compute unit - measured
@@ -80,7 +123,7 @@ __global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH a
     // the descriptor starts W + 2 elements ahead of the first sample (a four-byte boundary: W is even) so that
     // every offset below is non-negative, and ends with the last sample the tile touches
     const long first = (long)n_first * geo.sample_elems;
-    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(geo.src + first - (W + 2), clamp_range(((long)(n_last - n_first + 1) * geo.sample_elems + (W + 2)) * 2));
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(geo.src + first - (W + 2), clamp_range(((long)(n_last - n_first + 1) * geo.sample_elems + (W + 2)) * EB));
 
     // ---- filter operand: rows tid/4 + 64 i, eight reduction values at 8 (tid%4) ------------------------
     // Two filter tiles are in flight: the one of step g + 2, about to be written to LDS, and the one of step g + 3,
@@ -99,7 +142,7 @@ __global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH a
         const int jj = valid ? j : j0;
         const int n = jj / plane, pix = jj - n * plane;
         const int p = pix / W;
-        voff = valid ? (int)(((long)(n - n_first) * geo.sample_elems + pix) * 2) : OOB;
+        voff = valid ? (int)(((long)(n - n_first) * geo.sample_elems + pix) * EB) : OOB;
         rowinv = 0;
 #pragma unroll
         for (int r = 0; r < 3; r++) {
@@ -107,19 +150,20 @@ __global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH a
             if (!((unsigned)ih < (unsigned)geo.H)) rowinv |= 1u << r;
         }
     }
-    // the two elements beside the tile, for 32 channels: lanes of wavefront 0, side = lane / 32, channel = lane % 32.
+    // the two elements beside the tile, for the slice's channels: lanes of wavefront 0, side = lane / CH, channel = lane % CH.
     // The left one is needed (and inside the image row) when the tile's first pixel is not the first of its row,
     // the right one when the tile's last pixel is not the last of its row.
     int hoff = OOB;
     unsigned hrowinv = 0;
-    if (wave == 0) {
-        const int side = lane >> 5, ch = lane & 31;
+    const bool halo_lane = wave == 0 && lane < 2 * CH;
+    if (halo_lane) {
+        const int side = lane / CH, ch = lane % CH;
         const int j = side ? j0 + W3_TN - 1 : j0;
         if (j < d.N) {
             const int n = j / plane, pix = j - n * plane;
             const int p = pix / W, q = pix - p * W;
             const bool needed = side ? q < W - 1 : q > 0;
-            if (needed) hoff = (int)(((long)(n - n_first) * geo.sample_elems + (long)ch * plane + pix + (side ? 1 : -1)) * 2);
+            if (needed) hoff = (int)(((long)(n - n_first) * geo.sample_elems + (long)ch * plane + pix + (side ? 1 : -1)) * EB);
 #pragma unroll
             for (int r = 0; r < 3; r++) {
                 const int ih = MODE == 0 ? p + r - 1 : p + 1 - r;
@@ -147,7 +191,10 @@ __global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH a
 
     // Two windows are in flight: the one fetched for the row step after the next, and the one for the step after
     // that. [item][pixel of the pair]: eight channels each, ready for LDS; the halo element of this lane (wavefront 0).
-    struct Fetched { uintx4 wr[2][2]; unsigned hr; };
+    // Float layers: one item, [channel][pixel of the pair] as fetched, split when it is stored.
+    struct FetchedH { uintx4 wr[2][2]; unsigned hr; };
+    struct FetchedF { floatx2 raw[8]; float hr; };
+    typedef typename std::conditional<SPLIT, FetchedF, FetchedH>::type Fetched;
     Fetched fa, fb;
     fa.hr = 0; fb.hr = 0;
     const int g0 = __builtin_amdgcn_readfirstlane(tid >> 7); // channel group of the thread's first item: uniform per wavefront
@@ -158,6 +205,13 @@ __global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH a
         const int cb = row_step / 3, r = row_step - cb * 3;
         const int rowoff = MODE == 0 ? (r - 1) * W : (1 - r) * W;
         const int vo = voff | bit_to_all_ones(rowinv, r);
+        if constexpr (SPLIT) {
+            const int ch = cb * CH + 8 * g0;
+            const int soff = (ch * plane + rowoff + W + 2) * 4, step = plane * 4;
+#pragma unroll
+            for (int e = 0; e < 8; e++) f.raw[e] = __builtin_bit_cast(floatx2, __builtin_amdgcn_raw_buffer_load_b64(rsrc, vo, soff + e * step, 0));
+            if (halo_lane) f.hr = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, hoff | bit_to_all_ones(hrowinv, r), (cb * CH * plane + rowoff + W + 2) * 4, 0));
+        } else {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             const int ch = cb * KH + 8 * (g0 + 2 * i);
@@ -177,18 +231,44 @@ __global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH a
             const int soff = (cb * KH * plane + rowoff + W + 2) * 2;
             f.hr = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc, hoff | bit_to_all_ones(hrowinv, r), soff, 0);
         }
+        }
     };
     // A lane's two pixels are neighbouring LDS rows, lane after lane two rows on: sixteen lanes storing their first
     // pixels would meet only eight of the sixteen groups of four banks (160 bytes from lane to lane). Lanes 8-15 of
     // every sixteen therefore store their second pixel first: odd rows, the other eight groups (a third fewer
     // bank-conflict cycles in the kernel as a whole).
     auto store_window = [&](unsigned short* lds, const Fetched& f) {
+        if constexpr (SPLIT) {
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                // the pixel stored by instruction e: the lane's pixel e ^ swapped
+                uintx4 hi, lo;
+                unsigned h[4], l[4];
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const float a = (e ^ swapped) ? f.raw[2 * k].y : f.raw[2 * k].x, b = (e ^ swapped) ? f.raw[2 * k + 1].y : f.raw[2 * k + 1].x;
+                    split_pair(a, b, h[k], l[k]);
+                }
+                hi.x = h[0]; hi.y = h[1]; hi.z = h[2]; hi.w = h[3];
+                lo.x = l[0]; lo.y = l[1]; lo.z = l[2]; lo.w = l[3];
+                unsigned short* at = lds + (1 + 2 * (tid & 127) + (e ^ swapped)) * HSTRIDE + 8 * (tid >> 7);
+                *(uintx4*)at = hi;
+                *(uintx4*)(at + 16) = lo;
+            }
+            if (halo_lane) {
+                unsigned h, l;
+                split_pair(f.hr, 0.0f, h, l);
+                unsigned short* at = lds + ((lane / CH) ? W3_ROWS - 1 : 0) * HSTRIDE + (lane % CH);
+                at[0] = (unsigned short)h; at[16] = (unsigned short)l;
+            }
+        } else {
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int e = 0; e < 2; e++)
                 *(uintx4*)(lds + (1 + 2 * (tid & 127) + (e ^ swapped)) * HSTRIDE + 8 * ((tid >> 7) + 2 * i)) = f.wr[i][e];
         if (wave == 0) lds[((lane >> 5) ? W3_ROWS - 1 : 0) * HSTRIDE + (lane & 31)] = (unsigned short)f.hr;
+        }
     };
 
     floatx16 acc[NJ / 2][2][2]; // [64-column half][row block][column block]
@@ -241,10 +321,13 @@ __global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH a
     load_window(row_begin + 1, fb);
     load_window(row_begin + 2, fa);
     __syncthreads();
-    bf16x8 a0[2], a1[2];
-    uintx4 b0[NJ], b1[NJ];
-    read_a(As[0], 0, a0);
-    read_b(Bw[0], 0, 0, b0);
+    // Float layers multiply hi x hi in the first half of a step and hi x lo + lo x hi in the second, while the next step's
+    // hi fragments arrive: those take turns in two sets of registers.
+    // (the lo fragments read a step ahead as well, so that the first half only writes to LDS: measured the same)
+    bf16x8 a0[SPLIT ? 2 : 1][2], a1[2];
+    uintx4 b0[SPLIT ? 2 : 1][NJ], b1[NJ];
+    read_a(As[0], 0, a0[0]);
+    read_b(Bw[0], 0, 0, b0[0]);
     // one row step; `f` holds the window of the next row step (fetched two row steps ago): it is written to LDS in the
     // first half of the last tap, and the registers then take the fetch of the window three row steps ahead. `odd`: the
     // parity of the row step counted from row_begin, which fixes the parity of g (the filter registers of a step)
@@ -255,9 +338,10 @@ __global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH a
         for (int s = 0; s < 3; s++) {
             const int g = (row_step - row_begin) * 3 + s;
             const int cur = (3 * ODD + s) & 1, nxt = cur ^ 1; // = g & 1
+            const int rc = SPLIT ? cur : 0, rn = SPLIT ? nxt : 0;
             read_a(As[cur], 1, a1);
             read_b(Bw[wb], s, 1, b1);
-            multiply(a0, b0);
+            multiply(a0[rc], b0[rc]);
             LoadPackedH::template store<TM>(As[nxt], tid, ra[(3 * ODD + s + 1) & 1]);
             if (s == 2) store_window(Bw[wb ^ 1], f);
             // issue order of the first half: an LDS access behind every MFMA
@@ -266,12 +350,13 @@ __global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH a
             __syncthreads();
             al.template load<TM>(sa, row_begin * W3_DEPTH + (g + 3) * KH, k_end, tid, ra[(3 * ODD + s + 1) & 1]);
             if (s == 2) load_window(row_step + 3, f);
-            read_a(As[nxt], 0, a0);
-            read_b(s == 2 ? Bw[wb ^ 1] : Bw[wb], s == 2 ? 0 : s + 1, 0, b0);
-            multiply(a1, b1);
+            read_a(As[nxt], 0, a0[rn]);
+            read_b(s == 2 ? Bw[wb ^ 1] : Bw[wb], s == 2 ? 0 : s + 1, 0, b0[rn]);
+            if constexpr (SPLIT) { multiply(a0[rc], b1); multiply(a1, b0[rc]); }
+            else multiply(a1, b1);
             // second half: a memory instruction and an LDS read behind every MFMA
 #pragma unroll
-            for (int i = 0; i < 2 * NJ; i++) {
+            for (int i = 0; i < (SPLIT ? 4 : 2) * NJ; i++) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
@@ -287,7 +372,7 @@ __global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH a
     // applied, rounded to bfloat16) and writes it eight pixels - 16 bytes - per lane, gated by eight elements of the gate
     // tensor fetched the same way; lane by lane the block would leave in two-byte stores of 64-byte runs. Same values.
     // Needs planes of whole groups of eight pixels (a group stays in its sample) and 16-byte aligned tensors.
-    if (whole && ep.opix % 8 == 0 && (((uintptr_t)ep.out | (uintptr_t)ep.gate) & 15) == 0) {
+    if constexpr (!SPLIT) if (whole && ep.opix % 8 == 0 && (((uintptr_t)ep.out | (uintptr_t)ep.gate) & 15) == 0) {
         static_assert(NJ == 2 && WM == 1, "one 64 x 64 block per wavefront");
         constexpr int STG = 72; // row stride of the block in LDS, 16-bit units
         static_assert(4 * 64 * STG <= 2 * W3_ROWS * HSTRIDE, "the four blocks fit the window buffers");
@@ -345,7 +430,7 @@ __global__ void __launch_bounds__(NT, 3) conv3x3_bf16_kernel(const LoadPackedH a
     }
 #pragma unroll
     for (int q = 0; q < NJ / 2; q++) {
-        if (StoreNCHW<bf16_t>::TAIL && d.full_tiles > 0 && !whole)
+        if (StoreNCHW<E>::TAIL && d.full_tiles > 0 && !whole)
             ep.store_tail(acc[q], wm0, wn0 + 64 * q, lane, (long)(tile - d.full_tiles) * d.splits + ks, TM, W3_TN);
         else
             ep.store(acc[q], m0 + wm0, j0 + wn0 + 64 * q, lane, ks, d, !whole);
