@@ -55,6 +55,8 @@ SWEEP_POLICIES = ",".join([
     "BASELINE+bf16+fused", "VDNN_ALL+refined+ahead+bf16+fused+zvc", "VDNN_ALL+refined+bf16+fused+zvc+keep",
     "VDNN_ALL+refined+bf16+fused+zvc+budget5.9", "VDNN_ALL+refined+bf16+fused+zvc+keep+inplace+recompute",
     "VDNN_ALL+refined+bf16+fused+zvc+inplace+recompute+budget5.0", "VDNN_ALL+refined+bf16+fused+zvc+inplace+recompute+budget6.0",
+    "BASELINE+perf", "BASELINE+fused+perf", "BASELINE+wino", "VDNN_ALL+perf", "VDNN_ALL+refined+fused+zvc+budget3.0+perf",
+    "VDNN_ALL+refined+fused+zvc+inplace+recompute+budget4.0+perf",
 ])
 
 

@@ -65,10 +65,12 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_split_kernel(const Wgrad3x3S g
     const __amdgpu_buffer_rsrc_t rsA = make_rsrc(g.dy + (long)n_first * g.K * PQ, clamp_range((long)(n_last - n_first + 1) * g.K * PQ * 4));
     const __amdgpu_buffer_rsrc_t rsB = make_rsrc(g.x + (long)n_first * g.C * PQ, clamp_range((long)(n_last - n_first + 1) * g.C * PQ * 4));
 
-    // loader state: this thread's group of eight pixels of the slice and its row of the operands. Rows of dy: all
-    // threads (TM = 128) or the first half (TM = 64); rows of x: the first half (wavefronts 0 and 1).
-    const int pg = tid & 1, rl = tid >> 1;
-    const bool loads_a = rl < TM, loads_b = wave < 2;
+    // loader state: this thread's group of eight pixels of the slice and its row of the operands. TM = 128: rows of dy by
+    // all threads, rows of x by wavefronts 0 and 1, the two neighbouring elements by wavefronts 2 and 3. TM = 64: rows
+    // of dy by wavefronts 0 and 1, rows of x by wavefronts 2 and 3 (so that every wavefront splits one operand), the
+    // neighbouring elements by wavefronts 0 and 1.
+    const int pg = tid & 1, rl = tid >> 1, rlb = rl & 63;
+    const bool loads_a = rl < TM, loads_b = TM == 64 ? wave >= 2 : wave < 2;
     const int mrow = (loads_a && m0 + rl < g.K) ? (m0 + rl) * PQ * 4 : SENT;
     int pqA, offA, pB, qB, posB;
     {
@@ -79,9 +81,9 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_split_kernel(const Wgrad3x3S g
         pB = pq / W; qB = pq - pB * W;
         posB = (int)(((long)(n - n_first) * g.C * PQ + pq) * 4);
     }
-    const int colB = ((c0 + (rl & 63)) * PQ + (r - 1) * W) * 4; // the channel's plane and the filter row's shift
-    // wavefronts 2 and 3 also fetch the element before (after) the slice's run, one channel per lane
-    const bool loads_h = wave >= 2;
+    const int colB = ((c0 + rlb) * PQ + (r - 1) * W) * 4; // the channel's plane and the filter row's shift
+    // the element before (after) the slice's run, one channel per lane
+    const bool loads_h = TM == 64 ? wave < 2 : wave >= 2;
     const int side = wave & 1;
     int pH, qH, posH;
     {
@@ -152,7 +154,7 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_split_kernel(const Wgrad3x3S g
         if (loads_b) {
             uintx4 hi, lo;
             split8(f.rb, hi, lo);
-            unsigned short* at = Bs[buf] + rl * HSTRIDE + 8 * pg;
+            unsigned short* at = Bs[buf] + rlb * HSTRIDE + 8 * pg;
             *(uintx4*)at = hi; *(uintx4*)(at + 16) = lo;
         }
         if (loads_h) {
