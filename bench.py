@@ -369,6 +369,7 @@ def main():
                    "gbs": (v["bytes"] / (v["ms"] * 1e-3) / 1e9) if v["bytes"] else None}
                for k, v in sorted(prof.items(), key=lambda kv: -kv[1]["ms"])}
     fp32 = {k: v for k, v in results.items() if not (args.bf16 or is_bf16(k))}
+    same_sums = {k: v for k, v in fp32.items() if perf_kind(k) == perf_kind(head)}   # the headline's algorithm mode: its losses, bit for bit
     ratio = (results[head]["images_per_s"] / base["images_per_s"]) if base and head != "BASELINE" else None
 
     def brief(b):
@@ -397,13 +398,14 @@ def main():
         "conv_mfma_util": conv_all_tf / peak if conv_all_tf else None,
         # float only, same losses as the literal run bit for bit: the fastest VDNN configuration at >= 3x less memory than
         # BASELINE, and the fastest of those that move at least 0.5 GB over the link each way
-        "best_fp32_at_3x": brief(best_within(fp32, base, 3.0, False)),
-        "best_fp32_at_3x_over_the_link": brief(best_within(fp32, base, 3.0, True)),
+        "best_fp32_at_3x": brief(best_within(same_sums, base, 3.0, False)),
+        "best_fp32_at_3x_over_the_link": brief(best_within(same_sums, base, 3.0, True)),
     }
     details = {
         "policies": results, "kernels": kernels,
         "least_memory_fp32_at_85pct": smallest_within(fp32, base, 0.85),
         "best_any_dtype_at_3x": best_within(results, base, 3.0, False),
+        "best_fp32_any_mode_at_3x": best_within(fp32, base, 3.0, False),   # (the perf-optimal rows sum in another order)
         "baseline_peak_gb_replayed": baseline_peak / 1e9,
         "step_mfma_frac": args.batch * FLOP_PER_IMAGE / (results[head]["ms_per_step"] * 1e-3) / 1e12 / peak if args.cnn == "VGG16" else None,
     }
