@@ -323,7 +323,10 @@ __global__ void __launch_bounds__(NT, RESIDENT) conv3x3_bf16_kernel(const LoadPa
     __syncthreads();
     // Float layers multiply hi x hi in the first half of a step and hi x lo + lo x hi in the second, while the next step's
     // hi fragments arrive: those take turns in two sets of registers.
-    // (the lo fragments read a step ahead as well, so that the first half only writes to LDS: measured the same)
+    // (Measured within 1 % of this, same box and run: the lo fragments read a step ahead as well, so that the first half
+    // only writes to LDS; three windows in flight; three workgroups per compute unit at 18 spilled registers. A barrier
+    // per row step instead of per tap - the three filter tiles of a row step in buffers of their own, 72 KB of LDS -
+    // gained 3 % on the 28 x 28 layers and nothing elsewhere.)
     bf16x8 a0[SPLIT ? 2 : 1][2], a1[2];
     uintx4 b0[SPLIT ? 2 : 1][NJ], b1[NJ];
     read_a(As[0], 0, a0[0]);
