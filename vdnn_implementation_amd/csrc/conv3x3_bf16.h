@@ -198,7 +198,7 @@ __global__ void __launch_bounds__(NT, RESIDENT) conv3x3_bf16_kernel(const LoadPa
     Fetched fa, fb;
     fa.hr = 0; fb.hr = 0;
     const int g0 = __builtin_amdgcn_readfirstlane(tid >> 7); // channel group of the thread's first item: uniform per wavefront
-    const int swapped = (tid >> 3) & 1;                      // this lane stores its second pixel first
+    const int swapped = (tid >> 2) & 1;                      // this lane stores its second pixel first
     const unsigned sel_first = swapped ? 0x07060302u : 0x05040100u, sel_second = swapped ? 0x05040100u : 0x07060302u;
 
     auto load_window = [&](int row_step, Fetched& f) {
@@ -233,10 +233,10 @@ __global__ void __launch_bounds__(NT, RESIDENT) conv3x3_bf16_kernel(const LoadPa
         }
         }
     };
-    // A lane's two pixels are neighbouring LDS rows, lane after lane two rows on: sixteen lanes storing their first
-    // pixels would meet only eight of the sixteen groups of four banks (160 bytes from lane to lane). Lanes 8-15 of
-    // every sixteen therefore store their second pixel first: odd rows, the other eight groups (a third fewer
-    // bank-conflict cycles in the kernel as a whole).
+    // A lane's two pixels are neighbouring LDS rows, lane after lane two rows on (160 bytes = 40 words): the eight lanes
+    // that LDS takes together (rows_by_four_lanes in mfma_bf16.h) would meet on banks 0, 8, 16, 24 twice each. Lanes 4-7 of
+    // every eight therefore store their second pixel first: odd rows, 20 words on, the other four groups of banks
+    // (a 128-bit store of a wavefront: 8 cycles instead of 16, measured on the pattern alone).
     auto store_window = [&](unsigned short* lds, const Fetched& f) {
         if constexpr (SPLIT) {
 #pragma unroll

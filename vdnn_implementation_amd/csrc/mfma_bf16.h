@@ -19,8 +19,23 @@ constexpr int HSTRIDE = 40; // LDS row stride in 16-bit units
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 
+// LDS takes a 128-bit store eight lanes at a time, on 32 banks of four bytes (measured: 8 cycles per store when the
+// eight lanes' 32 words fall on 32 different banks, 16 otherwise). With rows of HSTRIDE = 40 halfwords (20 words)
+// four lanes per 64-byte row and two consecutive rows per eight lanes meet on four banks (20 + 12 = 32 = 0); rows
+// r and r + 4 (80 words = 16 mod 32) tile the banks. So the four lanes t%4 of a row take the rows in the order
+// 0 4 1 5 2 6 3 7 of every eight: which thread fetches which row is free.
+__device__ __forceinline__ int rows_by_four_lanes(int tid) {
+    const int b = tid >> 2;
+    return (b & ~7) | ((b & 1) << 2) | ((b >> 1) & 3);
+}
+// The same for two lanes per row (a 16-byte piece each, rows of 20 words): rows 0 2 4 6 1 3 5 7 of every eight.
+__device__ __forceinline__ int rows_by_two_lanes(int tid) {
+    const int b = tid >> 1;
+    return (b & ~7) | ((b & 3) << 1) | ((b >> 2) & 1);
+}
+
 // ---- dense bfloat16 reduction-major operand: element (row, kk) at base[row*ld + kk] --------------------
-// thread t: values 8*(t%4) .. +7 of rows t/4 + 64*i, one 128-bit load each
+// thread t: values 8*(t%4) .. +7 of rows rows_by_four_lanes(t) + 64*i, one 128-bit load each
 struct LoadPackedH {
     const unsigned short* base;
     long ld;        // elements between rows (a multiple of 8)
@@ -33,7 +48,7 @@ struct LoadPackedH {
         st.rsrc = make_rsrc(base, bytes);
 #pragma unroll
         for (int i = 0; i < T / 64; i++) {
-            const int row = row0 + (tid >> 2) + 64 * i;
+            const int row = row0 + rows_by_four_lanes(tid) + 64 * i;
             st.vrow[i] = row < rows ? (int)(((long)row * ld + 8 * (tid & 3)) * 2) : OOB;
         }
     }
@@ -46,7 +61,7 @@ struct LoadPackedH {
     template <int T>
     __device__ static __forceinline__ void store(unsigned short* lds, int tid, const Regs<T>& r) {
 #pragma unroll
-        for (int i = 0; i < T / 64; i++) *(uintx4*)(lds + ((tid >> 2) + 64 * i) * HSTRIDE + 8 * (tid & 3)) = r.v[i];
+        for (int i = 0; i < T / 64; i++) *(uintx4*)(lds + (rows_by_four_lanes(tid) + 64 * i) * HSTRIDE + 8 * (tid & 3)) = r.v[i];
     }
 };
 

@@ -75,7 +75,7 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_bf16_kernel(const Wgrad3x3 g, 
     const __amdgpu_buffer_rsrc_t rsB = make_rsrc(g.x + (long)n_first * g.C * PQ, clamp_range((long)(n_last - n_first + 1) * g.C * PQ * 2));
 
     // loader state: this thread's pixel group of the slice (eight pixels) and its row of the operands
-    const int pg = tid & 3, rl = tid >> 2;
+    const int pg = tid & 3, rl = rows_by_four_lanes(tid); // (the order of the rows over the lanes: no LDS bank conflicts in the stores)
     int mrow[AL];
 #pragma unroll
     for (int i = 0; i < AL; i++) { const int m = m0 + rl + 64 * i; mrow[i] = m < g.K ? m * PQ * 2 : SENT; }

@@ -69,7 +69,7 @@ __global__ void __launch_bounds__(NT, 2) wgrad3x3_split_kernel(const Wgrad3x3S g
     // all threads, rows of x by wavefronts 0 and 1, the two neighbouring elements by wavefronts 2 and 3. TM = 64: rows
     // of dy by wavefronts 0 and 1, rows of x by wavefronts 2 and 3 (so that every wavefront splits one operand), the
     // neighbouring elements by wavefronts 0 and 1.
-    const int pg = tid & 1, rl = tid >> 1, rlb = rl & 63;
+    const int pg = tid & 1, rl = rows_by_two_lanes(tid), rlb = rl & 63; // (that order of the rows: no LDS bank conflicts in the stores)
     const bool loads_a = rl < TM, loads_b = TM == 64 ? wave >= 2 : wave < 2;
     const int mrow = (loads_a && m0 + rl < g.K) ? (m0 + rl) * PQ * 4 : SENT;
     int pqA, offA, pB, qB, posB;
