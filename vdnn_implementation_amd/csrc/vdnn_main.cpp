@@ -70,6 +70,7 @@ int main(int argc, char** argv) {
         else if (!strcmp(argv[i], "--bf16")) opt.dataType = VDNN_DTYPE_BF16;
         else if (!strcmp(argv[i], "--offload-lag")) opt.offloadLag = atoi(need("--offload-lag needs a value"));
         else if (!strcmp(argv[i], "--prefetch-depth")) opt.prefetchDepth = atoi(need("--prefetch-depth needs a value"));
+        else if (!strcmp(argv[i], "--winograd")) vdnn_conv_perf_variant(1); /* VDNN_PERF_OPT_ALGO: Winograd where the default variant and it both apply */
         else if (!strcmp(argv[i], "--verbose")) opt.verbose = true;
         else M_ASSERT(0, "unknown flag");
     }
