@@ -213,24 +213,24 @@ __global__ void __launch_bounds__(NT, RESIDENT) conv3x3_bf16_kernel(const LoadPa
             if (halo_lane) f.hr = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, hoff | bit_to_all_ones(hrowinv, r), (cb * CH * plane + rowoff + W + 2) * 4, 0));
         } else {
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int ch = cb * KH + 8 * (g0 + 2 * i);
-            const int soff = (ch * plane + rowoff + W + 2) * 2, step = plane * 2;
-            unsigned c[8];
+            for (int i = 0; i < 2; i++) {
+                const int ch = cb * KH + 8 * (g0 + 2 * i);
+                const int soff = (ch * plane + rowoff + W + 2) * 2, step = plane * 2;
+                unsigned c[8];
 #pragma unroll
-            for (int e = 0; e < 8; e++) c[e] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rsrc, vo, soff + e * step, 0);
-            // 2 x 8 transpose of 16-bit values: the low halves are the first pixel's channels, the high halves the second's.
-            // wr[i][0] is the pixel this lane stores first: its first pixel in lanes 0-7 of every sixteen, its second in
-            // lanes 8-15 (store_window)
-            f.wr[i][0].x = __builtin_amdgcn_perm(c[1], c[0], sel_first); f.wr[i][0].y = __builtin_amdgcn_perm(c[3], c[2], sel_first);
-            f.wr[i][0].z = __builtin_amdgcn_perm(c[5], c[4], sel_first); f.wr[i][0].w = __builtin_amdgcn_perm(c[7], c[6], sel_first);
-            f.wr[i][1].x = __builtin_amdgcn_perm(c[1], c[0], sel_second); f.wr[i][1].y = __builtin_amdgcn_perm(c[3], c[2], sel_second);
-            f.wr[i][1].z = __builtin_amdgcn_perm(c[5], c[4], sel_second); f.wr[i][1].w = __builtin_amdgcn_perm(c[7], c[6], sel_second);
-        }
-        if (wave == 0) {
-            const int soff = (cb * KH * plane + rowoff + W + 2) * 2;
-            f.hr = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc, hoff | bit_to_all_ones(hrowinv, r), soff, 0);
-        }
+                for (int e = 0; e < 8; e++) c[e] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rsrc, vo, soff + e * step, 0);
+                // 2 x 8 transpose of 16-bit values: the low halves are the first pixel's channels, the high halves the second's.
+                // wr[i][0] is the pixel this lane stores first: its first pixel in lanes 0-3 of every eight, its second in
+                // lanes 4-7 (store_window)
+                f.wr[i][0].x = __builtin_amdgcn_perm(c[1], c[0], sel_first); f.wr[i][0].y = __builtin_amdgcn_perm(c[3], c[2], sel_first);
+                f.wr[i][0].z = __builtin_amdgcn_perm(c[5], c[4], sel_first); f.wr[i][0].w = __builtin_amdgcn_perm(c[7], c[6], sel_first);
+                f.wr[i][1].x = __builtin_amdgcn_perm(c[1], c[0], sel_second); f.wr[i][1].y = __builtin_amdgcn_perm(c[3], c[2], sel_second);
+                f.wr[i][1].z = __builtin_amdgcn_perm(c[5], c[4], sel_second); f.wr[i][1].w = __builtin_amdgcn_perm(c[7], c[6], sel_second);
+            }
+            if (wave == 0) {
+                const int soff = (cb * KH * plane + rowoff + W + 2) * 2;
+                f.hr = (unsigned)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc, hoff | bit_to_all_ones(hrowinv, r), soff, 0);
+            }
         }
     };
     // A lane's two pixels are neighbouring LDS rows, lane after lane two rows on (160 bytes = 40 words): the eight lanes
@@ -263,11 +263,11 @@ __global__ void __launch_bounds__(NT, RESIDENT) conv3x3_bf16_kernel(const LoadPa
             }
         } else {
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+            for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int e = 0; e < 2; e++)
-                *(uintx4*)(lds + (1 + 2 * (tid & 127) + (e ^ swapped)) * HSTRIDE + 8 * ((tid >> 7) + 2 * i)) = f.wr[i][e];
-        if (wave == 0) lds[((lane >> 5) ? W3_ROWS - 1 : 0) * HSTRIDE + (lane & 31)] = (unsigned short)f.hr;
+                for (int e = 0; e < 2; e++)
+                    *(uintx4*)(lds + (1 + 2 * (tid & 127) + (e ^ swapped)) * HSTRIDE + 8 * ((tid >> 7) + 2 * i)) = f.wr[i][e];
+            if (wave == 0) lds[((lane >> 5) ? W3_ROWS - 1 : 0) * HSTRIDE + (lane & 31)] = (unsigned short)f.hr;
         }
     };
 
@@ -375,61 +375,63 @@ __global__ void __launch_bounds__(NT, RESIDENT) conv3x3_bf16_kernel(const LoadPa
     // applied, rounded to bfloat16) and writes it eight pixels - 16 bytes - per lane, gated by eight elements of the gate
     // tensor fetched the same way; lane by lane the block would leave in two-byte stores of 64-byte runs. Same values.
     // Needs planes of whole groups of eight pixels (a group stays in its sample) and 16-byte aligned tensors.
-    if constexpr (!SPLIT) if (whole && ep.opix % 8 == 0 && (((uintptr_t)ep.out | (uintptr_t)ep.gate) & 15) == 0) {
-        static_assert(NJ == 2 && WM == 1, "one 64 x 64 block per wavefront");
-        constexpr int STG = 72; // row stride of the block in LDS, 16-bit units
-        static_assert(4 * 64 * STG <= 2 * W3_ROWS * HSTRIDE, "the four blocks fit the window buffers");
-        // the gate's elements first (what the lane will overwrite, if the gradient goes over the layer's own input):
-        // fetched one after the other behind each store they would cost a round trip to memory each
-        const int grp = lane & 7;
-        const int j = j0 + wn0 + 8 * grp;
-        const int n = j / ep.opix, pix = j - n * ep.opix;
-        const size_t base = (size_t)n * d.M * ep.opix + pix;
-        uintx4 gv[8];
-        if (ep.gate && j < d.N) {
+    if constexpr (!SPLIT) {
+        if (whole && ep.opix % 8 == 0 && (((uintptr_t)ep.out | (uintptr_t)ep.gate) & 15) == 0) {
+            static_assert(NJ == 2 && WM == 1, "one 64 x 64 block per wavefront");
+            constexpr int STG = 72; // row stride of the block in LDS, 16-bit units
+            static_assert(4 * 64 * STG <= 2 * W3_ROWS * HSTRIDE, "the four blocks fit the window buffers");
+            // the gate's elements first (what the lane will overwrite, if the gradient goes over the layer's own input):
+            // fetched one after the other behind each store they would cost a round trip to memory each
+            const int grp = lane & 7;
+            const int j = j0 + wn0 + 8 * grp;
+            const int n = j / ep.opix, pix = j - n * ep.opix;
+            const size_t base = (size_t)n * d.M * ep.opix + pix;
+            uintx4 gv[8];
+            if (ep.gate && j < d.N) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int m = m0 + (lane >> 3) + 8 * i;
-                gv[i] = m < d.M ? *(const uintx4*)(ep.gate + base + (size_t)m * ep.opix) : uintx4{0, 0, 0, 0};
-            }
-        }
-        __syncthreads(); // every wavefront has read its last fragments
-        unsigned short* stg = &Bw[0][0] + wave * (64 * STG);
-#pragma unroll
-        for (int it = 0; it < 2; it++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int row = it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
-                const int m = m0 + row;
-                const float b = (ep.bias && m < d.M) ? ep.bias[m] : 0.0f;
-#pragma unroll
-                for (int jt = 0; jt < 2; jt++) {
-                    float r = acc[0][it][jt][v];
-                    if (ep.bias) r += b;
-                    if (ep.relu) r = relu_value(r);
-                    stg[row * STG + jt * 32 + l32] = float_to_bf16_bits(r);
+                for (int i = 0; i < 8; i++) {
+                    const int m = m0 + (lane >> 3) + 8 * i;
+                    gv[i] = m < d.M ? *(const uintx4*)(ep.gate + base + (size_t)m * ep.opix) : uintx4{0, 0, 0, 0};
                 }
             }
-        __builtin_amdgcn_wave_barrier(); // the block is read by other lanes of the same wavefront: LDS keeps a wavefront's order
-        if (j < d.N) {
+            __syncthreads(); // every wavefront has read its last fragments
+            unsigned short* stg = &Bw[0][0] + wave * (64 * STG);
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int row = (lane >> 3) + 8 * i;
-                const int m = m0 + row;
-                if (m >= d.M) continue;
-                uintx4 val = *(const uintx4*)(stg + row * STG + 8 * grp);
-                const size_t idx = base + (size_t)m * ep.opix;
-                if (ep.gate) {
-                    // kept where gate > 0: a positive bfloat16 that is not a NaN has bits 0x0001 .. 0x7F80
-                    auto keep = [](unsigned w) {
-                        return ((((w & 0xFFFFu) - 1u) < 0x7F80u) ? 0x0000FFFFu : 0u) | ((((w >> 16) - 1u) < 0x7F80u) ? 0xFFFF0000u : 0u);
-                    };
-                    val.x &= keep(gv[i].x); val.y &= keep(gv[i].y); val.z &= keep(gv[i].z); val.w &= keep(gv[i].w);
+            for (int it = 0; it < 2; it++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int row = it * 32 + 8 * (v / 4) + 4 * lk + (v % 4);
+                    const int m = m0 + row;
+                    const float b = (ep.bias && m < d.M) ? ep.bias[m] : 0.0f;
+#pragma unroll
+                    for (int jt = 0; jt < 2; jt++) {
+                        float r = acc[0][it][jt][v];
+                        if (ep.bias) r += b;
+                        if (ep.relu) r = relu_value(r);
+                        stg[row * STG + jt * 32 + l32] = float_to_bf16_bits(r);
+                    }
                 }
-                *(uintx4*)(ep.out + idx) = val;
+            __builtin_amdgcn_wave_barrier(); // the block is read by other lanes of the same wavefront: LDS keeps a wavefront's order
+            if (j < d.N) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const int row = (lane >> 3) + 8 * i;
+                    const int m = m0 + row;
+                    if (m >= d.M) continue;
+                    uintx4 val = *(const uintx4*)(stg + row * STG + 8 * grp);
+                    const size_t idx = base + (size_t)m * ep.opix;
+                    if (ep.gate) {
+                        // kept where gate > 0: a positive bfloat16 that is not a NaN has bits 0x0001 .. 0x7F80
+                        auto keep = [](unsigned w) {
+                            return ((((w & 0xFFFFu) - 1u) < 0x7F80u) ? 0x0000FFFFu : 0u) | ((((w >> 16) - 1u) < 0x7F80u) ? 0xFFFF0000u : 0u);
+                        };
+                        val.x &= keep(gv[i].x); val.y &= keep(gv[i].y); val.z &= keep(gv[i].z); val.w &= keep(gv[i].w);
+                    }
+                    *(uintx4*)(ep.out + idx) = val;
+                }
             }
+            return;
         }
-        return;
     }
 #pragma unroll
     for (int q = 0; q < NJ / 2; q++) {
