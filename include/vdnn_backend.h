@@ -183,10 +183,13 @@ size_t vdnn_conv_workspace_bytes_dtype(const vdnn_shape_t* shape, int algo_mode,
  * (samples are independent in forward and backward data). */
 size_t vdnn_conv_winograd_chunk_bytes(size_t bytes);
 /* Tuning (no counterpart in the reference; cuDNN's perf-optimal choice is made by cudnnGet*Algorithm, layer.cu:1012-1090):
- * which kernels VDNN_PERF_OPT_ALGO takes for 3x3 / stride 1 / padding 1 layers with float activations where both
- * apply. 0 (default): the bfloat16 matrix cores with every float operand as two bfloat16 parts and three matrix
- * instructions per product (about 5e-6 of the largest output from the exact result; workspace = the filter's bytes);
- * 1: Winograd F(4x4, 3x3) / F(3x3, 4x4) (about 2e-5; workspace of a third to three quarters of a gigabyte). Returns
+ * which kernels VDNN_PERF_OPT_ALGO takes for layers with float activations where both apply. 0 (default): the
+ * bfloat16 matrix cores with every float operand as two bfloat16 parts and three matrix instructions per product
+ * (about 5e-6 of the largest output from the exact result; workspace = the filter's bytes) - forward and backward
+ * data of stride-1 layers (forward: any stride) with at most 32 taps and reduced channels a multiple of 16, backward
+ * filter of 3x3 / stride 1 / padding 1 layers with rows of whole groups of four pixels;
+ * 1: Winograd F(4x4, 3x3) / F(3x3, 4x4) for wide 3x3 / stride 1 / padding 1 layers (about 2e-5; workspace of a third
+ * to three quarters of a gigabyte), which also serves backward filter where variant 0 has no kernel. Returns
  * the previous value; other arguments only query. Process-wide, and it changes what vdnn_conv_workspace_bytes reports:
  * set it before networks are built. */
 int vdnn_conv_perf_variant(int variant);

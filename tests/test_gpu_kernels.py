@@ -421,6 +421,66 @@ def test_conv_split_bf16_against_oracle(ctx, geom):
         assert np.array_equal(dx_.download(x.shape), gated)
 
 
+# The same products through the general bfloat16 engine: stride-1 layers the windowed kernel does not take (and strided
+# forward), reduced channels a multiple of 16, at most 32 taps.
+SPLIT_GENERAL_GEOMS = [
+    (2, 48, 27, 27, 96, 5, 5, 2, 2, 1, 1),      # AlexNet conv2 geometry
+    (2, 64, 12, 12, 80, 5, 5, 0, 0, 1, 1),      # no padding; 80 rows: a ragged row tile
+    (3, 32, 13, 13, 48, 3, 3, 1, 1, 1, 1),      # odd planes, too narrow for Winograd
+    (2, 96, 13, 15, 64, 3, 3, 1, 1, 1, 1),      # 64 rows: the 64 x 256 tile, two items per thread
+    (1, 16, 20, 24, 32, 3, 5, 1, 2, 2, 1),      # strided: forward only
+    (3, 64, 9, 9, 128, 1, 1, 0, 0, 1, 1),       # one tap
+    (130, 16, 7, 7, 16, 3, 3, 1, 1, 1, 1),      # samples smaller than a tile: tiles over several samples
+    (2, 512, 6, 6, 160, 3, 3, 0, 0, 1, 1),      # deep reduction, few tiles: split
+    (2, 256, 13, 13, 384, 3, 3, 1, 1, 1, 1),    # AlexNet conv3 geometry: Winograd applies too, this variant is taken
+]
+
+
+@pytest.mark.parametrize("geom", SPLIT_GENERAL_GEOMS, ids=lambda g: "x".join(map(str, g)))
+def test_conv_split_general_against_oracle(ctx, geom):
+    """Forward (with the rectifier too) and backward data (plain and gated) of the perf-optimal mode through the general
+    bfloat16 engine with float operands as two bfloat16 parts, against the checker: held to 3e-5 (the mode's bound is
+    1e-4), other bits than the memory-optimal kernels' (the variant ran), the same bits twice."""
+    tight = 3e-5
+    n, c, h, w_, k, r, s_, ph, pw, sh, sw = geom
+    rng = np.random.default_rng(hash(geom) % (2 ** 31) + 9)
+    g, og = be.shape(*geom), oracle.shape(*geom)
+    filter_bytes = k * c * r * s_ * 4
+    x = rng.standard_normal((g.n, g.c, g.h, g.w)).astype(np.float32)
+    w = (rng.standard_normal((g.k, g.c, g.r, g.s)) * np.sqrt(2.0 / (g.c * g.r * g.s))).astype(np.float32)
+    b = rng.standard_normal(g.k).astype(np.float32)
+    want_y = oracle.conv_fwd(og, x, w, b)
+    dy = rng.standard_normal(want_y.shape).astype(np.float32)
+    want_dx = oracle.conv_bwd_data(og, dy, w)
+    assert lib.vdnn_conv_perf_variant(-1) == 0
+    assert int(lib.vdnn_conv_workspace_bytes(g, 1, 0)) == filter_bytes
+    bwd_applies = (sh, sw) == (1, 1) and k % 16 == 0
+    if bwd_applies:
+        assert int(lib.vdnn_conv_workspace_bytes(g, 1, 1)) == filter_bytes
+    with Dev(ctx) as d:
+        dx_, dw, db, ddy = d.up(x), d.up(w), d.up(b), d.up(dy)
+        y, y0, gx, gx0 = d.empty(want_y.shape), d.empty(want_y.shape), d.empty(x.shape), d.empty(x.shape)
+        ws = d.empty((filter_bytes // 4,))
+        announce("split general", geom, "fwd")
+        check(lib.vdnn_conv_fwd(ctx.handle, None, g, 1, dx_.ptr, dw.ptr, db.ptr, y.ptr, ws.ptr, filter_bytes))
+        first = y.download(want_y.shape)
+        assert_close(first, want_y, tight, "fwd")
+        check(lib.vdnn_conv_fwd(ctx.handle, None, g, 0, dx_.ptr, dw.ptr, db.ptr, y0.ptr, None, 0))
+        assert not np.array_equal(y0.download(want_y.shape), first)
+        check(lib.vdnn_conv_fwd_relu(ctx.handle, None, g, 1, dx_.ptr, dw.ptr, db.ptr, y.ptr, ws.ptr, filter_bytes))
+        assert np.array_equal(y.download(want_y.shape), np.maximum(first, 0))
+        announce("split general", geom, "bwd_data")
+        check(lib.vdnn_conv_bwd_data(ctx.handle, None, g, 1, ddy.ptr, dw.ptr, gx.ptr, ws.ptr, filter_bytes))
+        plain = gx.download(x.shape)
+        assert_close(plain, want_dx, tight, "bwd data")
+        check(lib.vdnn_conv_bwd_data(ctx.handle, None, g, 0, ddy.ptr, dw.ptr, gx0.ptr, None, 0))
+        assert np.array_equal(gx0.download(x.shape), plain) != bwd_applies
+        check(lib.vdnn_conv_bwd_data_relu(ctx.handle, None, g, 1, ddy.ptr, dw.ptr, dx_.ptr, gx.ptr, ws.ptr, filter_bytes))
+        assert np.array_equal(gx.download(x.shape), np.where(x > 0, plain, 0))
+        check(lib.vdnn_conv_bwd_data(ctx.handle, None, g, 1, ddy.ptr, dw.ptr, gx.ptr, ws.ptr, filter_bytes))
+        assert np.array_equal(gx.download(x.shape), plain)
+
+
 # (geometry, algorithm mode, whether the filter-gradient kernel of the shape adds up the bias gradient itself)
 FILTER_BIAS_GEOMS = [
     ((7, 3, 40, 36, 16, 3, 3, 1, 1, 1, 1), 0, True),       # first-layer kernel: the product's spare column multiplies dy by one

@@ -581,8 +581,9 @@ static int conv_half_engine(vdnn_ctx* ctx, hipStream_t st, const PassNames& name
 // ---- perf-optimal mode, float layers: 3x3 / stride 1 / padding 1 on the bfloat16 matrix cores ------------------
 // Every float operand as two bfloat16 parts, three matrix instructions per product (conv3x3_bf16.h): forward and
 // backward data through the windowed kernel, the split filter bank (as many bytes as the filter) in the workspace.
-// Which variant the perf-optimal mode takes where both apply: 0 = this one (faster on every VGG16 layer, closer to
-// the exact result, no transformed tensors), 1 = Winograd. vdnn_conv_perf_variant.
+// Which variant the perf-optimal mode takes where both apply: 0 = this one, through the windowed kernel or the general
+// engine (faster than Winograd on every VGG16 / AlexNet / OverFeat layer, closer to the exact result, no transformed
+// tensors; backward filter of the layers it does not take stays Winograd's), 1 = Winograd. vdnn_conv_perf_variant.
 static int g_perf_variant = 0;
 
 // MODE 0: rows = output channels, reduced = input channels; MODE 1: rows = input channels, reduced = output channels
@@ -614,6 +615,49 @@ static int launch_split3x3(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, cons
     const Win3x3T<float> geo{src, g.H, g.W, sample, sample * g.N, g.N};
     return launch_win3x3<MODE, float>(ctx, st, MODE == 0 ? kFwdSplitNames : kBwdDataSplitNames, al, geo, ep, rows, g.N * g.H * g.W, reduced * 18,
                                       2.0 * g.N * (double)g.K * g.C * 9 * g.P * g.Q, ctx->reduce_scratch_bytes);
+}
+
+// The same products through the general bfloat16 engine, for stride-1 layers the windowed kernel does not take (other
+// windows than 3x3, no or other padding, planes with odd rows): forward (MODE 0) and backward data (MODE 1), at most 32
+// taps, reduced channels a multiple of 16.
+static bool split_general_ok(const ConvGeo& g, int mode) {
+    const int reduced = mode == 0 ? g.C : g.K, rows = mode == 0 ? g.K : g.C;
+    return g.R * g.S <= 32 && reduced % 16 == 0 && g.C > 4 && (mode == 0 || (g.sh == 1 && g.sw == 1)) &&
+           (long)rows * reduced * g.R * g.S * 4 < (1l << 31);
+}
+
+static const PassNames kFwdSplitGenNames{"conv_fwd_splitgen_64x256", "conv_fwd_splitgen_128x128"};
+static const PassNames kBwdDataSplitGenNames{"conv_bwd_data_splitgen_64x256", "conv_bwd_data_splitgen_128x128"};
+
+template <int MODE>
+static int launch_split_general(vdnn_ctx* ctx, hipStream_t st, const ConvGeo& g, const float* src, const float* w, const StoreNCHW<float>& ep,
+                                void* workspace, size_t workspace_bytes, bool* taken) {
+    *taken = false;
+    const int RS = g.R * g.S;
+    const int rows = MODE == 0 ? g.K : g.C, reduced = MODE == 0 ? g.C : g.K;
+    const size_t bank = (size_t)rows * reduced * RS * 4;
+    if (!split_general_ok(g, MODE) || !workspace || workspace_bytes < bank || !aligned16(workspace)) return VDNN_OK;
+    const long sample = MODE == 0 ? (long)g.C * g.H * g.W : (long)g.K * g.P * g.Q;
+    const int opix = MODE == 0 ? g.P * g.Q : g.H * g.W;
+    if (!pixel_tile_span_ok(sample, opix, 256, 4)) return VDNN_OK;
+    *taken = true;
+    unsigned short* packed = (unsigned short*)workspace;
+    {
+        const long total = (long)rows * reduced * RS;
+        ProfScope prof(ctx, st, "conv_pack_filter", 0.0, 8.0 * (double)total);
+        hipLaunchKernelGGL(pack_filter_split_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, w, packed, rows, reduced, RS,
+                           MODE == 0 ? g.C * RS : RS, MODE == 0 ? RS : g.C * RS, total);
+        VDNN_LAUNCH_CHECK();
+    }
+    const LoadPackedH al{packed, (long)reduced * RS * 2, rows, (unsigned)bank};
+    const FastDiv dRS = FastDiv::make(RS), dS = FastDiv::make(g.S);
+    const double flops = 2.0 * g.N * (double)g.K * g.C * RS * g.P * g.Q;
+    if (MODE == 0) {
+        const LoadIm2colPixTapS<MODE> bl{{src, g.H, g.W, g.P, g.Q, g.R, g.S, g.ph, g.pw, g.sh, g.sw, sample, g.N, dRS, dS}};
+        return launch_by_m<LoadPackedH, LoadIm2colPixTapS<MODE>, float, true>(ctx, st, kFwdSplitGenNames, al, bl, ep, rows, g.N * opix, reduced * RS * 2, flops);
+    }
+    const LoadIm2colPixTapS<MODE> bl{{src, g.P, g.Q, g.H, g.W, g.R, g.S, g.ph, g.pw, 1, 1, sample, g.N, dRS, dS}};
+    return launch_by_m<LoadPackedH, LoadIm2colPixTapS<MODE>, float, true>(ctx, st, kBwdDataSplitGenNames, al, bl, ep, rows, g.N * opix, reduced * RS * 2, flops);
 }
 
 static int launch_pack_filter(vdnn_ctx* ctx, hipStream_t st, const float* w, float* packed, int rows, int Cred, int RS,
@@ -887,6 +931,8 @@ static int conv_fwd_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_shape_t
                 const StoreNCHW<float> eps{y, bias, g.P * g.Q, ctx->reduce_scratch, relu, nullptr};
                 const int rc = launch_split3x3<0>(ctx, st, g, x, w, eps, workspace, workspace_bytes, &taken);
                 if (taken || rc != VDNN_OK) return rc;
+                const int rcg = launch_split_general<0>(ctx, st, g, x, w, eps, workspace, workspace_bytes, &taken);
+                if (taken || rcg != VDNN_OK) return rcg;
             }
             const int rc = launch_winograd(ctx, st, g, false, x, w, bias, y, relu, nullptr, workspace, workspace_bytes, &taken);
             if (taken || rc != VDNN_OK) return rc;
@@ -1026,6 +1072,8 @@ static int conv_bwd_data_impl(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sh
                 const StoreNCHW<float> eps{dx, nullptr, g.H * g.W, ctx->reduce_scratch, 0, gate};
                 const int rc = launch_split3x3<1>(ctx, st, g, dy, w, eps, workspace, workspace_bytes, &taken);
                 if (taken || rc != VDNN_OK) return rc;
+                const int rcg = launch_split_general<1>(ctx, st, g, dy, w, eps, workspace, workspace_bytes, &taken);
+                if (taken || rcg != VDNN_OK) return rcg;
             }
             const int rc = launch_winograd(ctx, st, g, true, dy, w, nullptr, dx, 0, gate, workspace, workspace_bytes, &taken);
             if (taken || rc != VDNN_OK) return rc;
@@ -1372,7 +1420,7 @@ size_t vdnn_conv_workspace_bytes_dtype(const vdnn_shape_t* shape, int algo_mode,
     // for 128-bit operand loads; backward filter takes a staging area large enough for the split count that fills the chip.
     const int RS = g.R * g.S;
     const size_t filter_bytes = (size_t)g.K * g.C * RS * sizeof(float);
-    if (dtype == VDNN_DTYPE_F32 && pass != 2 && g_perf_variant == 0 && split3x3_ok(g, pass)) return filter_bytes;
+    if (dtype == VDNN_DTYPE_F32 && pass != 2 && g_perf_variant == 0 && (split3x3_ok(g, pass) || split_general_ok(g, pass))) return filter_bytes;
     if (dtype == VDNN_DTYPE_F32 && pass != 2 && wino_ok(g, pass == 1)) {
         const WinoPlan p = wino_plan(g, pass == 1);
         if (wino_plan_ok(p)) return p.total;

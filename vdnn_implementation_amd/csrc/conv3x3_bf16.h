@@ -53,33 +53,6 @@ struct Win3x3T {
 };
 typedef Win3x3T<bf16_t> Win3x3;
 
-// Filter bank of a float layer split into bfloat16 parts for the kernel below: 16-channel blocks, tap-major,
-// packed[row][((cb*RS + tap)*2 + part)*16 + l] = part of w[row*row_stride + (cb*16 + l)*red_stride + tap], part 0 = hi, 1 = lo
-// (row_stride / red_stride as in pack_filter_tap_bf16_kernel). One thread per filter element.
-static __global__ void __launch_bounds__(256) pack_filter_split_kernel(const float* __restrict__ w, unsigned short* __restrict__ packed,
-                                                                int rows, int Cred, int RS, int row_stride, int red_stride, long total) {
-    const long i = (long)blockIdx.x * 256 + threadIdx.x;
-    if (i >= total) return;
-    const int per_row = Cred * RS;
-    const int row = (int)(i / per_row), kk = (int)(i - (long)row * per_row);
-    const int l = kk & 15, slice = kk >> 4;
-    const int cb = slice / RS, tap = slice - cb * RS;
-    const float v = w[(long)row * row_stride + (long)(cb * 16 + l) * red_stride + tap];
-    const unsigned short hi = float_to_bf16_bits(v);
-    const unsigned short lo = float_to_bf16_bits(v - __builtin_bit_cast(float, (unsigned)hi << 16));
-    unsigned short* at = packed + (long)row * per_row * 2 + (long)slice * 32 + l;
-    at[0] = hi; at[16] = lo;
-}
-
-typedef float floatx2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-// (hi, lo) parts of two floats, each pair packed into one word (first value in the low half)
-__device__ __forceinline__ void split_pair(float a, float b, unsigned& hi, unsigned& lo) {
-    hi = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{a, b}, bf16x2));
-    const float ha = __builtin_bit_cast(float, hi << 16), hb = __builtin_bit_cast(float, hi & 0xFFFF0000u);
-    lo = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{a - ha, b - hb}, bf16x2));
-}
-
 template <int MODE, class E = bf16_t, int RESIDENT = 3>
 __global__ void __launch_bounds__(NT, RESIDENT) conv3x3_bf16_kernel(const LoadPackedH al, const Win3x3T<E> geo, const StoreNCHW<E> ep, const GemmDims d) {
     constexpr bool SPLIT = std::is_same<E, float>::value;

@@ -19,6 +19,34 @@ constexpr int HSTRIDE = 40; // LDS row stride in 16-bit units
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 
+// Filter bank of a float layer split into bfloat16 parts, for the kernels that multiply float layers on the bfloat16
+// matrix cores (conv3x3_bf16.h, LoadIm2colPixTapS below): 16-channel blocks, tap-major,
+// packed[row][((cb*RS + tap)*2 + part)*16 + l] = part of w[row*row_stride + (cb*16 + l)*red_stride + tap], part 0 = hi, 1 = lo
+// (row_stride / red_stride as in pack_filter_tap_bf16_kernel). One thread per filter element.
+static __global__ void __launch_bounds__(256) pack_filter_split_kernel(const float* __restrict__ w, unsigned short* __restrict__ packed,
+                                                                int rows, int Cred, int RS, int row_stride, int red_stride, long total) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int per_row = Cred * RS;
+    const int row = (int)(i / per_row), kk = (int)(i - (long)row * per_row);
+    const int l = kk & 15, slice = kk >> 4;
+    const int cb = slice / RS, tap = slice - cb * RS;
+    const float v = w[(long)row * row_stride + (long)(cb * 16 + l) * red_stride + tap];
+    const unsigned short hi = float_to_bf16_bits(v);
+    const unsigned short lo = float_to_bf16_bits(v - __builtin_bit_cast(float, (unsigned)hi << 16));
+    unsigned short* at = packed + (long)row * per_row * 2 + (long)slice * 32 + l;
+    at[0] = hi; at[16] = lo;
+}
+
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+// (hi, lo) parts of two floats, each pair packed into one word (first value in the low half)
+__device__ __forceinline__ void split_pair(float a, float b, unsigned& hi, unsigned& lo) {
+    hi = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{a, b}, bf16x2));
+    const float ha = __builtin_bit_cast(float, hi << 16), hb = __builtin_bit_cast(float, hi & 0xFFFF0000u);
+    lo = __builtin_bit_cast(unsigned, __builtin_convertvector(floatx2{a - ha, b - hb}, bf16x2));
+}
+
 // LDS takes a 128-bit store eight lanes at a time, on 32 banks of four bytes (measured: 8 cycles per store when the
 // eight lanes' 32 words fall on 32 different banks, 16 otherwise). With rows of HSTRIDE = 40 halfwords (20 words)
 // four lanes per 64-byte row and two consecutive rows per eight lanes meet on four banks (20 + 12 = 32 = 0); rows
@@ -104,6 +132,58 @@ struct LoadIm2colPixTapH {
         for (int i = 0; i < T / 64; i++) *(uintx4*)(lds + (tid % T) * HSTRIDE + 8 * (tid / T + (NT / T) * i)) = r.v[i];
     }
 };
+
+// The same operand of a float layer for the perf-optimal mode's products of bfloat16 parts (conv3x3_bf16.h): a slice is
+// one tap x 16 channels, an LDS row holds [hi of the 16 channels | lo of the 16 channels]. A lane owns one pixel and
+// fetches eight consecutive channels of it per item as floats, splits them (hi = bf16(v), lo = bf16(v - hi)) and
+// writes two 128-bit LDS pieces. kk0 counts the 16-bit values of a row of the filter operand (32 per slice).
+template <int MODE>
+struct LoadIm2colPixTapS {
+    LoadIm2colPix<MODE, false, float> base; // geometry and per-pixel state of the float engine's loader
+    static constexpr int ITEMS(int T) { return 2 * T / NT > 0 ? 2 * T / NT : 1; } // two channel groups per pixel
+    template <int T> struct Regs { float v[2 * T / NT > 0 ? 2 * T / NT : 1][8]; };
+    template <int T> using State = typename LoadIm2colPix<MODE, false, float>::template State<T>;
+    template <int T>
+    __device__ __forceinline__ void init(State<T>& st, int j0, int tid, int ncols, int k_begin) const {
+        base.template init<T>(st, j0, tid, ncols, k_begin);
+    }
+    template <int T>
+    __device__ __forceinline__ void load(State<T>& st, int kk0, int, int tid, Regs<T>& r) const {
+        static_assert(T == 128 || T == 256, "one or two items per thread");
+        const int plane = base.Hs * base.Ws;
+        const int slice = kk0 / KH;
+        const int cb = base.divRS.div(slice), tap = slice - cb * (base.R * base.S);
+        const int tr = base.divS.div(tap), ts = tap - tr * base.S;
+        const int tapoff = MODE == 0 ? tr * base.Ws + ts : (base.R - 1 - tr) * base.Ws + (base.S - 1 - ts);
+        const int voff = st.vbase | bit_to_all_ones(st.inv, tap);
+        const int g0 = __builtin_amdgcn_readfirstlane(tid / T);
+#pragma unroll
+        for (int i = 0; i < ITEMS(T); i++) {
+            const int ch = cb * 16 + 8 * (g0 + (NT / T) * i);
+            const int soff = (ch * plane + tapoff) * 4, step = plane * 4;
+#pragma unroll
+            for (int e = 0; e < 8; e++) r.v[i][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(st.rsrc, voff, soff + e * step, 0));
+        }
+    }
+    template <int T>
+    __device__ static __forceinline__ void store(unsigned short* lds, int tid, const Regs<T>& r) {
+#pragma unroll
+        for (int i = 0; i < ITEMS(T); i++) {
+            uintx4 hi, lo;
+            unsigned h[4], l[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) split_pair(r.v[i][2 * k], r.v[i][2 * k + 1], h[k], l[k]);
+            hi.x = h[0]; hi.y = h[1]; hi.z = h[2]; hi.w = h[3];
+            lo.x = l[0]; lo.y = l[1]; lo.z = l[2]; lo.w = l[3];
+            unsigned short* at = lds + (tid % T) * HSTRIDE + 8 * (tid / T + (NT / T) * i);
+            *(uintx4*)at = hi;
+            *(uintx4*)(at + 16) = lo;
+        }
+    }
+};
+// Operands whose slices are [hi | lo] parts: the engine multiplies hi x hi + hi x lo + lo x hi instead of the two halves.
+template <class BL> struct SplitProducts { static constexpr bool V = false; };
+template <int MODE> struct SplitProducts<LoadIm2colPixTapS<MODE>> { static constexpr bool V = true; };
 
 // Filter bank rounded to bfloat16 and re-laid-out for the blocked tap-major order:
 // packed[row][(cb*RS + tap)*32 + l] = bf16(w[row*row_stride + (cb*32 + l)*red_stride + tap])
@@ -197,13 +277,23 @@ __global__ void __launch_bounds__(NT, (MinResident<AL, BL>::V)) igemm_bf16_kerne
                 a[h][i] = *(const bf16x8*)(ap + i * 32 * HSTRIDE + 16 * h);
                 b[h][i] = *(const bf16x8*)(bp + i * 32 * HSTRIDE + 16 * h);
             }
+        if constexpr (SplitProducts<BL>::V) {
 #pragma unroll
-        for (int h = 0; h < 2; h++)
+            for (int p = 0; p < 3; p++)
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+                for (int i = 0; i < 2; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[h][i], b[h][j], acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[p == 2][i], b[p == 1][j], acc[i][j], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[h][i], b[h][j], acc[i][j], 0, 0, 0);
+        }
         AL::template store<TM>(As[nxt], tid, ra);
         BL::template store<TN>(Bs[nxt], tid, rb);
         __syncthreads();
