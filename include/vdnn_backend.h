@@ -168,11 +168,13 @@ int vdnn_memcpy_d2d_async(vdnn_ctx* ctx, void* dst_dev, const void* src_dev, siz
 int vdnn_out_dim(int in, int pad, int window, int stride);
 /* cudnnGetConvolution*WorkspaceSize (layer.cu:268-294). algo_mode is a vdnnAlgoMode_t value.
  * VDNN_MEMORY_OPT_ALGO always returns 0. VDNN_PERF_OPT_ALGO (the reference asks cuDNN for its fastest algorithm,
- * layer.cu:1013-1089): forward / backward data of 3x3, stride 1, padding 1 layers with at least 128 reduced and more
- * than 64 produced channels and float activations run as Winograd F(4x4, 3x3) and take the transformed filter plus the
- * transformed input and output of a chunk of samples (up to 512 MiB); other layers take a re-laid-out copy of the
- * filter; backward filter takes room for the partial sums of its split reduction. A pass handed less than this runs
- * the memory-optimal kernels. The _dtype form takes the element type of the activations (VDNN_DTYPE_*); the plain
+ * layer.cu:1013-1089), float activations: forward / backward data on the bfloat16 matrix cores (every float operand
+ * as two bfloat16 parts, see vdnn_conv_perf_variant) take the filter bank split that way - the filter's bytes; under
+ * the Winograd variant, forward / backward data of 3x3, stride 1, padding 1 layers with at least 128 reduced and more
+ * than 64 produced channels take the transformed filter plus the transformed input and output of a chunk of samples
+ * (up to 512 MiB), and so does backward filter where the default variant has no kernel; other layers take a
+ * re-laid-out copy of the filter; backward filter otherwise takes room for the partial sums of its split reduction
+ * where the context's staging area is too small. A pass handed less than this runs the memory-optimal kernels. The _dtype form takes the element type of the activations (VDNN_DTYPE_*); the plain
  * form assumes float. */
 size_t vdnn_conv_workspace_bytes(const vdnn_shape_t* shape, int algo_mode, int pass);
 size_t vdnn_conv_workspace_bytes_dtype(const vdnn_shape_t* shape, int algo_mode, int pass, int dtype);
@@ -236,7 +238,7 @@ int vdnn_conv_bwd_filter_sgd(vdnn_ctx* ctx, vdnn_stream_t stream, const vdnn_sha
 
 /* cudnnConvolutionBackwardBias and cudnnConvolutionBackwardFilter (layer.cu:631-637, 651-660) in one call: both read
  * dy, and for most shapes the filter-gradient kernel adds up the bias gradient from the values it streams (the
- * filter-row kernel of 3x3 / stride 1 / padding 1 layers, the first-layer kernel, the Winograd variant; float
+ * filter-row kernels of 3x3 / stride 1 / padding 1 layers, the first-layer kernel, the Winograd variant; float
  * activations) instead of a second pass over dy. vdnn_conv_bwd_filter_sums_bias says whether a shape's kernel does;
  * where it does not, the call runs the kernels of vdnn_conv_bwd_bias[_sgd] behind the filter gradient on the same
  * stream (a caller that wants them side by side on another stream issues the two calls itself). The bias gradient's

@@ -1415,9 +1415,11 @@ size_t vdnn_conv_workspace_bytes_dtype(const vdnn_shape_t* shape, int algo_mode,
     ConvGeo g;
     if (!shape || !geo_from_shape(shape, g)) return 0;
     if (algo_mode == 0 /* VDNN_MEMORY_OPT_ALGO */ || is_dense(g)) return 0;
-    // Perf-optimal mode: wide 3x3 layers with float activations run forward and backward data as Winograd F(4x4, 3x3)
-    // and take the transformed filter, input and output of a chunk of samples; other layers re-lay the filter bank out
-    // for 128-bit operand loads; backward filter takes a staging area large enough for the split count that fills the chip.
+    // Perf-optimal mode, float activations: forward and backward data on the bfloat16 matrix cores take the filter bank
+    // split into bfloat16 parts (the filter's bytes); under the Winograd variant, and for backward filter where the default
+    // has no kernel, wide 3x3 layers take the transformed filter, input and output of a chunk of samples; other layers
+    // re-lay the filter bank out for 128-bit operand loads; backward filter otherwise takes a staging area large enough
+    // for the split count that fills the chip.
     const int RS = g.R * g.S;
     const size_t filter_bytes = (size_t)g.K * g.C * RS * sizeof(float);
     if (dtype == VDNN_DTYPE_F32 && pass != 2 && g_perf_variant == 0 && (split3x3_ok(g, pass) || split_general_ok(g, pass))) return filter_bytes;
