@@ -239,6 +239,59 @@ def test_conv_perf_opt_variants(ctx, geom, winograd_variant):
         assert_close(got, gpu_conv_bwd_filter(ctx, g, x, dy, zero, np.float32(1.0), algo=0), TOL, "bwd filter, two split counts")
 
 
+def drawn_perf_geometries(seed, count, budget=2.5e8):
+    """Geometries for the perf-optimal mode's routes: channel counts at and beside the multiples of 16 / 64 / 128 its
+    kernels ask for, mostly 3x3 / stride 1 / padding 1 with rows of whole and broken pixel groups, the rest other
+    windows, strides and paddings."""
+    import random
+    rnd = random.Random(seed)
+    channels = [3, 8, 16, 16, 32, 48, 64, 64, 65, 80, 96, 128, 128, 130, 144, 192, 256]
+    out = []
+    while len(out) < count:
+        n, c, k = rnd.choice([1, 2, 3, 5, 9]), rnd.choice(channels), rnd.choice(channels)
+        if rnd.random() < 0.6:
+            r, s, ph, pw, sh, sw = 3, 3, 1, 1, 1, 1
+            h, w = rnd.choice([4, 6, 7, 12, 14, 16, 28]), rnd.choice([4, 6, 8, 10, 13, 14, 16, 18, 20, 28, 36])
+        else:
+            r, s = rnd.choice([(1, 1), (1, 3), (2, 2), (3, 3), (3, 5), (5, 5), (4, 7)])
+            ph, pw = rnd.choice([0, r // 2, r - 1]), rnd.choice([0, s // 2, s - 1])
+            sh, sw = rnd.choice([(1, 1), (1, 1), (1, 1), (2, 2), (2, 1)])
+            h, w = rnd.randint(max(1, r - 2 * ph), 30), rnd.randint(max(1, s - 2 * pw), 30)
+        p, q = (h + 2 * ph - r) // sh + 1, (w + 2 * pw - s) // sw + 1
+        if p < 1 or q < 1 or n * c * k * r * s * p * q > budget:
+            continue
+        out.append((n, c, h, w, k, r, s, ph, pw, sh, sw))
+    return out
+
+
+@pytest.mark.parametrize("variant", [0, 1], ids=["split-bf16", "winograd"])
+@pytest.mark.parametrize("geom", drawn_perf_geometries(11, 20), ids=lambda g: "x".join(map(str, g)))
+def test_conv_perf_opt_drawn_geometries_against_oracle(ctx, geom, variant):
+    """Whatever kernels the perf-optimal mode picks for a drawn geometry, with the workspace it asks for: forward,
+    backward data, backward filter applied to a filter, against the checker to the mode's tolerance."""
+    before = lib.vdnn_conv_perf_variant(variant)
+    try:
+        rng = np.random.default_rng(hash(geom) % (2 ** 31) + 13)
+        g, og = be.shape(*geom), oracle.shape(*geom)
+        x = rng.standard_normal((g.n, g.c, g.h, g.w)).astype(np.float32)
+        w = (rng.standard_normal((g.k, g.c, g.r, g.s)) * np.sqrt(2.0 / (g.c * g.r * g.s))).astype(np.float32)
+        b = rng.standard_normal(g.k).astype(np.float32)
+        announce("conv perf-opt drawn", geom, "fwd variant %d" % variant)
+        want_y = oracle.conv_fwd(og, x, w, b)
+        assert_close(gpu_conv_fwd(ctx, g, x, w, b, algo=1), want_y, TOL, "fwd")
+        dy = rng.standard_normal(want_y.shape).astype(np.float32)
+        announce("conv perf-opt drawn", geom, "bwd_data variant %d" % variant)
+        assert_close(gpu_conv_bwd_data(ctx, g, dy, w, algo=1), oracle.conv_bwd_data(og, dy, w), TOL, "bwd data")
+        announce("conv perf-opt drawn", geom, "bwd_filter variant %d" % variant)
+        zero = np.zeros_like(w)
+        assert_close(gpu_conv_bwd_filter(ctx, g, x, dy, zero, np.float32(1.0), algo=1),
+                     oracle.conv_bwd_filter_sgd(og, x, dy, zero, 1.0), TOL, "bwd filter")
+        got = gpu_conv_bwd_filter(ctx, g, x, dy, w, np.float32(-1e-5), algo=1)
+        assert_close(got, oracle.conv_bwd_filter_sgd(og, x, dy, w, -1e-5), 1e-6, "fused sgd")
+    finally:
+        lib.vdnn_conv_perf_variant(before)
+
+
 # Winograd F(4x4, 3x3): planes that are whole 4x4 tiles and planes that are not (tiles stored in part, rows that are not
 # whole groups of four pixels take the scalar loads), channel counts at and beside the limits
 WINOGRAD_GEOMS = [
