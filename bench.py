@@ -233,6 +233,85 @@ def zvc_standalone(be):
     return out
 
 
+def library_rates(be):
+    """Forward convolutions of three VGG16 layers at batch 128, one kernel at a time, HIP events around ten launches:
+    this library (float memory-optimal, float perf-optimal, bfloat16; NCHW) beside what the image's vendor libraries
+    reach on the same box through PyTorch (`conv2d` with the library's own search switched on, NCHW and channels-last;
+    `matmul` at the product shape of the deepest layer and at 8192 cubed). The perf-optimal rows are priced as issued:
+    three bfloat16 instructions per float product, a third of the bfloat16 peak. Context for the roofline fractions, not
+    part of the path: nothing here is called by the library, and PyTorch is imported by this function only."""
+    import ctypes as C
+    import numpy as np
+    lib, check = be.lib, be.check
+    layers = [(64, 64, 224), (256, 256, 56), (512, 512, 28)]
+    rows = []
+    rng = np.random.default_rng(0)
+    for name, dtype, algo, es, peak in (("f32_memory_opt", 0, 0, 4, 157.3), ("f32_perf_opt", 0, 1, 4, 2500.0 / 3), ("bf16", 1, 0, 2, 2500.0)):
+        ctx = be.Context(pool_bytes=8 << 30)
+        h = ctx.handle
+        try:
+            check(lib.vdnn_ctx_set_activation_dtype(h, dtype))
+            ev = [C.c_void_p(), C.c_void_p()]
+            for e in ev:
+                check(lib.vdnn_event_create(h, C.byref(e), 1))
+            for (c, k, hw) in layers:
+                g = be.shape(128, c, hw, hw, k, 3, 3, 1, 1, 1, 1)
+                x, y, w, b = ctx.alloc(128 * c * hw * hw * es), ctx.alloc(128 * k * hw * hw * es), ctx.alloc(k * c * 9 * 4), ctx.alloc(k * 4)
+                xv = rng.standard_normal(128 * c * hw * hw, dtype=np.float32)   # (random like PyTorch's: the clock follows the data)
+                if es == 2:
+                    xv = (xv.view(np.uint32) >> 16).astype(np.uint16)
+                check(lib.vdnn_memcpy_h2d(h, x.ptr, xv.ctypes.data, xv.nbytes))
+                wv = rng.standard_normal(k * c * 9, dtype=np.float32) * np.float32(np.sqrt(2.0 / (c * 9)))
+                check(lib.vdnn_memcpy_h2d(h, w.ptr, wv.ctypes.data, wv.nbytes))
+                bv = rng.standard_normal(k, dtype=np.float32)
+                check(lib.vdnn_memcpy_h2d(h, b.ptr, bv.ctypes.data, bv.nbytes))
+                nws = int(lib.vdnn_conv_workspace_bytes_dtype(g, algo, 0, dtype))
+                ws = ctx.alloc(max(nws, 256))
+                run = lambda: check(lib.vdnn_conv_fwd(h, None, g, algo, x.ptr, w.ptr, b.ptr, y.ptr, ws.ptr if nws else None, nws))
+                run(); ctx.synchronize()
+                check(lib.vdnn_event_record(h, ev[0], None))
+                for _ in range(10):
+                    run()
+                check(lib.vdnn_event_record(h, ev[1], None)); check(lib.vdnn_event_synchronize(h, ev[1]))
+                ms = C.c_float(); check(lib.vdnn_event_elapsed_ms(h, ev[0], ev[1], C.byref(ms)))
+                tf = 2.0 * 128 * hw * hw * c * k * 9 / (ms.value / 10) / 1e9
+                rows.append({"who": "this library, " + name, "what": "conv %d->%d @%d" % (c, k, hw), "ms": ms.value / 10, "tflops": tf, "of_peak": tf / peak})
+                for t in (x, y, w, b, ws):
+                    t.free()
+        finally:
+            ctx.close()
+    import torch
+    import torch.nn.functional as F
+    torch.backends.cudnn.benchmark = True
+    dev = "cuda:0"
+
+    def timed(fn):
+        fn(); torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            fn()
+        e1.record(); torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / 10
+    for dt, peak in ((torch.float32, 157.3), (torch.bfloat16, 2500.0)):
+        tag = "f32" if dt == torch.float32 else "bf16"
+        for (c, k, hw) in layers:
+            for fmt, fname in ((torch.contiguous_format, "NCHW"), (torch.channels_last, "channels-last")):
+                x = torch.randn(128, c, hw, hw, device=dev, dtype=dt).contiguous(memory_format=fmt)
+                w = torch.randn(k, c, 3, 3, device=dev, dtype=dt).contiguous(memory_format=fmt)
+                ms = timed(lambda: F.conv2d(x, w, padding=1))
+                tf = 2.0 * 128 * hw * hw * c * k * 9 / ms / 1e9
+                rows.append({"who": "vendor conv2d, %s %s" % (tag, fname), "what": "conv %d->%d @%d" % (c, k, hw), "ms": ms, "tflops": tf, "of_peak": tf / peak})
+                del x, w
+        for (m, n, k) in ((512, 100352, 4608), (8192, 8192, 8192)):
+            a, b = torch.randn(m, k, device=dev, dtype=dt), torch.randn(k, n, device=dev, dtype=dt)
+            ms = timed(lambda: torch.matmul(a, b))
+            tf = 2.0 * m * n * k / ms / 1e9
+            rows.append({"who": "vendor matmul, %s" % tag, "what": "%d x %d x %d" % (m, n, k), "ms": ms, "tflops": tf, "of_peak": tf / peak})
+            del a, b
+    return rows
+
+
 def cpu_baseline(batch, threads):
     """The checker's training step (forward, backward, SGD) on the host cores: VGG16, float."""
     import oracle
@@ -271,6 +350,7 @@ def main():
     ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (0: the box's CPU share, at most 16)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--zvc-standalone", action="store_true", help="also time the kernels of the compressed offload alone on the device")
+    ap.add_argument("--library-rates", action="store_true", help="also time single forward convolutions beside the vendor libraries' (through PyTorch); into --details")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus)
@@ -413,6 +493,11 @@ def main():
         log("[bench] compressed offload alone on the device")
         details["zvc_standalone"] = zvc_standalone(be)
         log("[bench]   %s" % json.dumps(details["zvc_standalone"]))
+    if args.library_rates:
+        log("[bench] single forward convolutions beside the vendor libraries'")
+        details["library_rates"] = library_rates(be)
+        for r in details["library_rates"]:
+            log("[bench]   %-36s %-26s %8.3f ms %7.0f TFLOP/s  %.2f of peak" % (r["who"], r["what"], r["ms"], r["tflops"], r["of_peak"]))
     if not args.no_cpu_baseline:
         threads = args.cpu_threads or min(16, os.cpu_count() or 1)
         cpu_batch = args.cpu_batch or 128
