@@ -234,7 +234,8 @@ def zvc_standalone(be):
 
 
 def library_rates(be):
-    """Forward convolutions of three VGG16 layers at batch 128, one kernel at a time, HIP events around ten launches:
+    """Forward convolutions of three VGG16 layers at batch 128, one kernel at a time, HIP events around ten launches after
+    twenty untimed ones:
     this library (float memory-optimal, float perf-optimal, bfloat16; NCHW) beside what the image's vendor libraries
     reach on the same box through PyTorch (`conv2d` with the library's own search switched on, NCHW and channels-last;
     `matmul` at the product shape of the deepest layer and at 8192 cubed). The perf-optimal rows are priced as issued:
@@ -268,7 +269,9 @@ def library_rates(be):
                 nws = int(lib.vdnn_conv_workspace_bytes_dtype(g, algo, 0, dtype))
                 ws = ctx.alloc(max(nws, 256))
                 run = lambda: check(lib.vdnn_conv_fwd(h, None, g, algo, x.ptr, w.ptr, b.ptr, y.ptr, ws.ptr if nws else None, nws))
-                run(); ctx.synchronize()
+                for _ in range(20):   # (the clock takes some milliseconds of load to come up after the upload)
+                    run()
+                ctx.synchronize()
                 check(lib.vdnn_event_record(h, ev[0], None))
                 for _ in range(10):
                     run()
@@ -286,7 +289,9 @@ def library_rates(be):
     dev = "cuda:0"
 
     def timed(fn):
-        fn(); torch.cuda.synchronize()
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(10):
