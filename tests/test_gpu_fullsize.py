@@ -163,17 +163,21 @@ def test_convolution_passes_at_full_size(ctx, layer, batch, bf16):
             for s in samples:
                 want = oracle.conv_bwd_data(one, dy.values(slice(s, s + 1)), wr)
                 compare_act(fetch(ctx, out, s * plane_in, (1, c, hw, hw), bf16), want, bf16, "%s bwd data sample %d algo %d" % (layer, s, algo))
-        announce("full size", layer, geom, "bf16" if bf16 else "f32", "bwd_filter")
-        gw = d.up(np.zeros_like(w))
-        p, n = workspace(d, g, 0, 2)
-        check(lib.vdnn_conv_bwd_filter(ctx.handle, None, g, 0, dx_.ptr, ddy.ptr, gw.ptr, p, n))
-        got = gw.download(w.shape)
+        # both algorithm modes (with float activations the perf-optimal one is another kernel, with another split of the batch)
+        got = {}
+        for algo in (0, 1):
+            announce("full size", layer, geom, "bf16" if bf16 else "f32", "algo", algo, "bwd_filter")
+            gw = d.up(np.zeros_like(w))
+            p, n = workspace(d, g, algo, 2)
+            check(lib.vdnn_conv_bwd_filter(ctx.handle, None, g, algo, dx_.ptr, ddy.ptr, gw.ptr, p, n))
+            got[algo] = gw.download(w.shape)
         four = oracle.shape(batch, 4, hw, hw, 4, 3, 3, 1, 1, 1, 1)
         for k0, c0 in ((0, 0), (k // 2 - 2, c // 2 + 4), (k - 4, c - 4)):
             xs = x.values((slice(None), slice(c0, c0 + 4)))
             dys = dy.values((slice(None), slice(k0, k0 + 4)))
             want = oracle.conv_bwd_filter_sgd(four, xs, dys, np.zeros((4, 4, 3, 3), np.float32), 1.0)
-            assert_close(got[k0:k0 + 4, c0:c0 + 4], want, TOL, "%s bwd filter block (%d, %d)" % (layer, k0, c0))
+            for algo in (0, 1):
+                assert_close(got[algo][k0:k0 + 4, c0:c0 + 4], want, TOL, "%s bwd filter block (%d, %d) algo %d" % (layer, k0, c0, algo))
         # the bias gradient reads the same dy: every channel against a float64 sum over the batch
         announce("full size", layer, geom, "bf16" if bf16 else "f32", "bwd_bias")
         gb = d.up(np.zeros_like(b))
