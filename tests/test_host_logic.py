@@ -413,6 +413,43 @@ def test_unfused_optimizer_costs_one_more_copy_of_the_parameters():
         assert abs(extra - fused["weight_bytes"]) < 64 * 512  # 32 parameter blocks, 512-byte granularity
 
 
+def test_workspace_sizes_of_the_algorithm_modes_vgg16_128():
+    """The workspace protocol of `layer.cu:268-294` (sizes asked per pass) for VGG16's layer shapes at batch 128: none in
+    the memory-optimal mode; in the perf-optimal mode the size of the filter for forward and backward data wherever the
+    reduced channels come in sixteens (the filter as two bfloat16 parts), and - with its Winograd variant selected - the
+    transformed filter plus a chunk's transformed tensors on the layers Winograd takes. Host arithmetic only."""
+    shapes = [(3, 64, 224), (64, 64, 224), (64, 128, 112), (128, 128, 112), (128, 256, 56), (256, 256, 56), (256, 512, 28),
+              (512, 512, 28), (512, 512, 14)]
+    assert lib.vdnn_conv_perf_variant(-1) == 0      # (an unknown value changes nothing and reports the current one)
+    try:
+        for c, k, hw in shapes:
+            g = be.shape(128, c, hw, hw, k, 3, 3, 1, 1, 1, 1)
+            filt = k * c * 9 * 4
+            assert [int(lib.vdnn_conv_workspace_bytes(g, 0, p)) for p in range(3)] == [0, 0, 0]
+            lib.vdnn_conv_perf_variant(0)
+            split = [int(lib.vdnn_conv_workspace_bytes(g, 1, p)) for p in range(3)]
+            assert split[:2] == ([0, 0] if c == 3 else [filt, filt])
+            assert lib.vdnn_conv_perf_variant(1) == 0
+            wino = [int(lib.vdnn_conv_workspace_bytes(g, 1, p)) for p in range(3)]
+            assert lib.vdnn_conv_perf_variant(0) == 1
+            if c >= 128:
+                # transformed filter (36 values per tap set) and at least one sample's transformed input and output
+                tiles = ((hw + 3) // 4) ** 2
+                for p in range(2):
+                    assert wino[p] >= 36 * k * c * 4 + 36 * (c + k) * tiles * 4 and wino[p] % 256 == 0
+                assert wino[2] >= 36 * k * c * 4
+                # backward filter of the split variant: more staging for its splits, or (14 x 14) Winograd's
+                assert split[2] == 0 or split[2] >= filt
+                if hw == 14:
+                    assert split[2] == wino[2]
+            else:
+                assert wino == split
+            # bfloat16 activations: the re-laid-out filter, whatever the variant
+            assert int(lib.vdnn_conv_workspace_bytes_dtype(g, 1, 0, 1)) == (0 if c == 3 else filt)
+    finally:
+        lib.vdnn_conv_perf_variant(0)
+
+
 def test_peak_memory_other_configs():
     for cnn, batch, base, allp in ((VGG16_64, 0, 9.57, 4.70), (OVERFEAT, 128, 1.90, 1.37), (ALEXNET, 32, 0.53, 0.44)):
         with plan(cnn, BASELINE, batch=batch) as net:
